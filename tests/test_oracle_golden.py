@@ -1,0 +1,147 @@
+"""The CPU oracle against every known-answer vector the reference's own tests hold for the hot path."""
+import numpy as np
+import pytest
+
+from conftest import cases_for
+from oracle import oracle as zo
+
+
+def T(d, dtype=np.float32):
+    return None if d is None else np.array(d["data"], dtype=dtype).reshape(d["shape"])
+
+
+@pytest.mark.parametrize("c", cases_for("convolve_tensor_with_bias"))
+def test_convolve_tensor_with_bias(c):
+    y = zo.convolve_tensor_with_bias(T(c["x"]), T(c["w"]), T(c["bias"]), c["stride"], c["dilations"])
+    assert list(y.shape) == c["expect"]["shape"]
+    np.testing.assert_array_equal(y, T(c["expect"]))
+
+
+@pytest.mark.parametrize("c", cases_for("conv_lean", "Conv"))
+def test_conv(c):
+    x, w, b = T(c["x"]), T(c["w"]), T(c["bias"])
+    if c["op"] == "conv_lean":
+        y = np.zeros(c["expect"]["shape"], np.float32)
+        zo.conv_lean(x, w, y, b, c["stride"], c["pads"], c["dilations"], c["group"], c["auto_pad"])
+    else:
+        y = zo.Conv(x, w, b, c["stride"], c["pads"], c["dilations"], c["group"], c["auto_pad"])
+    assert list(y.shape) == c["expect"]["shape"]
+    np.testing.assert_array_equal(y, T(c["expect"]))
+
+
+@pytest.mark.parametrize("c", cases_for("gemm"))
+def test_gemm(c):
+    y = zo.gemm(T(c["a"]), T(c["b"]), T(c["c"]), c["alpha"], c["beta"], c["transA"], c["transB"])
+    assert list(y.shape) == c["expect_shape"]
+    for i, v in c["expect_at"].items():
+        assert y.ravel()[int(i)] == v
+
+
+@pytest.mark.parametrize("c", cases_for("gemm_error"))
+def test_gemm_errors(c):
+    a, b = np.zeros(c["a_shape"], np.float32), np.zeros(c["b_shape"], np.float32)
+    with pytest.raises(zo.OracleError) as e:
+        zo.gemm(a, b, None, 1, 1, c["transA"], c["transB"])
+    assert e.value.name == c["error"]
+
+
+@pytest.mark.parametrize("c", cases_for("mat_mul"))
+def test_mat_mul(c):
+    y = zo.mat_mul(T(c["a"]), T(c["b"]))
+    assert list(y.shape) == c["expect_shape"]
+    for i, v in c["expect_at"].items():
+        assert y.ravel()[int(i)] == v
+
+
+@pytest.mark.parametrize("c", cases_for("mat_mul_error"))
+def test_mat_mul_errors(c):
+    with pytest.raises(zo.OracleError) as e:
+        zo.mat_mul(np.zeros(c["a_shape"], np.float32), np.zeros(c["b_shape"], np.float32))
+    assert e.value.name == c["error"]
+
+
+@pytest.mark.parametrize("c", cases_for("onnx_maxpool"))
+def test_maxpool(c):
+    y = zo.onnx_maxpool(T(c["x"]), c["kernel"], c["strides"], c["dilations"], c["pads"], c["auto_pad"], c["ceil_mode"])
+    assert list(y.shape) == c["expect"]["shape"]
+    np.testing.assert_array_equal(y, T(c["expect"]))
+    # the u8 variant is order preserving: identical on the same integers
+    yq = zo.onnx_maxpool(T(c["x"], np.uint8), c["kernel"], c["strides"], c["dilations"], c["pads"], c["auto_pad"], c["ceil_mode"])
+    np.testing.assert_array_equal(yq, T(c["expect"], np.uint8))
+
+
+@pytest.mark.parametrize("c", cases_for("ReLU"))
+def test_relu(c):
+    np.testing.assert_array_equal(zo.ReLU(T(c["x"])), T(c["expect"]))
+
+
+def test_relu_lean_keeps_previous_content():
+    # lib_activation_function_math.zig:25-27 has no else branch
+    y = np.full(4, 7.0, np.float32)
+    zo.ReLU_lean(np.array([1, -2, -4, 5], np.float32), y)
+    np.testing.assert_array_equal(y, [1, 7, 7, 5])
+
+
+@pytest.mark.parametrize("c", cases_for("leakyReLU"))
+def test_leaky(c):
+    y = zo.leakyReLU(T(c["x"]), c["slope"])
+    assert np.all(np.abs(y - T(c["expect"])) <= c["atol"])
+
+
+@pytest.mark.parametrize("c", cases_for("softmax"))
+def test_softmax(c):
+    y = zo.softmax(T(c["x"]))
+    if c["property"] == "rows_sum_to_1_within_0.1":
+        assert np.all(np.abs(y.sum(axis=1) - 1) < 0.1)
+    else:
+        assert y[0, 0] == y[0, 1] and y[1, 0] == y[1, 1]
+
+
+@pytest.mark.parametrize("c", cases_for("sum_tensors"))
+def test_sum_tensors(c):
+    np.testing.assert_array_equal(zo.sum_tensors_lean(T(c["a"]), T(c["b"])), T(c["expect"]))
+
+
+@pytest.mark.parametrize("c", cases_for("add_bias"))
+def test_add_bias(c):
+    t = T(c["t"]).copy()
+    np.testing.assert_array_equal(zo.add_bias(t, T(c["bias"])), T(c["expect"]))
+
+
+@pytest.mark.parametrize("c", cases_for("reshape"))
+def test_reshape(c):
+    x = T(c["x"], np.uint8)
+    if "error" in c:
+        with pytest.raises(zo.OracleError) as e:
+            zo.reshape_lean(x, c["new_shape"])
+        assert e.value.name == c["error"]
+    else:
+        y = zo.reshape_lean(x, c["new_shape"])
+        assert list(y.shape) == c["expect_shape"]
+        np.testing.assert_array_equal(y.ravel(), x.ravel())
+
+
+def test_conv_error_paths():
+    # group != 1 -> InvalidDimensions (op_convolution.zig:59-65)
+    x, w = np.zeros((1, 2, 4, 4), np.float32), np.zeros((2, 1, 3, 3), np.float32)
+    with pytest.raises(zo.OracleError) as e:
+        zo.conv_lean(x, w, np.zeros((1, 2, 2, 2), np.float32), None, [1, 1], None, None, 2, None)
+    assert e.value.name == "InvalidDimensions"
+    # auto_pad NOTSET without pads -> InvalidPadding (:120-125)
+    w = np.zeros((2, 2, 3, 3), np.float32)
+    with pytest.raises(zo.OracleError) as e:
+        zo.conv_lean(x, w, np.zeros((1, 2, 2, 2), np.float32), None, [1, 1], None, None, 1, "NOTSET")
+    assert e.value.name == "InvalidPadding"
+    # output shape mismatch -> InvalidDimensions (:212-217)
+    with pytest.raises(zo.OracleError) as e:
+        zo.conv_lean(x, w, np.zeros((1, 2, 3, 3), np.float32), None, [1, 1], None, None, 1, None)
+    assert e.value.name == "InvalidDimensions"
+    # rank != 4 -> InvalidDimensions (:44-46)
+    with pytest.raises(zo.OracleError) as e:
+        zo.conv_lean(x[0], w, np.zeros((1, 2, 2, 2), np.float32), None, [1, 1])
+    assert e.value.name == "InvalidDimensions"
+    # pads are ignored unless auto_pad == "NOTSET": the allocating wrapper then
+    # expects the padded shape and the lean call reports the mismatch (:725-728 vs :86)
+    with pytest.raises(zo.OracleError) as e:
+        zo.Conv(x, w, None, [1, 1], [1, 1, 1, 1], None, 1, None)
+    assert e.value.name == "InvalidDimensions"
