@@ -1,0 +1,199 @@
+/*
+ * zant_hip.h -- C ABI of the MI355X (gfx950) backend for Z-Ant's tensor-math hot path.
+ *
+ * One shared library (libzant_hip.so), plain pointers and sizes only.  Every
+ * operator entry point mirrors one `*_lean` function of the reference
+ * (src/Core/Tensor/TensorMath/tensor_math_standard.zig:43-149): the caller owns
+ * and pre-shapes the output, the call validates, enqueues hand-written HIP
+ * kernels on the context's stream and returns a status.  Tensor arguments are
+ * DEVICE pointers (row-major, contiguous, NCHW for rank 4); shape / attribute
+ * arrays are HOST pointers.  A Zig `Tensor(T)` is not `extern` (tensor.zig:25-31),
+ * so the Zig wrapper passes `t.data.ptr` and a copy of `t.shape`.
+ *
+ * Status codes: 0 = ok; negative values name the Zig error the reference would
+ * return (src/Utils/errorHandler.zig:36-84) so the wrapper can map them back and
+ * the generated `predict()` keeps its `catch return` behaviour
+ * (src/codeGen/math_handler.zig:107).  The library never aborts.
+ *
+ * Threading: one zant_ctx = one HIP stream; use one context per host thread.
+ * Calls are asynchronous; zant_hip_sync() waits for the stream.
+ */
+#ifndef ZANT_HIP_H
+#define ZANT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct zant_ctx zant_ctx;
+typedef struct zant_model zant_model;
+
+enum zant_status {
+    ZANT_OK = 0,
+    ZANT_InvalidDimensions = -1,            /* TensorMathError.InvalidDimensions */
+    ZANT_InvalidPadding = -2,               /* TensorMathError.InvalidPadding */
+    ZANT_InputTensorsWrongShape = -3,       /* TensorMathError.InputTensorsWrongShape */
+    ZANT_InputTensorDifferentShape = -4,    /* TensorMathError.InputTensorDifferentShape */
+    ZANT_InputTensorDimensionMismatch = -5, /* TensorMathError.InputTensorDimensionMismatch */
+    ZANT_IncompatibleBroadcastShapes = -6,  /* TensorMathError.IncompatibleBroadcastShapes */
+    ZANT_InputTensorDifferentSize = -7,     /* TensorMathError.InputTensorDifferentSize */
+    ZANT_EmptyTensor = -8,                  /* TensorError.EmptyTensor */
+    ZANT_ZeroSizeTensor = -9,               /* TensorError.ZeroSizeTensor */
+    ZANT_InvalidInput = -10,                /* TensorError.InvalidInput */
+    ZANT_InputArrayWrongSize = -11,         /* TensorError.InputArrayWrongSize */
+    ZANT_WrongStride = -12,                 /* TensorMathError.WrongStride */
+    ZANT_MemError = -13,                    /* TensorMathError.MemError (host or device allocation) */
+    ZANT_HipError = -100,                   /* a HIP runtime call failed; see zant_hip_last_error() */
+    ZANT_NullPointer = -101,
+    ZANT_ArenaOverflow = -102,
+    ZANT_NotFinalized = -103
+};
+
+/* AutoPadType of MaxPool, src/Core/Tensor/TensorMath/op_pooling.zig:9-14. */
+enum zant_auto_pad { ZANT_PAD_NOTSET = 0, ZANT_PAD_SAME_UPPER = 1, ZANT_PAD_SAME_LOWER = 2, ZANT_PAD_VALID = 3 };
+
+/* Activation fused into a producing kernel, or applied in dequantised space
+ * between two quantised tensors. */
+enum zant_act { ZANT_ACT_NONE = 0, ZANT_ACT_RELU = 1, ZANT_ACT_LEAKY = 2, ZANT_ACT_RELU6 = 3 };
+
+/* ---- context, memory, timing ------------------------------------------------ */
+
+/* Creates a context on `device`.  `stream` is a hipStream_t to enqueue on, or
+ * NULL to let the context create (and own) a stream at default priority. */
+int zant_hip_ctx_create(zant_ctx **out, int device, void *stream);
+void zant_hip_ctx_destroy(zant_ctx *ctx);
+int zant_hip_sync(zant_ctx *ctx);
+const char *zant_hip_status_name(int status);
+const char *zant_hip_last_error(zant_ctx *ctx);
+const char *zant_hip_version(void);
+
+/* Replaces setLogFunctionC (src/Core/Tensor/TensorMath/op_convolution.zig:37-41)
+ * and the generated library's setLogFunction (src/codeGen/skeleton.zig:93-97). */
+void setLogFunctionC(void (*func)(char *));
+void setLogFunction(void (*func)(char *));
+
+/* The activation arena: ONE device allocation that model-level forward passes
+ * carve their tensors from (the reference keeps one static array per node
+ * output, src/codeGen/predict.zig:265-272).  Reserving again grows it. */
+int zant_hip_arena_reserve(zant_ctx *ctx, size_t bytes);
+void *zant_hip_arena_ptr(zant_ctx *ctx, size_t offset);
+size_t zant_hip_arena_size(zant_ctx *ctx);
+
+int zant_hip_malloc(zant_ctx *ctx, void **dev_ptr, size_t bytes);
+int zant_hip_free(zant_ctx *ctx, void *dev_ptr);
+int zant_hip_upload(zant_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);
+int zant_hip_download(zant_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes);
+int zant_hip_memset(zant_ctx *ctx, void *dst_dev, int byte_value, size_t bytes);
+
+/* HIP-event stopwatch on the context's stream (what the benchmark times kernels with). */
+int zant_hip_timer_start(zant_ctx *ctx);
+int zant_hip_timer_stop(zant_ctx *ctx, float *elapsed_ms);
+
+/* ---- f32 operators ------------------------------------------------------------ */
+
+/* conv_lean = OnnxConvLean (op_convolution.zig:42-219).  stride/pads/dil are the
+ * Zig slices (pointer + length; pads/dil may be NULL = Zig null); group < 0 = null;
+ * auto_pad is the string the reference compares ("NOTSET", "VALID", "SAME_UPPER",
+ * "SAME_LOWER") or NULL.  As in the reference, pads are honoured only under
+ * "NOTSET" and group must be 1 or null.  fuse_act: ZANT_ACT_NONE, or
+ * ZANT_ACT_RELU to apply ReLU_lean to the result in the same kernel. */
+int zant_hip_conv2d_f32(zant_ctx *ctx, const float *x, const int64_t xdim[4], const float *w,
+                        const int64_t wdim[4], const float *bias, float *y, const int64_t ydim[4],
+                        const int64_t *stride, int n_stride, const int64_t *pads, int n_pads,
+                        const int64_t *dil, int n_dil, int64_t group, const char *auto_pad, int fuse_act);
+/* Shape the allocating wrapper OnnxConv expects (op_convolution.zig:647-732). Host only. */
+int zant_hip_conv2d_out_shape(const int64_t xdim[4], const int64_t wdim[4], const int64_t *stride, int n_stride,
+                              const int64_t *pads, int n_pads, const int64_t *dil, int n_dil, int64_t group,
+                              const char *auto_pad, int64_t ydim[4]);
+
+/* mat_mul_lean = lean_mat_mul (op_mat_mul.zig:92-172): last two dims only. */
+int zant_hip_matmul_f32(zant_ctx *ctx, const float *a, const int64_t *adim, int a_rank, const float *b,
+                        const int64_t *bdim, int b_rank, float *y);
+/* The checks of the allocating mat_mul (op_mat_mul.zig:22-55). Host only. */
+int zant_hip_matmul_check(const int64_t *adim, int a_rank, const int64_t *bdim, int b_rank);
+
+/* gemm_lean = lean_gemm (op_gemm.zig:91-185): Y = alpha*op(A)*op(B) + beta*C on
+ * {1,1,R,C} tensors, C broadcast over rows and/or columns.  Transposes are folded
+ * into the loads.  fuse_act as for conv. */
+int zant_hip_gemm_f32(zant_ctx *ctx, const float *a, const int64_t adim[4], const float *b, const int64_t bdim[4],
+                      const float *c, const int64_t *cdim, int c_rank, float alpha, float beta, int trans_a,
+                      int trans_b, float *y, const int64_t ydim[4], int fuse_act);
+/* The checks of the allocating gemm (op_gemm.zig:15-61); writes the result dims. Host only. */
+int zant_hip_gemm_check(const int64_t *adim, int a_rank, const int64_t *bdim, int b_rank, const int64_t *cdim,
+                        int c_rank, int has_c, int trans_a, int trans_b, int64_t ydim[4]);
+
+/* onnx_maxpool_lean = lean_onnx_maxpool (op_pooling.zig:570-659) and its shape
+ * function get_onnx_maxpool_output_shape (:477-567, host only). */
+int zant_hip_maxpool2d_f32(zant_ctx *ctx, const float *x, const int64_t xdim[4], float *y, const int64_t ydim[4],
+                           const int64_t kernel[2], const int64_t strides[2], const int64_t dil[2],
+                           const int64_t *pads, int n_pads, int auto_pad);
+int zant_hip_maxpool2d_out_shape(const int64_t xdim[4], const int64_t kernel[2], const int64_t strides[2],
+                                 const int64_t dil[2], const int64_t pads[4], int auto_pad, int ceil_mode,
+                                 int64_t ydim[4]);
+
+/* ReLU_lean (lib_activation_function_math.zig:22-28).  The reference writes only
+ * where x > 0 and relies on a zeroed output; this writes x > 0 ? x : 0 everywhere,
+ * which is the same result on the zeroed outputs the reference always passes. */
+int zant_hip_relu_f32(zant_ctx *ctx, const float *x, float *y, int64_t n);
+/* leakyReLU_lean (:68-77): x <= 0 ? slope*x : x. */
+int zant_hip_leaky_relu_f32(zant_ctx *ctx, const float *x, float slope, float *y, int64_t n);
+/* softmax_lean (:154-187): rows = shape[0], cols = shape[1]. */
+int zant_hip_softmax_f32(zant_ctx *ctx, const float *x, float *y, int64_t rows, int64_t cols);
+/* sum_tensors_lean (lib_elementWise_math.zig:70-210): same-size add, else
+ * right-aligned NumPy broadcast (rank <= 8).  Writes the output shape when
+ * ydim_out is not NULL. */
+int zant_hip_add_f32(zant_ctx *ctx, const float *a, const int64_t *adim, int a_rank, const float *b,
+                     const int64_t *bdim, int b_rank, float *y, int64_t *ydim_out, int *y_rank_out);
+/* add_bias (lib_elementWise_math.zig:22-45), in place over the last axis. */
+int zant_hip_add_bias_f32(zant_ctx *ctx, float *t, const int64_t *tdim, int t_rank, const float *bias,
+                          const int64_t *bdim, int b_rank);
+/* reshape_lean (lib_shape_math.zig:1139-1209): resolves 0 / -1 entries into
+ * ydim_out and copies the data unless y == x (a view). */
+int zant_hip_reshape(zant_ctx *ctx, const void *x, const int64_t *xdim, int x_rank, size_t elem_size,
+                     const int64_t *new_shape, int new_rank, void *y, int64_t *ydim_out);
+
+/* ---- int8 operators (ONNX definitions; the reference has none) ----------------- */
+
+/* QuantizeLinear: y = sat_u8(rne(x / y_scale[c]) + y_zp[c]); n_scale == 1 per tensor,
+ * else per `axis`.  y_scale / y_zp are device pointers (y_zp may be NULL = 0). */
+int zant_hip_quantize_linear_f32_u8(zant_ctx *ctx, const float *x, const int64_t *xdim, int rank,
+                                    const float *y_scale, const uint8_t *y_zp, int64_t n_scale, int axis,
+                                    uint8_t *y);
+/* DequantizeLinear: y = (x - x_zp[c]) * x_scale[c]. */
+int zant_hip_dequantize_linear_u8_f32(zant_ctx *ctx, const uint8_t *x, const int64_t *xdim, int rank,
+                                      const float *x_scale, const uint8_t *x_zp, int64_t n_scale, int axis,
+                                      float *y);
+/* QLinearConv (u8 x i8 -> i32 -> u8), explicit pads [top,left,bottom,right], any
+ * group dividing C and K (group == C: depthwise).  w_scale (n_wscale = 1 or K),
+ * w_zp (NULL = 0) and bias (NULL = 0) are device pointers; activation scales and
+ * zero points are host scalars.  Requantisation:
+ *   y = sat_u8(rne((float)acc * ((x_scale * w_scale[k]) / y_scale)) + y_zp)
+ * then, when act != ZANT_ACT_NONE, the fused DequantizeLinear -> act -> QuantizeLinear:
+ *   y = sat_u8(rne(act((y - y_zp) * y_scale) / act_scale) + act_zp). */
+int zant_hip_qlinearconv_u8i8(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], float x_scale,
+                              uint8_t x_zp, const int8_t *w, const int64_t wdim[4], const float *w_scale,
+                              int64_t n_wscale, const int8_t *w_zp, float y_scale, uint8_t y_zp,
+                              const int32_t *bias, uint8_t *y, const int64_t ydim[4], const int64_t stride[2],
+                              const int64_t pads[4], const int64_t dil[2], int64_t group, int act,
+                              float act_alpha, float act_scale, uint8_t act_zp);
+/* DequantizeLinear -> {none, ReLU, LeakyReLU(alpha), ReLU6} -> QuantizeLinear. */
+int zant_hip_qlinear_act_u8(zant_ctx *ctx, const uint8_t *x, int64_t n, float x_scale, uint8_t x_zp, int act,
+                            float alpha, float y_scale, uint8_t y_zp, uint8_t *y);
+/* DequantizeLinear(a) + DequantizeLinear(b) -> QuantizeLinear, same shape. */
+int zant_hip_qlinear_add_u8(zant_ctx *ctx, const uint8_t *a, float a_scale, uint8_t a_zp, const uint8_t *b,
+                            float b_scale, uint8_t b_zp, float y_scale, uint8_t y_zp, uint8_t *y, int64_t n);
+/* MaxPool on quantised values (same window rules as zant_hip_maxpool2d_f32). */
+int zant_hip_maxpool2d_u8(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], uint8_t *y,
+                          const int64_t ydim[4], const int64_t kernel[2], const int64_t strides[2],
+                          const int64_t dil[2], const int64_t *pads, int n_pads, int auto_pad);
+/* Global average pool of a quantised NCHW tensor -> [N,C,1,1]. */
+int zant_hip_qlinear_global_avgpool_u8(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], float x_scale,
+                                       uint8_t x_zp, float y_scale, uint8_t y_zp, uint8_t *y);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ZANT_HIP_H */

@@ -1,0 +1,130 @@
+"""Bit-exact parity of the HIP int8 family (through the C ABI) with the CPU oracle."""
+import numpy as np
+import pytest
+
+from oracle import oracle as zo
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def G():
+    import gpu_util
+    return gpu_util
+
+
+QCASES = [
+    # N, C, H, W, K, KH, KW, stride, pads, dil, group
+    (2, 8, 7, 7, 6, 3, 3, [1, 1], [1, 1, 1, 1], [1, 1], 1),
+    (2, 128, 28, 28, 128, 3, 3, [1, 1], [1, 1, 1, 1], [1, 1], 1),   # config-3 shape, small batch
+    (3, 3, 96, 96, 16, 3, 3, [1, 1], [1, 1, 1, 1], [1, 1], 1),      # tiny-YOLO first layer
+    (2, 256, 3, 3, 27, 1, 1, [1, 1], [0, 0, 0, 0], [1, 1], 1),      # tiny-YOLO head
+    (2, 3, 96, 96, 16, 3, 3, [2, 2], [1, 1, 1, 1], [1, 1], 1),      # MobileNet stem
+    (2, 96, 24, 24, 96, 3, 3, [1, 1], [1, 1, 1, 1], [1, 1], 96),    # depthwise
+    (2, 48, 25, 25, 48, 3, 3, [2, 2], [1, 1, 1, 1], [1, 1], 48),    # depthwise stride 2, odd size
+    (2, 16, 24, 24, 96, 1, 1, [1, 1], [0, 0, 0, 0], [1, 1], 1),     # pointwise expand
+    (1, 8, 6, 6, 4, 3, 3, [2, 1], [0, 1, 2, 0], [1, 1], 2),         # grouped, asymmetric pads
+    (1, 3, 9, 9, 5, 2, 2, [1, 1], [0, 0, 0, 0], [2, 2], 1),         # dilation
+    (4, 1280, 1, 1, 1000, 1, 1, [1, 1], [0, 0, 0, 0], [1, 1], 1),   # final Gemm as a 1x1 conv
+]
+
+
+@pytest.mark.parametrize("case", QCASES, ids=[str(i) for i in range(len(QCASES))])
+@pytest.mark.parametrize("act", [None, "leaky", "relu6"])
+def test_qlinearconv_bit_exact(G, case, act):
+    N, C, H, W, K, KH, KW, s, p, d, grp = case
+    g = np.random.default_rng(7 * N + C + K)
+    x = g.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+    w = g.integers(-127, 128, (K, C // grp, KH, KW), dtype=np.int8)
+    fan = (C // grp) * KH * KW
+    ws = (g.uniform(0.5, 1.5, K) * 0.08 / np.sqrt(fan)).astype(np.float32)   # spreads outputs over the u8 range
+    b = g.integers(-1000, 1001, K, dtype=np.int32)
+    kw = dict(act=act, act_alpha=0.1, act_scale=0.04, act_zp=30) if act else {}
+    ref = zo.qlinearconv(x, 0.02, 128, w, ws, None, 0.05, 128, b, s, p, d, grp, **kw)
+    y = G.tm.qlinearconv(G.dev(x), 0.02, 128, G.dev(w), G.dev(ws), None, 0.05, 128, G.dev(b), s, p, d, grp, **kw)
+    np.testing.assert_array_equal(G.host(y), ref)
+    assert len(np.unique(ref)) > 8  # the case really exercises requantisation
+
+
+def test_qlinearconv_per_tensor_scale_weight_zero_point_no_bias(G):
+    g = np.random.default_rng(1)
+    x = g.integers(0, 256, (2, 8, 9, 9), dtype=np.uint8)
+    w = g.integers(-127, 128, (12, 8, 3, 3), dtype=np.int8)
+    wz = g.integers(-5, 6, 12, dtype=np.int8)
+    ws = np.array([0.004], np.float32)
+    ref = zo.qlinearconv(x, 0.03, 7, w, ws, wz, 0.06, 100, None, [1, 1], [1, 1, 1, 1], [1, 1])
+    y = G.tm.qlinearconv(G.dev(x), 0.03, 7, G.dev(w), G.dev(ws), G.dev(wz), 0.06, 100, None, [1, 1], [1, 1, 1, 1], [1, 1])
+    np.testing.assert_array_equal(G.host(y), ref)
+
+
+def test_qlinearconv_errors(G):
+    import torch
+    x = torch.zeros((1, 4, 5, 5), dtype=torch.uint8, device="cuda:0")
+    w = torch.zeros((4, 2, 3, 3), dtype=torch.int8, device="cuda:0")
+    ws = torch.ones(4, device="cuda:0")
+    with pytest.raises(G.ZantError) as e:  # group does not match the weight's channels per group
+        G.tm.qlinearconv(x, 1.0, 0, w, ws, None, 1.0, 0, None, [1, 1], [1, 1, 1, 1], [1, 1], 1)
+    assert e.value.name == "InvalidDimensions"
+    with pytest.raises(G.ZantError) as e:  # wrong number of weight scales
+        G.tm.qlinearconv(x, 1.0, 0, w, ws[:3].contiguous(), None, 1.0, 0, None, [1, 1], [1, 1, 1, 1], [1, 1], 2)
+    assert e.value.name == "InputTensorDimensionMismatch"
+
+
+def test_quantize_dequantize_bit_exact(G):
+    g = np.random.default_rng(2)
+    x = (g.standard_normal((3, 5, 17, 9)) * 3).astype(np.float32)
+    x.ravel()[:8] = [0.5, 1.5, 2.5, -0.5, -1.5, 1e9, -1e9, 0.49999997]
+    for s, zp, axis in [(np.float32(0.05), 128, 1), (np.array([0.01, 0.02, 0.05, 0.1, 1.0], np.float32), np.array([128, 100, 0, 255, 3], np.uint8), 1),
+                        (np.array([0.5, 0.25, 1.0], np.float32), None, 0)]:
+        ref = zo.quantize_linear(x, s, zp, axis)
+        q = G.tm.quantize_linear(G.dev(x), s, zp, axis)
+        np.testing.assert_array_equal(G.host(q), ref)
+        np.testing.assert_array_equal(G.host(G.tm.dequantize_linear(q, s, zp, axis)), zo.dequantize_linear(ref, s, zp, axis))
+    t = np.array([0.5, 1.5, 2.5, -0.5, 3.5, 254.5, 255.5], np.float32)  # ties and saturation
+    np.testing.assert_array_equal(G.host(G.tm.quantize_linear(G.dev(t), 1.0, 0)), [0, 2, 2, 0, 4, 254, 255])
+
+
+@pytest.mark.parametrize("act,alpha", [("relu", 0.0), ("leaky", 0.1), ("relu6", 0.0), (None, 0.0)])
+@pytest.mark.parametrize("n", [256, 100003])
+def test_qlinear_act_bit_exact(G, act, alpha, n):
+    g = np.random.default_rng(n)
+    q = g.integers(0, 256, n, dtype=np.uint8)
+    q[:256] = np.arange(256)
+    y = G.tm.qlinear_act(G.dev(q), 0.05, 128, act, alpha, 0.03, 20)
+    np.testing.assert_array_equal(G.host(y), zo.qlinear_act(q, 0.05, 128, act, alpha, 0.03, 20))
+
+
+@pytest.mark.parametrize("n", [7, 4096, 1000003])
+def test_qlinear_add_bit_exact(G, n):
+    g = np.random.default_rng(n)
+    a = g.integers(0, 256, n, dtype=np.uint8); b = g.integers(0, 256, n, dtype=np.uint8)
+    y = G.tm.qlinear_add(G.dev(a), 0.02, 128, G.dev(b), 0.03, 120, 0.04, 125)
+    np.testing.assert_array_equal(G.host(y), zo.qlinear_add(a, 0.02, 128, b, 0.03, 120, 0.04, 125))
+
+
+def test_qlinear_global_avgpool_bit_exact(G):
+    g = np.random.default_rng(4)
+    for shape in [(3, 5, 3, 3), (8, 1280, 3, 3), (2, 7, 13, 11)]:
+        x = g.integers(0, 256, shape, dtype=np.uint8)
+        y = G.tm.qlinear_global_avgpool(G.dev(x), 0.05, 128, 0.02, 110)
+        np.testing.assert_array_equal(G.host(y), zo.qlinear_global_avgpool(x, 0.05, 128, 0.02, 110))
+
+
+def test_full_size_qlinearconv_properties(G):
+    """Config 3 at its real shape: a slice against the oracle plus batch-permutation equivariance."""
+    import torch
+    g = np.random.default_rng(3)
+    N, C, H, K = 128, 128, 28, 128
+    x = g.integers(0, 256, (N, C, H, H), dtype=np.uint8)
+    w = g.integers(-127, 128, (K, C, 3, 3), dtype=np.int8)
+    ws = g.uniform(0.001, 0.01, K).astype(np.float32)
+    b = g.integers(-1000, 1001, K, dtype=np.int32)
+    args = ([1, 1], [1, 1, 1, 1], [1, 1])
+    X, Wt, WS, Bt = G.dev(x), G.dev(w), G.dev(ws), G.dev(b)
+    y = G.tm.qlinearconv(X, 0.02, 128, Wt, WS, None, 0.05, 128, Bt, *args)
+    perm = torch.randperm(N, device="cuda:0")
+    yp = G.tm.qlinearconv(X[perm].contiguous(), 0.02, 128, Wt, WS, None, 0.05, 128, Bt, *args)
+    torch.cuda.synchronize()
+    assert torch.equal(yp, y[perm])
+    ref = zo.qlinearconv(x[60:62], 0.02, 128, w, ws, None, 0.05, 128, b, *args)
+    np.testing.assert_array_equal(G.host(y[60:62]), ref)

@@ -1,0 +1,41 @@
+"""Builds libzant_hip.so (the product) for gfx950 with hipcc.  Cross-compiles without a GPU.
+
+Usage: python z-ant_amd/build.py            (from the repository root)
+"""
+import glob
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libzant_hip.so")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    # never let the compiler form packed-f32 VALU ops; rounding of a*b+c stays two-step everywhere
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-ffp-contract=off",
+    "-Wall", "-Wno-unused-function",
+    "-I", os.path.join(ROOT, "include"), "-I", CSRC,
+]
+
+
+def sources():
+    return sorted(glob.glob(os.path.join(CSRC, "*.hip")))
+
+
+def build(verbose=True):
+    cmd = [HIPCC] + FLAGS + sources() + ["-o", LIB]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return LIB
+
+
+if __name__ == "__main__":
+    build()
+    print("built", LIB)
+    sys.exit(0)

@@ -1,0 +1,67 @@
+// Shared internals of libzant_hip.so: the context, status helpers and launch utilities.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <string>
+
+#include "zant_hip.h"
+
+struct zant_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    bool owns_stream = false;
+    // activation arena: one allocation, bump/plan addressed by offset
+    void *arena = nullptr;
+    size_t arena_bytes = 0;
+    // scratch for per-call packed weights / multiplier tables (grown on demand, never shrunk)
+    void *workspace = nullptr;
+    size_t workspace_bytes = 0;
+    hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+    int num_cus = 256;
+    std::string last_error;
+};
+
+extern void (*g_zant_log)(char *);
+static inline void zant_log(const char *msg) {
+    if (g_zant_log) g_zant_log(const_cast<char *>(msg));
+}
+
+// Records a failed HIP call on the context and yields ZANT_HipError.
+int zant_fail_hip(zant_ctx *ctx, hipError_t e, const char *what);
+
+#define ZANT_HIP_TRY(ctx, expr)                                      \
+    do {                                                             \
+        hipError_t _e = (expr);                                      \
+        if (_e != hipSuccess) return zant_fail_hip((ctx), _e, #expr); \
+    } while (0)
+
+// Checks the launch that was just enqueued.
+#define ZANT_LAUNCH_CHECK(ctx) ZANT_HIP_TRY(ctx, hipGetLastError())
+
+// Grows the context's workspace to at least `bytes` (stream-ordered use only).
+int zant_workspace(zant_ctx *ctx, size_t bytes, void **out);
+
+static inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
+static inline int64_t prod_dims(const int64_t *d, int rank) {
+    int64_t p = 1;
+    for (int i = 0; i < rank; ++i) p *= d[i];
+    return p;
+}
+
+// Geometry every 2-D convolution kernel takes (already validated, int32 safe).
+struct ConvGeom {
+    int N, C, H, W;      // input
+    int K, CG, KH, KW;   // filters, channels per group, kernel
+    int OH, OW;
+    int sh, sw, dh, dw;
+    int pt, pl;          // pad top / left (bottom/right are implied by OH/OW)
+    int groups;
+};
+
+// Resolves OnnxConvLean's stride / dilation defaults and pads; host only.
+int zant_conv_resolve(const int64_t xdim[4], const int64_t wdim[4], const int64_t *stride, int n_stride,
+                      const int64_t *pads, int n_pads, const int64_t *dil, int n_dil, int64_t group,
+                      const char *auto_pad, int64_t s[2], int64_t d[2], int64_t p[4]);

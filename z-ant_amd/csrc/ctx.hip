@@ -1,0 +1,183 @@
+// Context, arena, transfers, timing and status names of libzant_hip.so.
+#include "common.h"
+
+void (*g_zant_log)(char *) = nullptr;
+
+extern "C" void setLogFunctionC(void (*func)(char *)) { g_zant_log = func; }
+extern "C" void setLogFunction(void (*func)(char *)) { g_zant_log = func; }
+
+int zant_fail_hip(zant_ctx *ctx, hipError_t e, const char *what) {
+    if (ctx) {
+        ctx->last_error = std::string(what) + ": " + hipGetErrorString(e);
+        zant_log(ctx->last_error.c_str());
+    }
+    return ZANT_HipError;
+}
+
+int zant_workspace(zant_ctx *ctx, size_t bytes, void **out) {
+    if (bytes > ctx->workspace_bytes) {
+        // The old buffer may still be read by queued kernels: drain before replacing it.
+        ZANT_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+        if (ctx->workspace) ZANT_HIP_TRY(ctx, hipFree(ctx->workspace));
+        ctx->workspace = nullptr;
+        ctx->workspace_bytes = 0;
+        size_t want = bytes < (size_t(1) << 20) ? (size_t(1) << 20) : bytes;
+        ZANT_HIP_TRY(ctx, hipMalloc(&ctx->workspace, want));
+        ctx->workspace_bytes = want;
+    }
+    *out = ctx->workspace;
+    return ZANT_OK;
+}
+
+extern "C" int zant_hip_ctx_create(zant_ctx **out, int device, void *stream) {
+    if (!out) return ZANT_NullPointer;
+    *out = nullptr;
+    zant_ctx *ctx = new (std::nothrow) zant_ctx();
+    if (!ctx) return ZANT_MemError;
+    ctx->device = device;
+    hipError_t e = hipSetDevice(device);
+    if (e != hipSuccess) { delete ctx; return ZANT_HipError; }
+    if (stream) {
+        ctx->stream = static_cast<hipStream_t>(stream);
+    } else {
+        e = hipStreamCreate(&ctx->stream);  // default priority
+        if (e != hipSuccess) { delete ctx; return ZANT_HipError; }
+        ctx->owns_stream = true;
+    }
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device) == hipSuccess) ctx->num_cus = prop.multiProcessorCount;
+    if (hipEventCreate(&ctx->ev_start) != hipSuccess || hipEventCreate(&ctx->ev_stop) != hipSuccess) {
+        zant_hip_ctx_destroy(ctx);
+        return ZANT_HipError;
+    }
+    *out = ctx;
+    return ZANT_OK;
+}
+
+extern "C" void zant_hip_ctx_destroy(zant_ctx *ctx) {
+    if (!ctx) return;
+    (void)hipSetDevice(ctx->device);
+    if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->arena) (void)hipFree(ctx->arena);
+    if (ctx->workspace) (void)hipFree(ctx->workspace);
+    if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
+    if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);
+    if (ctx->owns_stream && ctx->stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+}
+
+extern "C" int zant_hip_sync(zant_ctx *ctx) {
+    if (!ctx) return ZANT_NullPointer;
+    ZANT_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return ZANT_OK;
+}
+
+extern "C" const char *zant_hip_last_error(zant_ctx *ctx) { return ctx ? ctx->last_error.c_str() : ""; }
+extern "C" const char *zant_hip_version(void) { return "zant-hip 0.1 (gfx950)"; }
+
+extern "C" const char *zant_hip_status_name(int s) {
+    switch (s) {
+    case ZANT_OK: return "OK";
+    case ZANT_InvalidDimensions: return "InvalidDimensions";
+    case ZANT_InvalidPadding: return "InvalidPadding";
+    case ZANT_InputTensorsWrongShape: return "InputTensorsWrongShape";
+    case ZANT_InputTensorDifferentShape: return "InputTensorDifferentShape";
+    case ZANT_InputTensorDimensionMismatch: return "InputTensorDimensionMismatch";
+    case ZANT_IncompatibleBroadcastShapes: return "IncompatibleBroadcastShapes";
+    case ZANT_InputTensorDifferentSize: return "InputTensorDifferentSize";
+    case ZANT_EmptyTensor: return "EmptyTensor";
+    case ZANT_ZeroSizeTensor: return "ZeroSizeTensor";
+    case ZANT_InvalidInput: return "InvalidInput";
+    case ZANT_InputArrayWrongSize: return "InputArrayWrongSize";
+    case ZANT_WrongStride: return "WrongStride";
+    case ZANT_MemError: return "MemError";
+    case ZANT_HipError: return "HipError";
+    case ZANT_NullPointer: return "NullPointer";
+    case ZANT_ArenaOverflow: return "ArenaOverflow";
+    case ZANT_NotFinalized: return "NotFinalized";
+    default: return "Unknown";
+    }
+}
+
+extern "C" int zant_hip_arena_reserve(zant_ctx *ctx, size_t bytes) {
+    if (!ctx) return ZANT_NullPointer;
+    if (bytes <= ctx->arena_bytes) return ZANT_OK;
+    ZANT_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    if (ctx->arena) ZANT_HIP_TRY(ctx, hipFree(ctx->arena));
+    ctx->arena = nullptr;
+    ctx->arena_bytes = 0;
+    hipError_t e = hipMalloc(&ctx->arena, bytes);
+    if (e != hipSuccess) { zant_fail_hip(ctx, e, "hipMalloc(arena)"); return ZANT_MemError; }
+    ctx->arena_bytes = bytes;
+    return ZANT_OK;
+}
+
+extern "C" void *zant_hip_arena_ptr(zant_ctx *ctx, size_t offset) {
+    if (!ctx || !ctx->arena || offset >= ctx->arena_bytes) return nullptr;
+    return static_cast<char *>(ctx->arena) + offset;
+}
+
+extern "C" size_t zant_hip_arena_size(zant_ctx *ctx) { return ctx ? ctx->arena_bytes : 0; }
+
+extern "C" int zant_hip_malloc(zant_ctx *ctx, void **dev_ptr, size_t bytes) {
+    if (!ctx || !dev_ptr) return ZANT_NullPointer;
+    hipError_t e = hipMalloc(dev_ptr, bytes ? bytes : 1);
+    if (e != hipSuccess) { zant_fail_hip(ctx, e, "hipMalloc"); return ZANT_MemError; }
+    return ZANT_OK;
+}
+
+extern "C" int zant_hip_free(zant_ctx *ctx, void *dev_ptr) {
+    if (!ctx) return ZANT_NullPointer;
+    if (!dev_ptr) return ZANT_OK;
+    ZANT_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    ZANT_HIP_TRY(ctx, hipFree(dev_ptr));
+    return ZANT_OK;
+}
+
+extern "C" int zant_hip_upload(zant_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes) {
+    if (!ctx || (bytes && (!dst_dev || !src_host))) return ZANT_NullPointer;
+    if (!bytes) return ZANT_OK;
+    ZANT_HIP_TRY(ctx, hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, ctx->stream));
+    ZANT_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));  // the host buffer may be pageable and reused
+    return ZANT_OK;
+}
+
+extern "C" int zant_hip_download(zant_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes) {
+    if (!ctx || (bytes && (!dst_host || !src_dev))) return ZANT_NullPointer;
+    if (!bytes) return ZANT_OK;
+    ZANT_HIP_TRY(ctx, hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    ZANT_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return ZANT_OK;
+}
+
+__global__ void zant_fill_bytes_kernel(uint8_t *p, uint8_t v, size_t n) {
+    size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    const size_t step = size_t(gridDim.x) * blockDim.x;
+    for (; i < n; i += step) p[i] = v;
+}
+
+extern "C" int zant_hip_memset(zant_ctx *ctx, void *dst_dev, int byte_value, size_t bytes) {
+    if (!ctx || (bytes && !dst_dev)) return ZANT_NullPointer;
+    if (!bytes) return ZANT_OK;
+    // A fill kernel rather than hipMemsetAsync so the call stays safe under graph capture.
+    size_t blocks = (bytes + 255) / 256;
+    if (blocks > 65535) blocks = 65535;
+    hipLaunchKernelGGL(zant_fill_bytes_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream,
+                       static_cast<uint8_t *>(dst_dev), (uint8_t)byte_value, bytes);
+    ZANT_LAUNCH_CHECK(ctx);
+    return ZANT_OK;
+}
+
+extern "C" int zant_hip_timer_start(zant_ctx *ctx) {
+    if (!ctx) return ZANT_NullPointer;
+    ZANT_HIP_TRY(ctx, hipEventRecord(ctx->ev_start, ctx->stream));
+    return ZANT_OK;
+}
+
+extern "C" int zant_hip_timer_stop(zant_ctx *ctx, float *elapsed_ms) {
+    if (!ctx || !elapsed_ms) return ZANT_NullPointer;
+    ZANT_HIP_TRY(ctx, hipEventRecord(ctx->ev_stop, ctx->stream));
+    ZANT_HIP_TRY(ctx, hipEventSynchronize(ctx->ev_stop));
+    ZANT_HIP_TRY(ctx, hipEventElapsedTime(elapsed_ms, ctx->ev_start, ctx->ev_stop));
+    return ZANT_OK;
+}

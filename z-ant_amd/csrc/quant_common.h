@@ -1,0 +1,36 @@
+// Device helpers shared by the int8 kernels: the single requantisation sequence and the fused
+// Dequantize -> activation -> Quantize step.
+#pragma once
+#include "common.h"
+
+// round-half-to-even (v_rndne_f32), add the zero point as a float (exact), saturate, convert.
+__device__ __forceinline__ uint8_t sat_u8_rne(float v, uint8_t zp) {
+    float r = __builtin_rintf(v) + float(zp);
+    r = __builtin_fmaxf(r, 0.0f);  // NaN -> 0
+    r = __builtin_fminf(r, 255.0f);
+    return uint8_t(r);
+}
+
+struct QAct {
+    int act;            // zant_act
+    float alpha;        // LeakyReLU slope
+    float in_scale;     // scale / zero point of the tensor the activation reads
+    int in_zp;
+    float out_scale;    // scale / zero point of the tensor it writes
+    uint8_t out_zp;
+};
+
+__device__ __forceinline__ float act_f32(float v, int act, float alpha) {
+    switch (act) {
+    case ZANT_ACT_RELU: return v > 0.0f ? v : 0.0f;
+    case ZANT_ACT_LEAKY: return v <= 0.0f ? alpha * v : v;
+    case ZANT_ACT_RELU6: return __builtin_fminf(__builtin_fmaxf(v, 0.0f), 6.0f);
+    default: return v;
+    }
+}
+
+// q -> sat_u8(rne(act((q - in_zp) * in_scale) / out_scale) + out_zp)
+__device__ __forceinline__ uint8_t qact_apply(uint8_t q, const QAct &a) {
+    const float v = act_f32(float(int(q) - a.in_zp) * a.in_scale, a.act, a.alpha);
+    return sat_u8_rne(v / a.out_scale, a.out_zp);
+}
