@@ -11,159 +11,330 @@
 // Output channels are the MFMA rows and output positions the MFMA columns, so each accumulator
 // register holds 32 consecutive NCHW positions and stores are 128-byte coalesced.
 // A direct kernel (one thread per output element) covers shapes the tiled kernel does not take.
+#include <algorithm>
+
 #include "common.h"
 
 namespace {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __attribute__((address_space(1))) const void *gptr_t;
+typedef __attribute__((address_space(3))) void *lptr_t;
 
 constexpr int CC = 8;  // input channels staged per chunk (4 MFMA k-steps per filter tap)
 
 struct TileGeom {
-    int NB, TH;          // images per workgroup, output rows per workgroup
-    int PH, PW, P1;      // staged patch rows / cols, floats per channel (NB*PH*PW)
+    int NB, TH;          // images per workgroup tile, output rows per tile
+    int PH, PW, P1;      // staged patch rows / cols, positions per channel (NB*PH*PW)
+    int P1s;             // P1 rounded up to a multiple of 4
     int n_row_tiles;     // ceil(OH / TH)
     int n_chunks;        // ceil(C / CC)
     int n_kblocks;       // ceil(K / K_BLK)
-    int n_sblocks;       // spatial workgroups
-    int positions;       // NB*TH*OW valid positions per workgroup
+    int n_sblocks;       // spatial tiles
+    int n_tiles;         // n_sblocks * n_kblocks
 };
 
-// Packs OIHW weights into [chunk][kblock][tap][cc][K_BLK] (zero padded) so a chunk's slab is one
-// contiguous, 16-byte aligned run whose LDS image has the output channel as the fastest axis.
+// Packs OIHW weights into [chunk][kblock][tap][half][K_BLK][4] (zero padded):
+// element (half, k, j) holds W[k][chunk*8 + half*4 + j][tap].  A chunk's slab is one contiguous
+// 16-byte aligned run, and one 128-bit LDS read per lane fetches the A operands of 4 k-steps.
+// Thread 0 also resets the tile counter the persistent convolution workgroups draw from.
 __global__ void pack_weights_f32_kernel(const float *__restrict__ w, float *__restrict__ wp, int K, int C, int T,
-                                        int n_chunks, int n_kblocks, int k_blk) {
+                                        int n_chunks, int n_kblocks, int k_blk, int *__restrict__ tile_counter,
+                                        int counter_init) {
     const int64_t total = int64_t(n_chunks) * n_kblocks * T * CC * k_blk;
     const int64_t step = int64_t(gridDim.x) * blockDim.x;
+    if (blockIdx.x == 0 && threadIdx.x == 0) *tile_counter = counter_init;
     for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += step) {
         int64_t r = i;
+        const int j = int(r & 3); r >>= 2;
         const int kk = int(r % k_blk); r /= k_blk;
-        const int cc = int(r % CC); r /= CC;
+        const int half = int(r & 1); r >>= 1;
         const int tap = int(r % T); r /= T;
         const int kb = int(r % n_kblocks); r /= n_kblocks;
         const int chunk = int(r);
-        const int k = kb * k_blk + kk, c = chunk * CC + cc;
+        const int k = kb * k_blk + kk, c = chunk * CC + half * 4 + j;
         wp[i] = (k < K && c < C) ? w[(int64_t(k) * C + c) * T + tap] : 0.0f;
     }
 }
 
-// MT: 32-position MFMA tiles per wave; WM x WN waves per workgroup (positions x output channels).
-template <int MT, int WM, int WN>
-__global__ void __launch_bounds__(WM *WN * 64, 2)
-conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, const float *__restrict__ bias,
-                     float *__restrict__ y, ConvGeom g, TileGeom t, int relu) {
+// A few zero words that padding lanes of the asynchronous global->LDS copies read from.
+__device__ float g_zero_words[4] = {0.f, 0.f, 0.f, 0.f};
+
+// Tile id -> first image, first output row, output-channel block.  XCD-aware: consecutive
+// workgroups sit on different XCDs, so each XCD gets a contiguous run of spatial tiles (halo rows
+// then hit that XCD's own L2).
+__device__ __forceinline__ void decode_tile(const TileGeom &t, int tile, int &n0, int &oh0, int &kb) {
+    kb = tile % t.n_kblocks;
+    int sb = tile / t.n_kblocks;
+    if ((t.n_sblocks & 7) == 0) sb = (sb & 7) * (t.n_sblocks >> 3) + (sb >> 3);
+    const int ig = sb / t.n_row_tiles;
+    n0 = ig * t.NB;
+    oh0 = (sb - ig * t.n_row_tiles) * t.TH;
+}
+
+// One (tile, chunk) step of the pipeline: start the asynchronous global->LDS copies of the NEXT step
+// into `dma` and run the matrix cores over THIS step's operands in `cmp`.
+//
+// The three LDS regions are passed as __restrict__ pointers on purpose: `dma`, `cmp` and `ptab` never
+// overlap within a step, and saying so is what lets the compiler leave the copies in flight across
+// the LDS reads of this step instead of draining them (vmcnt(0)) before the first one.
+template <int MT, int WM, int WN, int KV, int TT>
+__device__ __forceinline__ void conv_step(float *__restrict__ dma, const float *__restrict__ cmp,
+                                          const int2 *__restrict__ ptab, const float *__restrict__ x,
+                                          const float *__restrict__ wp, const ConvGeom &g, const TileGeom &t,
+                                          bool do_issue, int itile, int ichunk, const int (&lds_off)[MT],
+                                          f32x16 (&acc)[MT]) {
     constexpr int NT = WM * WN * 64;
     constexpr int K_BLK = WN * 32;
-    extern __shared__ float lds[];
-    const int T = g.KH * g.KW;
-    float *patch = lds;                 // [CC][P1]
-    float *wl = lds + CC * t.P1;        // [T][CC][K_BLK]
-
+    constexpr int PPI = NT / 4;  // patch positions covered by one staging instruction of the workgroup
+    const int T = TT > 0 ? TT : g.KH * g.KW;
+    const int w_chunk = T * CC * K_BLK;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave % WM, wn = wave / WM;
+    const int wn = wave / WM;
     const int l32 = lane & 31, lh = lane >> 5;
 
-    // XCD-aware order: consecutive workgroup ids go to different XCDs, so give each XCD a
-    // contiguous run of spatial tiles (neighbours share halo rows in that XCD's L2).
-    int sb = blockIdx.x;
-    if ((t.n_sblocks & 7) == 0) sb = (sb & 7) * (t.n_sblocks >> 3) + (sb >> 3);
-    const int kb = blockIdx.y;
-    const int ig = sb / t.n_row_tiles, rt = sb - ig * t.n_row_tiles;
-    const int n0 = ig * t.NB, oh0 = rt * t.TH;
-    const int64_t x_img = int64_t(g.C) * g.H * g.W;
-    const float *xb = x + int64_t(n0) * x_img;
-
-    // ---- per-lane constants: LDS base offset and output offset of each of this wave's tiles ----
-    int lds_off[MT];
-    int64_t out_off[MT];
-    const int rows_here = min(t.TH, g.OH - oh0);
-    const int imgs_here = min(t.NB, g.N - n0);
-    const int per_img = t.TH * g.OW;
-#pragma unroll
-    for (int i = 0; i < MT; ++i) {
-        const int p = (wm * MT + i) * 32 + l32;
-        const int img = p / per_img, rem = p - img * per_img;
-        const int r = rem / g.OW, c = rem - r * g.OW;
-        const bool ok = img < imgs_here && r < rows_here;
-        lds_off[i] = ok ? (img * t.PH + r * g.sh) * t.PW + c * g.sw : 0;
-        out_off[i] = ok ? (int64_t(n0 + img) * g.K * g.OH + (oh0 + r)) * g.OW + c : -1;
-    }
-
-    f32x16 acc[MT];
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[i][v] = 0.0f;
-
-    const int ih0 = oh0 * g.sh - g.pt;
-    const int patch_hw = t.PH * t.PW;
-    const int w_chunk = T * CC * K_BLK;  // floats per (chunk, kblock) slab, a multiple of 4
-
-    for (int chunk = 0; chunk < t.n_chunks; ++chunk) {
-        __syncthreads();  // every wave is done reading the previous chunk
-        // ---- stage the input patch: [cc][img][ph][pw], zero outside the image ----
-        for (int e = tid; e < t.P1; e += NT) {
-            const int img = e / patch_hw, rem = e - img * patch_hw;
-            const int ph = rem / t.PW, pw = rem - ph * t.PW;
-            const int ih = ih0 + ph, iw = pw - g.pl;
-            const bool ok = img < imgs_here && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W;
-            const int64_t goff = int64_t(img) * x_img + int64_t(ih) * g.W + iw;
-#pragma unroll
-            for (int cc = 0; cc < CC; ++cc) {
-                const int c = chunk * CC + cc;
-                float v = 0.0f;
-                if (ok && c < g.C) v = xb[goff + int64_t(c) * g.H * g.W];
-                patch[cc * t.P1 + e] = v;
-            }
+    if (do_issue) {
+        int n0, oh0, kb;
+        decode_tile(t, itile, n0, oh0, kb);
+        float *xl = dma + w_chunk;
+        // weight slab: contiguous 16-byte units, lane-consecutive in LDS
+        const float *wsrc = wp + (int64_t(ichunk) * t.n_kblocks + kb) * w_chunk;
+        const int units = w_chunk >> 2;
+        for (int u0 = 0; u0 < units; u0 += NT) {
+            const int u = u0 + tid;
+            if (u < units)
+                __builtin_amdgcn_global_load_lds((gptr_t)(wsrc + u * 4), (lptr_t)(dma + (u0 + wave * 64) * 4), 16, 0, 0);
         }
-        // ---- stage the weight slab (already in LDS order) ----
-        {
-            const float4 *src = reinterpret_cast<const float4 *>(wp + (int64_t(chunk) * t.n_kblocks + kb) * w_chunk);
-            float4 *dst = reinterpret_cast<float4 *>(wl);
-            for (int e = tid; e < (w_chunk >> 2); e += NT) dst[e] = src[e];
-        }
-        __syncthreads();
-        // ---- MFMA: per tap, 4 k-steps of 2 channels ----
-        const float *wa = wl + lh * K_BLK + wn * 32 + l32;
-        const float *pb = patch + lh * t.P1;
-        for (int kh = 0; kh < g.KH; ++kh) {
-            for (int kw = 0; kw < g.KW; ++kw) {
-                const int tap_off = kh * g.dh * t.PW + kw * g.dw;
-                const float *wt = wa + (kh * g.KW + kw) * CC * K_BLK;
+        // input patch: lane -> (position, channel j of a half); zero words for padding
+        const int64_t x_plane = int64_t(g.H) * g.W;
+        const float *xb = x + int64_t(n0) * g.C * x_plane;
+        const int ih0 = oh0 * g.sh - g.pt;
+        const int imgs_here = min(t.NB, g.N - n0);
+        const int j = tid & 3;
+        for (int p0 = 0; p0 < t.P1; p0 += PPI) {
+            const int pos = p0 + (tid >> 2);
+            if (pos < t.P1) {
+                const int2 e = ptab[pos];
+                const int ih = ih0 + (e.y & 0xffff);
+                const bool ok = e.x >= 0 && ih >= 0 && ih < g.H && (e.y >> 16) < imgs_here;
+                const float *src = xb + (e.x + ih0 * g.W) + int64_t(ichunk * CC + j) * x_plane;
 #pragma unroll
-                for (int cp = 0; cp < CC / 2; ++cp) {
-                    const float a = wt[cp * 2 * K_BLK];
-                    const float *pc = pb + cp * 2 * t.P1 + tap_off;
-                    float b[MT];
-#pragma unroll
-                    for (int i = 0; i < MT; ++i) b[i] = pc[lds_off[i]];
-#pragma unroll
-                    for (int i = 0; i < MT; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b[i], acc[i], 0, 0, 0);
+                for (int half = 0; half < 2; ++half) {
+                    const int c = ichunk * CC + half * 4 + j;
+                    const float *sp = (ok && c < g.C) ? src + half * 4 * x_plane : g_zero_words;
+                    __builtin_amdgcn_global_load_lds((gptr_t)sp, (lptr_t)(xl + (half * t.P1s + p0 + wave * 16) * 4), 4, 0, 0);
                 }
             }
         }
     }
 
-    // ---- epilogue: bias (+ReLU), coalesced NCHW stores ----
-    const int64_t plane = int64_t(g.OH) * g.OW;
-    float bv[16];
-    int kv[16];
+    // keep the copy-issue code and the MFMA loop apart: interleaving them only adds register pressure
+    __builtin_amdgcn_sched_barrier(0);
+
+    typedef float vkv __attribute__((ext_vector_type(KV)));
+    constexpr int SUBS = 4 / KV;  // LDS reads per tap and operand
+    const float *wlf = cmp + (lh * K_BLK + wn * 32 + l32) * 4;
+    const float *xlf = cmp + w_chunk + lh * t.P1s * 4;
+    vkv a0, a1, b0[MT], b1[MT];
+    int lkh = 0, lkw = 0, ltap = 0, lsub = 0;  // what the next load_grp() call fetches
+    auto load_grp = [&](vkv &a, vkv (&b)[MT]) {
+        const int off = (lkh * g.dh * t.PW + lkw * g.dw) * 4 + lsub * KV;
+        a = *reinterpret_cast<const vkv *>(wlf + ltap * 2 * K_BLK * 4 + lsub * KV);
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        kv[v] = kb * K_BLK + wn * 32 + (v >> 2) * 8 + lh * 4 + (v & 3);
-        bv[v] = (bias != nullptr && kv[v] < g.K) ? bias[kv[v]] : 0.0f;
+        for (int i = 0; i < MT; ++i) b[i] = *reinterpret_cast<const vkv *>(xlf + lds_off[i] * 4 + off);
+        if (++lsub == SUBS) {
+            lsub = 0;
+            ++ltap;
+            if (++lkw == g.KW) { lkw = 0; ++lkh; }
+        }
+    };
+    // MFMAs of k-steps [j0, j1) of a group.  Raised priority for the burst: of the two waves sharing a
+    // SIMD, the one that reaches its burst first keeps the matrix core and the other fetches operands
+    // meanwhile, instead of both interleaving bursts and then both stalling together.
+    auto mfma_part = [&](const vkv &a, const vkv (&b)[MT], int j0, int j1) {
+        __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+        for (int j = 0; j < KV; ++j)
+            if (j >= j0 && j < j1) {
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+                    acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j], b[i][j], acc[i], 0, 0, 0);
+            }
+        __builtin_amdgcn_s_setprio(0);
+    };
+    // One group: the next group's operand reads are issued in the middle of this group's MFMAs, so
+    // they have half a burst to land before anything waits on them.
+    auto run_grp = [&](const vkv &a, const vkv (&b)[MT], vkv &an, vkv (&bn)[MT], bool more) {
+        mfma_part(a, b, 0, KV / 2);
+        if (more) load_grp(an, bn);
+        mfma_part(a, b, KV / 2, KV);
+    };
+    if (TT > 0) {
+        constexpr int N_GRP = (TT > 0 ? TT : 1) * SUBS;
+        load_grp(a0, b0);
+#pragma unroll
+        for (int gp = 0; gp < N_GRP; gp += 2) {
+            run_grp(a0, b0, a1, b1, gp + 1 < N_GRP);
+            if (gp + 1 < N_GRP) run_grp(a1, b1, a0, b0, gp + 2 < N_GRP);
+        }
+    } else {
+        const int n_grp = T * SUBS;
+        load_grp(a0, b0);
+        for (int gp = 0; gp < n_grp; gp += 2) {
+            run_grp(a0, b0, a1, b1, gp + 1 < n_grp);
+            if (gp + 1 < n_grp) run_grp(a1, b1, a0, b0, gp + 2 < n_grp);
+        }
     }
+}
+
+// Persistent implicit-GEMM convolution.
+//   MT: 32-position MFMA tiles per wave; WM x WN waves per workgroup (positions x output channels);
+//   KV: k-steps fetched per LDS read (4 = 128-bit reads; 2 = 64-bit reads, fewer registers for MT = 8);
+//   TT: filter taps KH*KW when known at compile time (the tap loop is then fully unrolled, which lets
+//       the compiler count outstanding LDS reads exactly instead of draining them at a loop edge), 0 = any.
+// LDS holds two staging buffers, each [weights: T][2][K_BLK][4] + [patch: 2][P1s][4]: the 8 channels
+// of a chunk are split in two halves (one per MFMA k index) and the 4 channels of a half sit next to
+// each other, so ONE 128-bit LDS read per lane feeds 4 MFMA k-steps.  Global->LDS copies are
+// asynchronous (global_load_lds, no VGPR round trip) and run one (tile, chunk) step ahead of the
+// matrix cores, across tile boundaries as well: while a tile's bias/ReLU epilogue stores drain, the
+// first chunk of the workgroup's next tile is already landing.  Tiles are drawn from an atomic counter.
+template <int MT, int WM, int WN, int KV, int TT>
+__global__ void __launch_bounds__(WM *WN * 64, 2)
+conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, const float *__restrict__ bias,
+                     float *__restrict__ y, ConvGeom g, TileGeom t, int relu, int *__restrict__ tile_counter) {
+    constexpr int NT = WM * WN * 64;
+    constexpr int K_BLK = WN * 32;
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int T = TT > 0 ? TT : g.KH * g.KW;
+    const int w_chunk = T * CC * K_BLK;          // floats per (chunk, kblock) weight slab
+    const int buf_floats = w_chunk + CC * t.P1s;  // one staging buffer
+    float *buf0 = lds, *buf1 = lds + buf_floats;
+    int2 *ptab = reinterpret_cast<int2 *>(lds + 2 * buf_floats);  // [P1]: {offset in image group, img<<16 | ph}
+    int *sched = reinterpret_cast<int *>(ptab + t.P1s);            // [2]: tile ids handed out by thread 0
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave % WM, wn = wave / WM;
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int64_t x_img = int64_t(g.C) * g.H * g.W;
+    const int per_img = t.TH * g.OW;
+    const int patch_hw = t.PH * t.PW;
+
+    // ---- once per workgroup: the tile-independent part of the patch geometry ----
+    for (int e = tid; e < t.P1; e += NT) {
+        const int img = e / patch_hw, rem = e - img * patch_hw;
+        const int ph = rem / t.PW, pw = rem - ph * t.PW;
+        const int iw = pw - g.pl;
+        int2 v;
+        v.x = (iw >= 0 && iw < g.W) ? int(img * x_img) + ph * g.W + iw : -1;  // NB*C*H*W < 2^31 is checked on the host
+        v.y = (img << 16) | ph;
+        ptab[e] = v;
+    }
+    int lds_off[MT];  // float4 index of each of this lane's output positions inside a patch half
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
-        if (out_off[i] < 0) continue;
+        const int p = (wm * MT + i) * 32 + l32;
+        const int img = p / per_img, rem = p - img * per_img;
+        const int r = rem / g.OW, c = rem - r * g.OW;
+        lds_off[i] = (img < t.NB && r < t.TH) ? (img * t.PH + r * g.sh) * t.PW + c * g.sw : 0;
+    }
+    if (tid == 0) sched[0] = blockIdx.x + gridDim.x;  // the second tile is static, later ones come from the counter
+    __syncthreads();
+
+    int cur = blockIdx.x;
+    if (cur >= t.n_tiles) return;
+    f32x16 acc[MT];
+    // prologue: copies of the first step, with nothing to compute yet
+    {
+        int n0, oh0, kb;
+        decode_tile(t, cur, n0, oh0, kb);
+        const float *wsrc = wp + int64_t(kb) * w_chunk;
+        const int units = w_chunk >> 2;
+        for (int u0 = 0; u0 < units; u0 += NT) {
+            const int u = u0 + tid;
+            if (u < units)
+                __builtin_amdgcn_global_load_lds((gptr_t)(wsrc + u * 4), (lptr_t)(buf0 + (u0 + wave * 64) * 4), 16, 0, 0);
+        }
+        const int64_t x_plane = int64_t(g.H) * g.W;
+        const float *xb = x + int64_t(n0) * x_img;
+        const int ih0 = oh0 * g.sh - g.pt;
+        const int imgs_here = min(t.NB, g.N - n0);
+        const int j = tid & 3;
+        float *xl = buf0 + w_chunk;
+        for (int p0 = 0; p0 < t.P1; p0 += NT / 4) {
+            const int pos = p0 + (tid >> 2);
+            if (pos < t.P1) {
+                const int2 e = ptab[pos];
+                const int ih = ih0 + (e.y & 0xffff);
+                const bool ok = e.x >= 0 && ih >= 0 && ih < g.H && (e.y >> 16) < imgs_here;
+                const float *src = xb + (e.x + ih0 * g.W) + int64_t(j) * x_plane;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            if (kv[v] < g.K) {
-                float r = acc[i][v] + bv[v];
-                if (relu) r = r > 0.0f ? r : 0.0f;
-                y[out_off[i] + int64_t(kv[v]) * plane] = r;
+                for (int half = 0; half < 2; ++half) {
+                    const int c = half * 4 + j;
+                    const float *sp = (ok && c < g.C) ? src + half * 4 * x_plane : g_zero_words;
+                    __builtin_amdgcn_global_load_lds((gptr_t)sp, (lptr_t)(xl + (half * t.P1s + p0 + wave * 16) * 4), 4, 0, 0);
+                }
             }
         }
+    }
+    int step = 0;  // flattened (tile, chunk) counter; its parity selects the staging buffer
+    int tile_par = 0;
+    while (cur < t.n_tiles) {
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][v] = 0.0f;
+        int nxt = t.n_tiles;
+        for (int chunk = 0; chunk < t.n_chunks; ++chunk, ++step) {
+            __builtin_amdgcn_s_waitcnt(0);  // this thread's copies for this step have landed
+            __syncthreads();                // ... everyone's have; all waves are done with the other buffer
+            if (chunk == 0) {
+                nxt = sched[tile_par];  // written at least one barrier ago
+                if (tid == 0) sched[tile_par ^ 1] = atomicAdd(tile_counter, 1);
+            }
+            const bool same_tile = chunk + 1 < t.n_chunks;
+            const bool do_issue = same_tile || nxt < t.n_tiles;
+            const int itile = same_tile ? cur : nxt, ichunk = same_tile ? chunk + 1 : 0;
+            float *dma = (step & 1) ? buf0 : buf1;
+            const float *cmp = (step & 1) ? buf1 : buf0;
+            conv_step<MT, WM, WN, KV, TT>(dma, cmp, ptab, x, wp, g, t, do_issue, itile, ichunk, lds_off, acc);
+        }
+
+        // ---- epilogue: bias (+ReLU), coalesced NCHW stores; the next tile's first chunk is in flight ----
+        {
+            int n0, oh0, kb;
+            decode_tile(t, cur, n0, oh0, kb);
+            const int rows_here = min(t.TH, g.OH - oh0);
+            const int imgs_here = min(t.NB, g.N - n0);
+            const int64_t plane = int64_t(g.OH) * g.OW;
+            const int kbase = kb * K_BLK + wn * 32 + lh * 4;
+            const bool full_k = (kb + 1) * K_BLK <= g.K;
+            float bv[16];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int k = kbase + (v >> 2) * 8 + (v & 3);
+                bv[v] = (bias != nullptr && k < g.K) ? bias[k] : 0.0f;
+            }
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+                const int p = (wm * MT + i) * 32 + l32;
+                const int img = p / per_img, rem = p - img * per_img;
+                const int r = rem / g.OW, c = rem - r * g.OW;
+                if (img < imgs_here && r < rows_here) {
+                    float *yp = y + (int64_t(n0 + img) * g.K + kbase) * plane + int64_t(oh0 + r) * g.OW + c;
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int dk = (v >> 2) * 8 + (v & 3);
+                        if (full_k || kbase + dk < g.K) {
+                            float o = acc[i][v] + bv[v];
+                            if (relu) o = o > 0.0f ? o : 0.0f;
+                            yp[dk * plane] = o;
+                        }
+                    }
+                }
+            }
+        }
+        cur = nxt;
+        tile_par ^= 1;
     }
 }
 
@@ -208,7 +379,7 @@ struct MfmaPlan {
 // Picks the tile shape with the best useful-lane fraction whose LDS footprint allows two workgroups per CU.
 bool plan_mfma(const ConvGeom &g, MfmaPlan *best) {
     static const int kMT[] = {8, 7, 6, 5, 4, 3, 2, 1};
-    const size_t lds_cap = 72 * 1024;
+    const size_t lds_cap = 80 * 1024;  // two workgroups per CU within the 160 KB of LDS
     const int T = g.KH * g.KW;
     bool found = false;
     const int WN = g.K > 32 ? 2 : 1, WM = 4 / WN;
@@ -230,11 +401,17 @@ bool plan_mfma(const ConvGeom &g, MfmaPlan *best) {
         t.PH = (t.TH - 1) * g.sh + (g.KH - 1) * g.dh + 1;
         t.PW = (g.OW - 1) * g.sw + (g.KW - 1) * g.dw + 1;
         t.P1 = t.NB * t.PH * t.PW;
+        t.P1s = (t.P1 + 3) & ~3;
+        if (t.PH >= (1 << 16) || t.NB >= (1 << 15)) continue;  // packed into one int of the patch table
+        if (int64_t(t.NB) * g.C * g.H * g.W >= (int64_t(1) << 31)) continue;  // 32-bit offsets inside an image group
         t.n_chunks = (g.C + CC - 1) / CC;
         t.n_kblocks = (g.K + K_BLK - 1) / K_BLK;
         t.n_sblocks = ((g.N + t.NB - 1) / t.NB) * t.n_row_tiles;
-        t.positions = t.NB * t.TH * g.OW;
-        const size_t lds = (size_t(CC) * t.P1 + size_t(T) * CC * K_BLK) * sizeof(float);
+        const int64_t n_tiles = int64_t(t.n_sblocks) * t.n_kblocks;
+        if (n_tiles >= (int64_t(1) << 30)) continue;
+        t.n_tiles = int(n_tiles);
+        const size_t lds = 2 * (size_t(T) * CC * K_BLK + size_t(CC) * t.P1s) * sizeof(float)  // two staging buffers
+                           + size_t(t.P1s) * sizeof(int2) + 2 * sizeof(int);                   // patch table, scheduler slots
         if (lds > lds_cap) continue;
         const double useful = double(g.N) * g.OH * g.OW;
         const double eff = useful / (double(t.n_sblocks) * S);
@@ -246,25 +423,42 @@ bool plan_mfma(const ConvGeom &g, MfmaPlan *best) {
     return found;
 }
 
+template <int MT, int WM, int WN, int TT>
+void launch_mfma_tt(zant_ctx *ctx, const float *x, const float *wp, const float *bias, float *y, const ConvGeom &g,
+                    const MfmaPlan &p, int relu, int *counter, int grid) {
+    constexpr int KV = MT >= 8 ? 2 : 4;  // 64-bit operand reads keep 8 accumulator tiles inside 256 VGPRs
+    // more than 64 KB of dynamic LDS has to be opted into once per kernel
+    static bool attr_set = false;
+    if (!attr_set) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&conv_f32_mfma_kernel<MT, WM, WN, KV, TT>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((conv_f32_mfma_kernel<MT, WM, WN, KV, TT>), dim3(grid), dim3(WM * WN * 64), p.lds_bytes,
+                       ctx->stream, x, wp, bias, y, g, p.t, relu, counter);
+}
+
 template <int MT, int WM, int WN>
 void launch_mfma(zant_ctx *ctx, const float *x, const float *wp, const float *bias, float *y, const ConvGeom &g,
-                 const MfmaPlan &p, int relu) {
-    hipLaunchKernelGGL((conv_f32_mfma_kernel<MT, WM, WN>), dim3(p.t.n_sblocks, p.t.n_kblocks), dim3(WM * WN * 64),
-                       p.lds_bytes, ctx->stream, x, wp, bias, y, g, p.t, relu);
+                 const MfmaPlan &p, int relu, int *counter, int grid) {
+    const int T = g.KH * g.KW;
+    if (T == 9) launch_mfma_tt<MT, WM, WN, 9>(ctx, x, wp, bias, y, g, p, relu, counter, grid);
+    else if (T == 1) launch_mfma_tt<MT, WM, WN, 1>(ctx, x, wp, bias, y, g, p, relu, counter, grid);
+    else launch_mfma_tt<MT, WM, WN, 0>(ctx, x, wp, bias, y, g, p, relu, counter, grid);
 }
 
 template <int WM, int WN>
 bool dispatch_mt(zant_ctx *ctx, const float *x, const float *wp, const float *bias, float *y, const ConvGeom &g,
-                 const MfmaPlan &p, int relu) {
+                 const MfmaPlan &p, int relu, int *counter, int grid) {
     switch (p.MT) {
-    case 1: launch_mfma<1, WM, WN>(ctx, x, wp, bias, y, g, p, relu); return true;
-    case 2: launch_mfma<2, WM, WN>(ctx, x, wp, bias, y, g, p, relu); return true;
-    case 3: launch_mfma<3, WM, WN>(ctx, x, wp, bias, y, g, p, relu); return true;
-    case 4: launch_mfma<4, WM, WN>(ctx, x, wp, bias, y, g, p, relu); return true;
-    case 5: launch_mfma<5, WM, WN>(ctx, x, wp, bias, y, g, p, relu); return true;
-    case 6: launch_mfma<6, WM, WN>(ctx, x, wp, bias, y, g, p, relu); return true;
-    case 7: launch_mfma<7, WM, WN>(ctx, x, wp, bias, y, g, p, relu); return true;
-    case 8: launch_mfma<8, WM, WN>(ctx, x, wp, bias, y, g, p, relu); return true;
+    case 1: launch_mfma<1, WM, WN>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
+    case 2: launch_mfma<2, WM, WN>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
+    case 3: launch_mfma<3, WM, WN>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
+    case 4: launch_mfma<4, WM, WN>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
+    case 5: launch_mfma<5, WM, WN>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
+    case 6: launch_mfma<6, WM, WN>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
+    case 7: launch_mfma<7, WM, WN>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
+    case 8: launch_mfma<8, WM, WN>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
     default: return false;
     }
 }
@@ -379,15 +573,18 @@ extern "C" int zant_hip_conv2d_f32(zant_ctx *ctx, const float *x, const int64_t 
         const int T = g.KH * g.KW, K_BLK = plan.WN * 32;
         const size_t wp_floats = size_t(plan.t.n_chunks) * plan.t.n_kblocks * T * CC * K_BLK;
         void *ws = nullptr;
-        rc = zant_workspace(ctx, wp_floats * sizeof(float), &ws);
+        rc = zant_workspace(ctx, 256 + wp_floats * sizeof(float), &ws);  // [tile counter | packed weights]
         if (rc) return rc;
-        float *wp = static_cast<float *>(ws);
+        int *counter = static_cast<int *>(ws);
+        float *wp = reinterpret_cast<float *>(static_cast<char *>(ws) + 256);
+        // persistent workgroups: two per CU; the first two tiles of each are static, the rest dynamic
+        const int grid = int(std::min<int64_t>(plan.t.n_tiles, int64_t(ctx->num_cus) * 2));
         const unsigned pb = unsigned(std::min<int64_t>(ceil_div64(int64_t(wp_floats), 256), 1024));
         hipLaunchKernelGGL(pack_weights_f32_kernel, dim3(pb), dim3(256), 0, ctx->stream, w, wp, g.K, g.C, T,
-                           plan.t.n_chunks, plan.t.n_kblocks, K_BLK);
+                           plan.t.n_chunks, plan.t.n_kblocks, K_BLK, counter, 2 * grid);
         ZANT_LAUNCH_CHECK(ctx);
-        bool ok = plan.WN == 2 ? dispatch_mt<2, 2>(ctx, x, wp, bias, y, g, plan, relu)
-                               : dispatch_mt<4, 1>(ctx, x, wp, bias, y, g, plan, relu);
+        bool ok = plan.WN == 2 ? dispatch_mt<2, 2>(ctx, x, wp, bias, y, g, plan, relu, counter, grid)
+                               : dispatch_mt<4, 1>(ctx, x, wp, bias, y, g, plan, relu, counter, grid);
         if (ok) {
             ZANT_LAUNCH_CHECK(ctx);
             zant_log("OnnxConvLean4");
