@@ -1,0 +1,210 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X backend for Z-Ant's tensor-math hot path.
+
+Workload (N=1 GPU): the reference's README CNN (Conv32-ReLU-MaxPool-Conv64-ReLU-MaxPool-Flatten-Dense512-ReLU-
+Dense10-Softmax, f32) at batch 4096 -- the configuration the headline metric "batched inferences/sec at batch
+4096" is quoted on.  One step = one forward pass over one resident batch.  Prints ONE JSON line.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-operators]
+
+`value` is inferences/s with inputs resident in HBM; `roofline` is measured live with HIP events around the
+dominant kernel of the pass; `cpu_baseline` times the CPU oracle (a restatement of the reference's algorithm:
+the reference is Zig-only and no Zig toolchain exists here) on the host, one image at a time on one core, which
+is how the reference's generated predict() runs.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_F32_MFMA_TFLOPS = 157.3
+PEAK_I8_MFMA_TOPS = 5030.0
+PEAK_HBM_GBS = 8000.0
+BATCH = 4096
+
+
+def kernel_avg_ms(ctx, fn, iters):
+    """Average duration of the main kernel of `fn` (HIP events recorded by the library around that launch)."""
+    ctx.kernel_timing(True)
+    tot = 0.0
+    for _ in range(iters):
+        fn()
+        tot += ctx.kernel_ms()
+    ctx.kernel_timing(False)
+    return tot / iters
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-operators", action="store_true", help="skip the standalone operator figures (configs 2a, 2b, 3)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build targets ONE MI355X; the forward pass shards by batch with no collectives "
+                 "and no multi-GPU figure is produced. Run with --gpus 1.")
+
+    import numpy as np
+    import torch
+    import __graft_entry__ as ge
+
+    za = ge.load_package()  # raises if libzant_hip.so is not built: there is no fallback path
+    tm = za.tensor_math
+    from zant_amd import networks
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    ctx = tm.context()
+    params = networks.readme_cnn_params(seed=0)
+    net = networks.ReadmeCNN(BATCH, params, dev)
+    g = np.random.default_rng(1)
+    x_host = g.random((BATCH, 1, 28, 28), dtype=np.float32)  # ~U[0,1)
+    x = torch.from_numpy(x_host).to(dev)
+
+    # ---- parity gate on the first images of the batch (the oracle is only the checker) ----
+    out = net.forward(x)
+    torch.cuda.synchronize()
+    from oracle import oracle as zo
+
+    def oracle_forward(img):
+        y = zo.ReLU(zo.Conv(img, params["w1"], params["b1"], [1, 1], None, None, 1, None))
+        y = zo.onnx_maxpool(y, [2, 2], [2, 2], [1, 1], [0, 0, 0, 0])
+        y = zo.ReLU(zo.Conv(y, params["w2"], params["b2"], [1, 1], None, None, 1, None))
+        y = zo.onnx_maxpool(y, [2, 2], [2, 2], [1, 1], [0, 0, 0, 0])
+        y = zo.ReLU(zo.gemm(y.reshape(1, 1, 1, 1600), params["g1"], params["c1"], 1.0, 1.0, False, False))
+        y = zo.gemm(y, params["g2"], params["c2"], 1.0, 1.0, False, False)
+        return zo.softmax(y.reshape(1, 10))
+
+    ref = np.concatenate([oracle_forward(x_host[i:i + 1]) for i in (0, 1, 2, BATCH - 1)])
+    got = out[[0, 1, 2, BATCH - 1]].cpu().numpy()
+    np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-5)
+
+    # ---- timed region: W warm-up steps, then exactly K steps between synchronisations ----
+    for _ in range(args.warmup):
+        net.forward(x)
+    ctx.sync()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ctx.timer_start()
+    for _ in range(args.steps):
+        net.forward(x)
+    ev_ms = ctx.timer_stop()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms_per_step = max(ev_ms, wall_ms) / args.steps  # the host clock includes the final synchronisation
+    value = BATCH / (ms_per_step * 1e-3)
+
+    # ---- per-kernel durations of the pass (HIP events around each main kernel) ----
+    p = net.p
+    flops = networks.readme_cnn_flops_per_inference()
+    flat = net.p2.view(1, 1, BATCH, 1600)
+    kit = max(5, min(args.steps, 20))
+    kernels = {
+        "conv1+relu": (lambda: tm.conv_lean(x, p["w1"], net.a1, p["b1"], [1, 1], None, None, 1, None, "relu"),
+                       "hbm", (x.numel() + net.a1.numel()) * 4),
+        "maxpool1": (lambda: tm.onnx_maxpool_lean(net.a1, net.p1, [2, 2], [2, 2], [1, 1], [0, 0, 0, 0]),
+                     "hbm", (net.a1.numel() + net.p1.numel()) * 4),
+        "conv2+relu": (lambda: tm.conv_lean(net.p1, p["w2"], net.a2, p["b2"], [1, 1], None, None, 1, None, "relu"),
+                       "mfma", flops["conv2"] * BATCH),
+        "maxpool2": (lambda: tm.onnx_maxpool_lean(net.a2, net.p2, [2, 2], [2, 2], [1, 1], [0, 0, 0, 0]),
+                     "hbm", (net.a2.numel() + net.p2.numel()) * 4),
+        "gemm1+relu": (lambda: tm.gemm_lean(flat, p["g1"], p["c1"], 1.0, 1.0, False, False, net.h1, "relu"),
+                       "mfma", flops["gemm1"] * BATCH),
+        "gemm2": (lambda: tm.gemm_lean(net.h1, p["g2"], p["c2"], 1.0, 1.0, False, False, net.h2),
+                  "mfma", flops["gemm2"] * BATCH),
+        "softmax": (lambda: tm.softmax_lean(net.h2.view(BATCH, 10), net.out), "hbm", 2 * BATCH * 10 * 4),
+    }
+    per_kernel = {}
+    for name, (fn, bound, work) in kernels.items():
+        ms = kernel_avg_ms(ctx, fn, kit)
+        if bound == "mfma":
+            ach = work / (ms * 1e-3) / 1e12
+            per_kernel[name] = {"ms": round(ms, 4), "bound": "mfma", "achieved_tflops": round(ach, 2),
+                                "frac": round(ach / PEAK_F32_MFMA_TFLOPS, 4)}
+        else:
+            ach = work / (ms * 1e-3) / 1e9
+            per_kernel[name] = {"ms": round(ms, 4), "bound": "hbm", "achieved_gbs": round(ach, 1),
+                                "frac": round(ach / PEAK_HBM_GBS, 4)}
+    dominant = max(per_kernel, key=lambda k: per_kernel[k]["ms"])
+    dk = per_kernel[dominant]
+    if dk["bound"] == "mfma":
+        roofline = {"kernel": dominant, "bound": "mfma", "achieved": dk["achieved_tflops"], "peak": PEAK_F32_MFMA_TFLOPS,
+                    "unit": "TFLOP/s", "frac": dk["frac"], "traffic": None, "avg_ms": dk["ms"]}
+    else:
+        roofline = {"kernel": dominant, "bound": "hbm", "achieved": dk["achieved_gbs"], "peak": PEAK_HBM_GBS,
+                    "unit": "GB/s", "frac": dk["frac"], "traffic": None, "avg_ms": dk["ms"]}
+
+    # ---- standalone operator figures (the "conv TOPS" half of the metric): configs 2a, 2b, 3 ----
+    operators = None
+    if not args.no_operators:
+        operators = {}
+        torch.manual_seed(0)
+        xa = torch.randn(256, 64, 56, 56, device=dev)
+        wa = torch.randn(64, 64, 3, 3, device=dev) * (2.0 / 576) ** 0.5
+        ba = torch.randn(64, device=dev) * 0.1
+        ya = torch.zeros(256, 64, 56, 56, device=dev)
+        fn = lambda: tm.conv_lean(xa, wa, ya, ba, [1, 1], [1, 1, 1, 1], [1, 1], 1, "NOTSET")
+        fn(); ms = kernel_avg_ms(ctx, fn, kit)
+        fl = 2 * 256 * 64 * 56 * 56 * 64 * 9
+        operators["conv_f32_N256_C64_56x56_K64_3x3"] = {"ms": round(ms, 4), "tflops": round(fl / ms / 1e9, 2),
+                                                        "frac_f32_mfma_peak": round(fl / ms / 1e9 / PEAK_F32_MFMA_TFLOPS, 4)}
+        del xa, ya
+        ga = torch.randn(1, 1, 4096, 1600, device=dev)
+        gb = torch.randn(1, 1, 1600, 512, device=dev) * (2.0 / 1600) ** 0.5
+        gc = torch.randn(1, 1, 1, 512, device=dev) * 0.1
+        gy = torch.zeros(1, 1, 4096, 512, device=dev)
+        fn = lambda: tm.gemm_lean(ga, gb, gc, 1.0, 1.0, False, False, gy)
+        fn(); ms = kernel_avg_ms(ctx, fn, kit)
+        fl = 2 * 4096 * 1600 * 512
+        operators["gemm_f32_4096x1600x512"] = {"ms": round(ms, 4), "tflops": round(fl / ms / 1e9, 2),
+                                               "frac_f32_mfma_peak": round(fl / ms / 1e9 / PEAK_F32_MFMA_TFLOPS, 4)}
+        xq = torch.randint(0, 256, (128, 128, 28, 28), dtype=torch.uint8, device=dev)
+        wq = torch.randint(-127, 128, (128, 128, 3, 3), dtype=torch.int8, device=dev)
+        ws = torch.rand(128, device=dev) * 0.009 + 0.001
+        bq = torch.randint(-1000, 1001, (128,), dtype=torch.int32, device=dev)
+        yq = torch.zeros(128, 128, 28, 28, dtype=torch.uint8, device=dev)
+        fn = lambda: tm.qlinearconv_lean(xq, 0.02, 128, wq, ws, None, 0.05, 128, bq, yq, [1, 1], [1, 1, 1, 1], [1, 1])
+        fn(); ms = kernel_avg_ms(ctx, fn, 3)
+        op = 2 * 128 * 128 * 28 * 28 * 128 * 9
+        operators["qlinearconv_u8i8_N128_C128_28x28_K128_3x3"] = {"ms": round(ms, 4), "tops": round(op / ms / 1e9, 2),
+                                                                  "frac_i8_mfma_peak": round(op / ms / 1e9 / PEAK_I8_MFMA_TOPS, 5)}
+
+    # ---- CPU baseline: the oracle on one host core, one image at a time, over a bounded sample ----
+    cpu = None
+    if not args.no_cpu_baseline:
+        sample = 2048
+        t0 = time.perf_counter()
+        for i in range(sample):
+            oracle_forward(x_host[i:i + 1])
+        dt = time.perf_counter() - t0
+        cpu = {"value": round(sample / dt, 2), "unit": "inferences/s", "cores": 1, "kind": "port",
+               "host_cores": os.cpu_count(),
+               "sample": f"first {sample} images of the batch, batch 1 per call (how the reference's predict() runs), "
+                         f"{dt:.1f} s of CPU time"}
+
+    line = {
+        "metric": "batched inferences/sec + conv TOPS (% of MI355X peak) at batch 4096",
+        "value": round(value, 1), "unit": "inferences/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "config 1: README f32 CNN (Conv32-ReLU-Pool-Conv64-ReLU-Pool-Gemm512-ReLU-Gemm10-Softmax), "
+                               "input 4096x1x28x28 ~U[0,1), He-normal weights, seed 0", "batch": BATCH,
+                   "flop_per_inference": flops["total"],
+                   "tflops": round(flops["total"] * BATCH / (ms_per_step * 1e-3) / 1e12, 2)},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "kernels": per_kernel,
+        "operators": operators,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -91,6 +91,11 @@ int zant_hip_memset(zant_ctx *ctx, void *dst_dev, int byte_value, size_t bytes);
 /* HIP-event stopwatch on the context's stream (what the benchmark times kernels with). */
 int zant_hip_timer_start(zant_ctx *ctx);
 int zant_hip_timer_stop(zant_ctx *ctx, float *elapsed_ms);
+/* Per-kernel timing: while enabled, every operator brackets its MAIN kernel launch (not its small
+ * weight-packing helpers) with HIP events on the context's stream; zant_hip_kernel_ms() waits for
+ * the most recent one and returns its duration.  Off by default (two event records per call). */
+int zant_hip_kernel_timing(zant_ctx *ctx, int enable);
+int zant_hip_kernel_ms(zant_ctx *ctx, float *elapsed_ms);
 
 /* ---- f32 operators ------------------------------------------------------------ */
 

@@ -155,6 +155,9 @@ CONV_CASES = [
     (2, 16, 9, 11, 32, 1, 1, [1, 1], None, None, None),               # 1x1
     (1, 8, 12, 12, 8, 5, 5, [1, 1], None, None, "SAME_LOWER"),        # 5x5 (mnist-8 style)
     (1, 8, 10, 14, 20, 3, 2, [2, 1], [1, 0, 2, 1], [1, 1], "NOTSET"),   # rectangular everything
+    (2, 3, 20, 20, 16, 3, 3, [1, 1], [1, 1, 1, 1], [1, 1], "NOTSET"),   # 3 input channels (few-channel kernel)
+    (2, 3, 17, 17, 16, 3, 3, [2, 2], [1, 1, 1, 1], [1, 1], "NOTSET"),   # ... stride 2 stem
+    (2, 1, 12, 12, 8, 5, 5, [1, 1], None, None, "SAME_UPPER"),        # 1 channel, 5x5 (mnist-8 first layer)
 ]
 
 

@@ -36,6 +36,8 @@ PROTOTYPES = {
     "zant_hip_memset": (i32, [vp, vp, i32, sz]),
     "zant_hip_timer_start": (i32, [vp]),
     "zant_hip_timer_stop": (i32, [vp, C.POINTER(f32)]),
+    "zant_hip_kernel_timing": (i32, [vp, i32]),
+    "zant_hip_kernel_ms": (i32, [vp, C.POINTER(f32)]),
     "zant_hip_conv2d_f32": (i32, [vp, vp, c_i64p, vp, c_i64p, vp, vp, c_i64p, c_i64p, i32, c_i64p, i32, c_i64p, i32,
                                   i64, C.c_char_p, i32]),
     "zant_hip_conv2d_out_shape": (i32, [c_i64p, c_i64p, c_i64p, i32, c_i64p, i32, c_i64p, i32, i64, C.c_char_p, c_i64p]),
@@ -111,6 +113,14 @@ class Context:
     def timer_stop(self):
         ms = f32()
         self.check(lib.zant_hip_timer_stop(self.handle, C.byref(ms)))
+        return ms.value
+
+    def kernel_timing(self, enable):
+        self.check(lib.zant_hip_kernel_timing(self.handle, int(enable)))
+
+    def kernel_ms(self):
+        ms = f32()
+        self.check(lib.zant_hip_kernel_ms(self.handle, C.byref(ms)))
         return ms.value
 
     def close(self):

@@ -20,6 +20,8 @@ struct zant_ctx {
     void *workspace = nullptr;
     size_t workspace_bytes = 0;
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+    hipEvent_t ev_k0 = nullptr, ev_k1 = nullptr;  // bracket the last main kernel when kernel_timing is on
+    bool kernel_timing = false;
     int num_cus = 256;
     std::string last_error;
 };
@@ -40,6 +42,17 @@ int zant_fail_hip(zant_ctx *ctx, hipError_t e, const char *what);
 
 // Checks the launch that was just enqueued.
 #define ZANT_LAUNCH_CHECK(ctx) ZANT_HIP_TRY(ctx, hipGetLastError())
+
+// Brackets the main kernel of an operator with events when per-kernel timing is enabled.
+struct KernelTimer {
+    zant_ctx *ctx;
+    explicit KernelTimer(zant_ctx *c) : ctx(c) {
+        if (ctx->kernel_timing) (void)hipEventRecord(ctx->ev_k0, ctx->stream);
+    }
+    ~KernelTimer() {
+        if (ctx->kernel_timing) (void)hipEventRecord(ctx->ev_k1, ctx->stream);
+    }
+};
 
 // Grows the context's workspace to at least `bytes` (stream-ordered use only).
 int zant_workspace(zant_ctx *ctx, size_t bytes, void **out);

@@ -369,6 +369,44 @@ __global__ void __launch_bounds__(256) conv_f32_direct_kernel(const float *__res
     }
 }
 
+// Few-input-channel convolution (C*KH*KW = CKK small: first layers with 1 or 3 channels).  The
+// implicit-GEMM K is then far below one MFMA tile and the layer is bound by writing its output, so
+// each thread keeps the CKK input taps of one output position in registers and streams all K output
+// channels (weights are wave-uniform: scalar loads); a wave writes 256 contiguous bytes per channel.
+template <int CKK>
+__global__ void __launch_bounds__(256) conv_f32_smallc_kernel(const float *__restrict__ x, const float *__restrict__ w,
+                                                             const float *__restrict__ bias, float *__restrict__ y,
+                                                             ConvGeom g, int relu) {
+    const int64_t plane = int64_t(g.OH) * g.OW;
+    const int64_t total = int64_t(g.N) * plane;
+    const int64_t step = int64_t(gridDim.x) * blockDim.x;
+    const int taps = g.KH * g.KW;
+    for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += step) {
+        const int n = int(i / plane);
+        const int pos = int(i - int64_t(n) * plane);
+        const int oh = pos / g.OW, ow = pos - oh * g.OW;
+        float xin[CKK];
+#pragma unroll
+        for (int e = 0; e < CKK; ++e) {
+            const int c = e / taps, t = e - c * taps;
+            const int kh = t / g.KW, kw = t - kh * g.KW;
+            const int ih = oh * g.sh - g.pt + kh * g.dh, iw = ow * g.sw - g.pl + kw * g.dw;
+            const bool ok = ih >= 0 && ih < g.H && iw >= 0 && iw < g.W;
+            xin[e] = ok ? x[((int64_t(n) * g.C + c) * g.H + ih) * g.W + iw] : 0.0f;
+        }
+        float *yp = y + int64_t(n) * g.K * plane + pos;
+        for (int k = 0; k < g.K; ++k) {
+            const float *wk = w + int64_t(k) * CKK;
+            float acc = 0.0f;
+#pragma unroll
+            for (int e = 0; e < CKK; ++e) acc = __builtin_fmaf(xin[e], wk[e], acc);
+            float r = acc + (bias ? bias[k] : 0.0f);
+            if (relu) r = r > 0.0f ? r : 0.0f;
+            yp[int64_t(k) * plane] = r;
+        }
+    }
+}
+
 struct MfmaPlan {
     int MT, WM, WN;
     TileGeom t;
@@ -583,6 +621,7 @@ extern "C" int zant_hip_conv2d_f32(zant_ctx *ctx, const float *x, const int64_t 
         hipLaunchKernelGGL(pack_weights_f32_kernel, dim3(pb), dim3(256), 0, ctx->stream, w, wp, g.K, g.C, T,
                            plan.t.n_chunks, plan.t.n_kblocks, K_BLK, counter, 2 * grid);
         ZANT_LAUNCH_CHECK(ctx);
+        KernelTimer kt(ctx);
         bool ok = plan.WN == 2 ? dispatch_mt<2, 2>(ctx, x, wp, bias, y, g, plan, relu, counter, grid)
                                : dispatch_mt<4, 1>(ctx, x, wp, bias, y, g, plan, relu, counter, grid);
         if (ok) {
@@ -591,9 +630,22 @@ extern "C" int zant_hip_conv2d_f32(zant_ctx *ctx, const float *x, const int64_t 
             return ZANT_OK;
         }
     }
+    const int ckk = g.C * g.KH * g.KW;
+    if (ckk == 9 || ckk == 25 || ckk == 27) {
+        const int64_t positions = int64_t(g.N) * g.OH * g.OW;
+        const unsigned pb = unsigned(std::min<int64_t>(ceil_div64(positions, 256), int64_t(ctx->num_cus) * 16));
+        KernelTimer kt(ctx);
+        if (ckk == 9) hipLaunchKernelGGL(conv_f32_smallc_kernel<9>, dim3(pb), dim3(256), 0, ctx->stream, x, w, bias, y, g, relu);
+        else if (ckk == 25) hipLaunchKernelGGL(conv_f32_smallc_kernel<25>, dim3(pb), dim3(256), 0, ctx->stream, x, w, bias, y, g, relu);
+        else hipLaunchKernelGGL(conv_f32_smallc_kernel<27>, dim3(pb), dim3(256), 0, ctx->stream, x, w, bias, y, g, relu);
+        ZANT_LAUNCH_CHECK(ctx);
+        zant_log("OnnxConvLean4");
+        return ZANT_OK;
+    }
     const int64_t total = int64_t(g.N) * g.K * g.OH * g.OW;
     int64_t blocks = ceil_div64(total, 256);
     if (blocks > int64_t(ctx->num_cus) * 32) blocks = int64_t(ctx->num_cus) * 32;
+    KernelTimer kt(ctx);
     hipLaunchKernelGGL(conv_f32_direct_kernel, dim3(unsigned(blocks)), dim3(256), 0, ctx->stream, x, w, bias, y, g, relu);
     ZANT_LAUNCH_CHECK(ctx);
     zant_log("OnnxConvLean4");

@@ -46,7 +46,8 @@ extern "C" int zant_hip_ctx_create(zant_ctx **out, int device, void *stream) {
     }
     hipDeviceProp_t prop;
     if (hipGetDeviceProperties(&prop, device) == hipSuccess) ctx->num_cus = prop.multiProcessorCount;
-    if (hipEventCreate(&ctx->ev_start) != hipSuccess || hipEventCreate(&ctx->ev_stop) != hipSuccess) {
+    if (hipEventCreate(&ctx->ev_start) != hipSuccess || hipEventCreate(&ctx->ev_stop) != hipSuccess ||
+        hipEventCreate(&ctx->ev_k0) != hipSuccess || hipEventCreate(&ctx->ev_k1) != hipSuccess) {
         zant_hip_ctx_destroy(ctx);
         return ZANT_HipError;
     }
@@ -62,6 +63,8 @@ extern "C" void zant_hip_ctx_destroy(zant_ctx *ctx) {
     if (ctx->workspace) (void)hipFree(ctx->workspace);
     if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
     if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);
+    if (ctx->ev_k0) (void)hipEventDestroy(ctx->ev_k0);
+    if (ctx->ev_k1) (void)hipEventDestroy(ctx->ev_k1);
     if (ctx->owns_stream && ctx->stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
 }
@@ -179,5 +182,18 @@ extern "C" int zant_hip_timer_stop(zant_ctx *ctx, float *elapsed_ms) {
     ZANT_HIP_TRY(ctx, hipEventRecord(ctx->ev_stop, ctx->stream));
     ZANT_HIP_TRY(ctx, hipEventSynchronize(ctx->ev_stop));
     ZANT_HIP_TRY(ctx, hipEventElapsedTime(elapsed_ms, ctx->ev_start, ctx->ev_stop));
+    return ZANT_OK;
+}
+
+extern "C" int zant_hip_kernel_timing(zant_ctx *ctx, int enable) {
+    if (!ctx) return ZANT_NullPointer;
+    ctx->kernel_timing = enable != 0;
+    return ZANT_OK;
+}
+
+extern "C" int zant_hip_kernel_ms(zant_ctx *ctx, float *elapsed_ms) {
+    if (!ctx || !elapsed_ms) return ZANT_NullPointer;
+    ZANT_HIP_TRY(ctx, hipEventSynchronize(ctx->ev_k1));
+    ZANT_HIP_TRY(ctx, hipEventElapsedTime(elapsed_ms, ctx->ev_k0, ctx->ev_k1));
     return ZANT_OK;
 }

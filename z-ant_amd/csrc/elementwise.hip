@@ -57,9 +57,11 @@ int launch_unary(zant_ctx *ctx, const float *x, float *y, int64_t n, float slope
     if (n <= 0) return ZANT_OK;
     const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
     if (aligned) {
+        KernelTimer kt(ctx);
         hipLaunchKernelGGL(unary_f32_kernel<OP>, dim3(grid_for(n, kThreads * 4, ctx->num_cus)), dim3(kThreads), 0,
                            ctx->stream, x, y, n, slope);
     } else {
+        KernelTimer kt(ctx);
         hipLaunchKernelGGL(unary_f32_unaligned_kernel<OP>, dim3(grid_for(n, kThreads, ctx->num_cus)), dim3(kThreads),
                            0, ctx->stream, x, y, n, slope);
     }
@@ -258,9 +260,11 @@ int launch_maxpool(zant_ctx *ctx, const T *x, const int64_t xdim[4], T *y, const
     if (fast) {
         constexpr int PER = sizeof(T) == 1 ? 8 : 2;
         const int64_t items = g.NC * g.OH * ((g.OW + PER - 1) / PER);
+        KernelTimer kt(ctx);
         hipLaunchKernelGGL((maxpool_2x2s2_kernel<T, PER>), dim3(grid_for(items, kThreads, ctx->num_cus)),
                            dim3(kThreads), 0, ctx->stream, x, y, g);
     } else {
+        KernelTimer kt(ctx);
         hipLaunchKernelGGL(maxpool_generic_kernel<T>, dim3(grid_for(total, kThreads, ctx->num_cus)), dim3(kThreads), 0,
                            ctx->stream, x, y, g);
     }
@@ -285,6 +289,7 @@ extern "C" int zant_hip_softmax_f32(zant_ctx *ctx, const float *x, float *y, int
     if (rows < 0 || cols < 0) return ZANT_InvalidDimensions;
     if (rows == 0 || cols == 0) return ZANT_OK;
     if (!x || !y) return ZANT_NullPointer;
+    KernelTimer kt(ctx);
     hipLaunchKernelGGL(softmax_f32_kernel, dim3(grid_for(rows, kThreads / 64, ctx->num_cus)), dim3(kThreads), 0,
                        ctx->stream, x, y, rows, cols);
     ZANT_LAUNCH_CHECK(ctx);
@@ -302,6 +307,7 @@ extern "C" int zant_hip_add_f32(zant_ctx *ctx, const float *a, const int64_t *ad
         if (asz == 0) return ZANT_OK;
         if (!a || !b || !y) return ZANT_NullPointer;
         const int vec = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
+        KernelTimer kt(ctx);
         hipLaunchKernelGGL(add_same_f32_kernel, dim3(grid_for(asz, kThreads * 4, ctx->num_cus)), dim3(kThreads), 0,
                            ctx->stream, a, b, y, asz, vec);
         ZANT_LAUNCH_CHECK(ctx);
@@ -328,6 +334,7 @@ extern "C" int zant_hip_add_f32(zant_ctx *ctx, const float *a, const int64_t *ad
     if (ydim_out) for (int i = 0; i < g.rank; ++i) ydim_out[i] = g.out_dim[i];
     if (osz == 0) return ZANT_OK;
     if (!a || !b || !y) return ZANT_NullPointer;
+    KernelTimer kt(ctx);
     hipLaunchKernelGGL(add_bcast_f32_kernel, dim3(grid_for(osz, kThreads, ctx->num_cus)), dim3(kThreads), 0, ctx->stream,
                        a, b, y, osz, g);
     ZANT_LAUNCH_CHECK(ctx);
@@ -342,6 +349,7 @@ extern "C" int zant_hip_add_bias_f32(zant_ctx *ctx, float *t, const int64_t *tdi
     if (b_rank != 1) return ZANT_InputTensorsWrongShape;                       // :30-32
     if (bdim[0] != tdim[t_rank - 1]) return ZANT_InputTensorDimensionMismatch;  // :33-36
     if (!t || !bias) return ZANT_NullPointer;
+    KernelTimer kt(ctx);
     hipLaunchKernelGGL(add_bias_f32_kernel, dim3(grid_for(tsz, kThreads, ctx->num_cus)), dim3(kThreads), 0, ctx->stream,
                        t, bias, tsz, bdim[0]);
     ZANT_LAUNCH_CHECK(ctx);

@@ -196,6 +196,7 @@ int run_gemm(zant_ctx *ctx, const float *A, const float *B, const float *C, floa
     g.a_vec = (reinterpret_cast<uintptr_t>(A) & 15) == 0 && (g.lda & 3) == 0;
     g.b_vec = (reinterpret_cast<uintptr_t>(B) & 15) == 0 && (g.ldb & 3) == 0;
     const bool a_kc = !trans_a, b_kc = trans_b;
+    KernelTimer kt(ctx);
     if (N > 32) launch_gemm<2, 2, 2>(ctx, A, B, C, Y, g, a_kc, b_kc);   // 128 x 64 tile
     else launch_gemm<1, 4, 1>(ctx, A, B, C, Y, g, a_kc, b_kc);          // 128 x 32 tile
     ZANT_LAUNCH_CHECK(ctx);

@@ -97,6 +97,7 @@ extern "C" int zant_hip_qlinearconv_u8i8(zant_ctx *ctx, const uint8_t *x, const 
     const int64_t total = int64_t(g.N) * g.K * g.OH * g.OW;
     int64_t blocks = ceil_div64(total, 256);
     if (blocks > int64_t(ctx->num_cus) * 32) blocks = int64_t(ctx->num_cus) * 32;
+    KernelTimer kt(ctx);
     hipLaunchKernelGGL(qconv_direct_kernel, dim3(unsigned(blocks)), dim3(256), 0, ctx->stream, x, w, w_scale, w_zp, bias, y,
                        g, q);
     ZANT_LAUNCH_CHECK(ctx);

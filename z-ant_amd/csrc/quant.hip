@@ -159,6 +159,7 @@ extern "C" int zant_hip_quantize_linear_f32_u8(zant_ctx *ctx, const float *x, co
     if (rc) return rc;
     if (g.n == 0) return ZANT_OK;
     if (!x || !y || !y_scale) return ZANT_NullPointer;
+    KernelTimer kt(ctx);
     hipLaunchKernelGGL(quantize_kernel, dim3(grid_for(g.n, kThreads, ctx->num_cus)), dim3(kThreads), 0, ctx->stream, x,
                        y_scale, y_zp, y, g);
     ZANT_LAUNCH_CHECK(ctx);
@@ -174,6 +175,7 @@ extern "C" int zant_hip_dequantize_linear_u8_f32(zant_ctx *ctx, const uint8_t *x
     if (rc) return rc;
     if (g.n == 0) return ZANT_OK;
     if (!x || !y || !x_scale) return ZANT_NullPointer;
+    KernelTimer kt(ctx);
     hipLaunchKernelGGL(dequantize_kernel, dim3(grid_for(g.n, kThreads, ctx->num_cus)), dim3(kThreads), 0, ctx->stream, x,
                        x_scale, x_zp, y, g);
     ZANT_LAUNCH_CHECK(ctx);
@@ -189,6 +191,7 @@ extern "C" int zant_hip_qlinear_act_u8(zant_ctx *ctx, const uint8_t *x, int64_t 
     QAct qa;
     qa.act = act; qa.alpha = alpha; qa.in_scale = x_scale; qa.in_zp = x_zp; qa.out_scale = y_scale; qa.out_zp = y_zp;
     const int vec = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
+    KernelTimer kt(ctx);
     hipLaunchKernelGGL(qlinear_act_kernel, dim3(grid_for(n, kThreads * 16, ctx->num_cus)), dim3(kThreads), 0, ctx->stream,
                        x, y, n, qa, vec);
     ZANT_LAUNCH_CHECK(ctx);
@@ -203,6 +206,7 @@ extern "C" int zant_hip_qlinear_add_u8(zant_ctx *ctx, const uint8_t *a, float a_
     QAddArgs q;
     q.a_scale = a_scale; q.b_scale = b_scale; q.y_scale = y_scale; q.a_zp = a_zp; q.b_zp = b_zp; q.y_zp = y_zp;
     const int vec = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
+    KernelTimer kt(ctx);
     hipLaunchKernelGGL(qlinear_add_kernel, dim3(grid_for(n, kThreads * 16, ctx->num_cus)), dim3(kThreads), 0, ctx->stream,
                        a, b, y, n, q, vec);
     ZANT_LAUNCH_CHECK(ctx);
@@ -216,6 +220,7 @@ extern "C" int zant_hip_qlinear_global_avgpool_u8(zant_ctx *ctx, const uint8_t *
     if (planes < 0 || hw <= 0 || hw > (1 << 23)) return ZANT_InvalidDimensions;  // i32 sum cannot overflow
     if (planes == 0) return ZANT_OK;
     if (!x || !y) return ZANT_NullPointer;
+    KernelTimer kt(ctx);
     hipLaunchKernelGGL(qgap_kernel, dim3(grid_for(planes, kThreads / 64, ctx->num_cus)), dim3(kThreads), 0, ctx->stream, x,
                        y, planes, int(hw), x_scale, int(x_zp), y_scale, y_zp);
     ZANT_LAUNCH_CHECK(ctx);
