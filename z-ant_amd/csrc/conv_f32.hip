@@ -13,7 +13,7 @@
 // A direct kernel (one thread per output element) covers shapes the tiled kernel does not take.
 #include <algorithm>
 
-#include "common.h"
+#include "conv_tile.h"
 
 namespace {
 
@@ -23,16 +23,6 @@ typedef __attribute__((address_space(3))) void *lptr_t;
 
 constexpr int CC = 8;  // input channels staged per chunk (4 MFMA k-steps per filter tap)
 
-struct TileGeom {
-    int NB, TH;          // images per workgroup tile, output rows per tile
-    int PH, PW, P1;      // staged patch rows / cols, positions per channel (NB*PH*PW)
-    int P1s;             // P1 rounded up to a multiple of 4
-    int n_row_tiles;     // ceil(OH / TH)
-    int n_chunks;        // ceil(C / CC)
-    int n_kblocks;       // ceil(K / K_BLK)
-    int n_sblocks;       // spatial tiles
-    int n_tiles;         // n_sblocks * n_kblocks
-};
 
 // Packs OIHW weights into [chunk][kblock][tap][half][K_BLK][4] (zero padded):
 // element (half, k, j) holds W[k][chunk*8 + half*4 + j][tap].  A chunk's slab is one contiguous
@@ -59,18 +49,6 @@ __global__ void pack_weights_f32_kernel(const float *__restrict__ w, float *__re
 
 // A few zero words that padding lanes of the asynchronous global->LDS copies read from.
 __device__ float g_zero_words[4] = {0.f, 0.f, 0.f, 0.f};
-
-// Tile id -> first image, first output row, output-channel block.  XCD-aware: consecutive
-// workgroups sit on different XCDs, so each XCD gets a contiguous run of spatial tiles (halo rows
-// then hit that XCD's own L2).
-__device__ __forceinline__ void decode_tile(const TileGeom &t, int tile, int &n0, int &oh0, int &kb) {
-    kb = tile % t.n_kblocks;
-    int sb = tile / t.n_kblocks;
-    if ((t.n_sblocks & 7) == 0) sb = (sb & 7) * (t.n_sblocks >> 3) + (sb >> 3);
-    const int ig = sb / t.n_row_tiles;
-    n0 = ig * t.NB;
-    oh0 = (sb - ig * t.n_row_tiles) * t.TH;
-}
 
 // One (tile, chunk) step of the pipeline: start the asynchronous global->LDS copies of the NEXT step
 // into `dma` and run the matrix cores over THIS step's operands in `cmp`.
@@ -407,58 +385,12 @@ __global__ void __launch_bounds__(256) conv_f32_smallc_kernel(const float *__res
     }
 }
 
-struct MfmaPlan {
-    int MT, WM, WN;
-    TileGeom t;
-    size_t lds_bytes;
-    double eff;
-};
+typedef TilePlan MfmaPlan;
 
-// Picks the tile shape with the best useful-lane fraction whose LDS footprint allows two workgroups per CU.
+// Tile shape with the best useful-lane fraction whose LDS footprint allows two workgroups per CU.
 bool plan_mfma(const ConvGeom &g, MfmaPlan *best) {
-    static const int kMT[] = {8, 7, 6, 5, 4, 3, 2, 1};
-    const size_t lds_cap = 80 * 1024;  // two workgroups per CU within the 160 KB of LDS
-    const int T = g.KH * g.KW;
-    bool found = false;
     const int WN = g.K > 32 ? 2 : 1, WM = 4 / WN;
-    const int K_BLK = WN * 32;
-    for (int mt : kMT) {
-        const int S = WM * mt * 32;
-        const int per_img = g.OH * g.OW;
-        TileGeom t;
-        if (per_img <= S) {
-            t.NB = S / per_img; t.TH = g.OH;
-            if (t.NB > g.N) t.NB = g.N;
-        } else {
-            t.NB = 1; t.TH = S / g.OW;
-            if (t.TH < 1) continue;
-        }
-        t.n_row_tiles = (g.OH + t.TH - 1) / t.TH;
-        // even out the rows so the last tile is not nearly empty
-        t.TH = (g.OH + t.n_row_tiles - 1) / t.n_row_tiles;
-        t.PH = (t.TH - 1) * g.sh + (g.KH - 1) * g.dh + 1;
-        t.PW = (g.OW - 1) * g.sw + (g.KW - 1) * g.dw + 1;
-        t.P1 = t.NB * t.PH * t.PW;
-        t.P1s = (t.P1 + 3) & ~3;
-        if (t.PH >= (1 << 16) || t.NB >= (1 << 15)) continue;  // packed into one int of the patch table
-        if (int64_t(t.NB) * g.C * g.H * g.W >= (int64_t(1) << 31)) continue;  // 32-bit offsets inside an image group
-        t.n_chunks = (g.C + CC - 1) / CC;
-        t.n_kblocks = (g.K + K_BLK - 1) / K_BLK;
-        t.n_sblocks = ((g.N + t.NB - 1) / t.NB) * t.n_row_tiles;
-        const int64_t n_tiles = int64_t(t.n_sblocks) * t.n_kblocks;
-        if (n_tiles >= (int64_t(1) << 30)) continue;
-        t.n_tiles = int(n_tiles);
-        const size_t lds = 2 * (size_t(T) * CC * K_BLK + size_t(CC) * t.P1s) * sizeof(float)  // two staging buffers
-                           + size_t(t.P1s) * sizeof(int2) + 2 * sizeof(int);                   // patch table, scheduler slots
-        if (lds > lds_cap) continue;
-        const double useful = double(g.N) * g.OH * g.OW;
-        const double eff = useful / (double(t.n_sblocks) * S);
-        if (!found || eff > best->eff + 1e-9) {
-            best->MT = mt; best->WM = WM; best->WN = WN; best->t = t; best->lds_bytes = lds; best->eff = eff;
-            found = true;
-        }
-    }
-    return found;
+    return zant_plan_conv_tiles(g, WM, WN, 8, CC, sizeof(float), 80 * 1024, best);
 }
 
 template <int MT, int WM, int WN, int TT>

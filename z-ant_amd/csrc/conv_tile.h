@@ -1,0 +1,83 @@
+// Tiling shared by the implicit-GEMM convolution kernels (f32 and int8).
+//
+// A tile is NB whole images x TH whole output rows x all OW columns, for one block of output
+// channels.  Per chunk of input channels a tile stages a patch of P1 = NB*PH*PW input positions.
+// Both kernels use 32 bytes of LDS per patch position and chunk (8 f32 channels or 32 int8 channels)
+// and T*32*K_BLK bytes per weight slab, so one planner serves both.
+#pragma once
+#include "common.h"
+
+struct TileGeom {
+    int NB, TH;          // images per workgroup tile, output rows per tile
+    int PH, PW, P1;      // staged patch rows / cols, positions per chunk (NB*PH*PW)
+    int P1s;             // P1 rounded up to a multiple of 4
+    int n_row_tiles;     // ceil(OH / TH)
+    int n_chunks;        // ceil(C / channels per chunk)
+    int n_kblocks;       // ceil(K / K_BLK)
+    int n_sblocks;       // spatial tiles
+    int n_tiles;         // n_sblocks * n_kblocks
+};
+
+struct TilePlan {
+    int MT, WM, WN;
+    TileGeom t;
+    size_t lds_bytes;
+    double eff;          // useful fraction of the MFMA columns
+};
+
+// Tile id -> first image, first output row, output-channel block.  XCD-aware: consecutive
+// workgroups sit on different XCDs, so each XCD gets a contiguous run of spatial tiles (halo rows
+// then hit that XCD's own L2).
+__device__ __forceinline__ void decode_tile(const TileGeom &t, int tile, int &n0, int &oh0, int &kb) {
+    kb = tile % t.n_kblocks;
+    int sb = tile / t.n_kblocks;
+    if ((t.n_sblocks & 7) == 0) sb = (sb & 7) * (t.n_sblocks >> 3) + (sb >> 3);
+    const int ig = sb / t.n_row_tiles;
+    n0 = ig * t.NB;
+    oh0 = (sb - ig * t.n_row_tiles) * t.TH;
+}
+
+// Best tile shape for WM x WN waves (WN*32 output channels per workgroup) among MT = mt_max..1 whose
+// two staging buffers, patch table and scheduler slots fit in `lds_cap` bytes.
+// chunk_channels: input channels per chunk; elem_bytes: bytes per input element.
+inline bool zant_plan_conv_tiles(const ConvGeom &g, int WM, int WN, int mt_max, int chunk_channels, size_t elem_bytes,
+                                 size_t lds_cap, TilePlan *best) {
+    const int T = g.KH * g.KW;
+    const int K_BLK = WN * 32;
+    bool found = false;
+    for (int mt = mt_max; mt >= 1; --mt) {
+        const int S = WM * mt * 32;
+        const int per_img = g.OH * g.OW;
+        TileGeom t;
+        if (per_img <= S) {
+            t.NB = S / per_img; t.TH = g.OH;
+            if (t.NB > g.N) t.NB = g.N;
+        } else {
+            t.NB = 1; t.TH = S / g.OW;
+            if (t.TH < 1) continue;
+        }
+        t.n_row_tiles = (g.OH + t.TH - 1) / t.TH;
+        t.TH = (g.OH + t.n_row_tiles - 1) / t.n_row_tiles;  // even out the rows over the row tiles
+        t.PH = (t.TH - 1) * g.sh + (g.KH - 1) * g.dh + 1;
+        t.PW = (g.OW - 1) * g.sw + (g.KW - 1) * g.dw + 1;
+        t.P1 = t.NB * t.PH * t.PW;
+        t.P1s = (t.P1 + 3) & ~3;
+        if (t.PH >= (1 << 16) || t.NB >= (1 << 15)) continue;  // packed into one int of the patch table
+        if (int64_t(t.NB) * g.C * g.H * g.W * int64_t(elem_bytes) >= (int64_t(1) << 31)) continue;  // 32-bit offsets per image group
+        t.n_chunks = (g.C + chunk_channels - 1) / chunk_channels;
+        t.n_kblocks = (g.K + K_BLK - 1) / K_BLK;
+        t.n_sblocks = ((g.N + t.NB - 1) / t.NB) * t.n_row_tiles;
+        const int64_t n_tiles = int64_t(t.n_sblocks) * t.n_kblocks;
+        if (n_tiles >= (int64_t(1) << 30)) continue;
+        t.n_tiles = int(n_tiles);
+        const size_t lds = 2 * (size_t(T) * 32 * K_BLK + size_t(32) * t.P1s)  // two staging buffers
+                           + size_t(t.P1s) * 8 + 8;                          // patch table, scheduler slots
+        if (lds > lds_cap) continue;
+        const double eff = double(g.N) * g.OH * g.OW / (double(t.n_sblocks) * S);
+        if (!found || eff > best->eff + 1e-9) {
+            best->MT = mt; best->WM = WM; best->WN = WN; best->t = t; best->lds_bytes = lds; best->eff = eff;
+            found = true;
+        }
+    }
+    return found;
+}

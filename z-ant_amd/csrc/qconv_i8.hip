@@ -2,6 +2,18 @@
 // no quantised or grouped convolution).  Accumulation is exact integer arithmetic; the epilogue is the
 // single f32 requantisation sequence shared with the CPU checker, optionally followed by the fused
 // Dequantize -> activation -> Quantize step.
+//
+// Dense (group = 1) layers with >= 16 input channels run as an implicit GEMM on the int8 matrix cores
+// (v_mfma_i32_32x32x32_i8).  The MFMA wants 16 consecutive input channels per lane, which NCHW does
+// not have, so a first pass rewrites the activations once into a channel-blocked signed layout
+// [N][C/16][H][W][16] (u8 ^ 0x80 = value - 128); one 16-byte global->LDS copy then moves the 16
+// channels of a position, and one 128-bit LDS read is one MFMA operand.  The u8 zero point is folded
+// into a per-channel integer correction: sum (x - x_zp) w = sum (x - 128) w + (128 - x_zp) sum w,
+// with padding positions holding x_zp so that they contribute exactly 0.  Tiling, the asynchronous
+// double-buffered staging and the persistent tile loop are those of the f32 kernel.
+#include <algorithm>
+
+#include "conv_tile.h"
 #include "quant_common.h"
 
 namespace {
@@ -56,6 +68,394 @@ qconv_direct_kernel(const uint8_t *__restrict__ x, const int8_t *__restrict__ w,
     }
 }
 
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(1))) const void *gptr_t;
+typedef __attribute__((address_space(3))) void *lptr_t;
+
+constexpr int QCC = 32;  // input channels per chunk = one MFMA k-step per filter tap
+
+// NCHW u8 -> [N][CB][H][W][16] signed (value - 128); channels beyond C are 0 (their weights are 0 too).
+__global__ void __launch_bounds__(256) to_blocked_s8_kernel(const uint8_t *__restrict__ x, uint4 *__restrict__ xb, int N,
+                                                           int C, int CB, int64_t HW) {
+    const int64_t total = int64_t(N) * CB * HW;
+    const int64_t step = int64_t(gridDim.x) * blockDim.x;
+    for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += step) {
+        const int64_t hw = i % HW;
+        const int cb = int((i / HW) % CB);
+        const int64_t n = i / (HW * CB);
+        const uint8_t *src = x + (n * C + int64_t(cb) * 16) * HW + hw;
+        uint32_t w[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            uint32_t v = 0;
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                const int c = cb * 16 + q * 4 + b;
+                const uint32_t byte = c < C ? uint32_t(src[int64_t(q * 4 + b) * HW] ^ 0x80u) : 0u;
+                v |= byte << (8 * b);
+            }
+            w[q] = v;
+        }
+        xb[i] = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+}
+
+// Packs OIHW int8 weights into [chunk][kblock][tap][half][K_BLK][16] (zero padded), and writes the
+// per-channel requantisation multiplier, the integer correction (bias + (128 - x_zp) * sum w), the
+// 16-byte padding vector (x_zp - 128 in every lane) and the tile counter.
+__global__ void __launch_bounds__(256)
+qpack_kernel(const int8_t *__restrict__ w, const float *__restrict__ w_scale, const int32_t *__restrict__ bias,
+             int8_t *__restrict__ wp, float *__restrict__ mult, int32_t *__restrict__ corr, int8_t *__restrict__ padvec,
+             int *__restrict__ tile_counter, int counter_init, int K, int C, int T, int n_chunks, int n_kblocks, int k_blk,
+             float x_scale, float y_scale, int x_zp, int n_wscale) {
+    const int64_t total = int64_t(n_chunks) * n_kblocks * T * QCC * k_blk;
+    const int64_t step = int64_t(gridDim.x) * blockDim.x;
+    const int64_t gid = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (gid == 0) *tile_counter = counter_init;
+    if (gid < 16) padvec[gid] = int8_t(x_zp - 128);
+    for (int64_t i = gid; i < total; i += step) {
+        int64_t r = i;
+        const int j = int(r & 15); r >>= 4;
+        const int kk = int(r % k_blk); r /= k_blk;
+        const int half = int(r & 1); r >>= 1;
+        const int tap = int(r % T); r /= T;
+        const int kb = int(r % n_kblocks); r /= n_kblocks;
+        const int chunk = int(r);
+        const int k = kb * k_blk + kk, c = chunk * QCC + half * 16 + j;
+        wp[i] = (k < K && c < C) ? w[(int64_t(k) * C + c) * T + tap] : int8_t(0);
+    }
+    const int kpad = n_kblocks * k_blk;
+    for (int64_t k = gid; k < kpad; k += step) {
+        if (k < K) {
+            int sum = 0;
+            for (int e = 0; e < C * T; ++e) sum += int(w[k * C * T + e]);
+            corr[k] = (bias ? bias[k] : 0) + (128 - x_zp) * sum;
+            mult[k] = (x_scale * w_scale[n_wscale == 1 ? 0 : k]) / y_scale;
+        } else {
+            corr[k] = 0;
+            mult[k] = 0.0f;
+        }
+    }
+}
+
+// One (tile, chunk) step: start the global->LDS copies of the next step into `dma`, run the int8
+// matrix cores over this step's operands in `cmp`.  The LDS regions never overlap within a step and
+// are __restrict__ so that the copies stay in flight across this step's LDS reads.
+template <int MT, int WM, int WN, int TT>
+__device__ __forceinline__ void qconv_step(char *__restrict__ dma, const char *__restrict__ cmp,
+                                           const int2 *__restrict__ ptab, const int8_t *__restrict__ xb,
+                                           const int8_t *__restrict__ wp, const int8_t *__restrict__ padvec,
+                                           const ConvGeom &g, const TileGeom &t, int CB, bool do_issue, int itile,
+                                           int ichunk, const int (&lds_off)[MT], i32x16 (&acc)[MT]) {
+    constexpr int NT = WM * WN * 64;
+    constexpr int K_BLK = WN * 32;
+    const int T = TT > 0 ? TT : g.KH * g.KW;
+    const int w_chunk = T * QCC * K_BLK;  // bytes
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wn = wave / WM;
+    const int l32 = lane & 31, lh = lane >> 5;
+
+    if (do_issue) {
+        int n0, oh0, kb;
+        decode_tile(t, itile, n0, oh0, kb);
+        char *xl = dma + w_chunk;
+        const int8_t *wsrc = wp + (int64_t(ichunk) * t.n_kblocks + kb) * w_chunk;
+        const int units = w_chunk >> 4;
+        for (int u0 = 0; u0 < units; u0 += NT) {
+            const int u = u0 + tid;
+            if (u < units)
+                __builtin_amdgcn_global_load_lds((gptr_t)(wsrc + u * 16), (lptr_t)(dma + (u0 + wave * 64) * 16), 16, 0, 0);
+        }
+        const int64_t plane = int64_t(g.H) * g.W;
+        const int8_t *xg = xb + int64_t(n0) * CB * plane * 16;
+        const int ih0 = oh0 * g.sh - g.pt;
+        const int imgs_here = min(t.NB, g.N - n0);
+        for (int p0 = 0; p0 < t.P1; p0 += NT) {
+            const int pos = p0 + tid;
+            if (pos < t.P1) {
+                const int2 e = ptab[pos];
+                const int ih = ih0 + (e.y & 0xffff);
+                const bool ok = e.x >= 0 && ih >= 0 && ih < g.H && (e.y >> 16) < imgs_here;
+                const int8_t *src = xg + (int64_t(e.x + ih0 * g.W) + int64_t(ichunk * 2) * plane) * 16;
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    const int8_t *sp = (ok && ichunk * 2 + half < CB) ? src + half * plane * 16 : padvec;
+                    __builtin_amdgcn_global_load_lds((gptr_t)sp, (lptr_t)(xl + (half * t.P1s + p0 + wave * 64) * 16), 16, 0, 0);
+                }
+            }
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    const char *wl = cmp + (lh * K_BLK + wn * 32 + l32) * 16;
+    const char *xl = cmp + w_chunk + lh * t.P1s * 16;
+    i32x4 a0, a1, b0[MT], b1[MT];
+    int lkh = 0, lkw = 0, ltap = 0;
+    auto load_tap = [&](i32x4 &a, i32x4 (&b)[MT]) {
+        const int off = (lkh * g.dh * t.PW + lkw * g.dw) * 16;
+        a = *reinterpret_cast<const i32x4 *>(wl + ltap * 2 * K_BLK * 16);
+#pragma unroll
+        for (int i = 0; i < MT; ++i) b[i] = *reinterpret_cast<const i32x4 *>(xl + lds_off[i] * 16 + off);
+        ++ltap;
+        if (++lkw == g.KW) { lkw = 0; ++lkh; }
+    };
+    auto mfma_tap = [&](const i32x4 &a, const i32x4 (&b)[MT]) {
+        __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+        for (int i = 0; i < MT; ++i) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b[i], acc[i], 0, 0, 0);
+        __builtin_amdgcn_s_setprio(0);
+    };
+    if (TT > 0) {
+        constexpr int NTAP = TT > 0 ? TT : 1;
+        load_tap(a0, b0);
+#pragma unroll
+        for (int tp = 0; tp < NTAP; tp += 2) {
+            if (tp + 1 < NTAP) load_tap(a1, b1);
+            mfma_tap(a0, b0);
+            if (tp + 1 < NTAP) {
+                if (tp + 2 < NTAP) load_tap(a0, b0);
+                mfma_tap(a1, b1);
+            }
+        }
+    } else {
+        load_tap(a0, b0);
+        for (int tp = 0; tp < T; tp += 2) {
+            if (tp + 1 < T) load_tap(a1, b1);
+            mfma_tap(a0, b0);
+            if (tp + 1 < T) {
+                if (tp + 2 < T) load_tap(a0, b0);
+                mfma_tap(a1, b1);
+            }
+        }
+    }
+}
+
+// Persistent int8 implicit-GEMM convolution over the channel-blocked input.
+template <int MT, int WM, int WN, int TT>
+__global__ void __launch_bounds__(WM *WN * 64, 2)
+qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, const float *__restrict__ mult,
+                  const int32_t *__restrict__ corr, const int8_t *__restrict__ padvec, uint8_t *__restrict__ y, ConvGeom g,
+                  TileGeom t, int CB, QConvArgs q, int *__restrict__ tile_counter) {
+    constexpr int NT = WM * WN * 64;
+    constexpr int K_BLK = WN * 32;
+    extern __shared__ __attribute__((aligned(16))) char qlds[];
+    const int T = TT > 0 ? TT : g.KH * g.KW;
+    const int w_chunk = T * QCC * K_BLK;          // bytes per (chunk, kblock) weight slab
+    const int buf_bytes = w_chunk + QCC * t.P1s;  // one staging buffer
+    char *buf0 = qlds, *buf1 = qlds + buf_bytes;
+    int2 *ptab = reinterpret_cast<int2 *>(qlds + 2 * buf_bytes);
+    int *sched = reinterpret_cast<int *>(ptab + t.P1s);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave % WM, wn = wave / WM;
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int64_t plane_in = int64_t(g.H) * g.W;
+    const int per_img = t.TH * g.OW;
+    const int patch_hw = t.PH * t.PW;
+
+    for (int e = tid; e < t.P1; e += NT) {
+        const int img = e / patch_hw, rem = e - img * patch_hw;
+        const int ph = rem / t.PW, pw = rem - ph * t.PW;
+        const int iw = pw - g.pl;
+        int2 v;
+        v.x = (iw >= 0 && iw < g.W) ? int(img * CB * plane_in) + ph * g.W + iw : -1;
+        v.y = (img << 16) | ph;
+        ptab[e] = v;
+    }
+    int lds_off[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        const int p = (wm * MT + i) * 32 + l32;
+        const int img = p / per_img, rem = p - img * per_img;
+        const int r = rem / g.OW, c = rem - r * g.OW;
+        lds_off[i] = (img < t.NB && r < t.TH) ? (img * t.PH + r * g.sh) * t.PW + c * g.sw : 0;
+    }
+    if (tid == 0) sched[0] = blockIdx.x + gridDim.x;
+    __syncthreads();
+
+    int cur = blockIdx.x;
+    if (cur >= t.n_tiles) return;
+    i32x16 acc[MT];
+    // prologue: the first step's copies go through the same code path with nothing to compute
+    // (an all-zero pass over whatever the LDS holds into accumulators that are reset right after).
+    {
+        // issue only: replicate the copy part of qconv_step for (cur, chunk 0) into buf0
+        int n0, oh0, kb;
+        decode_tile(t, cur, n0, oh0, kb);
+        const int8_t *wsrc = wp + int64_t(kb) * w_chunk;
+        const int units = w_chunk >> 4;
+        for (int u0 = 0; u0 < units; u0 += NT) {
+            const int u = u0 + tid;
+            if (u < units)
+                __builtin_amdgcn_global_load_lds((gptr_t)(wsrc + u * 16), (lptr_t)(buf0 + (u0 + wave * 64) * 16), 16, 0, 0);
+        }
+        const int8_t *xg = xb + int64_t(n0) * CB * plane_in * 16;
+        const int ih0 = oh0 * g.sh - g.pt;
+        const int imgs_here = min(t.NB, g.N - n0);
+        char *xl = buf0 + w_chunk;
+        for (int p0 = 0; p0 < t.P1; p0 += NT) {
+            const int pos = p0 + tid;
+            if (pos < t.P1) {
+                const int2 e = ptab[pos];
+                const int ih = ih0 + (e.y & 0xffff);
+                const bool ok = e.x >= 0 && ih >= 0 && ih < g.H && (e.y >> 16) < imgs_here;
+                const int8_t *src = xg + int64_t(e.x + ih0 * g.W) * 16;
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    const int8_t *sp = (ok && half < CB) ? src + half * plane_in * 16 : padvec;
+                    __builtin_amdgcn_global_load_lds((gptr_t)sp, (lptr_t)(xl + (half * t.P1s + p0 + wave * 64) * 16), 16, 0, 0);
+                }
+            }
+        }
+    }
+    int step = 0, tile_par = 0;
+    while (cur < t.n_tiles) {
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][v] = 0;
+        int nxt = t.n_tiles;
+        for (int chunk = 0; chunk < t.n_chunks; ++chunk, ++step) {
+            __builtin_amdgcn_s_waitcnt(0);
+            __syncthreads();
+            if (chunk == 0) {
+                nxt = sched[tile_par];
+                if (tid == 0) sched[tile_par ^ 1] = atomicAdd(tile_counter, 1);
+            }
+            const bool same_tile = chunk + 1 < t.n_chunks;
+            const bool do_issue = same_tile || nxt < t.n_tiles;
+            const int itile = same_tile ? cur : nxt, ichunk = same_tile ? chunk + 1 : 0;
+            char *dma = (step & 1) ? buf0 : buf1;
+            const char *cmp = (step & 1) ? buf1 : buf0;
+            qconv_step<MT, WM, WN, TT>(dma, cmp, ptab, xb, wp, padvec, g, t, CB, do_issue, itile, ichunk, lds_off, acc);
+        }
+
+        // ---- epilogue: integer correction, requantisation (+ fused activation), NCHW u8 stores ----
+        {
+            int n0, oh0, kb;
+            decode_tile(t, cur, n0, oh0, kb);
+            const int rows_here = min(t.TH, g.OH - oh0);
+            const int imgs_here = min(t.NB, g.N - n0);
+            const int64_t plane = int64_t(g.OH) * g.OW;
+            const int kbase = kb * K_BLK + wn * 32 + lh * 4;
+            float mv[16];
+            int cv[16];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int k = kbase + (v >> 2) * 8 + (v & 3);  // < n_kblocks * K_BLK: the tables are padded
+                mv[v] = mult[k];
+                cv[v] = corr[k];
+            }
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+                const int p = (wm * MT + i) * 32 + l32;
+                const int img = p / per_img, rem = p - img * per_img;
+                const int r = rem / g.OW, c = rem - r * g.OW;
+                if (img < imgs_here && r < rows_here) {
+                    uint8_t *yp = y + (int64_t(n0 + img) * g.K + kbase) * plane + int64_t(oh0 + r) * g.OW + c;
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int dk = (v >> 2) * 8 + (v & 3);
+                        if (kbase + dk < g.K) yp[dk * plane] = requant(acc[i][v] + cv[v], mv[v], q);
+                    }
+                }
+            }
+        }
+        cur = nxt;
+        tile_par ^= 1;
+    }
+}
+
+template <int MT, int WM, int WN, int TT>
+void launch_qmfma_tt(zant_ctx *ctx, const int8_t *xb, const int8_t *wp, const float *mult, const int32_t *corr,
+                     const int8_t *padvec, uint8_t *y, const ConvGeom &g, const TilePlan &p, int CB, const QConvArgs &q,
+                     int *counter, int grid) {
+    static bool attr_set = false;
+    if (!attr_set) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&qconv_mfma_kernel<MT, WM, WN, TT>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((qconv_mfma_kernel<MT, WM, WN, TT>), dim3(grid), dim3(WM * WN * 64), p.lds_bytes, ctx->stream, xb,
+                       wp, mult, corr, padvec, y, g, p.t, CB, q, counter);
+}
+
+template <int MT, int WM, int WN>
+void launch_qmfma(zant_ctx *ctx, const int8_t *xb, const int8_t *wp, const float *mult, const int32_t *corr,
+                  const int8_t *padvec, uint8_t *y, const ConvGeom &g, const TilePlan &p, int CB, const QConvArgs &q,
+                  int *counter, int grid) {
+    const int T = g.KH * g.KW;
+    if (T == 9) launch_qmfma_tt<MT, WM, WN, 9>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid);
+    else if (T == 1) launch_qmfma_tt<MT, WM, WN, 1>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid);
+    else launch_qmfma_tt<MT, WM, WN, 0>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid);
+}
+
+template <int WM, int WN>
+bool dispatch_qmt(zant_ctx *ctx, const int8_t *xb, const int8_t *wp, const float *mult, const int32_t *corr,
+                  const int8_t *padvec, uint8_t *y, const ConvGeom &g, const TilePlan &p, int CB, const QConvArgs &q,
+                  int *counter, int grid) {
+    switch (p.MT) {
+    case 1: launch_qmfma<1, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid); return true;
+    case 2: launch_qmfma<2, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid); return true;
+    case 3: launch_qmfma<3, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid); return true;
+    case 4: launch_qmfma<4, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid); return true;
+    case 5: launch_qmfma<5, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid); return true;
+    case 6: launch_qmfma<6, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid); return true;
+    case 7: launch_qmfma<7, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid); return true;
+    default: return false;
+    }
+}
+
+static size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
+
+// The matrix-core path; returns ZANT_OK when it ran, 1 when the shape is left to the direct kernel.
+int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float *w_scale, const int32_t *bias, uint8_t *y,
+                   const ConvGeom &g, const QConvArgs &q) {
+    if (g.groups != 1 || g.C < 16 || int64_t(g.N) * g.OH * g.OW < 64) return 1;
+    const int CB = (g.C + 15) / 16;
+    if (int64_t(g.N) * CB * g.H * g.W >= (int64_t(1) << 27)) return 1;  // 16-byte units addressed with 32-bit offsets
+    TilePlan plan;
+    const int WN = g.K > 32 ? 2 : 1, WM = 4 / WN;
+    ConvGeom gp = g;
+    gp.C = CB;  // the planner's 32-bit offset check works in 16-byte units here
+    if (!zant_plan_conv_tiles(gp, WM, WN, 7, 2, 16, 80 * 1024, &plan) || plan.eff < 0.4) return 1;
+    const int T = g.KH * g.KW, K_BLK = WN * 32;
+    plan.t.n_chunks = (g.C + QCC - 1) / QCC;
+    const size_t wp_bytes = size_t(plan.t.n_chunks) * plan.t.n_kblocks * T * QCC * K_BLK;
+    const size_t kpad = size_t(plan.t.n_kblocks) * K_BLK;
+    const size_t xb_bytes = size_t(g.N) * CB * g.H * g.W * 16;
+    const size_t o_pad = 256, o_mult = 512, o_corr = o_mult + align256(kpad * 4), o_wp = o_corr + align256(kpad * 4),
+                 o_xb = o_wp + align256(wp_bytes), total = o_xb + xb_bytes;
+    void *ws = nullptr;
+    int rc = zant_workspace(ctx, total, &ws);
+    if (rc) return rc;
+    char *base = static_cast<char *>(ws);
+    int *counter = reinterpret_cast<int *>(base);
+    int8_t *padvec = reinterpret_cast<int8_t *>(base + o_pad);
+    float *mult = reinterpret_cast<float *>(base + o_mult);
+    int32_t *corr = reinterpret_cast<int32_t *>(base + o_corr);
+    int8_t *wp = reinterpret_cast<int8_t *>(base + o_wp);
+    int8_t *xb = reinterpret_cast<int8_t *>(base + o_xb);
+    const int grid = int(std::min<int64_t>(plan.t.n_tiles, int64_t(ctx->num_cus) * 2));
+    const unsigned pb = unsigned(std::min<int64_t>(ceil_div64(int64_t(wp_bytes), 256), 1024));
+    hipLaunchKernelGGL(qpack_kernel, dim3(pb), dim3(256), 0, ctx->stream, w, w_scale, bias, wp, mult, corr, padvec, counter,
+                       2 * grid, g.K, g.C, T, plan.t.n_chunks, plan.t.n_kblocks, K_BLK, q.x_scale, q.y_scale, q.x_zp,
+                       q.n_wscale);
+    ZANT_LAUNCH_CHECK(ctx);
+    const int64_t units = int64_t(g.N) * CB * g.H * g.W;
+    const unsigned tb = unsigned(std::min<int64_t>(ceil_div64(units, 256), int64_t(ctx->num_cus) * 16));
+    hipLaunchKernelGGL(to_blocked_s8_kernel, dim3(tb), dim3(256), 0, ctx->stream, x, reinterpret_cast<uint4 *>(xb), g.N, g.C,
+                       CB, int64_t(g.H) * g.W);
+    ZANT_LAUNCH_CHECK(ctx);
+    KernelTimer kt(ctx);
+    const bool ok = WN == 2 ? dispatch_qmt<2, 2>(ctx, xb, wp, mult, corr, padvec, y, g, plan, CB, q, counter, grid)
+                            : dispatch_qmt<4, 1>(ctx, xb, wp, mult, corr, padvec, y, g, plan, CB, q, counter, grid);
+    if (!ok) return 1;
+    ZANT_LAUNCH_CHECK(ctx);
+    return ZANT_OK;
+}
+
 }  // namespace
 
 extern "C" int zant_hip_qlinearconv_u8i8(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], float x_scale,
@@ -94,6 +494,10 @@ extern "C" int zant_hip_qlinearconv_u8i8(zant_ctx *ctx, const uint8_t *x, const 
     q.act.act = act; q.act.alpha = act_alpha; q.act.in_scale = y_scale; q.act.in_zp = y_zp;
     q.act.out_scale = act_scale; q.act.out_zp = act_zp;
 
+    if (w_zp == nullptr) {  // a non-zero weight zero point makes the correction position dependent: direct kernel
+        const int rc = run_qconv_mfma(ctx, x, w, w_scale, bias, y, g, q);
+        if (rc <= 0) return rc;
+    }
     const int64_t total = int64_t(g.N) * g.K * g.OH * g.OW;
     int64_t blocks = ceil_div64(total, 256);
     if (blocks > int64_t(ctx->num_cus) * 32) blocks = int64_t(ctx->num_cus) * 32;
