@@ -198,6 +198,72 @@ int zant_hip_maxpool2d_u8(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4]
 int zant_hip_qlinear_global_avgpool_u8(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], float x_scale,
                                        uint8_t x_zp, float y_scale, uint8_t y_zp, uint8_t *y);
 
+/* ---- generated-library level: a whole network in one preallocated arena -------- */
+
+/* The reference's code generator emits one static array per node output, a
+ * straight-line predict() that calls one *_lean operator per ONNX node, and a
+ * compiled-in input shape (src/codeGen/predict.zig:23-70, 265-377).  A zant_model
+ * is the GPU form of such a generated library: nodes are appended in ready order
+ * (src/codeGen/utils.zig:114-135), parameters are copied to the device once, and
+ * zant_model_finalize() fuses activations into their producers, turns Reshape
+ * into a view and assigns every activation an offset in ONE arena allocation by
+ * liveness, so that zant_model_run() performs no device allocation at all.
+ * Tensor handles are small non-negative ints; a negative return is a zant_status. */
+enum zant_dtype { ZANT_F32 = 0, ZANT_U8 = 1 };
+
+int zant_model_create(zant_ctx *ctx, zant_model **out);
+void zant_model_destroy(zant_model *m);
+/* The network input (batch compiled in, like the reference).  scale / zp describe a u8 input. */
+int zant_model_input(zant_model *m, int dtype, const int64_t *dims, int rank, float scale, int zp);
+/* f32 nodes; w / bias / b / c are HOST pointers copied at finalize. */
+int zant_model_conv(zant_model *m, int x, const float *w, const int64_t wdim[4], const float *bias,
+                    const int64_t *stride, int n_stride, const int64_t *pads, int n_pads, const int64_t *dil,
+                    int n_dil, int64_t group, const char *auto_pad);
+int zant_model_relu(zant_model *m, int x);
+int zant_model_leaky_relu(zant_model *m, int x, float slope);
+int zant_model_maxpool(zant_model *m, int x, const int64_t kernel[2], const int64_t strides[2],
+                       const int64_t dil[2], const int64_t pads[4], int auto_pad, int ceil_mode);
+int zant_model_reshape(zant_model *m, int x, const int64_t *new_shape, int rank);
+int zant_model_gemm(zant_model *m, int a, const float *b, const int64_t bdim[4], const float *c,
+                    const int64_t *cdim, int c_rank, float alpha, float beta, int trans_a, int trans_b);
+int zant_model_matmul(zant_model *m, int a, const float *b, const int64_t *bdim, int b_rank);
+int zant_model_add_const(zant_model *m, int x, const float *c, const int64_t *cdim, int c_rank);
+int zant_model_add(zant_model *m, int a, int b);
+int zant_model_softmax(zant_model *m, int x);
+/* int8 nodes; activation scales / zero points are tracked per tensor. */
+int zant_model_quantize(zant_model *m, int x, float y_scale, int y_zp);
+int zant_model_dequantize(zant_model *m, int x);
+int zant_model_qlinearconv(zant_model *m, int x, const int8_t *w, const int64_t wdim[4], const float *w_scale,
+                           int64_t n_wscale, const int32_t *bias, float y_scale, int y_zp,
+                           const int64_t stride[2], const int64_t pads[4], const int64_t dil[2], int64_t group);
+int zant_model_qlinear_act(zant_model *m, int x, int act, float alpha, float y_scale, int y_zp);
+int zant_model_qlinear_add(zant_model *m, int a, int b, float y_scale, int y_zp);
+int zant_model_qlinear_global_avgpool(zant_model *m, int x, float y_scale, int y_zp);
+/* Fuses, plans the arena (reserved on the context), uploads parameters.  The last node's output is
+ * the network output. */
+int zant_model_finalize(zant_model *m);
+int zant_model_output_dims(zant_model *m, int64_t *dims, int *rank, int *dtype);
+size_t zant_model_arena_bytes(zant_model *m);   /* planned arena size */
+size_t zant_model_unfused_bytes(zant_model *m); /* sum of all node outputs, the reference's static arrays */
+int zant_model_num_launches(zant_model *m);     /* operator calls per run after fusion */
+/* One forward pass, device in / device out, asynchronous, no allocation.  input_dev == NULL means the
+ * caller already wrote the input at zant_model_input_ptr(); output_dev == NULL leaves the result at
+ * zant_model_output_ptr() (both inside the arena, valid after finalize). */
+int zant_model_run(zant_model *m, const void *input_dev, void *output_dev);
+void *zant_model_input_ptr(zant_model *m);
+void *zant_model_output_ptr(zant_model *m);
+/* Host in / host out: upload, run, download (synchronous). */
+int zant_model_predict_host(zant_model *m, const void *input_host, void *output_host);
+/* Debug: copies tensor `id` (as planned in the arena) to the host after a run. */
+int zant_model_read_tensor(zant_model *m, int id, void *dst_host, size_t bytes);
+
+/* The reference's exported entry point (src/codeGen/predict.zig:34-39), served by the bound model:
+ * silent return when shape_len is 0, differs from the model's rank, or a dimension differs
+ * (predict.zig:317-335); otherwise *result points at library-owned host storage that stays valid
+ * until the next call. */
+int zant_model_bind_predict(zant_model *m);
+void predict(float *input, uint32_t *input_shape, uint32_t shape_len, float **result);
+
 #ifdef __cplusplus
 }
 #endif

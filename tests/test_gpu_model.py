@@ -1,0 +1,185 @@
+"""The generated-library level (zant_model): whole networks in one arena, against the CPU oracle."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import oracle as zo
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def G():
+    import gpu_util
+    return gpu_util
+
+
+def readme_cnn(G, batch, params):
+    from zant_amd.model import Model
+    m = Model(G.tm.context())
+    x = m.input((batch, 1, 28, 28))
+    t = m.conv(x, params["w1"], params["b1"], [1, 1], None, None, 1, None)
+    t = m.relu(t)
+    t = m.maxpool(t, [2, 2], [2, 2])
+    t = m.conv(t, params["w2"], params["b2"], [1, 1], None, None, 1, None)
+    t = m.relu(t)
+    t = m.maxpool(t, [2, 2], [2, 2])
+    t = m.reshape(t, [1, 1, batch, 1600])
+    t = m.gemm(t, params["g1"], params["c1"])
+    t = m.relu(t)
+    t = m.gemm(t, params["g2"], params["c2"])
+    t = m.reshape(t, [batch, 10])
+    t = m.softmax(t)
+    return m.finalize()
+
+
+def oracle_readme_cnn(img, p):
+    y = zo.ReLU(zo.Conv(img, p["w1"], p["b1"], [1, 1], None, None, 1, None))
+    y = zo.onnx_maxpool(y, [2, 2], [2, 2], [1, 1], [0, 0, 0, 0])
+    y = zo.ReLU(zo.Conv(y, p["w2"], p["b2"], [1, 1], None, None, 1, None))
+    y = zo.onnx_maxpool(y, [2, 2], [2, 2], [1, 1], [0, 0, 0, 0])
+    y = zo.ReLU(zo.gemm(y.reshape(1, 1, 1, 1600), p["g1"], p["c1"], 1.0, 1.0, False, False))
+    y = zo.gemm(y, p["g2"], p["c2"], 1.0, 1.0, False, False)
+    return zo.softmax(y.reshape(1, 10))
+
+
+def test_readme_cnn_matches_oracle_and_plans_one_arena(G):
+    from zant_amd import networks
+    params = networks.readme_cnn_params(seed=3)
+    params["b1"] = (np.random.default_rng(0).standard_normal(32) * 0.1).astype(np.float32)  # exercise the bias path
+    batch = 37
+    m = readme_cnn(G, batch, params)
+    x = np.random.default_rng(1).random((batch, 1, 28, 28), dtype=np.float32)
+    y = m.predict_host(x)
+    ref = np.concatenate([oracle_readme_cnn(x[i:i + 1], params) for i in range(batch)])
+    np.testing.assert_allclose(y, ref, rtol=G.RTOL, atol=G.ATOL)
+    # 12 nodes: 3 ReLUs ride in their producers, 2 Reshapes are views -> 7 kernel-launching nodes
+    assert m.num_launches == 7
+    # liveness planning: the arena is much smaller than one static array per node output
+    assert m.arena_bytes < 0.6 * m.unfused_bytes
+
+
+def test_run_on_device_pointers_allocates_nothing(G):
+    import torch
+    from zant_amd import networks
+    params = networks.readme_cnn_params(seed=0)
+    batch = 64
+    m = readme_cnn(G, batch, params)
+    x = torch.rand((batch, 1, 28, 28), device="cuda:0")
+    out = torch.zeros((batch, 10), device="cuda:0")
+    m.run(x.data_ptr(), out.data_ptr())
+    torch.cuda.synchronize()
+    first = out.clone()
+    free0, _ = torch.cuda.mem_get_info()
+    arena0 = G.za.lib.zant_hip_arena_size(G.tm.context().handle)
+    for _ in range(5):
+        m.run(x.data_ptr(), out.data_ptr())
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0 and G.za.lib.zant_hip_arena_size(G.tm.context().handle) == arena0
+    assert torch.equal(out, first)  # same input, same arena: bit-identical reruns
+    ref = np.concatenate([oracle_readme_cnn(G.host(x)[i:i + 1], params) for i in (0, batch - 1)])
+    np.testing.assert_allclose(G.host(out)[[0, batch - 1]], ref, rtol=G.RTOL, atol=G.ATOL)
+
+
+def test_mnist8_style_graph_folds_add_into_conv_bias(G):
+    """Conv(SAME_UPPER, no bias) -> Add({M,1,1}) -> Relu -> MaxPool -> Reshape -> MatMul -> Add, as the reference's
+    hardcoded_mnist8.zig:186-283 emits it."""
+    from zant_amd.model import Model
+    g = np.random.default_rng(5)
+    w1 = (g.standard_normal((8, 1, 5, 5)) * 0.2).astype(np.float32); b1 = g.standard_normal((8, 1, 1)).astype(np.float32)
+    w2 = (g.standard_normal((16, 8, 5, 5)) * 0.07).astype(np.float32); b2 = g.standard_normal((16, 1, 1)).astype(np.float32)
+    fc = (g.standard_normal((256, 10)) * 0.06).astype(np.float32); fb = g.standard_normal((1, 10)).astype(np.float32)
+    m = Model(G.tm.context())
+    x = m.input((1, 1, 28, 28))
+    t = m.conv(x, w1, None, [1, 1], None, [1, 1], 1, "SAME_UPPER")
+    t = m.add_const(t, b1)
+    t = m.relu(t)
+    t = m.maxpool(t, [2, 2], [2, 2])
+    t = m.conv(t, w2, None, [1, 1], None, [1, 1], 1, "SAME_UPPER")
+    t = m.add_const(t, b2)
+    t = m.relu(t)
+    t = m.maxpool(t, [3, 3], [3, 3])
+    t = m.reshape(t, [1, 256])
+    t = m.matmul(t, fc)
+    t = m.add_const(t, fb)
+    m.finalize()
+    assert m.num_launches == 6  # conv, pool, conv, pool, matmul, add
+    img = g.random((1, 1, 28, 28), dtype=np.float32)
+    y = m.predict_host(img)
+    r = zo.Conv(img, w1, None, [1, 1], None, [1, 1], 1, "SAME_UPPER")
+    r = zo.ReLU(zo.sum_tensors_lean(r, b1))
+    r = zo.onnx_maxpool(r, [2, 2], [2, 2], [1, 1], [0, 0, 0, 0])
+    r = zo.Conv(r, w2, None, [1, 1], None, [1, 1], 1, "SAME_UPPER")
+    r = zo.ReLU(zo.sum_tensors_lean(r, b2))
+    r = zo.onnx_maxpool(r, [3, 3], [3, 3], [1, 1], [0, 0, 0, 0])
+    r = zo.sum_tensors_lean(zo.mat_mul(r.reshape(1, 256), fc), fb)
+    np.testing.assert_allclose(y, r, rtol=G.RTOL, atol=1e-4)
+
+
+def test_predict_entry_point_follows_the_reference_abi(G):
+    from zant_amd import networks
+    params = networks.readme_cnn_params(seed=0)
+    m = readme_cnn(G, 1, params)
+    m.bind_predict()
+    lib = G.za.lib
+    img = np.random.default_rng(2).random((1, 1, 28, 28), dtype=np.float32)
+    result = C.c_void_p(0)
+
+    def call(shape):
+        arr = (C.c_uint32 * max(len(shape), 1))(*shape)
+        lib.predict(img.ctypes.data_as(C.c_void_p), arr, len(shape), C.byref(result))
+
+    # wrong rank, empty shape, wrong dimension: silent return, result untouched (predict.zig:317-335)
+    for bad in ([1, 28, 28], [], [1, 1, 28, 27], [2, 1, 28, 28]):
+        call(bad)
+        assert result.value is None
+    call([1, 1, 28, 28])
+    assert result.value is not None
+    out = np.ctypeslib.as_array(C.cast(result, C.POINTER(C.c_float)), shape=(10,)).copy()
+    np.testing.assert_allclose(out, oracle_readme_cnn(img, params).ravel(), rtol=G.RTOL, atol=G.ATOL)
+    first_ptr = result.value
+    call([1, 1, 28, 28])
+    assert result.value == first_ptr  # library-owned storage, reused by the next call
+    lib.zant_model_bind_predict(None)
+    result2 = C.c_void_p(0)
+    arr = (C.c_uint32 * 4)(1, 1, 28, 28)
+    lib.predict(img.ctypes.data_as(C.c_void_p), arr, 4, C.byref(result2))
+    assert result2.value is None  # no model bound: nothing happens
+
+
+def test_int8_network_fuses_activation_and_is_bit_exact(G):
+    """QLinearConv -> Dequant/LeakyReLU/Quant -> MaxPool -> QLinearConv -> ReLU6 -> residual add -> global average pool."""
+    from zant_amd.model import Model, U8
+    g = np.random.default_rng(7)
+    N = 5
+    x = g.integers(0, 256, (N, 3, 24, 24), dtype=np.uint8)
+    w1 = g.integers(-127, 128, (16, 3, 3, 3), dtype=np.int8); s1 = g.uniform(0.002, 0.004, 16).astype(np.float32)
+    b1 = g.integers(-500, 500, 16, dtype=np.int32)
+    w2 = g.integers(-127, 128, (16, 16, 3, 3), dtype=np.int8); s2 = g.uniform(0.0005, 0.001, 16).astype(np.float32)
+    wd = g.integers(-127, 128, (16, 1, 3, 3), dtype=np.int8); sd = g.uniform(0.002, 0.004, 16).astype(np.float32)
+    m = Model(G.tm.context())
+    t0 = m.input((N, 3, 24, 24), U8, 0.02, 128)
+    t1 = m.qlinearconv(t0, w1, s1, b1, 0.05, 128, [1, 1], [1, 1, 1, 1])
+    t2 = m.qlinear_act(t1, "leaky", 0.1, 0.04, 30)
+    t3 = m.maxpool(t2, [2, 2], [2, 2])
+    t4 = m.qlinearconv(t3, w2, s2, None, 0.05, 120, [1, 1], [1, 1, 1, 1])
+    t5 = m.qlinear_act(t4, "relu6", 0.0, 0.03, 0)
+    t6 = m.qlinearconv(t5, wd, sd, None, 0.06, 110, [1, 1], [1, 1, 1, 1], group=16)   # depthwise
+    t7 = m.qlinear_add(t6, t3, 0.07, 100)                                             # residual
+    t8 = m.qlinear_global_avgpool(t7, 0.05, 90)
+    m.finalize()
+    assert m.num_launches == 6  # both activations ride in their convolutions
+    y = m.predict_host(x)
+    r1 = zo.qlinearconv(x, 0.02, 128, w1, s1, None, 0.05, 128, b1, [1, 1], [1, 1, 1, 1], [1, 1])
+    r2 = zo.qlinear_act(r1, 0.05, 128, "leaky", 0.1, 0.04, 30)
+    r3 = zo.onnx_maxpool(r2, [2, 2], [2, 2], [1, 1], [0, 0, 0, 0])
+    r4 = zo.qlinearconv(r3, 0.04, 30, w2, s2, None, 0.05, 120, None, [1, 1], [1, 1, 1, 1], [1, 1])
+    r5 = zo.qlinear_act(r4, 0.05, 120, "relu6", 0.0, 0.03, 0)
+    r6 = zo.qlinearconv(r5, 0.03, 0, wd, sd, None, 0.06, 110, None, [1, 1], [1, 1, 1, 1], [1, 1], 16)
+    r7 = zo.qlinear_add(r6, 0.06, 110, r3, 0.04, 30, 0.07, 100)
+    r8 = zo.qlinear_global_avgpool(r7, 0.07, 100, 0.05, 90)
+    np.testing.assert_array_equal(y, r8)
+    np.testing.assert_array_equal(m.read_tensor(t3, r3.shape, np.uint8), r3)
+    assert len(np.unique(r8)) > 4

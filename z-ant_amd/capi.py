@@ -61,6 +61,37 @@ PROTOTYPES = {
     "zant_hip_qlinear_act_u8": (i32, [vp, vp, i64, f32, u8, i32, f32, f32, u8, vp]),
     "zant_hip_qlinear_add_u8": (i32, [vp, vp, f32, u8, vp, f32, u8, f32, u8, vp, i64]),
     "zant_hip_qlinear_global_avgpool_u8": (i32, [vp, vp, c_i64p, f32, u8, f32, u8, vp]),
+    "zant_model_create": (i32, [vp, C.POINTER(vp)]),
+    "zant_model_destroy": (None, [vp]),
+    "zant_model_input": (i32, [vp, i32, c_i64p, i32, f32, i32]),
+    "zant_model_conv": (i32, [vp, i32, vp, c_i64p, vp, c_i64p, i32, c_i64p, i32, c_i64p, i32, i64, C.c_char_p]),
+    "zant_model_relu": (i32, [vp, i32]),
+    "zant_model_leaky_relu": (i32, [vp, i32, f32]),
+    "zant_model_maxpool": (i32, [vp, i32, c_i64p, c_i64p, c_i64p, c_i64p, i32, i32]),
+    "zant_model_reshape": (i32, [vp, i32, c_i64p, i32]),
+    "zant_model_gemm": (i32, [vp, i32, vp, c_i64p, vp, c_i64p, i32, f32, f32, i32, i32]),
+    "zant_model_matmul": (i32, [vp, i32, vp, c_i64p, i32]),
+    "zant_model_add_const": (i32, [vp, i32, vp, c_i64p, i32]),
+    "zant_model_add": (i32, [vp, i32, i32]),
+    "zant_model_softmax": (i32, [vp, i32]),
+    "zant_model_quantize": (i32, [vp, i32, f32, i32]),
+    "zant_model_dequantize": (i32, [vp, i32]),
+    "zant_model_qlinearconv": (i32, [vp, i32, vp, c_i64p, vp, i64, vp, f32, i32, c_i64p, c_i64p, c_i64p, i64]),
+    "zant_model_qlinear_act": (i32, [vp, i32, i32, f32, f32, i32]),
+    "zant_model_qlinear_add": (i32, [vp, i32, i32, f32, i32]),
+    "zant_model_qlinear_global_avgpool": (i32, [vp, i32, f32, i32]),
+    "zant_model_finalize": (i32, [vp]),
+    "zant_model_output_dims": (i32, [vp, c_i64p, C.POINTER(i32), C.POINTER(i32)]),
+    "zant_model_arena_bytes": (sz, [vp]),
+    "zant_model_unfused_bytes": (sz, [vp]),
+    "zant_model_num_launches": (i32, [vp]),
+    "zant_model_run": (i32, [vp, vp, vp]),
+    "zant_model_input_ptr": (vp, [vp]),
+    "zant_model_output_ptr": (vp, [vp]),
+    "zant_model_predict_host": (i32, [vp, vp, vp]),
+    "zant_model_read_tensor": (i32, [vp, i32, vp, sz]),
+    "zant_model_bind_predict": (i32, [vp]),
+    "predict": (None, [vp, C.POINTER(C.c_uint32), C.c_uint32, C.POINTER(vp)]),
 }
 
 for _name, (_res, _args) in PROTOTYPES.items():

@@ -1,0 +1,677 @@
+// zant_model: the GPU form of a generated library (reference src/codeGen/predict.zig:23-70, 265-377).
+//
+// The reference emits one zero-initialised static array per node output, memsets all of them at the
+// top of every predict(), and calls one *_lean operator per ONNX node.  Here the node list is built
+// once (ready order), then finalize():
+//   - folds a constant per-channel Add into the preceding bias-less Conv (the mnist-8 pattern
+//     Conv -> Add({M,1,1}) -> Relu, src/codeGen/hardcoded/hardcoded_mnist8.zig:186-209),
+//   - fuses Relu into the Conv / Gemm that feeds it, and the Dequantize -> activation -> Quantize
+//     step into the QLinearConv that feeds it (one kernel epilogue instead of a pass over HBM),
+//   - turns Reshape into a view,
+//   - assigns every remaining activation an offset in ONE device allocation by liveness
+//     (first fit over [definition, last use] intervals), and uploads all parameters into one
+//     allocation.
+// run() then enqueues the operator kernels on arena pointers: no allocation, no memset (every
+// kernel writes its whole output).
+#include <algorithm>
+#include <vector>
+
+#include "common.h"
+
+namespace {
+
+enum OpKind {
+    OP_CONV, OP_RELU, OP_LEAKY, OP_MAXPOOL, OP_RESHAPE, OP_GEMM, OP_MATMUL, OP_ADD_CONST, OP_ADD, OP_SOFTMAX,
+    OP_QUANT, OP_DEQUANT, OP_QCONV, OP_QACT, OP_QADD, OP_QGAP
+};
+
+struct MTensor {
+    int dtype = ZANT_F32;
+    int rank = 0;
+    int64_t dim[8] = {0};
+    float scale = 1.0f;   // quantisation parameters of a u8 tensor
+    int zp = 0;
+    int alias_of = -1;    // shares storage with that tensor (views, fused activations)
+    size_t offset = 0;    // in the arena, valid for storage roots after finalize
+    int def = -1, last = -1;
+    size_t bytes() const {
+        size_t n = dtype == ZANT_F32 ? 4 : 1;
+        for (int i = 0; i < rank; ++i) n *= size_t(dim[i]);
+        return n;
+    }
+};
+
+struct Param {           // a host copy of a constant until finalize, then its place in the parameter block
+    std::vector<char> host;
+    size_t offset = 0;
+};
+
+struct MNode {
+    int op = 0;
+    int in0 = -1, in1 = -1, out = -1;
+    bool skip = false;            // fused into its producer or turned into a view
+    int fuse_act = ZANT_ACT_NONE; // activation applied in this node's epilogue
+    float act_alpha = 0.0f, act_scale = 1.0f;
+    int act_zp = 0;
+    int w = -1, b = -1, c = -1, ws = -1;  // parameter indices
+    int64_t wdim[4] = {0}, cdim[4] = {0};
+    int c_rank = 0;
+    int64_t stride[2] = {1, 1}, pads[4] = {0, 0, 0, 0}, dil[2] = {1, 1}, kernel[2] = {1, 1};
+    int n_stride = 2, n_pads = 0, n_dil = 0;
+    bool has_pads = false, has_dil = false;
+    int64_t group = 1;
+    std::string auto_pad;
+    bool has_auto_pad = false;
+    int pool_pad = ZANT_PAD_NOTSET;
+    float alpha = 1.0f, beta = 1.0f, slope = 0.0f;
+    int trans_a = 0, trans_b = 0;
+    int64_t n_wscale = 1;
+    int act = ZANT_ACT_NONE;
+    int b_rank = 0;
+    int64_t bdim[8] = {0};
+};
+
+}  // namespace
+
+struct zant_model {
+    zant_ctx *ctx = nullptr;
+    std::vector<MTensor> t;
+    std::vector<MNode> n;
+    std::vector<Param> p;
+    bool finalized = false;
+    int input = -1, output = -1;
+    void *params_dev = nullptr;
+    size_t arena_bytes = 0, unfused_bytes = 0;
+    int launches = 0;
+    std::vector<char> result_host;  // what predict() hands out
+};
+
+namespace {
+
+zant_model *g_predict_model = nullptr;
+
+int root_of(const zant_model *m, int id) {
+    while (m->t[id].alias_of >= 0) id = m->t[id].alias_of;
+    return id;
+}
+
+int add_tensor(zant_model *m, int dtype, const int64_t *dims, int rank, float scale, int zp) {
+    MTensor t;
+    t.dtype = dtype; t.rank = rank; t.scale = scale; t.zp = zp;
+    for (int i = 0; i < rank; ++i) t.dim[i] = dims[i];
+    m->t.push_back(t);
+    return int(m->t.size()) - 1;
+}
+
+int add_param(zant_model *m, const void *src, size_t bytes) {
+    Param p;
+    p.host.assign(static_cast<const char *>(src), static_cast<const char *>(src) + bytes);
+    m->p.push_back(std::move(p));
+    return int(m->p.size()) - 1;
+}
+
+bool valid_tensor(const zant_model *m, int id) { return m && id >= 0 && id < int(m->t.size()); }
+
+void *tensor_ptr(zant_model *m, int id) {
+    return static_cast<char *>(m->ctx->arena) + m->t[root_of(m, id)].offset;
+}
+
+const void *param_ptr(const zant_model *m, int idx) {
+    return idx < 0 ? nullptr : static_cast<const char *>(m->params_dev) + m->p[idx].offset;
+}
+
+int consumers(const zant_model *m, int tensor, int *only) {
+    int cnt = 0;
+    for (size_t i = 0; i < m->n.size(); ++i)
+        if (m->n[i].in0 == tensor || m->n[i].in1 == tensor) { ++cnt; *only = int(i); }
+    return cnt;
+}
+
+int producer(const zant_model *m, int tensor) {
+    for (size_t i = 0; i < m->n.size(); ++i)
+        if (m->n[i].out == tensor) return int(i);
+    return -1;
+}
+
+int append(zant_model *m, MNode &node, int dtype, const int64_t *dims, int rank, float scale, int zp) {
+    if (m->finalized) return ZANT_InvalidInput;
+    node.out = add_tensor(m, dtype, dims, rank, scale, zp);
+    m->n.push_back(node);
+    return node.out;
+}
+
+int run_node(zant_model *m, const MNode &nd) {
+    zant_ctx *ctx = m->ctx;
+    const MTensor &ti = m->t[nd.in0];
+    const MTensor &to = m->t[nd.out];
+    const void *x = tensor_ptr(m, nd.in0);
+    void *y = tensor_ptr(m, nd.out);
+    switch (nd.op) {
+    case OP_CONV:
+        return zant_hip_conv2d_f32(ctx, static_cast<const float *>(x), ti.dim, static_cast<const float *>(param_ptr(m, nd.w)),
+                                   nd.wdim, static_cast<const float *>(param_ptr(m, nd.b)), static_cast<float *>(y), to.dim,
+                                   nd.stride, nd.n_stride, nd.has_pads ? nd.pads : nullptr, nd.n_pads,
+                                   nd.has_dil ? nd.dil : nullptr, nd.n_dil, nd.group,
+                                   nd.has_auto_pad ? nd.auto_pad.c_str() : nullptr, nd.fuse_act);
+    case OP_RELU:
+        return zant_hip_relu_f32(ctx, static_cast<const float *>(x), static_cast<float *>(y), int64_t(ti.bytes() / 4));
+    case OP_LEAKY:
+        return zant_hip_leaky_relu_f32(ctx, static_cast<const float *>(x), nd.slope, static_cast<float *>(y),
+                                       int64_t(ti.bytes() / 4));
+    case OP_MAXPOOL:
+        if (ti.dtype == ZANT_U8)
+            return zant_hip_maxpool2d_u8(ctx, static_cast<const uint8_t *>(x), ti.dim, static_cast<uint8_t *>(y), to.dim,
+                                         nd.kernel, nd.stride, nd.dil, nd.pads, 4, nd.pool_pad);
+        return zant_hip_maxpool2d_f32(ctx, static_cast<const float *>(x), ti.dim, static_cast<float *>(y), to.dim, nd.kernel,
+                                      nd.stride, nd.dil, nd.pads, 4, nd.pool_pad);
+    case OP_GEMM:
+        return zant_hip_gemm_f32(ctx, static_cast<const float *>(x), ti.dim, static_cast<const float *>(param_ptr(m, nd.w)),
+                                 nd.wdim, static_cast<const float *>(param_ptr(m, nd.c)), nd.cdim, nd.c_rank, nd.alpha,
+                                 nd.beta, nd.trans_a, nd.trans_b, static_cast<float *>(y), to.dim, nd.fuse_act);
+    case OP_MATMUL:
+        return zant_hip_matmul_f32(ctx, static_cast<const float *>(x), ti.dim, ti.rank,
+                                   static_cast<const float *>(param_ptr(m, nd.w)), nd.bdim, nd.b_rank, static_cast<float *>(y));
+    case OP_ADD_CONST:
+        return zant_hip_add_f32(ctx, static_cast<const float *>(x), ti.dim, ti.rank,
+                                static_cast<const float *>(param_ptr(m, nd.c)), nd.cdim, nd.c_rank, static_cast<float *>(y),
+                                nullptr, nullptr);
+    case OP_ADD: {
+        const MTensor &tb = m->t[nd.in1];
+        return zant_hip_add_f32(ctx, static_cast<const float *>(x), ti.dim, ti.rank,
+                                static_cast<const float *>(tensor_ptr(m, nd.in1)), tb.dim, tb.rank, static_cast<float *>(y),
+                                nullptr, nullptr);
+    }
+    case OP_SOFTMAX:
+        return zant_hip_softmax_f32(ctx, static_cast<const float *>(x), static_cast<float *>(y), ti.dim[0], ti.dim[1]);
+    case OP_QUANT:
+        return zant_hip_quantize_linear_f32_u8(ctx, static_cast<const float *>(x), ti.dim, ti.rank,
+                                               static_cast<const float *>(param_ptr(m, nd.ws)),
+                                               static_cast<const uint8_t *>(param_ptr(m, nd.b)), 1, 1,
+                                               static_cast<uint8_t *>(y));
+    case OP_DEQUANT:
+        return zant_hip_dequantize_linear_u8_f32(ctx, static_cast<const uint8_t *>(x), ti.dim, ti.rank,
+                                                 static_cast<const float *>(param_ptr(m, nd.ws)),
+                                                 static_cast<const uint8_t *>(param_ptr(m, nd.b)), 1, 1,
+                                                 static_cast<float *>(y));
+    case OP_QCONV:
+        return zant_hip_qlinearconv_u8i8(ctx, static_cast<const uint8_t *>(x), ti.dim, ti.scale, uint8_t(ti.zp),
+                                         static_cast<const int8_t *>(param_ptr(m, nd.w)), nd.wdim,
+                                         static_cast<const float *>(param_ptr(m, nd.ws)), nd.n_wscale, nullptr,
+                                         nd.fuse_act ? nd.act_scale : to.scale, uint8_t(nd.fuse_act ? nd.act_zp : to.zp),
+                                         static_cast<const int32_t *>(param_ptr(m, nd.b)), static_cast<uint8_t *>(y), to.dim,
+                                         nd.stride, nd.pads, nd.dil, nd.group, nd.fuse_act, nd.act_alpha, to.scale,
+                                         uint8_t(to.zp));
+    case OP_QACT:
+        return zant_hip_qlinear_act_u8(ctx, static_cast<const uint8_t *>(x), int64_t(ti.bytes()), ti.scale, uint8_t(ti.zp),
+                                       nd.act, nd.act_alpha, to.scale, uint8_t(to.zp), static_cast<uint8_t *>(y));
+    case OP_QADD: {
+        const MTensor &tb = m->t[nd.in1];
+        return zant_hip_qlinear_add_u8(ctx, static_cast<const uint8_t *>(x), ti.scale, uint8_t(ti.zp),
+                                       static_cast<const uint8_t *>(tensor_ptr(m, nd.in1)), tb.scale, uint8_t(tb.zp), to.scale,
+                                       uint8_t(to.zp), static_cast<uint8_t *>(y), int64_t(ti.bytes()));
+    }
+    case OP_QGAP:
+        return zant_hip_qlinear_global_avgpool_u8(ctx, static_cast<const uint8_t *>(x), ti.dim, ti.scale, uint8_t(ti.zp),
+                                                  to.scale, uint8_t(to.zp), static_cast<uint8_t *>(y));
+    default:
+        return ZANT_InvalidInput;
+    }
+}
+
+}  // namespace
+
+extern "C" int zant_model_create(zant_ctx *ctx, zant_model **out) {
+    if (!ctx || !out) return ZANT_NullPointer;
+    zant_model *m = new (std::nothrow) zant_model();
+    if (!m) return ZANT_MemError;
+    m->ctx = ctx;
+    *out = m;
+    return ZANT_OK;
+}
+
+extern "C" void zant_model_destroy(zant_model *m) {
+    if (!m) return;
+    if (g_predict_model == m) g_predict_model = nullptr;
+    if (m->params_dev) {
+        (void)hipStreamSynchronize(m->ctx->stream);
+        (void)hipFree(m->params_dev);
+    }
+    delete m;
+}
+
+extern "C" int zant_model_input(zant_model *m, int dtype, const int64_t *dims, int rank, float scale, int zp) {
+    if (!m || !dims) return ZANT_NullPointer;
+    if (m->finalized || m->input >= 0 || rank < 1 || rank > 8 || (dtype != ZANT_F32 && dtype != ZANT_U8)) return ZANT_InvalidInput;
+    for (int i = 0; i < rank; ++i)
+        if (dims[i] <= 0) return ZANT_InvalidDimensions;
+    m->input = add_tensor(m, dtype, dims, rank, scale, zp);
+    return m->input;
+}
+
+extern "C" int zant_model_conv(zant_model *m, int x, const float *w, const int64_t wdim[4], const float *bias,
+                               const int64_t *stride, int n_stride, const int64_t *pads, int n_pads, const int64_t *dil,
+                               int n_dil, int64_t group, const char *auto_pad) {
+    if (!valid_tensor(m, x) || !w || !wdim || !stride) return ZANT_NullPointer;
+    const MTensor &tx = m->t[x];
+    if (tx.rank != 4 || tx.dtype != ZANT_F32) return ZANT_InvalidDimensions;
+    if (n_stride < 1 || n_stride > 2 || n_pads > 4 || n_dil > 2) return ZANT_InvalidInput;
+    // shape inference runs the operator's own rule; the generated code passes pads only with "NOTSET" in mind
+    int64_t s[2], d[2], p[4];
+    int rc = zant_conv_resolve(tx.dim, wdim, stride, n_stride, pads, n_pads, dil, n_dil, group, auto_pad, s, d, p);
+    if (rc) return rc;
+    const int64_t dkh = (wdim[2] - 1) * d[0] + 1, dkw = (wdim[3] - 1) * d[1] + 1;
+    const int64_t PH = tx.dim[2] + p[0] + p[2], PW = tx.dim[3] + p[1] + p[3];
+    if (PH < dkh || PW < dkw || tx.dim[1] != wdim[1]) return ZANT_InvalidDimensions;
+    const int64_t ydim[4] = {tx.dim[0], wdim[0], (PH - dkh) / s[0] + 1, (PW - dkw) / s[1] + 1};
+    MNode nd;
+    nd.op = OP_CONV; nd.in0 = x;
+    for (int i = 0; i < 4; ++i) nd.wdim[i] = wdim[i];
+    nd.w = add_param(m, w, size_t(wdim[0] * wdim[1] * wdim[2] * wdim[3]) * 4);
+    if (bias) nd.b = add_param(m, bias, size_t(wdim[0]) * 4);
+    nd.n_stride = n_stride;
+    for (int i = 0; i < n_stride; ++i) nd.stride[i] = stride[i];
+    nd.has_pads = pads != nullptr; nd.n_pads = n_pads;
+    for (int i = 0; pads && i < n_pads; ++i) nd.pads[i] = pads[i];
+    nd.has_dil = dil != nullptr; nd.n_dil = n_dil;
+    for (int i = 0; dil && i < n_dil; ++i) nd.dil[i] = dil[i];
+    nd.group = group;
+    nd.has_auto_pad = auto_pad != nullptr;
+    if (auto_pad) nd.auto_pad = auto_pad;
+    return append(m, nd, ZANT_F32, ydim, 4, 1.0f, 0);
+}
+
+static int unary_same_shape(zant_model *m, int x, int op, float slope) {
+    if (!valid_tensor(m, x)) return ZANT_NullPointer;
+    const MTensor tx = m->t[x];
+    if (tx.dtype != ZANT_F32) return ZANT_InvalidInput;
+    MNode nd;
+    nd.op = op; nd.in0 = x; nd.slope = slope;
+    return append(m, nd, ZANT_F32, tx.dim, tx.rank, 1.0f, 0);
+}
+
+extern "C" int zant_model_relu(zant_model *m, int x) { return unary_same_shape(m, x, OP_RELU, 0.0f); }
+extern "C" int zant_model_leaky_relu(zant_model *m, int x, float slope) { return unary_same_shape(m, x, OP_LEAKY, slope); }
+
+extern "C" int zant_model_maxpool(zant_model *m, int x, const int64_t kernel[2], const int64_t strides[2],
+                                  const int64_t dil[2], const int64_t pads[4], int auto_pad, int ceil_mode) {
+    if (!valid_tensor(m, x) || !kernel || !strides || !dil || !pads) return ZANT_NullPointer;
+    const MTensor tx = m->t[x];
+    if (tx.rank != 4) return ZANT_InvalidDimensions;
+    int64_t ydim[4];
+    int rc = zant_hip_maxpool2d_out_shape(tx.dim, kernel, strides, dil, pads, auto_pad, ceil_mode, ydim);
+    if (rc) return rc;
+    MNode nd;
+    nd.op = OP_MAXPOOL; nd.in0 = x; nd.pool_pad = auto_pad;
+    for (int i = 0; i < 2; ++i) { nd.kernel[i] = kernel[i]; nd.stride[i] = strides[i]; nd.dil[i] = dil[i]; }
+    for (int i = 0; i < 4; ++i) nd.pads[i] = pads[i];
+    return append(m, nd, tx.dtype, ydim, 4, tx.scale, tx.zp);
+}
+
+extern "C" int zant_model_reshape(zant_model *m, int x, const int64_t *new_shape, int rank) {
+    if (!valid_tensor(m, x) || !new_shape) return ZANT_NullPointer;
+    if (rank < 1 || rank > 8) return ZANT_InvalidInput;
+    const MTensor tx = m->t[x];
+    int64_t ydim[8];
+    // shape resolution of reshape_lean (0 copies, -1 infers); no data moves: the result is a view
+    int rc = zant_hip_reshape(m->ctx, nullptr, tx.dim, tx.rank, 1, new_shape, rank, nullptr, ydim);
+    if (rc) return rc;
+    MNode nd;
+    nd.op = OP_RESHAPE; nd.in0 = x;
+    return append(m, nd, tx.dtype, ydim, rank, tx.scale, tx.zp);
+}
+
+extern "C" int zant_model_gemm(zant_model *m, int a, const float *b, const int64_t bdim[4], const float *c,
+                               const int64_t *cdim, int c_rank, float alpha, float beta, int trans_a, int trans_b) {
+    if (!valid_tensor(m, a) || !b || !bdim) return ZANT_NullPointer;
+    const MTensor ta = m->t[a];
+    if (ta.dtype != ZANT_F32) return ZANT_InvalidInput;
+    int64_t ydim[4];
+    int rc = zant_hip_gemm_check(ta.dim, ta.rank, bdim, 4, cdim, c_rank, c != nullptr, trans_a, trans_b, ydim);
+    if (rc) return rc;
+    MNode nd;
+    nd.op = OP_GEMM; nd.in0 = a;
+    for (int i = 0; i < 4; ++i) nd.wdim[i] = bdim[i];
+    nd.w = add_param(m, b, size_t(bdim[0] * bdim[1] * bdim[2] * bdim[3]) * 4);
+    if (c) {
+        nd.c_rank = c_rank;
+        size_t n = 4;
+        for (int i = 0; i < c_rank; ++i) { nd.cdim[i] = cdim[i]; n *= size_t(cdim[i]); }
+        nd.c = add_param(m, c, n);
+    }
+    nd.alpha = alpha; nd.beta = beta; nd.trans_a = trans_a; nd.trans_b = trans_b;
+    return append(m, nd, ZANT_F32, ydim, 4, 1.0f, 0);
+}
+
+extern "C" int zant_model_matmul(zant_model *m, int a, const float *b, const int64_t *bdim, int b_rank) {
+    if (!valid_tensor(m, a) || !b || !bdim) return ZANT_NullPointer;
+    const MTensor ta = m->t[a];
+    if (ta.dtype != ZANT_F32 || b_rank > 8) return ZANT_InvalidInput;
+    int rc = zant_hip_matmul_check(ta.dim, ta.rank, bdim, b_rank);
+    if (rc) return rc;
+    MNode nd;
+    nd.op = OP_MATMUL; nd.in0 = a; nd.b_rank = b_rank;
+    size_t n = 4;
+    for (int i = 0; i < b_rank; ++i) { nd.bdim[i] = bdim[i]; n *= size_t(bdim[i]); }
+    nd.w = add_param(m, b, n);
+    int64_t ydim[8];
+    for (int i = 0; i < ta.rank; ++i) ydim[i] = ta.dim[i];
+    ydim[ta.rank - 1] = bdim[b_rank - 1];
+    return append(m, nd, ZANT_F32, ydim, ta.rank, 1.0f, 0);
+}
+
+extern "C" int zant_model_add_const(zant_model *m, int x, const float *c, const int64_t *cdim, int c_rank) {
+    if (!valid_tensor(m, x) || !c || !cdim) return ZANT_NullPointer;
+    const MTensor tx = m->t[x];
+    if (tx.dtype != ZANT_F32 || c_rank > 4 || c_rank < 1) return ZANT_InvalidInput;
+    int64_t ydim[8];
+    int yr = 0;
+    int rc = zant_hip_add_f32(m->ctx, nullptr, tx.dim, tx.rank, nullptr, cdim, c_rank, nullptr, ydim, &yr);
+    if (rc != ZANT_OK && rc != ZANT_NullPointer) return rc;  // shapes are validated before pointers are looked at
+    MNode nd;
+    nd.op = OP_ADD_CONST; nd.in0 = x; nd.c_rank = c_rank;
+    size_t n = 4;
+    for (int i = 0; i < c_rank; ++i) { nd.cdim[i] = cdim[i]; n *= size_t(cdim[i]); }
+    nd.c = add_param(m, c, n);
+    return append(m, nd, ZANT_F32, ydim, yr, 1.0f, 0);
+}
+
+extern "C" int zant_model_add(zant_model *m, int a, int b) {
+    if (!valid_tensor(m, a) || !valid_tensor(m, b)) return ZANT_NullPointer;
+    const MTensor ta = m->t[a], tb = m->t[b];
+    if (ta.dtype != ZANT_F32 || tb.dtype != ZANT_F32) return ZANT_InvalidInput;
+    int64_t ydim[8];
+    int yr = 0;
+    int rc = zant_hip_add_f32(m->ctx, nullptr, ta.dim, ta.rank, nullptr, tb.dim, tb.rank, nullptr, ydim, &yr);
+    if (rc != ZANT_OK && rc != ZANT_NullPointer) return rc;
+    MNode nd;
+    nd.op = OP_ADD; nd.in0 = a; nd.in1 = b;
+    return append(m, nd, ZANT_F32, ydim, yr, 1.0f, 0);
+}
+
+extern "C" int zant_model_softmax(zant_model *m, int x) {
+    if (!valid_tensor(m, x)) return ZANT_NullPointer;
+    const MTensor tx = m->t[x];
+    if (tx.dtype != ZANT_F32 || tx.rank < 2) return ZANT_InvalidInput;
+    MNode nd;
+    nd.op = OP_SOFTMAX; nd.in0 = x;
+    return append(m, nd, ZANT_F32, tx.dim, tx.rank, 1.0f, 0);
+}
+
+extern "C" int zant_model_quantize(zant_model *m, int x, float y_scale, int y_zp) {
+    if (!valid_tensor(m, x)) return ZANT_NullPointer;
+    const MTensor tx = m->t[x];
+    if (tx.dtype != ZANT_F32 || y_zp < 0 || y_zp > 255) return ZANT_InvalidInput;
+    MNode nd;
+    nd.op = OP_QUANT; nd.in0 = x;
+    const uint8_t zp8 = uint8_t(y_zp);
+    nd.ws = add_param(m, &y_scale, 4);
+    nd.b = add_param(m, &zp8, 1);
+    return append(m, nd, ZANT_U8, tx.dim, tx.rank, y_scale, y_zp);
+}
+
+extern "C" int zant_model_dequantize(zant_model *m, int x) {
+    if (!valid_tensor(m, x)) return ZANT_NullPointer;
+    const MTensor tx = m->t[x];
+    if (tx.dtype != ZANT_U8) return ZANT_InvalidInput;
+    MNode nd;
+    nd.op = OP_DEQUANT; nd.in0 = x;
+    const uint8_t zp8 = uint8_t(tx.zp);
+    nd.ws = add_param(m, &tx.scale, 4);
+    nd.b = add_param(m, &zp8, 1);
+    return append(m, nd, ZANT_F32, tx.dim, tx.rank, 1.0f, 0);
+}
+
+extern "C" int zant_model_qlinearconv(zant_model *m, int x, const int8_t *w, const int64_t wdim[4], const float *w_scale,
+                                      int64_t n_wscale, const int32_t *bias, float y_scale, int y_zp,
+                                      const int64_t stride[2], const int64_t pads[4], const int64_t dil[2], int64_t group) {
+    if (!valid_tensor(m, x) || !w || !wdim || !w_scale || !stride || !pads || !dil) return ZANT_NullPointer;
+    const MTensor tx = m->t[x];
+    if (tx.dtype != ZANT_U8 || tx.rank != 4 || y_zp < 0 || y_zp > 255) return ZANT_InvalidInput;
+    if (group < 1 || tx.dim[1] % group || wdim[0] % group || tx.dim[1] / group != wdim[1]) return ZANT_InvalidDimensions;
+    if (n_wscale != 1 && n_wscale != wdim[0]) return ZANT_InputTensorDimensionMismatch;
+    if (stride[0] <= 0 || stride[1] <= 0 || dil[0] <= 0 || dil[1] <= 0) return ZANT_WrongStride;
+    const int64_t dkh = (wdim[2] - 1) * dil[0] + 1, dkw = (wdim[3] - 1) * dil[1] + 1;
+    const int64_t PH = tx.dim[2] + pads[0] + pads[2], PW = tx.dim[3] + pads[1] + pads[3];
+    if (PH < dkh || PW < dkw) return ZANT_InvalidDimensions;
+    const int64_t ydim[4] = {tx.dim[0], wdim[0], (PH - dkh) / stride[0] + 1, (PW - dkw) / stride[1] + 1};
+    MNode nd;
+    nd.op = OP_QCONV; nd.in0 = x; nd.group = group; nd.n_wscale = n_wscale;
+    for (int i = 0; i < 4; ++i) { nd.wdim[i] = wdim[i]; nd.pads[i] = pads[i]; }
+    for (int i = 0; i < 2; ++i) { nd.stride[i] = stride[i]; nd.dil[i] = dil[i]; }
+    nd.w = add_param(m, w, size_t(wdim[0] * wdim[1] * wdim[2] * wdim[3]));
+    nd.ws = add_param(m, w_scale, size_t(n_wscale) * 4);
+    if (bias) nd.b = add_param(m, bias, size_t(wdim[0]) * 4);
+    return append(m, nd, ZANT_U8, ydim, 4, y_scale, y_zp);
+}
+
+extern "C" int zant_model_qlinear_act(zant_model *m, int x, int act, float alpha, float y_scale, int y_zp) {
+    if (!valid_tensor(m, x)) return ZANT_NullPointer;
+    const MTensor tx = m->t[x];
+    if (tx.dtype != ZANT_U8 || act < ZANT_ACT_NONE || act > ZANT_ACT_RELU6 || y_zp < 0 || y_zp > 255) return ZANT_InvalidInput;
+    MNode nd;
+    nd.op = OP_QACT; nd.in0 = x; nd.act = act; nd.act_alpha = alpha;
+    return append(m, nd, ZANT_U8, tx.dim, tx.rank, y_scale, y_zp);
+}
+
+extern "C" int zant_model_qlinear_add(zant_model *m, int a, int b, float y_scale, int y_zp) {
+    if (!valid_tensor(m, a) || !valid_tensor(m, b)) return ZANT_NullPointer;
+    const MTensor ta = m->t[a], tb = m->t[b];
+    if (ta.dtype != ZANT_U8 || tb.dtype != ZANT_U8 || y_zp < 0 || y_zp > 255) return ZANT_InvalidInput;
+    if (ta.rank != tb.rank || ta.bytes() != tb.bytes()) return ZANT_InputTensorDifferentSize;
+    MNode nd;
+    nd.op = OP_QADD; nd.in0 = a; nd.in1 = b;
+    return append(m, nd, ZANT_U8, ta.dim, ta.rank, y_scale, y_zp);
+}
+
+extern "C" int zant_model_qlinear_global_avgpool(zant_model *m, int x, float y_scale, int y_zp) {
+    if (!valid_tensor(m, x)) return ZANT_NullPointer;
+    const MTensor tx = m->t[x];
+    if (tx.dtype != ZANT_U8 || tx.rank != 4 || y_zp < 0 || y_zp > 255) return ZANT_InvalidInput;
+    const int64_t ydim[4] = {tx.dim[0], tx.dim[1], 1, 1};
+    MNode nd;
+    nd.op = OP_QGAP; nd.in0 = x;
+    return append(m, nd, ZANT_U8, ydim, 4, y_scale, y_zp);
+}
+
+extern "C" int zant_model_finalize(zant_model *m) {
+    if (!m) return ZANT_NullPointer;
+    if (m->finalized) return ZANT_OK;
+    if (m->input < 0 || m->n.empty()) return ZANT_InvalidInput;
+    zant_ctx *ctx = m->ctx;
+    const int nn = int(m->n.size());
+    m->output = m->n.back().out;
+
+    // ---- peephole fusions -----------------------------------------------------------------------
+    for (int i = 0; i < nn; ++i) {
+        MNode &nd = m->n[i];
+        if (nd.skip) continue;
+        int only = -1;
+        if (nd.op == OP_RESHAPE) {  // a view of its input
+            m->t[nd.out].alias_of = nd.in0;
+            nd.skip = true;
+            continue;
+        }
+        if (nd.op == OP_CONV && nd.b < 0 && consumers(m, nd.out, &only) == 1 && m->n[only].op == OP_ADD_CONST &&
+            m->n[only].in0 == nd.out) {
+            // Conv -> Add(constant of one value per output channel): that constant is the bias
+            MNode &ad = m->n[only];
+            int64_t cnt = 1;
+            for (int k = 0; k < ad.c_rank; ++k) cnt *= ad.cdim[k];
+            const bool per_channel = cnt == nd.wdim[0] &&
+                                     ((ad.c_rank == 3 && ad.cdim[0] == nd.wdim[0]) || (ad.c_rank == 4 && ad.cdim[1] == nd.wdim[0]) ||
+                                      (ad.c_rank == 1 && m->t[nd.out].dim[3] == 1 && m->t[nd.out].dim[2] == 1));
+            if (per_channel) {
+                nd.b = ad.c;
+                m->t[ad.out].alias_of = nd.out;
+                ad.skip = true;
+            }
+        }
+        if ((nd.op == OP_CONV || nd.op == OP_GEMM) && nd.fuse_act == ZANT_ACT_NONE) {
+            int out = nd.out;
+            // look through an Add that was just folded
+            int c1 = -1;
+            while (consumers(m, out, &c1) == 1 && m->n[c1].skip && m->n[c1].op == OP_ADD_CONST) out = m->n[c1].out;
+            if (consumers(m, out, &only) == 1 && m->n[only].op == OP_RELU && !m->n[only].skip) {
+                nd.fuse_act = ZANT_ACT_RELU;
+                m->t[m->n[only].out].alias_of = out;
+                m->n[only].skip = true;
+            }
+        }
+        if (nd.op == OP_QCONV && nd.fuse_act == ZANT_ACT_NONE && consumers(m, nd.out, &only) == 1 &&
+            m->n[only].op == OP_QACT && !m->n[only].skip) {
+            // the activation's output parameters become the kernel's second requantisation stage
+            const MNode &an = m->n[only];
+            const MTensor &ao = m->t[an.out];
+            nd.fuse_act = an.act;
+            nd.act_alpha = an.act_alpha;
+            // run_node passes (conv y_scale/zp) = this node's out tensor, (act scale/zp) = the activation's out tensor
+            nd.act_scale = m->t[nd.out].scale;
+            nd.act_zp = m->t[nd.out].zp;
+            m->t[nd.out].scale = ao.scale;  // the stored tensor now holds the activation's result
+            m->t[nd.out].zp = ao.zp;
+            m->t[an.out].alias_of = nd.out;
+            m->n[only].skip = true;
+        }
+    }
+    (void)producer;
+
+    // ---- liveness and first-fit arena planning --------------------------------------------------
+    const int nt = int(m->t.size());
+    for (int i = 0; i < nt; ++i) { m->t[i].def = -1; m->t[i].last = -1; }
+    m->t[root_of(m, m->input)].def = 0;
+    m->unfused_bytes = 0;
+    m->launches = 0;
+    for (int i = 0; i < nn; ++i) {
+        const MNode &nd = m->n[i];
+        m->unfused_bytes += m->t[nd.out].bytes();
+        if (!nd.skip) ++m->launches;
+        const int ro = root_of(m, nd.out);
+        if (m->t[ro].def < 0) m->t[ro].def = i + 1;
+        for (int in : {nd.in0, nd.in1})
+            if (in >= 0) { const int r = root_of(m, in); m->t[r].last = std::max(m->t[r].last, i + 1); }
+    }
+    m->t[root_of(m, m->output)].last = nn + 1;  // the output outlives the pass
+    m->t[root_of(m, m->input)].last = std::max(m->t[root_of(m, m->input)].last, 1);
+    struct Placed { size_t off, size; int def, last; };
+    std::vector<Placed> placed;
+    size_t arena = 0;
+    std::vector<int> order;
+    for (int i = 0; i < nt; ++i)
+        if (m->t[i].alias_of < 0 && m->t[i].def >= 0) order.push_back(i);
+    std::sort(order.begin(), order.end(), [&](int a, int b) { return m->t[a].def < m->t[b].def; });
+    for (int id : order) {
+        MTensor &t = m->t[id];
+        // the storage of a view chain must hold the largest member (they are all the same size here)
+        const size_t size = (t.bytes() + 255) & ~size_t(255);
+        const int last = std::max(t.last, t.def);
+        std::vector<std::pair<size_t, size_t>> busy;  // arena ranges alive during [def, last]
+        for (const Placed &p : placed)
+            if (!(p.last < t.def || p.def > last)) busy.emplace_back(p.off, p.off + p.size);
+        std::sort(busy.begin(), busy.end());
+        size_t off = 0;
+        for (const auto &b : busy) {
+            if (off + size <= b.first) break;
+            off = std::max(off, b.second);
+        }
+        t.offset = off;
+        placed.push_back({off, size, t.def, last});
+        arena = std::max(arena, off + size);
+    }
+    m->arena_bytes = arena;
+    int rc = zant_hip_arena_reserve(ctx, arena);
+    if (rc) return rc;
+
+    // ---- parameters: one allocation, one upload each ---------------------------------------------
+    size_t pbytes = 0;
+    for (Param &p : m->p) { p.offset = pbytes; pbytes += (p.host.size() + 255) & ~size_t(255); }
+    if (pbytes) {
+        hipError_t e = hipMalloc(&m->params_dev, pbytes);
+        if (e != hipSuccess) { zant_fail_hip(ctx, e, "hipMalloc(parameters)"); return ZANT_MemError; }
+        for (Param &p : m->p) {
+            rc = zant_hip_upload(ctx, static_cast<char *>(m->params_dev) + p.offset, p.host.data(), p.host.size());
+            if (rc) return rc;
+            std::vector<char>().swap(p.host);
+        }
+    }
+    m->result_host.resize(m->t[m->output].bytes());
+    m->finalized = true;
+    return ZANT_OK;
+}
+
+extern "C" int zant_model_output_dims(zant_model *m, int64_t *dims, int *rank, int *dtype) {
+    if (!m || !dims || !rank) return ZANT_NullPointer;
+    if (m->n.empty()) return ZANT_InvalidInput;
+    const MTensor &t = m->t[m->n.back().out];
+    *rank = t.rank;
+    for (int i = 0; i < t.rank; ++i) dims[i] = t.dim[i];
+    if (dtype) *dtype = t.dtype;
+    return ZANT_OK;
+}
+
+extern "C" size_t zant_model_arena_bytes(zant_model *m) { return m ? m->arena_bytes : 0; }
+extern "C" size_t zant_model_unfused_bytes(zant_model *m) { return m ? m->unfused_bytes : 0; }
+extern "C" int zant_model_num_launches(zant_model *m) { return m ? m->launches : 0; }
+
+extern "C" void *zant_model_input_ptr(zant_model *m) { return (m && m->finalized) ? tensor_ptr(m, m->input) : nullptr; }
+extern "C" void *zant_model_output_ptr(zant_model *m) { return (m && m->finalized) ? tensor_ptr(m, m->output) : nullptr; }
+
+extern "C" int zant_model_run(zant_model *m, const void *input_dev, void *output_dev) {
+    if (!m) return ZANT_NullPointer;
+    if (!m->finalized) return ZANT_NotFinalized;
+    zant_ctx *ctx = m->ctx;
+    if (m->arena_bytes > ctx->arena_bytes) return ZANT_ArenaOverflow;  // another model shrank nothing, but be explicit
+    const MTensor &tin = m->t[m->input];
+    if (input_dev && input_dev != tensor_ptr(m, m->input))
+        ZANT_HIP_TRY(ctx, hipMemcpyAsync(tensor_ptr(m, m->input), input_dev, tin.bytes(), hipMemcpyDeviceToDevice, ctx->stream));
+    for (const MNode &nd : m->n) {
+        if (nd.skip) continue;
+        const int rc = run_node(m, nd);
+        if (rc) return rc;
+    }
+    if (output_dev)
+        ZANT_HIP_TRY(ctx, hipMemcpyAsync(output_dev, tensor_ptr(m, m->output), m->t[m->output].bytes(), hipMemcpyDeviceToDevice,
+                                         ctx->stream));
+    return ZANT_OK;
+}
+
+extern "C" int zant_model_predict_host(zant_model *m, const void *input_host, void *output_host) {
+    if (!m || !input_host || !output_host) return ZANT_NullPointer;
+    if (!m->finalized) return ZANT_NotFinalized;
+    zant_ctx *ctx = m->ctx;
+    int rc = zant_hip_upload(ctx, tensor_ptr(m, m->input), input_host, m->t[m->input].bytes());
+    if (rc) return rc;
+    for (const MNode &nd : m->n) {
+        if (nd.skip) continue;
+        rc = run_node(m, nd);
+        if (rc) return rc;
+    }
+    return zant_hip_download(ctx, output_host, tensor_ptr(m, m->output), m->t[m->output].bytes());
+}
+
+extern "C" int zant_model_read_tensor(zant_model *m, int id, void *dst_host, size_t bytes) {
+    if (!valid_tensor(m, id) || !dst_host) return ZANT_NullPointer;
+    if (!m->finalized) return ZANT_NotFinalized;
+    if (bytes > m->t[id].bytes()) return ZANT_InvalidDimensions;
+    return zant_hip_download(m->ctx, dst_host, tensor_ptr(m, id), bytes);
+}
+
+extern "C" int zant_model_bind_predict(zant_model *m) {
+    if (m && !m->finalized) return ZANT_NotFinalized;
+    g_predict_model = m;
+    return ZANT_OK;
+}
+
+extern "C" void predict(float *input, uint32_t *input_shape, uint32_t shape_len, float **result) {
+    zant_log("Starting prediction...\n");
+    zant_model *m = g_predict_model;
+    if (!m || !input || !input_shape || !result) return;
+    const MTensor &tin = m->t[m->input];
+    if (shape_len == 0) return;                      // src/codeGen/predict.zig:324
+    if (shape_len != uint32_t(tin.rank)) return;     // :325
+    for (int i = 0; i < tin.rank; ++i)
+        if (int64_t(input_shape[i]) != tin.dim[i]) return;  // :329-334
+    if (tin.dtype != ZANT_F32 || m->t[m->output].dtype != ZANT_F32) return;
+    if (zant_model_predict_host(m, input, m->result_host.data()) != ZANT_OK) return;  // `catch return`: result untouched
+    *result = reinterpret_cast<float *>(m->result_host.data());
+    zant_log("Prediction completed.\n");
+}

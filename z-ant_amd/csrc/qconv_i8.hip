@@ -76,28 +76,46 @@ typedef __attribute__((address_space(3))) void *lptr_t;
 constexpr int QCC = 32;  // input channels per chunk = one MFMA k-step per filter tap
 
 // NCHW u8 -> [N][CB][H][W][16] signed (value - 128); channels beyond C are 0 (their weights are 0 too).
+// Each thread turns 4 consecutive positions x 16 channels: sixteen 4-byte loads (one per channel
+// row), a 4x4 byte transpose per group of 4 channels, four 16-byte stores.
 __global__ void __launch_bounds__(256) to_blocked_s8_kernel(const uint8_t *__restrict__ x, uint4 *__restrict__ xb, int N,
-                                                           int C, int CB, int64_t HW) {
-    const int64_t total = int64_t(N) * CB * HW;
+                                                           int C, int CB, int64_t HW, int vec_ok) {
+    const int64_t HW4 = (HW + 3) >> 2;
+    const int64_t total = int64_t(N) * CB * HW4;
     const int64_t step = int64_t(gridDim.x) * blockDim.x;
     for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += step) {
-        const int64_t hw = i % HW;
-        const int cb = int((i / HW) % CB);
-        const int64_t n = i / (HW * CB);
+        const int64_t hw = (i % HW4) << 2;
+        const int cb = int((i / HW4) % CB);
+        const int64_t n = i / (HW4 * CB);
         const uint8_t *src = x + (n * C + int64_t(cb) * 16) * HW + hw;
-        uint32_t w[4];
+        const int valid = int(min(int64_t(4), HW - hw));
+        uint32_t rows[16];  // rows[c] = 4 consecutive positions of channel c
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
+        for (int c = 0; c < 16; ++c) {
             uint32_t v = 0;
-#pragma unroll
-            for (int b = 0; b < 4; ++b) {
-                const int c = cb * 16 + q * 4 + b;
-                const uint32_t byte = c < C ? uint32_t(src[int64_t(q * 4 + b) * HW] ^ 0x80u) : 0u;
-                v |= byte << (8 * b);
+            if (cb * 16 + c < C) {
+                const uint8_t *p = src + int64_t(c) * HW;
+                if (vec_ok && valid == 4) {
+                    v = *reinterpret_cast<const uint32_t *>(p);
+                } else {
+                    for (int b = 0; b < valid; ++b) v |= uint32_t(p[b]) << (8 * b);
+                }
+                v ^= 0x80808080u;
             }
-            w[q] = v;
+            rows[c] = v;
         }
-        xb[i] = make_uint4(w[0], w[1], w[2], w[3]);
+        uint4 *dst = xb + (n * CB + cb) * HW + hw;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            if (b < valid) {
+                uint32_t o[4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    o[q] = ((rows[q * 4 + 0] >> (8 * b)) & 0xff) | (((rows[q * 4 + 1] >> (8 * b)) & 0xff) << 8) |
+                           (((rows[q * 4 + 2] >> (8 * b)) & 0xff) << 16) | (((rows[q * 4 + 3] >> (8 * b)) & 0xff) << 24);
+                dst[b] = make_uint4(o[0], o[1], o[2], o[3]);
+            }
+        }
     }
 }
 
@@ -125,16 +143,25 @@ qpack_kernel(const int8_t *__restrict__ w, const float *__restrict__ w_scale, co
         const int k = kb * k_blk + kk, c = chunk * QCC + half * 16 + j;
         wp[i] = (k < K && c < C) ? w[(int64_t(k) * C + c) * T + tap] : int8_t(0);
     }
+    // per output channel: one wavefront sums the channel's weights
     const int kpad = n_kblocks * k_blk;
-    for (int64_t k = gid; k < kpad; k += step) {
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = gid >> 6, n_waves = step >> 6;
+    for (int64_t k = wave; k < kpad; k += n_waves) {
+        int sum = 0;
         if (k < K) {
-            int sum = 0;
-            for (int e = 0; e < C * T; ++e) sum += int(w[k * C * T + e]);
-            corr[k] = (bias ? bias[k] : 0) + (128 - x_zp) * sum;
-            mult[k] = (x_scale * w_scale[n_wscale == 1 ? 0 : k]) / y_scale;
-        } else {
-            corr[k] = 0;
-            mult[k] = 0.0f;
+            const int8_t *wk = w + k * int64_t(C) * T;
+            for (int e = lane; e < C * T; e += 64) sum += int(wk[e]);
+        }
+        for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+        if (lane == 0) {
+            if (k < K) {
+                corr[k] = (bias ? bias[k] : 0) + (128 - x_zp) * sum;
+                mult[k] = (x_scale * w_scale[n_wscale == 1 ? 0 : k]) / y_scale;
+            } else {
+                corr[k] = 0;
+                mult[k] = 0.0f;
+            }
         }
     }
 }
@@ -438,15 +465,17 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
     int8_t *wp = reinterpret_cast<int8_t *>(base + o_wp);
     int8_t *xb = reinterpret_cast<int8_t *>(base + o_xb);
     const int grid = int(std::min<int64_t>(plan.t.n_tiles, int64_t(ctx->num_cus) * 2));
-    const unsigned pb = unsigned(std::min<int64_t>(ceil_div64(int64_t(wp_bytes), 256), 1024));
+    const unsigned pb = unsigned(std::min<int64_t>(std::max<int64_t>(ceil_div64(int64_t(wp_bytes), 256), ceil_div64(int64_t(kpad), 4)), 1024));
     hipLaunchKernelGGL(qpack_kernel, dim3(pb), dim3(256), 0, ctx->stream, w, w_scale, bias, wp, mult, corr, padvec, counter,
                        2 * grid, g.K, g.C, T, plan.t.n_chunks, plan.t.n_kblocks, K_BLK, q.x_scale, q.y_scale, q.x_zp,
                        q.n_wscale);
     ZANT_LAUNCH_CHECK(ctx);
-    const int64_t units = int64_t(g.N) * CB * g.H * g.W;
+    const int64_t hw = int64_t(g.H) * g.W;
+    const int64_t units = int64_t(g.N) * CB * ((hw + 3) / 4);
     const unsigned tb = unsigned(std::min<int64_t>(ceil_div64(units, 256), int64_t(ctx->num_cus) * 16));
+    const int vec_ok = (hw % 4 == 0) && (reinterpret_cast<uintptr_t>(x) % 4 == 0);
     hipLaunchKernelGGL(to_blocked_s8_kernel, dim3(tb), dim3(256), 0, ctx->stream, x, reinterpret_cast<uint4 *>(xb), g.N, g.C,
-                       CB, int64_t(g.H) * g.W);
+                       CB, hw, vec_ok);
     ZANT_LAUNCH_CHECK(ctx);
     KernelTimer kt(ctx);
     const bool ok = WN == 2 ? dispatch_qmt<2, 2>(ctx, xb, wp, mult, corr, padvec, y, g, plan, CB, q, counter, grid)
