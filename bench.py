@@ -63,14 +63,15 @@ def main():
     dev = torch.device("cuda:0")
     ctx = tm.context()
     params = networks.readme_cnn_params(seed=0)
-    net = networks.ReadmeCNN(BATCH, params, dev)
+    model = networks.build_readme_cnn_model(ctx, BATCH, params)  # what is timed: one zant_model_run per step
     g = np.random.default_rng(1)
     x_host = g.random((BATCH, 1, 28, 28), dtype=np.float32)  # ~U[0,1)
-    x = torch.from_numpy(x_host).to(dev)
+    ctx.check(za.lib.zant_hip_upload(ctx.handle, model.input_ptr, x_host.ctypes.data, x_host.nbytes))  # resident input
 
     # ---- parity gate on the first images of the batch (the oracle is only the checker) ----
-    out = net.forward(x)
-    torch.cuda.synchronize()
+    model.run()
+    out_host = np.zeros((BATCH, 10), np.float32)
+    ctx.check(za.lib.zant_hip_download(ctx.handle, out_host.ctypes.data, model.output_ptr, out_host.nbytes))
     from oracle import oracle as zo
 
     def oracle_forward(img):
@@ -83,55 +84,44 @@ def main():
         return zo.softmax(y.reshape(1, 10))
 
     ref = np.concatenate([oracle_forward(x_host[i:i + 1]) for i in (0, 1, 2, BATCH - 1)])
-    got = out[[0, 1, 2, BATCH - 1]].cpu().numpy()
-    np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(out_host[[0, 1, 2, BATCH - 1]], ref, rtol=1e-4, atol=1e-5)
 
     # ---- timed region: W warm-up steps, then exactly K steps between synchronisations ----
     for _ in range(args.warmup):
-        net.forward(x)
+        model.run()
     ctx.sync()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     ctx.timer_start()
     for _ in range(args.steps):
-        net.forward(x)
+        model.run()
     ev_ms = ctx.timer_stop()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
     ms_per_step = max(ev_ms, wall_ms) / args.steps  # the host clock includes the final synchronisation
     value = BATCH / (ms_per_step * 1e-3)
 
-    # ---- per-kernel durations of the pass (HIP events around each main kernel) ----
-    p = net.p
+    # ---- per-kernel durations of the pass: HIP events around the main kernel of every launching node ----
     flops = networks.readme_cnn_flops_per_inference()
-    flat = net.p2.view(1, 1, BATCH, 1600)
     kit = max(5, min(args.steps, 20))
-    kernels = {
-        "conv1+relu": (lambda: tm.conv_lean(x, p["w1"], net.a1, p["b1"], [1, 1], None, None, 1, None, "relu"),
-                       "hbm", (x.numel() + net.a1.numel()) * 4),
-        "maxpool1": (lambda: tm.onnx_maxpool_lean(net.a1, net.p1, [2, 2], [2, 2], [1, 1], [0, 0, 0, 0]),
-                     "hbm", (net.a1.numel() + net.p1.numel()) * 4),
-        "conv2+relu": (lambda: tm.conv_lean(net.p1, p["w2"], net.a2, p["b2"], [1, 1], None, None, 1, None, "relu"),
-                       "mfma", flops["conv2"] * BATCH),
-        "maxpool2": (lambda: tm.onnx_maxpool_lean(net.a2, net.p2, [2, 2], [2, 2], [1, 1], [0, 0, 0, 0]),
-                     "hbm", (net.a2.numel() + net.p2.numel()) * 4),
-        "gemm1+relu": (lambda: tm.gemm_lean(flat, p["g1"], p["c1"], 1.0, 1.0, False, False, net.h1, "relu"),
-                       "mfma", flops["gemm1"] * BATCH),
-        "gemm2": (lambda: tm.gemm_lean(net.h1, p["g2"], p["c2"], 1.0, 1.0, False, False, net.h2),
-                  "mfma", flops["gemm2"] * BATCH),
-        "softmax": (lambda: tm.softmax_lean(net.h2.view(BATCH, 10), net.out), "hbm", 2 * BATCH * 10 * 4),
-    }
+    acc = None
+    for _ in range(kit):
+        prof = model.profile()
+        acc = prof if acc is None else [(n, a[1] + p[1], o, b) for a, p, (n, _, o, b) in zip(acc, prof, prof)]
     per_kernel = {}
-    for name, (fn, bound, work) in kernels.items():
-        ms = kernel_avg_ms(ctx, fn, kit)
-        if bound == "mfma":
-            ach = work / (ms * 1e-3) / 1e12
-            per_kernel[name] = {"ms": round(ms, 4), "bound": "mfma", "achieved_tflops": round(ach, 2),
-                                "frac": round(ach / PEAK_F32_MFMA_TFLOPS, 4)}
+    for i, (name, ms_sum, ops, nbytes) in enumerate(acc):
+        ms = ms_sum / kit
+        key = f"{i}:{name}"
+        # the roofline that bounds each node: arithmetic intensity against the f32 MFMA / HBM ridge (157.3 TF / 8 TB/s)
+        mfma_bound = ops > 0 and ops / nbytes > PEAK_F32_MFMA_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9)
+        if mfma_bound:
+            ach = ops / (ms * 1e-3) / 1e12
+            per_kernel[key] = {"ms": round(ms, 4), "bound": "mfma", "achieved_tflops": round(ach, 2),
+                               "frac": round(ach / PEAK_F32_MFMA_TFLOPS, 4), "flop": ops, "bytes": nbytes}
         else:
-            ach = work / (ms * 1e-3) / 1e9
-            per_kernel[name] = {"ms": round(ms, 4), "bound": "hbm", "achieved_gbs": round(ach, 1),
-                                "frac": round(ach / PEAK_HBM_GBS, 4)}
+            ach = nbytes / (ms * 1e-3) / 1e9
+            per_kernel[key] = {"ms": round(ms, 4), "bound": "hbm", "achieved_gbs": round(ach, 1),
+                               "frac": round(ach / PEAK_HBM_GBS, 4), "flop": ops, "bytes": nbytes}
     dominant = max(per_kernel, key=lambda k: per_kernel[k]["ms"])
     dk = per_kernel[dominant]
     if dk["bound"] == "mfma":
@@ -196,7 +186,8 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "config 1: README f32 CNN (Conv32-ReLU-Pool-Conv64-ReLU-Pool-Gemm512-ReLU-Gemm10-Softmax), "
                                "input 4096x1x28x28 ~U[0,1), He-normal weights, seed 0", "batch": BATCH,
-                   "flop_per_inference": flops["total"],
+                   "flop_per_inference": flops["total"], "launches_per_step": model.num_launches,
+                   "arena_bytes": model.arena_bytes, "unfused_activation_bytes": model.unfused_bytes,
                    "tflops": round(flops["total"] * BATCH / (ms_per_step * 1e-3) / 1e12, 2)},
         "roofline": roofline,
         "cpu_baseline": cpu,

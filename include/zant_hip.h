@@ -254,6 +254,13 @@ void *zant_model_input_ptr(zant_model *m);
 void *zant_model_output_ptr(zant_model *m);
 /* Host in / host out: upload, run, download (synchronous). */
 int zant_model_predict_host(zant_model *m, const void *input_host, void *output_host);
+/* One pass with per-kernel timing: fills, for each kernel-launching node in execution order, the
+ * duration of its main kernel (ms), its algorithmic work (flops or integer ops; 0 for data movement)
+ * and its algorithmic bytes (inputs + parameters + output, each once).  Returns the number of entries
+ * written (at most `capacity`) or a negative status.  zant_model_launch_name() names entry i, e.g.
+ * "Conv+Relu+MaxPool". */
+int zant_model_profile(zant_model *m, float *ms, double *ops, double *bytes, int capacity);
+const char *zant_model_launch_name(zant_model *m, int i);
 /* Debug: copies tensor `id` (as planned in the arena) to the host after a run. */
 int zant_model_read_tensor(zant_model *m, int id, void *dst_host, size_t bytes);
 

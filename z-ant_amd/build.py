@@ -27,8 +27,18 @@ def sources():
     return sorted(glob.glob(os.path.join(CSRC, "*.hip")))
 
 
+HOST_TEST = os.path.join(HERE, "host", "test_host_mirror")
+
+
 def build(verbose=True):
     cmd = [HIPCC] + FLAGS + sources() + ["-o", LIB]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    # the C++ host mirror of the reference's operator interface: plain g++ over the C ABI (no HIP headers)
+    cmd = ["g++", "-std=c++17", "-O1", "-Wall", "-I", os.path.join(ROOT, "include"),
+           os.path.join(HERE, "host", "test_host_mirror.cpp"), "-o", HOST_TEST, "-L", HERE, "-lzant_hip",
+           "-Wl,-rpath,$ORIGIN/.."]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)

@@ -89,6 +89,8 @@ PROTOTYPES = {
     "zant_model_input_ptr": (vp, [vp]),
     "zant_model_output_ptr": (vp, [vp]),
     "zant_model_predict_host": (i32, [vp, vp, vp]),
+    "zant_model_profile": (i32, [vp, C.POINTER(f32), C.POINTER(C.c_double), C.POINTER(C.c_double), i32]),
+    "zant_model_launch_name": (C.c_char_p, [vp, i32]),
     "zant_model_read_tensor": (i32, [vp, i32, vp, sz]),
     "zant_model_bind_predict": (i32, [vp]),
     "predict": (None, [vp, C.POINTER(C.c_uint32), C.c_uint32, C.POINTER(vp)]),

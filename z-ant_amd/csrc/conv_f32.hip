@@ -385,6 +385,58 @@ __global__ void __launch_bounds__(256) conv_f32_smallc_kernel(const float *__res
     }
 }
 
+// Few-input-channel convolution fused with ReLU and a 2x2 / stride-2 max pool (stride-1, undilated
+// convolution).  One thread owns one POOLED position: it keeps the (KH+1) x (KW+1) input patch of each
+// channel in registers, forms the four convolution outputs of the pooling window for every output
+// channel, and writes only their (ReLU'd) maximum: the full-resolution activation never reaches HBM.
+template <int C, int KH, int KW>
+__global__ void __launch_bounds__(256)
+conv_f32_smallc_pool_kernel(const float *__restrict__ x, const float *__restrict__ w, const float *__restrict__ bias,
+                            float *__restrict__ y, ConvGeom g, int POH, int POW, int relu) {
+    constexpr int PH = KH + 1, PW = KW + 1, CKK = C * KH * KW;
+    const int64_t pplane = int64_t(POH) * POW;
+    const int64_t total = int64_t(g.N) * pplane;
+    const int64_t step = int64_t(gridDim.x) * blockDim.x;
+    for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += step) {
+        const int n = int(i / pplane);
+        const int pos = int(i - int64_t(n) * pplane);
+        const int ph = pos / POW, pw = pos - ph * POW;
+        const int ih0 = 2 * ph - g.pt, iw0 = 2 * pw - g.pl;
+        float patch[C][PH][PW];
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+#pragma unroll
+            for (int r = 0; r < PH; ++r)
+#pragma unroll
+                for (int q = 0; q < PW; ++q) {
+                    const int ih = ih0 + r, iw = iw0 + q;
+                    const bool ok = ih >= 0 && ih < g.H && iw >= 0 && iw < g.W;
+                    patch[c][r][q] = ok ? x[((int64_t(n) * C + c) * g.H + ih) * g.W + iw] : 0.0f;
+                }
+        float *yp = y + int64_t(n) * g.K * pplane + pos;
+        for (int k = 0; k < g.K; ++k) {
+            const float *wk = w + int64_t(k) * CKK;
+            float a00 = 0.f, a01 = 0.f, a10 = 0.f, a11 = 0.f;
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+#pragma unroll
+                for (int kh = 0; kh < KH; ++kh)
+#pragma unroll
+                    for (int kw = 0; kw < KW; ++kw) {
+                        const float wv = wk[(c * KH + kh) * KW + kw];
+                        a00 = __builtin_fmaf(patch[c][kh][kw], wv, a00);
+                        a01 = __builtin_fmaf(patch[c][kh][kw + 1], wv, a01);
+                        a10 = __builtin_fmaf(patch[c][kh + 1][kw], wv, a10);
+                        a11 = __builtin_fmaf(patch[c][kh + 1][kw + 1], wv, a11);
+                    }
+            const float b = bias ? bias[k] : 0.0f;
+            float r = fmaxf(fmaxf(a00 + b, a01 + b), fmaxf(a10 + b, a11 + b));
+            if (relu) r = r > 0.0f ? r : 0.0f;  // max and ReLU commute (both monotone)
+            yp[int64_t(k) * pplane] = r;
+        }
+    }
+}
+
 typedef TilePlan MfmaPlan;
 
 // Tile shape with the best useful-lane fraction whose LDS footprint allows two workgroups per CU.
@@ -581,5 +633,36 @@ extern "C" int zant_hip_conv2d_f32(zant_ctx *ctx, const float *x, const int64_t 
     hipLaunchKernelGGL(conv_f32_direct_kernel, dim3(unsigned(blocks)), dim3(256), 0, ctx->stream, x, w, bias, y, g, relu);
     ZANT_LAUNCH_CHECK(ctx);
     zant_log("OnnxConvLean4");
+    return ZANT_OK;
+}
+
+// Conv (+ReLU) + MaxPool 2x2/2 in one kernel for few-channel first layers; returns 1 when the shape is
+// not one this kernel takes (the caller then runs the two operators separately).
+int zant_conv2d_f32_fused_pool(zant_ctx *ctx, const float *x, const int64_t xdim[4], const float *w, const int64_t wdim[4],
+                               const float *bias, float *y, const int64_t ydim[4], const int64_t *stride, int n_stride,
+                               const int64_t *pads, int n_pads, const int64_t *dil, int n_dil, int64_t group,
+                               const char *auto_pad, int relu, bool query_only) {
+    int64_t s[2], d[2], p[4];
+    if (zant_conv_resolve(xdim, wdim, stride, n_stride, pads, n_pads, dil, n_dil, group, auto_pad, s, d, p)) return 1;
+    if (s[0] != 1 || s[1] != 1 || d[0] != 1 || d[1] != 1 || xdim[1] != wdim[1]) return 1;
+    const int C = int(wdim[1]), KH = int(wdim[2]), KW = int(wdim[3]);
+    const bool k133 = C == 1 && KH == 3 && KW == 3, k155 = C == 1 && KH == 5 && KW == 5, k333 = C == 3 && KH == 3 && KW == 3;
+    if (!k133 && !k155 && !k333) return 1;
+    const int64_t OH = xdim[2] + p[0] + p[2] - KH + 1, OW = xdim[3] + p[1] + p[3] - KW + 1;
+    if (OH < 2 || OW < 2) return 1;
+    if (ydim[0] != xdim[0] || ydim[1] != wdim[0] || ydim[2] != OH / 2 || ydim[3] != OW / 2) return 1;
+    if (query_only) return ZANT_OK;
+    ConvGeom g;
+    g.N = int(xdim[0]); g.C = C; g.H = int(xdim[2]); g.W = int(xdim[3]);
+    g.K = int(wdim[0]); g.CG = C; g.KH = KH; g.KW = KW; g.OH = int(OH); g.OW = int(OW);
+    g.sh = g.sw = g.dh = g.dw = 1; g.pt = int(p[0]); g.pl = int(p[1]); g.groups = 1;
+    const int POH = int(OH / 2), POW = int(OW / 2);
+    const int64_t positions = int64_t(g.N) * POH * POW;
+    const unsigned pb = unsigned(std::min<int64_t>(ceil_div64(positions, 256), int64_t(ctx->num_cus) * 16));
+    KernelTimer kt(ctx);
+    if (k133) hipLaunchKernelGGL((conv_f32_smallc_pool_kernel<1, 3, 3>), dim3(pb), dim3(256), 0, ctx->stream, x, w, bias, y, g, POH, POW, relu);
+    else if (k155) hipLaunchKernelGGL((conv_f32_smallc_pool_kernel<1, 5, 5>), dim3(pb), dim3(256), 0, ctx->stream, x, w, bias, y, g, POH, POW, relu);
+    else hipLaunchKernelGGL((conv_f32_smallc_pool_kernel<3, 3, 3>), dim3(pb), dim3(256), 0, ctx->stream, x, w, bias, y, g, POH, POW, relu);
+    ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
 }

@@ -74,7 +74,7 @@ inline bool zant_plan_conv_tiles(const ConvGeom &g, int WM, int WN, int mt_max, 
                            + size_t(t.P1s) * 8 + 8;                          // patch table, scheduler slots
         if (lds > lds_cap) continue;
         const double eff = double(g.N) * g.OH * g.OW / (double(t.n_sblocks) * S);
-        if (!found || eff > best->eff + 1e-9) {
+        if (!found || eff > best->eff + 0.01) {  // larger tiles win ties: fewer tiles, more operand reuse
             best->MT = mt; best->WM = WM; best->WN = WN; best->t = t; best->lds_bytes = lds; best->eff = eff;
             found = true;
         }

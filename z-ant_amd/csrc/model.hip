@@ -51,6 +51,7 @@ struct MNode {
     int in0 = -1, in1 = -1, out = -1;
     bool skip = false;            // fused into its producer or turned into a view
     int fuse_act = ZANT_ACT_NONE; // activation applied in this node's epilogue
+    bool fuse_pool = false;       // a following 2x2/2 MaxPool is computed in this node's kernel
     float act_alpha = 0.0f, act_scale = 1.0f;
     int act_zp = 0;
     int w = -1, b = -1, c = -1, ws = -1;  // parameter indices
@@ -148,6 +149,13 @@ int run_node(zant_model *m, const MNode &nd) {
     void *y = tensor_ptr(m, nd.out);
     switch (nd.op) {
     case OP_CONV:
+        if (nd.fuse_pool)
+            return zant_conv2d_f32_fused_pool(ctx, static_cast<const float *>(x), ti.dim,
+                                              static_cast<const float *>(param_ptr(m, nd.w)), nd.wdim,
+                                              static_cast<const float *>(param_ptr(m, nd.b)), static_cast<float *>(y), to.dim,
+                                              nd.stride, nd.n_stride, nd.has_pads ? nd.pads : nullptr, nd.n_pads,
+                                              nd.has_dil ? nd.dil : nullptr, nd.n_dil, nd.group,
+                                              nd.has_auto_pad ? nd.auto_pad.c_str() : nullptr, nd.fuse_act == ZANT_ACT_RELU, false);
         return zant_hip_conv2d_f32(ctx, static_cast<const float *>(x), ti.dim, static_cast<const float *>(param_ptr(m, nd.w)),
                                    nd.wdim, static_cast<const float *>(param_ptr(m, nd.b)), static_cast<float *>(y), to.dim,
                                    nd.stride, nd.n_stride, nd.has_pads ? nd.pads : nullptr, nd.n_pads,
@@ -480,6 +488,8 @@ extern "C" int zant_model_finalize(zant_model *m) {
     zant_ctx *ctx = m->ctx;
     const int nn = int(m->n.size());
     m->output = m->n.back().out;
+    m->unfused_bytes = 0;  // what one static array per node output (the reference's layout) would take
+    for (const MNode &nd : m->n) m->unfused_bytes += m->t[nd.out].bytes();
 
     // ---- peephole fusions -----------------------------------------------------------------------
     for (int i = 0; i < nn; ++i) {
@@ -517,6 +527,32 @@ extern "C" int zant_model_finalize(zant_model *m) {
                 m->n[only].skip = true;
             }
         }
+        if (nd.op == OP_CONV) {
+            // Conv (+ReLU) -> MaxPool 2x2/2 on a few-channel first layer: one kernel, pooled output only
+            int out = nd.out, c1 = -1;
+            while (consumers(m, out, &c1) == 1 && m->n[c1].skip && (m->n[c1].op == OP_ADD_CONST || m->n[c1].op == OP_RELU))
+                out = m->n[c1].out;
+            if (consumers(m, out, &only) == 1 && m->n[only].op == OP_MAXPOOL && !m->n[only].skip) {
+                MNode &pn = m->n[only];
+                const bool pool22 = pn.kernel[0] == 2 && pn.kernel[1] == 2 && pn.stride[0] == 2 && pn.stride[1] == 2 &&
+                                    pn.dil[0] == 1 && pn.dil[1] == 1 && pn.pads[0] == 0 && pn.pads[1] == 0 && pn.pads[2] == 0 &&
+                                    pn.pads[3] == 0 && (pn.pool_pad == ZANT_PAD_NOTSET || pn.pool_pad == ZANT_PAD_VALID);
+                const MTensor &tp = m->t[pn.out];
+                if (pool22 && m->t[nd.in0].dtype == ZANT_F32 &&
+                    zant_conv2d_f32_fused_pool(ctx, nullptr, m->t[nd.in0].dim, nullptr, nd.wdim, nullptr, nullptr, tp.dim, nd.stride,
+                                               nd.n_stride, nd.has_pads ? nd.pads : nullptr, nd.n_pads,
+                                               nd.has_dil ? nd.dil : nullptr, nd.n_dil, nd.group,
+                                               nd.has_auto_pad ? nd.auto_pad.c_str() : nullptr, 0, true) == ZANT_OK) {
+                    // the conv node now produces the pool's tensor; the intermediate tensors are never materialised
+                    nd.fuse_pool = true;
+                    const int conv_out = nd.out;
+                    nd.out = pn.out;
+                    pn.skip = true;
+                    pn.out = conv_out;  // keeps every tensor id owned by exactly one node
+                    pn.in0 = conv_out;
+                }
+            }
+        }
         if (nd.op == OP_QCONV && nd.fuse_act == ZANT_ACT_NONE && consumers(m, nd.out, &only) == 1 &&
             m->n[only].op == OP_QACT && !m->n[only].skip) {
             // the activation's output parameters become the kernel's second requantisation stage
@@ -539,12 +575,11 @@ extern "C" int zant_model_finalize(zant_model *m) {
     const int nt = int(m->t.size());
     for (int i = 0; i < nt; ++i) { m->t[i].def = -1; m->t[i].last = -1; }
     m->t[root_of(m, m->input)].def = 0;
-    m->unfused_bytes = 0;
     m->launches = 0;
     for (int i = 0; i < nn; ++i) {
         const MNode &nd = m->n[i];
-        m->unfused_bytes += m->t[nd.out].bytes();
-        if (!nd.skip) ++m->launches;
+        if (nd.skip) continue;  // fused away: its tensors are views of live ones or are never materialised
+        ++m->launches;
         const int ro = root_of(m, nd.out);
         if (m->t[ro].def < 0) m->t[ro].def = i + 1;
         for (int in : {nd.in0, nd.in1})
@@ -646,6 +681,105 @@ extern "C" int zant_model_predict_host(zant_model *m, const void *input_host, vo
         if (rc) return rc;
     }
     return zant_hip_download(ctx, output_host, tensor_ptr(m, m->output), m->t[m->output].bytes());
+}
+
+namespace {
+
+const char *op_name(const MNode &nd) {
+    switch (nd.op) {
+    case OP_CONV:
+        if (nd.fuse_pool) return nd.fuse_act ? "Conv+Relu+MaxPool" : "Conv+MaxPool";
+        return nd.fuse_act ? "Conv+Relu" : "Conv";
+    case OP_RELU: return "Relu";
+    case OP_LEAKY: return "LeakyRelu";
+    case OP_MAXPOOL: return "MaxPool";
+    case OP_RESHAPE: return "Reshape";
+    case OP_GEMM: return nd.fuse_act ? "Gemm+Relu" : "Gemm";
+    case OP_MATMUL: return "MatMul";
+    case OP_ADD_CONST: return "Add(const)";
+    case OP_ADD: return "Add";
+    case OP_SOFTMAX: return "Softmax";
+    case OP_QUANT: return "QuantizeLinear";
+    case OP_DEQUANT: return "DequantizeLinear";
+    case OP_QCONV:
+        if (nd.group > 1) return nd.fuse_act ? "QLinearConv(depthwise)+Act" : "QLinearConv(depthwise)";
+        return nd.fuse_act ? "QLinearConv+Act" : "QLinearConv";
+    case OP_QACT: return "QLinearAct";
+    case OP_QADD: return "QLinearAdd";
+    case OP_QGAP: return "QLinearGlobalAveragePool";
+    default: return "?";
+    }
+}
+
+void node_work(const zant_model *m, const MNode &nd, double *ops, double *bytes) {
+    const MTensor &ti = m->t[nd.in0];
+    const MTensor &to = m->t[nd.out];
+    double b = double(ti.bytes()) + double(to.bytes());
+    if (nd.in1 >= 0) b += double(m->t[nd.in1].bytes());
+    double o = 0.0;
+    switch (nd.op) {
+    case OP_CONV:
+    case OP_QCONV: {
+        // ops count the convolution's own output (before any fused pooling)
+        double outs = double(to.bytes()) / (nd.op == OP_CONV ? 4.0 : 1.0);
+        if (nd.fuse_pool) outs *= 4.0;
+        o = 2.0 * outs * double(nd.wdim[1] * nd.wdim[2] * nd.wdim[3]);
+        b += double(nd.wdim[0] * nd.wdim[1] * nd.wdim[2] * nd.wdim[3]) * (nd.op == OP_CONV ? 4.0 : 1.0);
+        break;
+    }
+    case OP_GEMM: {
+        const double K = double(nd.trans_a ? ti.dim[2] : ti.dim[3]);
+        o = 2.0 * double(to.dim[2]) * double(to.dim[3]) * K;
+        b += double(nd.wdim[2] * nd.wdim[3]) * 4.0;
+        break;
+    }
+    case OP_MATMUL: {
+        const double K = double(ti.dim[ti.rank - 1]);
+        o = 2.0 * double(to.dim[to.rank - 2]) * double(to.dim[to.rank - 1]) * K;
+        b += double(nd.bdim[nd.b_rank - 2] * nd.bdim[nd.b_rank - 1]) * 4.0;
+        break;
+    }
+    default: break;
+    }
+    *ops = o;
+    *bytes = b;
+}
+
+}  // namespace
+
+extern "C" int zant_model_profile(zant_model *m, float *ms, double *ops, double *bytes, int capacity) {
+    if (!m || !ms) return ZANT_NullPointer;
+    if (!m->finalized) return ZANT_NotFinalized;
+    zant_ctx *ctx = m->ctx;
+    const bool was = ctx->kernel_timing;
+    ctx->kernel_timing = true;
+    int cnt = 0, rc = ZANT_OK;
+    for (const MNode &nd : m->n) {
+        if (nd.skip) continue;
+        rc = run_node(m, nd);
+        if (rc) break;
+        if (cnt < capacity) {
+            rc = zant_hip_kernel_ms(ctx, &ms[cnt]);
+            if (rc) break;
+            double o = 0, b = 0;
+            node_work(m, nd, &o, &b);
+            if (ops) ops[cnt] = o;
+            if (bytes) bytes[cnt] = b;
+            ++cnt;
+        }
+    }
+    ctx->kernel_timing = was;
+    return rc ? rc : cnt;
+}
+
+extern "C" const char *zant_model_launch_name(zant_model *m, int i) {
+    if (!m) return "";
+    int cnt = 0;
+    for (const MNode &nd : m->n) {
+        if (nd.skip) continue;
+        if (cnt++ == i) return op_name(nd);
+    }
+    return "";
 }
 
 extern "C" int zant_model_read_tensor(zant_model *m, int id, void *dst_host, size_t bytes) {

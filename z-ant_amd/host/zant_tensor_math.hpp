@@ -1,0 +1,252 @@
+// Host-side C++ mirror of the reference's operator interface over the C ABI of libzant_hip.so.
+//
+// The reference is Zig: `Tensor(T)` (src/Core/Tensor/tensor.zig:25-31) and the `tensMath` facade
+// (src/Core/Tensor/TensorMath/tensor_math_standard.zig:43-149) whose operators come in a lean form
+// (caller supplies a pre-shaped output, returns an error union) and a standard form (validates,
+// allocates the output, calls the lean form).  This header keeps those names, argument order and
+// error behaviour; a Zig error becomes a thrown zant::Error whose code() is the zant_status.
+// Tensor data lives on the GPU; optional arguments are pointers / std::optional (null = Zig null).
+#pragma once
+#include <cstdint>
+#include <optional>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "zant_hip.h"
+
+namespace zant {
+
+class Error : public std::runtime_error {
+  public:
+    explicit Error(int code) : std::runtime_error(zant_hip_status_name(code)), code_(code) {}
+    int code() const { return code_; }
+
+  private:
+    int code_;
+};
+
+inline void check(int rc) {
+    if (rc != ZANT_OK) throw Error(rc);
+}
+
+// One context per thread, like one generated library instance.
+inline zant_ctx *&default_ctx() {
+    static zant_ctx *ctx = nullptr;
+    if (!ctx) check(zant_hip_ctx_create(&ctx, 0, nullptr));
+    return ctx;
+}
+
+// Tensor(T): data (device), size, shape, owns_memory -- tensor.zig:25-31.
+template <typename T>
+struct Tensor {
+    T *data = nullptr;
+    size_t size = 0;
+    std::vector<int64_t> shape;
+    bool owns_memory = false;
+
+    Tensor() = default;
+    Tensor(const Tensor &) = delete;
+    Tensor &operator=(const Tensor &) = delete;
+    Tensor(Tensor &&o) noexcept { *this = std::move(o); }
+    Tensor &operator=(Tensor &&o) noexcept {
+        deinit();
+        data = o.data; size = o.size; shape = std::move(o.shape); owns_memory = o.owns_memory;
+        o.data = nullptr; o.size = 0; o.owns_memory = false;
+        return *this;
+    }
+    ~Tensor() { deinit(); }
+
+    // fromShape: zero filled (tensor.zig:116-130)
+    static Tensor fromShape(const std::vector<int64_t> &shape) {
+        Tensor t;
+        t.shape = shape;
+        t.size = 1;
+        for (int64_t d : shape) t.size *= size_t(d);
+        void *p = nullptr;
+        check(zant_hip_malloc(default_ctx(), &p, t.size * sizeof(T)));
+        t.data = static_cast<T *>(p);
+        t.owns_memory = true;
+        check(zant_hip_memset(default_ctx(), t.data, 0, t.size * sizeof(T)));
+        return t;
+    }
+    // fromArray: copies host data (tensor.zig:63-100)
+    static Tensor fromArray(const T *host, const std::vector<int64_t> &shape) {
+        Tensor t = fromShape(shape);
+        check(zant_hip_upload(default_ctx(), t.data, host, t.size * sizeof(T)));
+        return t;
+    }
+    // fromConstBuffer: borrows device memory, e.g. a slice of the arena (tensor.zig:142-150)
+    static Tensor fromConstBuffer(T *device_data, const std::vector<int64_t> &shape) {
+        Tensor t;
+        t.shape = shape;
+        t.size = 1;
+        for (int64_t d : shape) t.size *= size_t(d);
+        t.data = device_data;
+        t.owns_memory = false;
+        return t;
+    }
+    std::vector<T> toHost() const {
+        std::vector<T> h(size);
+        check(zant_hip_download(default_ctx(), h.data(), data, size * sizeof(T)));
+        return h;
+    }
+    void deinit() {
+        if (owns_memory && data) (void)zant_hip_free(default_ctx(), data);
+        data = nullptr;
+        owns_memory = false;
+    }
+};
+
+enum class AutoPadType { NOTSET = 0, SAME_UPPER = 1, SAME_LOWER = 2, VALID = 3 };  // op_pooling.zig:9-14
+
+namespace tensMath {
+
+using Dims = std::vector<int64_t>;
+
+// conv_lean = OnnxConvLean (op_convolution.zig:42)
+inline void conv_lean(Tensor<float> *input, Tensor<float> *kernel, Tensor<float> *output, const Tensor<float> *bias,
+                      const Dims &stride, const Dims *pads, const Dims *dilations, std::optional<int64_t> group,
+                      const char *auto_pad) {
+    if (input->shape.size() != 4 || kernel->shape.size() != 4) throw Error(ZANT_InvalidDimensions);
+    check(zant_hip_conv2d_f32(default_ctx(), input->data, input->shape.data(), kernel->data, kernel->shape.data(),
+                              bias ? bias->data : nullptr, output->data, output->shape.data(), stride.data(),
+                              int(stride.size()), pads ? pads->data() : nullptr, pads ? int(pads->size()) : 0,
+                              dilations ? dilations->data() : nullptr, dilations ? int(dilations->size()) : 0,
+                              group ? *group : -1, auto_pad, ZANT_ACT_NONE));
+}
+
+// Conv = OnnxConv (op_convolution.zig:647)
+inline Tensor<float> Conv(Tensor<float> *input, Tensor<float> *kernel, const Tensor<float> *bias, const Dims &stride,
+                          const Dims *pads, const Dims *dilations, std::optional<int64_t> group, const char *auto_pad) {
+    if (input->shape.size() != 4 || kernel->shape.size() != 4) throw Error(ZANT_InvalidDimensions);
+    int64_t ydim[4];
+    check(zant_hip_conv2d_out_shape(input->shape.data(), kernel->shape.data(), stride.data(), int(stride.size()),
+                                    pads ? pads->data() : nullptr, pads ? int(pads->size()) : 0,
+                                    dilations ? dilations->data() : nullptr, dilations ? int(dilations->size()) : 0,
+                                    group ? *group : -1, auto_pad, ydim));
+    Tensor<float> out = Tensor<float>::fromShape({ydim[0], ydim[1], ydim[2], ydim[3]});
+    conv_lean(input, kernel, &out, bias, stride, pads, dilations, group, auto_pad);
+    return out;
+}
+
+// mat_mul_lean / mat_mul (op_mat_mul.zig:92, :22)
+inline void mat_mul_lean(const Tensor<float> *A, const Tensor<float> *B, Tensor<float> *Y) {
+    check(zant_hip_matmul_f32(default_ctx(), A->data, A->shape.data(), int(A->shape.size()), B->data, B->shape.data(),
+                              int(B->shape.size()), Y->data));
+}
+inline Tensor<float> mat_mul(const Tensor<float> *A, const Tensor<float> *B) {
+    check(zant_hip_matmul_check(A->shape.data(), int(A->shape.size()), B->shape.data(), int(B->shape.size())));
+    Dims out = A->shape;
+    out[out.size() - 1] = B->shape.back();
+    Tensor<float> Y = Tensor<float>::fromShape(out);
+    mat_mul_lean(A, B, &Y);
+    return Y;
+}
+
+// gemm_lean / gemm (op_gemm.zig:91, :15)
+inline void gemm_lean(Tensor<float> *A, Tensor<float> *B, Tensor<float> *C, float alpha, float beta, bool transA,
+                      bool transB, Tensor<float> *result) {
+    check(zant_hip_gemm_f32(default_ctx(), A->data, A->shape.data(), B->data, B->shape.data(), C ? C->data : nullptr,
+                            C ? C->shape.data() : nullptr, C ? int(C->shape.size()) : 0, alpha, beta, transA, transB,
+                            result->data, result->shape.data(), ZANT_ACT_NONE));
+}
+inline Tensor<float> gemm(Tensor<float> *A, Tensor<float> *B, Tensor<float> *C, float alpha, float beta, bool transA,
+                          bool transB) {
+    int64_t ydim[4];
+    check(zant_hip_gemm_check(A->shape.data(), int(A->shape.size()), B->shape.data(), int(B->shape.size()),
+                              C ? C->shape.data() : nullptr, C ? int(C->shape.size()) : 0, C != nullptr, transA, transB,
+                              ydim));
+    Tensor<float> Y = Tensor<float>::fromShape({ydim[0], ydim[1], ydim[2], ydim[3]});
+    gemm_lean(A, B, C, alpha, beta, transA, transB, &Y);
+    return Y;
+}
+
+// onnx_maxpool_lean / onnx_maxpool (op_pooling.zig:570, :663)
+template <typename T>
+inline void onnx_maxpool_lean(Tensor<T> *input, Tensor<T> *output, const Dims &kernel_shape, const Dims &strides,
+                              const Dims &dilations, const Dims &pads, AutoPadType auto_pad);
+template <>
+inline void onnx_maxpool_lean<float>(Tensor<float> *input, Tensor<float> *output, const Dims &k, const Dims &s,
+                                     const Dims &d, const Dims &p, AutoPadType ap) {
+    check(zant_hip_maxpool2d_f32(default_ctx(), input->data, input->shape.data(), output->data, output->shape.data(),
+                                 k.data(), s.data(), d.data(), p.data(), int(p.size()), int(ap)));
+}
+template <>
+inline void onnx_maxpool_lean<uint8_t>(Tensor<uint8_t> *input, Tensor<uint8_t> *output, const Dims &k, const Dims &s,
+                                       const Dims &d, const Dims &p, AutoPadType ap) {
+    check(zant_hip_maxpool2d_u8(default_ctx(), input->data, input->shape.data(), output->data, output->shape.data(),
+                                k.data(), s.data(), d.data(), p.data(), int(p.size()), int(ap)));
+}
+template <typename T>
+inline Tensor<T> onnx_maxpool(Tensor<T> *input, const Dims &k, const Dims &s, const Dims &d, const Dims &p,
+                              AutoPadType ap, bool ceil_mode) {
+    if (input->shape.size() != 4) throw Error(ZANT_InvalidDimensions);
+    int64_t ydim[4];
+    check(zant_hip_maxpool2d_out_shape(input->shape.data(), k.data(), s.data(), d.data(), p.data(), int(ap), ceil_mode,
+                                       ydim));
+    Tensor<T> out = Tensor<T>::fromShape({ydim[0], ydim[1], ydim[2], ydim[3]});
+    onnx_maxpool_lean<T>(input, &out, k, s, d, p, ap);
+    return out;
+}
+
+// ReLU_lean / ReLU, leakyReLU_lean / leakyReLU, softmax_lean / softmax (lib_activation_function_math.zig)
+inline void ReLU_lean(Tensor<float> *in, Tensor<float> *out) {
+    check(zant_hip_relu_f32(default_ctx(), in->data, out->data, int64_t(in->size)));
+}
+inline Tensor<float> ReLU(Tensor<float> *in) {
+    if (in->size == 0) throw Error(ZANT_ZeroSizeTensor);
+    Tensor<float> out = Tensor<float>::fromShape(in->shape);
+    ReLU_lean(in, &out);
+    return out;
+}
+inline void leakyReLU_lean(Tensor<float> *in, float slope, Tensor<float> *out) {
+    check(zant_hip_leaky_relu_f32(default_ctx(), in->data, slope, out->data, int64_t(in->size)));
+}
+inline Tensor<float> leakyReLU(Tensor<float> *in, float slope) {
+    if (in->size == 0) throw Error(ZANT_ZeroSizeTensor);
+    Tensor<float> out = Tensor<float>::fromShape(in->shape);
+    leakyReLU_lean(in, slope, &out);
+    return out;
+}
+inline void softmax_lean(Tensor<float> *in, Tensor<float> *out) {
+    check(zant_hip_softmax_f32(default_ctx(), in->data, out->data, in->shape[0], in->shape[1]));
+}
+inline Tensor<float> softmax(Tensor<float> *in) {
+    if (in->size == 0) throw Error(ZANT_ZeroSizeTensor);
+    Tensor<float> out = Tensor<float>::fromShape(in->shape);
+    softmax_lean(in, &out);
+    return out;
+}
+
+// sum_tensors_lean / sum_tensors, add_bias (lib_elementWise_math.zig:70, :52, :22)
+inline void sum_tensors_lean(Tensor<float> *t1, Tensor<float> *t2, Tensor<float> *out) {
+    int64_t ydim[8];
+    int yr = 0;
+    check(zant_hip_add_f32(default_ctx(), t1->data, t1->shape.data(), int(t1->shape.size()), t2->data, t2->shape.data(),
+                           int(t2->shape.size()), out->data, ydim, &yr));
+    out->shape.assign(ydim, ydim + yr);  // the lean op rewrites the output shape (:157)
+}
+inline Tensor<float> sum_tensors(Tensor<float> *t1, Tensor<float> *t2) {
+    if (t1->size != t2->size) throw Error(ZANT_InputTensorDifferentSize);
+    Tensor<float> out = Tensor<float>::fromShape(t2->shape);
+    sum_tensors_lean(t1, t2, &out);
+    return out;
+}
+inline void add_bias(Tensor<float> *tensor, Tensor<float> *bias) {
+    check(zant_hip_add_bias_f32(default_ctx(), tensor->data, tensor->shape.data(), int(tensor->shape.size()), bias->data,
+                                bias->shape.data(), int(bias->shape.size())));
+}
+
+// reshape_lean (lib_shape_math.zig:1139); -1 stands for the maxInt(usize) sentinel
+template <typename T>
+inline void reshape_lean(Tensor<T> *in, const Dims &newShape, std::optional<bool> /*allowZero*/, Tensor<T> *out) {
+    Dims resolved(newShape.size());
+    check(zant_hip_reshape(default_ctx(), in->data, in->shape.data(), int(in->shape.size()), sizeof(T), newShape.data(),
+                           int(newShape.size()), out->data, resolved.data()));
+    out->shape = resolved;
+    out->size = in->size;
+}
+
+}  // namespace tensMath
+}  // namespace zant

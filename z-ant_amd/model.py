@@ -136,6 +136,15 @@ class Model:
         if rc:
             raise ZantError(rc)
 
+    def profile(self):
+        """One pass with per-kernel timing -> [(name, ms, ops, bytes)] per kernel-launching node."""
+        n = self.num_launches
+        ms = (C.c_float * n)(); ops = (C.c_double * n)(); by = (C.c_double * n)()
+        rc = lib.zant_model_profile(self.handle, ms, ops, by, n)
+        if rc < 0:
+            raise ZantError(rc)
+        return [(lib.zant_model_launch_name(self.handle, i).decode(), ms[i], ops[i], by[i]) for i in range(rc)]
+
     def predict_host(self, x):
         x = np.ascontiguousarray(x)
         y = np.zeros(self.out_shape, self.out_dtype)

@@ -32,6 +32,26 @@ def readme_cnn_flops_per_inference():
     return {"conv1": conv1, "conv2": conv2, "gemm1": gemm1, "gemm2": gemm2, "total": conv1 + conv2 + gemm1 + gemm2}
 
 
+def build_readme_cnn_model(ctx, batch, params):
+    """The README CNN as a zant_model: the node list a generated predict() would call, fused and arena-planned."""
+    from .model import Model
+    m = Model(ctx)
+    t = m.input((batch, 1, 28, 28))
+    t = m.conv(t, params["w1"], params["b1"], [1, 1], None, None, 1, None)
+    t = m.relu(t)
+    t = m.maxpool(t, [2, 2], [2, 2])
+    t = m.conv(t, params["w2"], params["b2"], [1, 1], None, None, 1, None)
+    t = m.relu(t)
+    t = m.maxpool(t, [2, 2], [2, 2])
+    t = m.reshape(t, [1, 1, batch, 1600])
+    t = m.gemm(t, params["g1"], params["c1"])
+    t = m.relu(t)
+    t = m.gemm(t, params["g2"], params["c2"])
+    t = m.reshape(t, [batch, 10])
+    t = m.softmax(t)
+    return m.finalize()
+
+
 class ReadmeCNN:
     def __init__(self, batch, params, device="cuda:0"):
         self.n = batch
