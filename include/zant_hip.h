@@ -67,7 +67,7 @@ int zant_hip_ctx_create(zant_ctx **out, int device, void *stream);
 void zant_hip_ctx_destroy(zant_ctx *ctx);
 int zant_hip_sync(zant_ctx *ctx);
 const char *zant_hip_status_name(int status);
-const char *zant_hip_last_error(zant_ctx *ctx);
+const char *zant_hip_last_error(zant_ctx *ctx); /* ctx == NULL: the calling thread's last failed zant_hip_ctx_create */
 const char *zant_hip_version(void);
 
 /* Replaces setLogFunctionC (src/Core/Tensor/TensorMath/op_convolution.zig:37-41)

@@ -11,6 +11,11 @@ if not os.path.exists(lib_path):
         f"{lib_path} is not built. Run `python z-ant_amd/build.py` (hipcc, gfx950). "
         "This backend has no CPU fallback.")
 
+# torch ships its own copy of the HIP runtime.  Two runtimes in one process do not share the device (the second
+# one to initialise reports "no ROCm-capable device"), so torch's must be mapped before the library's dependency
+# on libamdhip64.so is resolved: the loader then binds the library to the copy that is already there.
+import torch  # noqa: E402,F401
+
 lib = C.CDLL(lib_path)
 
 c_i64p = C.POINTER(C.c_int64)
@@ -130,7 +135,7 @@ class Context:
         h = vp()
         rc = lib.zant_hip_ctx_create(C.byref(h), device, vp(stream) if stream else None)
         if rc:
-            raise ZantError(rc, "zant_hip_ctx_create")
+            raise ZantError(rc, "zant_hip_ctx_create: " + lib.zant_hip_last_error(None).decode())
         self.handle = h
 
     def check(self, rc):

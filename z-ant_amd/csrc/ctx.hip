@@ -6,6 +6,15 @@ void (*g_zant_log)(char *) = nullptr;
 extern "C" void setLogFunctionC(void (*func)(char *)) { g_zant_log = func; }
 extern "C" void setLogFunction(void (*func)(char *)) { g_zant_log = func; }
 
+// Failures with no context to hold them (context creation itself) are kept per thread.
+static thread_local std::string g_create_error;
+
+static int create_failed(hipError_t e, const char *what) {
+    g_create_error = std::string(what) + ": " + hipGetErrorString(e);
+    zant_log(g_create_error.c_str());
+    return ZANT_HipError;
+}
+
 int zant_fail_hip(zant_ctx *ctx, hipError_t e, const char *what) {
     if (ctx) {
         ctx->last_error = std::string(what) + ": " + hipGetErrorString(e);
@@ -36,20 +45,23 @@ extern "C" int zant_hip_ctx_create(zant_ctx **out, int device, void *stream) {
     if (!ctx) return ZANT_MemError;
     ctx->device = device;
     hipError_t e = hipSetDevice(device);
-    if (e != hipSuccess) { delete ctx; return ZANT_HipError; }
+    if (e != hipSuccess) { delete ctx; return create_failed(e, "hipSetDevice"); }
     if (stream) {
         ctx->stream = static_cast<hipStream_t>(stream);
     } else {
         e = hipStreamCreate(&ctx->stream);  // default priority
-        if (e != hipSuccess) { delete ctx; return ZANT_HipError; }
+        if (e != hipSuccess) { delete ctx; return create_failed(e, "hipStreamCreate"); }
         ctx->owns_stream = true;
     }
     hipDeviceProp_t prop;
     if (hipGetDeviceProperties(&prop, device) == hipSuccess) ctx->num_cus = prop.multiProcessorCount;
-    if (hipEventCreate(&ctx->ev_start) != hipSuccess || hipEventCreate(&ctx->ev_stop) != hipSuccess ||
-        hipEventCreate(&ctx->ev_k0) != hipSuccess || hipEventCreate(&ctx->ev_k1) != hipSuccess) {
-        zant_hip_ctx_destroy(ctx);
-        return ZANT_HipError;
+    hipEvent_t *evs[4] = {&ctx->ev_start, &ctx->ev_stop, &ctx->ev_k0, &ctx->ev_k1};
+    for (hipEvent_t *ev : evs) {
+        e = hipEventCreate(ev);
+        if (e != hipSuccess) {
+            zant_hip_ctx_destroy(ctx);
+            return create_failed(e, "hipEventCreate");
+        }
     }
     *out = ctx;
     return ZANT_OK;
@@ -75,7 +87,7 @@ extern "C" int zant_hip_sync(zant_ctx *ctx) {
     return ZANT_OK;
 }
 
-extern "C" const char *zant_hip_last_error(zant_ctx *ctx) { return ctx ? ctx->last_error.c_str() : ""; }
+extern "C" const char *zant_hip_last_error(zant_ctx *ctx) { return ctx ? ctx->last_error.c_str() : g_create_error.c_str(); }
 extern "C" const char *zant_hip_version(void) { return "zant-hip 0.1 (gfx950)"; }
 
 extern "C" const char *zant_hip_status_name(int s) {

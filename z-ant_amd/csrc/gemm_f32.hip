@@ -12,6 +12,7 @@
 namespace {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 constexpr int BK = 32;
 
 struct GemmArgs {
@@ -22,6 +23,7 @@ struct GemmArgs {
     int c_ld_r, c_ld_c;      // 0 strides for broadcast axes
     int relu;
     int a_vec, b_vec;        // 16-byte vector loads are legal for A / B
+    int dbg;
 };
 
 // Loads 4 consecutive floats p[0..3]; elements at or beyond `valid` read as 0.
@@ -57,7 +59,12 @@ gemm_f32_mfma_kernel(const float *__restrict__ A, const float *__restrict__ B, c
     const int l32 = lane & 31, lh = lane >> 5;
     // N tiles vary fastest so that workgroups sharing a row panel of A are dispatched together.
     const int n_tiles = (g.N + BN - 1) / BN;
-    const int bm = blockIdx.x / n_tiles, bn = blockIdx.x - bm * n_tiles;
+    // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2): give every XCD a contiguous range of
+    // tiles so that the tiles sharing a row panel of A meet in one L2.
+    const int per_xcd = (gridDim.x + 7) >> 3;
+    int sb = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if ((gridDim.x & 7) != 0) sb = blockIdx.x;
+    const int bm = sb / n_tiles, bn = sb - bm * n_tiles;
     const int m0 = bm * BM, n0 = bn * BN;
 
     float4 ra[A_V], rb[B_V];
@@ -170,6 +177,309 @@ gemm_f32_mfma_kernel(const float *__restrict__ A, const float *__restrict__ B, c
     }
 }
 
+// ------------------------------------------------------------------------------------------------------------
+// Fast path: asynchronous global->LDS staging (no VGPR round trip), a ring of S stages, 128-bit operand reads.
+// ------------------------------------------------------------------------------------------------------------
+typedef __attribute__((address_space(1))) const void *gptr_t;
+typedef __attribute__((address_space(3))) void *lptr_t;
+__device__ __attribute__((aligned(16))) const float g_gemm_zero[4] = {0.f, 0.f, 0.f, 0.f};
+
+// How an operand panel [ROWS x 32 k] is staged.  KC*: the matrix is stored with k contiguous ([rows][K]);
+// RC4: stored with the row index contiguous ([K][rows]).  In LDS a "unit" is 4 consecutive k of one row (16 bytes):
+//   KC layout  unit(row, u) at row*8 + (u ^ (row & 7))   (XOR swizzle: a 128-byte global row segment lands in one
+//              128-byte LDS row, and lanes that read 32 different rows at the same u still hit 8 different columns)
+//   RC layout  unit(row, u) at u*ROWS + row
+enum { KC16 = 0, KC4 = 1, RC4 = 2 };
+
+template <int MODE, int ROWS>
+constexpr int stage_instrs() { return MODE == KC16 ? ROWS / 8 : ROWS / 2; }
+
+// The copies of one operand panel for chunk k0.  Every wave issues the same number of instructions whatever the
+// masks are (masked lanes fetch zeros), so the number of copies in flight per wave is known at compile time.
+template <int MODE, int ROWS, int NW>
+__device__ __forceinline__ void stage_panel(float *dst, const float *__restrict__ src, int ld, int r0, int R, int k0,
+                                            int K, int wave, int lane) {
+    constexpr int INSTRS = stage_instrs<MODE, ROWS>();
+    static_assert(INSTRS % NW == 0, "staging instructions must divide over the waves");
+#pragma unroll
+    for (int ii = 0; ii < INSTRS / NW; ++ii) {
+        const int i = ii * NW + wave;
+        const float *sp;
+        if (MODE == KC16) {
+            const int U = i * 64 + lane, row = U >> 3, slot = U & 7;
+            const int k = k0 + ((slot ^ (row & 7)) << 2);
+            sp = (r0 + row < R && k < K) ? src + int64_t(r0 + row) * ld + k : g_gemm_zero;
+            __builtin_amdgcn_global_load_lds((gptr_t)sp, (lptr_t)(dst + i * 256), 16, 0, 0);
+        } else if (MODE == KC4) {
+            const int F = i * 64 + lane, row = F >> 5, slot = (F >> 2) & 7, j = F & 3;
+            const int k = k0 + ((slot ^ (row & 7)) << 2) + j;
+            sp = (r0 + row < R && k < K) ? src + int64_t(r0 + row) * ld + k : g_gemm_zero;
+            __builtin_amdgcn_global_load_lds((gptr_t)sp, (lptr_t)(dst + i * 64), 4, 0, 0);
+        } else {
+            const int F = i * 64 + lane, j = F & 3, row = (F >> 2) % ROWS, u = F / (4 * ROWS);
+            const int k = k0 + (u << 2) + j;
+            sp = (r0 + row < R && k < K) ? src + int64_t(k) * ld + r0 + row : g_gemm_zero;
+            __builtin_amdgcn_global_load_lds((gptr_t)sp, (lptr_t)(dst + i * 64), 4, 0, 0);
+        }
+    }
+}
+
+// Per-lane source pointers of a panel at chunk 0 for the unmasked fast path.  Rows beyond the matrix are clamped to
+// its last row: what they produce lands in accumulator rows / columns that are never stored.
+template <int MODE, int ROWS, int NW>
+__device__ __forceinline__ void stage_ptrs(const float *(&p)[stage_instrs<MODE, ROWS>() / NW], const float *src, int ld,
+                                           int r0, int R, int wave, int lane) {
+#pragma unroll
+    for (int ii = 0; ii < stage_instrs<MODE, ROWS>() / NW; ++ii) {
+        const int i = ii * NW + wave;
+        if (MODE == KC16) {
+            const int U = i * 64 + lane, row = U >> 3, slot = U & 7;
+            p[ii] = src + int64_t(min(r0 + row, R - 1)) * ld + ((slot ^ (row & 7)) << 2);
+        } else if (MODE == KC4) {
+            const int F = i * 64 + lane, row = F >> 5, slot = (F >> 2) & 7, j = F & 3;
+            p[ii] = src + int64_t(min(r0 + row, R - 1)) * ld + ((slot ^ (row & 7)) << 2) + j;
+        } else {
+            const int F = i * 64 + lane, j = F & 3, row = (F >> 2) % ROWS, u = F / (4 * ROWS);
+            p[ii] = src + int64_t((u << 2) + j) * ld + min(r0 + row, R - 1);
+        }
+    }
+}
+
+// Fast-path copies of one panel: chunk offset `koff` (floats) is uniform, nothing is masked.
+template <int MODE, int ROWS, int NW>
+__device__ __forceinline__ void stage_fast(float *dst, const float *const (&p)[stage_instrs<MODE, ROWS>() / NW],
+                                           int64_t koff, int wave) {
+#pragma unroll
+    for (int ii = 0; ii < stage_instrs<MODE, ROWS>() / NW; ++ii) {
+        const int i = ii * NW + wave;
+        if (MODE == KC16) __builtin_amdgcn_global_load_lds((gptr_t)(p[ii] + koff), (lptr_t)(dst + i * 256), 16, 0, 0);
+        else __builtin_amdgcn_global_load_lds((gptr_t)(p[ii] + koff), (lptr_t)(dst + i * 64), 4, 0, 0);
+    }
+}
+
+// LDS float offset of unit (row, u) of a panel.
+template <int MODE, int ROWS>
+__device__ __forceinline__ int unit_off(int row, int u) {
+    return MODE == RC4 ? (u * ROWS + row) * 4 : (row * 8 + (u ^ (row & 7))) * 4;
+}
+
+// Operand reads and their waits are written by hand.  The compiler cannot count LDS reads that are still in flight
+// when newer ones have been issued (it waits for ALL of them, lgkmcnt(0)), which exposes the full LDS latency once per
+// group.  LDS returns data in order, so after "lgkmcnt(n)" with n = number of reads issued later, a read has landed.
+__device__ __forceinline__ unsigned lds_addr(const float *p) {
+    return unsigned(reinterpret_cast<uintptr_t>((lptr_t)const_cast<float *>(p)));
+}
+template <int OFF>
+__device__ __forceinline__ void lds_read128(f32x4 &v, unsigned addr) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+}
+// Waits until at most N LDS reads are outstanding.  The operand registers are in/out operands so that nothing
+// that consumes them can be scheduled above the wait.
+template <int N, int MT>
+__device__ __forceinline__ void lds_wait(f32x4 (&a)[MT], f32x4 &b) {
+    static_assert(MT == 1 || MT == 2 || MT == 4, "unsupported tile count");
+    if constexpr (MT == 1) asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a[0]), "+v"(b) : "n"(N));
+    else if constexpr (MT == 2) asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(a[0]), "+v"(a[1]), "+v"(b) : "n"(N));
+    else asm volatile("s_waitcnt lgkmcnt(%5)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b) : "n"(N));
+}
+
+// The reads of group gi of the chunk at LDS byte address `stage`: MT units of A and one of B per lane.
+//   offa / offb: this lane's byte offsets of its group-0..3 units inside a stage (tile i of A adds i * 32 rows).
+template <int MT, int AM, int BMODE, int BM, int BN>
+__device__ __forceinline__ void read_group(unsigned stage, int gi, const unsigned (&offa)[BK / 8],
+                                           const unsigned (&offb)[BK / 8], f32x4 (&av)[MT], f32x4 &bv) {
+    constexpr int A_TILE = (AM == RC4 ? 32 * 16 : 32 * 128);  // bytes between rows r and r + 32 of a panel
+    const unsigned pa = stage + offa[gi], pb = stage + BM * BK * 4 + offb[gi];
+    lds_read128<0>(av[0], pa);
+    if constexpr (MT >= 2) lds_read128<A_TILE>(av[1], pa);
+    if constexpr (MT >= 4) {
+        lds_read128<2 * A_TILE>(av[2], pa);
+        lds_read128<3 * A_TILE>(av[3], pa);
+    }
+    lds_read128<0>(bv, pb);
+}
+
+// One pipeline step: start the copies of chunk `ichunk` into `dma`, multiply the chunk at LDS address `cmp_addr`,
+// request the first operands of the chunk at `nxt_addr`.
+template <int MT, int WM, int WN, int AM, int BMODE>
+__device__ __forceinline__ void gemm_step(float *__restrict__ dma, unsigned cmp_addr, unsigned nxt_addr,
+                                          const unsigned (&offa)[BK / 8], const unsigned (&offb)[BK / 8],
+                                          f32x4 (&a)[2][MT], f32x4 (&b)[2],
+                                          const float *__restrict__ A, const float *__restrict__ B, const GemmArgs &g,
+                                          const float *const (&pa)[stage_instrs<AM, WM * MT * 32>() / (WM * WN)],
+                                          const float *const (&pb)[stage_instrs<BMODE, WN * 32>() / (WM * WN)],
+                                          int m0, int n0, int ichunk, f32x16 (&acc)[MT]) {
+    constexpr int NW = WM * WN, BM = WM * MT * 32, BN = WN * 32;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave % WM, wn = wave / WM;
+    const int l32 = lane & 31, lh = lane >> 5;
+    if (g.dbg & 1) {} else
+    if ((ichunk + 1) * BK <= g.K) {  // whole chunk inside K: no masks, addresses are a uniform offset from chunk 0
+        stage_fast<AM, BM, NW>(dma, pa, AM == RC4 ? int64_t(ichunk) * BK * g.lda : int64_t(ichunk) * BK, wave);
+        stage_fast<BMODE, BN, NW>(dma + BM * BK, pb, BMODE == RC4 ? int64_t(ichunk) * BK * g.ldb : int64_t(ichunk) * BK, wave);
+    } else {
+        stage_panel<AM, BM, NW>(dma, A, g.lda, m0, g.M, ichunk * BK, g.K, wave, lane);
+        stage_panel<BMODE, BN, NW>(dma + BM * BK, B, g.ldb, n0, g.N, ichunk * BK, g.K, wave, lane);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    if (g.dbg & 2) return;
+    static_assert((BK / 8) % 2 == 0, "group 0 of every chunk uses operand registers 0");
+#pragma unroll
+    for (int gi = 0; gi < BK / 8; ++gi) {
+        const int cur = gi & 1;
+        // The next group's operands are requested before this group's MFMAs start: a whole burst to land.  After the
+        // last group that is group 0 of the next chunk, which the barrier of THIS step already proved complete, so the
+        // next step starts with its operands in registers (or on their way).
+        if (gi + 1 < BK / 8) read_group<MT, AM, BMODE, BM, BN>(cmp_addr, gi + 1, offa, offb, a[cur ^ 1], b[cur ^ 1]);
+        else read_group<MT, AM, BMODE, BM, BN>(nxt_addr, 0, offa, offb, a[0], b[0]);
+        lds_wait<MT + 1, MT>(a[cur], b[cur]);  // everything but the MT + 1 reads just issued has landed
+        __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][i][j], b[cur][j], acc[i], 0, 0, 0);
+        __builtin_amdgcn_s_setprio(0);
+    }
+}
+
+// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt in bits 3:0 and 15:14).
+constexpr int vmcnt_imm(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
+
+template <int MT, int WM, int WN, int AM, int BMODE, int S>
+__global__ void __launch_bounds__(WM *WN * 64)
+gemm_f32_dma_kernel(const float *__restrict__ A, const float *__restrict__ B, const float *__restrict__ C,
+                    float *__restrict__ Y, GemmArgs g) {
+    constexpr int NW = WM * WN, BM = WM * MT * 32, BN = WN * 32;
+    constexpr int STAGE = (BM + BN) * BK;  // floats
+    constexpr int P = (stage_instrs<AM, BM>() + stage_instrs<BMODE, BN>()) / NW;  // copies per wave and chunk
+    static_assert(S >= 3 && P * (S - 2) < 64, "vmcnt is a 6-bit counter");
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave % WM, wn = wave / WM;
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int n_tiles = (g.N + BN - 1) / BN;
+    const int per_xcd = (gridDim.x + 7) >> 3;
+    int sb = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);  // contiguous tile range per XCD (one L2 each)
+    if ((gridDim.x & 7) != 0) sb = blockIdx.x;
+    const int bm = sb / n_tiles, bn = sb - bm * n_tiles;
+    const int m0 = bm * BM, n0 = bn * BN;
+
+    f32x16 acc[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][v] = 0.0f;
+
+    const float *pa[stage_instrs<AM, BM>() / NW], *pb[stage_instrs<BMODE, BN>() / NW];
+    stage_ptrs<AM, BM, NW>(pa, A, g.lda, m0, g.M, wave, lane);
+    stage_ptrs<BMODE, BN, NW>(pb, B, g.ldb, n0, g.N, wave, lane);
+
+    const int n_chunks = (g.K + BK - 1) / BK;
+    // prologue: chunks 0 .. S-2 in flight (chunks beyond the end copy zeros: the count per wave stays fixed)
+#pragma unroll
+    for (int c = 0; c < S - 1; ++c) {
+        stage_panel<AM, BM, NW>(lds + c * STAGE, A, g.lda, m0, g.M, c * BK, g.K, wave, lane);
+        stage_panel<BMODE, BN, NW>(lds + c * STAGE + BM * BK, B, g.ldb, n0, g.N, c * BK, g.K, wave, lane);
+    }
+    // Chunk 0 must be complete for everyone before its first operands are fetched.
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(P * (S - 2)));
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    // this lane's operand units: group gi reads k-unit 2*gi + lh of rows (wm*MT + i)*32 + l32 (A) and wn*32 + l32 (B)
+    unsigned offa[BK / 8], offb[BK / 8];
+#pragma unroll
+    for (int gi = 0; gi < BK / 8; ++gi) {
+        offa[gi] = unsigned(unit_off<AM, BM>(wm * MT * 32 + l32, gi * 2 + lh)) * 4u;
+        offb[gi] = unsigned(unit_off<BMODE, BN>(wn * 32 + l32, gi * 2 + lh)) * 4u;
+    }
+    const unsigned lds0 = lds_addr(lds);
+    f32x4 ra[2][MT], rb[2];
+    read_group<MT, AM, BMODE, BM, BN>(lds0, 0, offa, offb, ra[0], rb[0]);
+    int cbuf = 0, dbuf = S - 1;
+    for (int c = 0; c < n_chunks; ++c) {
+        // After this barrier: chunk c+1 is complete for everyone (each wave waited for its own copies of it), and
+        // everyone is done with chunk c-1, whose stage is refilled now.  A bare s_barrier: __syncthreads() carries a
+        // fence that drains ALL outstanding copies, which would serialise the ring.  The step multiplies chunk c,
+        // whose first operands were fetched at the end of the previous step, and ends by fetching those of chunk c+1.
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(P * (S - 3)));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        const int nbuf = cbuf + 1 == S ? 0 : cbuf + 1;
+        gemm_step<MT, WM, WN, AM, BMODE>(lds + dbuf * STAGE, lds0 + cbuf * (STAGE * 4), lds0 + nbuf * (STAGE * 4), offa, offb,
+                                         ra, rb, A, B, g, pa, pb, m0, n0, c + S - 1, acc);
+        cbuf = nbuf;
+        dbuf = dbuf + 1 == S ? 0 : dbuf + 1;
+    }
+    lds_wait<0, MT>(ra[0], rb[0]);             // the last step's look-ahead reads
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // trailing zero copies must not outlive the workgroup's LDS
+
+    const int n = n0 + wn * 32 + l32;
+    if (n < g.N) {
+        // all C values first (independent loads in flight together), one per lane when C is broadcast along rows
+        float cv[MT][16];
+        if (g.c_mode) {
+            if (g.c_ld_r == 0) {
+                const float c0 = C[int64_t(n) * g.c_ld_c];
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) cv[i][v] = c0;
+            } else {
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int m = m0 + (wm * MT + i) * 32 + (v >> 2) * 8 + lh * 4 + (v & 3);
+                        cv[i][v] = C[int64_t(min(m, g.M - 1)) * g.c_ld_r + int64_t(n) * g.c_ld_c];
+                    }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int m = m0 + (wm * MT + i) * 32 + (v >> 2) * 8 + lh * 4 + (v & 3);
+                if (m < g.M) {
+                    float r = acc[i][v] * g.alpha;
+                    if (g.c_mode) r = r + cv[i][v] * g.beta;
+                    if (g.relu) r = r > 0.0f ? r : 0.0f;
+                    Y[int64_t(m) * g.N + n] = r;
+                }
+            }
+        }
+    }
+}
+
+template <int MT, int WM, int WN, int AM, int BMODE>
+void launch_gemm_dma(zant_ctx *ctx, const float *A, const float *B, const float *C, float *Y, const GemmArgs &g) {
+    constexpr int S = 5;
+    constexpr int BM = WM * MT * 32, BN = WN * 32;
+    constexpr size_t lds_bytes = size_t(S) * (BM + BN) * BK * sizeof(float);
+    auto kern = &gemm_f32_dma_kernel<MT, WM, WN, AM, BMODE, S>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
+        attr_set = true;
+    }
+    const unsigned blocks = unsigned(((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN));
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(WM * WN * 64), lds_bytes, ctx->stream, A, B, C, Y, g);
+}
+
+template <int MT, int WM, int WN>
+void dispatch_gemm_dma(zant_ctx *ctx, const float *A, const float *B, const float *C, float *Y, const GemmArgs &g,
+                       int am, int bmode) {
+#define ZANT_GEMM_CASE(a, b) if (am == a && bmode == b) return launch_gemm_dma<MT, WM, WN, a, b>(ctx, A, B, C, Y, g);
+    ZANT_GEMM_CASE(KC16, KC16) ZANT_GEMM_CASE(KC16, KC4) ZANT_GEMM_CASE(KC16, RC4)
+    ZANT_GEMM_CASE(KC4, KC16) ZANT_GEMM_CASE(KC4, KC4) ZANT_GEMM_CASE(KC4, RC4)
+    ZANT_GEMM_CASE(RC4, KC16) ZANT_GEMM_CASE(RC4, KC4) ZANT_GEMM_CASE(RC4, RC4)
+#undef ZANT_GEMM_CASE
+}
+
 template <int TM, int WM, int WN>
 void launch_gemm(zant_ctx *ctx, const float *A, const float *B, const float *C, float *Y, const GemmArgs &g,
                  bool a_kc, bool b_kc) {
@@ -193,12 +503,24 @@ int run_gemm(zant_ctx *ctx, const float *A, const float *B, const float *C, floa
     g.alpha = alpha; g.beta = beta;
     g.c_mode = c_mode; g.c_ld_r = int(c_ld_r); g.c_ld_c = int(c_ld_c);
     g.relu = relu;
+    g.dbg = getenv("ZANT_GEMM_DBG") ? atoi(getenv("ZANT_GEMM_DBG")) : 0;
     g.a_vec = (reinterpret_cast<uintptr_t>(A) & 15) == 0 && (g.lda & 3) == 0;
     g.b_vec = (reinterpret_cast<uintptr_t>(B) & 15) == 0 && (g.ldb & 3) == 0;
     const bool a_kc = !trans_a, b_kc = trans_b;
     KernelTimer kt(ctx);
-    if (N > 32) launch_gemm<2, 2, 2>(ctx, A, B, C, Y, g, a_kc, b_kc);   // 128 x 64 tile
-    else launch_gemm<1, 4, 1>(ctx, A, B, C, Y, g, a_kc, b_kc);          // 128 x 32 tile
+    const int am = a_kc ? (g.a_vec ? KC16 : KC4) : RC4;
+    const int bmode = b_kc ? (g.b_vec ? KC16 : KC4) : RC4;
+    const char *cfg = getenv("ZANT_GEMM_CFG");
+    int c = cfg ? atoi(cfg) : 0;
+    if (c == 1) launch_gemm_dma<1, 2, 2, KC16, RC4>(ctx, A, B, C, Y, g);
+    else if (c == 2) launch_gemm_dma<2, 2, 2, KC16, RC4>(ctx, A, B, C, Y, g);
+    else if (c == 3) launch_gemm_dma<1, 2, 4, KC16, RC4>(ctx, A, B, C, Y, g);
+    else if (c == 4) launch_gemm_dma<2, 1, 4, KC16, RC4>(ctx, A, B, C, Y, g);
+    else if (c == 5) launch_gemm_dma<1, 4, 1, KC16, RC4>(ctx, A, B, C, Y, g);
+    else if (c == 6) launch_gemm_dma<2, 2, 1, KC16, RC4>(ctx, A, B, C, Y, g);
+    else
+    if (N > 32) dispatch_gemm_dma<1, 4, 2>(ctx, A, B, C, Y, g, am, bmode);  // 128 x 64 tile, 8 waves
+    else launch_gemm<1, 4, 1>(ctx, A, B, C, Y, g, a_kc, b_kc);              // 128 x 32 tile
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
 }

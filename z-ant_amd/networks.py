@@ -78,3 +78,112 @@ class ReadmeCNN:
         tm.gemm_lean(self.h1, p["g2"], p["c2"], 1.0, 1.0, False, False, self.h2)
         tm.softmax_lean(self.h2.view(self.n, 10), self.out)
         return self.out
+
+
+# ------------------------------------------------------------------------------------------------
+# int8 networks of the benchmark configurations (tiny-YOLO style detector, MobileNetV2-0.35 @ 96)
+# ------------------------------------------------------------------------------------------------
+# An architecture is a list of layer dicts executed in order; "src"/"res" name earlier layer outputs.
+#   conv : QLinearConv  (k, stride, pad, cin, cout, group)   [+ act: None | "leaky" | "relu6"]
+#   pool : MaxPool 2x2/2 on the quantised values
+#   add  : quantised residual add with the output of layer `res`
+#   gap  : quantised global average pool
+# Activation scales / zero points are NOT chosen here: they come from a calibration pass recorded as a
+# fixture (tests/golden/int8_networks.json) and are passed in as `quant`.
+
+def _make_divisible(v, d=8):
+    return max(d, int(v + d / 2) // d * d)
+
+
+def tiny_yolo_arch():
+    """Six 3x3 pad-1 convolutions 3->16->32->64->128->256->256 with LeakyReLU(0.1), a 2x2/2 MaxPool after each of
+    the first five, and a 1x1 head to 3*(5+4) = 27 channels; 3x96x96 input -> 27x3x3 output."""
+    arch, cin = [], 3
+    for i, cout in enumerate([16, 32, 64, 128, 256, 256]):
+        arch.append(dict(op="conv", k=3, stride=1, pad=1, cin=cin, cout=cout, group=1, act="leaky", alpha=0.1))
+        if i < 5:
+            arch.append(dict(op="pool"))
+        cin = cout
+    arch.append(dict(op="conv", k=1, stride=1, pad=0, cin=256, cout=27, group=1, act=None))
+    return dict(name="tiny_yolo_int8", input=(3, 96, 96), layers=arch)
+
+
+def mobilenet_v2_035_arch():
+    """MobileNetV2, width 0.35, 96x96 input: 3x3/2 stem, 17 inverted-residual blocks (1x1 expand x6 + ReLU6,
+    3x3 depthwise + ReLU6, 1x1 linear projection, residual add where shapes match), 1x1 to 1280 + ReLU6, global
+    average pool, 1280->1000 classifier (a 1x1 QLinearConv on the pooled [N,1280,1,1] tensor)."""
+    w = 0.35
+    layers = [dict(op="conv", k=3, stride=2, pad=1, cin=3, cout=_make_divisible(32 * w), group=1, act="relu6")]
+    cin = layers[0]["cout"]
+    for t, c, n, s in [(6, 16, 1, 1), (6, 24, 2, 2), (6, 32, 3, 2), (6, 64, 4, 2), (6, 96, 3, 1), (6, 160, 3, 2), (6, 320, 1, 1)]:
+        cout = _make_divisible(c * w)
+        for i in range(n):
+            stride = s if i == 0 else 1
+            block_in = len(layers) - 1  # index of the layer whose output feeds this block
+            hidden = cin * t
+            layers.append(dict(op="conv", k=1, stride=1, pad=0, cin=cin, cout=hidden, group=1, act="relu6"))
+            layers.append(dict(op="conv", k=3, stride=stride, pad=1, cin=hidden, cout=hidden, group=hidden, act="relu6"))
+            layers.append(dict(op="conv", k=1, stride=1, pad=0, cin=hidden, cout=cout, group=1, act=None))
+            if stride == 1 and cin == cout:
+                layers.append(dict(op="add", res=block_in))
+            cin = cout
+    layers.append(dict(op="conv", k=1, stride=1, pad=0, cin=cin, cout=1280, group=1, act="relu6"))
+    layers.append(dict(op="gap"))
+    layers.append(dict(op="conv", k=1, stride=1, pad=0, cin=1280, cout=1000, group=1, act=None))
+    return dict(name="mobilenet_v2_035_int8", input=(3, 96, 96), layers=layers)
+
+
+def int8_params(arch, seed=0):
+    """Per-channel int8 weights ~U{-127..127}, per-channel scales sized like He initialisation, int32 biases."""
+    g = np.random.default_rng(seed)
+    params = []
+    for L in arch["layers"]:
+        if L["op"] != "conv":
+            params.append(None)
+            continue
+        cg = L["cin"] // L["group"]
+        fan_in = cg * L["k"] * L["k"]
+        w = g.integers(-127, 128, (L["cout"], cg, L["k"], L["k"]), dtype=np.int8)
+        ws = (np.sqrt(2.0 / fan_in) / 73.0 * g.uniform(0.5, 1.5, L["cout"])).astype(np.float32)
+        b = g.integers(-64, 65, L["cout"], dtype=np.int32)
+        params.append(dict(w=w, w_scale=ws, bias=b))
+    return params
+
+
+def int8_macs_per_inference(arch):
+    c, h, w = arch["input"]
+    macs = 0
+    for L in arch["layers"]:
+        if L["op"] == "conv":
+            oh = (h + 2 * L["pad"] - L["k"]) // L["stride"] + 1
+            ow = (w + 2 * L["pad"] - L["k"]) // L["stride"] + 1
+            macs += L["cout"] * oh * ow * (L["cin"] // L["group"]) * L["k"] * L["k"]
+            c, h, w = L["cout"], oh, ow
+        elif L["op"] == "pool":
+            h, w = h // 2, w // 2
+        elif L["op"] == "gap":
+            h, w = 1, 1
+    return macs
+
+
+def build_int8_model(ctx, arch, params, quant, batch):
+    """quant: {"input": [scale, zp], "layers": [[conv_scale, conv_zp, out_scale, out_zp] | [scale, zp] | None ...]}"""
+    from .model import Model, U8
+    m = Model(ctx)
+    c, h, w = arch["input"]
+    t = m.input((batch, c, h, w), U8, quant["input"][0], int(quant["input"][1]))
+    outs = []
+    for L, P, Q in zip(arch["layers"], params, quant["layers"]):
+        if L["op"] == "conv":
+            t = m.qlinearconv(t, P["w"], P["w_scale"], P["bias"], Q[0], int(Q[1]), [L["stride"]] * 2, [L["pad"]] * 4,
+                              [1, 1], L["group"])
+            if L["act"]:
+                t = m.qlinear_act(t, L["act"], L.get("alpha", 0.0), Q[2], int(Q[3]))
+        elif L["op"] == "pool":
+            t = m.maxpool(t, [2, 2], [2, 2])
+        elif L["op"] == "add":
+            t = m.qlinear_add(t, outs[L["res"]], Q[0], int(Q[1]))
+        elif L["op"] == "gap":
+            t = m.qlinear_global_avgpool(t, Q[0], int(Q[1]))
+        outs.append(t)
+    return m.finalize()
