@@ -8,6 +8,7 @@
 // MFMAs.  Rows of Y are the MFMA rows, columns the MFMA columns, so each accumulator register holds
 // 32 consecutive floats of a Y row (128-byte coalesced stores).
 #include "common.h"
+#include <type_traits>
 
 namespace {
 
@@ -23,7 +24,6 @@ struct GemmArgs {
     int c_ld_r, c_ld_c;      // 0 strides for broadcast axes
     int relu;
     int a_vec, b_vec;        // 16-byte vector loads are legal for A / B
-    int dbg;
 };
 
 // Loads 4 consecutive floats p[0..3]; elements at or beyond `valid` read as 0.
@@ -186,10 +186,14 @@ __device__ __attribute__((aligned(16))) const float g_gemm_zero[4] = {0.f, 0.f, 
 
 // How an operand panel [ROWS x 32 k] is staged.  KC*: the matrix is stored with k contiguous ([rows][K]);
 // RC4: stored with the row index contiguous ([K][rows]).  In LDS a "unit" is 4 consecutive k of one row (16 bytes):
-//   KC layout  unit(row, u) at row*8 + (u ^ (row & 7))   (XOR swizzle: a 128-byte global row segment lands in one
+//   KC layout  unit(row, u) at row*8 + (u ^ swz(row))     (XOR swizzle: a 128-byte global row segment lands in one
 //              128-byte LDS row, and lanes that read 32 different rows at the same u still hit 8 different columns)
 //   RC layout  unit(row, u) at u*ROWS + row
 enum { KC16 = 0, KC4 = 1, RC4 = 2 };
+
+// The LDS serves 128-bit reads 16 lanes at a time from 64 four-byte banks: 16 consecutive rows (two 128-byte rows
+// per 256-byte bank line) must land on 16 different 16-byte columns, so the XOR term steps every second row.
+__device__ __forceinline__ constexpr int swz(int row) { return (row >> 1) & 7; }
 
 template <int MODE, int ROWS>
 constexpr int stage_instrs() { return MODE == KC16 ? ROWS / 8 : ROWS / 2; }
@@ -207,12 +211,12 @@ __device__ __forceinline__ void stage_panel(float *dst, const float *__restrict_
         const float *sp;
         if (MODE == KC16) {
             const int U = i * 64 + lane, row = U >> 3, slot = U & 7;
-            const int k = k0 + ((slot ^ (row & 7)) << 2);
+            const int k = k0 + ((slot ^ swz(row)) << 2);
             sp = (r0 + row < R && k < K) ? src + int64_t(r0 + row) * ld + k : g_gemm_zero;
             __builtin_amdgcn_global_load_lds((gptr_t)sp, (lptr_t)(dst + i * 256), 16, 0, 0);
         } else if (MODE == KC4) {
             const int F = i * 64 + lane, row = F >> 5, slot = (F >> 2) & 7, j = F & 3;
-            const int k = k0 + ((slot ^ (row & 7)) << 2) + j;
+            const int k = k0 + ((slot ^ swz(row)) << 2) + j;
             sp = (r0 + row < R && k < K) ? src + int64_t(r0 + row) * ld + k : g_gemm_zero;
             __builtin_amdgcn_global_load_lds((gptr_t)sp, (lptr_t)(dst + i * 64), 4, 0, 0);
         } else {
@@ -234,10 +238,10 @@ __device__ __forceinline__ void stage_ptrs(const float *(&p)[stage_instrs<MODE, 
         const int i = ii * NW + wave;
         if (MODE == KC16) {
             const int U = i * 64 + lane, row = U >> 3, slot = U & 7;
-            p[ii] = src + int64_t(min(r0 + row, R - 1)) * ld + ((slot ^ (row & 7)) << 2);
+            p[ii] = src + int64_t(min(r0 + row, R - 1)) * ld + ((slot ^ swz(row)) << 2);
         } else if (MODE == KC4) {
             const int F = i * 64 + lane, row = F >> 5, slot = (F >> 2) & 7, j = F & 3;
-            p[ii] = src + int64_t(min(r0 + row, R - 1)) * ld + ((slot ^ (row & 7)) << 2) + j;
+            p[ii] = src + int64_t(min(r0 + row, R - 1)) * ld + ((slot ^ swz(row)) << 2) + j;
         } else {
             const int F = i * 64 + lane, j = F & 3, row = (F >> 2) % ROWS, u = F / (4 * ROWS);
             p[ii] = src + int64_t((u << 2) + j) * ld + min(r0 + row, R - 1);
@@ -257,10 +261,18 @@ __device__ __forceinline__ void stage_fast(float *dst, const float *const (&p)[s
     }
 }
 
+// Copy instruction ii of this wave's share of a panel (fast path).
+template <int MODE, int NW>
+__device__ __forceinline__ void stage_fast_one(float *dst, const float *p, int64_t koff, int wave, int ii) {
+    const int i = ii * NW + wave;
+    if (MODE == KC16) __builtin_amdgcn_global_load_lds((gptr_t)(p + koff), (lptr_t)(dst + i * 256), 16, 0, 0);
+    else __builtin_amdgcn_global_load_lds((gptr_t)(p + koff), (lptr_t)(dst + i * 64), 4, 0, 0);
+}
+
 // LDS float offset of unit (row, u) of a panel.
 template <int MODE, int ROWS>
 __device__ __forceinline__ int unit_off(int row, int u) {
-    return MODE == RC4 ? (u * ROWS + row) * 4 : (row * 8 + (u ^ (row & 7))) * 4;
+    return MODE == RC4 ? (u * ROWS + row) * 4 : (row * 8 + (u ^ swz(row))) * 4;
 }
 
 // Operand reads and their waits are written by hand.  The compiler cannot count LDS reads that are still in flight
@@ -314,18 +326,24 @@ __device__ __forceinline__ void gemm_step(float *__restrict__ dma, unsigned cmp_
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave % WM, wn = wave / WM;
     const int l32 = lane & 31, lh = lane >> 5;
-    if (g.dbg & 1) {} else
-    if ((ichunk + 1) * BK <= g.K) {  // whole chunk inside K: no masks, addresses are a uniform offset from chunk 0
-        stage_fast<AM, BM, NW>(dma, pa, AM == RC4 ? int64_t(ichunk) * BK * g.lda : int64_t(ichunk) * BK, wave);
-        stage_fast<BMODE, BN, NW>(dma + BM * BK, pb, BMODE == RC4 ? int64_t(ichunk) * BK * g.ldb : int64_t(ichunk) * BK, wave);
-    } else {
+    constexpr int PA = stage_instrs<AM, BM>() / NW, PB = stage_instrs<BMODE, BN>() / NW;
+    static_assert(PA + PB <= 4 * MT * (BK / 8), "one copy instruction per MFMA at most");
+    // Whole chunk inside K: no masks, addresses are a uniform offset from chunk 0, and the copy instructions are
+    // spread between the MFMAs (each is issued while the previous MFMA of the dependent chain executes).  Otherwise
+    // (the K tail and the zero chunks behind it) the masked copies are issued up front.
+    const bool fast = (ichunk + 1) * BK <= g.K;
+    const int64_t koffa = AM == RC4 ? int64_t(ichunk) * BK * g.lda : int64_t(ichunk) * BK;
+    const int64_t koffb = BMODE == RC4 ? int64_t(ichunk) * BK * g.ldb : int64_t(ichunk) * BK;
+    if (!fast) {
         stage_panel<AM, BM, NW>(dma, A, g.lda, m0, g.M, ichunk * BK, g.K, wave, lane);
         stage_panel<BMODE, BN, NW>(dma + BM * BK, B, g.ldb, n0, g.N, ichunk * BK, g.K, wave, lane);
     }
     __builtin_amdgcn_sched_barrier(0);
 
-    if (g.dbg & 2) return;
     static_assert((BK / 8) % 2 == 0, "group 0 of every chunk uses operand registers 0");
+    auto multiply = [&](auto fast_c) {
+    constexpr bool FAST = decltype(fast_c)::value;
+    int q = 0;  // MFMAs issued so far in this step (a constant after unrolling)
 #pragma unroll
     for (int gi = 0; gi < BK / 8; ++gi) {
         const int cur = gi & 1;
@@ -335,14 +353,22 @@ __device__ __forceinline__ void gemm_step(float *__restrict__ dma, unsigned cmp_
         if (gi + 1 < BK / 8) read_group<MT, AM, BMODE, BM, BN>(cmp_addr, gi + 1, offa, offb, a[cur ^ 1], b[cur ^ 1]);
         else read_group<MT, AM, BMODE, BM, BN>(nxt_addr, 0, offa, offb, a[0], b[0]);
         lds_wait<MT + 1, MT>(a[cur], b[cur]);  // everything but the MT + 1 reads just issued has landed
-        __builtin_amdgcn_s_setprio(1);
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int i = 0; i < MT; ++i)
+            for (int i = 0; i < MT; ++i) {
                 acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][i][j], b[cur][j], acc[i], 0, 0, 0);
-        __builtin_amdgcn_s_setprio(0);
+                if (FAST) {
+                    if (q < PA) stage_fast_one<AM, NW>(dma, pa[q < PA ? q : 0], koffa, wave, q);
+                    else if (q < PA + PB) stage_fast_one<BMODE, NW>(dma + BM * BK, pb[q >= PA && q < PA + PB ? q - PA : 0], koffb, wave, q - PA);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                ++q;
+            }
     }
+    };
+    if (fast) multiply(std::true_type{});
+    else multiply(std::false_type{});
 }
 
 // s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt in bits 3:0 and 15:14).
@@ -455,9 +481,8 @@ gemm_f32_dma_kernel(const float *__restrict__ A, const float *__restrict__ B, co
     }
 }
 
-template <int MT, int WM, int WN, int AM, int BMODE>
+template <int MT, int WM, int WN, int AM, int BMODE, int S = 5>
 void launch_gemm_dma(zant_ctx *ctx, const float *A, const float *B, const float *C, float *Y, const GemmArgs &g) {
-    constexpr int S = 5;
     constexpr int BM = WM * MT * 32, BN = WN * 32;
     constexpr size_t lds_bytes = size_t(S) * (BM + BN) * BK * sizeof(float);
     auto kern = &gemm_f32_dma_kernel<MT, WM, WN, AM, BMODE, S>;
@@ -503,23 +528,13 @@ int run_gemm(zant_ctx *ctx, const float *A, const float *B, const float *C, floa
     g.alpha = alpha; g.beta = beta;
     g.c_mode = c_mode; g.c_ld_r = int(c_ld_r); g.c_ld_c = int(c_ld_c);
     g.relu = relu;
-    g.dbg = getenv("ZANT_GEMM_DBG") ? atoi(getenv("ZANT_GEMM_DBG")) : 0;
     g.a_vec = (reinterpret_cast<uintptr_t>(A) & 15) == 0 && (g.lda & 3) == 0;
     g.b_vec = (reinterpret_cast<uintptr_t>(B) & 15) == 0 && (g.ldb & 3) == 0;
     const bool a_kc = !trans_a, b_kc = trans_b;
     KernelTimer kt(ctx);
     const int am = a_kc ? (g.a_vec ? KC16 : KC4) : RC4;
     const int bmode = b_kc ? (g.b_vec ? KC16 : KC4) : RC4;
-    const char *cfg = getenv("ZANT_GEMM_CFG");
-    int c = cfg ? atoi(cfg) : 0;
-    if (c == 1) launch_gemm_dma<1, 2, 2, KC16, RC4>(ctx, A, B, C, Y, g);
-    else if (c == 2) launch_gemm_dma<2, 2, 2, KC16, RC4>(ctx, A, B, C, Y, g);
-    else if (c == 3) launch_gemm_dma<1, 2, 4, KC16, RC4>(ctx, A, B, C, Y, g);
-    else if (c == 4) launch_gemm_dma<2, 1, 4, KC16, RC4>(ctx, A, B, C, Y, g);
-    else if (c == 5) launch_gemm_dma<1, 4, 1, KC16, RC4>(ctx, A, B, C, Y, g);
-    else if (c == 6) launch_gemm_dma<2, 2, 1, KC16, RC4>(ctx, A, B, C, Y, g);
-    else
-    if (N > 32) dispatch_gemm_dma<1, 4, 2>(ctx, A, B, C, Y, g, am, bmode);  // 128 x 64 tile, 8 waves
+    if (N > 32) dispatch_gemm_dma<1, 4, 2>(ctx, A, B, C, Y, g, am, bmode);  // 128 x 64 tile, 8 waves, 5 stages
     else launch_gemm<1, 4, 1>(ctx, A, B, C, Y, g, a_kc, b_kc);              // 128 x 32 tile
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
