@@ -57,7 +57,8 @@ enum zant_auto_pad { ZANT_PAD_NOTSET = 0, ZANT_PAD_SAME_UPPER = 1, ZANT_PAD_SAME
 
 /* Activation fused into a producing kernel, or applied in dequantised space
  * between two quantised tensors. */
-enum zant_act { ZANT_ACT_NONE = 0, ZANT_ACT_RELU = 1, ZANT_ACT_LEAKY = 2, ZANT_ACT_RELU6 = 3 };
+enum zant_act { ZANT_ACT_NONE = 0, ZANT_ACT_RELU = 1, ZANT_ACT_LEAKY = 2, ZANT_ACT_RELU6 = 3,
+                ZANT_ACT_SOFTMAX = 4 /* zant_hip_gemm_f32 only: lean_softmax over every output row */ };
 
 /* ---- context, memory, timing ------------------------------------------------ */
 
@@ -122,7 +123,9 @@ int zant_hip_matmul_check(const int64_t *adim, int a_rank, const int64_t *bdim, 
 
 /* gemm_lean = lean_gemm (op_gemm.zig:91-185): Y = alpha*op(A)*op(B) + beta*C on
  * {1,1,R,C} tensors, C broadcast over rows and/or columns.  Transposes are folded
- * into the loads.  fuse_act as for conv. */
+ * into the loads.  fuse_act as for conv; ZANT_ACT_SOFTMAX (the classifier head Gemm -> Softmax in one kernel,
+ * reference op_softmax.zig lean_softmax on the [rows, cols] result) is accepted for cols <= 16 without trans_a
+ * and returns InvalidInput otherwise. */
 int zant_hip_gemm_f32(zant_ctx *ctx, const float *a, const int64_t adim[4], const float *b, const int64_t bdim[4],
                       const float *c, const int64_t *cdim, int c_rank, float alpha, float beta, int trans_a,
                       int trans_b, float *y, const int64_t ydim[4], int fuse_act);

@@ -178,7 +178,8 @@ def test_conv_vs_oracle(G, case, relu):
     np.testing.assert_allclose(G.host(y), ref, rtol=G.RTOL, atol=G.ATOL)
 
 
-GEMM_CASES = [(64, 96, 48), (130, 70, 33), (1, 256, 10), (257, 1600, 512), (33, 5, 7), (128, 512, 10)]
+GEMM_CASES = [(64, 96, 48), (130, 70, 33), (1, 256, 10), (257, 1600, 512), (33, 5, 7), (128, 512, 10), (67, 1100, 16),
+              (19, 513, 1), (200, 64, 17)]
 
 
 @pytest.mark.parametrize("M,K,N", GEMM_CASES)
@@ -197,6 +198,26 @@ def test_gemm_vs_oracle(G, M, K, N, ta, tb):
         y = torch.full(ref.shape, -7.0, device="cuda:0")
         G.tm.gemm_lean(G.dev(a), G.dev(b), G.dev(c), alpha, beta, ta, tb, y, act)
         np.testing.assert_allclose(G.host(y), ref, rtol=G.RTOL, atol=G.ATOL)
+
+
+@pytest.mark.parametrize("M,K,N,tb", [(4096, 512, 10, 0), (37, 700, 16, 1), (5, 3, 2, 0), (64, 1024, 7, 0)])
+def test_gemm_with_fused_row_softmax(G, M, K, N, tb):
+    """The classifier head in one kernel: Gemm, then lean_softmax over each row of the [M, N] result."""
+    import torch
+    g = np.random.default_rng(M + K + N)
+    a = g.standard_normal((1, 1, M, K), dtype=np.float32)
+    b = (g.standard_normal((1, 1, N, K) if tb else (1, 1, K, N)) * np.sqrt(2.0 / K)).astype(np.float32)
+    c = (g.standard_normal((1, 1, 1, N)) * 0.1).astype(np.float32)
+    ref = zo.softmax(zo.gemm(a, b, c, 1.0, 1.0, False, bool(tb)).reshape(M, N))
+    y = torch.full((1, 1, M, N), -7.0, device="cuda:0")
+    G.tm.gemm_lean(G.dev(a), G.dev(b), G.dev(c), 1.0, 1.0, False, bool(tb), y, "softmax")
+    np.testing.assert_allclose(G.host(y).reshape(M, N), ref, rtol=G.RTOL, atol=G.ATOL)
+    np.testing.assert_allclose(G.host(y).reshape(M, N).sum(axis=1), 1.0, rtol=1e-5)
+    # not available for wide or transposed-A products
+    with pytest.raises(G.ZantError) as e:
+        G.tm.gemm_lean(torch.zeros(1, 1, 8, 4, device="cuda:0"), torch.zeros(1, 1, 4, 32, device="cuda:0"), None, 1.0, 1.0,
+                       False, False, torch.zeros(1, 1, 8, 32, device="cuda:0"), "softmax")
+    assert e.value.name == "InvalidInput"
 
 
 def test_matmul_vs_oracle_and_ignored_batch_dims(G):

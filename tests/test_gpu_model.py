@@ -54,9 +54,9 @@ def test_readme_cnn_matches_oracle_and_plans_one_arena(G):
     y = m.predict_host(x)
     ref = np.concatenate([oracle_readme_cnn(x[i:i + 1], params) for i in range(batch)])
     np.testing.assert_allclose(y, ref, rtol=G.RTOL, atol=G.ATOL)
-    # 12 nodes: 3 ReLUs ride in their producers, 2 Reshapes are views, the first MaxPool is computed inside the
-    # few-channel first convolution -> 6 kernel-launching nodes
-    assert m.num_launches == 6
+    # 12 nodes: 3 ReLUs ride in their producers, 2 Reshapes are views, both MaxPools are computed inside their
+    # convolutions, the Softmax inside the last Gemm -> 4 kernel-launching nodes
+    assert m.num_launches == 4  # conv+relu+pool, conv+relu+pool, gemm+relu, gemm+softmax
     # liveness planning: the arena is much smaller than one static array per node output
     assert m.arena_bytes < 0.6 * m.unfused_bytes
 
@@ -148,6 +148,34 @@ def test_predict_entry_point_follows_the_reference_abi(G):
     arr = (C.c_uint32 * 4)(1, 1, 28, 28)
     lib.predict(img.ctypes.data_as(C.c_void_p), arr, 4, C.byref(result2))
     assert result2.value is None  # no model bound: nothing happens
+
+
+@pytest.mark.parametrize("N,C,H,W,K,k,pad,relu", [
+    (9, 32, 12, 12, 64, 3, 0, True),     # the README CNN's second layer: several images per tile
+    (3, 16, 41, 37, 40, 3, 1, True),     # odd conv rows and columns (the pool drops the last), K not a multiple of 32
+    (2, 8, 70, 66, 96, 3, 1, False),     # several row tiles per image, three output-channel blocks, no ReLU
+    (5, 12, 20, 20, 32, (2, 3), 1, True),  # 2x3 filter (generic tap loop), 32-channel workgroups
+])
+def test_conv_with_fused_pool_on_the_matrix_cores(G, N, C, H, W, K, k, pad, relu):
+    from zant_amd.model import Model
+    g = np.random.default_rng(N * 1000 + C)
+    x = g.standard_normal((N, C, H, W), dtype=np.float32)
+    kh, kw = k if isinstance(k, tuple) else (k, k)
+    w = (g.standard_normal((K, C, kh, kw)) * np.sqrt(2.0 / (C * kh * kw))).astype(np.float32)
+    b = (g.standard_normal(K) * 0.1).astype(np.float32)
+    m = Model(G.tm.context())
+    t = m.conv(m.input((N, C, H, W)), w, b, [1, 1], [pad] * 4, [1, 1], 1, "NOTSET")
+    if relu:
+        t = m.relu(t)
+    t = m.maxpool(t, [2, 2], [2, 2])
+    m.finalize()
+    assert m.num_launches == 1
+    ref = zo.Conv(x, w, b, [1, 1], [pad] * 4, [1, 1], 1, "NOTSET")
+    if relu:
+        ref = zo.ReLU(ref)
+    ref = zo.onnx_maxpool(ref, [2, 2], [2, 2], [1, 1], [0, 0, 0, 0])
+    np.testing.assert_allclose(m.predict_host(x), ref, rtol=G.RTOL, atol=G.ATOL)
+    m.close()
 
 
 def test_int8_network_fuses_activation_and_is_bit_exact(G):

@@ -79,7 +79,7 @@ int zant_conv_resolve(const int64_t xdim[4], const int64_t wdim[4], const int64_
                       const int64_t *pads, int n_pads, const int64_t *dil, int n_dil, int64_t group,
                       const char *auto_pad, int64_t s[2], int64_t d[2], int64_t p[4]);
 
-// Internal (not part of the C ABI): Conv (+ReLU) + MaxPool 2x2/2 fused for few-channel first layers.
+// Internal (not part of the C ABI): Conv (+ReLU) + MaxPool 2x2/2 fused into the convolution kernels.
 // Returns ZANT_OK, a negative status, or 1 when the shape is not eligible.  query_only: just say whether it is.
 int zant_conv2d_f32_fused_pool(zant_ctx *ctx, const float *x, const int64_t xdim[4], const float *w, const int64_t wdim[4],
                                const float *bias, float *y, const int64_t ydim[4], const int64_t *stride, int n_stride,

@@ -176,7 +176,7 @@ __device__ __forceinline__ void conv_step(float *__restrict__ dma, const float *
 // asynchronous (global_load_lds, no VGPR round trip) and run one (tile, chunk) step ahead of the
 // matrix cores, across tile boundaries as well: while a tile's bias/ReLU epilogue stores drain, the
 // first chunk of the workgroup's next tile is already landing.  Tiles are drawn from an atomic counter.
-template <int MT, int WM, int WN, int KV, int TT>
+template <int MT, int WM, int WN, int KV, int TT, bool POOL = false>
 __global__ void __launch_bounds__(WM *WN * 64, 2)
 conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, const float *__restrict__ bias,
                      float *__restrict__ y, ConvGeom g, TileGeom t, int relu, int *__restrict__ tile_counter) {
@@ -207,12 +207,25 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
         v.y = (img << 16) | ph;
         ptab[e] = v;
     }
+    // With a fused 2x2/2 max pool the lane's tile registers 4j .. 4j+3 are the four members of ONE pooling window
+    // (pooled position (wm*MT/4 + j)*32 + l32), so the pool is a register-wise max in the epilogue.
+    const int per_img_p = POOL ? (t.TH / 2) * t.POW : 0;
     int lds_off[MT];  // float4 index of each of this lane's output positions inside a patch half
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
-        const int p = (wm * MT + i) * 32 + l32;
-        const int img = p / per_img, rem = p - img * per_img;
-        const int r = rem / g.OW, c = rem - r * g.OW;
+        int img, r, c;
+        if (POOL) {
+            const int pp = (wm * (MT / 4) + i / 4) * 32 + l32;
+            img = pp / per_img_p;
+            const int rem = pp - img * per_img_p, pr = rem / t.POW;
+            r = 2 * pr + ((i & 3) >> 1);
+            c = 2 * (rem - pr * t.POW) + (i & 1);
+        } else {
+            const int p = (wm * MT + i) * 32 + l32;
+            img = p / per_img;
+            const int rem = p - img * per_img;
+            r = rem / g.OW; c = rem - r * g.OW;
+        }
         lds_off[i] = (img < t.NB && r < t.TH) ? (img * t.PH + r * g.sh) * t.PW + c * g.sw : 0;
     }
     if (tid == 0) sched[0] = blockIdx.x + gridDim.x;  // the second tile is static, later ones come from the counter
@@ -292,6 +305,29 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
                 const int k = kbase + (v >> 2) * 8 + (v & 3);
                 bv[v] = (bias != nullptr && k < g.K) ? bias[k] : 0.0f;
             }
+            if constexpr (POOL) {
+                // max over the window, then bias and ReLU: both are monotone, so this equals pool(relu(conv + bias))
+                const int prows_here = min(t.TH / 2, g.OH / 2 - oh0 / 2);
+                const int64_t pplane = int64_t(g.OH / 2) * t.POW;
+#pragma unroll
+                for (int j = 0; j < MT / 4; ++j) {
+                    const int pp = (wm * (MT / 4) + j) * 32 + l32;
+                    const int img = pp / per_img_p, rem = pp - img * per_img_p;
+                    const int pr = rem / t.POW, pc = rem - pr * t.POW;
+                    if (img < imgs_here && pr < prows_here) {
+                        float *yp = y + (int64_t(n0 + img) * g.K + kbase) * pplane + int64_t(oh0 / 2 + pr) * t.POW + pc;
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            const int dk = (v >> 2) * 8 + (v & 3);
+                            if (full_k || kbase + dk < g.K) {
+                                float o = fmaxf(fmaxf(acc[4 * j][v], acc[4 * j + 1][v]), fmaxf(acc[4 * j + 2][v], acc[4 * j + 3][v])) + bv[v];
+                                if (relu) o = o > 0.0f ? o : 0.0f;
+                                yp[dk * pplane] = o;
+                            }
+                        }
+                    }
+                }
+            } else
 #pragma unroll
             for (int i = 0; i < MT; ++i) {
                 const int p = (wm * MT + i) * 32 + l32;
@@ -440,49 +476,88 @@ conv_f32_smallc_pool_kernel(const float *__restrict__ x, const float *__restrict
 typedef TilePlan MfmaPlan;
 
 // Tile shape with the best useful-lane fraction whose LDS footprint allows two workgroups per CU.
-bool plan_mfma(const ConvGeom &g, MfmaPlan *best) {
+bool plan_mfma(const ConvGeom &g, MfmaPlan *best, bool pool = false) {
     const int WN = g.K > 32 ? 2 : 1, WM = 4 / WN;
-    return zant_plan_conv_tiles(g, WM, WN, 8, CC, sizeof(float), 80 * 1024, best);
+    return zant_plan_conv_tiles(g, WM, WN, 8, CC, sizeof(float), 80 * 1024, best, pool);
 }
 
-template <int MT, int WM, int WN, int TT>
+template <int MT, int WM, int WN, int TT, bool POOL>
 void launch_mfma_tt(zant_ctx *ctx, const float *x, const float *wp, const float *bias, float *y, const ConvGeom &g,
                     const MfmaPlan &p, int relu, int *counter, int grid) {
     constexpr int KV = MT >= 8 ? 2 : 4;  // 64-bit operand reads keep 8 accumulator tiles inside 256 VGPRs
     // more than 64 KB of dynamic LDS has to be opted into once per kernel
     static bool attr_set = false;
     if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&conv_f32_mfma_kernel<MT, WM, WN, KV, TT>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&conv_f32_mfma_kernel<MT, WM, WN, KV, TT, POOL>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         attr_set = true;
     }
-    hipLaunchKernelGGL((conv_f32_mfma_kernel<MT, WM, WN, KV, TT>), dim3(grid), dim3(WM * WN * 64), p.lds_bytes,
+    hipLaunchKernelGGL((conv_f32_mfma_kernel<MT, WM, WN, KV, TT, POOL>), dim3(grid), dim3(WM * WN * 64), p.lds_bytes,
                        ctx->stream, x, wp, bias, y, g, p.t, relu, counter);
 }
 
-template <int MT, int WM, int WN>
+template <int MT, int WM, int WN, bool POOL>
 void launch_mfma(zant_ctx *ctx, const float *x, const float *wp, const float *bias, float *y, const ConvGeom &g,
                  const MfmaPlan &p, int relu, int *counter, int grid) {
     const int T = g.KH * g.KW;
-    if (T == 9) launch_mfma_tt<MT, WM, WN, 9>(ctx, x, wp, bias, y, g, p, relu, counter, grid);
-    else if (T == 1) launch_mfma_tt<MT, WM, WN, 1>(ctx, x, wp, bias, y, g, p, relu, counter, grid);
-    else launch_mfma_tt<MT, WM, WN, 0>(ctx, x, wp, bias, y, g, p, relu, counter, grid);
+    if (T == 9) launch_mfma_tt<MT, WM, WN, 9, POOL>(ctx, x, wp, bias, y, g, p, relu, counter, grid);
+    else if (T == 1 && !POOL) launch_mfma_tt<MT, WM, WN, 1, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid);
+    else launch_mfma_tt<MT, WM, WN, 0, POOL>(ctx, x, wp, bias, y, g, p, relu, counter, grid);
 }
 
 template <int WM, int WN>
 bool dispatch_mt(zant_ctx *ctx, const float *x, const float *wp, const float *bias, float *y, const ConvGeom &g,
-                 const MfmaPlan &p, int relu, int *counter, int grid) {
+                 const MfmaPlan &p, int relu, int *counter, int grid, bool pool) {
+    if (pool) {
+        switch (p.MT) {
+        case 4: launch_mfma<4, WM, WN, true>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
+        case 8: launch_mfma<8, WM, WN, true>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
+        default: return false;
+        }
+    }
     switch (p.MT) {
-    case 1: launch_mfma<1, WM, WN>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
-    case 2: launch_mfma<2, WM, WN>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
-    case 3: launch_mfma<3, WM, WN>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
-    case 4: launch_mfma<4, WM, WN>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
-    case 5: launch_mfma<5, WM, WN>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
-    case 6: launch_mfma<6, WM, WN>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
-    case 7: launch_mfma<7, WM, WN>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
-    case 8: launch_mfma<8, WM, WN>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
+    case 1: launch_mfma<1, WM, WN, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
+    case 2: launch_mfma<2, WM, WN, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
+    case 3: launch_mfma<3, WM, WN, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
+    case 4: launch_mfma<4, WM, WN, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
+    case 5: launch_mfma<5, WM, WN, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
+    case 6: launch_mfma<6, WM, WN, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
+    case 7: launch_mfma<7, WM, WN, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
+    case 8: launch_mfma<8, WM, WN, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
     default: return false;
     }
+}
+
+// Whether the implicit-GEMM kernel takes this convolution (optionally with the fused 2x2/2 max pool), and its plan.
+bool mfma_eligible(const ConvGeom &g, bool pool, MfmaPlan *plan) {
+    const int64_t macs_per_out = int64_t(g.C) * g.KH * g.KW;
+    const bool want = g.C >= 4 && macs_per_out >= 32 && int64_t(g.N) * g.OH * g.OW >= 64 &&
+                      int64_t(g.N) * g.C * g.H * g.W < (int64_t(1) << 40);
+    return want && plan_mfma(g, plan, pool) && plan->eff >= 0.5;
+}
+
+// Packs the weights, resets the tile counter and launches the persistent implicit-GEMM kernel.
+int run_conv_mfma(zant_ctx *ctx, const float *x, const float *w, const float *bias, float *y, const ConvGeom &g,
+                  const MfmaPlan &plan, int relu, bool pool) {
+    const int T = g.KH * g.KW, K_BLK = plan.WN * 32;
+    const size_t wp_floats = size_t(plan.t.n_chunks) * plan.t.n_kblocks * T * CC * K_BLK;
+    void *ws = nullptr;
+    int rc = zant_workspace(ctx, 256 + wp_floats * sizeof(float), &ws);  // [tile counter | packed weights]
+    if (rc) return rc;
+    int *counter = static_cast<int *>(ws);
+    float *wp = reinterpret_cast<float *>(static_cast<char *>(ws) + 256);
+    // persistent workgroups: two per CU; the first two tiles of each are static, the rest dynamic
+    const int grid = int(std::min<int64_t>(plan.t.n_tiles, int64_t(ctx->num_cus) * 2));
+    const unsigned pb = unsigned(std::min<int64_t>(ceil_div64(int64_t(wp_floats), 256), 1024));
+    hipLaunchKernelGGL(pack_weights_f32_kernel, dim3(pb), dim3(256), 0, ctx->stream, w, wp, g.K, g.C, T,
+                       plan.t.n_chunks, plan.t.n_kblocks, K_BLK, counter, 2 * grid);
+    ZANT_LAUNCH_CHECK(ctx);
+    KernelTimer kt(ctx);
+    const bool ok = plan.WN == 2 ? dispatch_mt<2, 2>(ctx, x, wp, bias, y, g, plan, relu, counter, grid, pool)
+                                 : dispatch_mt<4, 1>(ctx, x, wp, bias, y, g, plan, relu, counter, grid, pool);
+    if (!ok) return 1;
+    ZANT_LAUNCH_CHECK(ctx);
+    return ZANT_OK;
 }
 
 }  // namespace
@@ -588,30 +663,11 @@ extern "C" int zant_hip_conv2d_f32(zant_ctx *ctx, const float *x, const int64_t 
     zant_log("OnnxConvLean2");
 
     MfmaPlan plan;
-    const int64_t macs_per_out = int64_t(g.C) * g.KH * g.KW;
-    const bool want_mfma = g.C >= 4 && macs_per_out >= 32 && int64_t(g.N) * g.OH * g.OW >= 64 &&
-                           int64_t(g.N) * g.C * g.H * g.W < (int64_t(1) << 40);
-    if (want_mfma && plan_mfma(g, &plan) && plan.eff >= 0.5) {
-        const int T = g.KH * g.KW, K_BLK = plan.WN * 32;
-        const size_t wp_floats = size_t(plan.t.n_chunks) * plan.t.n_kblocks * T * CC * K_BLK;
-        void *ws = nullptr;
-        rc = zant_workspace(ctx, 256 + wp_floats * sizeof(float), &ws);  // [tile counter | packed weights]
-        if (rc) return rc;
-        int *counter = static_cast<int *>(ws);
-        float *wp = reinterpret_cast<float *>(static_cast<char *>(ws) + 256);
-        // persistent workgroups: two per CU; the first two tiles of each are static, the rest dynamic
-        const int grid = int(std::min<int64_t>(plan.t.n_tiles, int64_t(ctx->num_cus) * 2));
-        const unsigned pb = unsigned(std::min<int64_t>(ceil_div64(int64_t(wp_floats), 256), 1024));
-        hipLaunchKernelGGL(pack_weights_f32_kernel, dim3(pb), dim3(256), 0, ctx->stream, w, wp, g.K, g.C, T,
-                           plan.t.n_chunks, plan.t.n_kblocks, K_BLK, counter, 2 * grid);
-        ZANT_LAUNCH_CHECK(ctx);
-        KernelTimer kt(ctx);
-        bool ok = plan.WN == 2 ? dispatch_mt<2, 2>(ctx, x, wp, bias, y, g, plan, relu, counter, grid)
-                               : dispatch_mt<4, 1>(ctx, x, wp, bias, y, g, plan, relu, counter, grid);
-        if (ok) {
-            ZANT_LAUNCH_CHECK(ctx);
-            zant_log("OnnxConvLean4");
-            return ZANT_OK;
+    if (mfma_eligible(g, false, &plan)) {
+        rc = run_conv_mfma(ctx, x, w, bias, y, g, plan, relu, false);
+        if (rc <= 0) {
+            if (rc == ZANT_OK) zant_log("OnnxConvLean4");
+            return rc;
         }
     }
     const int ckk = g.C * g.KH * g.KW;
@@ -636,7 +692,8 @@ extern "C" int zant_hip_conv2d_f32(zant_ctx *ctx, const float *x, const int64_t 
     return ZANT_OK;
 }
 
-// Conv (+ReLU) + MaxPool 2x2/2 in one kernel for few-channel first layers; returns 1 when the shape is
+// Conv (+ReLU) + MaxPool 2x2/2 in one kernel (few-channel first layers: direct kernel; many-channel layers: the
+// implicit-GEMM kernel with a register-wise pool in its epilogue); returns 1 when the shape is
 // not one this kernel takes (the caller then runs the two operators separately).
 int zant_conv2d_f32_fused_pool(zant_ctx *ctx, const float *x, const int64_t xdim[4], const float *w, const int64_t wdim[4],
                                const float *bias, float *y, const int64_t ydim[4], const int64_t *stride, int n_stride,
@@ -647,15 +704,23 @@ int zant_conv2d_f32_fused_pool(zant_ctx *ctx, const float *x, const int64_t xdim
     if (s[0] != 1 || s[1] != 1 || d[0] != 1 || d[1] != 1 || xdim[1] != wdim[1]) return 1;
     const int C = int(wdim[1]), KH = int(wdim[2]), KW = int(wdim[3]);
     const bool k133 = C == 1 && KH == 3 && KW == 3, k155 = C == 1 && KH == 5 && KW == 5, k333 = C == 3 && KH == 3 && KW == 3;
-    if (!k133 && !k155 && !k333) return 1;
     const int64_t OH = xdim[2] + p[0] + p[2] - KH + 1, OW = xdim[3] + p[1] + p[3] - KW + 1;
     if (OH < 2 || OW < 2) return 1;
     if (ydim[0] != xdim[0] || ydim[1] != wdim[0] || ydim[2] != OH / 2 || ydim[3] != OW / 2) return 1;
-    if (query_only) return ZANT_OK;
+    for (int i = 0; i < 4; ++i)
+        if (xdim[i] <= 0 || wdim[i] <= 0 || xdim[i] > INT32_MAX || wdim[i] > INT32_MAX) return 1;
     ConvGeom g;
     g.N = int(xdim[0]); g.C = C; g.H = int(xdim[2]); g.W = int(xdim[3]);
     g.K = int(wdim[0]); g.CG = C; g.KH = KH; g.KW = KW; g.OH = int(OH); g.OW = int(OW);
     g.sh = g.sw = g.dh = g.dw = 1; g.pt = int(p[0]); g.pl = int(p[1]); g.groups = 1;
+    if (!k133 && !k155 && !k333) {
+        // many-channel layers: the implicit-GEMM kernel with the pool folded into its epilogue
+        MfmaPlan plan;
+        if (!mfma_eligible(g, true, &plan) || (plan.MT != 4 && plan.MT != 8)) return 1;
+        if (query_only) return ZANT_OK;
+        return run_conv_mfma(ctx, x, w, bias, y, g, plan, relu, true);
+    }
+    if (query_only) return ZANT_OK;
     const int POH = int(OH / 2), POW = int(OW / 2);
     const int64_t positions = int64_t(g.N) * POH * POW;
     const unsigned pb = unsigned(std::min<int64_t>(ceil_div64(positions, 256), int64_t(ctx->num_cus) * 16));

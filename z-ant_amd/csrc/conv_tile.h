@@ -16,6 +16,7 @@ struct TileGeom {
     int n_kblocks;       // ceil(K / K_BLK)
     int n_sblocks;       // spatial tiles
     int n_tiles;         // n_sblocks * n_kblocks
+    int POW;             // fused 2x2/2 max pool: pooled columns (OW / 2); 0 = no pooling
 };
 
 struct TilePlan {
@@ -40,24 +41,33 @@ __device__ __forceinline__ void decode_tile(const TileGeom &t, int tile, int &n0
 // Best tile shape for WM x WN waves (WN*32 output channels per workgroup) among MT = mt_max..1 whose
 // two staging buffers, patch table and scheduler slots fit in `lds_cap` bytes.
 // chunk_channels: input channels per chunk; elem_bytes: bytes per input element.
+// pool: the kernel's epilogue max-pools 2x2/2 (floor).  The MFMA column slots are then counted in POOLED positions:
+// tile registers 4j..4j+3 of a lane hold the four members of one window, so MT is a multiple of 4, TH is even and
+// a tile covers NB images x TH/2 pooled rows x OW/2 pooled columns.
 inline bool zant_plan_conv_tiles(const ConvGeom &g, int WM, int WN, int mt_max, int chunk_channels, size_t elem_bytes,
-                                 size_t lds_cap, TilePlan *best) {
+                                 size_t lds_cap, TilePlan *best, bool pool = false) {
     const int T = g.KH * g.KW;
     const int K_BLK = WN * 32;
     bool found = false;
     for (int mt = mt_max; mt >= 1; --mt) {
-        const int S = WM * mt * 32;
-        const int per_img = g.OH * g.OW;
+        if (pool && (mt & 3)) continue;
+        const int S = pool ? WM * (mt / 4) * 32 : WM * mt * 32;      // position slots (pooled positions when pooling)
+        const int rows = pool ? g.OH / 2 : g.OH, cols = pool ? g.OW / 2 : g.OW;
+        if (rows < 1 || cols < 1) continue;
+        const int per_img = rows * cols;
         TileGeom t;
+        t.POW = pool ? cols : 0;
+        int th;  // rows (pooled rows) per tile
         if (per_img <= S) {
-            t.NB = S / per_img; t.TH = g.OH;
+            t.NB = S / per_img; th = rows;
             if (t.NB > g.N) t.NB = g.N;
         } else {
-            t.NB = 1; t.TH = S / g.OW;
-            if (t.TH < 1) continue;
+            t.NB = 1; th = S / cols;
+            if (th < 1) continue;
         }
-        t.n_row_tiles = (g.OH + t.TH - 1) / t.TH;
-        t.TH = (g.OH + t.n_row_tiles - 1) / t.n_row_tiles;  // even out the rows over the row tiles
+        t.n_row_tiles = (rows + th - 1) / th;
+        th = (rows + t.n_row_tiles - 1) / t.n_row_tiles;  // even out the rows over the row tiles
+        t.TH = pool ? 2 * th : th;
         t.PH = (t.TH - 1) * g.sh + (g.KH - 1) * g.dh + 1;
         t.PW = (g.OW - 1) * g.sw + (g.KW - 1) * g.dw + 1;
         t.P1 = t.NB * t.PH * t.PW;
@@ -73,7 +83,7 @@ inline bool zant_plan_conv_tiles(const ConvGeom &g, int WM, int WN, int mt_max, 
         const size_t lds = 2 * (size_t(T) * 32 * K_BLK + size_t(32) * t.P1s)  // two staging buffers
                            + size_t(t.P1s) * 8 + 8;                          // patch table, scheduler slots
         if (lds > lds_cap) continue;
-        const double eff = double(g.N) * g.OH * g.OW / (double(t.n_sblocks) * S);
+        const double eff = double(g.N) * rows * cols / (double(t.n_sblocks) * S);
         if (!found || eff > best->eff + 0.01) {  // larger tiles win ties: fewer tiles, more operand reuse
             best->MT = mt; best->WM = WM; best->WN = WN; best->t = t; best->lds_bytes = lds; best->eff = eff;
             found = true;

@@ -505,6 +505,93 @@ void dispatch_gemm_dma(zant_ctx *ctx, const float *A, const float *B, const floa
 #undef ZANT_GEMM_CASE
 }
 
+// ------------------------------------------------------------------------------------------------------------
+// Skinny Gemm (N <= 16, A row-major): the classifier head.  HBM-bound on A: every wave owns 4 rows, its lanes split
+// K, B sits in LDS, and the 4 x 16 partial sums per lane are reduced across the wave by recursive halving (63
+// exchanges instead of 64 x 6), which leaves result (row r, column n) in lane r*16 + n -- where bias, ReLU or the
+// row softmax (16-lane groups) are applied before one coalesced store.
+// ------------------------------------------------------------------------------------------------------------
+constexpr int SK_KC = 512;  // k per LDS stage of B
+
+__global__ void __launch_bounds__(256)
+gemm_f32_skinny_kernel(const float *__restrict__ A, const float *__restrict__ B, const float *__restrict__ C,
+                       float *__restrict__ Y, GemmArgs g, int ldb_k, int ldb_n, int softmax) {
+    __shared__ f32x4 bs[SK_KC * 4];  // [k][4 units of 4 columns]; unit u of row k at u ^ ((k >> 2) & 3): conflict-free reads
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int row0 = (blockIdx.x * 4 + wave) * 4;
+    float v[64];
+#pragma unroll
+    for (int i = 0; i < 64; ++i) v[i] = 0.0f;
+
+    for (int kc = 0; kc < g.K; kc += SK_KC) {
+        const int kend = min(SK_KC, g.K - kc);
+        // this lane's A values of the whole stage first: 32 independent loads in flight while B is staged
+        float a[SK_KC / 64][4];
+#pragma unroll
+        for (int it = 0; it < SK_KC / 64; ++it)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int k = it * 64 + lane;
+                a[it][r] = (k < kend && row0 + r < g.M) ? A[int64_t(row0 + r) * g.lda + kc + k] : 0.0f;
+            }
+        // B stage: all of a thread's loads are issued before the first LDS store (fixed trip count, unrolled)
+        float bv[SK_KC * 16 / 256];
+#pragma unroll
+        for (int i = 0; i < SK_KC * 16 / 256; ++i) {
+            const int idx = i * 256 + tid, k = idx >> 4, n = idx & 15;
+            bv[i] = (k < kend && n < g.N) ? B[int64_t(kc + k) * ldb_k + int64_t(n) * ldb_n] : 0.0f;
+        }
+        if (kc) __syncthreads();
+#pragma unroll
+        for (int i = 0; i < SK_KC * 16 / 256; ++i) {
+            const int idx = i * 256 + tid, k = idx >> 4, n = idx & 15;
+            reinterpret_cast<float *>(bs)[(k * 4 + ((n >> 2) ^ ((k >> 2) & 3))) * 4 + (n & 3)] = bv[i];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int it = 0; it < SK_KC / 64; ++it) {
+            const int kq = it * 64 + lane;
+            if (it * 64 < kend) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const f32x4 b = bs[kq * 4 + (u ^ ((kq >> 2) & 3))];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) v[r * 16 + u * 4 + c] += a[it][r] * b[c];
+                }
+            }
+        }
+    }
+    // recursive halving: after the step with distance s a lane keeps the half of its values selected by (lane & s)
+#pragma unroll
+    for (int s = 32; s >= 1; s >>= 1) {
+        const bool up = (lane & s) != 0;
+#pragma unroll
+        for (int i = 0; i < s; ++i) {
+            const float keep = up ? v[i + s] : v[i];
+            const float give = up ? v[i] : v[i + s];
+            v[i] = keep + __shfl_xor(give, s, 64);
+        }
+    }
+    const int r = lane >> 4, n = lane & 15, m = row0 + r;
+    const bool valid = m < g.M && n < g.N;
+    float res = v[0] * g.alpha;
+    if (g.c_mode && valid) res = res + C[int64_t(m) * g.c_ld_r + int64_t(n) * g.c_ld_c] * g.beta;
+    if (g.relu) res = res > 0.0f ? res : 0.0f;
+    if (softmax) {  // lean_softmax on the row: exp(x - max) / sum
+        float mx = n < g.N ? res : -INFINITY;
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+        const float e = n < g.N ? expf(res - mx) : 0.0f;
+        float sum = e;
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+        res = e / sum;
+    }
+    if (valid) Y[int64_t(m) * g.N + n] = res;
+}
+
 template <int TM, int WM, int WN>
 void launch_gemm(zant_ctx *ctx, const float *A, const float *B, const float *C, float *Y, const GemmArgs &g,
                  bool a_kc, bool b_kc) {
@@ -519,7 +606,8 @@ void launch_gemm(zant_ctx *ctx, const float *A, const float *B, const float *C, 
 
 // M, N, K of op(A)[M,K] * op(B)[K,N]; lda/ldb are the stored row lengths.
 int run_gemm(zant_ctx *ctx, const float *A, const float *B, const float *C, float *Y, int64_t M, int64_t N, int64_t K,
-             bool trans_a, bool trans_b, float alpha, float beta, int c_mode, int64_t c_ld_r, int64_t c_ld_c, int relu) {
+             bool trans_a, bool trans_b, float alpha, float beta, int c_mode, int64_t c_ld_r, int64_t c_ld_c, int relu,
+             int softmax = 0) {
     if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return ZANT_InvalidDimensions;
     GemmArgs g;
     g.M = int(M); g.N = int(N); g.K = int(K);
@@ -531,7 +619,14 @@ int run_gemm(zant_ctx *ctx, const float *A, const float *B, const float *C, floa
     g.a_vec = (reinterpret_cast<uintptr_t>(A) & 15) == 0 && (g.lda & 3) == 0;
     g.b_vec = (reinterpret_cast<uintptr_t>(B) & 15) == 0 && (g.ldb & 3) == 0;
     const bool a_kc = !trans_a, b_kc = trans_b;
+    if (softmax && (trans_a || N > 16)) return ZANT_InvalidInput;
     KernelTimer kt(ctx);
+    if (!trans_a && N <= 16) {
+        hipLaunchKernelGGL(gemm_f32_skinny_kernel, dim3(unsigned((M + 15) / 16)), dim3(256), 0, ctx->stream, A, B, C, Y, g,
+                           trans_b ? 1 : g.ldb, trans_b ? g.ldb : 1, softmax);
+        ZANT_LAUNCH_CHECK(ctx);
+        return ZANT_OK;
+    }
     const int am = a_kc ? (g.a_vec ? KC16 : KC4) : RC4;
     const int bmode = b_kc ? (g.b_vec ? KC16 : KC4) : RC4;
     if (N > 32) dispatch_gemm_dma<1, 4, 2>(ctx, A, B, C, Y, g, am, bmode);  // 128 x 64 tile, 8 waves, 5 stages
@@ -587,7 +682,7 @@ extern "C" int zant_hip_gemm_f32(zant_ctx *ctx, const float *a, const int64_t ad
                                  const int64_t bdim[4], const float *c, const int64_t *cdim, int c_rank, float alpha,
                                  float beta, int trans_a, int trans_b, float *y, const int64_t ydim[4], int fuse_act) {
     if (!ctx || !adim || !bdim || !ydim) return ZANT_NullPointer;
-    if (fuse_act != ZANT_ACT_NONE && fuse_act != ZANT_ACT_RELU) return ZANT_InvalidInput;
+    if (fuse_act != ZANT_ACT_NONE && fuse_act != ZANT_ACT_RELU && fuse_act != ZANT_ACT_SOFTMAX) return ZANT_InvalidInput;
     const int64_t M = trans_a ? adim[3] : adim[2], K = trans_a ? adim[2] : adim[3];
     const int64_t Kb = trans_b ? bdim[3] : bdim[2], N = trans_b ? bdim[2] : bdim[3];
     if (K != Kb) return ZANT_InputTensorDimensionMismatch;
@@ -605,5 +700,5 @@ extern "C" int zant_hip_gemm_f32(zant_ctx *ctx, const float *a, const int64_t ad
         ld_c = c_cols == 1 ? 0 : 1;
     }
     return run_gemm(ctx, a, b, c, y, M, N, K, trans_a != 0, trans_b != 0, alpha, beta, c_mode, ld_r, ld_c,
-                    fuse_act == ZANT_ACT_RELU);
+                    fuse_act == ZANT_ACT_RELU, fuse_act == ZANT_ACT_SOFTMAX);
 }

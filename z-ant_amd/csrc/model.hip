@@ -527,8 +527,22 @@ extern "C" int zant_model_finalize(zant_model *m) {
                 m->n[only].skip = true;
             }
         }
+        if (nd.op == OP_GEMM && nd.fuse_act == ZANT_ACT_NONE && !nd.trans_a) {
+            // Gemm -> (Reshape views) -> Softmax over the same [rows, cols]: the classifier head in one kernel
+            int out = nd.out, c1 = -1;
+            while (consumers(m, out, &c1) == 1 && m->n[c1].op == OP_RESHAPE) out = m->n[c1].out;
+            if (consumers(m, out, &only) == 1 && m->n[only].op == OP_SOFTMAX && !m->n[only].skip) {
+                const MTensor &si = m->t[m->n[only].in0];
+                const MTensor &go = m->t[nd.out];
+                if (si.dim[0] == go.dim[2] && si.dim[1] == go.dim[3] && go.dim[3] <= 16) {
+                    nd.fuse_act = ZANT_ACT_SOFTMAX;
+                    m->t[m->n[only].out].alias_of = out;
+                    m->n[only].skip = true;
+                }
+            }
+        }
         if (nd.op == OP_CONV) {
-            // Conv (+ReLU) -> MaxPool 2x2/2 on a few-channel first layer: one kernel, pooled output only
+            // Conv (+ReLU) -> MaxPool 2x2/2: one kernel, pooled output only (where the convolution kernels take the shape)
             int out = nd.out, c1 = -1;
             while (consumers(m, out, &c1) == 1 && m->n[c1].skip && (m->n[c1].op == OP_ADD_CONST || m->n[c1].op == OP_RELU))
                 out = m->n[c1].out;
@@ -636,7 +650,8 @@ extern "C" int zant_model_finalize(zant_model *m) {
 extern "C" int zant_model_output_dims(zant_model *m, int64_t *dims, int *rank, int *dtype) {
     if (!m || !dims || !rank) return ZANT_NullPointer;
     if (m->n.empty()) return ZANT_InvalidInput;
-    const MTensor &t = m->t[m->n.back().out];
+    // before finalize the last node added; afterwards the recorded output (fusions may re-home a node's tensor)
+    const MTensor &t = m->t[m->finalized ? m->output : m->n.back().out];
     *rank = t.rank;
     for (int i = 0; i < t.rank; ++i) dims[i] = t.dim[i];
     if (dtype) *dtype = t.dtype;
@@ -694,7 +709,7 @@ const char *op_name(const MNode &nd) {
     case OP_LEAKY: return "LeakyRelu";
     case OP_MAXPOOL: return "MaxPool";
     case OP_RESHAPE: return "Reshape";
-    case OP_GEMM: return nd.fuse_act ? "Gemm+Relu" : "Gemm";
+    case OP_GEMM: return nd.fuse_act == ZANT_ACT_SOFTMAX ? "Gemm+Softmax" : nd.fuse_act ? "Gemm+Relu" : "Gemm";
     case OP_MATMUL: return "MatMul";
     case OP_ADD_CONST: return "Add(const)";
     case OP_ADD: return "Add";

@@ -14,7 +14,7 @@ import torch
 from .capi import Context, ZantError, dims, lib
 
 PAD = {"NOTSET": 0, "SAME_UPPER": 1, "SAME_LOWER": 2, "VALID": 3}
-ACT = {None: 0, "none": 0, "relu": 1, "leaky": 2, "relu6": 3}
+ACT = {None: 0, "none": 0, "relu": 1, "leaky": 2, "relu6": 3, "softmax": 4}
 
 _ctx = {}
 
