@@ -15,6 +15,7 @@
 
 #include "conv_tile.h"
 #include "quant_common.h"
+#include "quant_layout.h"
 
 namespace {
 
@@ -263,7 +264,7 @@ template <int MT, int WM, int WN, int TT>
 __global__ void __launch_bounds__(WM *WN * 64, 2)
 qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, const float *__restrict__ mult,
                   const int32_t *__restrict__ corr, const int8_t *__restrict__ padvec, uint8_t *__restrict__ y, ConvGeom g,
-                  TileGeom t, int CB, QConvArgs q, int *__restrict__ tile_counter) {
+                  TileGeom t, int CB, QConvArgs q, int *__restrict__ tile_counter, int y_blocked) {
     constexpr int NT = WM * WN * 64;
     constexpr int K_BLK = WN * 32;
     extern __shared__ __attribute__((aligned(16))) char qlds[];
@@ -374,6 +375,39 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
                 mv[v] = mult[k];
                 cv[v] = corr[k];
             }
+            if (y_blocked) {
+                // [N][KB][OH][OW][16] signed.  A lane holds 4 groups of 4 consecutive channels; lanes l and l+32 swap
+                // one dword per 16-channel block so that each stores 8 consecutive bytes: a half-wave then writes
+                // 32 positions x 16 bytes without gaps.
+                const int KB = (g.K + 15) >> 4;
+                const int cb0 = (kb * K_BLK + wn * 32) >> 4;
+#pragma unroll
+                for (int i = 0; i < MT; ++i) {
+                    const int p = (wm * MT + i) * 32 + l32;
+                    const int img = p / per_img, rem = p - img * per_img;
+                    const int r = rem / g.OW, c = rem - r * g.OW;
+                    uint32_t d[4];
+#pragma unroll
+                    for (int gq = 0; gq < 4; ++gq) {
+                        uint32_t w4 = 0;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            w4 |= uint32_t(requant(acc[i][gq * 4 + e] + cv[gq * 4 + e], mv[gq * 4 + e], q)) << (8 * e);
+                        d[gq] = w4 ^ 0x80808080u;
+                    }
+                    const bool ok = img < imgs_here && r < rows_here;
+#pragma unroll
+                    for (int b = 0; b < 2; ++b) {
+                        const uint32_t send = lh ? d[2 * b] : d[2 * b + 1];
+                        const uint32_t recv = uint32_t(__shfl_xor(int(send), 32, 64));
+                        const uint2 out = lh ? make_uint2(recv, d[2 * b + 1]) : make_uint2(d[2 * b], recv);
+                        if (ok && cb0 + b < KB) {
+                            uint8_t *yp = y + (((int64_t(n0 + img) * KB + cb0 + b) * g.OH + oh0 + r) * g.OW + c) * 16 + lh * 8;
+                            *reinterpret_cast<uint2 *>(yp) = out;
+                        }
+                    }
+                }
+            } else
 #pragma unroll
             for (int i = 0; i < MT; ++i) {
                 const int p = (wm * MT + i) * 32 + l32;
@@ -397,7 +431,7 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
 template <int MT, int WM, int WN, int TT>
 void launch_qmfma_tt(zant_ctx *ctx, const int8_t *xb, const int8_t *wp, const float *mult, const int32_t *corr,
                      const int8_t *padvec, uint8_t *y, const ConvGeom &g, const TilePlan &p, int CB, const QConvArgs &q,
-                     int *counter, int grid) {
+                     int *counter, int grid, int yb) {
     static bool attr_set = false;
     if (!attr_set) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&qconv_mfma_kernel<MT, WM, WN, TT>),
@@ -405,41 +439,47 @@ void launch_qmfma_tt(zant_ctx *ctx, const int8_t *xb, const int8_t *wp, const fl
         attr_set = true;
     }
     hipLaunchKernelGGL((qconv_mfma_kernel<MT, WM, WN, TT>), dim3(grid), dim3(WM * WN * 64), p.lds_bytes, ctx->stream, xb,
-                       wp, mult, corr, padvec, y, g, p.t, CB, q, counter);
+                       wp, mult, corr, padvec, y, g, p.t, CB, q, counter, yb);
 }
 
 template <int MT, int WM, int WN>
 void launch_qmfma(zant_ctx *ctx, const int8_t *xb, const int8_t *wp, const float *mult, const int32_t *corr,
                   const int8_t *padvec, uint8_t *y, const ConvGeom &g, const TilePlan &p, int CB, const QConvArgs &q,
-                  int *counter, int grid) {
+                  int *counter, int grid, int yb) {
     const int T = g.KH * g.KW;
-    if (T == 9) launch_qmfma_tt<MT, WM, WN, 9>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid);
-    else if (T == 1) launch_qmfma_tt<MT, WM, WN, 1>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid);
-    else launch_qmfma_tt<MT, WM, WN, 0>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid);
+    if (T == 9) launch_qmfma_tt<MT, WM, WN, 9>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb);
+    else if (T == 1) launch_qmfma_tt<MT, WM, WN, 1>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb);
+    else launch_qmfma_tt<MT, WM, WN, 0>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb);
 }
 
 template <int WM, int WN>
 bool dispatch_qmt(zant_ctx *ctx, const int8_t *xb, const int8_t *wp, const float *mult, const int32_t *corr,
                   const int8_t *padvec, uint8_t *y, const ConvGeom &g, const TilePlan &p, int CB, const QConvArgs &q,
-                  int *counter, int grid) {
+                  int *counter, int grid, int yb) {
     switch (p.MT) {
-    case 1: launch_qmfma<1, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid); return true;
-    case 2: launch_qmfma<2, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid); return true;
-    case 3: launch_qmfma<3, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid); return true;
-    case 4: launch_qmfma<4, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid); return true;
-    case 5: launch_qmfma<5, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid); return true;
-    case 6: launch_qmfma<6, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid); return true;
-    case 7: launch_qmfma<7, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid); return true;
+    case 1: launch_qmfma<1, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb); return true;
+    case 2: launch_qmfma<2, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb); return true;
+    case 3: launch_qmfma<3, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb); return true;
+    case 4: launch_qmfma<4, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb); return true;
+    case 5: launch_qmfma<5, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb); return true;
+    case 6: launch_qmfma<6, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb); return true;
+    case 7: launch_qmfma<7, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb); return true;
     default: return false;
     }
 }
 
 static size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
 
-// The matrix-core path; returns ZANT_OK when it ran, 1 when the shape is left to the direct kernel.
+unsigned to_blocked_grid(zant_ctx *ctx, int64_t N, int64_t CB, int64_t hw) {
+    const int64_t units = N * CB * ((hw + 3) / 4);
+    return unsigned(std::min<int64_t>(std::max<int64_t>(ceil_div64(units, 256), 1), int64_t(ctx->num_cus) * 16));
+}
+
+// The matrix-core path; returns ZANT_OK when it ran, 1 when the shape is left to the other kernels.
+// x_blocked / y_blocked: x, y are already / are to be written in the blocked signed layout.
 int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float *w_scale, const int32_t *bias, uint8_t *y,
-                   const ConvGeom &g, const QConvArgs &q) {
-    if (g.groups != 1 || g.C < 16 || int64_t(g.N) * g.OH * g.OW < 64) return 1;
+                   const ConvGeom &g, const QConvArgs &q, bool x_blocked, bool y_blocked) {
+    if (g.groups != 1 || g.C < 5 || int64_t(g.N) * g.OH * g.OW < 64) return 1;
     const int CB = (g.C + 15) / 16;
     if (int64_t(g.N) * CB * g.H * g.W >= (int64_t(1) << 27)) return 1;  // 16-byte units addressed with 32-bit offsets
     TilePlan plan;
@@ -451,7 +491,7 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
     plan.t.n_chunks = (g.C + QCC - 1) / QCC;
     const size_t wp_bytes = size_t(plan.t.n_chunks) * plan.t.n_kblocks * T * QCC * K_BLK;
     const size_t kpad = size_t(plan.t.n_kblocks) * K_BLK;
-    const size_t xb_bytes = size_t(g.N) * CB * g.H * g.W * 16;
+    const size_t xb_bytes = x_blocked ? 0 : size_t(g.N) * CB * g.H * g.W * 16;
     const size_t o_pad = 256, o_mult = 512, o_corr = o_mult + align256(kpad * 4), o_wp = o_corr + align256(kpad * 4),
                  o_xb = o_wp + align256(wp_bytes), total = o_xb + xb_bytes;
     void *ws = nullptr;
@@ -463,36 +503,297 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
     float *mult = reinterpret_cast<float *>(base + o_mult);
     int32_t *corr = reinterpret_cast<int32_t *>(base + o_corr);
     int8_t *wp = reinterpret_cast<int8_t *>(base + o_wp);
-    int8_t *xb = reinterpret_cast<int8_t *>(base + o_xb);
+    const int8_t *xb = x_blocked ? reinterpret_cast<const int8_t *>(x) : reinterpret_cast<const int8_t *>(base + o_xb);
     const int grid = int(std::min<int64_t>(plan.t.n_tiles, int64_t(ctx->num_cus) * 2));
     const unsigned pb = unsigned(std::min<int64_t>(std::max<int64_t>(ceil_div64(int64_t(wp_bytes), 256), ceil_div64(int64_t(kpad), 4)), 1024));
     hipLaunchKernelGGL(qpack_kernel, dim3(pb), dim3(256), 0, ctx->stream, w, w_scale, bias, wp, mult, corr, padvec, counter,
                        2 * grid, g.K, g.C, T, plan.t.n_chunks, plan.t.n_kblocks, K_BLK, q.x_scale, q.y_scale, q.x_zp,
                        q.n_wscale);
     ZANT_LAUNCH_CHECK(ctx);
-    const int64_t hw = int64_t(g.H) * g.W;
-    const int64_t units = int64_t(g.N) * CB * ((hw + 3) / 4);
-    const unsigned tb = unsigned(std::min<int64_t>(ceil_div64(units, 256), int64_t(ctx->num_cus) * 16));
-    const int vec_ok = (hw % 4 == 0) && (reinterpret_cast<uintptr_t>(x) % 4 == 0);
-    hipLaunchKernelGGL(to_blocked_s8_kernel, dim3(tb), dim3(256), 0, ctx->stream, x, reinterpret_cast<uint4 *>(xb), g.N, g.C,
-                       CB, hw, vec_ok);
-    ZANT_LAUNCH_CHECK(ctx);
+    if (!x_blocked) {
+        const int64_t hw = int64_t(g.H) * g.W;
+        const int vec_ok = (hw % 4 == 0) && (reinterpret_cast<uintptr_t>(x) % 4 == 0);
+        hipLaunchKernelGGL(to_blocked_s8_kernel, dim3(to_blocked_grid(ctx, g.N, CB, hw)), dim3(256), 0, ctx->stream, x,
+                           reinterpret_cast<uint4 *>(base + o_xb), g.N, g.C, CB, hw, vec_ok);
+        ZANT_LAUNCH_CHECK(ctx);
+    }
     KernelTimer kt(ctx);
-    const bool ok = WN == 2 ? dispatch_qmt<2, 2>(ctx, xb, wp, mult, corr, padvec, y, g, plan, CB, q, counter, grid)
-                            : dispatch_qmt<4, 1>(ctx, xb, wp, mult, corr, padvec, y, g, plan, CB, q, counter, grid);
+    const int yb = y_blocked ? 1 : 0;
+    const bool ok = WN == 2 ? dispatch_qmt<2, 2>(ctx, xb, wp, mult, corr, padvec, y, g, plan, CB, q, counter, grid, yb)
+                            : dispatch_qmt<4, 1>(ctx, xb, wp, mult, corr, padvec, y, g, plan, CB, q, counter, grid, yb);
     if (!ok) return 1;
+    ZANT_LAUNCH_CHECK(ctx);
+    return ZANT_OK;
+}
+
+// ------------------------------------------------------------------------------------------------------------------
+// First layers (1..4 input channels, 3x3): one thread per output position, 16 output channels at a time.  The C*9
+// taps of a position are gathered once into signed bytes (x - 128, padding = x_zp - 128) and every output channel is
+// 7 (or 3) v_dot4_i32_i8 against weights the whole wave shares (scalar loads).  The zero point is folded as in the
+// matrix-core path.  Optionally max-pools 2x2/2 the four positions of a window before the store.
+// Reads NCHW u8; writes NCHW u8 or the blocked signed layout (one 16-byte store per position and channel block).
+// ------------------------------------------------------------------------------------------------------------------
+template <int C>
+__global__ void __launch_bounds__(256)
+qconv_smallc_pack_kernel(const int8_t *__restrict__ w, const float *__restrict__ w_scale, const int32_t *__restrict__ bias,
+                         uint32_t *__restrict__ wpk, float *__restrict__ mult, int32_t *__restrict__ corr, int K, int kpad,
+                         float x_scale, float y_scale, int x_zp, int n_wscale) {
+    constexpr int NT = C * 9, ND = (NT + 3) / 4;
+    const int k = blockIdx.x * blockDim.x + threadIdx.x;
+    if (k >= kpad) return;
+    int sum = 0;
+    for (int d = 0; d < ND; ++d) {
+        uint32_t v = 0;
+        for (int e = 0; e < 4; ++e) {
+            const int t = d * 4 + e;
+            const int wv = (k < K && t < NT) ? int(w[int64_t(k) * NT + t]) : 0;
+            sum += wv;
+            v |= uint32_t(uint8_t(wv)) << (8 * e);
+        }
+        wpk[k * ND + d] = v;
+    }
+    corr[k] = k < K ? (bias ? bias[k] : 0) + (128 - x_zp) * sum : 0;
+    mult[k] = k < K ? (x_scale * w_scale[n_wscale == 1 ? 0 : k]) / y_scale : 0.0f;
+}
+
+template <int C>
+__global__ void __launch_bounds__(256)
+qconv_smallc_kernel(const uint8_t *__restrict__ x, const uint32_t *__restrict__ wpk, const float *__restrict__ mult,
+                    const int32_t *__restrict__ corr, uint8_t *__restrict__ y, ConvGeom g, QConvArgs q, int y_blocked,
+                    int pool) {
+    constexpr int NT = C * 9, ND = (NT + 3) / 4;
+    __shared__ uint8_t lut[256];  // the fused activation as a byte table (identity without one)
+    lut[threadIdx.x] = q.has_act ? qact_apply(uint8_t(threadIdx.x), q.act) : uint8_t(threadIdx.x);
+    __syncthreads();
+    const int OHo = pool ? g.OH / 2 : g.OH, OWo = pool ? g.OW / 2 : g.OW;
+    const int KB = (g.K + 15) >> 4;
+    const int n_win = pool ? 4 : 1;
+    const uint32_t pad_byte = uint32_t(q.x_zp ^ 0x80);
+    const int64_t total = int64_t(g.N) * OHo * OWo;
+    const int64_t step = int64_t(gridDim.x) * blockDim.x;
+    for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += step) {
+        const int owo = int(i % OWo);
+        const int oho = int((i / OWo) % OHo);
+        const int n = int(i / (int64_t(OWo) * OHo));
+        uint32_t xs[4][ND];
+#pragma unroll
+        for (int wd = 0; wd < 4; ++wd) {
+            if (wd < n_win) {
+                const int oh = pool ? 2 * oho + (wd >> 1) : oho, ow = pool ? 2 * owo + (wd & 1) : owo;
+#pragma unroll
+                for (int d = 0; d < ND; ++d) xs[wd][d] = 0;
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    const int c = t / 9, kh = (t % 9) / 3, kw = t % 3;
+                    const int ih = oh * g.sh - g.pt + kh, iw = ow * g.sw - g.pl + kw;
+                    uint32_t b = pad_byte;
+                    if (ih >= 0 && ih < g.H && iw >= 0 && iw < g.W)
+                        b = uint32_t(x[((int64_t(n) * C + c) * g.H + ih) * g.W + iw]) ^ 0x80u;
+                    xs[wd][t >> 2] |= b << (8 * (t & 3));
+                }
+            }
+        }
+        for (int kb = 0; kb < KB; ++kb) {
+            uint32_t out[4] = {0, 0, 0, 0};
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const int k = kb * 16 + j;  // the tables are padded to a multiple of 16 channels
+                const float m = mult[k];
+                const int cr = corr[k];
+                uint32_t wv[ND];
+#pragma unroll
+                for (int d = 0; d < ND; ++d) wv[d] = wpk[k * ND + d];
+                // requantisation is monotone in the accumulator (increasing for m >= 0), and so is the activation:
+                // the pooled byte is the byte of the largest (smallest for m < 0) accumulator of the window
+                const bool neg = m < 0.0f;
+                int best = INT32_MIN;
+#pragma unroll
+                for (int wd = 0; wd < 4; ++wd) {
+                    if (wd < n_win) {
+                        int acc = cr;
+#pragma unroll
+                        for (int d = 0; d < ND; ++d) acc = __builtin_amdgcn_sdot4(int(xs[wd][d]), int(wv[d]), acc, false);
+                        acc = neg ? -acc : acc;
+                        best = acc > best ? acc : best;
+                    }
+                }
+                best = neg ? -best : best;
+                const uint8_t r = lut[sat_u8_rne(float(best) * m, q.y_zp)];
+                out[j >> 2] |= uint32_t(r) << (8 * (j & 3));
+            }
+            if (y_blocked) {
+                uint4 *dst = reinterpret_cast<uint4 *>(y) + ((int64_t(n) * KB + kb) * OHo + oho) * OWo + owo;
+                *dst = make_uint4(out[0] ^ 0x80808080u, out[1] ^ 0x80808080u, out[2] ^ 0x80808080u, out[3] ^ 0x80808080u);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 16; ++j)
+                    if (kb * 16 + j < g.K)
+                        y[((int64_t(n) * g.K + kb * 16 + j) * OHo + oho) * OWo + owo] = uint8_t(out[j >> 2] >> (8 * (j & 3)));
+            }
+        }
+    }
+}
+
+bool smallc_eligible(const ConvGeom &g) {
+    return g.groups == 1 && g.C >= 1 && g.C <= 4 && g.KH == 3 && g.KW == 3 && g.dh == 1 && g.dw == 1;
+}
+
+template <int C>
+int launch_smallc(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float *w_scale, const int32_t *bias, uint8_t *y,
+                  const ConvGeom &g, const QConvArgs &q, bool y_blocked, bool pool) {
+    constexpr int ND = (C * 9 + 3) / 4;
+    const int kpad = ((g.K + 15) / 16) * 16;
+    const size_t o_mult = 0, o_corr = align256(size_t(kpad) * 4), o_w = 2 * o_corr, total = o_w + size_t(kpad) * ND * 4;
+    void *ws = nullptr;
+    const int rc = zant_workspace(ctx, total, &ws);
+    if (rc) return rc;
+    char *base = static_cast<char *>(ws);
+    float *mult = reinterpret_cast<float *>(base + o_mult);
+    int32_t *corr = reinterpret_cast<int32_t *>(base + o_corr);
+    uint32_t *wpk = reinterpret_cast<uint32_t *>(base + o_w);
+    hipLaunchKernelGGL(qconv_smallc_pack_kernel<C>, dim3((kpad + 255) / 256), dim3(256), 0, ctx->stream, w, w_scale, bias, wpk,
+                       mult, corr, g.K, kpad, q.x_scale, q.y_scale, q.x_zp, q.n_wscale);
+    ZANT_LAUNCH_CHECK(ctx);
+    const int64_t positions = int64_t(g.N) * (pool ? g.OH / 2 : g.OH) * (pool ? g.OW / 2 : g.OW);
+    const unsigned blocks = unsigned(std::min<int64_t>(std::max<int64_t>(ceil_div64(positions, 256), 1), int64_t(ctx->num_cus) * 32));
+    KernelTimer kt(ctx);
+    hipLaunchKernelGGL(qconv_smallc_kernel<C>, dim3(blocks), dim3(256), 0, ctx->stream, x, wpk, mult, corr, y, g, q,
+                       y_blocked ? 1 : 0, pool ? 1 : 0);
+    ZANT_LAUNCH_CHECK(ctx);
+    return ZANT_OK;
+}
+
+int run_qconv_smallc(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float *w_scale, const int32_t *bias, uint8_t *y,
+                     const ConvGeom &g, const QConvArgs &q, bool y_blocked, bool pool) {
+    switch (g.C) {
+    case 1: return launch_smallc<1>(ctx, x, w, w_scale, bias, y, g, q, y_blocked, pool);
+    case 2: return launch_smallc<2>(ctx, x, w, w_scale, bias, y, g, q, y_blocked, pool);
+    case 3: return launch_smallc<3>(ctx, x, w, w_scale, bias, y, g, q, y_blocked, pool);
+    default: return launch_smallc<4>(ctx, x, w, w_scale, bias, y, g, q, y_blocked, pool);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------------
+// Depthwise 3x3 on the blocked layout (HBM-bound): one thread per output unit (16 channels of one position): nine
+// 16-byte loads, one 16-byte store.  A workgroup works on one channel block, so its weights are wave-uniform: they are
+// pre-expanded to one dword per (tap, channel) with the weight in that channel's byte lane and zeros elsewhere, and
+// acc[ch] += v_dot4_i32_i8(x_dword, w_dword) picks the channel's byte without any unpacking.
+// ------------------------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+qdw_pack_kernel(const int8_t *__restrict__ w, const float *__restrict__ w_scale, const int32_t *__restrict__ bias,
+                uint32_t *__restrict__ wm, float *__restrict__ mult, int32_t *__restrict__ corr, int K, int kpad, float x_scale,
+                float y_scale, int x_zp, int n_wscale) {
+    const int k = blockIdx.x * blockDim.x + threadIdx.x;
+    if (k >= kpad) return;
+    int sum = 0;
+    const int cb = k >> 4, qd = (k >> 2) & 3, j = k & 3;
+    for (int t = 0; t < 9; ++t) {
+        const int wv = k < K ? int(w[int64_t(k) * 9 + t]) : 0;
+        sum += wv;
+        wm[((cb * 4 + qd) * 9 + t) * 4 + j] = uint32_t(uint8_t(wv)) << (8 * j);
+    }
+    corr[k] = k < K ? (bias ? bias[k] : 0) + (128 - x_zp) * sum : 0;
+    mult[k] = k < K ? (x_scale * w_scale[n_wscale == 1 ? 0 : k]) / y_scale : 0.0f;
+}
+
+__global__ void __launch_bounds__(256)
+qdw3x3_blocked_kernel(const uint4 *__restrict__ x, const uint32_t *__restrict__ wm, const float *__restrict__ mult,
+                      const int32_t *__restrict__ corr, uint4 *__restrict__ y, ConvGeom g, QConvArgs q, int CB,
+                      int blocks_per_cb) {
+    __shared__ uint8_t lut[256];
+    lut[threadIdx.x] = uint8_t((q.has_act ? qact_apply(uint8_t(threadIdx.x), q.act) : uint8_t(threadIdx.x)) ^ 0x80);
+    __syncthreads();
+    const int cb = blockIdx.x / blocks_per_cb, blk = blockIdx.x - cb * blocks_per_cb;
+    const int64_t per_cb = int64_t(g.N) * g.OH * g.OW;
+    const uint32_t pad4 = uint32_t(q.x_zp ^ 0x80) * 0x01010101u;
+    const uint32_t *wcb = wm + cb * 144;
+    for (int64_t i = int64_t(blk) * 256 + threadIdx.x; i < per_cb; i += int64_t(blocks_per_cb) * 256) {
+        const int ow = int(i % g.OW);
+        const int oh = int((i / g.OW) % g.OH);
+        const int64_t n = i / (int64_t(g.OW) * g.OH);
+        const uint4 *xp = x + (n * CB + cb) * int64_t(g.H) * g.W;
+        uint4 xv[9];
+#pragma unroll
+        for (int t = 0; t < 9; ++t) {
+            const int ih = oh * g.sh - g.pt + t / 3, iw = ow * g.sw - g.pl + t % 3;
+            xv[t] = (ih >= 0 && ih < g.H && iw >= 0 && iw < g.W) ? xp[ih * g.W + iw] : make_uint4(pad4, pad4, pad4, pad4);
+        }
+        uint32_t out[4];
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+            int acc[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j] = corr[cb * 16 + qd * 4 + j];
+#pragma unroll
+            for (int t = 0; t < 9; ++t) {
+                const uint32_t xd = qd == 0 ? xv[t].x : qd == 1 ? xv[t].y : qd == 2 ? xv[t].z : xv[t].w;
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[j] = __builtin_amdgcn_sdot4(int(xd), int(wcb[(qd * 9 + t) * 4 + j]), acc[j], false);
+            }
+            uint32_t o = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                o |= uint32_t(lut[sat_u8_rne(float(acc[j]) * mult[cb * 16 + qd * 4 + j], q.y_zp)]) << (8 * j);
+            out[qd] = o;
+        }
+        y[((n * CB + cb) * g.OH + oh) * int64_t(g.OW) + ow] = make_uint4(out[0], out[1], out[2], out[3]);
+    }
+}
+
+bool dw_eligible(const ConvGeom &g) {
+    return g.groups == g.C && g.K == g.C && g.CG == 1 && g.KH == 3 && g.KW == 3 && g.dh == 1 && g.dw == 1;
+}
+
+// x, y blocked.
+int run_qdw_blocked(zant_ctx *ctx, const uint8_t *xb, const int8_t *w, const float *w_scale, const int32_t *bias, uint8_t *yb,
+                    const ConvGeom &g, const QConvArgs &q, size_t ws_offset) {
+    const int CB = (g.C + 15) / 16, kpad = CB * 16;
+    const size_t o_mult = ws_offset, o_corr = o_mult + align256(size_t(kpad) * 4), o_w = o_corr + align256(size_t(kpad) * 4),
+                 total = o_w + size_t(CB) * 144 * 4;
+    void *ws = nullptr;
+    const int rc = zant_workspace(ctx, total, &ws);
+    if (rc) return rc;
+    char *base = static_cast<char *>(ws);
+    float *mult = reinterpret_cast<float *>(base + o_mult);
+    int32_t *corr = reinterpret_cast<int32_t *>(base + o_corr);
+    uint32_t *wm = reinterpret_cast<uint32_t *>(base + o_w);
+    hipLaunchKernelGGL(qdw_pack_kernel, dim3((kpad + 255) / 256), dim3(256), 0, ctx->stream, w, w_scale, bias, wm, mult, corr,
+                       g.K, kpad, q.x_scale, q.y_scale, q.x_zp, q.n_wscale);
+    ZANT_LAUNCH_CHECK(ctx);
+    const int64_t per_cb = int64_t(g.N) * g.OH * g.OW;
+    const int64_t want = std::max<int64_t>(1, (int64_t(ctx->num_cus) * 16 + CB - 1) / CB);
+    const int blocks_per_cb = int(std::min<int64_t>(std::max<int64_t>(ceil_div64(per_cb, 256), 1), want));
+    KernelTimer kt(ctx);
+    hipLaunchKernelGGL(qdw3x3_blocked_kernel, dim3(unsigned(CB) * blocks_per_cb), dim3(256), 0, ctx->stream,
+                       reinterpret_cast<const uint4 *>(xb), wm, mult, corr, reinterpret_cast<uint4 *>(yb), g, q, CB,
+                       blocks_per_cb);
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
 }
 
 }  // namespace
 
-extern "C" int zant_hip_qlinearconv_u8i8(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], float x_scale,
-                                         uint8_t x_zp, const int8_t *w, const int64_t wdim[4], const float *w_scale,
-                                         int64_t n_wscale, const int8_t *w_zp, float y_scale, uint8_t y_zp,
-                                         const int32_t *bias, uint8_t *y, const int64_t ydim[4], const int64_t stride[2],
-                                         const int64_t pads[4], const int64_t dil[2], int64_t group, int act,
-                                         float act_alpha, float act_scale, uint8_t act_zp) {
+int zant_to_blocked(zant_ctx *ctx, const uint8_t *x, int64_t N, int64_t C, int64_t HW, uint8_t *xb) {
+    if (!ctx) return ZANT_NullPointer;
+    if (N <= 0 || C <= 0 || HW <= 0) return ZANT_OK;
+    if (!x || !xb) return ZANT_NullPointer;
+    const int64_t CB = (C + 15) / 16;
+    const int vec_ok = (HW % 4 == 0) && (reinterpret_cast<uintptr_t>(x) % 4 == 0);
+    KernelTimer kt(ctx);
+    hipLaunchKernelGGL(to_blocked_s8_kernel, dim3(to_blocked_grid(ctx, N, CB, HW)), dim3(256), 0, ctx->stream, x,
+                       reinterpret_cast<uint4 *>(xb), int(N), int(C), int(CB), HW, vec_ok);
+    ZANT_LAUNCH_CHECK(ctx);
+    return ZANT_OK;
+}
+
+// fuse_pool (internal callers only): ydim is the 2x2/2 max-pooled shape; only the first-layer kernel takes it.
+int zant_qlinearconv_layout_pool(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], float x_scale, uint8_t x_zp,
+                                 const int8_t *w, const int64_t wdim[4], const float *w_scale, int64_t n_wscale,
+                                 const int8_t *w_zp, float y_scale, uint8_t y_zp, const int32_t *bias, uint8_t *y,
+                                 const int64_t ydim[4], const int64_t stride[2], const int64_t pads[4], const int64_t dil[2],
+                                 int64_t group, int act, float act_alpha, float act_scale, uint8_t act_zp, int x_layout,
+                                 int y_layout, int fuse_pool, bool query_only) {
     if (!ctx || !xdim || !wdim || !ydim || !stride || !pads || !dil) return ZANT_NullPointer;
     for (int i = 0; i < 4; ++i)
         if (xdim[i] <= 0 || wdim[i] <= 0 || xdim[i] > INT32_MAX || wdim[i] > INT32_MAX) return ZANT_InvalidDimensions;
@@ -506,10 +807,10 @@ extern "C" int zant_hip_qlinearconv_u8i8(zant_ctx *ctx, const uint8_t *x, const 
     const int64_t PH = xdim[2] + pads[0] + pads[2], PW = xdim[3] + pads[1] + pads[3];
     if (PH < dkh || PW < dkw) return ZANT_InvalidDimensions;
     const int64_t OH = (PH - dkh) / stride[0] + 1, OW = (PW - dkw) / stride[1] + 1;
-    if (ydim[0] != xdim[0] || ydim[1] != K || ydim[2] != OH || ydim[3] != OW) return ZANT_InvalidDimensions;
+    const int64_t OHo = fuse_pool ? OH / 2 : OH, OWo = fuse_pool ? OW / 2 : OW;
+    if (ydim[0] != xdim[0] || ydim[1] != K || ydim[2] != OHo || ydim[3] != OWo) return ZANT_InvalidDimensions;
     // the i32 accumulator must not overflow: |x - zp| <= 255, |w - wzp| <= 255
     if (wdim[1] * wdim[2] * wdim[3] > (int64_t(1) << 31) / (255 * 255) - 1) return ZANT_InvalidDimensions;
-    if (!x || !w || !w_scale || !y) return ZANT_NullPointer;
 
     ConvGeom g;
     g.N = int(xdim[0]); g.C = int(C); g.H = int(xdim[2]); g.W = int(xdim[3]);
@@ -517,22 +818,78 @@ extern "C" int zant_hip_qlinearconv_u8i8(zant_ctx *ctx, const uint8_t *x, const 
     g.OH = int(OH); g.OW = int(OW);
     g.sh = int(stride[0]); g.sw = int(stride[1]); g.dh = int(dil[0]); g.dw = int(dil[1]);
     g.pt = int(pads[0]); g.pl = int(pads[1]); g.groups = int(group);
+    const bool xb = x_layout == ZANT_LAYOUT_BLOCKED16, yb = y_layout == ZANT_LAYOUT_BLOCKED16;
+    const bool smallc = w_zp == nullptr && !xb && smallc_eligible(g);
+    if (fuse_pool && (!smallc || OHo < 1 || OWo < 1)) return 1;  // only the first-layer kernel pools
+    if (query_only) return ZANT_OK;
+    if (!x || !w || !w_scale || !y) return ZANT_NullPointer;
+
     QConvArgs q;
     q.x_scale = x_scale; q.y_scale = y_scale; q.x_zp = x_zp; q.y_zp = y_zp; q.n_wscale = int(n_wscale);
     q.has_act = act != ZANT_ACT_NONE;
     q.act.act = act; q.act.alpha = act_alpha; q.act.in_scale = y_scale; q.act.in_zp = y_zp;
     q.act.out_scale = act_scale; q.act.out_zp = act_zp;
 
+    if (smallc) return run_qconv_smallc(ctx, x, w, w_scale, bias, y, g, q, yb, fuse_pool != 0);
+
+    const size_t x_blk = zant_blocked_bytes(xdim), y_blk = zant_blocked_bytes(ydim);
+    if (w_zp == nullptr && dw_eligible(g)) {
+        // the depthwise kernel works blocked -> blocked; NCHW operands pass through conversions in the workspace
+        const size_t o_x = 0, o_y = xb ? 0 : align256(x_blk), o_tab = o_y + (yb ? 0 : align256(y_blk));
+        const int CB = (g.C + 15) / 16;
+        void *ws = nullptr;
+        int rc = zant_workspace(ctx, o_tab + 2 * align256(size_t(CB) * 64) + size_t(CB) * 144 * 4, &ws);
+        if (rc) return rc;
+        char *base = static_cast<char *>(ws);
+        const uint8_t *xin = x;
+        if (!xb) {
+            rc = zant_to_blocked(ctx, x, g.N, g.C, int64_t(g.H) * g.W, reinterpret_cast<uint8_t *>(base + o_x));
+            if (rc) return rc;
+            xin = reinterpret_cast<uint8_t *>(base + o_x);
+        }
+        uint8_t *yout = yb ? y : reinterpret_cast<uint8_t *>(base + o_y);
+        rc = run_qdw_blocked(ctx, xin, w, w_scale, bias, yout, g, q, o_tab);
+        if (rc) return rc;
+        return yb ? ZANT_OK : zant_from_blocked(ctx, yout, g.N, g.K, int64_t(g.OH) * g.OW, y);
+    }
     if (w_zp == nullptr) {  // a non-zero weight zero point makes the correction position dependent: direct kernel
-        const int rc = run_qconv_mfma(ctx, x, w, w_scale, bias, y, g, q);
+        const int rc = run_qconv_mfma(ctx, x, w, w_scale, bias, y, g, q, xb, yb);
         if (rc <= 0) return rc;
+    }
+    // direct kernel: NCHW only; blocked operands pass through conversions in the workspace
+    const uint8_t *xin = x;
+    uint8_t *yout = y;
+    if (xb || yb) {
+        const size_t x_n = size_t(g.N) * g.C * g.H * g.W, y_n = size_t(g.N) * g.K * g.OH * g.OW;
+        void *ws = nullptr;
+        int rc = zant_workspace(ctx, align256(x_n) + y_n, &ws);
+        if (rc) return rc;
+        if (xb) {
+            rc = zant_from_blocked(ctx, x, g.N, g.C, int64_t(g.H) * g.W, static_cast<uint8_t *>(ws));
+            if (rc) return rc;
+            xin = static_cast<uint8_t *>(ws);
+        }
+        if (yb) yout = static_cast<uint8_t *>(ws) + align256(x_n);
     }
     const int64_t total = int64_t(g.N) * g.K * g.OH * g.OW;
     int64_t blocks = ceil_div64(total, 256);
     if (blocks > int64_t(ctx->num_cus) * 32) blocks = int64_t(ctx->num_cus) * 32;
-    KernelTimer kt(ctx);
-    hipLaunchKernelGGL(qconv_direct_kernel, dim3(unsigned(blocks)), dim3(256), 0, ctx->stream, x, w, w_scale, w_zp, bias, y,
-                       g, q);
-    ZANT_LAUNCH_CHECK(ctx);
-    return ZANT_OK;
+    {
+        KernelTimer kt(ctx);
+        hipLaunchKernelGGL(qconv_direct_kernel, dim3(unsigned(blocks)), dim3(256), 0, ctx->stream, xin, w, w_scale, w_zp, bias,
+                           yout, g, q);
+        ZANT_LAUNCH_CHECK(ctx);
+    }
+    return yb ? zant_to_blocked(ctx, yout, g.N, g.K, int64_t(g.OH) * g.OW, y) : ZANT_OK;
+}
+
+extern "C" int zant_hip_qlinearconv_u8i8(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], float x_scale,
+                                         uint8_t x_zp, const int8_t *w, const int64_t wdim[4], const float *w_scale,
+                                         int64_t n_wscale, const int8_t *w_zp, float y_scale, uint8_t y_zp,
+                                         const int32_t *bias, uint8_t *y, const int64_t ydim[4], const int64_t stride[2],
+                                         const int64_t pads[4], const int64_t dil[2], int64_t group, int act,
+                                         float act_alpha, float act_scale, uint8_t act_zp) {
+    return zant_qlinearconv_layout_pool(ctx, x, xdim, x_scale, x_zp, w, wdim, w_scale, n_wscale, w_zp, y_scale, y_zp, bias, y,
+                                        ydim, stride, pads, dil, group, act, act_alpha, act_scale, act_zp, ZANT_LAYOUT_NCHW,
+                                        ZANT_LAYOUT_NCHW, 0, false);
 }

@@ -4,6 +4,7 @@
 // are bit-identical with the CPU checker: IEEE divide, round-half-to-even, add zero point, saturate.
 // All are HBM-bound byte streams: 16 bytes per lane per access on the contiguous axis.
 #include "quant_common.h"
+#include "quant_layout.h"
 
 namespace {
 
@@ -44,10 +45,11 @@ __global__ void __launch_bounds__(kThreads) dequantize_kernel(const uint8_t *__r
 
 // u8 -> u8 through a 256-entry table held in LDS (the function of one byte is evaluated 256 times
 // with the exact f32 sequence, then applied 16 bytes per lane).
+// flip: the bytes of x and y hold value ^ flip (0x80 for the blocked signed layout), folded into the table.
 __global__ void __launch_bounds__(kThreads) qlinear_act_kernel(const uint8_t *__restrict__ x, uint8_t *__restrict__ y,
-                                                              int64_t n, QAct qa, int vec) {
+                                                              int64_t n, QAct qa, int vec, int flip) {
     __shared__ uint8_t lut[256];
-    lut[threadIdx.x] = qact_apply(uint8_t(threadIdx.x), qa);
+    lut[threadIdx.x] = uint8_t(qact_apply(uint8_t(threadIdx.x ^ flip), qa) ^ flip);
     __syncthreads();
     const int64_t step = int64_t(gridDim.x) * blockDim.x;
     const int64_t i0 = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -85,7 +87,8 @@ __device__ __forceinline__ uint8_t qadd_one(uint8_t a, uint8_t b, const QAddArgs
 }
 
 __global__ void __launch_bounds__(kThreads) qlinear_add_kernel(const uint8_t *__restrict__ a, const uint8_t *__restrict__ b,
-                                                              uint8_t *__restrict__ y, int64_t n, QAddArgs q, int vec) {
+                                                              uint8_t *__restrict__ y, int64_t n, QAddArgs q, int vec,
+                                                              uint32_t flip4) {
     const int64_t step = int64_t(gridDim.x) * blockDim.x;
     const int64_t i0 = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
     int64_t done = 0;
@@ -96,6 +99,8 @@ __global__ void __launch_bounds__(kThreads) qlinear_add_kernel(const uint8_t *__
         uint4 *y16 = reinterpret_cast<uint4 *>(y);
         for (int64_t i = i0; i < n16; i += step) {
             uint4 va = a16[i], vb = b16[i], vy;
+            va.x ^= flip4; va.y ^= flip4; va.z ^= flip4; va.w ^= flip4;
+            vb.x ^= flip4; vb.y ^= flip4; vb.z ^= flip4; vb.w ^= flip4;
             const uint32_t *wa = reinterpret_cast<const uint32_t *>(&va);
             const uint32_t *wb = reinterpret_cast<const uint32_t *>(&vb);
             uint32_t *wy = reinterpret_cast<uint32_t *>(&vy);
@@ -105,13 +110,114 @@ __global__ void __launch_bounds__(kThreads) qlinear_add_kernel(const uint8_t *__
 #pragma unroll
                 for (int k = 0; k < 4; ++k)
                     r |= uint32_t(qadd_one(uint8_t(wa[j] >> (8 * k)), uint8_t(wb[j] >> (8 * k)), q)) << (8 * k);
-                wy[j] = r;
+                wy[j] = r ^ flip4;
             }
             y16[i] = vy;
         }
         done = n16 << 4;
     }
-    for (int64_t i = done + i0; i < n; i += step) y[i] = qadd_one(a[i], b[i], q);
+    const uint8_t f = uint8_t(flip4);
+    for (int64_t i = done + i0; i < n; i += step) y[i] = uint8_t(qadd_one(a[i] ^ f, b[i] ^ f, q) ^ f);
+}
+
+// [N][CB][HW][16] signed -> NCHW u8.  One thread per (n, cb, 4 positions): four 16-byte loads, byte transpose,
+// sixteen 4-byte stores (one per channel row).
+__global__ void __launch_bounds__(kThreads) from_blocked_kernel(const uint4 *__restrict__ xb, uint8_t *__restrict__ y, int N,
+                                                               int C, int CB, int64_t HW, int vec_ok) {
+    const int64_t HW4 = (HW + 3) >> 2;
+    const int64_t total = int64_t(N) * CB * HW4;
+    const int64_t step = int64_t(gridDim.x) * blockDim.x;
+    for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += step) {
+        const int64_t hw = (i % HW4) << 2;
+        const int cb = int((i / HW4) % CB);
+        const int64_t n = i / (HW4 * CB);
+        const int valid = int(min(int64_t(4), HW - hw));
+        const uint4 *src = xb + (n * CB + cb) * HW + hw;
+        uint32_t u[4][4];  // [position][dword of 4 channels]
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const uint4 v = b < valid ? src[b] : make_uint4(0, 0, 0, 0);
+            u[b][0] = v.x ^ 0x80808080u; u[b][1] = v.y ^ 0x80808080u; u[b][2] = v.z ^ 0x80808080u; u[b][3] = v.w ^ 0x80808080u;
+        }
+        uint8_t *dst = y + (n * C + int64_t(cb) * 16) * HW + hw;
+#pragma unroll
+        for (int c = 0; c < 16; ++c) {
+            if (cb * 16 + c < C) {
+                const int q = c >> 2, sh = 8 * (c & 3);
+                const uint32_t row = ((u[0][q] >> sh) & 0xff) | (((u[1][q] >> sh) & 0xff) << 8) |
+                                     (((u[2][q] >> sh) & 0xff) << 16) | (((u[3][q] >> sh) & 0xff) << 24);
+                uint8_t *p = dst + int64_t(c) * HW;
+                if (vec_ok && valid == 4) {
+                    *reinterpret_cast<uint32_t *>(p) = row;
+                } else {
+                    for (int b = 0; b < valid; ++b) p[b] = uint8_t(row >> (8 * b));
+                }
+            }
+        }
+    }
+}
+
+// Signed byte-wise max of two dwords (the blocked layout stores value - 128, so signed order = value order).
+__device__ __forceinline__ uint32_t max_s8x4(uint32_t a, uint32_t b) {
+    uint32_t r = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int x = int8_t(a >> (8 * k)), y = int8_t(b >> (8 * k));
+        r |= uint32_t(uint8_t(x > y ? x : y)) << (8 * k);
+    }
+    return r;
+}
+__device__ __forceinline__ uint4 max_s8x16(uint4 a, uint4 b) {
+    return make_uint4(max_s8x4(a.x, b.x), max_s8x4(a.y, b.y), max_s8x4(a.z, b.z), max_s8x4(a.w, b.w));
+}
+
+// 2x2 / stride 2 max pool on [planes][H][W] 16-byte units: one thread per output unit.
+__global__ void __launch_bounds__(kThreads) maxpool2x2_blocked_kernel(const uint4 *__restrict__ x, uint4 *__restrict__ y,
+                                                                     int64_t planes, int H, int W, int OH, int OW) {
+    const int64_t total = planes * OH * OW;
+    const int64_t step = int64_t(gridDim.x) * blockDim.x;
+    for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += step) {
+        const int ow = int(i % OW);
+        const int oh = int((i / OW) % OH);
+        const int64_t p = i / (int64_t(OW) * OH);
+        const uint4 *r0 = x + (p * H + 2 * oh) * W + 2 * ow;
+        y[i] = max_s8x16(max_s8x16(r0[0], r0[1]), max_s8x16(r0[W], r0[W + 1]));
+    }
+}
+
+// Global average pool of a blocked tensor: one thread per (n, cb, 4-channel dword); exact i32 sums, then the fixed
+// f32 sequence.  Writes NCHW u8 ([N][C]) or the blocked form ([N][CB][16], value ^ 0x80).
+__global__ void __launch_bounds__(kThreads) qgap_blocked_kernel(const uint32_t *__restrict__ x, uint8_t *__restrict__ y,
+                                                               int64_t planes, int C, int CB, int hw, float x_scale,
+                                                               int x_zp, float y_scale, uint8_t y_zp, int y_blocked) {
+    const int64_t total = planes * 4;
+    const int64_t step = int64_t(gridDim.x) * blockDim.x;
+    for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += step) {
+        const int64_t p = i >> 2;
+        const int q = int(i & 3);
+        const uint32_t *src = x + p * int64_t(hw) * 4 + q;
+        int s[4] = {0, 0, 0, 0};
+        for (int j = 0; j < hw; ++j) {
+            const uint32_t v = src[int64_t(j) * 4] ^ 0x80808080u;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) s[k] += int((v >> (8 * k)) & 0xff) - x_zp;
+        }
+        uint32_t out = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const float mean = (float(s[k]) * x_scale) / float(hw);
+            out |= uint32_t(sat_u8_rne(mean / y_scale, y_zp)) << (8 * k);
+        }
+        if (y_blocked) {
+            reinterpret_cast<uint32_t *>(y)[i] = out ^ 0x80808080u;
+        } else {
+            const int64_t n = p / CB;
+            const int c0 = int(p % CB) * 16 + q * 4;
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                if (c0 + k < C) y[n * C + c0 + k] = uint8_t(out >> (8 * k));
+        }
+    }
 }
 
 // One wavefront per (n, c) plane: exact i32 sum, then the fixed f32 sequence.
@@ -182,8 +288,8 @@ extern "C" int zant_hip_dequantize_linear_u8_f32(zant_ctx *ctx, const uint8_t *x
     return ZANT_OK;
 }
 
-extern "C" int zant_hip_qlinear_act_u8(zant_ctx *ctx, const uint8_t *x, int64_t n, float x_scale, uint8_t x_zp, int act,
-                                       float alpha, float y_scale, uint8_t y_zp, uint8_t *y) {
+int zant_qlinear_act_flip(zant_ctx *ctx, const uint8_t *x, int64_t n, float x_scale, uint8_t x_zp, int act, float alpha,
+                          float y_scale, uint8_t y_zp, uint8_t *y, int flip) {
     if (!ctx) return ZANT_NullPointer;
     if (act < ZANT_ACT_NONE || act > ZANT_ACT_RELU6) return ZANT_InvalidInput;
     if (n <= 0) return ZANT_OK;
@@ -193,13 +299,18 @@ extern "C" int zant_hip_qlinear_act_u8(zant_ctx *ctx, const uint8_t *x, int64_t 
     const int vec = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
     KernelTimer kt(ctx);
     hipLaunchKernelGGL(qlinear_act_kernel, dim3(grid_for(n, kThreads * 16, ctx->num_cus)), dim3(kThreads), 0, ctx->stream,
-                       x, y, n, qa, vec);
+                       x, y, n, qa, vec, flip & 0xff);
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
 }
 
-extern "C" int zant_hip_qlinear_add_u8(zant_ctx *ctx, const uint8_t *a, float a_scale, uint8_t a_zp, const uint8_t *b,
-                                       float b_scale, uint8_t b_zp, float y_scale, uint8_t y_zp, uint8_t *y, int64_t n) {
+extern "C" int zant_hip_qlinear_act_u8(zant_ctx *ctx, const uint8_t *x, int64_t n, float x_scale, uint8_t x_zp, int act,
+                                       float alpha, float y_scale, uint8_t y_zp, uint8_t *y) {
+    return zant_qlinear_act_flip(ctx, x, n, x_scale, x_zp, act, alpha, y_scale, y_zp, y, 0);
+}
+
+int zant_qlinear_add_flip(zant_ctx *ctx, const uint8_t *a, float a_scale, uint8_t a_zp, const uint8_t *b, float b_scale,
+                          uint8_t b_zp, float y_scale, uint8_t y_zp, uint8_t *y, int64_t n, int flip) {
     if (!ctx) return ZANT_NullPointer;
     if (n <= 0) return ZANT_OK;
     if (!a || !b || !y) return ZANT_NullPointer;
@@ -208,7 +319,53 @@ extern "C" int zant_hip_qlinear_add_u8(zant_ctx *ctx, const uint8_t *a, float a_
     const int vec = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
     KernelTimer kt(ctx);
     hipLaunchKernelGGL(qlinear_add_kernel, dim3(grid_for(n, kThreads * 16, ctx->num_cus)), dim3(kThreads), 0, ctx->stream,
-                       a, b, y, n, q, vec);
+                       a, b, y, n, q, vec, uint32_t(flip & 0xff) * 0x01010101u);
+    ZANT_LAUNCH_CHECK(ctx);
+    return ZANT_OK;
+}
+
+extern "C" int zant_hip_qlinear_add_u8(zant_ctx *ctx, const uint8_t *a, float a_scale, uint8_t a_zp, const uint8_t *b,
+                                       float b_scale, uint8_t b_zp, float y_scale, uint8_t y_zp, uint8_t *y, int64_t n) {
+    return zant_qlinear_add_flip(ctx, a, a_scale, a_zp, b, b_scale, b_zp, y_scale, y_zp, y, n, 0);
+}
+
+int zant_from_blocked(zant_ctx *ctx, const uint8_t *xb, int64_t N, int64_t C, int64_t HW, uint8_t *y) {
+    if (!ctx) return ZANT_NullPointer;
+    if (N <= 0 || C <= 0 || HW <= 0) return ZANT_OK;
+    if (!xb || !y) return ZANT_NullPointer;
+    const int64_t CB = (C + 15) / 16, units = N * CB * ((HW + 3) / 4);
+    const int vec_ok = (HW % 4 == 0) && (reinterpret_cast<uintptr_t>(y) % 4 == 0);
+    KernelTimer kt(ctx);
+    hipLaunchKernelGGL(from_blocked_kernel, dim3(grid_for(units, kThreads, ctx->num_cus)), dim3(kThreads), 0, ctx->stream,
+                       reinterpret_cast<const uint4 *>(xb), y, int(N), int(C), int(CB), HW, vec_ok);
+    ZANT_LAUNCH_CHECK(ctx);
+    return ZANT_OK;
+}
+
+int zant_maxpool2x2_blocked(zant_ctx *ctx, const uint8_t *xb, const int64_t xdim[4], uint8_t *yb) {
+    if (!ctx || !xdim) return ZANT_NullPointer;
+    const int64_t planes = xdim[0] * ((xdim[1] + 15) / 16), OH = xdim[2] / 2, OW = xdim[3] / 2;
+    if (planes <= 0 || OH <= 0 || OW <= 0) return ZANT_OK;
+    if (!xb || !yb) return ZANT_NullPointer;
+    KernelTimer kt(ctx);
+    hipLaunchKernelGGL(maxpool2x2_blocked_kernel, dim3(grid_for(planes * OH * OW, kThreads, ctx->num_cus)), dim3(kThreads), 0,
+                       ctx->stream, reinterpret_cast<const uint4 *>(xb), reinterpret_cast<uint4 *>(yb), planes, int(xdim[2]),
+                       int(xdim[3]), int(OH), int(OW));
+    ZANT_LAUNCH_CHECK(ctx);
+    return ZANT_OK;
+}
+
+int zant_qgap_blocked(zant_ctx *ctx, const uint8_t *xb, const int64_t xdim[4], float x_scale, uint8_t x_zp, float y_scale,
+                      uint8_t y_zp, uint8_t *y, int y_layout) {
+    if (!ctx || !xdim) return ZANT_NullPointer;
+    const int64_t CB = (xdim[1] + 15) / 16, planes = xdim[0] * CB, hw = xdim[2] * xdim[3];
+    if (planes < 0 || hw <= 0 || hw > (1 << 23)) return ZANT_InvalidDimensions;
+    if (planes == 0) return ZANT_OK;
+    if (!xb || !y) return ZANT_NullPointer;
+    KernelTimer kt(ctx);
+    hipLaunchKernelGGL(qgap_blocked_kernel, dim3(grid_for(planes * 4, kThreads, ctx->num_cus)), dim3(kThreads), 0, ctx->stream,
+                       reinterpret_cast<const uint32_t *>(xb), y, planes, int(xdim[1]), int(CB), int(hw), x_scale, int(x_zp),
+                       y_scale, y_zp, y_layout == ZANT_LAYOUT_BLOCKED16);
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
 }

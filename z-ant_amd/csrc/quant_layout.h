@@ -1,0 +1,43 @@
+// Internal interface of the int8 kernels that work on the channel-blocked activation layout.
+//
+// ZANT_LAYOUT_BLOCKED16 stores a [N, C, H, W] u8 tensor as [N][ceil(C/16)][H][W][16] bytes, every byte holding
+// value ^ 0x80 (the two's-complement int8 "value - 128").  Sixteen channels of one position are one 16-byte unit:
+// one global->LDS copy, one int8 MFMA operand, one vector store.  Bytes of channels >= C are unspecified but
+// initialised (every consumer multiplies them by zero weights or drops them).  The public C ABI only ever sees
+// NCHW u8; the model executor keeps int8 activations in this layout between layers.
+#pragma once
+#include "common.h"
+
+enum zant_layout { ZANT_LAYOUT_NCHW = 0, ZANT_LAYOUT_BLOCKED16 = 1 };
+
+static inline size_t zant_blocked_bytes(const int64_t dim[4]) {
+    return size_t(dim[0]) * size_t((dim[1] + 15) / 16) * size_t(dim[2]) * size_t(dim[3]) * 16;
+}
+
+// zant_hip_qlinearconv_u8i8 with the layout of x and y chosen by the caller.
+// fuse_pool: also max-pool 2x2/2 (floor, no padding) in the same kernel; ydim is then the pooled shape.  Only the
+// first-layer kernel (1..4 input channels, 3x3, NCHW input) does that: other shapes return 1 and run nothing.
+// query_only: validate and report eligibility (ZANT_OK / 1 / error status) without touching any pointer.
+int zant_qlinearconv_layout_pool(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], float x_scale, uint8_t x_zp,
+                                 const int8_t *w, const int64_t wdim[4], const float *w_scale, int64_t n_wscale,
+                                 const int8_t *w_zp, float y_scale, uint8_t y_zp, const int32_t *bias, uint8_t *y,
+                                 const int64_t ydim[4], const int64_t stride[2], const int64_t pads[4], const int64_t dil[2],
+                                 int64_t group, int act, float act_alpha, float act_scale, uint8_t act_zp, int x_layout,
+                                 int y_layout, int fuse_pool, bool query_only);
+
+// Layout conversions (HW = H * W).
+int zant_to_blocked(zant_ctx *ctx, const uint8_t *x, int64_t N, int64_t C, int64_t HW, uint8_t *xb);
+int zant_from_blocked(zant_ctx *ctx, const uint8_t *xb, int64_t N, int64_t C, int64_t HW, uint8_t *y);
+
+// MaxPool 2x2 / stride 2 / no padding (floor) on a blocked tensor; ydim = [N, C, H/2, W/2].
+int zant_maxpool2x2_blocked(zant_ctx *ctx, const uint8_t *xb, const int64_t xdim[4], uint8_t *yb);
+
+// Elementwise operators on buffers whose bytes hold value ^ flip (flip = 0x80 for blocked tensors, 0 for NCHW).
+int zant_qlinear_act_flip(zant_ctx *ctx, const uint8_t *x, int64_t n, float x_scale, uint8_t x_zp, int act, float alpha,
+                          float y_scale, uint8_t y_zp, uint8_t *y, int flip);
+int zant_qlinear_add_flip(zant_ctx *ctx, const uint8_t *a, float a_scale, uint8_t a_zp, const uint8_t *b, float b_scale,
+                          uint8_t b_zp, float y_scale, uint8_t y_zp, uint8_t *y, int64_t n, int flip);
+
+// Global average pool of a blocked tensor; y is [N, C, 1, 1] in y_layout.
+int zant_qgap_blocked(zant_ctx *ctx, const uint8_t *xb, const int64_t xdim[4], float x_scale, uint8_t x_zp, float y_scale,
+                      uint8_t y_zp, uint8_t *y, int y_layout);
