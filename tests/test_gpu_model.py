@@ -199,7 +199,7 @@ def test_int8_network_fuses_activation_and_is_bit_exact(G):
     t7 = m.qlinear_add(t6, t3, 0.07, 100)                                             # residual
     t8 = m.qlinear_global_avgpool(t7, 0.05, 90)
     m.finalize()
-    assert m.num_launches == 6  # both activations ride in their convolutions
+    assert m.num_launches == 5  # both activations ride in their convolutions, the MaxPool in the first one
     y = m.predict_host(x)
     r1 = zo.qlinearconv(x, 0.02, 128, w1, s1, None, 0.05, 128, b1, [1, 1], [1, 1, 1, 1], [1, 1])
     r2 = zo.qlinear_act(r1, 0.05, 128, "leaky", 0.1, 0.04, 30)

@@ -17,6 +17,7 @@
 #include <vector>
 
 #include "common.h"
+#include "quant_layout.h"
 
 namespace {
 
@@ -31,6 +32,7 @@ struct MTensor {
     int64_t dim[8] = {0};
     float scale = 1.0f;   // quantisation parameters of a u8 tensor
     int zp = 0;
+    int layout = ZANT_LAYOUT_NCHW;  // how the storage root keeps a rank-4 u8 tensor (set by finalize)
     int alias_of = -1;    // shares storage with that tensor (views, fused activations)
     size_t offset = 0;    // in the arena, valid for storage roots after finalize
     int def = -1, last = -1;
@@ -39,6 +41,7 @@ struct MTensor {
         for (int i = 0; i < rank; ++i) n *= size_t(dim[i]);
         return n;
     }
+    size_t storage_bytes() const { return layout == ZANT_LAYOUT_BLOCKED16 ? zant_blocked_bytes(dim) : bytes(); }
 };
 
 struct Param {           // a host copy of a constant until finalize, then its place in the parameter block
@@ -147,6 +150,7 @@ int run_node(zant_model *m, const MNode &nd) {
     const MTensor &to = m->t[nd.out];
     const void *x = tensor_ptr(m, nd.in0);
     void *y = tensor_ptr(m, nd.out);
+    const int lin = m->t[root_of(m, nd.in0)].layout, lout = m->t[root_of(m, nd.out)].layout;
     switch (nd.op) {
     case OP_CONV:
         if (nd.fuse_pool)
@@ -167,6 +171,8 @@ int run_node(zant_model *m, const MNode &nd) {
         return zant_hip_leaky_relu_f32(ctx, static_cast<const float *>(x), nd.slope, static_cast<float *>(y),
                                        int64_t(ti.bytes() / 4));
     case OP_MAXPOOL:
+        if (ti.dtype == ZANT_U8 && lin == ZANT_LAYOUT_BLOCKED16)
+            return zant_maxpool2x2_blocked(ctx, static_cast<const uint8_t *>(x), ti.dim, static_cast<uint8_t *>(y));
         if (ti.dtype == ZANT_U8)
             return zant_hip_maxpool2d_u8(ctx, static_cast<const uint8_t *>(x), ti.dim, static_cast<uint8_t *>(y), to.dim,
                                          nd.kernel, nd.stride, nd.dil, nd.pads, 4, nd.pool_pad);
@@ -202,23 +208,28 @@ int run_node(zant_model *m, const MNode &nd) {
                                                  static_cast<const uint8_t *>(param_ptr(m, nd.b)), 1, 1,
                                                  static_cast<float *>(y));
     case OP_QCONV:
-        return zant_hip_qlinearconv_u8i8(ctx, static_cast<const uint8_t *>(x), ti.dim, ti.scale, uint8_t(ti.zp),
-                                         static_cast<const int8_t *>(param_ptr(m, nd.w)), nd.wdim,
-                                         static_cast<const float *>(param_ptr(m, nd.ws)), nd.n_wscale, nullptr,
-                                         nd.fuse_act ? nd.act_scale : to.scale, uint8_t(nd.fuse_act ? nd.act_zp : to.zp),
-                                         static_cast<const int32_t *>(param_ptr(m, nd.b)), static_cast<uint8_t *>(y), to.dim,
-                                         nd.stride, nd.pads, nd.dil, nd.group, nd.fuse_act, nd.act_alpha, to.scale,
-                                         uint8_t(to.zp));
+        return zant_qlinearconv_layout_pool(ctx, static_cast<const uint8_t *>(x), ti.dim, ti.scale, uint8_t(ti.zp),
+                                            static_cast<const int8_t *>(param_ptr(m, nd.w)), nd.wdim,
+                                            static_cast<const float *>(param_ptr(m, nd.ws)), nd.n_wscale, nullptr,
+                                            nd.fuse_act ? nd.act_scale : to.scale, uint8_t(nd.fuse_act ? nd.act_zp : to.zp),
+                                            static_cast<const int32_t *>(param_ptr(m, nd.b)), static_cast<uint8_t *>(y), to.dim,
+                                            nd.stride, nd.pads, nd.dil, nd.group, nd.fuse_act, nd.act_alpha, to.scale,
+                                            uint8_t(to.zp), lin, lout, nd.fuse_pool ? 1 : 0, false);
     case OP_QACT:
-        return zant_hip_qlinear_act_u8(ctx, static_cast<const uint8_t *>(x), int64_t(ti.bytes()), ti.scale, uint8_t(ti.zp),
-                                       nd.act, nd.act_alpha, to.scale, uint8_t(to.zp), static_cast<uint8_t *>(y));
+        return zant_qlinear_act_flip(ctx, static_cast<const uint8_t *>(x), int64_t(m->t[root_of(m, nd.in0)].storage_bytes()),
+                                     ti.scale, uint8_t(ti.zp), nd.act, nd.act_alpha, to.scale, uint8_t(to.zp),
+                                     static_cast<uint8_t *>(y), lin == ZANT_LAYOUT_BLOCKED16 ? 0x80 : 0);
     case OP_QADD: {
         const MTensor &tb = m->t[nd.in1];
-        return zant_hip_qlinear_add_u8(ctx, static_cast<const uint8_t *>(x), ti.scale, uint8_t(ti.zp),
-                                       static_cast<const uint8_t *>(tensor_ptr(m, nd.in1)), tb.scale, uint8_t(tb.zp), to.scale,
-                                       uint8_t(to.zp), static_cast<uint8_t *>(y), int64_t(ti.bytes()));
+        return zant_qlinear_add_flip(ctx, static_cast<const uint8_t *>(x), ti.scale, uint8_t(ti.zp),
+                                     static_cast<const uint8_t *>(tensor_ptr(m, nd.in1)), tb.scale, uint8_t(tb.zp), to.scale,
+                                     uint8_t(to.zp), static_cast<uint8_t *>(y),
+                                     int64_t(m->t[root_of(m, nd.in0)].storage_bytes()), lin == ZANT_LAYOUT_BLOCKED16 ? 0x80 : 0);
     }
     case OP_QGAP:
+        if (lin == ZANT_LAYOUT_BLOCKED16)
+            return zant_qgap_blocked(ctx, static_cast<const uint8_t *>(x), ti.dim, ti.scale, uint8_t(ti.zp), to.scale,
+                                     uint8_t(to.zp), static_cast<uint8_t *>(y), lout);
         return zant_hip_qlinear_global_avgpool_u8(ctx, static_cast<const uint8_t *>(x), ti.dim, ti.scale, uint8_t(ti.zp),
                                                   to.scale, uint8_t(to.zp), static_cast<uint8_t *>(y));
     default:
@@ -585,6 +596,93 @@ extern "C" int zant_model_finalize(zant_model *m) {
     }
     (void)producer;
 
+    // ---- first int8 layer: QLinearConv (+activation) -> MaxPool 2x2/2 in the few-channel kernel -------------------
+    for (int i = 0; i < nn; ++i) {
+        MNode &nd = m->n[i];
+        int only = -1;
+        if (nd.skip || nd.op != OP_QCONV || consumers(m, nd.out, &only) != 1) continue;
+        // (a fused activation's tensor is an alias of nd.out, so its consumers count as consumers of nd.out's storage;
+        //  look for the pool among the readers of either id)
+        int out = nd.out, c1 = -1;
+        while (consumers(m, out, &c1) == 1 && m->n[c1].skip && m->n[c1].op == OP_QACT) out = m->n[c1].out;
+        if (consumers(m, out, &only) != 1 || m->n[only].op != OP_MAXPOOL || m->n[only].skip) continue;
+        MNode &pn = m->n[only];
+        const bool pool22 = pn.kernel[0] == 2 && pn.kernel[1] == 2 && pn.stride[0] == 2 && pn.stride[1] == 2 &&
+                            pn.dil[0] == 1 && pn.dil[1] == 1 && pn.pads[0] == 0 && pn.pads[1] == 0 && pn.pads[2] == 0 &&
+                            pn.pads[3] == 0 && (pn.pool_pad == ZANT_PAD_NOTSET || pn.pool_pad == ZANT_PAD_VALID);
+        const MTensor &ti = m->t[nd.in0];
+        const MTensor &tp = m->t[pn.out];
+        if (!pool22 || root_of(m, nd.in0) != root_of(m, m->input)) continue;
+        if (zant_qlinearconv_layout_pool(ctx, nullptr, ti.dim, ti.scale, uint8_t(ti.zp), nullptr, nd.wdim, nullptr, nd.n_wscale,
+                                         nullptr, 1.0f, 0, nullptr, nullptr, tp.dim, nd.stride, nd.pads, nd.dil, nd.group,
+                                         nd.fuse_act, 0.0f, 1.0f, 0, ZANT_LAYOUT_NCHW, ZANT_LAYOUT_NCHW, 1, true) != ZANT_OK)
+            continue;
+        // the pool's tensor carries the same scale / zero point as the tensor it pooled
+        m->t[pn.out].scale = m->t[nd.out].scale;
+        m->t[pn.out].zp = m->t[nd.out].zp;
+        nd.fuse_pool = true;
+        const int conv_out = nd.out;
+        nd.out = pn.out;
+        pn.skip = true;
+        pn.out = conv_out;
+        pn.in0 = conv_out;
+    }
+
+    // ---- layouts: int8 activations stay channel-blocked between the operators that have blocked kernels ----------
+    {
+        const int ntl = int(m->t.size());
+        auto blocked_op = [&](const MNode &nd) {
+            return nd.op == OP_QCONV || nd.op == OP_QACT || nd.op == OP_QADD || nd.op == OP_QGAP ||
+                   (nd.op == OP_MAXPOOL && m->t[nd.in0].dtype == ZANT_U8);
+        };
+        for (const MNode &nd : m->n) {
+            if (nd.skip || !blocked_op(nd)) continue;
+            MTensor &ro = m->t[root_of(m, nd.out)];
+            if (ro.dtype == ZANT_U8 && ro.rank == 4) ro.layout = ZANT_LAYOUT_BLOCKED16;
+        }
+        auto demote = [&](int id, bool &changed) {
+            MTensor &r = m->t[root_of(m, id)];
+            if (r.layout != ZANT_LAYOUT_NCHW) { r.layout = ZANT_LAYOUT_NCHW; changed = true; }
+        };
+        bool changed = true;
+        while (changed) {
+            changed = false;
+            demote(m->input, changed);
+            demote(m->output, changed);
+            for (const MNode &nd : m->n) {
+                if (nd.op == OP_RESHAPE) { demote(nd.in0, changed); demote(nd.out, changed); continue; }  // views need NCHW
+                if (nd.skip) continue;
+                const int li = m->t[root_of(m, nd.in0)].layout, lo = m->t[root_of(m, nd.out)].layout;
+                if (!blocked_op(nd)) {
+                    demote(nd.in0, changed);
+                    if (nd.in1 >= 0) demote(nd.in1, changed);
+                    continue;
+                }
+                if (nd.op == OP_QCONV) {
+                    if (nd.fuse_pool) demote(nd.in0, changed);
+                } else if (nd.op == OP_QGAP) {
+                    if (li == ZANT_LAYOUT_NCHW) demote(nd.out, changed);
+                } else if (nd.op == OP_QADD) {
+                    const int l1 = m->t[root_of(m, nd.in1)].layout;
+                    if (li == ZANT_LAYOUT_NCHW || l1 == ZANT_LAYOUT_NCHW || lo == ZANT_LAYOUT_NCHW) {
+                        demote(nd.in0, changed); demote(nd.in1, changed); demote(nd.out, changed);
+                    }
+                } else if (nd.op == OP_MAXPOOL) {
+                    const bool pool22 = nd.kernel[0] == 2 && nd.kernel[1] == 2 && nd.stride[0] == 2 && nd.stride[1] == 2 &&
+                                        nd.dil[0] == 1 && nd.dil[1] == 1 && nd.pads[0] == 0 && nd.pads[1] == 0 &&
+                                        nd.pads[2] == 0 && nd.pads[3] == 0 &&
+                                        (nd.pool_pad == ZANT_PAD_NOTSET || nd.pool_pad == ZANT_PAD_VALID) &&
+                                        m->t[nd.out].dim[2] == m->t[nd.in0].dim[2] / 2 &&
+                                        m->t[nd.out].dim[3] == m->t[nd.in0].dim[3] / 2;
+                    if (!pool22 || li == ZANT_LAYOUT_NCHW || lo == ZANT_LAYOUT_NCHW) { demote(nd.in0, changed); demote(nd.out, changed); }
+                } else {  // OP_QACT: elementwise, same layout on both sides
+                    if (li == ZANT_LAYOUT_NCHW || lo == ZANT_LAYOUT_NCHW) { demote(nd.in0, changed); demote(nd.out, changed); }
+                }
+            }
+        }
+        (void)ntl;
+    }
+
     // ---- liveness and first-fit arena planning --------------------------------------------------
     const int nt = int(m->t.size());
     for (int i = 0; i < nt; ++i) { m->t[i].def = -1; m->t[i].last = -1; }
@@ -611,7 +709,7 @@ extern "C" int zant_model_finalize(zant_model *m) {
     for (int id : order) {
         MTensor &t = m->t[id];
         // the storage of a view chain must hold the largest member (they are all the same size here)
-        const size_t size = (t.bytes() + 255) & ~size_t(255);
+        const size_t size = (t.storage_bytes() + 255) & ~size_t(255);
         const int last = std::max(t.last, t.def);
         std::vector<std::pair<size_t, size_t>> busy;  // arena ranges alive during [def, last]
         for (const Placed &p : placed)
@@ -717,6 +815,7 @@ const char *op_name(const MNode &nd) {
     case OP_QUANT: return "QuantizeLinear";
     case OP_DEQUANT: return "DequantizeLinear";
     case OP_QCONV:
+        if (nd.fuse_pool) return nd.fuse_act ? "QLinearConv+Act+MaxPool" : "QLinearConv+MaxPool";
         if (nd.group > 1) return nd.fuse_act ? "QLinearConv(depthwise)+Act" : "QLinearConv(depthwise)";
         return nd.fuse_act ? "QLinearConv+Act" : "QLinearConv";
     case OP_QACT: return "QLinearAct";
@@ -801,6 +900,16 @@ extern "C" int zant_model_read_tensor(zant_model *m, int id, void *dst_host, siz
     if (!valid_tensor(m, id) || !dst_host) return ZANT_NullPointer;
     if (!m->finalized) return ZANT_NotFinalized;
     if (bytes > m->t[id].bytes()) return ZANT_InvalidDimensions;
+    const MTensor &t = m->t[id];
+    if (m->t[root_of(m, id)].layout == ZANT_LAYOUT_BLOCKED16) {  // hand out NCHW u8 like everywhere outside the executor
+        void *ws = nullptr;
+        int rc = zant_workspace(m->ctx, t.bytes(), &ws);
+        if (rc) return rc;
+        rc = zant_from_blocked(m->ctx, static_cast<const uint8_t *>(tensor_ptr(m, id)), t.dim[0], t.dim[1], t.dim[2] * t.dim[3],
+                               static_cast<uint8_t *>(ws));
+        if (rc) return rc;
+        return zant_hip_download(m->ctx, dst_host, ws, bytes);
+    }
     return zant_hip_download(m->ctx, dst_host, tensor_ptr(m, id), bytes);
 }
 

@@ -34,6 +34,11 @@ __device__ __forceinline__ uint8_t requant(int acc, float m, const QConvArgs &q)
     if (q.has_act) r = qact_apply(r, q.act);
     return r;
 }
+// The same with the fused activation taken from a 256-entry byte table (identity without one): the activation is a
+// function of one byte, and evaluating its f32 sequence (an IEEE divide among it) per output costs more than the MFMAs.
+__device__ __forceinline__ uint8_t requant_lut(int acc, float m, const QConvArgs &q, const uint8_t *lut) {
+    return lut[sat_u8_rne(float(acc) * m, q.y_zp)];
+}
 
 // One thread per output element; any stride / dilation / pads / group.
 __global__ void __launch_bounds__(256)
@@ -274,11 +279,13 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
     char *buf0 = qlds, *buf1 = qlds + buf_bytes;
     int2 *ptab = reinterpret_cast<int2 *>(qlds + 2 * buf_bytes);
     int *sched = reinterpret_cast<int *>(ptab + t.P1s);
+    uint8_t *lut = reinterpret_cast<uint8_t *>(sched + 2);  // [256] fused activation table
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave % WM, wn = wave / WM;
     const int l32 = lane & 31, lh = lane >> 5;
     const int64_t plane_in = int64_t(g.H) * g.W;
+    lut[tid & 255] = q.has_act ? qact_apply(uint8_t(tid & 255), q.act) : uint8_t(tid & 255);  // NT == 256
     const int per_img = t.TH * g.OW;
     const int patch_hw = t.PH * t.PW;
 
@@ -392,7 +399,7 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
                         uint32_t w4 = 0;
 #pragma unroll
                         for (int e = 0; e < 4; ++e)
-                            w4 |= uint32_t(requant(acc[i][gq * 4 + e] + cv[gq * 4 + e], mv[gq * 4 + e], q)) << (8 * e);
+                            w4 |= uint32_t(requant_lut(acc[i][gq * 4 + e] + cv[gq * 4 + e], mv[gq * 4 + e], q, lut)) << (8 * e);
                         d[gq] = w4 ^ 0x80808080u;
                     }
                     const bool ok = img < imgs_here && r < rows_here;
@@ -418,7 +425,7 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
                         const int dk = (v >> 2) * 8 + (v & 3);
-                        if (kbase + dk < g.K) yp[dk * plane] = requant(acc[i][v] + cv[v], mv[v], q);
+                        if (kbase + dk < g.K) yp[dk * plane] = requant_lut(acc[i][v] + cv[v], mv[v], q, lut);
                     }
                 }
             }
@@ -438,7 +445,7 @@ void launch_qmfma_tt(zant_ctx *ctx, const int8_t *xb, const int8_t *wp, const fl
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         attr_set = true;
     }
-    hipLaunchKernelGGL((qconv_mfma_kernel<MT, WM, WN, TT>), dim3(grid), dim3(WM * WN * 64), p.lds_bytes, ctx->stream, xb,
+    hipLaunchKernelGGL((qconv_mfma_kernel<MT, WM, WN, TT>), dim3(grid), dim3(WM * WN * 64), p.lds_bytes + 256, ctx->stream, xb,
                        wp, mult, corr, padvec, y, g, p.t, CB, q, counter, yb);
 }
 

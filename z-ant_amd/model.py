@@ -1,6 +1,7 @@
 """Python handle of a zant_model: the GPU form of a library the reference's code generator would emit
 (src/codeGen/predict.zig): nodes appended in ready order, one arena, one `run` per forward pass."""
 import ctypes as C
+import sys
 
 import numpy as np
 
@@ -171,6 +172,8 @@ class Model:
             self.handle = None
 
     def __del__(self):
+        if sys is None or sys.is_finalizing():  # the HIP runtime may already be gone at interpreter exit; the OS reclaims the rest
+            return
         try:
             self.close()
         except Exception:
