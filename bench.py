@@ -22,6 +22,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+# HBM bytes per launch of the pass's kernels at batch 4096, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# file scaled by a 256 MiB copy (summary and commands: profiles/cnn_f32_b4096_hbm_traffic.md).  Counters cannot be read
+# from inside the process, so `roofline.traffic` reports the figure of that run for the dominant kernel.
+MEASURED_HBM_BYTES = {"Conv+Relu+MaxPool@1": 115.69e6, "Conv+Relu+MaxPool@0": 107.64e6, "Gemm+Relu@2": 60.97e6,
+                      "Gemm+Softmax@3": 8.94e6}
 PEAK_F32_MFMA_TFLOPS = 157.3
 PEAK_I8_MFMA_TOPS = 5030.0
 PEAK_HBM_GBS = 8000.0
@@ -46,6 +51,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-operators", action="store_true", help="skip the standalone operator figures (configs 2a, 2b, 3)")
+    ap.add_argument("--no-networks", action="store_true", help="skip the int8 network figures (configs 4, 5)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB device copy (3x): the known-size reference for scaling the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run of this command")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build targets ONE MI355X; the forward pass shards by batch with no collectives "
@@ -101,6 +110,14 @@ def main():
     ms_per_step = max(ev_ms, wall_ms) / args.steps  # the host clock includes the final synchronisation
     value = BATCH / (ms_per_step * 1e-3)
 
+    if args.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     # ---- per-kernel durations of the pass: HIP events around the main kernel of every launching node ----
     flops = networks.readme_cnn_flops_per_inference()
     kit = max(5, min(args.steps, 20))
@@ -124,12 +141,14 @@ def main():
                                "frac": round(ach / PEAK_HBM_GBS, 4), "flop": ops, "bytes": nbytes}
     dominant = max(per_kernel, key=lambda k: per_kernel[k]["ms"])
     dk = per_kernel[dominant]
+    idx, nm = dominant.split(":", 1)
+    traffic = MEASURED_HBM_BYTES.get(f"{nm}@{idx}")
     if dk["bound"] == "mfma":
         roofline = {"kernel": dominant, "bound": "mfma", "achieved": dk["achieved_tflops"], "peak": PEAK_F32_MFMA_TFLOPS,
-                    "unit": "TFLOP/s", "frac": dk["frac"], "traffic": None, "avg_ms": dk["ms"]}
+                    "unit": "TFLOP/s", "frac": dk["frac"], "traffic": traffic, "avg_ms": dk["ms"]}
     else:
         roofline = {"kernel": dominant, "bound": "hbm", "achieved": dk["achieved_gbs"], "peak": PEAK_HBM_GBS,
-                    "unit": "GB/s", "frac": dk["frac"], "traffic": None, "avg_ms": dk["ms"]}
+                    "unit": "GB/s", "frac": dk["frac"], "traffic": traffic, "avg_ms": dk["ms"]}
 
     # ---- standalone operator figures (the "conv TOPS" half of the metric): configs 2a, 2b, 3 ----
     operators = None
@@ -166,17 +185,45 @@ def main():
         operators["qlinearconv_u8i8_N128_C128_28x28_K128_3x3"] = {"ms": round(ms, 4), "tops": round(op / ms / 1e9, 2),
                                                                   "frac_i8_mfma_peak": round(op / ms / 1e9 / PEAK_I8_MFMA_TOPS, 5)}
 
+    # ---- int8 networks (configs 4 and 5): whole-network throughput with the calibrated scales of the golden fixture ----
+    nets_out = None
+    if not args.no_networks:
+        nets_out = {}
+        gold = json.load(open(os.path.join(ROOT, "tests", "golden", "int8_networks.json")))
+        for name, arch, nb in (("tiny_yolo_int8", networks.tiny_yolo_arch(), 512),
+                               ("mobilenet_v2_035_int8", networks.mobilenet_v2_035_arch(), 1024)):
+            qparams = networks.int8_params(arch, seed=gold[name]["param_seed"])
+            qm = networks.build_int8_model(ctx, arch, qparams, gold[name]["quant"], nb)
+            xq = np.random.default_rng(2).integers(0, 256, (nb,) + tuple(arch["input"]), dtype=np.uint8)
+            # parity gate: the two golden images at the head of the batch must reproduce the oracle's bytes
+            xg = np.random.default_rng(gold[name]["input_seed"]).integers(0, 256, (2,) + tuple(arch["input"]), dtype=np.uint8)
+            xq[:2] = xg
+            yq = qm.predict_host(xq)
+            assert np.array_equal(yq[:2].ravel(), np.array(gold[name]["expected_u8"], np.uint8)), name
+            for _ in range(3):
+                qm.run()
+            ctx.sync()
+            ctx.timer_start()
+            for _ in range(kit):
+                qm.run()
+            ms = ctx.timer_stop() / kit
+            macs = gold[name]["macs_per_inference"]
+            nets_out[name] = {"batch": nb, "ms_per_step": round(ms, 4), "inferences_per_s": round(nb / ms * 1e3, 1),
+                              "tops": round(2.0 * macs * nb / ms / 1e9, 2), "launches_per_step": qm.num_launches,
+                              "arena_bytes": qm.arena_bytes}
+            qm.close()
+
     # ---- CPU baseline: the oracle on one host core, one image at a time, over a bounded sample ----
     cpu = None
     if not args.no_cpu_baseline:
-        sample = 2048
+        sample = 3 * BATCH  # about 15 s of CPU work
         t0 = time.perf_counter()
         for i in range(sample):
-            oracle_forward(x_host[i:i + 1])
+            oracle_forward(x_host[i % BATCH:i % BATCH + 1])
         dt = time.perf_counter() - t0
         cpu = {"value": round(sample / dt, 2), "unit": "inferences/s", "cores": 1, "kind": "port",
                "host_cores": os.cpu_count(),
-               "sample": f"first {sample} images of the batch, batch 1 per call (how the reference's predict() runs), "
+               "sample": f"{sample} images (the batch, three times over), batch 1 per call (how the reference's predict() runs), "
                          f"{dt:.1f} s of CPU time"}
 
     line = {
@@ -193,6 +240,7 @@ def main():
         "cpu_baseline": cpu,
         "kernels": per_kernel,
         "operators": operators,
+        "networks": nets_out,
     }
     print(json.dumps(line))
 
