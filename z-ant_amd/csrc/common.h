@@ -57,6 +57,22 @@ struct KernelTimer {
 // Grows the context's workspace to at least `bytes` (stream-ordered use only).
 int zant_workspace(zant_ctx *ctx, size_t bytes, void **out);
 
+// Weight-derived scratch of one operator instance (packed weights, requantisation tables, tile counters).  The model
+// executor owns one per node, so packing happens once; calls through the C ABI pass none and pack on every call
+// (the caller may have changed the weights).
+struct zant_pack_slot {
+    void *dev = nullptr;
+    size_t bytes = 0;
+    bool ready = false;   // the packed contents are valid
+    unsigned runs = 0;    // launches so far; its parity selects the tile counter of a launch
+};
+void zant_pack_slot_free(zant_ctx *ctx, zant_pack_slot *slot);
+// Hands out `static_bytes` of weight-derived scratch (the slot's own allocation, or the front of the context
+// workspace when slot == nullptr) and `dyn_bytes` of per-call scratch (always workspace).  *need_pack says whether
+// the static part must be (re)filled; *parity which of the two tile counters this launch draws from.
+int zant_pack_region(zant_ctx *ctx, zant_pack_slot *slot, size_t static_bytes, size_t dyn_bytes, void **stat, void **dyn,
+                     bool *need_pack, int *parity);
+
 static inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 static inline int64_t prod_dims(const int64_t *d, int rank) {
     int64_t p = 1;
@@ -84,4 +100,10 @@ int zant_conv_resolve(const int64_t xdim[4], const int64_t wdim[4], const int64_
 int zant_conv2d_f32_fused_pool(zant_ctx *ctx, const float *x, const int64_t xdim[4], const float *w, const int64_t wdim[4],
                                const float *bias, float *y, const int64_t ydim[4], const int64_t *stride, int n_stride,
                                const int64_t *pads, int n_pads, const int64_t *dil, int n_dil, int64_t group,
-                               const char *auto_pad, int relu, bool query_only);
+                               const char *auto_pad, int relu, bool query_only, zant_pack_slot *slot = nullptr);
+
+// zant_hip_conv2d_f32 with a pack slot (see above).
+int zant_conv2d_f32_slot(zant_ctx *ctx, const float *x, const int64_t xdim[4], const float *w, const int64_t wdim[4],
+                         const float *bias, float *y, const int64_t ydim[4], const int64_t *stride, int n_stride,
+                         const int64_t *pads, int n_pads, const int64_t *dil, int n_dil, int64_t group, const char *auto_pad,
+                         int fuse_act, zant_pack_slot *slot);

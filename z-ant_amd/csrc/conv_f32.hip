@@ -179,7 +179,7 @@ __device__ __forceinline__ void conv_step(float *__restrict__ dma, const float *
 template <int MT, int WM, int WN, int KV, int TT, bool POOL = false>
 __global__ void __launch_bounds__(WM *WN * 64, 2)
 conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, const float *__restrict__ bias,
-                     float *__restrict__ y, ConvGeom g, TileGeom t, int relu, int *__restrict__ tile_counter) {
+                     float *__restrict__ y, ConvGeom g, TileGeom t, int relu, int *__restrict__ tile_counters, int parity) {
     constexpr int NT = WM * WN * 64;
     constexpr int K_BLK = WN * 32;
     extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -229,6 +229,9 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
         lds_off[i] = (img < t.NB && r < t.TH) ? (img * t.PH + r * g.sh) * t.PW + c * g.sw : 0;
     }
     if (tid == 0) sched[0] = blockIdx.x + gridDim.x;  // the second tile is static, later ones come from the counter
+    // Two counters take turns: this launch draws from tile_counters[parity] and re-arms the other one for the next
+    // launch of the same operator, so that packed weights and counters can be kept across calls without a reset pass.
+    if (tid == 0 && blockIdx.x == 0) tile_counters[parity ^ 1] = 2 * int(gridDim.x);
     __syncthreads();
 
     int cur = blockIdx.x;
@@ -280,7 +283,7 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
             __syncthreads();                // ... everyone's have; all waves are done with the other buffer
             if (chunk == 0) {
                 nxt = sched[tile_par];  // written at least one barrier ago
-                if (tid == 0) sched[tile_par ^ 1] = atomicAdd(tile_counter, 1);
+                if (tid == 0) sched[tile_par ^ 1] = atomicAdd(tile_counters + parity, 1);
             }
             const bool same_tile = chunk + 1 < t.n_chunks;
             const bool do_issue = same_tile || nxt < t.n_tiles;
@@ -483,7 +486,7 @@ bool plan_mfma(const ConvGeom &g, MfmaPlan *best, bool pool = false) {
 
 template <int MT, int WM, int WN, int TT, bool POOL>
 void launch_mfma_tt(zant_ctx *ctx, const float *x, const float *wp, const float *bias, float *y, const ConvGeom &g,
-                    const MfmaPlan &p, int relu, int *counter, int grid) {
+                    const MfmaPlan &p, int relu, int *counter, int grid, int parity) {
     constexpr int KV = MT >= 8 ? 2 : 4;  // 64-bit operand reads keep 8 accumulator tiles inside 256 VGPRs
     // more than 64 KB of dynamic LDS has to be opted into once per kernel
     static bool attr_set = false;
@@ -493,37 +496,37 @@ void launch_mfma_tt(zant_ctx *ctx, const float *x, const float *wp, const float 
         attr_set = true;
     }
     hipLaunchKernelGGL((conv_f32_mfma_kernel<MT, WM, WN, KV, TT, POOL>), dim3(grid), dim3(WM * WN * 64), p.lds_bytes,
-                       ctx->stream, x, wp, bias, y, g, p.t, relu, counter);
+                       ctx->stream, x, wp, bias, y, g, p.t, relu, counter, parity);
 }
 
 template <int MT, int WM, int WN, bool POOL>
 void launch_mfma(zant_ctx *ctx, const float *x, const float *wp, const float *bias, float *y, const ConvGeom &g,
-                 const MfmaPlan &p, int relu, int *counter, int grid) {
+                 const MfmaPlan &p, int relu, int *counter, int grid, int parity) {
     const int T = g.KH * g.KW;
-    if (T == 9) launch_mfma_tt<MT, WM, WN, 9, POOL>(ctx, x, wp, bias, y, g, p, relu, counter, grid);
-    else if (T == 1 && !POOL) launch_mfma_tt<MT, WM, WN, 1, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid);
-    else launch_mfma_tt<MT, WM, WN, 0, POOL>(ctx, x, wp, bias, y, g, p, relu, counter, grid);
+    if (T == 9) launch_mfma_tt<MT, WM, WN, 9, POOL>(ctx, x, wp, bias, y, g, p, relu, counter, grid, parity);
+    else if (T == 1 && !POOL) launch_mfma_tt<MT, WM, WN, 1, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid, parity);
+    else launch_mfma_tt<MT, WM, WN, 0, POOL>(ctx, x, wp, bias, y, g, p, relu, counter, grid, parity);
 }
 
 template <int WM, int WN>
 bool dispatch_mt(zant_ctx *ctx, const float *x, const float *wp, const float *bias, float *y, const ConvGeom &g,
-                 const MfmaPlan &p, int relu, int *counter, int grid, bool pool) {
+                 const MfmaPlan &p, int relu, int *counter, int grid, bool pool, int parity) {
     if (pool) {
         switch (p.MT) {
-        case 4: launch_mfma<4, WM, WN, true>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
-        case 8: launch_mfma<8, WM, WN, true>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
+        case 4: launch_mfma<4, WM, WN, true>(ctx, x, wp, bias, y, g, p, relu, counter, grid, parity); return true;
+        case 8: launch_mfma<8, WM, WN, true>(ctx, x, wp, bias, y, g, p, relu, counter, grid, parity); return true;
         default: return false;
         }
     }
     switch (p.MT) {
-    case 1: launch_mfma<1, WM, WN, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
-    case 2: launch_mfma<2, WM, WN, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
-    case 3: launch_mfma<3, WM, WN, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
-    case 4: launch_mfma<4, WM, WN, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
-    case 5: launch_mfma<5, WM, WN, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
-    case 6: launch_mfma<6, WM, WN, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
-    case 7: launch_mfma<7, WM, WN, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
-    case 8: launch_mfma<8, WM, WN, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid); return true;
+    case 1: launch_mfma<1, WM, WN, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid, parity); return true;
+    case 2: launch_mfma<2, WM, WN, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid, parity); return true;
+    case 3: launch_mfma<3, WM, WN, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid, parity); return true;
+    case 4: launch_mfma<4, WM, WN, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid, parity); return true;
+    case 5: launch_mfma<5, WM, WN, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid, parity); return true;
+    case 6: launch_mfma<6, WM, WN, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid, parity); return true;
+    case 7: launch_mfma<7, WM, WN, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid, parity); return true;
+    case 8: launch_mfma<8, WM, WN, false>(ctx, x, wp, bias, y, g, p, relu, counter, grid, parity); return true;
     default: return false;
     }
 }
@@ -538,23 +541,27 @@ bool mfma_eligible(const ConvGeom &g, bool pool, MfmaPlan *plan) {
 
 // Packs the weights, resets the tile counter and launches the persistent implicit-GEMM kernel.
 int run_conv_mfma(zant_ctx *ctx, const float *x, const float *w, const float *bias, float *y, const ConvGeom &g,
-                  const MfmaPlan &plan, int relu, bool pool) {
+                  const MfmaPlan &plan, int relu, bool pool, zant_pack_slot *slot) {
     const int T = g.KH * g.KW, K_BLK = plan.WN * 32;
     const size_t wp_floats = size_t(plan.t.n_chunks) * plan.t.n_kblocks * T * CC * K_BLK;
-    void *ws = nullptr;
-    int rc = zant_workspace(ctx, 256 + wp_floats * sizeof(float), &ws);  // [tile counter | packed weights]
+    void *ws = nullptr, *dyn = nullptr;
+    bool need_pack = true;
+    int parity = 0;
+    int rc = zant_pack_region(ctx, slot, 256 + wp_floats * sizeof(float), 0, &ws, &dyn, &need_pack, &parity);  // [tile counters | packed weights]
     if (rc) return rc;
     int *counter = static_cast<int *>(ws);
     float *wp = reinterpret_cast<float *>(static_cast<char *>(ws) + 256);
     // persistent workgroups: two per CU; the first two tiles of each are static, the rest dynamic
     const int grid = int(std::min<int64_t>(plan.t.n_tiles, int64_t(ctx->num_cus) * 2));
     const unsigned pb = unsigned(std::min<int64_t>(ceil_div64(int64_t(wp_floats), 256), 1024));
-    hipLaunchKernelGGL(pack_weights_f32_kernel, dim3(pb), dim3(256), 0, ctx->stream, w, wp, g.K, g.C, T,
-                       plan.t.n_chunks, plan.t.n_kblocks, K_BLK, counter, 2 * grid);
-    ZANT_LAUNCH_CHECK(ctx);
+    if (need_pack) {
+        hipLaunchKernelGGL(pack_weights_f32_kernel, dim3(pb), dim3(256), 0, ctx->stream, w, wp, g.K, g.C, T,
+                           plan.t.n_chunks, plan.t.n_kblocks, K_BLK, counter, 2 * grid);
+        ZANT_LAUNCH_CHECK(ctx);
+    }
     KernelTimer kt(ctx);
-    const bool ok = plan.WN == 2 ? dispatch_mt<2, 2>(ctx, x, wp, bias, y, g, plan, relu, counter, grid, pool)
-                                 : dispatch_mt<4, 1>(ctx, x, wp, bias, y, g, plan, relu, counter, grid, pool);
+    const bool ok = plan.WN == 2 ? dispatch_mt<2, 2>(ctx, x, wp, bias, y, g, plan, relu, counter, grid, pool, parity)
+                                 : dispatch_mt<4, 1>(ctx, x, wp, bias, y, g, plan, relu, counter, grid, pool, parity);
     if (!ok) return 1;
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
@@ -636,6 +643,14 @@ extern "C" int zant_hip_conv2d_f32(zant_ctx *ctx, const float *x, const int64_t 
                                    const int64_t wdim[4], const float *bias, float *y, const int64_t ydim[4],
                                    const int64_t *stride, int n_stride, const int64_t *pads, int n_pads,
                                    const int64_t *dil, int n_dil, int64_t group, const char *auto_pad, int fuse_act) {
+    return zant_conv2d_f32_slot(ctx, x, xdim, w, wdim, bias, y, ydim, stride, n_stride, pads, n_pads, dil, n_dil, group, auto_pad,
+                                fuse_act, nullptr);
+}
+
+int zant_conv2d_f32_slot(zant_ctx *ctx, const float *x, const int64_t xdim[4], const float *w, const int64_t wdim[4],
+                         const float *bias, float *y, const int64_t ydim[4], const int64_t *stride, int n_stride,
+                         const int64_t *pads, int n_pads, const int64_t *dil, int n_dil, int64_t group, const char *auto_pad,
+                         int fuse_act, zant_pack_slot *slot) {
     if (!ctx || !xdim || !wdim || !ydim) return ZANT_NullPointer;
     zant_log("OnnxConvLean1");
     int64_t s[2], d[2], p[4];
@@ -664,7 +679,7 @@ extern "C" int zant_hip_conv2d_f32(zant_ctx *ctx, const float *x, const int64_t 
 
     MfmaPlan plan;
     if (mfma_eligible(g, false, &plan)) {
-        rc = run_conv_mfma(ctx, x, w, bias, y, g, plan, relu, false);
+        rc = run_conv_mfma(ctx, x, w, bias, y, g, plan, relu, false, slot);
         if (rc <= 0) {
             if (rc == ZANT_OK) zant_log("OnnxConvLean4");
             return rc;
@@ -698,7 +713,7 @@ extern "C" int zant_hip_conv2d_f32(zant_ctx *ctx, const float *x, const int64_t 
 int zant_conv2d_f32_fused_pool(zant_ctx *ctx, const float *x, const int64_t xdim[4], const float *w, const int64_t wdim[4],
                                const float *bias, float *y, const int64_t ydim[4], const int64_t *stride, int n_stride,
                                const int64_t *pads, int n_pads, const int64_t *dil, int n_dil, int64_t group,
-                               const char *auto_pad, int relu, bool query_only) {
+                               const char *auto_pad, int relu, bool query_only, zant_pack_slot *slot) {
     int64_t s[2], d[2], p[4];
     if (zant_conv_resolve(xdim, wdim, stride, n_stride, pads, n_pads, dil, n_dil, group, auto_pad, s, d, p)) return 1;
     if (s[0] != 1 || s[1] != 1 || d[0] != 1 || d[1] != 1 || xdim[1] != wdim[1]) return 1;
@@ -718,7 +733,7 @@ int zant_conv2d_f32_fused_pool(zant_ctx *ctx, const float *x, const int64_t xdim
         MfmaPlan plan;
         if (!mfma_eligible(g, true, &plan) || (plan.MT != 4 && plan.MT != 8)) return 1;
         if (query_only) return ZANT_OK;
-        return run_conv_mfma(ctx, x, w, bias, y, g, plan, relu, true);
+        return run_conv_mfma(ctx, x, w, bias, y, g, plan, relu, true, slot);
     }
     if (query_only) return ZANT_OK;
     const int POH = int(OH / 2), POW = int(OW / 2);

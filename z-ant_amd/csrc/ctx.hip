@@ -38,6 +38,44 @@ int zant_workspace(zant_ctx *ctx, size_t bytes, void **out) {
     return ZANT_OK;
 }
 
+void zant_pack_slot_free(zant_ctx *ctx, zant_pack_slot *slot) {
+    if (!slot || !slot->dev) return;
+    if (ctx && ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    (void)hipFree(slot->dev);
+    slot->dev = nullptr; slot->bytes = 0; slot->ready = false; slot->runs = 0;
+}
+
+int zant_pack_region(zant_ctx *ctx, zant_pack_slot *slot, size_t static_bytes, size_t dyn_bytes, void **stat, void **dyn,
+                     bool *need_pack, int *parity) {
+    const size_t sa = (static_bytes + 255) & ~size_t(255);
+    if (!slot) {
+        void *ws = nullptr;
+        const int rc = zant_workspace(ctx, sa + dyn_bytes, &ws);
+        if (rc) return rc;
+        *stat = ws;
+        *dyn = static_cast<char *>(ws) + sa;
+        *need_pack = true;
+        *parity = 0;
+        return ZANT_OK;
+    }
+    if (!slot->dev || slot->bytes < sa) {
+        zant_pack_slot_free(ctx, slot);
+        ZANT_HIP_TRY(ctx, hipMalloc(&slot->dev, sa));
+        slot->bytes = sa;
+    }
+    *dyn = nullptr;
+    if (dyn_bytes) {
+        const int rc = zant_workspace(ctx, dyn_bytes, dyn);
+        if (rc) return rc;
+    }
+    *stat = slot->dev;
+    *need_pack = !slot->ready;
+    slot->ready = true;  // the caller packs in stream order before the first consumer
+    *parity = int(slot->runs & 1u);
+    ++slot->runs;
+    return ZANT_OK;
+}
+
 extern "C" int zant_hip_ctx_create(zant_ctx **out, int device, void *stream) {
     if (!out) return ZANT_NullPointer;
     *out = nullptr;

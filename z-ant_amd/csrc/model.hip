@@ -73,6 +73,7 @@ struct MNode {
     int act = ZANT_ACT_NONE;
     int b_rank = 0;
     int64_t bdim[8] = {0};
+    mutable zant_pack_slot slot;  // packed weights / tables of this node, filled by its first launch
 };
 
 }  // namespace
@@ -159,12 +160,12 @@ int run_node(zant_model *m, const MNode &nd) {
                                               static_cast<const float *>(param_ptr(m, nd.b)), static_cast<float *>(y), to.dim,
                                               nd.stride, nd.n_stride, nd.has_pads ? nd.pads : nullptr, nd.n_pads,
                                               nd.has_dil ? nd.dil : nullptr, nd.n_dil, nd.group,
-                                              nd.has_auto_pad ? nd.auto_pad.c_str() : nullptr, nd.fuse_act == ZANT_ACT_RELU, false);
-        return zant_hip_conv2d_f32(ctx, static_cast<const float *>(x), ti.dim, static_cast<const float *>(param_ptr(m, nd.w)),
-                                   nd.wdim, static_cast<const float *>(param_ptr(m, nd.b)), static_cast<float *>(y), to.dim,
-                                   nd.stride, nd.n_stride, nd.has_pads ? nd.pads : nullptr, nd.n_pads,
-                                   nd.has_dil ? nd.dil : nullptr, nd.n_dil, nd.group,
-                                   nd.has_auto_pad ? nd.auto_pad.c_str() : nullptr, nd.fuse_act);
+                                              nd.has_auto_pad ? nd.auto_pad.c_str() : nullptr, nd.fuse_act == ZANT_ACT_RELU, false, &nd.slot);
+        return zant_conv2d_f32_slot(ctx, static_cast<const float *>(x), ti.dim, static_cast<const float *>(param_ptr(m, nd.w)),
+                                    nd.wdim, static_cast<const float *>(param_ptr(m, nd.b)), static_cast<float *>(y), to.dim,
+                                    nd.stride, nd.n_stride, nd.has_pads ? nd.pads : nullptr, nd.n_pads,
+                                    nd.has_dil ? nd.dil : nullptr, nd.n_dil, nd.group,
+                                    nd.has_auto_pad ? nd.auto_pad.c_str() : nullptr, nd.fuse_act, &nd.slot);
     case OP_RELU:
         return zant_hip_relu_f32(ctx, static_cast<const float *>(x), static_cast<float *>(y), int64_t(ti.bytes() / 4));
     case OP_LEAKY:
@@ -214,7 +215,7 @@ int run_node(zant_model *m, const MNode &nd) {
                                             nd.fuse_act ? nd.act_scale : to.scale, uint8_t(nd.fuse_act ? nd.act_zp : to.zp),
                                             static_cast<const int32_t *>(param_ptr(m, nd.b)), static_cast<uint8_t *>(y), to.dim,
                                             nd.stride, nd.pads, nd.dil, nd.group, nd.fuse_act, nd.act_alpha, to.scale,
-                                            uint8_t(to.zp), lin, lout, nd.fuse_pool ? 1 : 0, false);
+                                            uint8_t(to.zp), lin, lout, nd.fuse_pool ? 1 : 0, false, &nd.slot);
     case OP_QACT:
         return zant_qlinear_act_flip(ctx, static_cast<const uint8_t *>(x), int64_t(m->t[root_of(m, nd.in0)].storage_bytes()),
                                      ti.scale, uint8_t(ti.zp), nd.act, nd.act_alpha, to.scale, uint8_t(to.zp),
@@ -255,6 +256,7 @@ extern "C" void zant_model_destroy(zant_model *m) {
         (void)hipStreamSynchronize(m->ctx->stream);
         (void)hipFree(m->params_dev);
     }
+    for (MNode &nd : m->n) zant_pack_slot_free(m->ctx, &nd.slot);
     delete m;
 }
 
@@ -615,7 +617,7 @@ extern "C" int zant_model_finalize(zant_model *m) {
         if (!pool22 || root_of(m, nd.in0) != root_of(m, m->input)) continue;
         if (zant_qlinearconv_layout_pool(ctx, nullptr, ti.dim, ti.scale, uint8_t(ti.zp), nullptr, nd.wdim, nullptr, nd.n_wscale,
                                          nullptr, 1.0f, 0, nullptr, nullptr, tp.dim, nd.stride, nd.pads, nd.dil, nd.group,
-                                         nd.fuse_act, 0.0f, 1.0f, 0, ZANT_LAYOUT_NCHW, ZANT_LAYOUT_NCHW, 1, true) != ZANT_OK)
+                                         nd.fuse_act, 0.0f, 1.0f, 0, ZANT_LAYOUT_NCHW, ZANT_LAYOUT_NCHW, 1, true, nullptr) != ZANT_OK)
             continue;
         // the pool's tensor carries the same scale / zero point as the tensor it pooled
         m->t[pn.out].scale = m->t[nd.out].scale;
@@ -741,6 +743,15 @@ extern "C" int zant_model_finalize(zant_model *m) {
         }
     }
     m->result_host.resize(m->t[m->output].bytes());
+    // One pass over whatever the arena holds: every node packs its weights and sizes its scratch now, so that
+    // zant_model_run allocates nothing and launches no packing kernels.
+    ZANT_HIP_TRY(ctx, hipMemsetAsync(ctx->arena, 0, arena, ctx->stream));
+    for (const MNode &nd : m->n) {
+        if (nd.skip) continue;
+        rc = run_node(m, nd);
+        if (rc) return rc;
+    }
+    ZANT_HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
     m->finalized = true;
     return ZANT_OK;
 }

@@ -269,7 +269,7 @@ template <int MT, int WM, int WN, int TT>
 __global__ void __launch_bounds__(WM *WN * 64, 2)
 qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, const float *__restrict__ mult,
                   const int32_t *__restrict__ corr, const int8_t *__restrict__ padvec, uint8_t *__restrict__ y, ConvGeom g,
-                  TileGeom t, int CB, QConvArgs q, int *__restrict__ tile_counter, int y_blocked) {
+                  TileGeom t, int CB, QConvArgs q, int *__restrict__ tile_counters, int parity, int y_blocked) {
     constexpr int NT = WM * WN * 64;
     constexpr int K_BLK = WN * 32;
     extern __shared__ __attribute__((aligned(16))) char qlds[];
@@ -307,6 +307,8 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
         lds_off[i] = (img < t.NB && r < t.TH) ? (img * t.PH + r * g.sh) * t.PW + c * g.sw : 0;
     }
     if (tid == 0) sched[0] = blockIdx.x + gridDim.x;
+    // this launch draws tiles from tile_counters[parity] and re-arms the other counter for the operator's next launch
+    if (tid == 0 && blockIdx.x == 0) tile_counters[parity ^ 1] = 2 * int(gridDim.x);
     __syncthreads();
 
     int cur = blockIdx.x;
@@ -356,7 +358,7 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
             __syncthreads();
             if (chunk == 0) {
                 nxt = sched[tile_par];
-                if (tid == 0) sched[tile_par ^ 1] = atomicAdd(tile_counter, 1);
+                if (tid == 0) sched[tile_par ^ 1] = atomicAdd(tile_counters + parity, 1);
             }
             const bool same_tile = chunk + 1 < t.n_chunks;
             const bool do_issue = same_tile || nxt < t.n_tiles;
@@ -438,7 +440,7 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
 template <int MT, int WM, int WN, int TT>
 void launch_qmfma_tt(zant_ctx *ctx, const int8_t *xb, const int8_t *wp, const float *mult, const int32_t *corr,
                      const int8_t *padvec, uint8_t *y, const ConvGeom &g, const TilePlan &p, int CB, const QConvArgs &q,
-                     int *counter, int grid, int yb) {
+                     int *counter, int grid, int yb, int parity) {
     static bool attr_set = false;
     if (!attr_set) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&qconv_mfma_kernel<MT, WM, WN, TT>),
@@ -446,31 +448,31 @@ void launch_qmfma_tt(zant_ctx *ctx, const int8_t *xb, const int8_t *wp, const fl
         attr_set = true;
     }
     hipLaunchKernelGGL((qconv_mfma_kernel<MT, WM, WN, TT>), dim3(grid), dim3(WM * WN * 64), p.lds_bytes + 256, ctx->stream, xb,
-                       wp, mult, corr, padvec, y, g, p.t, CB, q, counter, yb);
+                       wp, mult, corr, padvec, y, g, p.t, CB, q, counter, parity, yb);
 }
 
 template <int MT, int WM, int WN>
 void launch_qmfma(zant_ctx *ctx, const int8_t *xb, const int8_t *wp, const float *mult, const int32_t *corr,
                   const int8_t *padvec, uint8_t *y, const ConvGeom &g, const TilePlan &p, int CB, const QConvArgs &q,
-                  int *counter, int grid, int yb) {
+                  int *counter, int grid, int yb, int parity) {
     const int T = g.KH * g.KW;
-    if (T == 9) launch_qmfma_tt<MT, WM, WN, 9>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb);
-    else if (T == 1) launch_qmfma_tt<MT, WM, WN, 1>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb);
-    else launch_qmfma_tt<MT, WM, WN, 0>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb);
+    if (T == 9) launch_qmfma_tt<MT, WM, WN, 9>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb, parity);
+    else if (T == 1) launch_qmfma_tt<MT, WM, WN, 1>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb, parity);
+    else launch_qmfma_tt<MT, WM, WN, 0>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb, parity);
 }
 
 template <int WM, int WN>
 bool dispatch_qmt(zant_ctx *ctx, const int8_t *xb, const int8_t *wp, const float *mult, const int32_t *corr,
                   const int8_t *padvec, uint8_t *y, const ConvGeom &g, const TilePlan &p, int CB, const QConvArgs &q,
-                  int *counter, int grid, int yb) {
+                  int *counter, int grid, int yb, int parity) {
     switch (p.MT) {
-    case 1: launch_qmfma<1, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb); return true;
-    case 2: launch_qmfma<2, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb); return true;
-    case 3: launch_qmfma<3, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb); return true;
-    case 4: launch_qmfma<4, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb); return true;
-    case 5: launch_qmfma<5, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb); return true;
-    case 6: launch_qmfma<6, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb); return true;
-    case 7: launch_qmfma<7, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb); return true;
+    case 1: launch_qmfma<1, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb, parity); return true;
+    case 2: launch_qmfma<2, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb, parity); return true;
+    case 3: launch_qmfma<3, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb, parity); return true;
+    case 4: launch_qmfma<4, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb, parity); return true;
+    case 5: launch_qmfma<5, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb, parity); return true;
+    case 6: launch_qmfma<6, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb, parity); return true;
+    case 7: launch_qmfma<7, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb, parity); return true;
     default: return false;
     }
 }
@@ -485,7 +487,7 @@ unsigned to_blocked_grid(zant_ctx *ctx, int64_t N, int64_t CB, int64_t hw) {
 // The matrix-core path; returns ZANT_OK when it ran, 1 when the shape is left to the other kernels.
 // x_blocked / y_blocked: x, y are already / are to be written in the blocked signed layout.
 int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float *w_scale, const int32_t *bias, uint8_t *y,
-                   const ConvGeom &g, const QConvArgs &q, bool x_blocked, bool y_blocked) {
+                   const ConvGeom &g, const QConvArgs &q, bool x_blocked, bool y_blocked, zant_pack_slot *slot) {
     if (g.groups != 1 || g.C < 5 || int64_t(g.N) * g.OH * g.OW < 64) return 1;
     const int CB = (g.C + 15) / 16;
     if (int64_t(g.N) * CB * g.H * g.W >= (int64_t(1) << 27)) return 1;  // 16-byte units addressed with 32-bit offsets
@@ -500,9 +502,11 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
     const size_t kpad = size_t(plan.t.n_kblocks) * K_BLK;
     const size_t xb_bytes = x_blocked ? 0 : size_t(g.N) * CB * g.H * g.W * 16;
     const size_t o_pad = 256, o_mult = 512, o_corr = o_mult + align256(kpad * 4), o_wp = o_corr + align256(kpad * 4),
-                 o_xb = o_wp + align256(wp_bytes), total = o_xb + xb_bytes;
-    void *ws = nullptr;
-    int rc = zant_workspace(ctx, total, &ws);
+                 static_bytes = o_wp + align256(wp_bytes);
+    void *ws = nullptr, *dyn = nullptr;
+    bool need_pack = true;
+    int parity = 0;
+    int rc = zant_pack_region(ctx, slot, static_bytes, xb_bytes, &ws, &dyn, &need_pack, &parity);
     if (rc) return rc;
     char *base = static_cast<char *>(ws);
     int *counter = reinterpret_cast<int *>(base);
@@ -510,24 +514,26 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
     float *mult = reinterpret_cast<float *>(base + o_mult);
     int32_t *corr = reinterpret_cast<int32_t *>(base + o_corr);
     int8_t *wp = reinterpret_cast<int8_t *>(base + o_wp);
-    const int8_t *xb = x_blocked ? reinterpret_cast<const int8_t *>(x) : reinterpret_cast<const int8_t *>(base + o_xb);
+    const int8_t *xb = x_blocked ? reinterpret_cast<const int8_t *>(x) : static_cast<const int8_t *>(dyn);
     const int grid = int(std::min<int64_t>(plan.t.n_tiles, int64_t(ctx->num_cus) * 2));
     const unsigned pb = unsigned(std::min<int64_t>(std::max<int64_t>(ceil_div64(int64_t(wp_bytes), 256), ceil_div64(int64_t(kpad), 4)), 1024));
-    hipLaunchKernelGGL(qpack_kernel, dim3(pb), dim3(256), 0, ctx->stream, w, w_scale, bias, wp, mult, corr, padvec, counter,
-                       2 * grid, g.K, g.C, T, plan.t.n_chunks, plan.t.n_kblocks, K_BLK, q.x_scale, q.y_scale, q.x_zp,
-                       q.n_wscale);
-    ZANT_LAUNCH_CHECK(ctx);
+    if (need_pack) {
+        hipLaunchKernelGGL(qpack_kernel, dim3(pb), dim3(256), 0, ctx->stream, w, w_scale, bias, wp, mult, corr, padvec, counter,
+                           2 * grid, g.K, g.C, T, plan.t.n_chunks, plan.t.n_kblocks, K_BLK, q.x_scale, q.y_scale, q.x_zp,
+                           q.n_wscale);
+        ZANT_LAUNCH_CHECK(ctx);
+    }
     if (!x_blocked) {
         const int64_t hw = int64_t(g.H) * g.W;
         const int vec_ok = (hw % 4 == 0) && (reinterpret_cast<uintptr_t>(x) % 4 == 0);
         hipLaunchKernelGGL(to_blocked_s8_kernel, dim3(to_blocked_grid(ctx, g.N, CB, hw)), dim3(256), 0, ctx->stream, x,
-                           reinterpret_cast<uint4 *>(base + o_xb), g.N, g.C, CB, hw, vec_ok);
+                           static_cast<uint4 *>(dyn), g.N, g.C, CB, hw, vec_ok);
         ZANT_LAUNCH_CHECK(ctx);
     }
     KernelTimer kt(ctx);
     const int yb = y_blocked ? 1 : 0;
-    const bool ok = WN == 2 ? dispatch_qmt<2, 2>(ctx, xb, wp, mult, corr, padvec, y, g, plan, CB, q, counter, grid, yb)
-                            : dispatch_qmt<4, 1>(ctx, xb, wp, mult, corr, padvec, y, g, plan, CB, q, counter, grid, yb);
+    const bool ok = WN == 2 ? dispatch_qmt<2, 2>(ctx, xb, wp, mult, corr, padvec, y, g, plan, CB, q, counter, grid, yb, parity)
+                            : dispatch_qmt<4, 1>(ctx, xb, wp, mult, corr, padvec, y, g, plan, CB, q, counter, grid, yb, parity);
     if (!ok) return 1;
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
@@ -647,20 +653,24 @@ bool smallc_eligible(const ConvGeom &g) {
 
 template <int C>
 int launch_smallc(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float *w_scale, const int32_t *bias, uint8_t *y,
-                  const ConvGeom &g, const QConvArgs &q, bool y_blocked, bool pool) {
+                  const ConvGeom &g, const QConvArgs &q, bool y_blocked, bool pool, zant_pack_slot *slot) {
     constexpr int ND = (C * 9 + 3) / 4;
     const int kpad = ((g.K + 15) / 16) * 16;
     const size_t o_mult = 0, o_corr = align256(size_t(kpad) * 4), o_w = 2 * o_corr, total = o_w + size_t(kpad) * ND * 4;
-    void *ws = nullptr;
-    const int rc = zant_workspace(ctx, total, &ws);
+    void *ws = nullptr, *dyn = nullptr;
+    bool need_pack = true;
+    int parity = 0;
+    const int rc = zant_pack_region(ctx, slot, total, 0, &ws, &dyn, &need_pack, &parity);
     if (rc) return rc;
     char *base = static_cast<char *>(ws);
     float *mult = reinterpret_cast<float *>(base + o_mult);
     int32_t *corr = reinterpret_cast<int32_t *>(base + o_corr);
     uint32_t *wpk = reinterpret_cast<uint32_t *>(base + o_w);
-    hipLaunchKernelGGL(qconv_smallc_pack_kernel<C>, dim3((kpad + 255) / 256), dim3(256), 0, ctx->stream, w, w_scale, bias, wpk,
-                       mult, corr, g.K, kpad, q.x_scale, q.y_scale, q.x_zp, q.n_wscale);
-    ZANT_LAUNCH_CHECK(ctx);
+    if (need_pack) {
+        hipLaunchKernelGGL(qconv_smallc_pack_kernel<C>, dim3((kpad + 255) / 256), dim3(256), 0, ctx->stream, w, w_scale, bias,
+                           wpk, mult, corr, g.K, kpad, q.x_scale, q.y_scale, q.x_zp, q.n_wscale);
+        ZANT_LAUNCH_CHECK(ctx);
+    }
     const int64_t positions = int64_t(g.N) * (pool ? g.OH / 2 : g.OH) * (pool ? g.OW / 2 : g.OW);
     const unsigned blocks = unsigned(std::min<int64_t>(std::max<int64_t>(ceil_div64(positions, 256), 1), int64_t(ctx->num_cus) * 32));
     KernelTimer kt(ctx);
@@ -671,12 +681,12 @@ int launch_smallc(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float 
 }
 
 int run_qconv_smallc(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float *w_scale, const int32_t *bias, uint8_t *y,
-                     const ConvGeom &g, const QConvArgs &q, bool y_blocked, bool pool) {
+                     const ConvGeom &g, const QConvArgs &q, bool y_blocked, bool pool, zant_pack_slot *slot) {
     switch (g.C) {
-    case 1: return launch_smallc<1>(ctx, x, w, w_scale, bias, y, g, q, y_blocked, pool);
-    case 2: return launch_smallc<2>(ctx, x, w, w_scale, bias, y, g, q, y_blocked, pool);
-    case 3: return launch_smallc<3>(ctx, x, w, w_scale, bias, y, g, q, y_blocked, pool);
-    default: return launch_smallc<4>(ctx, x, w, w_scale, bias, y, g, q, y_blocked, pool);
+    case 1: return launch_smallc<1>(ctx, x, w, w_scale, bias, y, g, q, y_blocked, pool, slot);
+    case 2: return launch_smallc<2>(ctx, x, w, w_scale, bias, y, g, q, y_blocked, pool, slot);
+    case 3: return launch_smallc<3>(ctx, x, w, w_scale, bias, y, g, q, y_blocked, pool, slot);
+    default: return launch_smallc<4>(ctx, x, w, w_scale, bias, y, g, q, y_blocked, pool, slot);
     }
 }
 
@@ -752,22 +762,25 @@ bool dw_eligible(const ConvGeom &g) {
     return g.groups == g.C && g.K == g.C && g.CG == 1 && g.KH == 3 && g.KW == 3 && g.dh == 1 && g.dw == 1;
 }
 
-// x, y blocked.
+size_t qdw_table_bytes(int C) {
+    const int CB = (C + 15) / 16;
+    return 2 * align256(size_t(CB) * 64) + size_t(CB) * 144 * 4;
+}
+
+// x, y blocked; `tables` holds qdw_table_bytes(C) bytes that are (re)filled when need_pack is set.
 int run_qdw_blocked(zant_ctx *ctx, const uint8_t *xb, const int8_t *w, const float *w_scale, const int32_t *bias, uint8_t *yb,
-                    const ConvGeom &g, const QConvArgs &q, size_t ws_offset) {
+                    const ConvGeom &g, const QConvArgs &q, void *tables, bool need_pack) {
     const int CB = (g.C + 15) / 16, kpad = CB * 16;
-    const size_t o_mult = ws_offset, o_corr = o_mult + align256(size_t(kpad) * 4), o_w = o_corr + align256(size_t(kpad) * 4),
-                 total = o_w + size_t(CB) * 144 * 4;
-    void *ws = nullptr;
-    const int rc = zant_workspace(ctx, total, &ws);
-    if (rc) return rc;
-    char *base = static_cast<char *>(ws);
-    float *mult = reinterpret_cast<float *>(base + o_mult);
+    const size_t o_corr = align256(size_t(kpad) * 4), o_w = 2 * o_corr;
+    char *base = static_cast<char *>(tables);
+    float *mult = reinterpret_cast<float *>(base);
     int32_t *corr = reinterpret_cast<int32_t *>(base + o_corr);
     uint32_t *wm = reinterpret_cast<uint32_t *>(base + o_w);
-    hipLaunchKernelGGL(qdw_pack_kernel, dim3((kpad + 255) / 256), dim3(256), 0, ctx->stream, w, w_scale, bias, wm, mult, corr,
-                       g.K, kpad, q.x_scale, q.y_scale, q.x_zp, q.n_wscale);
-    ZANT_LAUNCH_CHECK(ctx);
+    if (need_pack) {
+        hipLaunchKernelGGL(qdw_pack_kernel, dim3((kpad + 255) / 256), dim3(256), 0, ctx->stream, w, w_scale, bias, wm, mult,
+                           corr, g.K, kpad, q.x_scale, q.y_scale, q.x_zp, q.n_wscale);
+        ZANT_LAUNCH_CHECK(ctx);
+    }
     const int64_t per_cb = int64_t(g.N) * g.OH * g.OW;
     const int64_t want = std::max<int64_t>(1, (int64_t(ctx->num_cus) * 16 + CB - 1) / CB);
     const int blocks_per_cb = int(std::min<int64_t>(std::max<int64_t>(ceil_div64(per_cb, 256), 1), want));
@@ -800,7 +813,7 @@ int zant_qlinearconv_layout_pool(zant_ctx *ctx, const uint8_t *x, const int64_t 
                                  const int8_t *w_zp, float y_scale, uint8_t y_zp, const int32_t *bias, uint8_t *y,
                                  const int64_t ydim[4], const int64_t stride[2], const int64_t pads[4], const int64_t dil[2],
                                  int64_t group, int act, float act_alpha, float act_scale, uint8_t act_zp, int x_layout,
-                                 int y_layout, int fuse_pool, bool query_only) {
+                                 int y_layout, int fuse_pool, bool query_only, zant_pack_slot *slot) {
     if (!ctx || !xdim || !wdim || !ydim || !stride || !pads || !dil) return ZANT_NullPointer;
     for (int i = 0; i < 4; ++i)
         if (xdim[i] <= 0 || wdim[i] <= 0 || xdim[i] > INT32_MAX || wdim[i] > INT32_MAX) return ZANT_InvalidDimensions;
@@ -837,30 +850,31 @@ int zant_qlinearconv_layout_pool(zant_ctx *ctx, const uint8_t *x, const int64_t 
     q.act.act = act; q.act.alpha = act_alpha; q.act.in_scale = y_scale; q.act.in_zp = y_zp;
     q.act.out_scale = act_scale; q.act.out_zp = act_zp;
 
-    if (smallc) return run_qconv_smallc(ctx, x, w, w_scale, bias, y, g, q, yb, fuse_pool != 0);
+    if (smallc) return run_qconv_smallc(ctx, x, w, w_scale, bias, y, g, q, yb, fuse_pool != 0, slot);
 
     const size_t x_blk = zant_blocked_bytes(xdim), y_blk = zant_blocked_bytes(ydim);
     if (w_zp == nullptr && dw_eligible(g)) {
         // the depthwise kernel works blocked -> blocked; NCHW operands pass through conversions in the workspace
-        const size_t o_x = 0, o_y = xb ? 0 : align256(x_blk), o_tab = o_y + (yb ? 0 : align256(y_blk));
-        const int CB = (g.C + 15) / 16;
-        void *ws = nullptr;
-        int rc = zant_workspace(ctx, o_tab + 2 * align256(size_t(CB) * 64) + size_t(CB) * 144 * 4, &ws);
+        const size_t o_y = xb ? 0 : align256(x_blk), dyn_bytes = o_y + (yb ? 0 : align256(y_blk));
+        void *tables = nullptr, *dyn = nullptr;
+        bool need_pack = true;
+        int parity = 0;
+        int rc = zant_pack_region(ctx, slot, qdw_table_bytes(g.C), dyn_bytes, &tables, &dyn, &need_pack, &parity);
         if (rc) return rc;
-        char *base = static_cast<char *>(ws);
+        char *base = static_cast<char *>(dyn);
         const uint8_t *xin = x;
         if (!xb) {
-            rc = zant_to_blocked(ctx, x, g.N, g.C, int64_t(g.H) * g.W, reinterpret_cast<uint8_t *>(base + o_x));
+            rc = zant_to_blocked(ctx, x, g.N, g.C, int64_t(g.H) * g.W, reinterpret_cast<uint8_t *>(base));
             if (rc) return rc;
-            xin = reinterpret_cast<uint8_t *>(base + o_x);
+            xin = reinterpret_cast<uint8_t *>(base);
         }
         uint8_t *yout = yb ? y : reinterpret_cast<uint8_t *>(base + o_y);
-        rc = run_qdw_blocked(ctx, xin, w, w_scale, bias, yout, g, q, o_tab);
+        rc = run_qdw_blocked(ctx, xin, w, w_scale, bias, yout, g, q, tables, need_pack);
         if (rc) return rc;
         return yb ? ZANT_OK : zant_from_blocked(ctx, yout, g.N, g.K, int64_t(g.OH) * g.OW, y);
     }
     if (w_zp == nullptr) {  // a non-zero weight zero point makes the correction position dependent: direct kernel
-        const int rc = run_qconv_mfma(ctx, x, w, w_scale, bias, y, g, q, xb, yb);
+        const int rc = run_qconv_mfma(ctx, x, w, w_scale, bias, y, g, q, xb, yb, slot);
         if (rc <= 0) return rc;
     }
     // direct kernel: NCHW only; blocked operands pass through conversions in the workspace
@@ -898,5 +912,5 @@ extern "C" int zant_hip_qlinearconv_u8i8(zant_ctx *ctx, const uint8_t *x, const 
                                          float act_alpha, float act_scale, uint8_t act_zp) {
     return zant_qlinearconv_layout_pool(ctx, x, xdim, x_scale, x_zp, w, wdim, w_scale, n_wscale, w_zp, y_scale, y_zp, bias, y,
                                         ydim, stride, pads, dil, group, act, act_alpha, act_scale, act_zp, ZANT_LAYOUT_NCHW,
-                                        ZANT_LAYOUT_NCHW, 0, false);
+                                        ZANT_LAYOUT_NCHW, 0, false, nullptr);
 }

@@ -18,12 +18,13 @@ static inline size_t zant_blocked_bytes(const int64_t dim[4]) {
 // fuse_pool: also max-pool 2x2/2 (floor, no padding) in the same kernel; ydim is then the pooled shape.  Only the
 // first-layer kernel (1..4 input channels, 3x3, NCHW input) does that: other shapes return 1 and run nothing.
 // query_only: validate and report eligibility (ZANT_OK / 1 / error status) without touching any pointer.
+// slot: where weight-derived scratch is kept across calls (nullptr: repacked on every call).
 int zant_qlinearconv_layout_pool(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], float x_scale, uint8_t x_zp,
                                  const int8_t *w, const int64_t wdim[4], const float *w_scale, int64_t n_wscale,
                                  const int8_t *w_zp, float y_scale, uint8_t y_zp, const int32_t *bias, uint8_t *y,
                                  const int64_t ydim[4], const int64_t stride[2], const int64_t pads[4], const int64_t dil[2],
                                  int64_t group, int act, float act_alpha, float act_scale, uint8_t act_zp, int x_layout,
-                                 int y_layout, int fuse_pool, bool query_only);
+                                 int y_layout, int fuse_pool, bool query_only, zant_pack_slot *slot);
 
 // Layout conversions (HW = H * W).
 int zant_to_blocked(zant_ctx *ctx, const uint8_t *x, int64_t N, int64_t C, int64_t HW, uint8_t *xb);
