@@ -273,6 +273,11 @@ int zant_model_read_tensor(zant_model *m, int id, void *dst_host, size_t bytes);
  * until the next call. */
 int zant_model_bind_predict(zant_model *m);
 void predict(float *input, uint32_t *input_shape, uint32_t shape_len, float **result);
+/* predict() for callers that only know the batch: `n` must equal the leading dimension the bound model was built
+ * with (the reference compiles the batch into predict's shape check, predict.zig:328-334); otherwise it returns
+ * silently with *result untouched, as predict does.  No counterpart in the reference: it exists for the batched
+ * measurements (batch 4096 / 512 / 1024). */
+void predict_batched(float *input, uint32_t n, float **result);
 
 #ifdef __cplusplus
 }

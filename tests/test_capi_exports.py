@@ -12,7 +12,7 @@ HEADER = os.path.join(ROOT, "include", "zant_hip.h")
 def declared_symbols():
     text = open(HEADER).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    names = re.findall(r"\b(zant_hip_\w+|zant_model_\w+|setLogFunctionC|setLogFunction|predict)\s*\(", text)
+    names = re.findall(r"\b(zant_hip_\w+|zant_model_\w+|setLogFunctionC|setLogFunction|predict_batched|predict)\s*\(", text)
     return sorted(set(names))
 
 

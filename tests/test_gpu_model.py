@@ -119,6 +119,25 @@ def test_mnist8_style_graph_folds_add_into_conv_bias(G):
     np.testing.assert_allclose(y, r, rtol=G.RTOL, atol=1e-4)
 
 
+def test_real_mnist8_onnx_weights_against_the_oracle(G):
+    """The bundled mnist-8.onnx (the reference's datasets/models/mnist-8, kept as a data fixture) read by the package's
+    ONNX reader and run by the executor, against the oracle executing the same graph node by node.  Covers SAME_UPPER
+    5x5 convolutions, broadcast-Add biases {C,1,1}, a 3x3/3 MaxPool, a folded constant Reshape and MatMul + Add."""
+    import os
+    from zant_amd import onnx_front
+    graph = onnx_front.read_graph(os.path.join(os.path.dirname(__file__), "golden", "mnist-8.onnx"))
+    assert [n["op"] for n in graph["nodes"]].count("Conv") == 2 and graph["inputs"][0][1] == [1, 1, 28, 28]
+    m = onnx_front.build_model(G.tm.context(), graph)
+    assert m.num_launches == 5  # conv(+add+relu+pool), conv(+add+relu), pool 3x3, matmul, add
+    g = np.random.default_rng(8)
+    for k in range(4):
+        img = g.random((1, 1, 28, 28), dtype=np.float32) * (255.0 if k % 2 else 1.0)  # raw 0..255 pixels and 0..1
+        ref = onnx_front.run_graph(graph, zo, img)
+        y = m.predict_host(img)
+        np.testing.assert_allclose(y, ref, rtol=G.RTOL, atol=1e-4 * max(1.0, float(np.abs(ref).max())))
+    m.close()
+
+
 def test_predict_entry_point_follows_the_reference_abi(G):
     from zant_amd import networks
     params = networks.readme_cnn_params(seed=0)
@@ -143,6 +162,12 @@ def test_predict_entry_point_follows_the_reference_abi(G):
     first_ptr = result.value
     call([1, 1, 28, 28])
     assert result.value == first_ptr  # library-owned storage, reused by the next call
+    # the batched form: only the batch is passed and must be the compiled-in one
+    rb = C.c_void_p(0)
+    lib.predict_batched(img.ctypes.data_as(C.c_void_p), 2, C.byref(rb))
+    assert rb.value is None
+    lib.predict_batched(img.ctypes.data_as(C.c_void_p), 1, C.byref(rb))
+    assert rb.value == first_ptr
     lib.zant_model_bind_predict(None)
     result2 = C.c_void_p(0)
     arr = (C.c_uint32 * 4)(1, 1, 28, 28)

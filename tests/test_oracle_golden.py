@@ -145,3 +145,23 @@ def test_conv_error_paths():
     with pytest.raises(zo.OracleError) as e:
         zo.Conv(x, w, None, [1, 1], [1, 1, 1, 1], None, 1, None)
     assert e.value.name == "InvalidDimensions"
+
+
+def test_onnx_reader_decodes_the_bundled_mnist8_graph():
+    """The reader needs no GPU: node list, attributes and initialiser shapes of mnist-8.onnx are what the reference's
+    hand-written translation of the same file lists (src/codeGen/hardcoded/hardcoded_mnist8.zig:140-288)."""
+    import importlib.util
+    import os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("onnx_front", os.path.join(root, "z-ant_amd", "onnx_front.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    g = mod.read_graph(os.path.join(root, "tests", "golden", "mnist-8.onnx"))
+    assert [n["op"] for n in g["nodes"]] == ["Reshape", "Conv", "Add", "Relu", "MaxPool", "Conv", "Add", "Relu", "MaxPool",
+                                             "Reshape", "MatMul", "Add"]
+    assert g["nodes"][1]["attrs"]["auto_pad"] == "SAME_UPPER" and g["nodes"][1]["attrs"]["kernel_shape"] == [5, 5]
+    assert g["nodes"][8]["attrs"]["kernel_shape"] == [3, 3] and g["nodes"][8]["attrs"]["strides"] == [3, 3]
+    shapes = {k: v.shape for k, v in g["initializers"].items()}
+    assert shapes["Parameter5"] == (8, 1, 5, 5) and shapes["Parameter87"] == (16, 8, 5, 5)
+    assert shapes["Parameter6"] == (8, 1, 1) and shapes["Parameter193"] == (16, 4, 4, 10) and shapes["Parameter194"] == (1, 10)
+    assert g["inputs"] == [("Input3", [1, 1, 28, 28])] and g["outputs"] == [("Plus214_Output_0", [1, 10])]

@@ -9,3 +9,4 @@ for device memory and streams.  There is no CPU fallback: importing fails if the
 from .capi import Context, ZantError, lib, lib_path, status_name  # noqa: F401
 from . import tensor_math  # noqa: F401
 from . import model  # noqa: F401
+from . import onnx_front  # noqa: F401

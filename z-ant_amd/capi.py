@@ -99,6 +99,7 @@ PROTOTYPES = {
     "zant_model_read_tensor": (i32, [vp, i32, vp, sz]),
     "zant_model_bind_predict": (i32, [vp]),
     "predict": (None, [vp, C.POINTER(C.c_uint32), C.c_uint32, C.POINTER(vp)]),
+    "predict_batched": (None, [vp, C.c_uint32, C.POINTER(vp)]),
 }
 
 for _name, (_res, _args) in PROTOTYPES.items():

@@ -47,6 +47,22 @@ __global__ void pack_weights_f32_kernel(const float *__restrict__ w, float *__re
     }
 }
 
+// LDS byte address of a pointer into the workgroup's shared memory.
+__device__ __forceinline__ unsigned lds_addr_of(const void *p) {
+    return unsigned(reinterpret_cast<uintptr_t>((lptr_t) const_cast<void *>(p)));
+}
+// Starts a 64-bit LDS read without the compiler's knowledge (it inserts no waits of its own for it) ...
+__device__ __forceinline__ int2 lds_read64_async(unsigned addr) {
+    int2 v;
+    asm volatile("ds_read_b64 %0, %1" : "=v"(v) : "v"(addr));
+    return v;
+}
+// ... and this waits for every outstanding LDS operation; the values are in/out operands so that their users stay
+// behind the wait.
+__device__ __forceinline__ void lds_wait_all(int2 &a, int2 &b, int2 &c, int2 &d) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+}
+
 // A few zero words that padding lanes of the asynchronous global->LDS copies read from.
 __device__ float g_zero_words[4] = {0.f, 0.f, 0.f, 0.f};
 
@@ -89,18 +105,31 @@ __device__ __forceinline__ void conv_step(float *__restrict__ dma, const float *
         const int ih0 = oh0 * g.sh - g.pt;
         const int imgs_here = min(t.NB, g.N - n0);
         const int j = tid & 3;
-        for (int p0 = 0; p0 < t.P1; p0 += PPI) {
-            const int pos = p0 + (tid >> 2);
-            if (pos < t.P1) {
-                const int2 e = ptab[pos];
-                const int ih = ih0 + (e.y & 0xffff);
-                const bool ok = e.x >= 0 && ih >= 0 && ih < g.H && (e.y >> 16) < imgs_here;
-                const float *src = xb + (e.x + ih0 * g.W) + int64_t(ichunk * CC + j) * x_plane;
+        // The patch table lives in LDS.  The compiler drains every outstanding asynchronous copy before an LDS read
+        // it issues itself in this loop (one round trip to L2 per iteration, which made staging cost ~18 % of a
+        // step), so the table is read with hand-written ds_read_b64, one iteration ahead of its use.
+        const unsigned ptab_addr = lds_addr_of(ptab);
+        for (int p0 = 0; p0 < t.P1; p0 += 4 * PPI) {
+            // four table entries per round; nothing read this way stays in flight across a loop edge (a register
+            // copy there would run before the data has landed)
+            int2 e[4];
 #pragma unroll
-                for (int half = 0; half < 2; ++half) {
-                    const int c = ichunk * CC + half * 4 + j;
-                    const float *sp = (ok && c < g.C) ? src + half * 4 * x_plane : g_zero_words;
-                    __builtin_amdgcn_global_load_lds((gptr_t)sp, (lptr_t)(xl + (half * t.P1s + p0 + wave * 16) * 4), 4, 0, 0);
+            for (int u = 0; u < 4; ++u)
+                e[u] = lds_read64_async(ptab_addr + unsigned(min(p0 + u * PPI + (tid >> 2), t.P1 - 1)) * 8u);
+            lds_wait_all(e[0], e[1], e[2], e[3]);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int pos = p0 + u * PPI + (tid >> 2);
+                if (pos < t.P1) {
+                    const int ih = ih0 + (e[u].y & 0xffff);
+                    const bool ok = e[u].x >= 0 && ih >= 0 && ih < g.H && (e[u].y >> 16) < imgs_here;
+                    const float *src = xb + (e[u].x + ih0 * g.W) + int64_t(ichunk * CC + j) * x_plane;
+#pragma unroll
+                    for (int half = 0; half < 2; ++half) {
+                        const int c = ichunk * CC + half * 4 + j;
+                        const float *sp = (ok && c < g.C) ? src + half * 4 * x_plane : g_zero_words;
+                        __builtin_amdgcn_global_load_lds((gptr_t)sp, (lptr_t)(xl + (half * t.P1s + p0 + u * PPI + wave * 16) * 4), 4, 0, 0);
+                    }
                 }
             }
         }
@@ -480,8 +509,16 @@ typedef TilePlan MfmaPlan;
 
 // Tile shape with the best useful-lane fraction whose LDS footprint allows two workgroups per CU.
 bool plan_mfma(const ConvGeom &g, MfmaPlan *best, bool pool = false) {
-    const int WN = g.K > 32 ? 2 : 1, WM = 4 / WN;
-    return zant_plan_conv_tiles(g, WM, WN, 8, CC, sizeof(float), 80 * 1024, best, pool);
+    if (g.K <= 32) return zant_plan_conv_tiles(g, 4, 1, 8, CC, sizeof(float), 80 * 1024, best, pool);
+    // 64 output channels per workgroup (2 x 2 waves) stage the input patch once per 64 channels; 32 per workgroup
+    // (4 x 1 waves) stage it twice but have twice the position slots, which can fit small feature maps much better
+    // (e.g. 5 whole 5x5 pooled images in 128 slots instead of 2 in 64).  Take the narrow shape only for a clear win.
+    MfmaPlan wide, narrow;
+    const bool ok_w = zant_plan_conv_tiles(g, 2, 2, 8, CC, sizeof(float), 80 * 1024, &wide, pool);
+    const bool ok_n = zant_plan_conv_tiles(g, 4, 1, 8, CC, sizeof(float), 80 * 1024, &narrow, pool);
+    if (ok_n && (!ok_w || narrow.eff > wide.eff + 0.1)) { *best = narrow; return true; }
+    if (ok_w) { *best = wide; return true; }
+    return false;
 }
 
 template <int MT, int WM, int WN, int TT, bool POOL>

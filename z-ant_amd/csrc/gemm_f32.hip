@@ -366,6 +366,9 @@ __device__ __forceinline__ void gemm_step(float *__restrict__ dma, unsigned cmp_
                 ++q;
             }
     }
+    // The look-ahead reads were issued a whole burst ago; make sure they have landed before the step ends: a value
+    // still in flight across the loop edge would be at the mercy of any register copy the compiler puts there.
+    lds_wait<0, MT>(a[0], b[0]);
     };
     if (fast) multiply(std::true_type{});
     else multiply(std::false_type{});

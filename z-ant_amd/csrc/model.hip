@@ -944,3 +944,13 @@ extern "C" void predict(float *input, uint32_t *input_shape, uint32_t shape_len,
     *result = reinterpret_cast<float *>(m->result_host.data());
     zant_log("Prediction completed.\n");
 }
+
+extern "C" void predict_batched(float *input, uint32_t n, float **result) {
+    zant_model *m = g_predict_model;
+    if (!m || !input || !result) return;
+    const MTensor &tin = m->t[m->input];
+    if (tin.rank < 1 || int64_t(n) != tin.dim[0]) return;
+    uint32_t shape[8];
+    for (int i = 0; i < tin.rank; ++i) shape[i] = uint32_t(tin.dim[i]);
+    predict(input, shape, uint32_t(tin.rank), result);
+}

@@ -1,0 +1,265 @@
+"""A minimal ONNX reader for the operator set of the hot path: decodes the protobuf wire format directly (no onnx
+package), folds Reshape on initialisers, and builds a ``Model`` (the executor behind the generated ``predict()``).
+
+The reference parses ONNX in Zig (src/onnx/protobuf.zig:31-203, src/onnx/onnx.zig) and turns each node into one
+``tensMath.*_lean`` call (src/codeGen/math_handler.zig:31-108); this does the same for Conv, Add, Relu, LeakyRelu,
+MaxPool, Reshape, MatMul, Gemm and Softmax, which covers the bundled mnist-8 network.
+"""
+import struct
+
+import numpy as np
+
+# ------------------------------------------------------------------------------------------------ protobuf wire format
+
+
+def _varint(buf, pos):
+    result = shift = 0
+    while True:
+        b = buf[pos]
+        pos += 1
+        result |= (b & 0x7F) << shift
+        if not b & 0x80:
+            return result, pos
+        shift += 7
+
+
+def _fields(buf):
+    """Yields (field number, wire type, value) of one message; length-delimited values are memoryviews."""
+    pos, end = 0, len(buf)
+    while pos < end:
+        key, pos = _varint(buf, pos)
+        num, wt = key >> 3, key & 7
+        if wt == 0:
+            val, pos = _varint(buf, pos)
+        elif wt == 1:
+            val, pos = bytes(buf[pos:pos + 8]), pos + 8
+        elif wt == 2:
+            n, pos = _varint(buf, pos)
+            val, pos = buf[pos:pos + n], pos + n
+        elif wt == 5:
+            val, pos = bytes(buf[pos:pos + 4]), pos + 4
+        else:
+            raise ValueError(f"unsupported protobuf wire type {wt}")
+        yield num, wt, val
+
+
+def _signed(v):
+    return v - (1 << 64) if v >= 1 << 63 else v
+
+
+def _packed_ints(wt, val):
+    if wt == 0:
+        return [_signed(val)]
+    out, pos = [], 0
+    while pos < len(val):
+        v, pos = _varint(val, pos)
+        out.append(_signed(v))
+    return out
+
+
+_DTYPES = {1: np.float32, 2: np.uint8, 3: np.int8, 6: np.int32, 7: np.int64, 11: np.float64}
+
+
+def _tensor(buf):
+    dims, dtype, name, raw, floats, ints = [], 1, "", None, [], []
+    for num, wt, val in _fields(buf):
+        if num == 1:
+            dims += _packed_ints(wt, val)
+        elif num == 2:
+            dtype = val
+        elif num == 8:
+            name = bytes(val).decode()
+        elif num == 9:
+            raw = bytes(val)
+        elif num == 4:
+            floats += [struct.unpack("<f", val)[0]] if wt == 5 else list(np.frombuffer(bytes(val), "<f4"))
+        elif num in (5, 7):
+            ints += _packed_ints(wt, val)
+    np_dtype = _DTYPES[dtype]
+    if raw is not None:
+        arr = np.frombuffer(raw, dtype=np.dtype(np_dtype).newbyteorder("<")).astype(np_dtype)
+    elif floats:
+        arr = np.array(floats, np_dtype)
+    else:
+        arr = np.array(ints, np_dtype)
+    return name, arr.reshape(dims)
+
+
+def _attribute(buf):
+    name, out, ints, floats = "", None, [], []
+    for num, wt, val in _fields(buf):
+        if num == 1:
+            name = bytes(val).decode()
+        elif num == 2:
+            out = struct.unpack("<f", val)[0]
+        elif num == 3:
+            out = _signed(val)
+        elif num == 4:
+            out = bytes(val).decode()
+        elif num == 5:
+            out = _tensor(val)[1]
+        elif num == 7:
+            floats += [struct.unpack("<f", val)[0]] if wt == 5 else list(np.frombuffer(bytes(val), "<f4"))
+        elif num == 8:
+            ints += _packed_ints(wt, val)
+    if ints:
+        out = ints
+    elif floats:
+        out = floats
+    return name, out
+
+
+def _node(buf):
+    node = {"inputs": [], "outputs": [], "op": "", "attrs": {}}
+    for num, _, val in _fields(buf):
+        if num == 1:
+            node["inputs"].append(bytes(val).decode())
+        elif num == 2:
+            node["outputs"].append(bytes(val).decode())
+        elif num == 4:
+            node["op"] = bytes(val).decode()
+        elif num == 5:
+            k, v = _attribute(val)
+            node["attrs"][k] = v
+    return node
+
+
+def _value_info(buf):
+    name, dims = "", []
+    for num, _, val in _fields(buf):
+        if num == 1:
+            name = bytes(val).decode()
+        elif num == 2:  # TypeProto
+            for n2, _, v2 in _fields(val):
+                if n2 == 1:  # tensor_type
+                    for n3, _, v3 in _fields(v2):
+                        if n3 == 2:  # shape
+                            for n4, _, v4 in _fields(v3):
+                                if n4 == 1:  # dim
+                                    d = 1
+                                    for n5, _, v5 in _fields(v4):
+                                        if n5 == 1:
+                                            d = v5
+                                    dims.append(int(d))
+    return name, dims
+
+
+def read_graph(path):
+    """-> {"nodes": [...], "initializers": {name: ndarray}, "inputs": [(name, dims)], "outputs": [(name, dims)]}"""
+    buf = memoryview(open(path, "rb").read())
+    graph = None
+    for num, _, val in _fields(buf):
+        if num == 7:
+            graph = val
+    if graph is None:
+        raise ValueError("no graph in the ONNX file")
+    g = {"nodes": [], "initializers": {}, "inputs": [], "outputs": []}
+    for num, _, val in _fields(graph):
+        if num == 1:
+            g["nodes"].append(_node(val))
+        elif num == 5:
+            name, arr = _tensor(val)
+            g["initializers"][name] = arr
+        elif num == 11:
+            g["inputs"].append(_value_info(val))
+        elif num == 12:
+            g["outputs"].append(_value_info(val))
+    g["inputs"] = [(n, d) for n, d in g["inputs"] if n not in g["initializers"]]
+    return g
+
+
+# ------------------------------------------------------------------------------------------------ graph -> executor
+
+def _pool_or_conv_attrs(a, rank2_default):
+    strides = a.get("strides", rank2_default)
+    pads = a.get("pads")
+    dil = a.get("dilations", [1, 1])
+    auto_pad = a.get("auto_pad", "NOTSET")
+    return strides, pads, dil, auto_pad
+
+
+def run_graph(graph, ops, x):
+    """Executes the graph with ``ops`` (an object with the reference-named operators: the CPU oracle module, or any
+    other implementation with the same signatures) on the numpy input ``x``.  Used by tests as the checker's driver."""
+    vals = dict(graph["initializers"])
+    vals[graph["inputs"][0][0]] = x
+    for nd in graph["nodes"]:
+        i = [vals[n] for n in nd["inputs"] if n]
+        a = nd["attrs"]
+        if nd["op"] == "Conv":
+            s, p, d, ap = _pool_or_conv_attrs(a, [1, 1])
+            y = ops.Conv(i[0], i[1], i[2] if len(i) > 2 else None, s, p if p is not None else ([0, 0, 0, 0] if ap == "NOTSET" else None), d,
+                         a.get("group", 1), ap)
+        elif nd["op"] == "Add":
+            y = ops.sum_tensors_lean(i[0], i[1])
+        elif nd["op"] == "Relu":
+            y = ops.ReLU(i[0])
+        elif nd["op"] == "MaxPool":
+            s, p, d, ap = _pool_or_conv_attrs(a, [1, 1])
+            y = ops.onnx_maxpool(i[0], a["kernel_shape"], s, d, p if p is not None else [0, 0, 0, 0], ap)
+        elif nd["op"] == "Reshape":
+            y = ops.reshape_lean(i[0], [int(v) for v in i[1]])
+        elif nd["op"] == "MatMul":
+            y = ops.mat_mul(i[0], i[1])
+        elif nd["op"] == "Softmax":
+            y = ops.softmax(i[0])
+        else:
+            raise NotImplementedError(nd["op"])
+        vals[nd["outputs"][0]] = y
+    return vals[graph["outputs"][0][0]]
+
+
+def build_model(ctx, graph):
+    """Turns the graph into a finalized ``Model``: one executor node per ONNX node, initialisers as parameters, Reshape
+    of an initialiser folded on the host (as the reference's code generator does for constant inputs)."""
+    from .model import Model
+    m = Model(ctx)
+    consts = dict(graph["initializers"])
+    name, dims = graph["inputs"][0]
+    tens = {name: m.input(tuple(dims))}
+
+    def reshape_const(arr, shape):
+        shape = [arr.shape[k] if v == 0 else int(v) for k, v in enumerate(shape)]
+        return arr.reshape(shape)
+
+    for nd in graph["nodes"]:
+        ins, a, out = nd["inputs"], nd["attrs"], nd["outputs"][0]
+        op = nd["op"]
+        if op == "Reshape" and ins[0] in consts:
+            consts[out] = reshape_const(consts[ins[0]], consts[ins[1]])
+            continue
+        if op == "Conv":
+            s, p, d, ap = _pool_or_conv_attrs(a, [1, 1])
+            bias = consts[ins[2]] if len(ins) > 2 and ins[2] else None
+            if p is None and ap == "NOTSET":
+                p = [0, 0, 0, 0]
+            t = m.conv(tens[ins[0]], consts[ins[1]].astype(np.float32), bias, s, p, d, a.get("group", 1), ap)
+        elif op == "Add":
+            if ins[1] in consts:
+                t = m.add_const(tens[ins[0]], consts[ins[1]].astype(np.float32))
+            elif ins[0] in consts:
+                t = m.add_const(tens[ins[1]], consts[ins[0]].astype(np.float32))
+            else:
+                t = m.add(tens[ins[0]], tens[ins[1]])
+        elif op == "Relu":
+            t = m.relu(tens[ins[0]])
+        elif op == "LeakyRelu":
+            t = m.leaky_relu(tens[ins[0]], a.get("alpha", 0.01))
+        elif op == "MaxPool":
+            s, p, d, ap = _pool_or_conv_attrs(a, [1, 1])
+            t = m.maxpool(tens[ins[0]], a["kernel_shape"], s, d, p if p is not None else [0, 0, 0, 0], ap,
+                          bool(a.get("ceil_mode", 0)))
+        elif op == "Reshape":
+            t = m.reshape(tens[ins[0]], [int(v) for v in consts[ins[1]]])
+        elif op == "MatMul":
+            t = m.matmul(tens[ins[0]], consts[ins[1]].astype(np.float32))
+        elif op == "Gemm":
+            c = consts[ins[2]].astype(np.float32) if len(ins) > 2 and ins[2] else None
+            t = m.gemm(tens[ins[0]], consts[ins[1]].astype(np.float32), c, a.get("alpha", 1.0), a.get("beta", 1.0),
+                       bool(a.get("transA", 0)), bool(a.get("transB", 0)))
+        elif op == "Softmax":
+            t = m.softmax(tens[ins[0]])
+        else:
+            raise NotImplementedError(f"ONNX operator {op} is outside the hot path")
+        tens[out] = t
+    return m.finalize()
