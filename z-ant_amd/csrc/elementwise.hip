@@ -28,20 +28,33 @@ __device__ __forceinline__ float unary_op(float v, float slope) {
 template <int OP>
 __global__ void __launch_bounds__(kThreads) unary_f32_kernel(const float *__restrict__ x, float *__restrict__ y,
                                                             int64_t n, float slope) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
     const int64_t n4 = n >> 2;
-    const int64_t step = int64_t(gridDim.x) * blockDim.x;
-    int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
-    const float4 *x4 = reinterpret_cast<const float4 *>(x);
-    float4 *y4 = reinterpret_cast<float4 *>(y);
-    for (int64_t j = i; j < n4; j += step) {
-        float4 v = x4[j];
-        v.x = unary_op<OP>(v.x, slope);
-        v.y = unary_op<OP>(v.y, slope);
-        v.z = unary_op<OP>(v.z, slope);
-        v.w = unary_op<OP>(v.w, slope);
-        y4[j] = v;
+    const int64_t base = int64_t(blockIdx.x) * (kThreads * ZANT_STREAM_U) + threadIdx.x;
+    const f4 *x4 = reinterpret_cast<const f4 *>(x);
+    f4 *y4 = reinterpret_cast<f4 *>(y);
+    f4 v[ZANT_STREAM_U];
+#pragma unroll
+    for (int u = 0; u < ZANT_STREAM_U; ++u) {
+        const int64_t j = base + u * kThreads;
+        if (j < n4) v[u] = __builtin_nontemporal_load(x4 + j);
     }
-    for (int64_t j = (n4 << 2) + i; j < n; j += step) y[j] = unary_op<OP>(x[j], slope);
+#pragma unroll
+    for (int u = 0; u < ZANT_STREAM_U; ++u) {
+        const int64_t j = base + u * kThreads;
+        if (j < n4) {
+            f4 r;
+            r.x = unary_op<OP>(v[u].x, slope);
+            r.y = unary_op<OP>(v[u].y, slope);
+            r.z = unary_op<OP>(v[u].z, slope);
+            r.w = unary_op<OP>(v[u].w, slope);
+            __builtin_nontemporal_store(r, y4 + j);
+        }
+    }
+    if (blockIdx.x == 0) {  // the 0..3 elements behind the last full vector
+        const int64_t j = (n4 << 2) + threadIdx.x;
+        if (j < n) y[j] = unary_op<OP>(x[j], slope);
+    }
 }
 
 template <int OP>
@@ -58,8 +71,8 @@ int launch_unary(zant_ctx *ctx, const float *x, float *y, int64_t n, float slope
     const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
     if (aligned) {
         KernelTimer kt(ctx);
-        hipLaunchKernelGGL(unary_f32_kernel<OP>, dim3(grid_for(n, kThreads * 4, ctx->num_cus)), dim3(kThreads), 0,
-                           ctx->stream, x, y, n, slope);
+        hipLaunchKernelGGL(unary_f32_kernel<OP>, dim3(zant_stream_grid(n >> 2)), dim3(kThreads), 0, ctx->stream, x, y, n,
+                           slope);
     } else {
         KernelTimer kt(ctx);
         hipLaunchKernelGGL(unary_f32_unaligned_kernel<OP>, dim3(grid_for(n, kThreads, ctx->num_cus)), dim3(kThreads),
@@ -106,21 +119,35 @@ __global__ void __launch_bounds__(kThreads) softmax_f32_kernel(const float *__re
 
 __global__ void __launch_bounds__(kThreads) add_same_f32_kernel(const float *__restrict__ a, const float *__restrict__ b,
                                                                float *__restrict__ y, int64_t n, int vec) {
-    const int64_t step = int64_t(gridDim.x) * blockDim.x;
-    const int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
-    int64_t done = 0;
-    if (vec) {
-        const int64_t n4 = n >> 2;
-        const float4 *a4 = reinterpret_cast<const float4 *>(a);
-        const float4 *b4 = reinterpret_cast<const float4 *>(b);
-        float4 *y4 = reinterpret_cast<float4 *>(y);
-        for (int64_t j = i; j < n4; j += step) {
-            const float4 u = a4[j], v = b4[j];
-            y4[j] = make_float4(u.x + v.x, u.y + v.y, u.z + v.z, u.w + v.w);
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    if (!vec) {  // unaligned operands: scalar, one element per thread of the same grid shape
+        const int64_t base = int64_t(blockIdx.x) * (kThreads * ZANT_STREAM_U * 4) + threadIdx.x;
+        for (int u = 0; u < ZANT_STREAM_U * 4; ++u) {
+            const int64_t j = base + u * kThreads;
+            if (j < n) y[j] = a[j] + b[j];
         }
-        done = n4 << 2;
+        return;
     }
-    for (int64_t j = done + i; j < n; j += step) y[j] = a[j] + b[j];
+    const int64_t n4 = n >> 2;
+    const int64_t base = int64_t(blockIdx.x) * (kThreads * ZANT_STREAM_U) + threadIdx.x;
+    const f4 *a4 = reinterpret_cast<const f4 *>(a);
+    const f4 *b4 = reinterpret_cast<const f4 *>(b);
+    f4 *y4 = reinterpret_cast<f4 *>(y);
+    f4 va[ZANT_STREAM_U], vb[ZANT_STREAM_U];
+#pragma unroll
+    for (int u = 0; u < ZANT_STREAM_U; ++u) {
+        const int64_t j = base + u * kThreads;
+        if (j < n4) { va[u] = __builtin_nontemporal_load(a4 + j); vb[u] = __builtin_nontemporal_load(b4 + j); }
+    }
+#pragma unroll
+    for (int u = 0; u < ZANT_STREAM_U; ++u) {
+        const int64_t j = base + u * kThreads;
+        if (j < n4) __builtin_nontemporal_store(va[u] + vb[u], y4 + j);
+    }
+    if (blockIdx.x == 0) {
+        const int64_t j = (n4 << 2) + threadIdx.x;
+        if (j < n) y[j] = a[j] + b[j];
+    }
 }
 
 struct BcastArgs {
@@ -308,8 +335,8 @@ extern "C" int zant_hip_add_f32(zant_ctx *ctx, const float *a, const int64_t *ad
         if (!a || !b || !y) return ZANT_NullPointer;
         const int vec = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
         KernelTimer kt(ctx);
-        hipLaunchKernelGGL(add_same_f32_kernel, dim3(grid_for(asz, kThreads * 4, ctx->num_cus)), dim3(kThreads), 0,
-                           ctx->stream, a, b, y, asz, vec);
+        hipLaunchKernelGGL(add_same_f32_kernel, dim3(zant_stream_grid((asz + 3) >> 2)), dim3(kThreads), 0, ctx->stream, a, b,
+                           y, asz, vec);
         ZANT_LAUNCH_CHECK(ctx);
         return ZANT_OK;
     }

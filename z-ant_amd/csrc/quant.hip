@@ -33,6 +33,72 @@ __global__ void __launch_bounds__(kThreads) quantize_kernel(const float *__restr
     }
 }
 
+// Per-tensor scale, 16-byte aligned x: one float4 in, four bytes out per vector (both coalesced across the lanes).
+__global__ void __launch_bounds__(kThreads) quantize_vec_kernel(const float *__restrict__ x, const float *__restrict__ scale,
+                                                               const uint8_t *__restrict__ zp, uint8_t *__restrict__ y,
+                                                               int64_t n) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    const float s = scale[0];
+    const uint8_t z = zp ? zp[0] : uint8_t(0);
+    const int64_t n4 = n >> 2;
+    const int64_t base = int64_t(blockIdx.x) * (kThreads * ZANT_STREAM_U) + threadIdx.x;
+    const f4 *x4 = reinterpret_cast<const f4 *>(x);
+    uint32_t *y4 = reinterpret_cast<uint32_t *>(y);
+    f4 v[ZANT_STREAM_U];
+#pragma unroll
+    for (int u = 0; u < ZANT_STREAM_U; ++u) {
+        const int64_t j = base + u * kThreads;
+        if (j < n4) v[u] = __builtin_nontemporal_load(x4 + j);
+    }
+#pragma unroll
+    for (int u = 0; u < ZANT_STREAM_U; ++u) {
+        const int64_t j = base + u * kThreads;
+        if (j < n4) {
+            const uint32_t r = uint32_t(sat_u8_rne(v[u].x / s, z)) | (uint32_t(sat_u8_rne(v[u].y / s, z)) << 8) |
+                               (uint32_t(sat_u8_rne(v[u].z / s, z)) << 16) | (uint32_t(sat_u8_rne(v[u].w / s, z)) << 24);
+            __builtin_nontemporal_store(r, y4 + j);
+        }
+    }
+    if (blockIdx.x == 0) {
+        const int64_t j = (n4 << 2) + threadIdx.x;
+        if (j < n) y[j] = sat_u8_rne(x[j] / s, z);
+    }
+}
+
+__global__ void __launch_bounds__(kThreads) dequantize_vec_kernel(const uint8_t *__restrict__ x, const float *__restrict__ scale,
+                                                                 const uint8_t *__restrict__ zp, float *__restrict__ y,
+                                                                 int64_t n) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    const float s = scale[0];
+    const int z = zp ? int(zp[0]) : 0;
+    const int64_t n4 = n >> 2;
+    const int64_t base = int64_t(blockIdx.x) * (kThreads * ZANT_STREAM_U) + threadIdx.x;
+    const uint32_t *x4 = reinterpret_cast<const uint32_t *>(x);
+    f4 *y4 = reinterpret_cast<f4 *>(y);
+    uint32_t v[ZANT_STREAM_U];
+#pragma unroll
+    for (int u = 0; u < ZANT_STREAM_U; ++u) {
+        const int64_t j = base + u * kThreads;
+        if (j < n4) v[u] = __builtin_nontemporal_load(x4 + j);
+    }
+#pragma unroll
+    for (int u = 0; u < ZANT_STREAM_U; ++u) {
+        const int64_t j = base + u * kThreads;
+        if (j < n4) {
+            f4 r;
+            r.x = float(int(v[u] & 255) - z) * s;
+            r.y = float(int((v[u] >> 8) & 255) - z) * s;
+            r.z = float(int((v[u] >> 16) & 255) - z) * s;
+            r.w = float(int(v[u] >> 24) - z) * s;
+            __builtin_nontemporal_store(r, y4 + j);
+        }
+    }
+    if (blockIdx.x == 0) {
+        const int64_t j = (n4 << 2) + threadIdx.x;
+        if (j < n) y[j] = float(int(x[j]) - z) * s;
+    }
+}
+
 __global__ void __launch_bounds__(kThreads) dequantize_kernel(const uint8_t *__restrict__ x, const float *__restrict__ scale,
                                                              const uint8_t *__restrict__ zp, float *__restrict__ y,
                                                              AxisGeom g) {
@@ -51,27 +117,43 @@ __global__ void __launch_bounds__(kThreads) qlinear_act_kernel(const uint8_t *__
     __shared__ uint8_t lut[256];
     lut[threadIdx.x] = uint8_t(qact_apply(uint8_t(threadIdx.x ^ flip), qa) ^ flip);
     __syncthreads();
-    const int64_t step = int64_t(gridDim.x) * blockDim.x;
-    const int64_t i0 = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
-    int64_t done = 0;
-    if (vec) {
-        const int64_t n16 = n >> 4;
-        const uint4 *x16 = reinterpret_cast<const uint4 *>(x);
-        uint4 *y16 = reinterpret_cast<uint4 *>(y);
-        for (int64_t i = i0; i < n16; i += step) {
-            uint4 v = x16[i];
-            uint32_t *w = reinterpret_cast<uint32_t *>(&v);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint32_t u = w[j];
-                w[j] = uint32_t(lut[u & 255]) | (uint32_t(lut[(u >> 8) & 255]) << 8) |
-                       (uint32_t(lut[(u >> 16) & 255]) << 16) | (uint32_t(lut[u >> 24]) << 24);
-            }
-            y16[i] = v;
+    typedef unsigned u4 __attribute__((ext_vector_type(4)));
+    if (!vec) {
+        const int64_t base = int64_t(blockIdx.x) * (kThreads * ZANT_STREAM_U * 16) + threadIdx.x;
+        for (int u = 0; u < ZANT_STREAM_U * 16; ++u) {
+            const int64_t j = base + u * kThreads;
+            if (j < n) y[j] = lut[x[j]];
         }
-        done = n16 << 4;
+        return;
     }
-    for (int64_t i = done + i0; i < n; i += step) y[i] = lut[x[i]];
+    const int64_t n16 = n >> 4;
+    const int64_t base = int64_t(blockIdx.x) * (kThreads * ZANT_STREAM_U) + threadIdx.x;
+    const u4 *x16 = reinterpret_cast<const u4 *>(x);
+    u4 *y16 = reinterpret_cast<u4 *>(y);
+    u4 v[ZANT_STREAM_U];
+#pragma unroll
+    for (int u = 0; u < ZANT_STREAM_U; ++u) {
+        const int64_t j = base + u * kThreads;
+        if (j < n16) v[u] = __builtin_nontemporal_load(x16 + j);
+    }
+#pragma unroll
+    for (int u = 0; u < ZANT_STREAM_U; ++u) {
+        const int64_t j = base + u * kThreads;
+        if (j < n16) {
+            u4 r;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t w = v[u][k];
+                r[k] = uint32_t(lut[w & 255]) | (uint32_t(lut[(w >> 8) & 255]) << 8) | (uint32_t(lut[(w >> 16) & 255]) << 16) |
+                       (uint32_t(lut[w >> 24]) << 24);
+            }
+            __builtin_nontemporal_store(r, y16 + j);
+        }
+    }
+    if (blockIdx.x == 0) {
+        const int64_t j = (n16 << 4) + threadIdx.x;
+        if (j < n) y[j] = lut[x[j]];
+    }
 }
 
 struct QAddArgs {
@@ -89,35 +171,47 @@ __device__ __forceinline__ uint8_t qadd_one(uint8_t a, uint8_t b, const QAddArgs
 __global__ void __launch_bounds__(kThreads) qlinear_add_kernel(const uint8_t *__restrict__ a, const uint8_t *__restrict__ b,
                                                               uint8_t *__restrict__ y, int64_t n, QAddArgs q, int vec,
                                                               uint32_t flip4) {
-    const int64_t step = int64_t(gridDim.x) * blockDim.x;
-    const int64_t i0 = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
-    int64_t done = 0;
-    if (vec) {
-        const int64_t n16 = n >> 4;
-        const uint4 *a16 = reinterpret_cast<const uint4 *>(a);
-        const uint4 *b16 = reinterpret_cast<const uint4 *>(b);
-        uint4 *y16 = reinterpret_cast<uint4 *>(y);
-        for (int64_t i = i0; i < n16; i += step) {
-            uint4 va = a16[i], vb = b16[i], vy;
-            va.x ^= flip4; va.y ^= flip4; va.z ^= flip4; va.w ^= flip4;
-            vb.x ^= flip4; vb.y ^= flip4; vb.z ^= flip4; vb.w ^= flip4;
-            const uint32_t *wa = reinterpret_cast<const uint32_t *>(&va);
-            const uint32_t *wb = reinterpret_cast<const uint32_t *>(&vb);
-            uint32_t *wy = reinterpret_cast<uint32_t *>(&vy);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                uint32_t r = 0;
-#pragma unroll
-                for (int k = 0; k < 4; ++k)
-                    r |= uint32_t(qadd_one(uint8_t(wa[j] >> (8 * k)), uint8_t(wb[j] >> (8 * k)), q)) << (8 * k);
-                wy[j] = r ^ flip4;
-            }
-            y16[i] = vy;
-        }
-        done = n16 << 4;
-    }
+    typedef unsigned u4 __attribute__((ext_vector_type(4)));
     const uint8_t f = uint8_t(flip4);
-    for (int64_t i = done + i0; i < n; i += step) y[i] = uint8_t(qadd_one(a[i] ^ f, b[i] ^ f, q) ^ f);
+    if (!vec) {
+        const int64_t base = int64_t(blockIdx.x) * (kThreads * ZANT_STREAM_U * 16) + threadIdx.x;
+        for (int u = 0; u < ZANT_STREAM_U * 16; ++u) {
+            const int64_t j = base + u * kThreads;
+            if (j < n) y[j] = uint8_t(qadd_one(a[j] ^ f, b[j] ^ f, q) ^ f);
+        }
+        return;
+    }
+    const int64_t n16 = n >> 4;
+    const int64_t base = int64_t(blockIdx.x) * (kThreads * ZANT_STREAM_U) + threadIdx.x;
+    const u4 *a16 = reinterpret_cast<const u4 *>(a);
+    const u4 *b16 = reinterpret_cast<const u4 *>(b);
+    u4 *y16 = reinterpret_cast<u4 *>(y);
+    u4 va[ZANT_STREAM_U], vb[ZANT_STREAM_U];
+#pragma unroll
+    for (int u = 0; u < ZANT_STREAM_U; ++u) {
+        const int64_t j = base + u * kThreads;
+        if (j < n16) { va[u] = __builtin_nontemporal_load(a16 + j); vb[u] = __builtin_nontemporal_load(b16 + j); }
+    }
+#pragma unroll
+    for (int u = 0; u < ZANT_STREAM_U; ++u) {
+        const int64_t j = base + u * kThreads;
+        if (j < n16) {
+            u4 r;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const uint32_t wa = va[u][w] ^ flip4, wb = vb[u][w] ^ flip4;
+                uint32_t o = 0;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) o |= uint32_t(qadd_one(uint8_t(wa >> (8 * k)), uint8_t(wb >> (8 * k)), q)) << (8 * k);
+                r[w] = o ^ flip4;
+            }
+            __builtin_nontemporal_store(r, y16 + j);
+        }
+    }
+    if (blockIdx.x == 0) {
+        const int64_t j = (n16 << 4) + threadIdx.x;
+        if (j < n) y[j] = uint8_t(qadd_one(a[j] ^ f, b[j] ^ f, q) ^ f);
+    }
 }
 
 // [N][CB][HW][16] signed -> NCHW u8.  One thread per (n, cb, 4 positions): four 16-byte loads, byte transpose,
@@ -266,6 +360,10 @@ extern "C" int zant_hip_quantize_linear_f32_u8(zant_ctx *ctx, const float *x, co
     if (g.n == 0) return ZANT_OK;
     if (!x || !y || !y_scale) return ZANT_NullPointer;
     KernelTimer kt(ctx);
+    if (!g.per_axis && ((reinterpret_cast<uintptr_t>(x) & 15) | (reinterpret_cast<uintptr_t>(y) & 3)) == 0)
+        hipLaunchKernelGGL(quantize_vec_kernel, dim3(zant_stream_grid((g.n + 3) >> 2)), dim3(kThreads), 0, ctx->stream, x, y_scale,
+                           y_zp, y, g.n);
+    else
     hipLaunchKernelGGL(quantize_kernel, dim3(grid_for(g.n, kThreads, ctx->num_cus)), dim3(kThreads), 0, ctx->stream, x,
                        y_scale, y_zp, y, g);
     ZANT_LAUNCH_CHECK(ctx);
@@ -282,6 +380,10 @@ extern "C" int zant_hip_dequantize_linear_u8_f32(zant_ctx *ctx, const uint8_t *x
     if (g.n == 0) return ZANT_OK;
     if (!x || !y || !x_scale) return ZANT_NullPointer;
     KernelTimer kt(ctx);
+    if (!g.per_axis && ((reinterpret_cast<uintptr_t>(y) & 15) | (reinterpret_cast<uintptr_t>(x) & 3)) == 0)
+        hipLaunchKernelGGL(dequantize_vec_kernel, dim3(zant_stream_grid((g.n + 3) >> 2)), dim3(kThreads), 0, ctx->stream, x,
+                           x_scale, x_zp, y, g.n);
+    else
     hipLaunchKernelGGL(dequantize_kernel, dim3(grid_for(g.n, kThreads, ctx->num_cus)), dim3(kThreads), 0, ctx->stream, x,
                        x_scale, x_zp, y, g);
     ZANT_LAUNCH_CHECK(ctx);
@@ -298,8 +400,8 @@ int zant_qlinear_act_flip(zant_ctx *ctx, const uint8_t *x, int64_t n, float x_sc
     qa.act = act; qa.alpha = alpha; qa.in_scale = x_scale; qa.in_zp = x_zp; qa.out_scale = y_scale; qa.out_zp = y_zp;
     const int vec = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
     KernelTimer kt(ctx);
-    hipLaunchKernelGGL(qlinear_act_kernel, dim3(grid_for(n, kThreads * 16, ctx->num_cus)), dim3(kThreads), 0, ctx->stream,
-                       x, y, n, qa, vec, flip & 0xff);
+    hipLaunchKernelGGL(qlinear_act_kernel, dim3(zant_stream_grid((n + 15) >> 4)), dim3(kThreads), 0, ctx->stream, x, y, n, qa,
+                       vec, flip & 0xff);
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
 }
@@ -318,8 +420,8 @@ int zant_qlinear_add_flip(zant_ctx *ctx, const uint8_t *a, float a_scale, uint8_
     q.a_scale = a_scale; q.b_scale = b_scale; q.y_scale = y_scale; q.a_zp = a_zp; q.b_zp = b_zp; q.y_zp = y_zp;
     const int vec = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
     KernelTimer kt(ctx);
-    hipLaunchKernelGGL(qlinear_add_kernel, dim3(grid_for(n, kThreads * 16, ctx->num_cus)), dim3(kThreads), 0, ctx->stream,
-                       a, b, y, n, q, vec, uint32_t(flip & 0xff) * 0x01010101u);
+    hipLaunchKernelGGL(qlinear_add_kernel, dim3(zant_stream_grid((n + 15) >> 4)), dim3(kThreads), 0, ctx->stream, a, b, y, n, q,
+                       vec, uint32_t(flip & 0xff) * 0x01010101u);
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
 }
