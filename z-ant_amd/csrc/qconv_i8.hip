@@ -569,18 +569,20 @@ qconv_smallc_pack_kernel(const int8_t *__restrict__ w, const float *__restrict__
     mult[k] = k < K ? (x_scale * w_scale[n_wscale == 1 ? 0 : k]) / y_scale : 0.0f;
 }
 
-template <int C>
+// S: stride when it is 1 or 2 (the input patch of a position -- or of a 2x2 pooling window -- then has a fixed size
+// and is fetched with independent, clamped, branch-free byte loads that all stay in flight together), 0 = any stride
+// (taps fetched one by one under their bounds checks).
+template <int C, int S, bool POOL>
 __global__ void __launch_bounds__(256)
 qconv_smallc_kernel(const uint8_t *__restrict__ x, const uint32_t *__restrict__ wpk, const float *__restrict__ mult,
-                    const int32_t *__restrict__ corr, uint8_t *__restrict__ y, ConvGeom g, QConvArgs q, int y_blocked,
-                    int pool) {
+                    const int32_t *__restrict__ corr, uint8_t *__restrict__ y, ConvGeom g, QConvArgs q, int y_blocked) {
     constexpr int NT = C * 9, ND = (NT + 3) / 4;
+    constexpr int NWIN = POOL ? 4 : 1;
     __shared__ uint8_t lut[256];  // the fused activation as a byte table (identity without one)
     lut[threadIdx.x] = q.has_act ? qact_apply(uint8_t(threadIdx.x), q.act) : uint8_t(threadIdx.x);
     __syncthreads();
-    const int OHo = pool ? g.OH / 2 : g.OH, OWo = pool ? g.OW / 2 : g.OW;
+    const int OHo = POOL ? g.OH / 2 : g.OH, OWo = POOL ? g.OW / 2 : g.OW;
     const int KB = (g.K + 15) >> 4;
-    const int n_win = pool ? 4 : 1;
     const uint32_t pad_byte = uint32_t(q.x_zp ^ 0x80);
     const int64_t total = int64_t(g.N) * OHo * OWo;
     const int64_t step = int64_t(gridDim.x) * blockDim.x;
@@ -588,13 +590,50 @@ qconv_smallc_kernel(const uint8_t *__restrict__ x, const uint32_t *__restrict__ 
         const int owo = int(i % OWo);
         const int oho = int((i / OWo) % OHo);
         const int n = int(i / (int64_t(OWo) * OHo));
-        uint32_t xs[4][ND];
+        uint32_t xs[NWIN][ND];
 #pragma unroll
-        for (int wd = 0; wd < 4; ++wd) {
-            if (wd < n_win) {
-                const int oh = pool ? 2 * oho + (wd >> 1) : oho, ow = pool ? 2 * owo + (wd & 1) : owo;
+        for (int wd = 0; wd < NWIN; ++wd)
 #pragma unroll
-                for (int d = 0; d < ND; ++d) xs[wd][d] = 0;
+            for (int d = 0; d < ND; ++d) xs[wd][d] = 0;
+        if constexpr (S > 0) {
+            constexpr int PR = (POOL ? S : 0) + 3;  // patch rows = columns
+            const int ih0 = (POOL ? 2 * oho : oho) * S - g.pt, iw0 = (POOL ? 2 * owo : owo) * S - g.pl;
+            int roff[PR], coff[PR];
+            bool rok[PR], cok[PR];
+#pragma unroll
+            for (int r = 0; r < PR; ++r) {
+                const int ih = ih0 + r, iw = iw0 + r;
+                rok[r] = ih >= 0 && ih < g.H;
+                cok[r] = iw >= 0 && iw < g.W;
+                roff[r] = min(max(ih, 0), g.H - 1) * g.W;
+                coff[r] = min(max(iw, 0), g.W - 1);
+            }
+            uint32_t patch[C][PR][PR];
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                const uint8_t *xc = x + (int64_t(n) * C + c) * g.H * g.W;
+#pragma unroll
+                for (int r = 0; r < PR; ++r)
+#pragma unroll
+                    for (int cc = 0; cc < PR; ++cc) patch[c][r][cc] = xc[roff[r] + coff[cc]];
+            }
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+#pragma unroll
+                for (int r = 0; r < PR; ++r)
+#pragma unroll
+                    for (int cc = 0; cc < PR; ++cc) patch[c][r][cc] = (rok[r] && cok[cc]) ? (patch[c][r][cc] ^ 0x80u) : pad_byte;
+#pragma unroll
+            for (int wd = 0; wd < NWIN; ++wd)
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    const int c = t / 9, kh = (t % 9) / 3, kw = t % 3;
+                    xs[wd][t >> 2] |= patch[c][(wd >> 1) * S + kh][(wd & 1) * S + kw] << (8 * (t & 3));
+                }
+        } else {
+#pragma unroll
+            for (int wd = 0; wd < NWIN; ++wd) {
+                const int oh = POOL ? 2 * oho + (wd >> 1) : oho, ow = POOL ? 2 * owo + (wd & 1) : owo;
 #pragma unroll
                 for (int t = 0; t < NT; ++t) {
                     const int c = t / 9, kh = (t % 9) / 3, kw = t % 3;
@@ -621,14 +660,12 @@ qconv_smallc_kernel(const uint8_t *__restrict__ x, const uint32_t *__restrict__ 
                 const bool neg = m < 0.0f;
                 int best = INT32_MIN;
 #pragma unroll
-                for (int wd = 0; wd < 4; ++wd) {
-                    if (wd < n_win) {
-                        int acc = cr;
+                for (int wd = 0; wd < NWIN; ++wd) {
+                    int acc = cr;
 #pragma unroll
-                        for (int d = 0; d < ND; ++d) acc = __builtin_amdgcn_sdot4(int(xs[wd][d]), int(wv[d]), acc, false);
-                        acc = neg ? -acc : acc;
-                        best = acc > best ? acc : best;
-                    }
+                    for (int d = 0; d < ND; ++d) acc = __builtin_amdgcn_sdot4(int(xs[wd][d]), int(wv[d]), acc, false);
+                    acc = neg ? -acc : acc;
+                    best = acc > best ? acc : best;
                 }
                 best = neg ? -best : best;
                 const uint8_t r = lut[sat_u8_rne(float(best) * m, q.y_zp)];
@@ -674,8 +711,12 @@ int launch_smallc(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float 
     const int64_t positions = int64_t(g.N) * (pool ? g.OH / 2 : g.OH) * (pool ? g.OW / 2 : g.OW);
     const unsigned blocks = unsigned(std::min<int64_t>(std::max<int64_t>(ceil_div64(positions, 256), 1), int64_t(ctx->num_cus) * 32));
     KernelTimer kt(ctx);
-    hipLaunchKernelGGL(qconv_smallc_kernel<C>, dim3(blocks), dim3(256), 0, ctx->stream, x, wpk, mult, corr, y, g, q,
-                       y_blocked ? 1 : 0, pool ? 1 : 0);
+    const int yb = y_blocked ? 1 : 0;
+    const int S = (g.sh == g.sw && (g.sh == 1 || g.sh == 2)) ? g.sh : 0;
+#define ZANT_SMALLC(SV, PV) hipLaunchKernelGGL((qconv_smallc_kernel<C, SV, PV>), dim3(blocks), dim3(256), 0, ctx->stream, x, wpk, mult, corr, y, g, q, yb)
+    if (pool) { if (S == 1) ZANT_SMALLC(1, true); else if (S == 2) ZANT_SMALLC(2, true); else ZANT_SMALLC(0, true); }
+    else { if (S == 1) ZANT_SMALLC(1, false); else if (S == 2) ZANT_SMALLC(2, false); else ZANT_SMALLC(0, false); }
+#undef ZANT_SMALLC
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
 }
