@@ -164,6 +164,13 @@ def main():
         fl = 2 * 256 * 64 * 56 * 56 * 64 * 9
         operators["conv_f32_N256_C64_56x56_K64_3x3"] = {"ms": round(ms, 4), "tflops": round(fl / ms / 1e9, 2),
                                                         "frac_f32_mfma_peak": round(fl / ms / 1e9 / PEAK_F32_MFMA_TFLOPS, 4)}
+        if not args.no_cpu_baseline:  # the oracle on one core over a slice of the same operator (2 of the 256 images)
+            xs, wsl, bs = xa[:2].cpu().numpy(), wa.cpu().numpy(), ba.cpu().numpy()
+            t0 = time.perf_counter()
+            zo.Conv(xs, wsl, bs, [1, 1], [1, 1, 1, 1], [1, 1], 1, "NOTSET")
+            dt = time.perf_counter() - t0
+            operators["conv_f32_N256_C64_56x56_K64_3x3"]["cpu_oracle_1core"] = {
+                "gflops": round(fl * 2 / 256 / dt / 1e9, 2), "sample": f"2 of 256 images, {dt:.1f} s"}
         del xa, ya
         ga = torch.randn(1, 1, 4096, 1600, device=dev)
         gb = torch.randn(1, 1, 1600, 512, device=dev) * (2.0 / 1600) ** 0.5
@@ -174,6 +181,13 @@ def main():
         fl = 2 * 4096 * 1600 * 512
         operators["gemm_f32_4096x1600x512"] = {"ms": round(ms, 4), "tflops": round(fl / ms / 1e9, 2),
                                                "frac_f32_mfma_peak": round(fl / ms / 1e9 / PEAK_F32_MFMA_TFLOPS, 4)}
+        if not args.no_cpu_baseline:
+            gas = ga[:, :, :256].cpu().numpy()
+            t0 = time.perf_counter()
+            zo.gemm(gas, gb.cpu().numpy(), gc.cpu().numpy(), 1.0, 1.0, False, False)
+            dt = time.perf_counter() - t0
+            operators["gemm_f32_4096x1600x512"]["cpu_oracle_1core"] = {
+                "gflops": round(fl * 256 / 4096 / dt / 1e9, 2), "sample": f"256 of 4096 rows, {dt:.1f} s"}
         xq = torch.randint(0, 256, (128, 128, 28, 28), dtype=torch.uint8, device=dev)
         wq = torch.randint(-127, 128, (128, 128, 3, 3), dtype=torch.int8, device=dev)
         ws = torch.rand(128, device=dev) * 0.009 + 0.001
@@ -184,6 +198,13 @@ def main():
         op = 2 * 128 * 128 * 28 * 28 * 128 * 9
         operators["qlinearconv_u8i8_N128_C128_28x28_K128_3x3"] = {"ms": round(ms, 4), "tops": round(op / ms / 1e9, 2),
                                                                   "frac_i8_mfma_peak": round(op / ms / 1e9 / PEAK_I8_MFMA_TOPS, 5)}
+        if not args.no_cpu_baseline:
+            t0 = time.perf_counter()
+            zo.qlinearconv(xq[:2].cpu().numpy(), 0.02, 128, wq.cpu().numpy(), ws.cpu().numpy(), None, 0.05, 128,
+                           bq.cpu().numpy(), [1, 1], [1, 1, 1, 1], [1, 1])
+            dt = time.perf_counter() - t0
+            operators["qlinearconv_u8i8_N128_C128_28x28_K128_3x3"]["cpu_oracle_1core"] = {
+                "gops": round(op * 2 / 128 / dt / 1e9, 2), "sample": f"2 of 128 images, {dt:.1f} s"}
 
     # ---- int8 networks (configs 4 and 5): whole-network throughput with the calibrated scales of the golden fixture ----
     nets_out = None

@@ -37,7 +37,7 @@ __device__ __forceinline__ uint8_t requant(int acc, float m, const QConvArgs &q)
 // The same with the fused activation taken from a 256-entry byte table (identity without one): the activation is a
 // function of one byte, and evaluating its f32 sequence (an IEEE divide among it) per output costs more than the MFMAs.
 __device__ __forceinline__ uint8_t requant_lut(int acc, float m, const QConvArgs &q, const uint8_t *lut) {
-    return lut[sat_u8_rne(float(acc) * m, q.y_zp)];
+    return lut[sat_u8_rne_finite(float(acc) * m, float(q.y_zp))];
 }
 
 // One thread per output element; any stride / dilation / pads / group.
@@ -668,7 +668,7 @@ qconv_smallc_kernel(const uint8_t *__restrict__ x, const uint32_t *__restrict__ 
                     best = acc > best ? acc : best;
                 }
                 best = neg ? -best : best;
-                const uint8_t r = lut[sat_u8_rne(float(best) * m, q.y_zp)];
+                const uint8_t r = lut[sat_u8_rne_finite(float(best) * m, float(q.y_zp))];
                 out[j >> 2] |= uint32_t(r) << (8 * (j & 3));
             }
             if (y_blocked) {
@@ -792,7 +792,7 @@ qdw3x3_blocked_kernel(const uint4 *__restrict__ x, const uint32_t *__restrict__ 
             uint32_t o = 0;
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                o |= uint32_t(lut[sat_u8_rne(float(acc[j]) * mult[cb * 16 + qd * 4 + j], q.y_zp)]) << (8 * j);
+                o |= uint32_t(lut[sat_u8_rne_finite(float(acc[j]) * mult[cb * 16 + qd * 4 + j], float(q.y_zp))]) << (8 * j);
             out[qd] = o;
         }
         y[((n * CB + cb) * g.OH + oh) * int64_t(g.OW) + ow] = make_uint4(out[0], out[1], out[2], out[3]);

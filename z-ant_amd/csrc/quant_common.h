@@ -11,6 +11,13 @@ __device__ __forceinline__ uint8_t sat_u8_rne(float v, uint8_t zp) {
     return uint8_t(r);
 }
 
+// The same for finite inputs (an int32 accumulator times a finite multiplier), as a byte in the low bits of a dword:
+// v_cvt_pk_u8_f32 converts with saturation to [0, 255], which replaces the clamp and the conversion.  The value is
+// already integral after rint + zero point, so the conversion's own rounding never acts.
+__device__ __forceinline__ uint32_t sat_u8_rne_finite(float v, float zp_f) {
+    return __builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(v) + zp_f, 0u, 0u);
+}
+
 struct QAct {
     int act;            // zant_act
     float alpha;        // LeakyReLU slope
