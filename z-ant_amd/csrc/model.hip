@@ -730,6 +730,23 @@ extern "C" int zant_model_finalize(zant_model *m) {
     int rc = zant_hip_arena_reserve(ctx, arena);
     if (rc) return rc;
 
+    // ---- wide Gemm weights are kept k-contiguous ([N][K], i.e. transB): both operands of the matrix-core kernel are then
+    // staged with 16-byte copies, half as many copy instructions per chunk as with a row-major B ---------------------
+    for (MNode &nd : m->n) {
+        if (nd.skip || nd.op != OP_GEMM || nd.trans_b || nd.wdim[0] != 1 || nd.wdim[1] != 1 || nd.wdim[3] <= 32) continue;
+        const int64_t K = nd.wdim[2], N = nd.wdim[3];
+        if (K % 4) continue;  // 16-byte copies need k-rows of a multiple of 4 floats
+        std::vector<char> &h = m->p[nd.w].host;
+        std::vector<char> tr(h.size());
+        const float *src = reinterpret_cast<const float *>(h.data());
+        float *dst = reinterpret_cast<float *>(tr.data());
+        for (int64_t k = 0; k < K; ++k)
+            for (int64_t n = 0; n < N; ++n) dst[n * K + k] = src[k * N + n];
+        h.swap(tr);
+        nd.wdim[2] = N; nd.wdim[3] = K;
+        nd.trans_b = 1;
+    }
+
     // ---- parameters: one allocation, one upload each ---------------------------------------------
     size_t pbytes = 0;
     for (Param &p : m->p) { p.offset = pbytes; pbytes += (p.host.size() + 255) & ~size_t(255); }
