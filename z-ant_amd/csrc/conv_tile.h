@@ -24,6 +24,7 @@ struct TilePlan {
     TileGeom t;
     size_t lds_bytes;
     double eff;          // useful fraction of the MFMA columns
+    double score;        // eff weighted by how much of the GPU the tiles fill (what plans are ranked by)
 };
 
 // Tile id -> first image, first output row, output-channel block.  XCD-aware: consecutive
@@ -44,8 +45,10 @@ __device__ __forceinline__ void decode_tile(const TileGeom &t, int tile, int &n0
 // pool: the kernel's epilogue max-pools 2x2/2 (floor).  The MFMA column slots are then counted in POOLED positions:
 // tile registers 4j..4j+3 of a lane hold the four members of one window, so MT is a multiple of 4, TH is even and
 // a tile covers NB images x TH/2 pooled rows x OW/2 pooled columns.
+// target_tiles > 0: plans are ranked by eff * min(1, n_tiles / target_tiles) -- a layer too small to give every
+// workgroup slot of the GPU a tile is better off with smaller tiles than with fuller ones.
 inline bool zant_plan_conv_tiles(const ConvGeom &g, int WM, int WN, int mt_max, int chunk_channels, size_t elem_bytes,
-                                 size_t lds_cap, TilePlan *best, bool pool = false) {
+                                 size_t lds_cap, TilePlan *best, bool pool = false, int target_tiles = 0) {
     const int T = g.KH * g.KW;
     const int K_BLK = WN * 32;
     bool found = false;
@@ -84,8 +87,11 @@ inline bool zant_plan_conv_tiles(const ConvGeom &g, int WM, int WN, int mt_max, 
                            + size_t(t.P1s) * 8 + 8;                          // patch table, scheduler slots
         if (lds > lds_cap) continue;
         const double eff = double(g.N) * rows * cols / (double(t.n_sblocks) * S);
-        if (!found || eff > best->eff + 0.01) {  // larger tiles win ties: fewer tiles, more operand reuse
+        double score = eff;
+        if (target_tiles > 0 && t.n_tiles < target_tiles) score *= double(t.n_tiles) / target_tiles;
+        if (!found || score > best->score + 0.01) {  // larger tiles win ties: fewer tiles, more operand reuse
             best->MT = mt; best->WM = WM; best->WN = WN; best->t = t; best->lds_bytes = lds; best->eff = eff;
+            best->score = score;
             found = true;
         }
     }

@@ -172,6 +172,83 @@ qpack_kernel(const int8_t *__restrict__ w, const float *__restrict__ w_scale, co
     }
 }
 
+// Bytes of the weight region of a staging buffer: the slab rounded up to one 16-byte unit per thread and round.
+__device__ __host__ __forceinline__ int w_region_bytes(int w_chunk, int nt) { return ((w_chunk / 16 + nt - 1) / nt) * nt * 16; }
+
+// The asynchronous copies of one (tile, chunk) step into the staging buffer `dma`.  Every thread issues the same
+// number of copies whatever the geometry (lanes past the end of the slab repeat its last unit, patch slots past P1
+// -- the patch region is padded to a multiple of the workgroup size -- copy the padding vector), so the number of
+// copies a wave has in flight per step is a constant the ring's waits can count with.
+template <int WM, int WN, int TT>
+__device__ __forceinline__ void qconv_issue(char *__restrict__ dma, const int2 *__restrict__ ptab,
+                                            const int8_t *__restrict__ xb, const int8_t *__restrict__ wp,
+                                            const int8_t *__restrict__ padvec, const ConvGeom &g, const TileGeom &t, int CB,
+                                            int itile, int ichunk) {
+    constexpr int NT = WM * WN * 64;
+    constexpr int K_BLK = WN * 32;
+    const int T = TT > 0 ? TT : g.KH * g.KW;
+    const int w_chunk = T * QCC * K_BLK;  // bytes
+    const int tid = threadIdx.x, wave = tid >> 6;
+    int n0, oh0, kb;
+    decode_tile(t, itile, n0, oh0, kb);
+    char *xl = dma + w_region_bytes(w_chunk, NT);
+    const int8_t *wsrc = wp + (int64_t(ichunk) * t.n_kblocks + kb) * w_chunk;
+    const int units = w_chunk >> 4;
+    for (int u0 = 0; u0 < units; u0 += NT) {
+        const int u = min(u0 + tid, units - 1);
+        __builtin_amdgcn_global_load_lds((gptr_t)(wsrc + u * 16), (lptr_t)(dma + (u0 + wave * 64) * 16), 16, 0, 0);
+    }
+    const int64_t plane = int64_t(g.H) * g.W;
+    const int8_t *xg = xb + int64_t(n0) * CB * plane * 16;
+    const int ih0 = oh0 * g.sh - g.pt;
+    const int imgs_here = min(t.NB, g.N - n0);
+    for (int p0 = 0; p0 < t.P1s; p0 += NT) {
+        const int2 e = ptab[p0 + tid];  // entries past P1 say "padding"
+        const int ih = ih0 + (e.y & 0xffff);
+        const bool ok = e.x >= 0 && ih >= 0 && ih < g.H && (e.y >> 16) < imgs_here;
+        const int8_t *src = xg + (int64_t(e.x + ih0 * g.W) + int64_t(ichunk * 2) * plane) * 16;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const int8_t *sp = (ok && ichunk * 2 + half < CB) ? src + half * plane * 16 : padvec;
+            __builtin_amdgcn_global_load_lds((gptr_t)sp, (lptr_t)(xl + (half * t.P1s + p0 + wave * 64) * 16), 16, 0, 0);
+        }
+    }
+}
+
+// LDS reads the compiler does not see (it would drain every outstanding asynchronous copy before an LDS read of its
+// own that it cannot prove independent of them).  The *_wait functions take the values as in/out operands so that their
+// users stay behind the wait; nothing read this way is kept in flight across a loop edge.
+__device__ __forceinline__ unsigned lds_addr_of(const void *p) {
+    return unsigned(reinterpret_cast<uintptr_t>((lptr_t) const_cast<void *>(p)));
+}
+__device__ __forceinline__ uint32_t lds_read_u8_async(unsigned addr) {
+    uint32_t v;
+    asm volatile("ds_read_u8 %0, %1" : "=v"(v) : "v"(addr));
+    return v;
+}
+__device__ __forceinline__ uint32_t lds_read_b32_async(unsigned addr) {
+    uint32_t v;
+    asm volatile("ds_read_b32 %0, %1" : "=v"(v) : "v"(addr));
+    return v;
+}
+__device__ __forceinline__ void lds_wait16(uint32_t (&v)[16]) {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]), "+v"(v[8]),
+                   "+v"(v[9]), "+v"(v[10]), "+v"(v[11]), "+v"(v[12]), "+v"(v[13]), "+v"(v[14]), "+v"(v[15]));
+}
+
+// Waits until at most n of this wave's vector-memory operations are outstanding (n is wave-uniform, 0..63).
+__device__ __forceinline__ void wait_vmcnt(int n) {
+#define ZANT_VM(k) case k: __builtin_amdgcn_s_waitcnt(((k) & 15) | (((k) >> 4) << 14) | 0x0F70); break;
+#define ZANT_VM8(b) ZANT_VM(b) ZANT_VM(b + 1) ZANT_VM(b + 2) ZANT_VM(b + 3) ZANT_VM(b + 4) ZANT_VM(b + 5) ZANT_VM(b + 6) ZANT_VM(b + 7)
+    switch (n) {
+        ZANT_VM8(0) ZANT_VM8(8) ZANT_VM8(16) ZANT_VM8(24) ZANT_VM8(32) ZANT_VM8(40) ZANT_VM8(48) ZANT_VM8(56)
+    default: __builtin_amdgcn_s_waitcnt(0x0F70); break;
+    }
+#undef ZANT_VM8
+#undef ZANT_VM
+}
+
 // One (tile, chunk) step: start the global->LDS copies of the next step into `dma`, run the int8
 // matrix cores over this step's operands in `cmp`.  The LDS regions never overlap within a step and
 // are __restrict__ so that the copies stay in flight across this step's LDS reads.
@@ -189,40 +266,11 @@ __device__ __forceinline__ void qconv_step(char *__restrict__ dma, const char *_
     const int wn = wave / WM;
     const int l32 = lane & 31, lh = lane >> 5;
 
-    if (do_issue) {
-        int n0, oh0, kb;
-        decode_tile(t, itile, n0, oh0, kb);
-        char *xl = dma + w_chunk;
-        const int8_t *wsrc = wp + (int64_t(ichunk) * t.n_kblocks + kb) * w_chunk;
-        const int units = w_chunk >> 4;
-        for (int u0 = 0; u0 < units; u0 += NT) {
-            const int u = u0 + tid;
-            if (u < units)
-                __builtin_amdgcn_global_load_lds((gptr_t)(wsrc + u * 16), (lptr_t)(dma + (u0 + wave * 64) * 16), 16, 0, 0);
-        }
-        const int64_t plane = int64_t(g.H) * g.W;
-        const int8_t *xg = xb + int64_t(n0) * CB * plane * 16;
-        const int ih0 = oh0 * g.sh - g.pt;
-        const int imgs_here = min(t.NB, g.N - n0);
-        for (int p0 = 0; p0 < t.P1; p0 += NT) {
-            const int pos = p0 + tid;
-            if (pos < t.P1) {
-                const int2 e = ptab[pos];
-                const int ih = ih0 + (e.y & 0xffff);
-                const bool ok = e.x >= 0 && ih >= 0 && ih < g.H && (e.y >> 16) < imgs_here;
-                const int8_t *src = xg + (int64_t(e.x + ih0 * g.W) + int64_t(ichunk * 2) * plane) * 16;
-#pragma unroll
-                for (int half = 0; half < 2; ++half) {
-                    const int8_t *sp = (ok && ichunk * 2 + half < CB) ? src + half * plane * 16 : padvec;
-                    __builtin_amdgcn_global_load_lds((gptr_t)sp, (lptr_t)(xl + (half * t.P1s + p0 + wave * 64) * 16), 16, 0, 0);
-                }
-            }
-        }
-    }
+    if (do_issue) qconv_issue<WM, WN, TT>(dma, ptab, xb, wp, padvec, g, t, CB, itile, ichunk);
     __builtin_amdgcn_sched_barrier(0);
 
     const char *wl = cmp + (lh * K_BLK + wn * 32 + l32) * 16;
-    const char *xl = cmp + w_chunk + lh * t.P1s * 16;
+    const char *xl = cmp + w_region_bytes(w_chunk, NT) + lh * t.P1s * 16;
     i32x4 a0, a1, b0[MT], b1[MT];
     int lkh = 0, lkw = 0, ltap = 0;
     auto load_tap = [&](i32x4 &a, i32x4 (&b)[MT]) {
@@ -264,37 +312,42 @@ __device__ __forceinline__ void qconv_step(char *__restrict__ dma, const char *_
     }
 }
 
-// Persistent int8 implicit-GEMM convolution over the channel-blocked input.
+// Persistent int8 implicit-GEMM convolution over the channel-blocked input.  A workgroup walks its tiles
+// (blockIdx.x, blockIdx.x + gridDim.x, ...) chunk by chunk; the (tile, chunk) steps form one sequence whose operand
+// copies run n_stages - 1 steps ahead of the matrix cores through a ring of n_stages LDS buffers, so that a step's
+// copy latency is hidden even when the step itself is only a few MFMAs (1x1 layers, small feature maps).
 template <int MT, int WM, int WN, int TT>
 __global__ void __launch_bounds__(WM *WN * 64, 2)
 qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, const float *__restrict__ mult,
                   const int32_t *__restrict__ corr, const int8_t *__restrict__ padvec, uint8_t *__restrict__ y, ConvGeom g,
-                  TileGeom t, int CB, QConvArgs q, int *__restrict__ tile_counters, int parity, int y_blocked) {
+                  TileGeom t, int CB, QConvArgs q, int n_stages, int y_blocked) {
     constexpr int NT = WM * WN * 64;
     constexpr int K_BLK = WN * 32;
     extern __shared__ __attribute__((aligned(16))) char qlds[];
     const int T = TT > 0 ? TT : g.KH * g.KW;
-    const int w_chunk = T * QCC * K_BLK;          // bytes per (chunk, kblock) weight slab
-    const int buf_bytes = w_chunk + QCC * t.P1s;  // one staging buffer
-    char *buf0 = qlds, *buf1 = qlds + buf_bytes;
-    int2 *ptab = reinterpret_cast<int2 *>(qlds + 2 * buf_bytes);
-    int *sched = reinterpret_cast<int *>(ptab + t.P1s);
-    uint8_t *lut = reinterpret_cast<uint8_t *>(sched + 2);  // [256] fused activation table
+    const int w_chunk = T * QCC * K_BLK;                           // bytes per (chunk, kblock) weight slab
+    const int buf_bytes = w_region_bytes(w_chunk, NT) + QCC * t.P1s;  // one staging buffer (P1s: multiple of NT)
+    int2 *ptab = reinterpret_cast<int2 *>(qlds + n_stages * buf_bytes);
+    uint8_t *lut = reinterpret_cast<uint8_t *>(ptab + t.P1s);  // [256] fused activation table
+    const int kpad = t.n_kblocks * K_BLK;
+    float *mult_l = reinterpret_cast<float *>(lut + 256);       // [kpad] requantisation multipliers ...
+    int *corr_l = reinterpret_cast<int *>(mult_l + kpad);       // [kpad] ... and integer corrections, copied once
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave % WM, wn = wave / WM;
     const int l32 = lane & 31, lh = lane >> 5;
     const int64_t plane_in = int64_t(g.H) * g.W;
-    lut[tid & 255] = q.has_act ? qact_apply(uint8_t(tid & 255), q.act) : uint8_t(tid & 255);  // NT == 256
     const int per_img = t.TH * g.OW;
     const int patch_hw = t.PH * t.PW;
+    lut[tid & 255] = q.has_act ? qact_apply(uint8_t(tid & 255), q.act) : uint8_t(tid & 255);  // NT == 256
+    for (int k = tid; k < kpad; k += NT) { mult_l[k] = mult[k]; corr_l[k] = corr[k]; }
 
-    for (int e = tid; e < t.P1; e += NT) {
+    for (int e = tid; e < t.P1s; e += NT) {
         const int img = e / patch_hw, rem = e - img * patch_hw;
         const int ph = rem / t.PW, pw = rem - ph * t.PW;
         const int iw = pw - g.pl;
         int2 v;
-        v.x = (iw >= 0 && iw < g.W) ? int(img * CB * plane_in) + ph * g.W + iw : -1;
+        v.x = (e < t.P1 && iw >= 0 && iw < g.W) ? int(img * CB * plane_in) + ph * g.W + iw : -1;
         v.y = (img << 16) | ph;
         ptab[e] = v;
     }
@@ -306,67 +359,43 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
         const int r = rem / g.OW, c = rem - r * g.OW;
         lds_off[i] = (img < t.NB && r < t.TH) ? (img * t.PH + r * g.sh) * t.PW + c * g.sw : 0;
     }
-    if (tid == 0) sched[0] = blockIdx.x + gridDim.x;
-    // this launch draws tiles from tile_counters[parity] and re-arms the other counter for the operator's next launch
-    if (tid == 0 && blockIdx.x == 0) tile_counters[parity ^ 1] = 2 * int(gridDim.x);
     __syncthreads();
 
-    int cur = blockIdx.x;
-    if (cur >= t.n_tiles) return;
+    if (int(blockIdx.x) >= t.n_tiles) return;
+    const int my_tiles = (t.n_tiles - int(blockIdx.x) + int(gridDim.x) - 1) / int(gridDim.x);
+    const int n_steps = my_tiles * t.n_chunks;
+    // copies per thread and step (see qconv_issue)
+    const int P = w_region_bytes(w_chunk, NT) / (16 * NT) + 2 * (t.P1s / NT);
     i32x16 acc[MT];
-    // prologue: the first step's copies go through the same code path with nothing to compute
-    // (an all-zero pass over whatever the LDS holds into accumulators that are reset right after).
-    {
-        // issue only: replicate the copy part of qconv_step for (cur, chunk 0) into buf0
-        int n0, oh0, kb;
-        decode_tile(t, cur, n0, oh0, kb);
-        const int8_t *wsrc = wp + int64_t(kb) * w_chunk;
-        const int units = w_chunk >> 4;
-        for (int u0 = 0; u0 < units; u0 += NT) {
-            const int u = u0 + tid;
-            if (u < units)
-                __builtin_amdgcn_global_load_lds((gptr_t)(wsrc + u * 16), (lptr_t)(buf0 + (u0 + wave * 64) * 16), 16, 0, 0);
-        }
-        const int8_t *xg = xb + int64_t(n0) * CB * plane_in * 16;
-        const int ih0 = oh0 * g.sh - g.pt;
-        const int imgs_here = min(t.NB, g.N - n0);
-        char *xl = buf0 + w_chunk;
-        for (int p0 = 0; p0 < t.P1; p0 += NT) {
-            const int pos = p0 + tid;
-            if (pos < t.P1) {
-                const int2 e = ptab[pos];
-                const int ih = ih0 + (e.y & 0xffff);
-                const bool ok = e.x >= 0 && ih >= 0 && ih < g.H && (e.y >> 16) < imgs_here;
-                const int8_t *src = xg + int64_t(e.x + ih0 * g.W) * 16;
+    // prologue: the first n_stages - 1 steps' copies
+    for (int s0 = 0; s0 < n_stages - 1 && s0 < n_steps; ++s0)
+        qconv_issue<WM, WN, TT>(qlds + s0 * buf_bytes, ptab, xb, wp, padvec, g, t, CB,
+                                int(blockIdx.x) + (s0 / t.n_chunks) * int(gridDim.x), s0 % t.n_chunks);
+    int cbuf = 0, dbuf = n_stages - 1;    // ring slots of the step being multiplied / of the step being copied
+    int itile = int(blockIdx.x), ichunk = 0;  // (tile, chunk) of the step whose copies are issued next
+    for (int s0 = 0; s0 < n_stages - 1; ++s0)
+        if (++ichunk == t.n_chunks) { ichunk = 0; itile += int(gridDim.x); }
+    int cur = int(blockIdx.x), chunk = 0;
+    for (int s0 = 0; s0 < n_steps; ++s0) {
+        if (chunk == 0) {
 #pragma unroll
-                for (int half = 0; half < 2; ++half) {
-                    const int8_t *sp = (ok && half < CB) ? src + half * plane_in * 16 : padvec;
-                    __builtin_amdgcn_global_load_lds((gptr_t)sp, (lptr_t)(xl + (half * t.P1s + p0 + wave * 64) * 16), 16, 0, 0);
-                }
-            }
-        }
-    }
-    int step = 0, tile_par = 0;
-    while (cur < t.n_tiles) {
+            for (int i = 0; i < MT; ++i)
 #pragma unroll
-        for (int i = 0; i < MT; ++i)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][v] = 0;
-        int nxt = t.n_tiles;
-        for (int chunk = 0; chunk < t.n_chunks; ++chunk, ++step) {
-            __builtin_amdgcn_s_waitcnt(0);
-            __syncthreads();
-            if (chunk == 0) {
-                nxt = sched[tile_par];
-                if (tid == 0) sched[tile_par ^ 1] = atomicAdd(tile_counters + parity, 1);
-            }
-            const bool same_tile = chunk + 1 < t.n_chunks;
-            const bool do_issue = same_tile || nxt < t.n_tiles;
-            const int itile = same_tile ? cur : nxt, ichunk = same_tile ? chunk + 1 : 0;
-            char *dma = (step & 1) ? buf0 : buf1;
-            const char *cmp = (step & 1) ? buf1 : buf0;
-            qconv_step<MT, WM, WN, TT>(dma, cmp, ptab, xb, wp, padvec, g, t, CB, do_issue, itile, ichunk, lds_off, acc);
+                for (int v = 0; v < 16; ++v) acc[i][v] = 0;
         }
+        // This wave's copies of step s0 have landed once no more than the copies of the later steps are outstanding
+        // (loads complete in order); after the barrier everybody's have, and everybody is done with step s0 - 1,
+        // whose ring slot is refilled now.  A bare s_barrier: __syncthreads() would drain every outstanding copy.
+        wait_vmcnt(P * min(n_stages - 2, n_steps - 1 - s0));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        qconv_step<MT, WM, WN, TT>(qlds + dbuf * buf_bytes, qlds + cbuf * buf_bytes, ptab, xb, wp, padvec, g, t, CB,
+                                   s0 + n_stages - 1 < n_steps, itile, ichunk, lds_off, acc);
+        if (++ichunk == t.n_chunks) { ichunk = 0; itile += int(gridDim.x); }
+        cbuf = cbuf + 1 == n_stages ? 0 : cbuf + 1;
+        dbuf = dbuf + 1 == n_stages ? 0 : dbuf + 1;
+        if (++chunk < t.n_chunks) continue;
+        chunk = 0;
 
         // ---- epilogue: integer correction, requantisation (+ fused activation), NCHW u8 stores ----
         {
@@ -376,35 +405,44 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
             const int imgs_here = min(t.NB, g.N - n0);
             const int64_t plane = int64_t(g.OH) * g.OW;
             const int kbase = kb * K_BLK + wn * 32 + lh * 4;
-            float mv[16];
-            int cv[16];
+            // multipliers and corrections of this lane's 16 channels, then per tile the 16 activation-table lookups,
+            // all through hand-issued LDS reads: the next steps' copies stay in flight behind the epilogue
+            uint32_t mraw[16], craw[16];
+            const unsigned lut_a = lds_addr_of(lut), mult_a = lds_addr_of(mult_l), corr_a = lds_addr_of(corr_l);
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int k = kbase + (v >> 2) * 8 + (v & 3);  // < n_kblocks * K_BLK: the tables are padded
-                mv[v] = mult[k];
-                cv[v] = corr[k];
+                mraw[v] = lds_read_b32_async(mult_a + unsigned(k) * 4u);
+                craw[v] = lds_read_b32_async(corr_a + unsigned(k) * 4u);
             }
-            if (y_blocked) {
-                // [N][KB][OH][OW][16] signed.  A lane holds 4 groups of 4 consecutive channels; lanes l and l+32 swap
-                // one dword per 16-channel block so that each stores 8 consecutive bytes: a half-wave then writes
-                // 32 positions x 16 bytes without gaps.
-                const int KB = (g.K + 15) >> 4;
-                const int cb0 = (kb * K_BLK + wn * 32) >> 4;
+            lds_wait16(mraw);
+            lds_wait16(craw);
+            float mv[16];
+            int cv[16];
 #pragma unroll
-                for (int i = 0; i < MT; ++i) {
-                    const int p = (wm * MT + i) * 32 + l32;
-                    const int img = p / per_img, rem = p - img * per_img;
-                    const int r = rem / g.OW, c = rem - r * g.OW;
+            for (int v = 0; v < 16; ++v) { mv[v] = __uint_as_float(mraw[v]); cv[v] = int(craw[v]); }
+            const float zpf = float(q.y_zp);
+            const int KB = (g.K + 15) >> 4;
+            const int cb0 = (kb * K_BLK + wn * 32) >> 4;
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+                const int p = (wm * MT + i) * 32 + l32;
+                const int img = p / per_img, rem = p - img * per_img;
+                const int r = rem / g.OW, c = rem - r * g.OW;
+                const bool ok = img < imgs_here && r < rows_here;
+                uint32_t ob[16];  // the 16 output bytes of this position
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    ob[v] = lds_read_u8_async(lut_a + sat_u8_rne_finite(float(acc[i][v] + cv[v]) * mv[v], zpf));
+                lds_wait16(ob);
+                if (y_blocked) {
+                    // [N][KB][OH][OW][16] signed.  A lane holds 4 groups of 4 consecutive channels; lanes l and l+32
+                    // swap one dword per 16-channel block so that each stores 8 consecutive bytes: a half-wave then
+                    // writes 32 positions x 16 bytes without gaps.
                     uint32_t d[4];
 #pragma unroll
-                    for (int gq = 0; gq < 4; ++gq) {
-                        uint32_t w4 = 0;
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            w4 |= uint32_t(requant_lut(acc[i][gq * 4 + e] + cv[gq * 4 + e], mv[gq * 4 + e], q, lut)) << (8 * e);
-                        d[gq] = w4 ^ 0x80808080u;
-                    }
-                    const bool ok = img < imgs_here && r < rows_here;
+                    for (int gq = 0; gq < 4; ++gq)
+                        d[gq] = (ob[gq * 4] | (ob[gq * 4 + 1] << 8) | (ob[gq * 4 + 2] << 16) | (ob[gq * 4 + 3] << 24)) ^ 0x80808080u;
 #pragma unroll
                     for (int b = 0; b < 2; ++b) {
                         const uint32_t send = lh ? d[2 * b] : d[2 * b + 1];
@@ -415,64 +453,55 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
                             *reinterpret_cast<uint2 *>(yp) = out;
                         }
                     }
-                }
-            } else
-#pragma unroll
-            for (int i = 0; i < MT; ++i) {
-                const int p = (wm * MT + i) * 32 + l32;
-                const int img = p / per_img, rem = p - img * per_img;
-                const int r = rem / g.OW, c = rem - r * g.OW;
-                if (img < imgs_here && r < rows_here) {
+                } else if (ok) {
                     uint8_t *yp = y + (int64_t(n0 + img) * g.K + kbase) * plane + int64_t(oh0 + r) * g.OW + c;
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
                         const int dk = (v >> 2) * 8 + (v & 3);
-                        if (kbase + dk < g.K) yp[dk * plane] = requant_lut(acc[i][v] + cv[v], mv[v], q, lut);
+                        if (kbase + dk < g.K) yp[dk * plane] = uint8_t(ob[v]);
                     }
                 }
             }
         }
-        cur = nxt;
-        tile_par ^= 1;
+        cur += int(gridDim.x);
     }
 }
 
 template <int MT, int WM, int WN, int TT>
 void launch_qmfma_tt(zant_ctx *ctx, const int8_t *xb, const int8_t *wp, const float *mult, const int32_t *corr,
                      const int8_t *padvec, uint8_t *y, const ConvGeom &g, const TilePlan &p, int CB, const QConvArgs &q,
-                     int *counter, int grid, int yb, int parity) {
+                     int grid, int yb, int n_stages) {
     static bool attr_set = false;
     if (!attr_set) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&qconv_mfma_kernel<MT, WM, WN, TT>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         attr_set = true;
     }
-    hipLaunchKernelGGL((qconv_mfma_kernel<MT, WM, WN, TT>), dim3(grid), dim3(WM * WN * 64), p.lds_bytes + 256, ctx->stream, xb,
-                       wp, mult, corr, padvec, y, g, p.t, CB, q, counter, parity, yb);
+    hipLaunchKernelGGL((qconv_mfma_kernel<MT, WM, WN, TT>), dim3(grid), dim3(WM * WN * 64), p.lds_bytes, ctx->stream, xb,
+                       wp, mult, corr, padvec, y, g, p.t, CB, q, n_stages, yb);
 }
 
 template <int MT, int WM, int WN>
 void launch_qmfma(zant_ctx *ctx, const int8_t *xb, const int8_t *wp, const float *mult, const int32_t *corr,
                   const int8_t *padvec, uint8_t *y, const ConvGeom &g, const TilePlan &p, int CB, const QConvArgs &q,
-                  int *counter, int grid, int yb, int parity) {
+                  int grid, int yb, int n_stages) {
     const int T = g.KH * g.KW;
-    if (T == 9) launch_qmfma_tt<MT, WM, WN, 9>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb, parity);
-    else if (T == 1) launch_qmfma_tt<MT, WM, WN, 1>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb, parity);
-    else launch_qmfma_tt<MT, WM, WN, 0>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb, parity);
+    if (T == 9) launch_qmfma_tt<MT, WM, WN, 9>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, grid, yb, n_stages);
+    else if (T == 1) launch_qmfma_tt<MT, WM, WN, 1>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, grid, yb, n_stages);
+    else launch_qmfma_tt<MT, WM, WN, 0>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, grid, yb, n_stages);
 }
 
 template <int WM, int WN>
 bool dispatch_qmt(zant_ctx *ctx, const int8_t *xb, const int8_t *wp, const float *mult, const int32_t *corr,
                   const int8_t *padvec, uint8_t *y, const ConvGeom &g, const TilePlan &p, int CB, const QConvArgs &q,
-                  int *counter, int grid, int yb, int parity) {
+                  int grid, int yb, int n_stages) {
     switch (p.MT) {
-    case 1: launch_qmfma<1, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb, parity); return true;
-    case 2: launch_qmfma<2, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb, parity); return true;
-    case 3: launch_qmfma<3, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb, parity); return true;
-    case 4: launch_qmfma<4, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb, parity); return true;
-    case 5: launch_qmfma<5, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb, parity); return true;
-    case 6: launch_qmfma<6, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb, parity); return true;
-    case 7: launch_qmfma<7, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, counter, grid, yb, parity); return true;
+    case 1: launch_qmfma<1, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, grid, yb, n_stages); return true;
+    case 2: launch_qmfma<2, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, grid, yb, n_stages); return true;
+    case 3: launch_qmfma<3, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, grid, yb, n_stages); return true;
+    case 4: launch_qmfma<4, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, grid, yb, n_stages); return true;
+    case 5: launch_qmfma<5, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, grid, yb, n_stages); return true;
+    case 6: launch_qmfma<6, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, grid, yb, n_stages); return true;
     default: return false;
     }
 }
@@ -492,12 +521,34 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
     const int CB = (g.C + 15) / 16;
     if (int64_t(g.N) * CB * g.H * g.W >= (int64_t(1) << 27)) return 1;  // 16-byte units addressed with 32-bit offsets
     TilePlan plan;
-    const int WN = g.K > 32 ? 2 : 1, WM = 4 / WN;
     ConvGeom gp = g;
     gp.C = CB;  // the planner's 32-bit offset check works in 16-byte units here
-    if (!zant_plan_conv_tiles(gp, WM, WN, 7, 2, 16, 80 * 1024, &plan) || plan.eff < 0.4) return 1;
+    // at most 6 position tiles per wave: with 7 the epilogue spills, and a scratch reload drains the copy ring.
+    // Both workgroup shapes are tried for more than 32 output channels; plans are ranked by useful MFMA columns times
+    // how much of the GPU's 2 x CUs workgroup slots they fill.
+    const int target = 2 * ctx->num_cus;
+    int WN = 1, WM = 4;
+    bool have = zant_plan_conv_tiles(gp, 4, 1, 6, 2, 16, 80 * 1024, &plan, false, target);
+    if (g.K > 32) {
+        TilePlan wide;
+        if (zant_plan_conv_tiles(gp, 2, 2, 6, 2, 16, 80 * 1024, &wide, false, target) && (!have || wide.score >= plan.score - 0.02)) {
+            plan = wide; WN = 2; WM = 2; have = true;
+        }
+    }
+    if (!have || plan.eff < 0.4) return 1;
     const int T = g.KH * g.KW, K_BLK = WN * 32;
     plan.t.n_chunks = (g.C + QCC - 1) / QCC;
+    // Ring of staging buffers: as many stages (2..4) as fit beside the tables in half a CU's LDS, and as the 6-bit
+    // vmcnt counter can tell apart.  The patch region is padded to one slot per thread and round.
+    constexpr int NT = 256;
+    plan.t.P1s = ((plan.t.P1 + NT - 1) / NT) * NT;
+    const size_t buf_bytes = size_t(w_region_bytes(T * QCC * K_BLK, NT)) + size_t(QCC) * plan.t.P1s;
+    const size_t fixed_bytes = size_t(plan.t.P1s) * 8 + 256 + size_t(plan.t.n_kblocks) * K_BLK * 8;
+    const int copies = w_region_bytes(T * QCC * K_BLK, NT) / (16 * NT) + 2 * (plan.t.P1s / NT);
+    int n_stages = 4;
+    while (n_stages > 2 && (n_stages * buf_bytes + fixed_bytes > 80 * 1024 || copies * (n_stages - 2) > 63)) --n_stages;
+    if (n_stages * buf_bytes + fixed_bytes > 80 * 1024) return 1;
+    plan.lds_bytes = n_stages * buf_bytes + fixed_bytes;
     const size_t wp_bytes = size_t(plan.t.n_chunks) * plan.t.n_kblocks * T * QCC * K_BLK;
     const size_t kpad = size_t(plan.t.n_kblocks) * K_BLK;
     const size_t xb_bytes = x_blocked ? 0 : size_t(g.N) * CB * g.H * g.W * 16;
@@ -532,8 +583,8 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
     }
     KernelTimer kt(ctx);
     const int yb = y_blocked ? 1 : 0;
-    const bool ok = WN == 2 ? dispatch_qmt<2, 2>(ctx, xb, wp, mult, corr, padvec, y, g, plan, CB, q, counter, grid, yb, parity)
-                            : dispatch_qmt<4, 1>(ctx, xb, wp, mult, corr, padvec, y, g, plan, CB, q, counter, grid, yb, parity);
+    const bool ok = WN == 2 ? dispatch_qmt<2, 2>(ctx, xb, wp, mult, corr, padvec, y, g, plan, CB, q, grid, yb, n_stages)
+                            : dispatch_qmt<4, 1>(ctx, xb, wp, mult, corr, padvec, y, g, plan, CB, q, grid, yb, n_stages);
     if (!ok) return 1;
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
