@@ -45,10 +45,18 @@ __device__ __forceinline__ void decode_tile(const TileGeom &t, int tile, int &n0
 // pool: the kernel's epilogue max-pools 2x2/2 (floor).  The MFMA column slots are then counted in POOLED positions:
 // tile registers 4j..4j+3 of a lane hold the four members of one window, so MT is a multiple of 4, TH is even and
 // a tile covers NB images x TH/2 pooled rows x OW/2 pooled columns.
-// target_tiles > 0: plans are ranked by eff * min(1, n_tiles / target_tiles) -- a layer too small to give every
-// workgroup slot of the GPU a tile is better off with smaller tiles than with fuller ones.
+// target_tiles > 0 (= 2 x CUs, the workgroup slots of the GPU): plans are ranked by an estimate of the kernel time,
+// the larger of (a) the MFMA time of the busiest workgroup slot -- which penalises padding lanes and layers too small
+// to give every slot a tile -- and (b) the time to copy every tile's operands from L2 into LDS at ~6 TB/s: the int8
+// matrix cores outrun that copy stream for all but the largest tiles, so operand reuse per staged byte decides.
+// mfma_cycles_per_tap: matrix-core cycles per wave, filter tap and position tile of one chunk.
+// copy_threads > 0: the kernel pads the patch region to one 32-byte slot and the weight slab to one 16-byte unit per
+// copying thread and round, and keeps 8 bytes of requantisation table per output channel in LDS; the footprint and the
+// staging estimate then count those padded sizes.
+// n_buffers: staging buffers that must fit (2 = double buffering; more for a deeper copy ring).
 inline bool zant_plan_conv_tiles(const ConvGeom &g, int WM, int WN, int mt_max, int chunk_channels, size_t elem_bytes,
-                                 size_t lds_cap, TilePlan *best, bool pool = false, int target_tiles = 0) {
+                                 size_t lds_cap, TilePlan *best, bool pool = false, int target_tiles = 0,
+                                 int mfma_cycles_per_tap = 32, int copy_threads = 0, int n_buffers = 2) {
     const int T = g.KH * g.KW;
     const int K_BLK = WN * 32;
     bool found = false;
@@ -74,7 +82,7 @@ inline bool zant_plan_conv_tiles(const ConvGeom &g, int WM, int WN, int mt_max, 
         t.PH = (t.TH - 1) * g.sh + (g.KH - 1) * g.dh + 1;
         t.PW = (g.OW - 1) * g.sw + (g.KW - 1) * g.dw + 1;
         t.P1 = t.NB * t.PH * t.PW;
-        t.P1s = (t.P1 + 3) & ~3;
+        t.P1s = copy_threads > 0 ? (t.P1 + copy_threads - 1) / copy_threads * copy_threads : (t.P1 + 3) & ~3;
         if (t.PH >= (1 << 16) || t.NB >= (1 << 15)) continue;  // packed into one int of the patch table
         if (int64_t(t.NB) * g.C * g.H * g.W * int64_t(elem_bytes) >= (int64_t(1) << 31)) continue;  // 32-bit offsets per image group
         t.n_chunks = (g.C + chunk_channels - 1) / chunk_channels;
@@ -83,13 +91,23 @@ inline bool zant_plan_conv_tiles(const ConvGeom &g, int WM, int WN, int mt_max, 
         const int64_t n_tiles = int64_t(t.n_sblocks) * t.n_kblocks;
         if (n_tiles >= (int64_t(1) << 30)) continue;
         t.n_tiles = int(n_tiles);
-        const size_t lds = 2 * (size_t(T) * 32 * K_BLK + size_t(32) * t.P1s)  // two staging buffers
-                           + size_t(t.P1s) * 8 + 8;                          // patch table, scheduler slots
+        size_t w_slab = size_t(T) * 32 * K_BLK, fixed = size_t(t.P1s) * 8 + 8;  // fixed: patch table, scheduler slots
+        if (copy_threads > 0) {
+            const size_t round = size_t(copy_threads) * 16;
+            w_slab = (w_slab + round - 1) / round * round;
+            fixed = size_t(t.P1s) * 8 + 256 + size_t(t.n_kblocks) * K_BLK * 8;
+        }
+        const size_t lds = n_buffers * (w_slab + size_t(32) * t.P1s) + fixed;  // the staging buffers
         if (lds > lds_cap) continue;
         const double eff = double(g.N) * rows * cols / (double(t.n_sblocks) * S);
         double score = eff;
-        if (target_tiles > 0 && t.n_tiles < target_tiles) score *= double(t.n_tiles) / target_tiles;
-        if (!found || score > best->score + 0.01) {  // larger tiles win ties: fewer tiles, more operand reuse
+        if (target_tiles > 0) {
+            const double rounds = double((t.n_tiles + target_tiles - 1) / target_tiles);
+            const double mfma = rounds * 2.0 * t.n_chunks * mt * T * mfma_cycles_per_tap;                 // cycles
+            const double stage = double(t.n_tiles) * t.n_chunks * (double(w_slab) + 32.0 * t.P1s) / 2500.0;  // cycles at 6 TB/s
+            score = 1.0e6 / (mfma > stage ? mfma : stage);
+        }
+        if (!found || score > best->score * 1.02) {  // larger tiles win ties: fewer tiles, more operand reuse
             best->MT = mt; best->WM = WM; best->WN = WN; best->t = t; best->lds_bytes = lds; best->eff = eff;
             best->score = score;
             found = true;

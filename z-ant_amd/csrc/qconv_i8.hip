@@ -524,30 +524,36 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
     ConvGeom gp = g;
     gp.C = CB;  // the planner's 32-bit offset check works in 16-byte units here
     // at most 6 position tiles per wave: with 7 the epilogue spills, and a scratch reload drains the copy ring.
-    // Both workgroup shapes are tried for more than 32 output channels; plans are ranked by useful MFMA columns times
-    // how much of the GPU's 2 x CUs workgroup slots they fill.
+    // Both workgroup shapes are tried for more than 32 output channels; plans are ranked by the planner's time estimate
+    // over the GPU's 2 x CUs workgroup slots.
     const int target = 2 * ctx->num_cus;
     int WN = 1, WM = 4;
-    bool have = zant_plan_conv_tiles(gp, 4, 1, 6, 2, 16, 80 * 1024, &plan, false, target);
+    // The footprint counts two staging buffers: larger tiles (more operand reuse per staged byte) beat a deeper ring.
+    bool have = zant_plan_conv_tiles(gp, 4, 1, 6, 2, 16, 80 * 1024, &plan, false, target, 32, 256);
     if (g.K > 32) {
         TilePlan wide;
-        if (zant_plan_conv_tiles(gp, 2, 2, 6, 2, 16, 80 * 1024, &wide, false, target) && (!have || wide.score >= plan.score - 0.02)) {
+        if (zant_plan_conv_tiles(gp, 2, 2, 6, 2, 16, 80 * 1024, &wide, false, target, 32, 256) && (!have || wide.score >= plan.score * 0.98)) {
             plan = wide; WN = 2; WM = 2; have = true;
         }
     }
     if (!have || plan.eff < 0.4) return 1;
     const int T = g.KH * g.KW, K_BLK = WN * 32;
     plan.t.n_chunks = (g.C + QCC - 1) / QCC;
-    // Ring of staging buffers: as many stages (2..4) as fit beside the tables in half a CU's LDS, and as the 6-bit
-    // vmcnt counter can tell apart.  The patch region is padded to one slot per thread and round.
+    // Ring of staging buffers: as many stages as fit beside the tables in the LDS share of a workgroup -- half a CU's
+    // 160 KB when two workgroups share a CU, all of it when the layer has no more tiles than the GPU has CUs (short
+    // per-tile sequences, where a deeper ring hides more of the copy latency) -- and as the 6-bit vmcnt counter can
+    // tell apart.  The patch region is padded to one slot per thread and round.
     constexpr int NT = 256;
     plan.t.P1s = ((plan.t.P1 + NT - 1) / NT) * NT;
     const size_t buf_bytes = size_t(w_region_bytes(T * QCC * K_BLK, NT)) + size_t(QCC) * plan.t.P1s;
     const size_t fixed_bytes = size_t(plan.t.P1s) * 8 + 256 + size_t(plan.t.n_kblocks) * K_BLK * 8;
     const int copies = w_region_bytes(T * QCC * K_BLK, NT) / (16 * NT) + 2 * (plan.t.P1s / NT);
-    int n_stages = 4;
-    while (n_stages > 2 && (n_stages * buf_bytes + fixed_bytes > 80 * 1024 || copies * (n_stages - 2) > 63)) --n_stages;
-    if (n_stages * buf_bytes + fixed_bytes > 80 * 1024) return 1;
+    const bool sparse = plan.t.n_tiles <= ctx->num_cus;
+    const size_t lds_cap = sparse ? 160 * 1024 : 80 * 1024;
+    int n_stages = sparse ? 8 : 4;
+    if (n_stages > plan.t.n_chunks + 1) n_stages = std::max(plan.t.n_chunks + 1, 2);
+    while (n_stages > 2 && (n_stages * buf_bytes + fixed_bytes > lds_cap || copies * (n_stages - 2) > 63)) --n_stages;
+    if (n_stages * buf_bytes + fixed_bytes > lds_cap) return 1;
     plan.lds_bytes = n_stages * buf_bytes + fixed_bytes;
     const size_t wp_bytes = size_t(plan.t.n_chunks) * plan.t.n_kblocks * T * QCC * K_BLK;
     const size_t kpad = size_t(plan.t.n_kblocks) * K_BLK;
