@@ -95,7 +95,7 @@ inline bool zant_plan_conv_tiles(const ConvGeom &g, int WM, int WN, int mt_max, 
         if (copy_threads > 0) {
             const size_t round = size_t(copy_threads) * 16;
             w_slab = (w_slab + round - 1) / round * round;
-            fixed = size_t(t.P1s) * 8 + 256 + size_t(t.n_kblocks) * K_BLK * 8;
+            fixed = size_t(t.P1s) * 8 + 512 + size_t(t.n_kblocks) * K_BLK * 8;
         }
         const size_t lds = n_buffers * (w_slab + size_t(32) * t.P1s) + fixed;  // the staging buffers
         if (lds > lds_cap) continue;

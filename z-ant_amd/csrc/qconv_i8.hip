@@ -237,6 +237,16 @@ __device__ __forceinline__ void lds_wait16(uint32_t (&v)[16]) {
                    "+v"(v[9]), "+v"(v[10]), "+v"(v[11]), "+v"(v[12]), "+v"(v[13]), "+v"(v[14]), "+v"(v[15]));
 }
 
+// p / d for 0 <= p < 2^20 and d > 0, with inv = 1.0f / d: the float quotient is off by at most one, which the
+// remainder corrects.  Far fewer instructions than the general 32-bit division sequence.
+__device__ __forceinline__ int small_div(int p, int d, float inv) {
+    int q = int(float(p) * inv);
+    const int r = p - q * d;
+    q += r >= d ? 1 : 0;
+    q -= r < 0 ? 1 : 0;
+    return q;
+}
+
 // Waits until at most n of this wave's vector-memory operations are outstanding (n is wave-uniform, 0..63).
 __device__ __forceinline__ void wait_vmcnt(int n) {
 #define ZANT_VM(k) case k: __builtin_amdgcn_s_waitcnt(((k) & 15) | (((k) >> 4) << 14) | 0x0F70); break;
@@ -323,14 +333,18 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
                   TileGeom t, int CB, QConvArgs q, int n_stages, int y_blocked) {
     constexpr int NT = WM * WN * 64;
     constexpr int K_BLK = WN * 32;
-    extern __shared__ __attribute__((aligned(16))) char qlds[];
+    extern __shared__ __attribute__((aligned(256))) char qlds_raw[];
     const int T = TT > 0 ? TT : g.KH * g.KW;
     const int w_chunk = T * QCC * K_BLK;                           // bytes per (chunk, kblock) weight slab
     const int buf_bytes = w_region_bytes(w_chunk, NT) + QCC * t.P1s;  // one staging buffer (P1s: multiple of NT)
-    int2 *ptab = reinterpret_cast<int2 *>(qlds + n_stages * buf_bytes);
-    uint8_t *lut = reinterpret_cast<uint8_t *>(ptab + t.P1s);  // [256] fused activation table
+    // LDS: [256-byte activation table, 256-aligned][n_stages staging buffers][patch table][multipliers][corrections]
+    const unsigned lut_a = (lds_addr_of(qlds_raw) + 255u) & ~255u;
+    char *qlds = qlds_raw + (lut_a - lds_addr_of(qlds_raw));
+    uint8_t *lut = reinterpret_cast<uint8_t *>(qlds);
+    char *ring = qlds + 256;
+    int2 *ptab = reinterpret_cast<int2 *>(ring + n_stages * buf_bytes);
     const int kpad = t.n_kblocks * K_BLK;
-    float *mult_l = reinterpret_cast<float *>(lut + 256);       // [kpad] requantisation multipliers ...
+    float *mult_l = reinterpret_cast<float *>(ptab + t.P1s);    // [kpad] requantisation multipliers ...
     int *corr_l = reinterpret_cast<int *>(mult_l + kpad);       // [kpad] ... and integer corrections, copied once
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -339,57 +353,80 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
     const int64_t plane_in = int64_t(g.H) * g.W;
     const int per_img = t.TH * g.OW;
     const int patch_hw = t.PH * t.PW;
-    lut[tid & 255] = q.has_act ? qact_apply(uint8_t(tid & 255), q.act) : uint8_t(tid & 255);  // NT == 256
+    const float inv_per_img = 1.0f / float(per_img), inv_ow = 1.0f / float(g.OW);
+    // The tables first (plain LDS writes), the copies after them: an LDS write behind an asynchronous copy would wait
+    // for the copy.  The activation table holds output bytes as they are stored (blocked tensors keep value ^ 0x80).
+    {
+        const uint8_t b = uint8_t(tid & 255);
+        lut[tid & 255] = uint8_t((q.has_act ? qact_apply(b, q.act) : b) ^ (y_blocked ? 0x80 : 0));  // NT == 256
+    }
     for (int k = tid; k < kpad; k += NT) { mult_l[k] = mult[k]; corr_l[k] = corr[k]; }
-
-    for (int e = tid; e < t.P1s; e += NT) {
-        const int img = e / patch_hw, rem = e - img * patch_hw;
-        const int ph = rem / t.PW, pw = rem - ph * t.PW;
-        const int iw = pw - g.pl;
-        int2 v;
-        v.x = (e < t.P1 && iw >= 0 && iw < g.W) ? int(img * CB * plane_in) + ph * g.W + iw : -1;
-        v.y = (img << 16) | ph;
-        ptab[e] = v;
+    {
+        const float inv_patch = 1.0f / float(patch_hw), inv_pw = 1.0f / float(t.PW);
+        for (int e = tid; e < t.P1s; e += NT) {
+            const int img = small_div(e, patch_hw, inv_patch), rem = e - img * patch_hw;
+            const int ph = small_div(rem, t.PW, inv_pw), pw = rem - ph * t.PW;
+            const int iw = pw - g.pl;
+            int2 v;
+            v.x = (e < t.P1 && iw >= 0 && iw < g.W) ? int(img * CB * plane_in) + ph * g.W + iw : -1;
+            v.y = (img << 16) | ph;
+            ptab[e] = v;   // read back by this same thread only (qconv_issue)
+        }
     }
-    int lds_off[MT];
-#pragma unroll
-    for (int i = 0; i < MT; ++i) {
-        const int p = (wm * MT + i) * 32 + l32;
-        const int img = p / per_img, rem = p - img * per_img;
-        const int r = rem / g.OW, c = rem - r * g.OW;
-        lds_off[i] = (img < t.NB && r < t.TH) ? (img * t.PH + r * g.sh) * t.PW + c * g.sw : 0;
-    }
-    __syncthreads();
-
     if (int(blockIdx.x) >= t.n_tiles) return;
     const int my_tiles = (t.n_tiles - int(blockIdx.x) + int(gridDim.x) - 1) / int(gridDim.x);
     const int n_steps = my_tiles * t.n_chunks;
     // copies per thread and step (see qconv_issue)
     const int P = w_region_bytes(w_chunk, NT) / (16 * NT) + 2 * (t.P1s / NT);
-    i32x16 acc[MT];
-    // prologue: the first n_stages - 1 steps' copies
+    // prologue: the first n_stages - 1 steps' copies, in flight behind the index arithmetic below
     for (int s0 = 0; s0 < n_stages - 1 && s0 < n_steps; ++s0)
-        qconv_issue<WM, WN, TT>(qlds + s0 * buf_bytes, ptab, xb, wp, padvec, g, t, CB,
+        qconv_issue<WM, WN, TT>(ring + s0 * buf_bytes, ptab, xb, wp, padvec, g, t, CB,
                                 int(blockIdx.x) + (s0 / t.n_chunks) * int(gridDim.x), s0 % t.n_chunks);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // Position slot i of this lane: image, row and column inside the tile.  pos[i] packs them for the epilogue
+    // (image << 20 | row << 10 | column; -1 = the slot is beyond the tile).
+    int lds_off[MT], pos[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        const int p = (wm * MT + i) * 32 + l32;
+        const int img = small_div(p, per_img, inv_per_img), rem = p - img * per_img;
+        const int r = small_div(rem, g.OW, inv_ow), c = rem - r * g.OW;
+        const bool in_tile = img < t.NB && r < t.TH;
+        lds_off[i] = in_tile ? (img * t.PH + r * g.sh) * t.PW + c * g.sw : 0;
+        pos[i] = in_tile ? (img << 20) | (r << 10) | c : -1;
+    }
+    // everybody's table writes are visible after the first barrier of the loop below
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0) only
+    const unsigned mult_a = lds_addr_of(mult_l), corr_a = lds_addr_of(corr_l);
+
+    i32x16 acc[MT];
     int cbuf = 0, dbuf = n_stages - 1;    // ring slots of the step being multiplied / of the step being copied
     int itile = int(blockIdx.x), ichunk = 0;  // (tile, chunk) of the step whose copies are issued next
     for (int s0 = 0; s0 < n_stages - 1; ++s0)
         if (++ichunk == t.n_chunks) { ichunk = 0; itile += int(gridDim.x); }
     int cur = int(blockIdx.x), chunk = 0;
     for (int s0 = 0; s0 < n_steps; ++s0) {
-        if (chunk == 0) {
-#pragma unroll
-            for (int i = 0; i < MT; ++i)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) acc[i][v] = 0;
-        }
         // This wave's copies of step s0 have landed once no more than the copies of the later steps are outstanding
         // (loads complete in order); after the barrier everybody's have, and everybody is done with step s0 - 1,
         // whose ring slot is refilled now.  A bare s_barrier: __syncthreads() would drain every outstanding copy.
         wait_vmcnt(P * min(n_stages - 2, n_steps - 1 - s0));
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        qconv_step<MT, WM, WN, TT>(qlds + dbuf * buf_bytes, qlds + cbuf * buf_bytes, ptab, xb, wp, padvec, g, t, CB,
+        if (chunk == 0) {
+            // accumulators start from the integer corrections of this lane's 16 output channels
+            const int kb = cur % t.n_kblocks;
+            const int kbase = kb * K_BLK + wn * 32 + lh * 4;
+            uint32_t craw[16];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) craw[v] = lds_read_b32_async(corr_a + unsigned(kbase + (v >> 2) * 8 + (v & 3)) * 4u);
+            lds_wait16(craw);
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][v] = int(craw[v]);
+        }
+        qconv_step<MT, WM, WN, TT>(ring + dbuf * buf_bytes, ring + cbuf * buf_bytes, ptab, xb, wp, padvec, g, t, CB,
                                    s0 + n_stages - 1 < n_steps, itile, ichunk, lds_off, acc);
         if (++ichunk == t.n_chunks) { ichunk = 0; itile += int(gridDim.x); }
         cbuf = cbuf + 1 == n_stages ? 0 : cbuf + 1;
@@ -397,7 +434,7 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
         if (++chunk < t.n_chunks) continue;
         chunk = 0;
 
-        // ---- epilogue: integer correction, requantisation (+ fused activation), NCHW u8 stores ----
+        // ---- epilogue: requantisation (+ fused activation), stores ----
         {
             int n0, oh0, kb;
             decode_tile(t, cur, n0, oh0, kb);
@@ -405,44 +442,49 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
             const int imgs_here = min(t.NB, g.N - n0);
             const int64_t plane = int64_t(g.OH) * g.OW;
             const int kbase = kb * K_BLK + wn * 32 + lh * 4;
-            // multipliers and corrections of this lane's 16 channels, then per tile the 16 activation-table lookups,
-            // all through hand-issued LDS reads: the next steps' copies stay in flight behind the epilogue
-            uint32_t mraw[16], craw[16];
-            const unsigned lut_a = lds_addr_of(lut), mult_a = lds_addr_of(mult_l), corr_a = lds_addr_of(corr_l);
+            // multipliers of this lane's 16 channels, then per position the 16 activation-table lookups, all through
+            // hand-issued LDS reads: the next steps' copies stay in flight behind the epilogue
+            uint32_t mraw[16];
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int k = kbase + (v >> 2) * 8 + (v & 3);  // < n_kblocks * K_BLK: the tables are padded
-                mraw[v] = lds_read_b32_async(mult_a + unsigned(k) * 4u);
-                craw[v] = lds_read_b32_async(corr_a + unsigned(k) * 4u);
-            }
+            for (int v = 0; v < 16; ++v) mraw[v] = lds_read_b32_async(mult_a + unsigned(kbase + (v >> 2) * 8 + (v & 3)) * 4u);
             lds_wait16(mraw);
-            lds_wait16(craw);
             float mv[16];
-            int cv[16];
 #pragma unroll
-            for (int v = 0; v < 16; ++v) { mv[v] = __uint_as_float(mraw[v]); cv[v] = int(craw[v]); }
+            for (int v = 0; v < 16; ++v) mv[v] = __uint_as_float(mraw[v]);
             const float zpf = float(q.y_zp);
             const int KB = (g.K + 15) >> 4;
             const int cb0 = (kb * K_BLK + wn * 32) >> 4;
+            const bool use_lut = q.has_act || !y_blocked;
 #pragma unroll
             for (int i = 0; i < MT; ++i) {
-                const int p = (wm * MT + i) * 32 + l32;
-                const int img = p / per_img, rem = p - img * per_img;
-                const int r = rem / g.OW, c = rem - r * g.OW;
-                const bool ok = img < imgs_here && r < rows_here;
-                uint32_t ob[16];  // the 16 output bytes of this position
-#pragma unroll
-                for (int v = 0; v < 16; ++v)
-                    ob[v] = lds_read_u8_async(lut_a + sat_u8_rne_finite(float(acc[i][v] + cv[v]) * mv[v], zpf));
-                lds_wait16(ob);
+                const int img = pos[i] >> 20, r = (pos[i] >> 10) & 1023, c = pos[i] & 1023;
+                const bool ok = pos[i] >= 0 && img < imgs_here && r < rows_here;
                 if (y_blocked) {
                     // [N][KB][OH][OW][16] signed.  A lane holds 4 groups of 4 consecutive channels; lanes l and l+32
                     // swap one dword per 16-channel block so that each stores 8 consecutive bytes: a half-wave then
                     // writes 32 positions x 16 bytes without gaps.
                     uint32_t d[4];
+                    if (use_lut) {
+                        uint32_t ob[16];
+                        // the converted byte lands in the low byte of the (256-aligned) table address
 #pragma unroll
-                    for (int gq = 0; gq < 4; ++gq)
-                        d[gq] = (ob[gq * 4] | (ob[gq * 4 + 1] << 8) | (ob[gq * 4 + 2] << 16) | (ob[gq * 4 + 3] << 24)) ^ 0x80808080u;
+                        for (int v = 0; v < 16; ++v)
+                            ob[v] = lds_read_u8_async(__builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(float(acc[i][v]) * mv[v]) + zpf, 0u, lut_a));
+                        lds_wait16(ob);
+#pragma unroll
+                        for (int gq = 0; gq < 4; ++gq)
+                            d[gq] = ob[gq * 4] | (ob[gq * 4 + 1] << 8) | (ob[gq * 4 + 2] << 16) | (ob[gq * 4 + 3] << 24);
+                    } else {
+                        // no activation: the saturating conversion packs the four bytes of a dword itself
+#pragma unroll
+                        for (int gq = 0; gq < 4; ++gq) {
+                            uint32_t w4 = 0;
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                w4 = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(float(acc[i][gq * 4 + e]) * mv[gq * 4 + e]) + zpf, unsigned(e), w4);
+                            d[gq] = w4 ^ 0x80808080u;
+                        }
+                    }
 #pragma unroll
                     for (int b = 0; b < 2; ++b) {
                         const uint32_t send = lh ? d[2 * b] : d[2 * b + 1];
@@ -450,15 +492,22 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
                         const uint2 out = lh ? make_uint2(recv, d[2 * b + 1]) : make_uint2(d[2 * b], recv);
                         if (ok && cb0 + b < KB) {
                             uint8_t *yp = y + (((int64_t(n0 + img) * KB + cb0 + b) * g.OH + oh0 + r) * g.OW + c) * 16 + lh * 8;
-                            *reinterpret_cast<uint2 *>(yp) = out;
+                            __builtin_nontemporal_store(*reinterpret_cast<const unsigned long long *>(&out), reinterpret_cast<unsigned long long *>(yp));
                         }
                     }
-                } else if (ok) {
-                    uint8_t *yp = y + (int64_t(n0 + img) * g.K + kbase) * plane + int64_t(oh0 + r) * g.OW + c;
+                } else {
+                    uint32_t ob[16];  // the 16 output bytes of this position
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int dk = (v >> 2) * 8 + (v & 3);
-                        if (kbase + dk < g.K) yp[dk * plane] = uint8_t(ob[v]);
+                    for (int v = 0; v < 16; ++v)
+                        ob[v] = lds_read_u8_async(__builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(float(acc[i][v]) * mv[v]) + zpf, 0u, lut_a));
+                    lds_wait16(ob);
+                    if (ok) {
+                        uint8_t *yp = y + (int64_t(n0 + img) * g.K + kbase) * plane + int64_t(oh0 + r) * g.OW + c;
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            const int dk = (v >> 2) * 8 + (v & 3);
+                            if (kbase + dk < g.K) yp[dk * plane] = uint8_t(ob[v]);
+                        }
                     }
                 }
             }
@@ -546,7 +595,7 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
     constexpr int NT = 256;
     plan.t.P1s = ((plan.t.P1 + NT - 1) / NT) * NT;
     const size_t buf_bytes = size_t(w_region_bytes(T * QCC * K_BLK, NT)) + size_t(QCC) * plan.t.P1s;
-    const size_t fixed_bytes = size_t(plan.t.P1s) * 8 + 256 + size_t(plan.t.n_kblocks) * K_BLK * 8;
+    const size_t fixed_bytes = size_t(plan.t.P1s) * 8 + 512 + size_t(plan.t.n_kblocks) * K_BLK * 8;  // 256: table, 256: its alignment
     const int copies = w_region_bytes(T * QCC * K_BLK, NT) / (16 * NT) + 2 * (plan.t.P1s / NT);
     const bool sparse = plan.t.n_tiles <= ctx->num_cus;
     const size_t lds_cap = sparse ? 160 * 1024 : 80 * 1024;
