@@ -905,19 +905,126 @@ qdw3x3_blocked_kernel(const uint4 *__restrict__ x, const uint32_t *__restrict__ 
     }
 }
 
+// The same on the int8 matrix cores.  A wavefront takes 32 output positions x 32 channels (two channel blocks): lane
+// (p, h) loads the nine 16-byte taps of position p in channel block h -- exactly the B operand of
+// v_mfma_i32_32x32x32_i8 -- and multiplies them by nine DIAGONAL 32x32 weight matrices (row c holds tap t's weight of
+// channel c in column c), built once per workgroup in registers.  1/32 of the multiplies are useful, yet nine MFMAs
+// replace 144 dot instructions per lane, which is what bounded the VALU version.  The accumulators come out as 16
+// channels of one position per lane, requantised and stored like the dense kernel's blocked epilogue.
+__global__ void __launch_bounds__(256)
+qdw3x3_mfma_kernel(const uint4 *__restrict__ x, const uint32_t *__restrict__ wm, const float *__restrict__ mult,
+                   const int32_t *__restrict__ corr, uint8_t *__restrict__ y, ConvGeom g, QConvArgs q, int CB,
+                   int blocks_per_pair) {
+    __shared__ uint8_t lut[256];
+    lut[threadIdx.x] = uint8_t((q.has_act ? qact_apply(uint8_t(threadIdx.x), q.act) : uint8_t(threadIdx.x)) ^ 0x80);
+    __syncthreads();
+    const int pair = blockIdx.x / blocks_per_pair, blk = blockIdx.x - pair * blocks_per_pair;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lh = lane >> 5;
+    const int cb = 2 * pair + lh;
+    const bool cb_ok = cb < CB;
+    i32x4 a[9];
+    {
+        const int k = pair * 32 + l32, kcb = k >> 4, qd = (k >> 2) & 3, j = k & 3;
+        const bool mine = (l32 >> 4) == lh;  // the diagonal element of row l32 lies in this lane's half of the columns
+#pragma unroll
+        for (int t = 0; t < 9; ++t) {
+            const int wv = mine ? int(wm[((kcb * 4 + qd) * 9 + t) * 4 + j]) : 0;
+            a[t][0] = qd == 0 ? wv : 0;
+            a[t][1] = qd == 1 ? wv : 0;
+            a[t][2] = qd == 2 ? wv : 0;
+            a[t][3] = qd == 3 ? wv : 0;
+        }
+    }
+    float mv[16];
+    int cv[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const int k = pair * 32 + (v >> 2) * 8 + lh * 4 + (v & 3);
+        mv[v] = mult[k];
+        cv[v] = corr[k];
+    }
+    const unsigned total = unsigned(g.N) * unsigned(g.OH) * unsigned(g.OW);  // < 2^31 (checked by the host)
+    const unsigned n_ptiles = (total + 31u) / 32u;
+    const unsigned per_img = unsigned(g.OH) * unsigned(g.OW);                // < 2^20 (checked by the host)
+    const float inv_per_img = 1.0f / float(per_img), inv_ow = 1.0f / float(g.OW);
+    const bool small_total = total < (1u << 20);
+    const uint32_t pad4 = uint32_t(q.x_zp ^ 0x80) * 0x01010101u;
+    const float zpf = float(q.y_zp);
+    i32x16 cvec;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) cvec[v] = cv[v];
+    const char *xbytes = reinterpret_cast<const char *>(x);  // the whole tensor is < 4 GB (checked by the host)
+    const unsigned plane = unsigned(g.H) * unsigned(g.W);
+    for (unsigned pt = unsigned(blk) * 4u + unsigned(wave); pt < n_ptiles; pt += unsigned(blocks_per_pair) * 4u) {
+        const unsigned i = pt * 32u + unsigned(l32);
+        const bool valid = i < total;
+        const unsigned ii = valid ? i : total - 1u;
+        const unsigned n = small_total ? unsigned(small_div(int(ii), int(per_img), inv_per_img)) : ii / per_img;
+        const int rem = int(ii - n * per_img);
+        const int oh = small_div(rem, g.OW, inv_ow), ow = rem - oh * g.OW;
+        // Every tap is loaded from an address inside the tensor (a tap outside the image reads its clamped neighbour)
+        // and replaced by the padding vector afterwards: no divergent control flow around the loads.
+        const int ih0 = oh * g.sh - g.pt, iw0 = ow * g.sw - g.pl;  // top-left tap
+        const unsigned base = (n * unsigned(CB) + unsigned(cb_ok ? cb : 0)) * plane * 16u;
+        bool rv[3], cvd[3];
+        unsigned rowb[3], colb[3];
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            const int ih = ih0 + k, iw = iw0 + k;
+            rv[k] = cb_ok && ih >= 0 && ih < g.H;
+            cvd[k] = iw >= 0 && iw < g.W;
+            rowb[k] = base + unsigned(min(max(ih, 0), g.H - 1)) * unsigned(g.W) * 16u;
+            colb[k] = unsigned(min(max(iw, 0), g.W - 1)) * 16u;
+        }
+        uint4 xv[9];
+#pragma unroll
+        for (int t = 0; t < 9; ++t) xv[t] = *reinterpret_cast<const uint4 *>(xbytes + (rowb[t / 3] + colb[t % 3]));
+        i32x16 acc;
+#pragma unroll
+        for (int t = 0; t < 9; ++t) {
+            const bool ok = rv[t / 3] && cvd[t % 3];
+            i32x4 b;
+            b[0] = int(ok ? xv[t].x : pad4); b[1] = int(ok ? xv[t].y : pad4);
+            b[2] = int(ok ? xv[t].z : pad4); b[3] = int(ok ? xv[t].w : pad4);
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[t], b, t == 0 ? cvec : acc, 0, 0, 0);
+        }
+        uint32_t d[4];
+#pragma unroll
+        for (int gq = 0; gq < 4; ++gq) {
+            uint32_t o = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                o |= uint32_t(lut[sat_u8_rne_finite(float(acc[gq * 4 + e]) * mv[gq * 4 + e], zpf)]) << (8 * e);
+            d[gq] = o;
+        }
+        // lanes p and p + 32 exchange one dword per channel block so that each stores 8 consecutive bytes
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            const uint32_t send = lh ? d[2 * b] : d[2 * b + 1];
+            const uint32_t recv = uint32_t(__shfl_xor(int(send), 32, 64));
+            const uint2 out = lh ? make_uint2(recv, d[2 * b + 1]) : make_uint2(d[2 * b], recv);
+            const int cbo = 2 * pair + b;
+            if (valid && cbo < CB) {
+                uint8_t *yp = y + (((int64_t(n) * CB + cbo) * g.OH + oh) * int64_t(g.OW) + ow) * 16 + lh * 8;
+                *reinterpret_cast<uint2 *>(yp) = out;
+            }
+        }
+    }
+}
+
 bool dw_eligible(const ConvGeom &g) {
     return g.groups == g.C && g.K == g.C && g.CG == 1 && g.KH == 3 && g.KW == 3 && g.dh == 1 && g.dw == 1;
 }
 
 size_t qdw_table_bytes(int C) {
-    const int CB = (C + 15) / 16;
+    const int CB = ((C + 31) / 32) * 2;  // the matrix-core kernel works on pairs of channel blocks
     return 2 * align256(size_t(CB) * 64) + size_t(CB) * 144 * 4;
 }
 
 // x, y blocked; `tables` holds qdw_table_bytes(C) bytes that are (re)filled when need_pack is set.
 int run_qdw_blocked(zant_ctx *ctx, const uint8_t *xb, const int8_t *w, const float *w_scale, const int32_t *bias, uint8_t *yb,
                     const ConvGeom &g, const QConvArgs &q, void *tables, bool need_pack) {
-    const int CB = (g.C + 15) / 16, kpad = CB * 16;
+    const int CB = (g.C + 15) / 16, n_pairs = (CB + 1) / 2, kpad = n_pairs * 32;
     const size_t o_corr = align256(size_t(kpad) * 4), o_w = 2 * o_corr;
     char *base = static_cast<char *>(tables);
     float *mult = reinterpret_cast<float *>(base);
@@ -929,12 +1036,20 @@ int run_qdw_blocked(zant_ctx *ctx, const uint8_t *xb, const int8_t *w, const flo
         ZANT_LAUNCH_CHECK(ctx);
     }
     const int64_t per_cb = int64_t(g.N) * g.OH * g.OW;
-    const int64_t want = std::max<int64_t>(1, (int64_t(ctx->num_cus) * 16 + CB - 1) / CB);
-    const int blocks_per_cb = int(std::min<int64_t>(std::max<int64_t>(ceil_div64(per_cb, 256), 1), want));
     KernelTimer kt(ctx);
-    hipLaunchKernelGGL(qdw3x3_blocked_kernel, dim3(unsigned(CB) * blocks_per_cb), dim3(256), 0, ctx->stream,
-                       reinterpret_cast<const uint4 *>(xb), wm, mult, corr, reinterpret_cast<uint4 *>(yb), g, q, CB,
-                       blocks_per_cb);
+    if (per_cb < (int64_t(1) << 31) - 64 && int64_t(g.OH) * g.OW < (1 << 20) &&
+        int64_t(g.N) * CB * g.H * g.W * 16 < (int64_t(1) << 32)) {
+        const int64_t want = std::max<int64_t>(1, (int64_t(ctx->num_cus) * 8 + n_pairs - 1) / n_pairs);
+        const int blocks_per_pair = int(std::min<int64_t>(std::max<int64_t>(ceil_div64(per_cb, 128), 1), want));
+        hipLaunchKernelGGL(qdw3x3_mfma_kernel, dim3(unsigned(n_pairs) * blocks_per_pair), dim3(256), 0, ctx->stream,
+                           reinterpret_cast<const uint4 *>(xb), wm, mult, corr, yb, g, q, CB, blocks_per_pair);
+    } else {
+        const int64_t want = std::max<int64_t>(1, (int64_t(ctx->num_cus) * 16 + CB - 1) / CB);
+        const int blocks_per_cb = int(std::min<int64_t>(std::max<int64_t>(ceil_div64(per_cb, 256), 1), want));
+        hipLaunchKernelGGL(qdw3x3_blocked_kernel, dim3(unsigned(CB) * blocks_per_cb), dim3(256), 0, ctx->stream,
+                           reinterpret_cast<const uint4 *>(xb), wm, mult, corr, reinterpret_cast<uint4 *>(yb), g, q, CB,
+                           blocks_per_cb);
+    }
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
 }
