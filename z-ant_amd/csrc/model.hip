@@ -23,7 +23,7 @@ namespace {
 
 enum OpKind {
     OP_CONV, OP_RELU, OP_LEAKY, OP_MAXPOOL, OP_RESHAPE, OP_GEMM, OP_MATMUL, OP_ADD_CONST, OP_ADD, OP_SOFTMAX,
-    OP_QUANT, OP_DEQUANT, OP_QCONV, OP_QACT, OP_QADD, OP_QGAP
+    OP_QUANT, OP_DEQUANT, OP_QCONV, OP_QACT, OP_QADD, OP_QGAP, OP_QBLOCK
 };
 
 struct MTensor {
@@ -74,6 +74,8 @@ struct MNode {
     int b_rank = 0;
     int64_t bdim[8] = {0};
     mutable zant_pack_slot slot;  // packed weights / tables of this node, filled by its first launch
+    // OP_QBLOCK (a fused inverted residual block): the expansion, depthwise, projection and residual Add nodes
+    int blk_expand = -1, blk_dw = -1, blk_project = -1, blk_add = -1;
 };
 
 }  // namespace
@@ -143,6 +145,38 @@ int append(zant_model *m, MNode &node, int dtype, const int64_t *dims, int rank,
     node.out = add_tensor(m, dtype, dims, rank, scale, zp);
     m->n.push_back(node);
     return node.out;
+}
+
+// One QLinearConv node as the fused block kernel takes it.  x_scale / x_zp: the tensor the node reads.
+zant_qconv_desc qconv_desc(const zant_model *m, const MNode &cv, float x_scale, int x_zp) {
+    const MTensor &to = m->t[cv.out];
+    zant_qconv_desc d;
+    d.w = static_cast<const int8_t *>(param_ptr(m, cv.w));
+    d.w_scale = static_cast<const float *>(param_ptr(m, cv.ws));
+    d.n_wscale = cv.n_wscale;
+    d.bias = static_cast<const int32_t *>(param_ptr(m, cv.b));
+    d.K = cv.wdim[0];
+    d.C = cv.group > 1 ? cv.wdim[0] : cv.wdim[1];
+    d.x_scale = x_scale; d.x_zp = x_zp;
+    d.y_scale = cv.fuse_act ? cv.act_scale : to.scale;
+    d.y_zp = cv.fuse_act ? cv.act_zp : to.zp;
+    d.act = cv.fuse_act; d.act_alpha = cv.act_alpha;
+    d.act_scale = to.scale; d.act_zp = to.zp;
+    return d;
+}
+
+// The three convolutions of a fused block (each reads what the one before it stores) and the residual Add's output.
+void fill_block_descs(const zant_model *m, const MNode &nd, zant_qconv_desc d[3], float *add_scale, int *add_zp) {
+    const MNode &ex = m->n[nd.blk_expand], &dw = m->n[nd.blk_dw], &pj = m->n[nd.blk_project];
+    const MTensor &ti = m->t[nd.in0];
+    d[0] = qconv_desc(m, ex, ti.scale, ti.zp);
+    d[1] = qconv_desc(m, dw, m->t[ex.out].scale, m->t[ex.out].zp);
+    d[2] = qconv_desc(m, pj, m->t[dw.out].scale, m->t[dw.out].zp);
+    if (nd.blk_add >= 0) {
+        const MTensor &ao = m->t[m->n[nd.blk_add].out];
+        *add_scale = ao.scale;
+        *add_zp = ao.zp;
+    }
 }
 
 int run_node(zant_model *m, const MNode &nd) {
@@ -226,6 +260,14 @@ int run_node(zant_model *m, const MNode &nd) {
                                      static_cast<const uint8_t *>(tensor_ptr(m, nd.in1)), tb.scale, uint8_t(tb.zp), to.scale,
                                      uint8_t(to.zp), static_cast<uint8_t *>(y),
                                      int64_t(m->t[root_of(m, nd.in0)].storage_bytes()), lin == ZANT_LAYOUT_BLOCKED16 ? 0x80 : 0);
+    }
+    case OP_QBLOCK: {
+        zant_qconv_desc d[3];
+        float add_scale = 1.0f;
+        int add_zp = 0;
+        fill_block_descs(m, nd, d, &add_scale, &add_zp);
+        return zant_qblock_blocked(ctx, static_cast<const uint8_t *>(x), ti.dim, &d[0], &d[1], m->n[nd.blk_dw].stride[0], &d[2],
+                                   nd.blk_add >= 0, add_scale, add_zp, static_cast<uint8_t *>(y), to.dim, false, &nd.slot);
     }
     case OP_QGAP:
         if (lin == ZANT_LAYOUT_BLOCKED16)
@@ -685,6 +727,73 @@ extern "C" int zant_model_finalize(zant_model *m) {
         (void)ntl;
     }
 
+    // ---- inverted residual blocks: 1x1 expansion -> depthwise 3x3 -> 1x1 projection (-> Add with the block input) in one
+    // kernel; the expanded tensors are never materialised -------------------------------------------------------------
+    {
+        auto is_1x1 = [](const MNode &c) {
+            return c.op == OP_QCONV && !c.skip && !c.fuse_pool && c.group == 1 && c.wdim[2] == 1 && c.wdim[3] == 1 &&
+                   c.stride[0] == 1 && c.stride[1] == 1 && c.pads[0] == 0 && c.pads[1] == 0 && c.pads[2] == 0 && c.pads[3] == 0;
+        };
+        // the single live reader of a tensor, looking through the activation nodes already folded into their producers
+        auto next_reader = [&](int tensor) {
+            int only = -1;
+            while (consumers(m, tensor, &only) == 1 && m->n[only].skip && m->n[only].op == OP_QACT) tensor = m->n[only].out;
+            return consumers(m, tensor, &only) == 1 && !m->n[only].skip ? only : -1;
+        };
+        for (int i = 0; i < nn; ++i) {
+            MNode &ex = m->n[i];
+            if (!is_1x1(ex) || m->t[root_of(m, ex.in0)].layout != ZANT_LAYOUT_BLOCKED16) continue;
+            const int id = next_reader(ex.out);
+            if (id < 0) continue;
+            MNode &dw = m->n[id];
+            if (dw.op != OP_QCONV || dw.fuse_pool || dw.group != dw.wdim[0] || dw.wdim[1] != 1 || dw.wdim[2] != 3 ||
+                dw.wdim[3] != 3 || dw.group != ex.wdim[0] || dw.stride[0] != dw.stride[1] || dw.stride[0] < 1 ||
+                dw.stride[0] > 2 || dw.dil[0] != 1 || dw.dil[1] != 1 || dw.pads[0] != 1 || dw.pads[1] != 1 || dw.pads[2] != 1 ||
+                dw.pads[3] != 1)
+                continue;
+            const int ip = next_reader(dw.out);
+            if (ip < 0 || !is_1x1(m->n[ip]) || m->n[ip].fuse_act != ZANT_ACT_NONE) continue;
+            MNode &pj = m->n[ip];
+            int ia = next_reader(pj.out);
+            if (ia >= 0) {
+                const MNode &ad = m->n[ia];
+                const int other = ad.in0 == pj.out ? ad.in1 : ad.in0;
+                if (ad.op != OP_QADD || other < 0 || root_of(m, other) != root_of(m, ex.in0)) ia = -1;
+            }
+            const int last = ia >= 0 ? ia : ip;
+            if (m->t[root_of(m, m->n[last].out)].layout != ZANT_LAYOUT_BLOCKED16) continue;
+            MNode blk;
+            blk.op = OP_QBLOCK;
+            blk.in0 = ex.in0;
+            blk.out = m->n[last].out;
+            blk.blk_expand = i; blk.blk_dw = id; blk.blk_project = ip; blk.blk_add = ia;
+            zant_qconv_desc d[3];
+            float add_scale = 1.0f;
+            int add_zp = 0;
+            fill_block_descs(m, blk, d, &add_scale, &add_zp);
+            if (zant_qblock_blocked(ctx, nullptr, m->t[ex.in0].dim, &d[0], &d[1], dw.stride[0], &d[2], ia >= 0, add_scale, add_zp,
+                                    nullptr, m->t[blk.out].dim, true, nullptr) != ZANT_OK)
+                continue;
+            // the block node takes the place of its last member (ready order); the members keep their tensor ids
+            ex.skip = true; dw.skip = true; pj.skip = true;
+            if (ia >= 0) m->n[ia].skip = true;
+            MNode &slot_node = m->n[last];
+            const MNode keep = slot_node;
+            slot_node.op = OP_QBLOCK;
+            slot_node.skip = false;
+            slot_node.in0 = blk.in0; slot_node.in1 = -1;
+            slot_node.blk_expand = i; slot_node.blk_dw = id; slot_node.blk_project = ip; slot_node.blk_add = ia;
+            // the member's own fields move to a spare node appended at the end (skipped, never run)
+            MNode spare = keep;
+            spare.skip = true;
+            spare.in0 = -1; spare.in1 = -1;  // no longer a reader of anything
+            spare.slot = zant_pack_slot();
+            m->n.push_back(spare);
+            const int moved = int(m->n.size()) - 1;
+            if (last == ip) m->n[last].blk_project = moved; else m->n[last].blk_add = moved;
+        }
+    }
+
     // ---- liveness and first-fit arena planning --------------------------------------------------
     const int nt = int(m->t.size());
     for (int i = 0; i < nt; ++i) { m->t[i].def = -1; m->t[i].last = -1; }
@@ -849,6 +958,7 @@ const char *op_name(const MNode &nd) {
     case OP_QACT: return "QLinearAct";
     case OP_QADD: return "QLinearAdd";
     case OP_QGAP: return "QLinearGlobalAveragePool";
+    case OP_QBLOCK: return nd.blk_add >= 0 ? "InvertedResidual(1x1+dw3x3+1x1+Add)" : "InvertedResidual(1x1+dw3x3+1x1)";
     default: return "?";
     }
 }
@@ -879,6 +989,14 @@ void node_work(const zant_model *m, const MNode &nd, double *ops, double *bytes)
         const double K = double(ti.dim[ti.rank - 1]);
         o = 2.0 * double(to.dim[to.rank - 2]) * double(to.dim[to.rank - 1]) * K;
         b += double(nd.bdim[nd.b_rank - 2] * nd.bdim[nd.b_rank - 1]) * 4.0;
+        break;
+    }
+    case OP_QBLOCK: {
+        const MNode &ex = m->n[nd.blk_expand], &dw = m->n[nd.blk_dw], &pj = m->n[nd.blk_project];
+        const double pos_in = double(ti.dim[0] * ti.dim[2] * ti.dim[3]), pos_out = double(to.dim[0] * to.dim[2] * to.dim[3]);
+        o = 2.0 * (pos_in * double(ex.wdim[0] * ex.wdim[1]) + pos_out * double(dw.wdim[0]) * 9.0 +
+                   pos_out * double(pj.wdim[0] * pj.wdim[1]));
+        b += double(ex.wdim[0] * ex.wdim[1] + dw.wdim[0] * 9 + pj.wdim[0] * pj.wdim[1]);
         break;
     }
     default: break;

@@ -1,0 +1,499 @@
+// MobileNetV2's inverted residual block as ONE kernel on the int8 matrix cores:
+//   1x1 expansion (+ activation) -> depthwise 3x3, pads 1, stride 1 or 2 (+ activation) -> 1x1 projection
+//   (-> QLinearAdd with the block input).
+// Run layer by layer, the expanded tensors (6x the block input) cross HBM four times and every small layer pays a
+// kernel launch; here they live only in LDS and a block is one launch.  The arithmetic of each stage is exactly that
+// of the stand-alone kernels (exact int32 accumulation, the one f32 requantisation sequence, the activation as a
+// 256-entry table), so the fused block is bit-identical to running the three QLinearConv nodes one after another.
+//
+// A workgroup (4 wavefronts) walks tiles of NB images x TH output rows.  Per tile:
+//   A  the input patch ((TH-1)*stride+3 rows, W+2 columns, halo included) is copied into LDS, channel-blocked;
+//   B  expansion: wave w takes (32 patch positions) x (32 expanded channels) pairs, one v_mfma_i32_32x32x32_i8 per 32
+//      input channels, requantises and writes the bytes (value ^ 0x80) to the expanded patch in LDS;
+//   C  patch positions outside the image are overwritten with the depthwise zero point (they are its padding);
+//   D  depthwise + projection: wave w takes 32 output positions; per 32 expanded channels nine MFMAs with DIAGONAL
+//      weight matrices (row c = tap weight of channel c in column c) compute the depthwise sums of 32 positions x 32
+//      channels, the requantised bytes are exchanged between lanes p and p+32 so that each lane holds 16 consecutive
+//      channels of its position -- the B operand of the projection MFMA -- and the projection accumulates over the
+//      expanded channels in registers.  The result is requantised (and added to the block input) and stored.
+#include <algorithm>
+#include <cmath>
+#include <initializer_list>
+#include <type_traits>
+
+#include "quant_common.h"
+#include "quant_layout.h"
+
+namespace {
+
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+struct QBlockArgs {
+    int N, H, W, OH, OW, stride;
+    int CBin, Cin32, Ce32, CBo;        // input channel blocks (16) / chunks (32); expanded chunks; output blocks
+    int NB, TH, PH, PW, P, Ppad, Q;    // tile: images, output rows, patch rows / columns / positions, output positions
+    int n_row_tiles, n_tiles;
+    int o_xl, o_e, o_w1, o_w2, o_wdw, o_tab, o_ptab;  // LDS byte offsets
+    float zp1f, zp2f, zp3f;            // zero points of the three convolutions' own outputs
+    QAct act1, act2;
+    int has_act1, has_act2;
+    uint32_t pad_e4;                   // the depthwise input zero point ^ 0x80 in every byte
+    int has_res, fast_div;             // fast_div: the scales allow the unscaled division sequence
+    float ry_rcp;                      // refined reciprocal of ry_scale
+    float ra_scale, rb_scale, ry_scale;  // residual add: a = projection output, b = block input, y = sum
+    int ra_zp, rb_zp, ry_zp;
+};
+
+__device__ __forceinline__ i32x4 as_i32x4(const uint4 &v) {
+    i32x4 r;
+    r[0] = int(v.x); r[1] = int(v.y); r[2] = int(v.z); r[3] = int(v.w);
+    return r;
+}
+
+// s / y, correctly rounded.  The general f32 division scales its operands against overflow and underflow of the
+// intermediate terms, then runs reciprocal refinement and two residual corrections.  When the caller knows that no scaling
+// can be needed (|s| and y within 2^+-40), the refined reciprocal r is the same for every element and the rest is five
+// instructions with the same correctly rounded result.
+__device__ __forceinline__ float div_by(float s, float y, float r, int fast) {
+    if (!fast) return s / y;
+    const float q0 = s * r;
+    const float e0 = __builtin_fmaf(-y, q0, s);
+    const float q1 = __builtin_fmaf(e0, r, q0);
+    const float e1 = __builtin_fmaf(-y, q1, s);
+    return __builtin_fmaf(e1, r, q1);
+}
+
+template <int CO32, int MQ>
+__global__ void __launch_bounds__(256, CO32 <= 2 ? 2 : 1)  // wide projections need the whole CU's LDS anyway
+qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 *__restrict__ w1p,
+              const uint4 *__restrict__ w2p, const uint32_t *__restrict__ wm, const float *__restrict__ mult1,
+              const int32_t *__restrict__ corr1, const float *__restrict__ mult2, const int32_t *__restrict__ corr2,
+              const float *__restrict__ mult3, const int32_t *__restrict__ corr3, QBlockArgs a) {
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    uint8_t *lut1 = reinterpret_cast<uint8_t *>(lds), *lut2 = lut1 + 256;
+    uint4 *XL = reinterpret_cast<uint4 *>(lds + a.o_xl);   // [Cin32*2][Ppad] units of 16 channels
+    uint4 *E = reinterpret_cast<uint4 *>(lds + a.o_e);     // [Ce32*2][Ppad]
+    uint4 *W1 = reinterpret_cast<uint4 *>(lds + a.o_w1);   // [Cin32][Ce32][2][32] units
+    uint4 *W2 = reinterpret_cast<uint4 *>(lds + a.o_w2);   // [Ce32][CO32][2][32] units
+    uint32_t *WDW = reinterpret_cast<uint32_t *>(lds + a.o_wdw);  // [Ce/4][9][4] dwords
+    const int Ce = a.Ce32 * 32;
+    float *m1 = reinterpret_cast<float *>(lds + a.o_tab);
+    int *c1 = reinterpret_cast<int *>(m1 + Ce);
+    float *m2 = reinterpret_cast<float *>(c1 + Ce);
+    int *c2 = reinterpret_cast<int *>(m2 + Ce);
+    float *m3 = reinterpret_cast<float *>(c2 + Ce);
+    int *c3 = reinterpret_cast<int *>(m3 + CO32 * 32);
+    int *ptab = reinterpret_cast<int *>(lds + a.o_ptab);   // [P] image << 20 | patch row << 10 | patch column
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, lh = lane >> 5;
+
+    // ---- once per workgroup: tables and weights into LDS ----
+    {
+        const uint8_t b = uint8_t(tid);
+        lut1[tid] = uint8_t((a.has_act1 ? qact_apply(b, a.act1) : b) ^ 0x80);
+        lut2[tid] = uint8_t((a.has_act2 ? qact_apply(b, a.act2) : b) ^ 0x80);
+    }
+    for (int i = tid; i < a.Cin32 * a.Ce32 * 64; i += 256) W1[i] = w1p[i];
+    for (int i = tid; i < a.Ce32 * CO32 * 64; i += 256) W2[i] = w2p[i];
+    for (int i = tid; i < Ce * 9; i += 256) WDW[i] = wm[i];
+    for (int k = tid; k < Ce; k += 256) { m1[k] = mult1[k]; c1[k] = corr1[k]; m2[k] = mult2[k]; c2[k] = corr2[k]; }
+    for (int k = tid; k < CO32 * 32; k += 256) { m3[k] = mult3[k]; c3[k] = corr3[k]; }
+    {
+        const int patch = a.PH * a.PW;
+        const float inv_patch = 1.0f / float(patch), inv_pw = 1.0f / float(a.PW);
+        for (int p = tid; p < a.P; p += 256) {
+            const int img = small_div(p, patch, inv_patch), rem = p - img * patch;
+            const int ph = small_div(rem, a.PW, inv_pw), pw = rem - ph * a.PW;
+            ptab[p] = (img << 20) | (ph << 10) | pw;
+        }
+    }
+    __syncthreads();
+
+    const float inv_p = 1.0f / float(a.P), inv_nptiles = 1.0f / float(a.Ppad >> 5);
+    const float inv_tile_img = 1.0f / float(a.TH * a.OW), inv_ow = 1.0f / float(a.OW);
+    const int n_ptiles = a.Ppad >> 5, nq_tiles = (a.Q + 31) >> 5;
+    const uint4 pad_e = make_uint4(a.pad_e4, a.pad_e4, a.pad_e4, a.pad_e4);
+    // the diagonal element of row l32 lies in this lane's half of the columns; which dword of the 16-byte operand
+    const bool diag_mine = (l32 >> 4) == lh;
+    const int diag_q = (l32 >> 2) & 3;
+    const uint32_t dm0 = diag_mine && diag_q == 0 ? 0xffffffffu : 0u, dm1 = diag_mine && diag_q == 1 ? 0xffffffffu : 0u,
+                   dm2 = diag_mine && diag_q == 2 ? 0xffffffffu : 0u, dm3 = diag_mine && diag_q == 3 ? 0xffffffffu : 0u;
+
+    for (int tile = blockIdx.x; tile < a.n_tiles; tile += gridDim.x) {
+        const int ig = tile / a.n_row_tiles, rt = tile - ig * a.n_row_tiles;
+        const int n0 = ig * a.NB, oh0 = rt * a.TH, ih0 = oh0 * a.stride - 1;
+
+        // ---- A: input patch -> LDS (positions outside the image are left as they are: C overwrites what they yield) ----
+        for (int u = tid; u < a.CBin * a.P; u += 256) {
+            const int cb = small_div(u, a.P, inv_p), p = u - cb * a.P;
+            const int e = ptab[p];
+            const int n = n0 + (e >> 20), ih = ih0 + ((e >> 10) & 1023), iw = (e & 1023) - 1;
+            if (n < a.N && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W)
+                XL[cb * a.Ppad + p] = x[((int64_t(n) * a.CBin + cb) * a.H + ih) * int64_t(a.W) + iw];
+        }
+        __syncthreads();
+
+        // ---- B: expansion.  A wave keeps one block of 32 expanded channels (its multipliers, corrections and, for one
+        // chunk of input channels, its weights) in registers and walks the position tiles with it. ----
+        {
+            // (channel block, position tile) units in channel-block-major order, split evenly over the four waves
+            const int units = a.Ce32 * n_ptiles, u_begin = (units * wave) >> 2, u_end = (units * (wave + 1)) >> 2;
+            int kb = small_div(u_begin, n_ptiles, inv_nptiles), ptile = u_begin - kb * n_ptiles;
+            for (int u = u_begin; u < u_end;) {
+                const int kch = kb * 32 + lh * 4;
+                i32x16 cvec;
+                float mv[16];
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    cvec[v] = c1[kch + (v >> 2) * 8 + (v & 3)];
+                    mv[v] = m1[kch + (v >> 2) * 8 + (v & 3)];
+                }
+                const i32x4 wa0 = as_i32x4(W1[kb * 64 + lh * 32 + l32]);
+                char *erow = reinterpret_cast<char *>(E) + (kb * 2 * a.Ppad + l32) * 16 + lh * 8;
+                for (; ptile < n_ptiles && u < u_end; ++ptile, ++u) {
+                    const int p = ptile * 32 + l32;
+                    i32x16 acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wa0, as_i32x4(XL[lh * a.Ppad + p]), cvec, 0, 0, 0);
+                    for (int chunk = 1; chunk < a.Cin32; ++chunk)
+                        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(as_i32x4(W1[(chunk * a.Ce32 + kb) * 64 + lh * 32 + l32]),
+                                                                    as_i32x4(XL[(2 * chunk + lh) * a.Ppad + p]), acc, 0, 0, 0);
+                    uint32_t d[4];
+#pragma unroll
+                    for (int gq = 0; gq < 4; ++gq) {
+                        uint32_t o = 0;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            o |= uint32_t(lut1[sat_u8_rne_finite(float(acc[gq * 4 + e]) * mv[gq * 4 + e], a.zp1f)]) << (8 * e);
+                        d[gq] = o;
+                    }
+                    // lanes p and p + 32 exchange one dword per 16-channel block so that each writes 8 consecutive bytes
+#pragma unroll
+                    for (int b = 0; b < 2; ++b) {
+                        const uint32_t send = lh ? d[2 * b] : d[2 * b + 1];
+                        const uint32_t recv = uint32_t(__shfl_xor(int(send), 32, 64));
+                        const uint2 out = lh ? make_uint2(recv, d[2 * b + 1]) : make_uint2(d[2 * b], recv);
+                        *reinterpret_cast<uint2 *>(erow + (b * a.Ppad + ptile * 32) * 16) = out;
+                    }
+                }
+                ptile = 0;
+                ++kb;
+            }
+        }
+        __syncthreads();
+
+        // ---- C: the depthwise convolution's padding ----
+        for (int p = tid; p < a.P; p += 256) {
+            const int e = ptab[p];
+            const int ih = ih0 + ((e >> 10) & 1023), pw = e & 1023;
+            if (pw == 0 || pw == a.PW - 1 || ih < 0 || ih >= a.H)
+                for (int cb = 0; cb < a.Ce32 * 2; ++cb) E[cb * a.Ppad + p] = pad_e;
+        }
+        __syncthreads();
+
+        // ---- D: depthwise 3x3 + projection.  A wave takes MQ tiles of 32 output positions at a time; per chunk of 32
+        // expanded channels the nine diagonal operands and the requantisation tables are set up once for all of them. ----
+        const int q_per_wave = (nq_tiles + 3) >> 2, q_end = min(nq_tiles, (wave + 1) * q_per_wave);
+        for (int q0 = wave * q_per_wave; q0 < q_end; q0 += MQ) {
+            int p0[MQ], qimg[MQ], qr[MQ], qc[MQ];
+            bool qvalid[MQ];
+#pragma unroll
+            for (int j = 0; j < MQ; ++j) {
+                const int q = (q0 + j) * 32 + l32;
+                qvalid[j] = q0 + j < q_end && q < a.Q;
+                const int qq = qvalid[j] ? q : 0;
+                qimg[j] = small_div(qq, a.TH * a.OW, inv_tile_img);
+                const int rem = qq - qimg[j] * a.TH * a.OW;
+                qr[j] = small_div(rem, a.OW, inv_ow);
+                qc[j] = rem - qr[j] * a.OW;
+                p0[j] = (qimg[j] * a.PH + qr[j] * a.stride) * a.PW + qc[j] * a.stride;  // top-left tap in the patch
+            }
+            i32x16 acc3[MQ][CO32];
+#pragma unroll
+            for (int kb3 = 0; kb3 < CO32; ++kb3)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int cv = c3[kb3 * 32 + lh * 4 + (v >> 2) * 8 + (v & 3)];
+#pragma unroll
+                    for (int j = 0; j < MQ; ++j) acc3[j][kb3][v] = cv;
+                }
+            for (int ch = 0; ch < a.Ce32; ++ch) {
+                const int kch = ch * 32 + lh * 4;
+                i32x16 cvec;
+                float mv[16];
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    cvec[v] = c2[kch + (v >> 2) * 8 + (v & 3)];
+                    mv[v] = m2[kch + (v >> 2) * 8 + (v & 3)];
+                }
+                const uint32_t *wk = WDW + ((ch * 32 + l32) >> 2) * 36 + (l32 & 3);
+                i32x4 wa[9];
+#pragma unroll
+                for (int t = 0; t < 9; ++t) {
+                    const uint32_t wd = wk[t * 4];
+                    wa[t][0] = int(wd & dm0); wa[t][1] = int(wd & dm1); wa[t][2] = int(wd & dm2); wa[t][3] = int(wd & dm3);
+                }
+                i32x4 w2a[CO32];
+#pragma unroll
+                for (int kb3 = 0; kb3 < CO32; ++kb3) w2a[kb3] = as_i32x4(W2[(ch * CO32 + kb3) * 64 + lh * 32 + l32]);
+#pragma unroll
+                for (int j = 0; j < MQ; ++j) {
+                    const uint4 *ep = E + (2 * ch + lh) * a.Ppad + p0[j];
+                    i32x16 acc2 = __builtin_amdgcn_mfma_i32_32x32x32_i8(wa[0], as_i32x4(ep[0]), cvec, 0, 0, 0);
+#pragma unroll
+                    for (int t = 1; t < 9; ++t)
+                        acc2 = __builtin_amdgcn_mfma_i32_32x32x32_i8(wa[t], as_i32x4(ep[(t / 3) * a.PW + (t % 3)]), acc2, 0, 0, 0);
+                    uint32_t d[4];
+#pragma unroll
+                    for (int gq = 0; gq < 4; ++gq) {
+                        uint32_t o = 0;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            o |= uint32_t(lut2[sat_u8_rne_finite(float(acc2[gq * 4 + e]) * mv[gq * 4 + e], a.zp2f)]) << (8 * e);
+                        d[gq] = o;
+                    }
+                    // lane (p, 0) gathers channels 0..15 of the chunk, lane (p, 1) channels 16..31
+                    const uint32_t r0 = uint32_t(__shfl_xor(int(lh ? d[0] : d[2]), 32, 64));
+                    const uint32_t r1 = uint32_t(__shfl_xor(int(lh ? d[1] : d[3]), 32, 64));
+                    i32x4 db;
+                    db[0] = int(lh ? r0 : d[0]); db[1] = int(lh ? d[2] : r0);
+                    db[2] = int(lh ? r1 : d[1]); db[3] = int(lh ? d[3] : r1);
+#pragma unroll
+                    for (int kb3 = 0; kb3 < CO32; ++kb3)
+                        acc3[j][kb3] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w2a[kb3], db, acc3[j][kb3], 0, 0, 0);
+                }
+            }
+            auto store_tiles = [&](auto res_tag, auto fast_tag) {
+                constexpr bool RES = decltype(res_tag)::value, FAST = decltype(fast_tag)::value;
+#pragma unroll
+                for (int j = 0; j < MQ; ++j) {
+                    const int n = n0 + qimg[j], oh = oh0 + qr[j];
+                    const bool ok = qvalid[j] && n < a.N && oh < a.OH;
+#pragma unroll
+                    for (int kb3 = 0; kb3 < CO32; ++kb3) {
+#pragma unroll
+                        for (int gq = 0; gq < 4; ++gq) {
+                            const int cbq = kb3 * 2 + (gq >> 1);
+                            const bool st = ok && cbq < a.CBo;
+                            const int64_t off = (((int64_t(n) * a.CBo + cbq) * a.OH + oh) * int64_t(a.OW) + qc[j]) * 16 + (gq & 1) * 8 + lh * 4;
+                            uint32_t xr = 0;
+                            if (RES && st)
+                                xr = *reinterpret_cast<const uint32_t *>(reinterpret_cast<const char *>(x) + off) ^ 0x80808080u;
+                            uint32_t o = 0;
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                uint32_t v = sat_u8_rne_finite(float(acc3[j][kb3][gq * 4 + e]) * m3[kb3 * 32 + gq * 8 + lh * 4 + e], a.zp3f);
+                                if (RES) {
+                                    const float fa = float(int(v) - a.ra_zp) * a.ra_scale;
+                                    const float fb = float(int((xr >> (8 * e)) & 0xffu) - a.rb_zp) * a.rb_scale;
+                                    // finite operands: the saturating conversion replaces the clamp
+                                    v = FAST ? sat_u8_rne_finite(div_by(fa + fb, a.ry_scale, a.ry_rcp, 1), float(a.ry_zp))
+                                             : uint32_t(sat_u8_rne((fa + fb) / a.ry_scale, uint8_t(a.ry_zp)));
+                                }
+                                o |= v << (8 * e);
+                            }
+                            if (st) *reinterpret_cast<uint32_t *>(y + off) = o ^ 0x80808080u;
+                        }
+                    }
+                }
+            };
+            if (!a.has_res) store_tiles(std::false_type(), std::false_type());
+            else if (a.fast_div) store_tiles(std::true_type(), std::true_type());
+            else store_tiles(std::true_type(), std::false_type());
+        }
+        __syncthreads();  // the next tile overwrites the patches
+    }
+}
+
+size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
+size_t align16(size_t v) { return (v + 15) & ~size_t(15); }
+
+bool conv1x1(const zant_qconv_desc *d) { return d && d->K > 0 && d->C > 0 && (d->n_wscale == 1 || d->n_wscale == d->K); }
+
+}  // namespace
+
+int zant_qblock_blocked(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], const zant_qconv_desc *expand,
+                        const zant_qconv_desc *dw, int64_t dw_stride, const zant_qconv_desc *project, int residual,
+                        float add_scale, int add_zp, uint8_t *y, const int64_t ydim[4], bool query_only, zant_pack_slot *slot) {
+    if (!ctx || !xdim || !ydim || !expand || !dw || !project) return ZANT_NullPointer;
+    if (!conv1x1(expand) || !conv1x1(dw) || !conv1x1(project)) return 1;
+    const int64_t N = xdim[0], Cin = xdim[1], H = xdim[2], W = xdim[3];
+    const int64_t Ce = expand->K, Co = project->K;
+    if (N <= 0 || H <= 0 || W <= 0 || expand->C != Cin || dw->C != Ce || dw->K != Ce || project->C != Ce) return 1;
+    if (dw_stride != 1 && dw_stride != 2) return 1;
+    const int64_t OH = (H + 2 - 3) / dw_stride + 1, OW = (W + 2 - 3) / dw_stride + 1;
+    if (ydim[0] != N || ydim[1] != Co || ydim[2] != OH || ydim[3] != OW) return 1;
+    if (residual && (Co != Cin || OH != H || OW != W)) return 1;
+    if (Cin > 512 || Ce > 2048 || Co > 128 || W + 2 > 1023 || N > INT32_MAX / 2) return 1;
+    if (N * ((Cin + 15) / 16) * H * W >= (int64_t(1) << 27) || N * ((Co + 15) / 16) * OH * OW >= (int64_t(1) << 27)) return 1;
+
+    QBlockArgs a;
+    a.N = int(N); a.H = int(H); a.W = int(W); a.OH = int(OH); a.OW = int(OW); a.stride = int(dw_stride);
+    a.CBin = int((Cin + 15) / 16); a.Cin32 = int((Cin + 31) / 32); a.Ce32 = int((Ce + 31) / 32); a.CBo = int((Co + 15) / 16);
+    const int CO32 = int((Co + 31) / 32), CeP = a.Ce32 * 32;
+    a.PW = int(W) + 2;
+    // LDS: fixed part, then per patch position the input and expanded bytes and one table entry
+    const size_t w1_bytes = size_t(a.Cin32) * a.Ce32 * 1024, w2_bytes = size_t(a.Ce32) * CO32 * 1024;
+    const size_t wdw_bytes = size_t(CeP) * 9 * 4, tab_bytes = (size_t(CeP) * 4 + size_t(CO32) * 32 * 2) * 4;
+    const size_t fixed = 512 + w1_bytes + w2_bytes + wdw_bytes + tab_bytes;
+    if (CO32 > 4) return 1;
+    // Tile = NB whole images, or TH output rows of one image.  Among the shapes that fit -- in half a CU's LDS first, so
+    // that two workgroups share a CU -- the one with the fewest wave instructions per image by a model of the kernel's
+    // stages: B works on (32 positions x 32 expanded channels) units split over 4 waves, D on tiles of 32 output
+    // positions, MQ at a time per wave; partly filled units and the halo rows cost as much as full ones.
+    const int mq_cap = CO32 == 1 ? 4 : CO32 == 2 ? 2 : 1;
+    const int64_t p_img = ((OH - 1) * dw_stride + 3) * a.PW;
+    auto lds_for = [&](int64_t P) {
+        const int64_t Ppad = (P + 31) & ~int64_t(31);
+        return size_t(512) + size_t(a.Cin32 * 2 + a.Ce32 * 2) * size_t(Ppad) * 16 + w1_bytes + w2_bytes + wdw_bytes + tab_bytes +
+               align16(size_t(P) * 4);
+    };
+    auto tile_cost = [&](int64_t P, int64_t Q) {
+        const int64_t b_units = int64_t(a.Ce32) * ((P + 31) / 32), nq = (Q + 31) / 32, qpw = (nq + 3) / 4;
+        const int64_t rounds = (qpw + mq_cap - 1) / mq_cap, mq = (qpw + rounds - 1) / rounds;
+        const double epi = residual ? 350.0 : 150.0;
+        return double((b_units + 3) / 4) * 150.0 + double(rounds) * (a.Ce32 * (100.0 + mq * 170.0) + mq * epi) +
+               double(P) * (a.CBin + a.Ce32 * 2) / 256.0 * 15.0 + 300.0;
+    };
+    bool found = false;
+    size_t cap_used = 0;
+    // 76 KB: what two workgroups per CU leave each other after the allocation granularity
+    for (size_t cap : {size_t(76 * 1024), size_t(160 * 1024)}) {
+        const int64_t slots = int64_t(ctx->num_cus) * (cap <= 80 * 1024 ? 2 : 1);
+        double best = 0.0;
+        int bNB = 0, bTH = 0;
+        if (lds_for(p_img) <= cap) {
+            for (int64_t nb = 1; nb <= std::min<int64_t>(N, 2047) && lds_for(nb * p_img) <= cap; ++nb) {
+                const int64_t tiles = (N + nb - 1) / nb, waves = (tiles + slots - 1) / slots;
+                const double c = tile_cost(nb * p_img, nb * OH * OW) * double(waves);  // time of the busiest workgroup slot
+                if (!bNB || c < best * 0.98) { best = c; bNB = int(nb); bTH = int(OH); }
+            }
+        } else {
+            for (int64_t th = 1; th <= OH; ++th) {
+                const int64_t P = ((th - 1) * dw_stride + 3) * a.PW;
+                if (lds_for(P) > cap) break;
+                const int64_t nrt = (OH + th - 1) / th;
+                if ((OH + nrt - 1) / nrt != th) continue;  // only evened-out row tiles
+                const int64_t tiles = N * nrt, waves = (tiles + slots - 1) / slots;
+                const double c = tile_cost(P, th * OW) * double(waves);
+                if (!bNB || c < best * 0.98) { best = c; bNB = 1; bTH = int(th); }
+            }
+            if (bNB && bTH < std::min<int64_t>(OH, 4) && cap < 160 * 1024) bNB = 0;  // too much halo: take the whole CU's LDS
+        }
+        if (!bNB) continue;
+        a.NB = bNB; a.TH = bTH;
+        a.PH = (bTH - 1) * int(dw_stride) + 3;
+        if (a.PH > 1023) continue;
+        a.P = bNB * a.PH * a.PW;
+        a.Ppad = (a.P + 31) & ~31;
+        a.Q = bNB * bTH * int(OW);
+        a.n_row_tiles = int((OH + bTH - 1) / bTH);
+        const int64_t n_tiles = ((N + bNB - 1) / bNB) * a.n_row_tiles;
+        if (n_tiles > INT32_MAX || a.P >= (1 << 20) || a.Q >= (1 << 20)) continue;
+        a.n_tiles = int(n_tiles);
+        size_t o = 512;
+        a.o_xl = int(o); o += size_t(a.Cin32) * 2 * a.Ppad * 16;
+        a.o_e = int(o); o += size_t(a.Ce32) * 2 * a.Ppad * 16;
+        a.o_w1 = int(o); o += w1_bytes;
+        a.o_w2 = int(o); o += w2_bytes;
+        a.o_wdw = int(o); o += wdw_bytes;
+        a.o_tab = int(o); o += tab_bytes;
+        a.o_ptab = int(o); o += align16(size_t(a.P) * 4);
+        if (o > cap) continue;
+        cap_used = o;
+        found = true;
+        break;
+    }
+    if (!found) return 1;
+    if (query_only) return ZANT_OK;
+    if (!x || !y || !expand->w || !expand->w_scale || !dw->w || !dw->w_scale || !project->w || !project->w_scale)
+        return ZANT_NullPointer;
+
+    // packed weights and tables of the three convolutions
+    const size_t kp1 = size_t(CeP), kp3 = size_t(CO32) * 32;
+    const size_t o_w1p = 256, o_m1 = o_w1p + align256(w1_bytes), o_c1 = o_m1 + align256(kp1 * 4), o_w2p = o_c1 + align256(kp1 * 4),
+                 o_m3 = o_w2p + align256(w2_bytes), o_c3 = o_m3 + align256(kp3 * 4), o_wm = o_c3 + align256(kp3 * 4),
+                 o_m2 = o_wm + align256(wdw_bytes), o_c2 = o_m2 + align256(kp1 * 4), static_bytes = o_c2 + align256(kp1 * 4);
+    void *ws = nullptr, *dyn = nullptr;
+    bool need_pack = true;
+    int parity = 0;
+    int rc = zant_pack_region(ctx, slot, static_bytes, 0, &ws, &dyn, &need_pack, &parity);
+    if (rc) return rc;
+    char *base = static_cast<char *>(ws);
+    int8_t *w1p = reinterpret_cast<int8_t *>(base + o_w1p), *w2p = reinterpret_cast<int8_t *>(base + o_w2p);
+    float *m1 = reinterpret_cast<float *>(base + o_m1), *m2 = reinterpret_cast<float *>(base + o_m2),
+          *m3 = reinterpret_cast<float *>(base + o_m3);
+    int32_t *c1 = reinterpret_cast<int32_t *>(base + o_c1), *c2 = reinterpret_cast<int32_t *>(base + o_c2),
+            *c3 = reinterpret_cast<int32_t *>(base + o_c3);
+    uint32_t *wmk = reinterpret_cast<uint32_t *>(base + o_wm);
+    if (need_pack) {
+        int8_t *padvec = reinterpret_cast<int8_t *>(base + 16);
+        int *word = reinterpret_cast<int *>(base);
+        rc = zant_qpack_dense(ctx, expand->w, expand->w_scale, expand->n_wscale, expand->bias, int(Ce), int(Cin), 1, 32,
+                              expand->x_scale, expand->x_zp, expand->y_scale, w1p, m1, c1, padvec, word);
+        if (rc) return rc;
+        rc = zant_qpack_depthwise(ctx, dw->w, dw->w_scale, dw->n_wscale, dw->bias, int(Ce), CeP, dw->x_scale, dw->x_zp,
+                                  dw->y_scale, wmk, m2, c2);
+        if (rc) return rc;
+        rc = zant_qpack_dense(ctx, project->w, project->w_scale, project->n_wscale, project->bias, int(Co), int(Ce), 1, 32,
+                              project->x_scale, project->x_zp, project->y_scale, w2p, m3, c3, padvec + 16, word);
+        if (rc) return rc;
+    }
+
+    a.zp1f = float(expand->y_zp); a.zp2f = float(dw->y_zp); a.zp3f = float(project->y_zp);
+    a.has_act1 = expand->act != ZANT_ACT_NONE;
+    a.act1.act = expand->act; a.act1.alpha = expand->act_alpha; a.act1.in_scale = expand->y_scale; a.act1.in_zp = expand->y_zp;
+    a.act1.out_scale = expand->act_scale; a.act1.out_zp = uint8_t(expand->act_zp);
+    a.has_act2 = dw->act != ZANT_ACT_NONE;
+    a.act2.act = dw->act; a.act2.alpha = dw->act_alpha; a.act2.in_scale = dw->y_scale; a.act2.in_zp = dw->y_zp;
+    a.act2.out_scale = dw->act_scale; a.act2.out_zp = uint8_t(dw->act_zp);
+    a.pad_e4 = uint32_t((dw->x_zp ^ 0x80) & 0xff) * 0x01010101u;
+    a.has_res = residual ? 1 : 0;
+    a.ra_scale = project->y_scale; a.ra_zp = project->y_zp;
+    a.rb_scale = expand->x_scale; a.rb_zp = expand->x_zp;
+    a.ry_scale = add_scale; a.ry_zp = add_zp;
+    {
+        // |fa + fb| <= 256 * (a_scale + b_scale); all three scales far inside the range where f32 division needs no scaling
+        auto tame = [](float v) { return v > 1e-9f && v < 1e9f; };
+        a.fast_div = residual && tame(a.ra_scale) && tame(a.rb_scale) && tame(add_scale);
+        float r = 0.0f;
+        if (a.fast_div) {
+            const volatile float r0 = 1.0f / add_scale;  // correctly rounded: at least as good a seed as the hardware estimate
+            r = std::fmaf(std::fmaf(-add_scale, r0, 1.0f), r0, r0);
+        }
+        a.ry_rcp = r;
+    }
+
+    const int per_cu = cap_used <= 76 * 1024 ? 2 : 1;
+    const int grid = int(std::min<int64_t>(a.n_tiles, int64_t(ctx->num_cus) * per_cu));
+    KernelTimer kt(ctx);
+    // position tiles a wave handles together in stage D: what its share of the tile needs, within the register budget
+    const int nq_tiles = (a.Q + 31) / 32;
+    const int q_per_wave = (nq_tiles + 3) / 4;
+    const int rounds = (q_per_wave + mq_cap - 1) / mq_cap;
+    const int MQv = std::max(1, (q_per_wave + rounds - 1) / rounds);
+#define ZANT_QBLOCK_LAUNCH(CO, M)                                                                                           \
+    do {                                                                                                                    \
+        static bool attr_set = false;                                                                                       \
+        if (!attr_set) {                                                                                                    \
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&qblock_kernel<CO, M>),                               \
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                             \
+            attr_set = true;                                                                                                \
+        }                                                                                                                   \
+        hipLaunchKernelGGL((qblock_kernel<CO, M>), dim3(grid), dim3(256), cap_used, ctx->stream,                           \
+                           reinterpret_cast<const uint4 *>(x), y, reinterpret_cast<const uint4 *>(w1p),                    \
+                           reinterpret_cast<const uint4 *>(w2p), wmk, m1, c1, m2, c2, m3, c3, a);                          \
+    } while (0)
+    switch (CO32 * 10 + MQv) {
+    case 11: ZANT_QBLOCK_LAUNCH(1, 1); break;
+    case 12: ZANT_QBLOCK_LAUNCH(1, 2); break;
+    case 13: ZANT_QBLOCK_LAUNCH(1, 3); break;
+    case 14: ZANT_QBLOCK_LAUNCH(1, 4); break;
+    case 21: ZANT_QBLOCK_LAUNCH(2, 1); break;
+    case 22: ZANT_QBLOCK_LAUNCH(2, 2); break;
+    case 31: ZANT_QBLOCK_LAUNCH(3, 1); break;
+    default: ZANT_QBLOCK_LAUNCH(4, 1); break;
+    }
+#undef ZANT_QBLOCK_LAUNCH
+    ZANT_LAUNCH_CHECK(ctx);
+    return ZANT_OK;
+}

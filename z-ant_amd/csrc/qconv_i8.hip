@@ -237,16 +237,6 @@ __device__ __forceinline__ void lds_wait16(uint32_t (&v)[16]) {
                    "+v"(v[9]), "+v"(v[10]), "+v"(v[11]), "+v"(v[12]), "+v"(v[13]), "+v"(v[14]), "+v"(v[15]));
 }
 
-// p / d for 0 <= p < 2^20 and d > 0, with inv = 1.0f / d: the float quotient is off by at most one, which the
-// remainder corrects.  Far fewer instructions than the general 32-bit division sequence.
-__device__ __forceinline__ int small_div(int p, int d, float inv) {
-    int q = int(float(p) * inv);
-    const int r = p - q * d;
-    q += r >= d ? 1 : 0;
-    q -= r < 0 ? 1 : 0;
-    return q;
-}
-
 // Waits until at most n of this wave's vector-memory operations are outstanding (n is wave-uniform, 0..63).
 __device__ __forceinline__ void wait_vmcnt(int n) {
 #define ZANT_VM(k) case k: __builtin_amdgcn_s_waitcnt(((k) & 15) | (((k) >> 4) << 14) | 0x0F70); break;
@@ -1055,6 +1045,26 @@ int run_qdw_blocked(zant_ctx *ctx, const uint8_t *xb, const int8_t *w, const flo
 }
 
 }  // namespace
+
+int zant_qpack_dense(zant_ctx *ctx, const int8_t *w, const float *w_scale, int64_t n_wscale, const int32_t *bias, int K, int C,
+                     int T, int k_blk, float x_scale, int x_zp, float y_scale, int8_t *wp, float *mult, int32_t *corr,
+                     int8_t *padvec, int *scratch_word) {
+    const int n_chunks = (C + QCC - 1) / QCC, n_kblocks = (K + k_blk - 1) / k_blk;
+    const int64_t wp_bytes = int64_t(n_chunks) * n_kblocks * T * QCC * k_blk, kpad = int64_t(n_kblocks) * k_blk;
+    const unsigned pb = unsigned(std::min<int64_t>(std::max<int64_t>(ceil_div64(wp_bytes, 256), ceil_div64(kpad, 4)), 1024));
+    hipLaunchKernelGGL(qpack_kernel, dim3(pb), dim3(256), 0, ctx->stream, w, w_scale, bias, wp, mult, corr, padvec, scratch_word,
+                       0, K, C, T, n_chunks, n_kblocks, k_blk, x_scale, y_scale, x_zp, int(n_wscale));
+    ZANT_LAUNCH_CHECK(ctx);
+    return ZANT_OK;
+}
+
+int zant_qpack_depthwise(zant_ctx *ctx, const int8_t *w, const float *w_scale, int64_t n_wscale, const int32_t *bias, int K,
+                         int kpad, float x_scale, int x_zp, float y_scale, uint32_t *wm, float *mult, int32_t *corr) {
+    hipLaunchKernelGGL(qdw_pack_kernel, dim3((kpad + 255) / 256), dim3(256), 0, ctx->stream, w, w_scale, bias, wm, mult, corr, K,
+                       kpad, x_scale, y_scale, x_zp, int(n_wscale));
+    ZANT_LAUNCH_CHECK(ctx);
+    return ZANT_OK;
+}
 
 int zant_to_blocked(zant_ctx *ctx, const uint8_t *x, int64_t N, int64_t C, int64_t HW, uint8_t *xb) {
     if (!ctx) return ZANT_NullPointer;

@@ -41,3 +41,13 @@ __device__ __forceinline__ uint8_t qact_apply(uint8_t q, const QAct &a) {
     const float v = act_f32(float(int(q) - a.in_zp) * a.in_scale, a.act, a.alpha);
     return sat_u8_rne(v / a.out_scale, a.out_zp);
 }
+
+// p / d for 0 <= p < 2^20 and d > 0, with inv = 1.0f / d: the float quotient is off by at most one, which the
+// remainder corrects.  Far fewer instructions than the general 32-bit division sequence.
+__device__ __forceinline__ int small_div(int p, int d, float inv) {
+    int q = int(float(p) * inv);
+    const int r = p - q * d;
+    q += r >= d ? 1 : 0;
+    q -= r < 0 ? 1 : 0;
+    return q;
+}

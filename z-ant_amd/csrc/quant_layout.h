@@ -42,3 +42,36 @@ int zant_qlinear_add_flip(zant_ctx *ctx, const uint8_t *a, float a_scale, uint8_
 // Global average pool of a blocked tensor; y is [N, C, 1, 1] in y_layout.
 int zant_qgap_blocked(zant_ctx *ctx, const uint8_t *xb, const int64_t xdim[4], float x_scale, uint8_t x_zp, float y_scale,
                       uint8_t y_zp, uint8_t *y, int y_layout);
+
+// Weight packing shared by the int8 matrix-core kernels (device pointers; launches on the context's stream).
+// Dense: [chunk of 32 input channels][block of k_blk output channels][tap][half][k_blk][16] int8, zero padded; per
+// output channel the requantisation multiplier (x_scale * w_scale / y_scale) and the integer correction
+// (bias + (128 - x_zp) * sum of weights); padvec = 16 bytes of x_zp - 128; scratch_word: one int that gets cleared.
+int zant_qpack_dense(zant_ctx *ctx, const int8_t *w, const float *w_scale, int64_t n_wscale, const int32_t *bias, int K, int C,
+                     int T, int k_blk, float x_scale, int x_zp, float y_scale, int8_t *wp, float *mult, int32_t *corr,
+                     int8_t *padvec, int *scratch_word);
+// Depthwise 3x3: one dword per (channel, tap) with the weight in byte (channel % 4) and zeros elsewhere, at
+// wm[((channel / 4) * 9 + tap) * 4 + channel % 4]; multipliers and corrections as above, for kpad channels.
+int zant_qpack_depthwise(zant_ctx *ctx, const int8_t *w, const float *w_scale, int64_t n_wscale, const int32_t *bias, int K,
+                         int kpad, float x_scale, int x_zp, float y_scale, uint32_t *wm, float *mult, int32_t *corr);
+
+// One QLinearConv of a fused block: weights, requantisation and the optional fused activation (conv output quantised
+// with y_scale / y_zp, the activation's output with act_scale / act_zp).
+struct zant_qconv_desc {
+    const int8_t *w;
+    const float *w_scale;
+    int64_t n_wscale;
+    const int32_t *bias;
+    int64_t K, C;          // output channels, input channels (depthwise: C == K)
+    float x_scale; int x_zp;
+    float y_scale; int y_zp;
+    int act; float act_alpha; float act_scale; int act_zp;
+};
+
+// MobileNetV2's inverted residual block in one kernel, on blocked tensors: 1x1 expansion (+activation) -> depthwise 3x3,
+// pads 1, stride 1 or 2 (+activation) -> 1x1 projection (-> QLinearAdd with the block input when `residual`).  The
+// expanded tensors live only in LDS.  query_only: report eligibility (ZANT_OK / 1) without touching pointers.
+// residual: y = sat(rne(((p - p_zp) * p_scale + (x - x_zp) * x_scale) / add_scale) + add_zp), p the projection output.
+int zant_qblock_blocked(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], const zant_qconv_desc *expand,
+                        const zant_qconv_desc *dw, int64_t dw_stride, const zant_qconv_desc *project, int residual,
+                        float add_scale, int add_zp, uint8_t *y, const int64_t ydim[4], bool query_only, zant_pack_slot *slot);
