@@ -82,6 +82,15 @@ int launch_unary(zant_ctx *ctx, const float *x, float *y, int64_t n, float slope
     return ZANT_OK;
 }
 
+// p / d for 0 <= p < 2^20, d > 0, inv = 1.0f / d (the float quotient is off by at most one; the remainder corrects it).
+__device__ __forceinline__ int small_div_host(int p, int d, float inv) {
+    int q = int(float(p) * inv);
+    const int r = p - q * d;
+    q += r >= d ? 1 : 0;
+    q -= r < 0 ? 1 : 0;
+    return q;
+}
+
 // ---- softmax: one wavefront per row ------------------------------------------------------------
 
 __device__ __forceinline__ float wave_max(float v) {
@@ -113,6 +122,45 @@ __global__ void __launch_bounds__(kThreads) softmax_f32_kernel(const float *__re
         s = wave_sum(s);
         for (int64_t j = lane; j < cols; j += 64) yr[j] = yr[j] / s;
     }
+}
+
+// Rows of at most 16 values: one thread per row, the row in registers (a wavefront per row would leave most lanes
+// idle).  A workgroup's 256 rows are one contiguous span: it crosses HBM as whole 16-byte vectors into LDS and back,
+// and each thread picks its row out of LDS.  Sequential max / sum over the row, in column order like the reference.
+__global__ void __launch_bounds__(kThreads) softmax_small_f32_kernel(const float *__restrict__ x, float *__restrict__ y,
+                                                                    int64_t rows, int cols, int vec) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    __shared__ __attribute__((aligned(16))) float buf[kThreads * 16];
+    const int64_t row0 = int64_t(blockIdx.x) * kThreads;
+    const int nrows = int(min(int64_t(kThreads), rows - row0)), nel = nrows * cols;
+    const float *xb = x + row0 * cols;
+    float *yb = y + row0 * cols;
+    const int nvec = vec ? nel >> 2 : 0;
+    for (int i = threadIdx.x; i < nvec; i += kThreads) reinterpret_cast<f4 *>(buf)[i] = __builtin_nontemporal_load(reinterpret_cast<const f4 *>(xb) + i);
+    for (int i = (nvec << 2) + threadIdx.x; i < nel; i += kThreads) buf[i] = xb[i];
+    __syncthreads();
+    if (int(threadIdx.x) < nrows) {
+        float *row = buf + threadIdx.x * cols;
+        float v[16];
+        float m = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            v[j] = j < cols ? row[j] : -INFINITY;
+            m = fmaxf(m, v[j]);
+        }
+        float sum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            v[j] = j < cols ? expf(v[j] - m) : 0.0f;
+            sum += v[j];
+        }
+#pragma unroll
+        for (int j = 0; j < 16; ++j)
+            if (j < cols) row[j] = v[j] / sum;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < nvec; i += kThreads) __builtin_nontemporal_store(reinterpret_cast<const f4 *>(buf)[i], reinterpret_cast<f4 *>(yb) + i);
+    for (int i = (nvec << 2) + threadIdx.x; i < nel; i += kThreads) yb[i] = buf[i];
 }
 
 // ---- add ----------------------------------------------------------------------------------------
@@ -169,6 +217,31 @@ __global__ void __launch_bounds__(kThreads) add_bcast_f32_kernel(const float *__
             ib += pos * g.sb[d];
         }
         y[i] = a[ia] + b[ib];
+    }
+}
+
+// One operand has the output's shape, the other a single axis of length C and ones elsewhere (a per-channel term):
+// y[i] = big[i] + small[(i / inner) % C].  With inner a multiple of 4 the four floats of a vector share a channel.
+__global__ void __launch_bounds__(kThreads) add_channel_f32_kernel(const float *__restrict__ big, const float *__restrict__ small,
+                                                                  float *__restrict__ y, uint32_t n4, uint32_t inner4, uint32_t C) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    const uint32_t base = blockIdx.x * (kThreads * ZANT_STREAM_U) + threadIdx.x;
+    const f4 *b4 = reinterpret_cast<const f4 *>(big);
+    f4 *y4 = reinterpret_cast<f4 *>(y);
+    f4 v[ZANT_STREAM_U];
+    float c[ZANT_STREAM_U];
+#pragma unroll
+    for (int u = 0; u < ZANT_STREAM_U; ++u) {
+        const uint32_t j = base + u * kThreads;
+        if (j < n4) {
+            v[u] = __builtin_nontemporal_load(b4 + j);
+            c[u] = small[(j / inner4) % C];
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < ZANT_STREAM_U; ++u) {
+        const uint32_t j = base + u * kThreads;
+        if (j < n4) __builtin_nontemporal_store(v[u] + c[u], y4 + j);
     }
 }
 
@@ -244,6 +317,80 @@ __global__ void __launch_bounds__(kThreads) maxpool_2x2s2_kernel(const T *__rest
     }
 }
 
+// 2x2 / stride 2 with even rows of inputs read as vectors: a thread turns two row segments of 2 * VEC inputs into VEC
+// outputs (f32: VEC = 1, two 8-byte loads; u8: VEC = 8, two 16-byte loads, one 8-byte store).  A workgroup covers
+// kThreads * ZANT_STREAM_U consecutive output vectors of the flattened [NC * OH, OW / VEC] grid and issues all its
+// loads before its stores, nontemporal both ways (the streaming pattern of the elementwise kernels).  Needs W even
+// (f32) or a multiple of 16 (u8), OW a multiple of VEC and aligned bases; the host checks.
+template <typename T, int VEC>
+__global__ void __launch_bounds__(kThreads) maxpool_2x2s2_stream_kernel(const T *__restrict__ x, T *__restrict__ y, PoolGeom g,
+                                                                      int64_t total_vec, int ow_vec, float inv_ow_vec,
+                                                                      float inv_oh) {
+    typedef unsigned u4 __attribute__((ext_vector_type(4)));
+    typedef unsigned u2 __attribute__((ext_vector_type(2)));
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    constexpr bool F32 = sizeof(T) == 4;
+    const int64_t base = int64_t(blockIdx.x) * (kThreads * ZANT_STREAM_U) + threadIdx.x;
+    // flat row index of the first vector of this workgroup, then block-local arithmetic in 32 bits
+    const int64_t row0 = (int64_t(blockIdx.x) * (kThreads * ZANT_STREAM_U)) / ow_vec;
+    const int col0 = int((int64_t(blockIdx.x) * (kThreads * ZANT_STREAM_U)) - row0 * ow_vec);
+    const int64_t nc0 = row0 / g.OH;
+    const int oh0 = int(row0 - nc0 * g.OH);
+    u4 r0[ZANT_STREAM_U], r1[ZANT_STREAM_U];
+    int64_t dst[ZANT_STREAM_U];
+#pragma unroll
+    for (int u = 0; u < ZANT_STREAM_U; ++u) {
+        const int local = col0 + int(threadIdx.x) + u * kThreads;         // < ow_vec + kThreads * ZANT_STREAM_U
+        const int drow = small_div_host(local, ow_vec, inv_ow_vec), oc = local - drow * ow_vec;
+        const int ohl = oh0 + drow;                                       // rows past this plane roll over
+        const int dnc = small_div_host(ohl, g.OH, inv_oh), oh = ohl - dnc * g.OH;
+        const int64_t nc = nc0 + dnc;
+        const T *p0 = x + (nc * g.H + 2 * oh) * int64_t(g.W) + int64_t(oc) * 2 * VEC;
+        dst[u] = (nc * g.OH + oh) * int64_t(g.OW) + int64_t(oc) * VEC;
+        if (base + u * kThreads < total_vec) {
+            if (F32) {
+                const f2 a = __builtin_nontemporal_load(reinterpret_cast<const f2 *>(p0));
+                const f2 b = __builtin_nontemporal_load(reinterpret_cast<const f2 *>(p0 + g.W));
+                r0[u][0] = __float_as_uint(a[0]); r0[u][1] = __float_as_uint(a[1]);
+                r1[u][0] = __float_as_uint(b[0]); r1[u][1] = __float_as_uint(b[1]);
+            } else {
+                r0[u] = __builtin_nontemporal_load(reinterpret_cast<const u4 *>(p0));
+                r1[u] = __builtin_nontemporal_load(reinterpret_cast<const u4 *>(p0 + g.W));
+            }
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < ZANT_STREAM_U; ++u) {
+        if (base + u * kThreads >= total_vec) continue;
+        if (F32) {
+            const float m = fmaxf(fmaxf(__uint_as_float(r0[u][0]), __uint_as_float(r0[u][1])),
+                                  fmaxf(__uint_as_float(r1[u][0]), __uint_as_float(r1[u][1])));
+            __builtin_nontemporal_store(m, reinterpret_cast<float *>(y) + dst[u]);
+        } else {
+            u2 o;
+#pragma unroll
+            for (int d = 0; d < 2; ++d) {
+                uint32_t w = 0;
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    // bytewise max of the two rows, then of horizontal neighbours
+                    const uint32_t a = r0[u][d * 2 + h], b = r1[u][d * 2 + h];
+                    uint32_t m = 0;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t ba = (a >> (8 * e)) & 0xffu, bb = (b >> (8 * e)) & 0xffu;
+                        m |= (ba > bb ? ba : bb) << (8 * e);
+                    }
+                    const uint32_t p01 = max(m & 0xffu, (m >> 8) & 0xffu), p23 = max((m >> 16) & 0xffu, m >> 24);
+                    w |= (p01 | (p23 << 8)) << (16 * h);
+                }
+                o[d] = w;
+            }
+            __builtin_nontemporal_store(o, reinterpret_cast<u2 *>(reinterpret_cast<uint8_t *>(y) + dst[u]));
+        }
+    }
+}
+
 int pool_geom(const int64_t xdim[4], const int64_t ydim[4], const int64_t kernel[2], const int64_t strides[2],
               const int64_t dil[2], const int64_t *pads, int n_pads, int auto_pad, PoolGeom *g) {
     if (!xdim || !ydim || !kernel || !strides || !dil) return ZANT_NullPointer;
@@ -284,7 +431,17 @@ int launch_maxpool(zant_ctx *ctx, const T *x, const int64_t xdim[4], T *y, const
     if (!x || !y) return ZANT_NullPointer;
     const bool fast = g.kh == 2 && g.kw == 2 && g.sh == 2 && g.sw == 2 && g.dh == 1 && g.dw == 1 && g.pt == 0 &&
                       g.pl == 0 && 2 * g.OH <= g.H && 2 * g.OW <= g.W;
-    if (fast) {
+    constexpr int VEC = sizeof(T) == 1 ? 8 : 1;
+    const bool stream = fast && g.H >= 2 * g.OH && g.OW % VEC == 0 && g.W % (sizeof(T) == 1 ? 16 : 2) == 0 &&
+                        (reinterpret_cast<uintptr_t>(x) % (sizeof(T) == 1 ? 16 : 8)) == 0 &&
+                        (reinterpret_cast<uintptr_t>(y) % (sizeof(T) == 1 ? 8 : 4)) == 0 && g.OW / VEC < (1 << 18) && g.OH < (1 << 18);
+    if (stream) {
+        const int ow_vec = g.OW / VEC;
+        const int64_t total_vec = g.NC * g.OH * ow_vec;
+        KernelTimer kt(ctx);
+        hipLaunchKernelGGL((maxpool_2x2s2_stream_kernel<T, VEC>), dim3(zant_stream_grid(total_vec)), dim3(kThreads), 0, ctx->stream,
+                           x, y, g, total_vec, ow_vec, 1.0f / float(ow_vec), 1.0f / float(g.OH));
+    } else if (fast) {
         constexpr int PER = sizeof(T) == 1 ? 8 : 2;
         const int64_t items = g.NC * g.OH * ((g.OW + PER - 1) / PER);
         KernelTimer kt(ctx);
@@ -317,8 +474,14 @@ extern "C" int zant_hip_softmax_f32(zant_ctx *ctx, const float *x, float *y, int
     if (rows == 0 || cols == 0) return ZANT_OK;
     if (!x || !y) return ZANT_NullPointer;
     KernelTimer kt(ctx);
-    hipLaunchKernelGGL(softmax_f32_kernel, dim3(grid_for(rows, kThreads / 64, ctx->num_cus)), dim3(kThreads), 0,
-                       ctx->stream, x, y, rows, cols);
+    if (cols <= 16)
+        hipLaunchKernelGGL(softmax_small_f32_kernel, dim3(unsigned((rows + kThreads - 1) / kThreads)), dim3(kThreads), 0,
+                           ctx->stream, x, y, rows, int(cols),
+                           // every workgroup's span starts on a 16-byte boundary when 256 * cols floats do
+                           ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0 ? 1 : 0);
+    else
+        hipLaunchKernelGGL(softmax_f32_kernel, dim3(grid_for(rows, kThreads / 64, ctx->num_cus)), dim3(kThreads), 0,
+                           ctx->stream, x, y, rows, cols);
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
 }
@@ -362,6 +525,30 @@ extern "C" int zant_hip_add_f32(zant_ctx *ctx, const float *a, const int64_t *ad
     if (osz == 0) return ZANT_OK;
     if (!a || !b || !y) return ZANT_NullPointer;
     KernelTimer kt(ctx);
+    {
+        // per-channel fast path: one operand is the whole output, the other varies along exactly one axis
+        auto single_axis = [&](const int64_t *sv, int64_t *axis_len, int64_t *inner) {
+            int axis = -1;
+            for (int i = 0; i < g.rank; ++i)
+                if (sv[i] > 1) { if (axis >= 0) return false; axis = i; }
+            if (axis < 0) return false;
+            *axis_len = sv[axis];
+            *inner = 1;
+            for (int i = axis + 1; i < g.rank; ++i) *inner *= g.out_dim[i];
+            return sv[axis] == g.out_dim[axis];
+        };
+        int64_t clen = 0, inner = 0;
+        const float *big = nullptr, *small = nullptr;
+        if (asz == osz && single_axis(s2, &clen, &inner)) { big = a; small = b; }
+        else if (bsz == osz && single_axis(s1, &clen, &inner)) { big = b; small = a; }
+        if (big && inner % 4 == 0 && osz < (int64_t(1) << 32) &&
+            ((reinterpret_cast<uintptr_t>(big) | reinterpret_cast<uintptr_t>(y)) & 15) == 0) {
+            hipLaunchKernelGGL(add_channel_f32_kernel, dim3(zant_stream_grid(osz >> 2)), dim3(kThreads), 0, ctx->stream, big, small,
+                               y, uint32_t(osz >> 2), uint32_t(inner >> 2), uint32_t(clen));
+            ZANT_LAUNCH_CHECK(ctx);
+            return ZANT_OK;
+        }
+    }
     hipLaunchKernelGGL(add_bcast_f32_kernel, dim3(grid_for(osz, kThreads, ctx->num_cus)), dim3(kThreads), 0, ctx->stream,
                        a, b, y, osz, g);
     ZANT_LAUNCH_CHECK(ctx);

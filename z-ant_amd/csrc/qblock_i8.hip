@@ -51,19 +51,6 @@ __device__ __forceinline__ i32x4 as_i32x4(const uint4 &v) {
     return r;
 }
 
-// s / y, correctly rounded.  The general f32 division scales its operands against overflow and underflow of the
-// intermediate terms, then runs reciprocal refinement and two residual corrections.  When the caller knows that no scaling
-// can be needed (|s| and y within 2^+-40), the refined reciprocal r is the same for every element and the rest is five
-// instructions with the same correctly rounded result.
-__device__ __forceinline__ float div_by(float s, float y, float r, int fast) {
-    if (!fast) return s / y;
-    const float q0 = s * r;
-    const float e0 = __builtin_fmaf(-y, q0, s);
-    const float q1 = __builtin_fmaf(e0, r, q0);
-    const float e1 = __builtin_fmaf(-y, q1, s);
-    return __builtin_fmaf(e1, r, q1);
-}
-
 template <int CO32, int MQ>
 __global__ void __launch_bounds__(256, CO32 <= 2 ? 2 : 1)  // wide projections need the whole CU's LDS anyway
 qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 *__restrict__ w1p,
@@ -451,17 +438,8 @@ int zant_qblock_blocked(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], 
     a.ra_scale = project->y_scale; a.ra_zp = project->y_zp;
     a.rb_scale = expand->x_scale; a.rb_zp = expand->x_zp;
     a.ry_scale = add_scale; a.ry_zp = add_zp;
-    {
-        // |fa + fb| <= 256 * (a_scale + b_scale); all three scales far inside the range where f32 division needs no scaling
-        auto tame = [](float v) { return v > 1e-9f && v < 1e9f; };
-        a.fast_div = residual && tame(a.ra_scale) && tame(a.rb_scale) && tame(add_scale);
-        float r = 0.0f;
-        if (a.fast_div) {
-            const volatile float r0 = 1.0f / add_scale;  // correctly rounded: at least as good a seed as the hardware estimate
-            r = std::fmaf(std::fmaf(-add_scale, r0, 1.0f), r0, r0);
-        }
-        a.ry_rcp = r;
-    }
+    a.fast_div = residual && zant_fast_div_ok(a.ra_scale, a.rb_scale, add_scale);
+    a.ry_rcp = a.fast_div ? zant_refined_rcp(add_scale) : 0.0f;
 
     const int per_cu = cap_used <= 76 * 1024 ? 2 : 1;
     const int grid = int(std::min<int64_t>(a.n_tiles, int64_t(ctx->num_cus) * per_cu));

@@ -160,6 +160,8 @@ struct QAddArgs {
     float a_scale, b_scale, y_scale;
     int a_zp, b_zp;
     uint8_t y_zp;
+    int fast_div;   // the unscaled division sequence applies (see div_by)
+    float y_rcp;    // refined reciprocal of y_scale for it
 };
 
 __device__ __forceinline__ uint8_t qadd_one(uint8_t a, uint8_t b, const QAddArgs &q) {
@@ -181,6 +183,12 @@ __global__ void __launch_bounds__(kThreads) qlinear_add_kernel(const uint8_t *__
         }
         return;
     }
+    // the dequantised value of every stored byte, once per workgroup: two table reads replace two subtract-convert-
+    // multiply chains per output byte
+    __shared__ float ta[256], tb[256];
+    ta[threadIdx.x] = float(int(uint8_t(threadIdx.x) ^ f) - q.a_zp) * q.a_scale;
+    tb[threadIdx.x] = float(int(uint8_t(threadIdx.x) ^ f) - q.b_zp) * q.b_scale;
+    __syncthreads();
     const int64_t n16 = n >> 4;
     const int64_t base = int64_t(blockIdx.x) * (kThreads * ZANT_STREAM_U) + threadIdx.x;
     const u4 *a16 = reinterpret_cast<const u4 *>(a);
@@ -192,6 +200,7 @@ __global__ void __launch_bounds__(kThreads) qlinear_add_kernel(const uint8_t *__
         const int64_t j = base + u * kThreads;
         if (j < n16) { va[u] = __builtin_nontemporal_load(a16 + j); vb[u] = __builtin_nontemporal_load(b16 + j); }
     }
+    const float zpf = float(q.y_zp);
 #pragma unroll
     for (int u = 0; u < ZANT_STREAM_U; ++u) {
         const int64_t j = base + u * kThreads;
@@ -199,10 +208,16 @@ __global__ void __launch_bounds__(kThreads) qlinear_add_kernel(const uint8_t *__
             u4 r;
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
-                const uint32_t wa = va[u][w] ^ flip4, wb = vb[u][w] ^ flip4;
+                const uint32_t wa = va[u][w], wb = vb[u][w];
                 uint32_t o = 0;
 #pragma unroll
-                for (int k = 0; k < 4; ++k) o |= uint32_t(qadd_one(uint8_t(wa >> (8 * k)), uint8_t(wb >> (8 * k)), q)) << (8 * k);
+                for (int k = 0; k < 4; ++k) {
+                    const float sum = ta[(wa >> (8 * k)) & 0xffu] + tb[(wb >> (8 * k)) & 0xffu];
+                    if (q.fast_div)  // finite: the saturating conversion clamps and packs
+                        o = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(div_by(sum, q.y_scale, q.y_rcp, 1)) + zpf, unsigned(k), o);
+                    else
+                        o |= uint32_t(sat_u8_rne(sum / q.y_scale, q.y_zp)) << (8 * k);
+                }
                 r[w] = o ^ flip4;
             }
             __builtin_nontemporal_store(r, y16 + j);
@@ -316,14 +331,28 @@ __global__ void __launch_bounds__(kThreads) qgap_blocked_kernel(const uint32_t *
 
 // One wavefront per (n, c) plane: exact i32 sum, then the fixed f32 sequence.
 __global__ void __launch_bounds__(kThreads) qgap_kernel(const uint8_t *__restrict__ x, uint8_t *__restrict__ y, int64_t planes,
-                                                       int hw, float x_scale, int x_zp, float y_scale, uint8_t y_zp) {
+                                                       int hw, float x_scale, int x_zp, float y_scale, uint8_t y_zp, int vec) {
     const int lane = threadIdx.x & 63;
     const int64_t wave = (int64_t(blockIdx.x) * blockDim.x + threadIdx.x) >> 6;
     const int64_t nwaves = (int64_t(gridDim.x) * blockDim.x) >> 6;
     for (int64_t p = wave; p < planes; p += nwaves) {
         const uint8_t *src = x + p * hw;
         int s = 0;
-        for (int j = lane; j < hw; j += 64) s += int(src[j]) - x_zp;
+        if (vec) {  // planes of whole 16-byte vectors: v_sad_u8 adds the four bytes of a dword in one instruction
+            typedef unsigned u4 __attribute__((ext_vector_type(4)));
+            const u4 *src16 = reinterpret_cast<const u4 *>(src);
+            unsigned su = 0;
+            for (int j = lane; j < (hw >> 4); j += 64) {
+                const u4 v = __builtin_nontemporal_load(src16 + j);
+                su = __builtin_amdgcn_sad_u8(v[0], 0u, su);
+                su = __builtin_amdgcn_sad_u8(v[1], 0u, su);
+                su = __builtin_amdgcn_sad_u8(v[2], 0u, su);
+                su = __builtin_amdgcn_sad_u8(v[3], 0u, su);
+            }
+            s = int(su) - (lane == 0 ? hw * x_zp : 0);
+        } else {
+            for (int j = lane; j < hw; j += 64) s += int(src[j]) - x_zp;
+        }
         for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
         if (lane == 0) {
             const float mean = (float(s) * x_scale) / float(hw);
@@ -418,6 +447,8 @@ int zant_qlinear_add_flip(zant_ctx *ctx, const uint8_t *a, float a_scale, uint8_
     if (!a || !b || !y) return ZANT_NullPointer;
     QAddArgs q;
     q.a_scale = a_scale; q.b_scale = b_scale; q.y_scale = y_scale; q.a_zp = a_zp; q.b_zp = b_zp; q.y_zp = y_zp;
+    q.fast_div = zant_fast_div_ok(a_scale, b_scale, y_scale) ? 1 : 0;
+    q.y_rcp = q.fast_div ? zant_refined_rcp(y_scale) : 0.0f;
     const int vec = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
     KernelTimer kt(ctx);
     hipLaunchKernelGGL(qlinear_add_kernel, dim3(zant_stream_grid((n + 15) >> 4)), dim3(kThreads), 0, ctx->stream, a, b, y, n, q,
@@ -481,7 +512,8 @@ extern "C" int zant_hip_qlinear_global_avgpool_u8(zant_ctx *ctx, const uint8_t *
     if (!x || !y) return ZANT_NullPointer;
     KernelTimer kt(ctx);
     hipLaunchKernelGGL(qgap_kernel, dim3(grid_for(planes, kThreads / 64, ctx->num_cus)), dim3(kThreads), 0, ctx->stream, x,
-                       y, planes, int(hw), x_scale, int(x_zp), y_scale, y_zp);
+                       y, planes, int(hw), x_scale, int(x_zp), y_scale, y_zp,
+                       (hw % 16 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0) ? 1 : 0);
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
 }

@@ -1,6 +1,8 @@
 // Device helpers shared by the int8 kernels: the single requantisation sequence and the fused
 // Dequantize -> activation -> Quantize step.
 #pragma once
+#include <cmath>
+
 #include "common.h"
 
 // round-half-to-even (v_rndne_f32), add the zero point as a float (exact), saturate, convert.
@@ -50,4 +52,29 @@ __device__ __forceinline__ int small_div(int p, int d, float inv) {
     q += r >= d ? 1 : 0;
     q -= r < 0 ? 1 : 0;
     return q;
+}
+
+// s / y, correctly rounded.  The general f32 division scales its operands against overflow and underflow of the
+// intermediate terms, then runs reciprocal refinement and two residual corrections.  When the caller knows that no scaling
+// can be needed (|s| and y within 2^+-40), the refined reciprocal r is the same for every element and the rest is five
+// instructions with the same correctly rounded result.
+__device__ __forceinline__ float div_by(float s, float y, float r, int fast) {
+    if (!fast) return s / y;
+    const float q0 = s * r;
+    const float e0 = __builtin_fmaf(-y, q0, s);
+    const float q1 = __builtin_fmaf(e0, r, q0);
+    const float e1 = __builtin_fmaf(-y, q1, s);
+    return __builtin_fmaf(e1, r, q1);
+}
+
+// Host side of div_by: whether the unscaled sequence applies to sums of two dequantised bytes divided by y_scale
+// (|sum| <= 256 * (a_scale + b_scale); all scales far inside the range where f32 division needs no operand scaling), and
+// the refined reciprocal it takes (a correctly rounded 1 / y as the seed, one Newton step as in the hardware sequence).
+static inline bool zant_fast_div_ok(float a_scale, float b_scale, float y_scale) {
+    auto tame = [](float v) { return v > 1e-9f && v < 1e9f; };
+    return tame(a_scale) && tame(b_scale) && tame(y_scale);
+}
+static inline float zant_refined_rcp(float y) {
+    const volatile float r0 = 1.0f / y;
+    return std::fmaf(std::fmaf(-y, r0, 1.0f), r0, r0);
 }
