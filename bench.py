@@ -5,7 +5,7 @@ Workload (N=1 GPU): the reference's README CNN (Conv32-ReLU-MaxPool-Conv64-ReLU-
 Dense10-Softmax, f32) at batch 4096 -- the configuration the headline metric "batched inferences/sec at batch
 4096" is quoted on.  One step = one forward pass over one resident batch.  Prints ONE JSON line.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-operators]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-operators] [--no-networks]
 
 `value` is inferences/s with inputs resident in HBM; `roofline` is measured live with HIP events around the
 dominant kernel of the pass; `cpu_baseline` times the CPU oracle (a restatement of the reference's algorithm:
@@ -205,6 +205,45 @@ def main():
             dt = time.perf_counter() - t0
             operators["qlinearconv_u8i8_N128_C128_28x28_K128_3x3"]["cpu_oracle_1core"] = {
                 "gops": round(op * 2 / 128 / dt / 1e9, 2), "sample": f"2 of 128 images, {dt:.1f} s"}
+
+    # ---- HBM-bound operators (pool / activation / requantisation / residual add): algorithmic bytes / kernel time ----
+    if operators is not None:
+        def hbm(name, fn, nbytes):
+            fn()
+            ms = kernel_avg_ms(ctx, fn, 5)
+            operators[name] = {"ms": round(ms, 4), "gbs": round(nbytes / ms / 1e6, 1),
+                               "frac_hbm_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
+
+        xf = torch.randn(4096, 32, 26, 26, device=dev)
+        yf = torch.empty_like(xf)
+        hbm("relu_f32_4096x32x26x26", lambda: tm.ReLU_lean(xf, yf), 2 * xf.numel() * 4)
+        hbm("leaky_relu_f32_4096x32x26x26", lambda: tm.leakyReLU_lean(xf, 0.1, yf), 2 * xf.numel() * 4)
+        yp = torch.empty(4096, 32, 13, 13, device=dev)
+        hbm("maxpool2x2_f32_4096x32x26x26", lambda: tm.onnx_maxpool_lean(xf, yp, [2, 2], [2, 2], [1, 1], [0, 0, 0, 0]),
+            xf.numel() * 5)
+        bf = torch.randn(4096, 32, 26, 26, device=dev)
+        hbm("add_f32_same_shape", lambda: tm.sum_tensors_lean(xf, bf, yf), 3 * xf.numel() * 4)
+        bc = torch.randn(32, 1, 1, device=dev)
+        hbm("add_f32_per_channel_broadcast", lambda: tm.sum_tensors_lean(xf, bc, yf), 2 * xf.numel() * 4)
+        del bf, yp
+        sm = torch.randn(1 << 20, 10, device=dev)
+        so = torch.empty_like(sm)
+        hbm("softmax_f32_1Mx10", lambda: tm.softmax_lean(sm, so), 2 * sm.numel() * 4)
+        del sm, so, xf, yf
+        qa = torch.randint(0, 256, (1024, 96, 48, 48), dtype=torch.uint8, device=dev)
+        qb = torch.randint(0, 256, qa.shape, dtype=torch.uint8, device=dev)
+        hbm("qlinear_relu6_u8_1024x96x48x48", lambda: tm.qlinear_act(qa, 0.05, 128, "relu6", 0.0, 0.03, 0), 2 * qa.numel())
+        hbm("qlinear_add_u8_1024x96x48x48", lambda: tm.qlinear_add(qa, 0.05, 128, qb, 0.04, 120, 0.07, 100), 3 * qa.numel())
+        qp = torch.empty(1024, 96, 24, 24, dtype=torch.uint8, device=dev)
+        hbm("maxpool2x2_u8_1024x96x48x48", lambda: tm.onnx_maxpool_lean(qa, qp, [2, 2], [2, 2], [1, 1], [0, 0, 0, 0]),
+            qa.numel() * 5 // 4)
+        hbm("qlinear_global_avgpool_u8_1024x96x48x48", lambda: tm.qlinear_global_avgpool(qa, 0.05, 128, 0.05, 128), qa.numel())
+        ff = torch.randn(1024, 96, 48, 48, device=dev)
+        s1 = torch.tensor([0.05], device=dev)
+        z1 = torch.tensor([128], dtype=torch.uint8, device=dev)
+        hbm("quantize_linear_f32_u8", lambda: tm.quantize_linear(ff, s1, z1, 1), ff.numel() * 5)
+        hbm("dequantize_linear_u8_f32", lambda: tm.dequantize_linear(qa, s1, z1, 1), ff.numel() * 5)
+        del qa, qb, qp, ff
 
     # ---- int8 networks (configs 4 and 5): whole-network throughput with the calibrated scales of the golden fixture ----
     nets_out = None
