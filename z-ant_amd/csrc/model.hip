@@ -727,6 +727,39 @@ extern "C" int zant_model_finalize(zant_model *m) {
         (void)ntl;
     }
 
+    // ---- QLinearConv (+activation) -> MaxPool 2x2/2 between blocked tensors: the pool rides in the matrix-core kernel ----
+    for (int i = 0; i < nn; ++i) {
+        MNode &nd = m->n[i];
+        if (nd.skip || nd.op != OP_QCONV || nd.fuse_pool) continue;
+        int out = nd.out, c1 = -1, only = -1;
+        while (consumers(m, out, &c1) == 1 && m->n[c1].skip && m->n[c1].op == OP_QACT) out = m->n[c1].out;
+        if (consumers(m, out, &only) != 1 || m->n[only].op != OP_MAXPOOL || m->n[only].skip) continue;
+        MNode &pn = m->n[only];
+        const bool pool22 = pn.kernel[0] == 2 && pn.kernel[1] == 2 && pn.stride[0] == 2 && pn.stride[1] == 2 &&
+                            pn.dil[0] == 1 && pn.dil[1] == 1 && pn.pads[0] == 0 && pn.pads[1] == 0 && pn.pads[2] == 0 &&
+                            pn.pads[3] == 0 && (pn.pool_pad == ZANT_PAD_NOTSET || pn.pool_pad == ZANT_PAD_VALID);
+        const MTensor &ti = m->t[nd.in0];
+        const MTensor &to = m->t[nd.out];
+        const MTensor &tp = m->t[pn.out];
+        if (!pool22 || m->t[root_of(m, nd.in0)].layout != ZANT_LAYOUT_BLOCKED16 ||
+            m->t[root_of(m, pn.out)].layout != ZANT_LAYOUT_BLOCKED16)
+            continue;
+        if (zant_qlinearconv_layout_pool(ctx, nullptr, ti.dim, ti.scale, uint8_t(ti.zp), nullptr, nd.wdim, nullptr, nd.n_wscale,
+                                         nullptr, nd.fuse_act ? nd.act_scale : to.scale, uint8_t(nd.fuse_act ? nd.act_zp : to.zp),
+                                         nullptr, nullptr, tp.dim, nd.stride, nd.pads, nd.dil, nd.group, nd.fuse_act, nd.act_alpha,
+                                         to.scale, uint8_t(to.zp), ZANT_LAYOUT_BLOCKED16, ZANT_LAYOUT_BLOCKED16, 1, true,
+                                         nullptr) != ZANT_OK)
+            continue;
+        m->t[pn.out].scale = m->t[nd.out].scale;
+        m->t[pn.out].zp = m->t[nd.out].zp;
+        nd.fuse_pool = true;
+        const int conv_out = nd.out;
+        nd.out = pn.out;
+        pn.skip = true;
+        pn.out = conv_out;
+        pn.in0 = conv_out;
+    }
+
     // ---- inverted residual blocks: 1x1 expansion -> depthwise 3x3 -> 1x1 projection (-> Add with the block input) in one
     // kernel; the expanded tensors are never materialised -------------------------------------------------------------
     {

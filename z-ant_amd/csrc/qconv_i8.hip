@@ -316,7 +316,7 @@ __device__ __forceinline__ void qconv_step(char *__restrict__ dma, const char *_
 // (blockIdx.x, blockIdx.x + gridDim.x, ...) chunk by chunk; the (tile, chunk) steps form one sequence whose operand
 // copies run n_stages - 1 steps ahead of the matrix cores through a ring of n_stages LDS buffers, so that a step's
 // copy latency is hidden even when the step itself is only a few MFMAs (1x1 layers, small feature maps).
-template <int MT, int WM, int WN, int TT>
+template <int MT, int WM, int WN, int TT, bool POOL = false>
 __global__ void __launch_bounds__(WM *WN * 64, 2)
 qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, const float *__restrict__ mult,
                   const int32_t *__restrict__ corr, const int8_t *__restrict__ padvec, uint8_t *__restrict__ y, ConvGeom g,
@@ -375,16 +375,33 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
     __builtin_amdgcn_sched_barrier(0);
 
     // Position slot i of this lane: image, row and column inside the tile.  pos[i] packs them for the epilogue
-    // (image << 20 | row << 10 | column; -1 = the slot is beyond the tile).
+    // (image << 20 | row << 10 | column; -1 = the slot is beyond the tile).  With a fused 2x2/2 max pool, slots
+    // 4j .. 4j+3 are the four members of ONE pooling window (pooled position (wm*MT/4 + j)*32 + l32) and pos[4j] holds
+    // the POOLED row and column: the pool is a register-wise reduction in the epilogue.
     int lds_off[MT], pos[MT];
+    const int per_img_p = POOL ? (t.TH / 2) * t.POW : 1;
+    const float inv_per_img_p = 1.0f / float(per_img_p), inv_pow = 1.0f / float(POOL ? t.POW : 1);
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
-        const int p = (wm * MT + i) * 32 + l32;
-        const int img = small_div(p, per_img, inv_per_img), rem = p - img * per_img;
-        const int r = small_div(rem, g.OW, inv_ow), c = rem - r * g.OW;
+        int img, r, c, pr = 0, pc = 0;
+        if (POOL) {
+            const int pp = (wm * (MT / 4) + i / 4) * 32 + l32;
+            img = small_div(pp, per_img_p, inv_per_img_p);
+            const int rem = pp - img * per_img_p;
+            pr = small_div(rem, t.POW, inv_pow);
+            pc = rem - pr * t.POW;
+            r = 2 * pr + ((i & 3) >> 1);
+            c = 2 * pc + (i & 1);
+        } else {
+            const int p = (wm * MT + i) * 32 + l32;
+            img = small_div(p, per_img, inv_per_img);
+            const int rem = p - img * per_img;
+            r = small_div(rem, g.OW, inv_ow);
+            c = rem - r * g.OW;
+        }
         const bool in_tile = img < t.NB && r < t.TH;
         lds_off[i] = in_tile ? (img * t.PH + r * g.sh) * t.PW + c * g.sw : 0;
-        pos[i] = in_tile ? (img << 20) | (r << 10) | c : -1;
+        pos[i] = in_tile ? (img << 20) | ((POOL ? pr : r) << 10) | (POOL ? pc : c) : -1;
     }
     // everybody's table writes are visible after the first barrier of the loop below
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0) only
@@ -428,9 +445,12 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
         {
             int n0, oh0, kb;
             decode_tile(t, cur, n0, oh0, kb);
-            const int rows_here = min(t.TH, g.OH - oh0);
+            // output geometry: the convolution's own, or the pooled one
+            const int OHo = POOL ? g.OH / 2 : g.OH, OWo = POOL ? t.POW : g.OW;
+            if (POOL) oh0 >>= 1;
+            const int rows_here = min(POOL ? t.TH / 2 : t.TH, OHo - oh0);
             const int imgs_here = min(t.NB, g.N - n0);
-            const int64_t plane = int64_t(g.OH) * g.OW;
+            const int64_t plane = int64_t(OHo) * OWo;
             const int kbase = kb * K_BLK + wn * 32 + lh * 4;
             // multipliers of this lane's 16 channels, then per position the 16 activation-table lookups, all through
             // hand-issued LDS reads: the next steps' copies stay in flight behind the epilogue
@@ -445,8 +465,20 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
             const int KB = (g.K + 15) >> 4;
             const int cb0 = (kb * K_BLK + wn * 32) >> 4;
             const bool use_lut = q.has_act || !y_blocked;
+            if (POOL) {
+                // Requantisation and the activation are monotone (non-decreasing for a positive multiplier, non-increasing
+                // for a negative one), so the window's maximum output comes from its largest or smallest accumulator.
 #pragma unroll
-            for (int i = 0; i < MT; ++i) {
+                for (int j = 0; j < MT / 4; ++j)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int a0 = acc[4 * j][v], a1 = acc[4 * j + 1][v], a2 = acc[4 * j + 2][v], a3 = acc[4 * j + 3][v];
+                        const int mx = max(max(a0, a1), max(a2, a3)), mn = min(min(a0, a1), min(a2, a3));
+                        acc[4 * j][v] = mv[v] >= 0.0f ? mx : mn;
+                    }
+            }
+#pragma unroll
+            for (int i = 0; i < MT; i += (POOL ? 4 : 1)) {
                 const int img = pos[i] >> 20, r = (pos[i] >> 10) & 1023, c = pos[i] & 1023;
                 const bool ok = pos[i] >= 0 && img < imgs_here && r < rows_here;
                 if (y_blocked) {
@@ -481,7 +513,7 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
                         const uint32_t recv = uint32_t(__shfl_xor(int(send), 32, 64));
                         const uint2 out = lh ? make_uint2(recv, d[2 * b + 1]) : make_uint2(d[2 * b], recv);
                         if (ok && cb0 + b < KB) {
-                            uint8_t *yp = y + (((int64_t(n0 + img) * KB + cb0 + b) * g.OH + oh0 + r) * g.OW + c) * 16 + lh * 8;
+                            uint8_t *yp = y + (((int64_t(n0 + img) * KB + cb0 + b) * OHo + oh0 + r) * OWo + c) * 16 + lh * 8;
                             __builtin_nontemporal_store(*reinterpret_cast<const unsigned long long *>(&out), reinterpret_cast<unsigned long long *>(yp));
                         }
                     }
@@ -492,7 +524,7 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
                         ob[v] = lds_read_u8_async(__builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(float(acc[i][v]) * mv[v]) + zpf, 0u, lut_a));
                     lds_wait16(ob);
                     if (ok) {
-                        uint8_t *yp = y + (int64_t(n0 + img) * g.K + kbase) * plane + int64_t(oh0 + r) * g.OW + c;
+                        uint8_t *yp = y + (int64_t(n0 + img) * g.K + kbase) * plane + int64_t(oh0 + r) * OWo + c;
 #pragma unroll
                         for (int v = 0; v < 16; ++v) {
                             const int dk = (v >> 2) * 8 + (v & 3);
@@ -506,17 +538,17 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
     }
 }
 
-template <int MT, int WM, int WN, int TT>
+template <int MT, int WM, int WN, int TT, bool POOL = false>
 void launch_qmfma_tt(zant_ctx *ctx, const int8_t *xb, const int8_t *wp, const float *mult, const int32_t *corr,
                      const int8_t *padvec, uint8_t *y, const ConvGeom &g, const TilePlan &p, int CB, const QConvArgs &q,
                      int grid, int yb, int n_stages) {
     static bool attr_set = false;
     if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&qconv_mfma_kernel<MT, WM, WN, TT>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&qconv_mfma_kernel<MT, WM, WN, TT, POOL>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         attr_set = true;
     }
-    hipLaunchKernelGGL((qconv_mfma_kernel<MT, WM, WN, TT>), dim3(grid), dim3(WM * WN * 64), p.lds_bytes, ctx->stream, xb,
+    hipLaunchKernelGGL((qconv_mfma_kernel<MT, WM, WN, TT, POOL>), dim3(grid), dim3(WM * WN * 64), p.lds_bytes, ctx->stream, xb,
                        wp, mult, corr, padvec, y, g, p.t, CB, q, n_stages, yb);
 }
 
@@ -533,7 +565,15 @@ void launch_qmfma(zant_ctx *ctx, const int8_t *xb, const int8_t *wp, const float
 template <int WM, int WN>
 bool dispatch_qmt(zant_ctx *ctx, const int8_t *xb, const int8_t *wp, const float *mult, const int32_t *corr,
                   const int8_t *padvec, uint8_t *y, const ConvGeom &g, const TilePlan &p, int CB, const QConvArgs &q,
-                  int grid, int yb, int n_stages) {
+                  int grid, int yb, int n_stages, bool pool) {
+    if (pool) {  // four window members per lane: MT = 4
+        if (p.MT != 4) return false;
+        const int T = g.KH * g.KW;
+        if (T == 9) launch_qmfma_tt<4, WM, WN, 9, true>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, grid, yb, n_stages);
+        else if (T == 1) launch_qmfma_tt<4, WM, WN, 1, true>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, grid, yb, n_stages);
+        else launch_qmfma_tt<4, WM, WN, 0, true>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, grid, yb, n_stages);
+        return true;
+    }
     switch (p.MT) {
     case 1: launch_qmfma<1, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, grid, yb, n_stages); return true;
     case 2: launch_qmfma<2, WM, WN>(ctx, xb, wp, mult, corr, padvec, y, g, p, CB, q, grid, yb, n_stages); return true;
@@ -555,8 +595,12 @@ unsigned to_blocked_grid(zant_ctx *ctx, int64_t N, int64_t CB, int64_t hw) {
 // The matrix-core path; returns ZANT_OK when it ran, 1 when the shape is left to the other kernels.
 // x_blocked / y_blocked: x, y are already / are to be written in the blocked signed layout.
 int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float *w_scale, const int32_t *bias, uint8_t *y,
-                   const ConvGeom &g, const QConvArgs &q, bool x_blocked, bool y_blocked, zant_pack_slot *slot) {
+                   const ConvGeom &g, const QConvArgs &q, bool x_blocked, bool y_blocked, zant_pack_slot *slot, bool pool = false,
+                   bool plan_only = false) {
     if (g.groups != 1 || g.C < 5 || int64_t(g.N) * g.OH * g.OW < 64) return 1;
+    // a fused 2x2/2 max pool needs whole windows and an activation that keeps the order of its inputs
+    if (pool && (g.OH < 2 || g.OW < 2 || (q.has_act && !(q.act.alpha >= 0.0f && q.act.in_scale > 0.0f && q.act.out_scale > 0.0f))))
+        return 1;
     const int CB = (g.C + 15) / 16;
     if (int64_t(g.N) * CB * g.H * g.W >= (int64_t(1) << 27)) return 1;  // 16-byte units addressed with 32-bit offsets
     TilePlan plan;
@@ -568,10 +612,10 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
     const int target = 2 * ctx->num_cus;
     int WN = 1, WM = 4;
     // The footprint counts two staging buffers: larger tiles (more operand reuse per staged byte) beat a deeper ring.
-    bool have = zant_plan_conv_tiles(gp, 4, 1, 6, 2, 16, 80 * 1024, &plan, false, target, 32, 256);
+    bool have = zant_plan_conv_tiles(gp, 4, 1, 6, 2, 16, 80 * 1024, &plan, pool, target, 32, 256);
     if (g.K > 32) {
         TilePlan wide;
-        if (zant_plan_conv_tiles(gp, 2, 2, 6, 2, 16, 80 * 1024, &wide, false, target, 32, 256) && (!have || wide.score >= plan.score * 0.98)) {
+        if (zant_plan_conv_tiles(gp, 2, 2, 6, 2, 16, 80 * 1024, &wide, pool, target, 32, 256) && (!have || wide.score >= plan.score * 0.98)) {
             plan = wide; WN = 2; WM = 2; have = true;
         }
     }
@@ -593,6 +637,7 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
     if (n_stages > plan.t.n_chunks + 1) n_stages = std::max(plan.t.n_chunks + 1, 2);
     while (n_stages > 2 && (n_stages * buf_bytes + fixed_bytes > lds_cap || copies * (n_stages - 2) > 63)) --n_stages;
     if (n_stages * buf_bytes + fixed_bytes > lds_cap) return 1;
+    if (plan_only) return ZANT_OK;
     plan.lds_bytes = n_stages * buf_bytes + fixed_bytes;
     const size_t wp_bytes = size_t(plan.t.n_chunks) * plan.t.n_kblocks * T * QCC * K_BLK;
     const size_t kpad = size_t(plan.t.n_kblocks) * K_BLK;
@@ -628,8 +673,8 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
     }
     KernelTimer kt(ctx);
     const int yb = y_blocked ? 1 : 0;
-    const bool ok = WN == 2 ? dispatch_qmt<2, 2>(ctx, xb, wp, mult, corr, padvec, y, g, plan, CB, q, grid, yb, n_stages)
-                            : dispatch_qmt<4, 1>(ctx, xb, wp, mult, corr, padvec, y, g, plan, CB, q, grid, yb, n_stages);
+    const bool ok = WN == 2 ? dispatch_qmt<2, 2>(ctx, xb, wp, mult, corr, padvec, y, g, plan, CB, q, grid, yb, n_stages, pool)
+                            : dispatch_qmt<4, 1>(ctx, xb, wp, mult, corr, padvec, y, g, plan, CB, q, grid, yb, n_stages, pool);
     if (!ok) return 1;
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
@@ -1079,7 +1124,8 @@ int zant_to_blocked(zant_ctx *ctx, const uint8_t *x, int64_t N, int64_t C, int64
     return ZANT_OK;
 }
 
-// fuse_pool (internal callers only): ydim is the 2x2/2 max-pooled shape; only the first-layer kernel takes it.
+// fuse_pool (internal callers only): ydim is the 2x2/2 max-pooled shape; the first-layer kernel and the matrix-core
+// kernel (blocked tensors on both sides) take it.
 int zant_qlinearconv_layout_pool(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], float x_scale, uint8_t x_zp,
                                  const int8_t *w, const int64_t wdim[4], const float *w_scale, int64_t n_wscale,
                                  const int8_t *w_zp, float y_scale, uint8_t y_zp, const int32_t *bias, uint8_t *y,
@@ -1112,16 +1158,20 @@ int zant_qlinearconv_layout_pool(zant_ctx *ctx, const uint8_t *x, const int64_t 
     g.pt = int(pads[0]); g.pl = int(pads[1]); g.groups = int(group);
     const bool xb = x_layout == ZANT_LAYOUT_BLOCKED16, yb = y_layout == ZANT_LAYOUT_BLOCKED16;
     const bool smallc = w_zp == nullptr && !xb && smallc_eligible(g);
-    if (fuse_pool && (!smallc || OHo < 1 || OWo < 1)) return 1;  // only the first-layer kernel pools
-    if (query_only) return ZANT_OK;
-    if (!x || !w || !w_scale || !y) return ZANT_NullPointer;
-
     QConvArgs q;
     q.x_scale = x_scale; q.y_scale = y_scale; q.x_zp = x_zp; q.y_zp = y_zp; q.n_wscale = int(n_wscale);
     q.has_act = act != ZANT_ACT_NONE;
     q.act.act = act; q.act.alpha = act_alpha; q.act.in_scale = y_scale; q.act.in_zp = y_zp;
     q.act.out_scale = act_scale; q.act.out_zp = act_zp;
 
+    // Pooling rides in the first-layer kernel (NCHW input) or in the matrix-core kernel (blocked on both sides).
+    const bool pool_mfma = fuse_pool && !smallc && xb && yb && w_zp == nullptr && !dw_eligible(g) && OHo >= 1 && OWo >= 1 &&
+                           run_qconv_mfma(ctx, nullptr, nullptr, nullptr, nullptr, nullptr, g, q, true, true, nullptr, true, true) == ZANT_OK;
+    if (fuse_pool && !pool_mfma && (!smallc || OHo < 1 || OWo < 1)) return 1;
+    if (query_only) return ZANT_OK;
+    if (!x || !w || !w_scale || !y) return ZANT_NullPointer;
+
+    if (pool_mfma) return run_qconv_mfma(ctx, x, w, w_scale, bias, y, g, q, true, true, slot, true, false);
     if (smallc) return run_qconv_smallc(ctx, x, w, w_scale, bias, y, g, q, yb, fuse_pool != 0, slot);
 
     const size_t x_blk = zant_blocked_bytes(xdim), y_blk = zant_blocked_bytes(ydim);

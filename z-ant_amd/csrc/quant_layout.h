@@ -15,8 +15,9 @@ static inline size_t zant_blocked_bytes(const int64_t dim[4]) {
 }
 
 // zant_hip_qlinearconv_u8i8 with the layout of x and y chosen by the caller.
-// fuse_pool: also max-pool 2x2/2 (floor, no padding) in the same kernel; ydim is then the pooled shape.  Only the
-// first-layer kernel (1..4 input channels, 3x3, NCHW input) does that: other shapes return 1 and run nothing.
+// fuse_pool: also max-pool 2x2/2 (floor, no padding) in the same kernel; ydim is then the pooled shape.  The first-layer
+// kernel (1..4 input channels, 3x3, NCHW input) and the matrix-core kernel (blocked x and y, an order-preserving
+// activation) do that: other shapes return 1 and run nothing.
 // query_only: validate and report eligibility (ZANT_OK / 1 / error status) without touching any pointer.
 // slot: where weight-derived scratch is kept across calls (nullptr: repacked on every call).
 int zant_qlinearconv_layout_pool(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], float x_scale, uint8_t x_zp,
