@@ -12,6 +12,7 @@
 // with padding positions holding x_zp so that they contribute exactly 0.  Tiling, the asynchronous
 // double-buffered staging and the persistent tile loop are those of the f32 kernel.
 #include <algorithm>
+#include <type_traits>
 
 #include "conv_tile.h"
 #include "quant_common.h"
@@ -80,6 +81,12 @@ typedef __attribute__((address_space(1))) const void *gptr_t;
 typedef __attribute__((address_space(3))) void *lptr_t;
 
 constexpr int QCC = 32;  // input channels per chunk = one MFMA k-step per filter tap
+
+__device__ __forceinline__ i32x4 as_i32x4_q(const uint4 &v) {
+    i32x4 r;
+    r[0] = int(v.x); r[1] = int(v.y); r[2] = int(v.z); r[3] = int(v.w);
+    return r;
+}
 
 // NCHW u8 -> [N][CB][H][W][16] signed (value - 128); channels beyond C are 0 (their weights are 0 too).
 // Each thread turns 4 consecutive positions x 16 channels: sixteen 4-byte loads (one per channel
@@ -862,8 +869,242 @@ int launch_smallc(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float 
     return ZANT_OK;
 }
 
+// ------------------------------------------------------------------------------------------------------------------
+// First layers on the matrix cores (1..4 input channels, 3x3, stride 1 or 2, pads <= 1, NCHW u8 input).
+// The GEMM's reduction index is k = (channel, filter row) * 4 + filter column, the fourth column carrying a zero weight:
+// 16 consecutive k are then four 4-byte pieces of input rows, each ONE (unaligned) dword load -- the B operand of
+// v_mfma_i32_32x32x32_i8 needs no byte gathering at all.  A lane pair (p, 0), (p, 1) holds output position p; a
+// wavefront turns 32 positions x 32 output channels per MFMA chain.  With the fused 2x2/2 max pool (stride 1) the four
+// window members are four chains over shifted views of the same row dwords, reduced on the accumulators.
+// ------------------------------------------------------------------------------------------------------------------
+typedef uint32_t __attribute__((aligned(1))) u32_unaligned;
+
+template <int C>
+__global__ void __launch_bounds__(256)
+qfirst_pack_kernel(const int8_t *__restrict__ w, const float *__restrict__ w_scale, const int32_t *__restrict__ bias,
+                   int8_t *__restrict__ wpk, float *__restrict__ mult, int32_t *__restrict__ corr, int K, int kb32, float x_scale,
+                   float y_scale, int x_zp, int n_wscale) {
+    constexpr int RW = C * 3, NCH = (RW + 7) / 8;
+    const int total = kb32 * NCH * 2 * 32 * 16;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gridDim.x * blockDim.x) {
+        int r = i;
+        const int kwi = r & 3; r >>= 2;
+        const int j = r & 3; r >>= 2;
+        const int kk = r & 31; r >>= 5;
+        const int half = r & 1; r >>= 1;
+        const int ch = r % NCH, kb = r / NCH;
+        const int k = kb * 32 + kk, rw = ch * 8 + half * 4 + j;
+        wpk[i] = (k < K && rw < RW && kwi < 3) ? w[(int64_t(k) * C + rw / 3) * 9 + (rw % 3) * 3 + kwi] : int8_t(0);
+    }
+    for (int k = blockIdx.x * blockDim.x + threadIdx.x; k < kb32 * 32; k += gridDim.x * blockDim.x) {
+        int sum = 0;
+        if (k < K)
+            for (int t = 0; t < C * 9; ++t) sum += int(w[int64_t(k) * C * 9 + t]);
+        corr[k] = k < K ? (bias ? bias[k] : 0) + (128 - x_zp) * sum : 0;
+        mult[k] = k < K ? (x_scale * w_scale[n_wscale == 1 ? 0 : k]) / y_scale : 0.0f;
+    }
+}
+
+template <int C, int S, bool POOL, int NV>  // NV: accumulator values per lane that are real channels (8 when K <= 16)
+__global__ void __launch_bounds__(256, 2)
+qfirst_mfma_kernel(const uint8_t *__restrict__ x, const uint4 *__restrict__ wpk, const float *__restrict__ mult,
+                   const int32_t *__restrict__ corr, uint8_t *__restrict__ y, ConvGeom g, QConvArgs q, int y_blocked, int kb32) {
+    constexpr int RW = C * 3, NCH = (RW + 7) / 8;
+    constexpr int PR = POOL ? 4 : 3, NWIN = POOL ? 4 : 1;
+    __shared__ uint8_t lut[256];  // the fused activation as a byte table, in the byte values the output stores
+    lut[threadIdx.x] = uint8_t((q.has_act ? qact_apply(uint8_t(threadIdx.x), q.act) : uint8_t(threadIdx.x)) ^ (y_blocked ? 0x80 : 0));
+    __syncthreads();
+    const int lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
+    const int OHo = POOL ? g.OH / 2 : g.OH, OWo = POOL ? g.OW / 2 : g.OW;
+    const int KB16 = (g.K + 15) >> 4;
+    const unsigned per_img = unsigned(OHo) * unsigned(OWo), total = unsigned(g.N) * per_img;  // < 2^31 (host)
+    const unsigned n_ptiles = (total + 31u) / 32u;
+    const float inv_per_img = 1.0f / float(per_img), inv_owo = 1.0f / float(OWo);
+    const bool small_total = total < (1u << 20);
+    const uint32_t padb = uint32_t(q.x_zp ^ 0x80) & 0xffu, pad4 = padb * 0x01010101u;
+    const float zpf = float(q.y_zp);
+    const int64_t plane_in = int64_t(g.H) * g.W;
+    const unsigned wave_id = (blockIdx.x * blockDim.x + threadIdx.x) >> 6, n_waves = (gridDim.x * blockDim.x) >> 6;
+    i32x16 cvec;
+    float mv[16];
+    i32x4 wa_all[NCH];
+    bool tables_loaded = false;
+    // The row loads of the NEXT tile are issued before this tile's arithmetic: with two wavefronts per SIMD the load
+    // latency would otherwise sit on the critical path of every tile.
+    struct TileMeta { unsigned n; int oho, owo, ih0, sh; bool valid; };
+    uint32_t raw[C][PR];
+    TileMeta nxt;
+    auto issue = [&](unsigned pt, TileMeta &m) {
+        const unsigned i = pt * 32u + unsigned(l32);
+        m.valid = i < total;
+        const unsigned ii = m.valid ? i : total - 1u;
+        m.n = small_total ? unsigned(small_div(int(ii), int(per_img), inv_per_img)) : ii / per_img;
+        const int rem = int(ii - m.n * per_img);
+        m.oho = small_div(rem, OWo, inv_owo);
+        m.owo = rem - m.oho * OWo;
+        m.ih0 = (POOL ? 2 * m.oho : m.oho) * S - g.pt;
+        const int iw0 = (POOL ? 2 * m.owo : m.owo) * S - g.pl;
+        // one dword per (channel, patch row): columns iw0 .. iw0+3, read from a start clamped into the row
+        const int iw0c = min(max(iw0, 0), g.W - 4);
+        m.sh = iw0 - iw0c;
+        const uint8_t *xn = x + int64_t(m.n) * C * plane_in + iw0c;
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+#pragma unroll
+            for (int r = 0; r < PR; ++r) {
+                const int ih = m.ih0 + r;
+                raw[c][r] = *reinterpret_cast<const u32_unaligned *>(xn + c * plane_in + int64_t(min(max(ih, 0), g.H - 1)) * g.W);
+            }
+    };
+    if (wave_id < n_ptiles) issue(wave_id, nxt);
+    for (unsigned pt = wave_id; pt < n_ptiles; pt += n_waves) {
+        const TileMeta cur = nxt;
+        const unsigned n = cur.n;
+        const int oho = cur.oho, owo = cur.owo, ih0 = cur.ih0, sh = cur.sh;
+        const bool valid = cur.valid;
+        // shifted into place; columns outside the image (and rows outside it) take the padding byte
+        uint32_t row[C][PR];
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+#pragma unroll
+            for (int r = 0; r < PR; ++r) {
+                const int ih = ih0 + r;
+                const uint32_t d = (ih >= 0 && ih < g.H) ? raw[c][r] ^ 0x80808080u : pad4;
+                // bytes of (hi:lo) >> 8 * s: a start clamped at the left edge shifts the row up behind one padding byte,
+                // one clamped at the right edge shifts it down with padding bytes following
+                row[c][r] = __builtin_amdgcn_alignbyte(sh < 0 ? d : pad4, sh < 0 ? pad4 : d, sh < 0 ? 3u : unsigned(sh));
+            }
+        if (pt + n_waves < n_ptiles) issue(pt + n_waves, nxt);
+        for (int kb = 0; kb < kb32; ++kb) {
+            const int kch = kb * 32 + lh * 4;
+            if (kb32 > 1 || !tables_loaded) {  // one block of output channels: the tables stay in registers across tiles
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    cvec[v] = corr[kch + (v >> 2) * 8 + (v & 3)];
+                    mv[v] = mult[kch + (v >> 2) * 8 + (v & 3)];
+                }
+#pragma unroll
+                for (int ch = 0; ch < NCH; ++ch) wa_all[ch] = as_i32x4_q(wpk[((kb * NCH + ch) * 2 + lh) * 32 + l32]);
+                tables_loaded = true;
+            }
+            i32x16 acc[NWIN];
+#pragma unroll
+            for (int ch = 0; ch < NCH; ++ch) {
+                const i32x4 wa = wa_all[ch];
+#pragma unroll
+                for (int wd = 0; wd < NWIN; ++wd) {
+                    const int dy = wd >> 1, dx = wd & 1;
+                    i32x4 b;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        // reduction rows ch*8 + j (lanes (p, 0)) and ch*8 + 4 + j (lanes (p, 1)): (channel, filter row)
+                        const int ra = ch * 8 + j, rb = ch * 8 + 4 + j;
+                        const uint32_t va = ra < RW ? row[ra / 3][ra % 3 + dy] >> (8 * dx) : 0u;
+                        const uint32_t vb = rb < RW ? row[rb / 3][rb % 3 + dy] >> (8 * dx) : 0u;
+                        b[j] = int(lh ? vb : va);
+                    }
+                    acc[wd] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wa, b, ch == 0 ? cvec : acc[wd], 0, 0, 0);
+                }
+            }
+            if (POOL) {
+                // requantisation and the activation keep (multiplier >= 0) or reverse (< 0) the order of the accumulators
+#pragma unroll
+                for (int v = 0; v < NV; ++v) {
+                    const int a0 = acc[0][v], a1 = acc[NWIN > 1 ? 1 : 0][v], a2 = acc[NWIN > 2 ? 2 : 0][v], a3 = acc[NWIN > 3 ? 3 : 0][v];
+                    const int mx = max(max(a0, a1), max(a2, a3)), mn = min(min(a0, a1), min(a2, a3));
+                    acc[0][v] = mv[v] >= 0.0f ? mx : mn;
+                }
+            }
+            uint32_t ob[16];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) ob[v] = v < NV ? uint32_t(lut[sat_u8_rne_finite(float(acc[0][v]) * mv[v], zpf)]) : 0u;
+            if (y_blocked) {
+                uint32_t d[4];
+#pragma unroll
+                for (int gq = 0; gq < 4; ++gq) d[gq] = ob[gq * 4] | (ob[gq * 4 + 1] << 8) | (ob[gq * 4 + 2] << 16) | (ob[gq * 4 + 3] << 24);
+#pragma unroll
+                for (int b = 0; b < 2; ++b) {
+                    const uint32_t send = lh ? d[2 * b] : d[2 * b + 1];
+                    const uint32_t recv = uint32_t(__shfl_xor(int(send), 32, 64));
+                    const uint2 out = lh ? make_uint2(recv, d[2 * b + 1]) : make_uint2(d[2 * b], recv);
+                    const int cbq = kb * 2 + b;
+                    if (valid && cbq < KB16) {
+                        uint8_t *yp = y + (((int64_t(n) * KB16 + cbq) * OHo + oho) * int64_t(OWo) + owo) * 16 + lh * 8;
+                        *reinterpret_cast<uint2 *>(yp) = out;
+                    }
+                }
+            } else if (valid) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int k = kch + (v >> 2) * 8 + (v & 3);
+                    if (k < g.K) y[((int64_t(n) * g.K + k) * OHo + oho) * int64_t(OWo) + owo] = uint8_t(ob[v]);
+                }
+            }
+        }
+    }
+}
+
+bool qfirst_eligible(const ConvGeom &g, bool pool) {
+    const int S = (g.sh == g.sw && (g.sh == 1 || g.sh == 2)) ? g.sh : 0;
+    if (S == 0 || (pool && S != 1) || g.W < 4 || g.pl > 1 || g.pt > 1) return false;
+    // the rightmost patch may hang over the row by at most three columns (it is read from a clamped start)
+    const int last = ((pool ? (g.OW / 2) * 2 : g.OW) - 1) * S - g.pl;
+    if (last + 3 - (g.W - 1) > 3) return false;
+    const int64_t OHo = pool ? g.OH / 2 : g.OH, OWo = pool ? g.OW / 2 : g.OW;
+    return OHo >= 1 && OWo >= 1 && int64_t(g.N) * OHo * OWo < (int64_t(1) << 31) - 64 && OHo * OWo < (1 << 20);
+}
+
+template <int C>
+int launch_qfirst(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float *w_scale, const int32_t *bias, uint8_t *y,
+                  const ConvGeom &g, const QConvArgs &q, bool y_blocked, bool pool, zant_pack_slot *slot) {
+    constexpr int RW = C * 3, NCH = (RW + 7) / 8;
+    const int kb32 = (g.K + 31) / 32;
+    const size_t o_mult = 0, o_corr = align256(size_t(kb32) * 32 * 4), o_w = 2 * o_corr, w_bytes = size_t(kb32) * NCH * 2 * 32 * 16;
+    void *ws = nullptr, *dyn = nullptr;
+    bool need_pack = true;
+    int parity = 0;
+    const int rc = zant_pack_region(ctx, slot, o_w + w_bytes, 0, &ws, &dyn, &need_pack, &parity);
+    if (rc) return rc;
+    char *base = static_cast<char *>(ws);
+    float *mult = reinterpret_cast<float *>(base + o_mult);
+    int32_t *corr = reinterpret_cast<int32_t *>(base + o_corr);
+    int8_t *wpk = reinterpret_cast<int8_t *>(base + o_w);
+    if (need_pack) {
+        hipLaunchKernelGGL(qfirst_pack_kernel<C>, dim3(unsigned(std::min<size_t>((w_bytes + 255) / 256, 256))), dim3(256), 0,
+                           ctx->stream, w, w_scale, bias, wpk, mult, corr, g.K, kb32, q.x_scale, q.y_scale, q.x_zp, q.n_wscale);
+        ZANT_LAUNCH_CHECK(ctx);
+    }
+    const int64_t positions = int64_t(g.N) * (pool ? g.OH / 2 : g.OH) * (pool ? g.OW / 2 : g.OW);
+    const unsigned blocks = unsigned(std::min<int64_t>(std::max<int64_t>(ceil_div64(positions, 128), 1), int64_t(ctx->num_cus) * 16));
+    KernelTimer kt(ctx);
+    const int yb = y_blocked ? 1 : 0;
+#define ZANT_QFIRST(SV, PV)                                                                                                 \
+    do {                                                                                                                    \
+        if (g.K <= 16)                                                                                                      \
+            hipLaunchKernelGGL((qfirst_mfma_kernel<C, SV, PV, 8>), dim3(blocks), dim3(256), 0, ctx->stream, x,             \
+                               reinterpret_cast<const uint4 *>(wpk), mult, corr, y, g, q, yb, kb32);                       \
+        else                                                                                                                \
+            hipLaunchKernelGGL((qfirst_mfma_kernel<C, SV, PV, 16>), dim3(blocks), dim3(256), 0, ctx->stream, x,            \
+                               reinterpret_cast<const uint4 *>(wpk), mult, corr, y, g, q, yb, kb32);                       \
+    } while (0)
+    if (pool) ZANT_QFIRST(1, true);
+    else if (g.sh == 1) ZANT_QFIRST(1, false);
+    else ZANT_QFIRST(2, false);
+#undef ZANT_QFIRST
+    ZANT_LAUNCH_CHECK(ctx);
+    return ZANT_OK;
+}
+
 int run_qconv_smallc(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float *w_scale, const int32_t *bias, uint8_t *y,
                      const ConvGeom &g, const QConvArgs &q, bool y_blocked, bool pool, zant_pack_slot *slot) {
+    if (qfirst_eligible(g, pool)) {
+        switch (g.C) {
+        case 1: return launch_qfirst<1>(ctx, x, w, w_scale, bias, y, g, q, y_blocked, pool, slot);
+        case 2: return launch_qfirst<2>(ctx, x, w, w_scale, bias, y, g, q, y_blocked, pool, slot);
+        case 3: return launch_qfirst<3>(ctx, x, w, w_scale, bias, y, g, q, y_blocked, pool, slot);
+        default: return launch_qfirst<4>(ctx, x, w, w_scale, bias, y, g, q, y_blocked, pool, slot);
+        }
+    }
     switch (g.C) {
     case 1: return launch_smallc<1>(ctx, x, w, w_scale, bias, y, g, q, y_blocked, pool, slot);
     case 2: return launch_smallc<2>(ctx, x, w, w_scale, bias, y, g, q, y_blocked, pool, slot);
