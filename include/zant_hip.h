@@ -264,7 +264,9 @@ int zant_model_predict_host(zant_model *m, const void *input_host, void *output_
  * "Conv+Relu+MaxPool". */
 int zant_model_profile(zant_model *m, float *ms, double *ops, double *bytes, int capacity);
 const char *zant_model_launch_name(zant_model *m, int i);
-/* Debug: copies tensor `id` (as planned in the arena) to the host after a run. */
+/* Debug: copies tensor `id` (as planned in the arena) to the host after a run.  Tensors that a fusion removed (the
+ * output of a convolution whose pool, or of a residual block's inner layers, run in the same kernel) are never
+ * materialised: ZANT_InvalidInput. */
 int zant_model_read_tensor(zant_model *m, int id, void *dst_host, size_t bytes);
 
 /* The reference's exported entry point (src/codeGen/predict.zig:34-39), served by the bound model:

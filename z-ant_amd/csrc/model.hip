@@ -1079,6 +1079,7 @@ extern "C" int zant_model_read_tensor(zant_model *m, int id, void *dst_host, siz
     if (!valid_tensor(m, id) || !dst_host) return ZANT_NullPointer;
     if (!m->finalized) return ZANT_NotFinalized;
     if (bytes > m->t[id].bytes()) return ZANT_InvalidDimensions;
+    if (m->t[root_of(m, id)].def < 0) return ZANT_InvalidInput;  // fused away: the tensor is never materialised
     const MTensor &t = m->t[id];
     if (m->t[root_of(m, id)].layout == ZANT_LAYOUT_BLOCKED16) {  // hand out NCHW u8 like everywhere outside the executor
         void *ws = nullptr;
