@@ -39,6 +39,7 @@ struct QBlockArgs {
     QAct act1, act2;
     int has_act1, has_act2;
     uint32_t pad_e4;                   // the depthwise input zero point ^ 0x80 in every byte
+    int half_last;                     // the last chunk of expanded channels holds at most 16 real ones
     int has_res, fast_div;             // fast_div: the scales allow the unscaled division sequence
     float ry_rcp;                      // refined reciprocal of ry_scale
     float ra_scale, rb_scale, ry_scale;  // residual add: a = projection output, b = block input, y = sum
@@ -137,6 +138,7 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
                     mv[v] = m1[kch + (v >> 2) * 8 + (v & 3)];
                 }
                 const i32x4 wa0 = as_i32x4(W1[kb * 64 + lh * 32 + l32]);
+                const bool half = a.half_last && kb == a.Ce32 - 1;
                 char *erow = reinterpret_cast<char *>(E) + (kb * 2 * a.Ppad + l32) * 16 + lh * 8;
                 for (; ptile < n_ptiles && u < u_end; ++ptile, ++u) {
                     const int p = ptile * 32 + l32;
@@ -144,14 +146,26 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
                     for (int chunk = 1; chunk < a.Cin32; ++chunk)
                         acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(as_i32x4(W1[(chunk * a.Ce32 + kb) * 64 + lh * 32 + l32]),
                                                                     as_i32x4(XL[(2 * chunk + lh) * a.Ppad + p]), acc, 0, 0, 0);
-                    uint32_t d[4];
+                    // a last block with at most 16 real channels: accumulator rows 16..31 (values 8..15) are padding
+                    uint32_t d[4] = {0u, 0u, 0u, 0u};
+                    if (half) {
 #pragma unroll
-                    for (int gq = 0; gq < 4; ++gq) {
-                        uint32_t o = 0;
+                        for (int gq = 0; gq < 2; ++gq) {
+                            uint32_t o = 0;
 #pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            o |= uint32_t(lut1[sat_u8_rne_finite(float(acc[gq * 4 + e]) * mv[gq * 4 + e], a.zp1f)]) << (8 * e);
-                        d[gq] = o;
+                            for (int e = 0; e < 4; ++e)
+                                o |= uint32_t(lut1[sat_u8_rne_finite(float(acc[gq * 4 + e]) * mv[gq * 4 + e], a.zp1f)]) << (8 * e);
+                            d[gq] = o;
+                        }
+                    } else {
+#pragma unroll
+                        for (int gq = 0; gq < 4; ++gq) {
+                            uint32_t o = 0;
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                o |= uint32_t(lut1[sat_u8_rne_finite(float(acc[gq * 4 + e]) * mv[gq * 4 + e], a.zp1f)]) << (8 * e);
+                            d[gq] = o;
+                        }
                     }
                     // lanes p and p + 32 exchange one dword per 16-channel block so that each writes 8 consecutive bytes
 #pragma unroll
@@ -159,7 +173,7 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
                         const uint32_t send = lh ? d[2 * b] : d[2 * b + 1];
                         const uint32_t recv = uint32_t(__shfl_xor(int(send), 32, 64));
                         const uint2 out = lh ? make_uint2(recv, d[2 * b + 1]) : make_uint2(d[2 * b], recv);
-                        *reinterpret_cast<uint2 *>(erow + (b * a.Ppad + ptile * 32) * 16) = out;
+                        if (b == 0 || !half) *reinterpret_cast<uint2 *>(erow + (b * a.Ppad + ptile * 32) * 16) = out;
                     }
                 }
                 ptile = 0;
@@ -205,6 +219,7 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
                 }
             for (int ch = 0; ch < a.Ce32; ++ch) {
                 const int kch = ch * 32 + lh * 4;
+                const bool half = a.half_last && ch == a.Ce32 - 1;
                 i32x16 cvec;
                 float mv[16];
 #pragma unroll
@@ -229,14 +244,25 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
 #pragma unroll
                     for (int t = 1; t < 9; ++t)
                         acc2 = __builtin_amdgcn_mfma_i32_32x32x32_i8(wa[t], as_i32x4(ep[(t / 3) * a.PW + (t % 3)]), acc2, 0, 0, 0);
-                    uint32_t d[4];
+                    uint32_t d[4] = {0u, 0u, 0u, 0u};
+                    if (half) {
 #pragma unroll
-                    for (int gq = 0; gq < 4; ++gq) {
-                        uint32_t o = 0;
+                        for (int gq = 0; gq < 2; ++gq) {
+                            uint32_t o = 0;
 #pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            o |= uint32_t(lut2[sat_u8_rne_finite(float(acc2[gq * 4 + e]) * mv[gq * 4 + e], a.zp2f)]) << (8 * e);
-                        d[gq] = o;
+                            for (int e = 0; e < 4; ++e)
+                                o |= uint32_t(lut2[sat_u8_rne_finite(float(acc2[gq * 4 + e]) * mv[gq * 4 + e], a.zp2f)]) << (8 * e);
+                            d[gq] = o;
+                        }
+                    } else {
+#pragma unroll
+                        for (int gq = 0; gq < 4; ++gq) {
+                            uint32_t o = 0;
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                o |= uint32_t(lut2[sat_u8_rne_finite(float(acc2[gq * 4 + e]) * mv[gq * 4 + e], a.zp2f)]) << (8 * e);
+                            d[gq] = o;
+                        }
                     }
                     // lane (p, 0) gathers channels 0..15 of the chunk, lane (p, 1) channels 16..31
                     const uint32_t r0 = uint32_t(__shfl_xor(int(lh ? d[0] : d[2]), 32, 64));
@@ -434,6 +460,7 @@ int zant_qblock_blocked(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], 
     a.act2.act = dw->act; a.act2.alpha = dw->act_alpha; a.act2.in_scale = dw->y_scale; a.act2.in_zp = dw->y_zp;
     a.act2.out_scale = dw->act_scale; a.act2.out_zp = uint8_t(dw->act_zp);
     a.pad_e4 = uint32_t((dw->x_zp ^ 0x80) & 0xff) * 0x01010101u;
+    a.half_last = (Ce % 32 != 0 && Ce % 32 <= 16) ? 1 : 0;
     a.has_res = residual ? 1 : 0;
     a.ra_scale = project->y_scale; a.ra_zp = project->y_zp;
     a.rb_scale = expand->x_scale; a.rb_zp = expand->x_zp;
