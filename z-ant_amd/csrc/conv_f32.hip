@@ -512,11 +512,12 @@ bool plan_mfma(const ConvGeom &g, MfmaPlan *best, bool pool = false) {
     if (g.K <= 32) return zant_plan_conv_tiles(g, 4, 1, 8, CC, sizeof(float), 80 * 1024, best, pool);
     // 64 output channels per workgroup (2 x 2 waves) stage the input patch once per 64 channels; 32 per workgroup
     // (4 x 1 waves) stage it twice but have twice the position slots, which can fit small feature maps much better
-    // (e.g. 5 whole 5x5 pooled images in 128 slots instead of 2 in 64).  Take the narrow shape only for a clear win.
+    // (e.g. 5 whole 5x5 pooled images in 128 slots instead of 2 in 64).  Take the narrow shape only for a clear win: at
+    // 0.98 against 0.78 useful columns the two measured the same time, and the wide one reads the input once.
     MfmaPlan wide, narrow;
     const bool ok_w = zant_plan_conv_tiles(g, 2, 2, 8, CC, sizeof(float), 80 * 1024, &wide, pool);
     const bool ok_n = zant_plan_conv_tiles(g, 4, 1, 8, CC, sizeof(float), 80 * 1024, &narrow, pool);
-    if (ok_n && (!ok_w || narrow.eff > wide.eff + 0.1)) { *best = narrow; return true; }
+    if (ok_n && (!ok_w || narrow.eff > wide.eff + 0.25)) { *best = narrow; return true; }
     if (ok_w) { *best = wide; return true; }
     return false;
 }
