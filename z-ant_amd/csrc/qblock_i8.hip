@@ -440,15 +440,14 @@ int zant_qblock_blocked(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], 
     uint32_t *wmk = reinterpret_cast<uint32_t *>(base + o_wm);
     if (need_pack) {
         int8_t *padvec = reinterpret_cast<int8_t *>(base + 16);
-        int *word = reinterpret_cast<int *>(base);
         rc = zant_qpack_dense(ctx, expand->w, expand->w_scale, expand->n_wscale, expand->bias, int(Ce), int(Cin), 1, 32,
-                              expand->x_scale, expand->x_zp, expand->y_scale, w1p, m1, c1, padvec, word);
+                              expand->x_scale, expand->x_zp, expand->y_scale, w1p, m1, c1, padvec);
         if (rc) return rc;
         rc = zant_qpack_depthwise(ctx, dw->w, dw->w_scale, dw->n_wscale, dw->bias, int(Ce), CeP, dw->x_scale, dw->x_zp,
                                   dw->y_scale, wmk, m2, c2);
         if (rc) return rc;
         rc = zant_qpack_dense(ctx, project->w, project->w_scale, project->n_wscale, project->bias, int(Co), int(Ce), 1, 32,
-                              project->x_scale, project->x_zp, project->y_scale, w2p, m3, c3, padvec + 16, word);
+                              project->x_scale, project->x_zp, project->y_scale, w2p, m3, c3, padvec + 16);
         if (rc) return rc;
     }
 

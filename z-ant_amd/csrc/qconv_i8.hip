@@ -134,16 +134,15 @@ __global__ void __launch_bounds__(256) to_blocked_s8_kernel(const uint8_t *__res
 
 // Packs OIHW int8 weights into [chunk][kblock][tap][half][K_BLK][16] (zero padded), and writes the
 // per-channel requantisation multiplier, the integer correction (bias + (128 - x_zp) * sum w), the
-// 16-byte padding vector (x_zp - 128 in every lane) and the tile counter.
+// 16-byte padding vector (x_zp - 128 in every lane).
 __global__ void __launch_bounds__(256)
 qpack_kernel(const int8_t *__restrict__ w, const float *__restrict__ w_scale, const int32_t *__restrict__ bias,
              int8_t *__restrict__ wp, float *__restrict__ mult, int32_t *__restrict__ corr, int8_t *__restrict__ padvec,
-             int *__restrict__ tile_counter, int counter_init, int K, int C, int T, int n_chunks, int n_kblocks, int k_blk,
+             int K, int C, int T, int n_chunks, int n_kblocks, int k_blk,
              float x_scale, float y_scale, int x_zp, int n_wscale) {
     const int64_t total = int64_t(n_chunks) * n_kblocks * T * QCC * k_blk;
     const int64_t step = int64_t(gridDim.x) * blockDim.x;
     const int64_t gid = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (gid == 0) *tile_counter = counter_init;
     if (gid < 16) padvec[gid] = int8_t(x_zp - 128);
     for (int64_t i = gid; i < total; i += step) {
         int64_t r = i;
@@ -657,7 +656,6 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
     int rc = zant_pack_region(ctx, slot, static_bytes, xb_bytes, &ws, &dyn, &need_pack, &parity);
     if (rc) return rc;
     char *base = static_cast<char *>(ws);
-    int *counter = reinterpret_cast<int *>(base);
     int8_t *padvec = reinterpret_cast<int8_t *>(base + o_pad);
     float *mult = reinterpret_cast<float *>(base + o_mult);
     int32_t *corr = reinterpret_cast<int32_t *>(base + o_corr);
@@ -666,8 +664,8 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
     const int grid = int(std::min<int64_t>(plan.t.n_tiles, int64_t(ctx->num_cus) * 2));
     const unsigned pb = unsigned(std::min<int64_t>(std::max<int64_t>(ceil_div64(int64_t(wp_bytes), 256), ceil_div64(int64_t(kpad), 4)), 1024));
     if (need_pack) {
-        hipLaunchKernelGGL(qpack_kernel, dim3(pb), dim3(256), 0, ctx->stream, w, w_scale, bias, wp, mult, corr, padvec, counter,
-                           2 * grid, g.K, g.C, T, plan.t.n_chunks, plan.t.n_kblocks, K_BLK, q.x_scale, q.y_scale, q.x_zp,
+        hipLaunchKernelGGL(qpack_kernel, dim3(pb), dim3(256), 0, ctx->stream, w, w_scale, bias, wp, mult, corr, padvec,
+                           g.K, g.C, T, plan.t.n_chunks, plan.t.n_kblocks, K_BLK, q.x_scale, q.y_scale, q.x_zp,
                            q.n_wscale);
         ZANT_LAUNCH_CHECK(ctx);
     }
@@ -1334,12 +1332,12 @@ int run_qdw_blocked(zant_ctx *ctx, const uint8_t *xb, const int8_t *w, const flo
 
 int zant_qpack_dense(zant_ctx *ctx, const int8_t *w, const float *w_scale, int64_t n_wscale, const int32_t *bias, int K, int C,
                      int T, int k_blk, float x_scale, int x_zp, float y_scale, int8_t *wp, float *mult, int32_t *corr,
-                     int8_t *padvec, int *scratch_word) {
+                     int8_t *padvec) {
     const int n_chunks = (C + QCC - 1) / QCC, n_kblocks = (K + k_blk - 1) / k_blk;
     const int64_t wp_bytes = int64_t(n_chunks) * n_kblocks * T * QCC * k_blk, kpad = int64_t(n_kblocks) * k_blk;
     const unsigned pb = unsigned(std::min<int64_t>(std::max<int64_t>(ceil_div64(wp_bytes, 256), ceil_div64(kpad, 4)), 1024));
-    hipLaunchKernelGGL(qpack_kernel, dim3(pb), dim3(256), 0, ctx->stream, w, w_scale, bias, wp, mult, corr, padvec, scratch_word,
-                       0, K, C, T, n_chunks, n_kblocks, k_blk, x_scale, y_scale, x_zp, int(n_wscale));
+    hipLaunchKernelGGL(qpack_kernel, dim3(pb), dim3(256), 0, ctx->stream, w, w_scale, bias, wp, mult, corr, padvec,
+                       K, C, T, n_chunks, n_kblocks, k_blk, x_scale, y_scale, x_zp, int(n_wscale));
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
 }

@@ -47,10 +47,10 @@ int zant_qgap_blocked(zant_ctx *ctx, const uint8_t *xb, const int64_t xdim[4], f
 // Weight packing shared by the int8 matrix-core kernels (device pointers; launches on the context's stream).
 // Dense: [chunk of 32 input channels][block of k_blk output channels][tap][half][k_blk][16] int8, zero padded; per
 // output channel the requantisation multiplier (x_scale * w_scale / y_scale) and the integer correction
-// (bias + (128 - x_zp) * sum of weights); padvec = 16 bytes of x_zp - 128; scratch_word: one int that gets cleared.
+// (bias + (128 - x_zp) * sum of weights); padvec = 16 bytes of x_zp - 128.
 int zant_qpack_dense(zant_ctx *ctx, const int8_t *w, const float *w_scale, int64_t n_wscale, const int32_t *bias, int K, int C,
                      int T, int k_blk, float x_scale, int x_zp, float y_scale, int8_t *wp, float *mult, int32_t *corr,
-                     int8_t *padvec, int *scratch_word);
+                     int8_t *padvec);
 // Depthwise 3x3: one dword per (channel, tap) with the weight in byte (channel % 4) and zeros elsewhere, at
 // wm[((channel / 4) * 9 + tap) * 4 + channel % 4]; multipliers and corrections as above, for kpad channels.
 int zant_qpack_depthwise(zant_ctx *ctx, const int8_t *w, const float *w_scale, int64_t n_wscale, const int32_t *bias, int K,
