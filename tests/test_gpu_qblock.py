@@ -49,6 +49,11 @@ CASES = [
     ((41, 37), 8, [(48, 16, 2, "relu6", "relu6", 1)], 2, 3),                     # row tiles, stride 2, odd sizes
     ((12, 12), 16, [(96, 16, 1, "relu6", "relu6", 1), (96, 24, 2, "relu6", "relu6", 1)], 6, 4),  # two blocks in a row
     ((9, 9), 8, [(48, 8, 1, "relu6", "relu6", 0)], 3, 5),                        # pad-0 depthwise: not the pattern, unfused
+    ((1, 1), 8, [(16, 8, 1, "relu6", "relu6", 1)], 7, 3),                        # one pixel, one half-filled expanded chunk
+    ((2, 3), 5, [(30, 128, 2, "relu6", "relu6", 1)], 1, 3),                      # batch 1, ragged input channels, 128 outputs
+    ((3, 3), 8, [(48, 8, 1, "relu6", "relu6", 1)], 1030, 3),                     # more images than one pass of tiles
+    ((24, 24), 40, [(240, 40, 1, "relu6", "relu6", 1)], 2, 3),                   # three input blocks, many expanded chunks
+    ((17, 5), 8, [(16, 24, 2, None, "leaky", 1)], 3, 3),                         # tall narrow map, stride 2
 ]
 
 
