@@ -369,9 +369,13 @@ int zant_qblock_blocked(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], 
     };
     bool found = false;
     size_t cap_used = 0;
-    // 76 KB: what two workgroups per CU leave each other after the allocation granularity
+    double best_time = 0.0;
+    // 76 KB: what two workgroups per CU leave each other after the allocation granularity.  Both sizes are planned and
+    // the cheaper taken: two workgroups on a CU run at half speed each but overlap each other's barriers and latencies,
+    // which the estimate credits with a factor 1.5 against the single large workgroup.
     for (size_t cap : {size_t(76 * 1024), size_t(160 * 1024)}) {
-        const int64_t slots = int64_t(ctx->num_cus) * (cap <= 80 * 1024 ? 2 : 1);
+        const bool two = cap <= 80 * 1024;
+        const int64_t slots = int64_t(ctx->num_cus) * (two ? 2 : 1);
         double best = 0.0;
         int bNB = 0, bTH = 0;
         if (lds_for(p_img) <= cap) {
@@ -390,31 +394,34 @@ int zant_qblock_blocked(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], 
                 const double c = tile_cost(P, th * OW) * double(waves);
                 if (!bNB || c < best * 0.98) { best = c; bNB = 1; bTH = int(th); }
             }
-            if (bNB && bTH < std::min<int64_t>(OH, 4) && cap < 160 * 1024) bNB = 0;  // too much halo: take the whole CU's LDS
         }
         if (!bNB) continue;
-        a.NB = bNB; a.TH = bTH;
-        a.PH = (bTH - 1) * int(dw_stride) + 3;
-        if (a.PH > 1023) continue;
-        a.P = bNB * a.PH * a.PW;
-        a.Ppad = (a.P + 31) & ~31;
-        a.Q = bNB * bTH * int(OW);
-        a.n_row_tiles = int((OH + bTH - 1) / bTH);
-        const int64_t n_tiles = ((N + bNB - 1) / bNB) * a.n_row_tiles;
-        if (n_tiles > INT32_MAX || a.P >= (1 << 20) || a.Q >= (1 << 20)) continue;
-        a.n_tiles = int(n_tiles);
+        const double time = best * (two ? 2.0 : 1.5);
+        if (found && time >= best_time) continue;
+        QBlockArgs t = a;
+        t.NB = bNB; t.TH = bTH;
+        t.PH = (bTH - 1) * int(dw_stride) + 3;
+        if (t.PH > 1023) continue;
+        t.P = bNB * t.PH * t.PW;
+        t.Ppad = (t.P + 31) & ~31;
+        t.Q = bNB * bTH * int(OW);
+        t.n_row_tiles = int((OH + bTH - 1) / bTH);
+        const int64_t n_tiles = ((N + bNB - 1) / bNB) * t.n_row_tiles;
+        if (n_tiles > INT32_MAX || t.P >= (1 << 20) || t.Q >= (1 << 20)) continue;
+        t.n_tiles = int(n_tiles);
         size_t o = 512;
-        a.o_xl = int(o); o += size_t(a.Cin32) * 2 * a.Ppad * 16;
-        a.o_e = int(o); o += size_t(a.Ce32) * 2 * a.Ppad * 16;
-        a.o_w1 = int(o); o += w1_bytes;
-        a.o_w2 = int(o); o += w2_bytes;
-        a.o_wdw = int(o); o += wdw_bytes;
-        a.o_tab = int(o); o += tab_bytes;
-        a.o_ptab = int(o); o += align16(size_t(a.P) * 4);
+        t.o_xl = int(o); o += size_t(t.Cin32) * 2 * t.Ppad * 16;
+        t.o_e = int(o); o += size_t(t.Ce32) * 2 * t.Ppad * 16;
+        t.o_w1 = int(o); o += w1_bytes;
+        t.o_w2 = int(o); o += w2_bytes;
+        t.o_wdw = int(o); o += wdw_bytes;
+        t.o_tab = int(o); o += tab_bytes;
+        t.o_ptab = int(o); o += align16(size_t(t.P) * 4);
         if (o > cap) continue;
+        a = t;
         cap_used = o;
+        best_time = time;
         found = true;
-        break;
     }
     if (!found) return 1;
     if (query_only) return ZANT_OK;
