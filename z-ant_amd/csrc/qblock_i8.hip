@@ -58,7 +58,7 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
               const uint4 *__restrict__ w2p, const uint32_t *__restrict__ wm, const float *__restrict__ mult1,
               const int32_t *__restrict__ corr1, const float *__restrict__ mult2, const int32_t *__restrict__ corr2,
               const float *__restrict__ mult3, const int32_t *__restrict__ corr3, QBlockArgs a) {
-    extern __shared__ __attribute__((aligned(16))) char lds[];
+    extern __shared__ __attribute__((aligned(256))) char lds[];  // the activation tables need 256-byte alignment
     uint8_t *lut1 = reinterpret_cast<uint8_t *>(lds), *lut2 = lut1 + 256;
     uint4 *XL = reinterpret_cast<uint4 *>(lds + a.o_xl);   // [Cin32*2][Ppad] units of 16 channels
     uint4 *E = reinterpret_cast<uint4 *>(lds + a.o_e);     // [Ce32*2][Ppad]
@@ -75,6 +75,7 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
     int *ptab = reinterpret_cast<int *>(lds + a.o_ptab);   // [P] image << 20 | patch row << 10 | patch column
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, lh = lane >> 5;
+    const unsigned lut1_a = lds_address(lut1), lut2_a = lds_address(lut2);
 
     // ---- once per workgroup: tables and weights into LDS ----
     {
@@ -154,7 +155,7 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
                             uint32_t o = 0;
 #pragma unroll
                             for (int e = 0; e < 4; ++e)
-                                o |= uint32_t(lut1[sat_u8_rne_finite(float(acc[gq * 4 + e]) * mv[gq * 4 + e], a.zp1f)]) << (8 * e);
+                                o |= requant_lookup(float(acc[gq * 4 + e]) * mv[gq * 4 + e], a.zp1f, lut1_a) << (8 * e);
                             d[gq] = o;
                         }
                     } else {
@@ -163,7 +164,7 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
                             uint32_t o = 0;
 #pragma unroll
                             for (int e = 0; e < 4; ++e)
-                                o |= uint32_t(lut1[sat_u8_rne_finite(float(acc[gq * 4 + e]) * mv[gq * 4 + e], a.zp1f)]) << (8 * e);
+                                o |= requant_lookup(float(acc[gq * 4 + e]) * mv[gq * 4 + e], a.zp1f, lut1_a) << (8 * e);
                             d[gq] = o;
                         }
                     }
@@ -251,7 +252,7 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
                             uint32_t o = 0;
 #pragma unroll
                             for (int e = 0; e < 4; ++e)
-                                o |= uint32_t(lut2[sat_u8_rne_finite(float(acc2[gq * 4 + e]) * mv[gq * 4 + e], a.zp2f)]) << (8 * e);
+                                o |= requant_lookup(float(acc2[gq * 4 + e]) * mv[gq * 4 + e], a.zp2f, lut2_a) << (8 * e);
                             d[gq] = o;
                         }
                     } else {
@@ -260,7 +261,7 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
                             uint32_t o = 0;
 #pragma unroll
                             for (int e = 0; e < 4; ++e)
-                                o |= uint32_t(lut2[sat_u8_rne_finite(float(acc2[gq * 4 + e]) * mv[gq * 4 + e], a.zp2f)]) << (8 * e);
+                                o |= requant_lookup(float(acc2[gq * 4 + e]) * mv[gq * 4 + e], a.zp2f, lut2_a) << (8 * e);
                             d[gq] = o;
                         }
                     }

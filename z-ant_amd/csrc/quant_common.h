@@ -78,3 +78,15 @@ static inline float zant_refined_rcp(float y) {
     const volatile float r0 = 1.0f / y;
     return std::fmaf(std::fmaf(-y, r0, 1.0f), r0, r0);
 }
+
+// Requantisation followed by a 256-entry byte table that sits at a 256-byte aligned LDS address: the saturating
+// conversion writes its byte into the low byte of `table` (its third operand), which makes the result the entry's
+// address -- no separate address addition per value.
+__device__ __forceinline__ unsigned lds_address(const void *p) {
+    return unsigned(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void *) const_cast<void *>(p)));
+}
+__device__ __forceinline__ uint32_t requant_lookup(float v, float zp_f, unsigned table) {
+    const unsigned addr = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(v) + zp_f, 0u, table);
+    return *reinterpret_cast<const __attribute__((address_space(3))) uint8_t *>(addr);
+}
+
