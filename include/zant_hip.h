@@ -174,6 +174,17 @@ int zant_hip_quantize_linear_f32_u8(zant_ctx *ctx, const float *x, const int64_t
 int zant_hip_dequantize_linear_u8_f32(zant_ctx *ctx, const uint8_t *x, const int64_t *xdim, int rank,
                                       const float *x_scale, const uint8_t *x_zp, int64_t n_scale, int axis,
                                       float *y);
+/* The same operators for the other code types ONNX defines: int8 codes (saturating to [-128, 127]) and
+ * DequantizeLinear of int32 (accumulators, biases).  The zero point has the code type. */
+int zant_hip_quantize_linear_f32_i8(zant_ctx *ctx, const float *x, const int64_t *xdim, int rank,
+                                    const float *y_scale, const int8_t *y_zp, int64_t n_scale, int axis,
+                                    int8_t *y);
+int zant_hip_dequantize_linear_i8_f32(zant_ctx *ctx, const int8_t *x, const int64_t *xdim, int rank,
+                                      const float *x_scale, const int8_t *x_zp, int64_t n_scale, int axis,
+                                      float *y);
+int zant_hip_dequantize_linear_i32_f32(zant_ctx *ctx, const int32_t *x, const int64_t *xdim, int rank,
+                                       const float *x_scale, const int32_t *x_zp, int64_t n_scale, int axis,
+                                       float *y);
 /* QLinearConv (u8 x i8 -> i32 -> u8), explicit pads [top,left,bottom,right], any
  * group dividing C and K (group == C: depthwise).  w_scale (n_wscale = 1 or K),
  * w_zp (NULL = 0) and bias (NULL = 0) are device pointers; activation scales and

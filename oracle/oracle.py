@@ -258,21 +258,31 @@ def reshape_lean(x, new_shape):
 
 # ----------------------------------------------------------------------------- int8 family
 
-def quantize_linear(x, y_scale, y_zp=None, axis=1):
+def quantize_linear(x, y_scale, y_zp=None, axis=1, signed=False):
+    """signed (or an int8 zero point): int8 output saturating to [-128, 127]; otherwise uint8."""
     x = _f32(x); y_scale = np.atleast_1d(_f32(y_scale))
-    zp = None if y_zp is None else np.atleast_1d(np.ascontiguousarray(y_zp, dtype=np.uint8))
-    y = np.zeros(x.shape, np.uint8)
+    signed = signed or (y_zp is not None and np.asarray(y_zp).dtype == np.int8)
+    dt = np.int8 if signed else np.uint8
+    zp = None if y_zp is None else np.atleast_1d(np.ascontiguousarray(y_zp, dtype=dt))
+    y = np.zeros(x.shape, dt)
     xd, r = _dims(x.shape)
-    _chk(_lib.zo_quantize_linear_f32_u8(_ptr(x), xd, r, _ptr(y_scale), _ptr(zp), C.c_int64(y_scale.size), axis, _ptr(y)))
+    fn = _lib.zo_quantize_linear_f32_i8 if signed else _lib.zo_quantize_linear_f32_u8
+    _chk(fn(_ptr(x), xd, r, _ptr(y_scale), _ptr(zp), C.c_int64(y_scale.size), axis, _ptr(y)))
     return y
 
 
 def dequantize_linear(x, x_scale, x_zp=None, axis=1):
-    x = np.ascontiguousarray(x, dtype=np.uint8); x_scale = np.atleast_1d(_f32(x_scale))
-    zp = None if x_zp is None else np.atleast_1d(np.ascontiguousarray(x_zp, dtype=np.uint8))
+    """x: uint8, int8 or int32 (the zero point has x's type)."""
+    x = np.ascontiguousarray(x)
+    if x.dtype not in (np.uint8, np.int8, np.int32):
+        x = x.astype(np.uint8)
+    x_scale = np.atleast_1d(_f32(x_scale))
+    zp = None if x_zp is None else np.atleast_1d(np.ascontiguousarray(x_zp, dtype=x.dtype))
     y = np.zeros(x.shape, np.float32)
     xd, r = _dims(x.shape)
-    _chk(_lib.zo_dequantize_linear_u8_f32(_ptr(x), xd, r, _ptr(x_scale), _ptr(zp), C.c_int64(x_scale.size), axis, _ptr(y)))
+    fn = {np.dtype(np.uint8): _lib.zo_dequantize_linear_u8_f32, np.dtype(np.int8): _lib.zo_dequantize_linear_i8_f32,
+          np.dtype(np.int32): _lib.zo_dequantize_linear_i32_f32}[x.dtype]
+    _chk(fn(_ptr(x), xd, r, _ptr(x_scale), _ptr(zp), C.c_int64(x_scale.size), axis, _ptr(y)))
     return y
 
 

@@ -641,6 +641,54 @@ int zo_dequantize_linear_u8_f32(const uint8_t *x, const int64_t *xdim, int rank,
     return ZO_OK;
 }
 
+/* QuantizeLinear to int8: the same sequence saturating to [-128, 127] (ONNX QuantizeLinear, int8 output). */
+int zo_quantize_linear_f32_i8(const float *x, const int64_t *xdim, int rank, const float *y_scale,
+                              const int8_t *y_zp, int64_t n_scale, int axis, int8_t *y) {
+    int64_t n = 1, inner, alen;
+    for (int i = 0; i < rank; ++i) n *= xdim[i];
+    if (n_scale > 1 && (axis < -rank || axis >= rank)) return ZO_InvalidDimensions;
+    axis_geometry(xdim, rank, axis, n_scale, &inner, &alen);
+    if (n_scale > 1 && n_scale != alen) return ZO_InputTensorDimensionMismatch;
+    for (int64_t i = 0; i < n; ++i) {
+        const int64_t c = n_scale > 1 ? (i / inner) % alen : 0;
+        float r = rintf(x[i] / y_scale[c]) + (float)(y_zp ? y_zp[c] : 0);
+        r = fmaxf(r, -128.0f); /* NaN -> -128 */
+        r = fminf(r, 127.0f);
+        y[i] = (int8_t)r;
+    }
+    return ZO_OK;
+}
+
+/* DequantizeLinear from int8 and from int32 (the accumulator / bias type): y = (x - zp) * scale. */
+int zo_dequantize_linear_i8_f32(const int8_t *x, const int64_t *xdim, int rank, const float *x_scale,
+                                const int8_t *x_zp, int64_t n_scale, int axis, float *y) {
+    int64_t n = 1, inner, alen;
+    for (int i = 0; i < rank; ++i) n *= xdim[i];
+    if (n_scale > 1 && (axis < -rank || axis >= rank)) return ZO_InvalidDimensions;
+    axis_geometry(xdim, rank, axis, n_scale, &inner, &alen);
+    if (n_scale > 1 && n_scale != alen) return ZO_InputTensorDimensionMismatch;
+    for (int64_t i = 0; i < n; ++i) {
+        const int64_t c = n_scale > 1 ? (i / inner) % alen : 0;
+        y[i] = (float)((int)x[i] - (int)(x_zp ? x_zp[c] : 0)) * x_scale[c];
+    }
+    return ZO_OK;
+}
+
+int zo_dequantize_linear_i32_f32(const int32_t *x, const int64_t *xdim, int rank, const float *x_scale,
+                                 const int32_t *x_zp, int64_t n_scale, int axis, float *y) {
+    int64_t n = 1, inner, alen;
+    for (int i = 0; i < rank; ++i) n *= xdim[i];
+    if (n_scale > 1 && (axis < -rank || axis >= rank)) return ZO_InvalidDimensions;
+    axis_geometry(xdim, rank, axis, n_scale, &inner, &alen);
+    if (n_scale > 1 && n_scale != alen) return ZO_InputTensorDimensionMismatch;
+    for (int64_t i = 0; i < n; ++i) {
+        const int64_t c = n_scale > 1 ? (i / inner) % alen : 0;
+        /* the difference in 64 bits (it cannot wrap), converted to f32 once */
+        y[i] = (float)((int64_t)x[i] - (int64_t)(x_zp ? x_zp[c] : 0)) * x_scale[c];
+    }
+    return ZO_OK;
+}
+
 int zo_qconv_acc_i32(const uint8_t *x, const int64_t xdim[4], uint8_t x_zp, const int8_t *w,
                      const int64_t wdim[4], const int8_t *w_zp, const int32_t *bias, int32_t *acc,
                      const int64_t ydim[4], const int64_t stride[2], const int64_t pads[4],

@@ -84,6 +84,27 @@ def test_quantize_dequantize_bit_exact(G):
     np.testing.assert_array_equal(G.host(G.tm.quantize_linear(G.dev(t), 1.0, 0)), [0, 2, 2, 0, 4, 254, 255])
 
 
+def test_signed_and_int32_codes_bit_exact(G):
+    import torch
+    g = np.random.default_rng(12)
+    x = (g.standard_normal((3, 4, 9, 7)) * 40).astype(np.float32)
+    x.ravel()[:8] = [0.5, 1.5, -0.5, -2.5, 127.5, -128.5, 1e9, -1e9]
+    for s, zp, axis in [(np.float32(0.7), None, 1), (np.array([0.3, 0.5, 1.0, 2.0], np.float32), np.array([-128, -7, 0, 127], np.int8), 1)]:
+        ref = zo.quantize_linear(x, s, zp, axis, signed=True)
+        zt = None if zp is None else torch.from_numpy(zp)
+        q = G.tm.quantize_linear(G.dev(x), s, zt, axis, signed=True)
+        assert q.dtype == torch.int8
+        np.testing.assert_array_equal(G.host(q), ref)
+        np.testing.assert_array_equal(G.host(G.tm.dequantize_linear(q, s, zt, axis)), zo.dequantize_linear(ref, s, zp, axis))
+    acc = g.integers(-2**31, 2**31, (2, 5, 3), dtype=np.int64).astype(np.int32)
+    acc.ravel()[:2] = [2**31 - 1, -2**31]
+    sc = np.array([1e-3, 0.5, 2.0, 7.0, 1.0], np.float32)
+    np.testing.assert_array_equal(G.host(G.tm.dequantize_linear(G.dev(acc), sc, None, 1)), zo.dequantize_linear(acc, sc, None, 1))
+    zp32 = np.array([-2**31, 5, 0, -9, 2**31 - 1], np.int32)
+    np.testing.assert_array_equal(G.host(G.tm.dequantize_linear(G.dev(acc), sc, torch.from_numpy(zp32), 1)),
+                                  zo.dequantize_linear(acc, sc, zp32, 1))
+
+
 @pytest.mark.parametrize("act,alpha", [("relu", 0.0), ("leaky", 0.1), ("relu6", 0.0), (None, 0.0)])
 @pytest.mark.parametrize("n", [256, 100003])
 def test_qlinear_act_bit_exact(G, act, alpha, n):

@@ -143,6 +143,29 @@ def test_quantize_per_axis_and_dequantize_roundtrip():
     np.testing.assert_array_equal(zo.quantize_linear(d, s, zp, axis=1), q)
 
 
+def test_signed_and_int32_codes():
+    """int8 QuantizeLinear saturates to [-128, 127] with the same rounding; int8 / int32 DequantizeLinear are (x - zp) * s."""
+    x = np.array([0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 126.5, 127.5, 1000.0, -128.5, -129.5, -1000.0], np.float32)
+    y = zo.quantize_linear(x, 1.0, None, signed=True)
+    assert y.dtype == np.int8
+    np.testing.assert_array_equal(y, [0, 2, 2, 0, -2, -2, 126, 127, 127, -128, -128, -128])
+    np.testing.assert_array_equal(zo.quantize_linear(x[:4], 1.0, np.array([-3], np.int8)), [-3, -1, -1, -3])
+    g = rng(11)
+    v = g.standard_normal((2, 3, 5)).astype(np.float32) * 4
+    s = np.array([0.02, 0.05, 0.1], np.float32); zp = np.array([-5, 0, 17], np.int8)
+    q = zo.quantize_linear(v, s, zp, axis=1)
+    ref = np.clip(np.rint(v / s[None, :, None]) + zp[None, :, None].astype(np.float32), -128, 127).astype(np.int8)
+    np.testing.assert_array_equal(q, ref)
+    d = zo.dequantize_linear(q, s, zp, axis=1)
+    np.testing.assert_array_equal(d, (q.astype(np.int32) - zp[None, :, None]).astype(np.float32) * s[None, :, None])
+    np.testing.assert_array_equal(zo.quantize_linear(d, s, zp, axis=1), q)  # identity on in-range codes
+    acc = np.array([0, 1, -1, 2**31 - 1, -2**31, 123456789], np.int32)
+    np.testing.assert_array_equal(zo.dequantize_linear(acc, np.float32(0.5)), acc.astype(np.float64).astype(np.float32) * np.float32(0.5))
+    # the difference cannot wrap: (2^31 - 1) - (-2^31) = 2^32 - 1
+    z = zo.dequantize_linear(np.array([2**31 - 1], np.int32), np.float32(1.0), np.array([-2**31], np.int32))
+    assert z[0] == np.float32(2.0**32)
+
+
 @pytest.mark.parametrize("act,alpha", [("relu", 0.0), ("leaky", 0.1), ("relu6", 0.0), (None, 0.0)])
 def test_qlinear_act_matches_dequant_act_quant(act, alpha):
     q = np.arange(256, dtype=np.uint8)

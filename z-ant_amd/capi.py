@@ -61,6 +61,9 @@ PROTOTYPES = {
     "zant_hip_reshape": (i32, [vp, vp, c_i64p, i32, sz, c_i64p, i32, vp, c_i64p]),
     "zant_hip_quantize_linear_f32_u8": (i32, [vp, vp, c_i64p, i32, vp, vp, i64, i32, vp]),
     "zant_hip_dequantize_linear_u8_f32": (i32, [vp, vp, c_i64p, i32, vp, vp, i64, i32, vp]),
+    "zant_hip_quantize_linear_f32_i8": (i32, [vp, vp, c_i64p, i32, vp, vp, i64, i32, vp]),
+    "zant_hip_dequantize_linear_i8_f32": (i32, [vp, vp, c_i64p, i32, vp, vp, i64, i32, vp]),
+    "zant_hip_dequantize_linear_i32_f32": (i32, [vp, vp, c_i64p, i32, vp, vp, i64, i32, vp]),
     "zant_hip_qlinearconv_u8i8": (i32, [vp, vp, c_i64p, f32, u8, vp, c_i64p, vp, i64, vp, f32, u8, vp, vp, c_i64p,
                                         c_i64p, c_i64p, c_i64p, i64, i32, f32, f32, u8]),
     "zant_hip_qlinear_act_u8": (i32, [vp, vp, i64, f32, u8, i32, f32, f32, u8, vp]),

@@ -23,13 +23,23 @@ struct AxisGeom {
     int per_axis;
 };
 
+__device__ __forceinline__ int8_t sat_i8_rne(float v, int8_t zp) {
+    float r = __builtin_rintf(v) + float(zp);
+    r = __builtin_fmaxf(r, -128.0f);  // NaN -> -128
+    r = __builtin_fminf(r, 127.0f);
+    return int8_t(r);
+}
+__device__ __forceinline__ uint8_t sat_q(float v, uint8_t zp) { return sat_u8_rne(v, zp); }
+__device__ __forceinline__ int8_t sat_q(float v, int8_t zp) { return sat_i8_rne(v, zp); }
+
+// Any axis layout, u8 or i8 codes.
+template <typename Q>
 __global__ void __launch_bounds__(kThreads) quantize_kernel(const float *__restrict__ x, const float *__restrict__ scale,
-                                                           const uint8_t *__restrict__ zp, uint8_t *__restrict__ y,
-                                                           AxisGeom g) {
+                                                           const Q *__restrict__ zp, Q *__restrict__ y, AxisGeom g) {
     const int64_t step = int64_t(gridDim.x) * blockDim.x;
     for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < g.n; i += step) {
         const int64_t c = g.per_axis ? (i / g.inner) % g.alen : 0;
-        y[i] = sat_u8_rne(x[i] / scale[c], zp ? zp[c] : uint8_t(0));
+        y[i] = sat_q(x[i] / scale[c], zp ? zp[c] : Q(0));
     }
 }
 
@@ -99,13 +109,14 @@ __global__ void __launch_bounds__(kThreads) dequantize_vec_kernel(const uint8_t 
     }
 }
 
-__global__ void __launch_bounds__(kThreads) dequantize_kernel(const uint8_t *__restrict__ x, const float *__restrict__ scale,
-                                                             const uint8_t *__restrict__ zp, float *__restrict__ y,
-                                                             AxisGeom g) {
+// Any axis layout; u8, i8 or i32 codes (the difference is taken in 64 bits: an i32 pair can differ by 2^32).
+template <typename Q>
+__global__ void __launch_bounds__(kThreads) dequantize_kernel(const Q *__restrict__ x, const float *__restrict__ scale,
+                                                             const Q *__restrict__ zp, float *__restrict__ y, AxisGeom g) {
     const int64_t step = int64_t(gridDim.x) * blockDim.x;
     for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < g.n; i += step) {
         const int64_t c = g.per_axis ? (i / g.inner) % g.alen : 0;
-        y[i] = float(int(x[i]) - int(zp ? zp[c] : uint8_t(0))) * scale[c];
+        y[i] = float(int64_t(x[i]) - int64_t(zp ? zp[c] : Q(0))) * scale[c];
     }
 }
 
@@ -393,8 +404,8 @@ extern "C" int zant_hip_quantize_linear_f32_u8(zant_ctx *ctx, const float *x, co
         hipLaunchKernelGGL(quantize_vec_kernel, dim3(zant_stream_grid((g.n + 3) >> 2)), dim3(kThreads), 0, ctx->stream, x, y_scale,
                            y_zp, y, g.n);
     else
-    hipLaunchKernelGGL(quantize_kernel, dim3(grid_for(g.n, kThreads, ctx->num_cus)), dim3(kThreads), 0, ctx->stream, x,
-                       y_scale, y_zp, y, g);
+        hipLaunchKernelGGL(quantize_kernel<uint8_t>, dim3(grid_for(g.n, kThreads, ctx->num_cus)), dim3(kThreads), 0, ctx->stream,
+                           x, y_scale, y_zp, y, g);
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
 }
@@ -413,10 +424,61 @@ extern "C" int zant_hip_dequantize_linear_u8_f32(zant_ctx *ctx, const uint8_t *x
         hipLaunchKernelGGL(dequantize_vec_kernel, dim3(zant_stream_grid((g.n + 3) >> 2)), dim3(kThreads), 0, ctx->stream, x,
                            x_scale, x_zp, y, g.n);
     else
-    hipLaunchKernelGGL(dequantize_kernel, dim3(grid_for(g.n, kThreads, ctx->num_cus)), dim3(kThreads), 0, ctx->stream, x,
+        hipLaunchKernelGGL(dequantize_kernel<uint8_t>, dim3(grid_for(g.n, kThreads, ctx->num_cus)), dim3(kThreads), 0, ctx->stream,
+                           x, x_scale, x_zp, y, g);
+    ZANT_LAUNCH_CHECK(ctx);
+    return ZANT_OK;
+}
+
+namespace {
+
+template <typename Q>
+int launch_quantize(zant_ctx *ctx, const float *x, const int64_t *xdim, int rank, const float *y_scale, const Q *y_zp,
+                    int64_t n_scale, int axis, Q *y) {
+    if (!ctx) return ZANT_NullPointer;
+    AxisGeom g;
+    int rc = axis_geom(xdim, rank, n_scale, axis, &g);
+    if (rc) return rc;
+    if (g.n == 0) return ZANT_OK;
+    if (!x || !y || !y_scale) return ZANT_NullPointer;
+    KernelTimer kt(ctx);
+    hipLaunchKernelGGL(quantize_kernel<Q>, dim3(grid_for(g.n, kThreads, ctx->num_cus)), dim3(kThreads), 0, ctx->stream, x, y_scale,
+                       y_zp, y, g);
+    ZANT_LAUNCH_CHECK(ctx);
+    return ZANT_OK;
+}
+
+template <typename Q>
+int launch_dequantize(zant_ctx *ctx, const Q *x, const int64_t *xdim, int rank, const float *x_scale, const Q *x_zp,
+                      int64_t n_scale, int axis, float *y) {
+    if (!ctx) return ZANT_NullPointer;
+    AxisGeom g;
+    int rc = axis_geom(xdim, rank, n_scale, axis, &g);
+    if (rc) return rc;
+    if (g.n == 0) return ZANT_OK;
+    if (!x || !y || !x_scale) return ZANT_NullPointer;
+    KernelTimer kt(ctx);
+    hipLaunchKernelGGL(dequantize_kernel<Q>, dim3(grid_for(g.n, kThreads, ctx->num_cus)), dim3(kThreads), 0, ctx->stream, x,
                        x_scale, x_zp, y, g);
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
+}
+
+}  // namespace
+
+extern "C" int zant_hip_quantize_linear_f32_i8(zant_ctx *ctx, const float *x, const int64_t *xdim, int rank,
+                                               const float *y_scale, const int8_t *y_zp, int64_t n_scale, int axis, int8_t *y) {
+    return launch_quantize<int8_t>(ctx, x, xdim, rank, y_scale, y_zp, n_scale, axis, y);
+}
+
+extern "C" int zant_hip_dequantize_linear_i8_f32(zant_ctx *ctx, const int8_t *x, const int64_t *xdim, int rank,
+                                                 const float *x_scale, const int8_t *x_zp, int64_t n_scale, int axis, float *y) {
+    return launch_dequantize<int8_t>(ctx, x, xdim, rank, x_scale, x_zp, n_scale, axis, y);
+}
+
+extern "C" int zant_hip_dequantize_linear_i32_f32(zant_ctx *ctx, const int32_t *x, const int64_t *xdim, int rank,
+                                                  const float *x_scale, const int32_t *x_zp, int64_t n_scale, int axis, float *y) {
+    return launch_dequantize<int32_t>(ctx, x, xdim, rank, x_scale, x_zp, n_scale, axis, y);
 }
 
 int zant_qlinear_act_flip(zant_ctx *ctx, const uint8_t *x, int64_t n, float x_scale, uint8_t x_zp, int act, float alpha,

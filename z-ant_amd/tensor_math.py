@@ -233,23 +233,30 @@ def _scalar_tensor(v, dtype, device):
     return torch.as_tensor(v, dtype=dtype, device=device).reshape(-1).contiguous()
 
 
-def quantize_linear(x, y_scale, y_zp=None, axis=1):
+def quantize_linear(x, y_scale, y_zp=None, axis=1, signed=False):
+    """signed (or an int8 zero point tensor): int8 codes saturating to [-128, 127]; otherwise uint8."""
     ctx = context()
+    signed = signed or (torch.is_tensor(y_zp) and y_zp.dtype == torch.int8)
+    dt = torch.int8 if signed else torch.uint8
     s = _scalar_tensor(y_scale, torch.float32, x.device)
-    zp = None if y_zp is None else _scalar_tensor(y_zp, torch.uint8, x.device)
-    y = torch.zeros(x.shape, dtype=torch.uint8, device=x.device)
+    zp = None if y_zp is None else _scalar_tensor(y_zp, dt, x.device)
+    y = torch.zeros(x.shape, dtype=dt, device=x.device)
     xd, r = dims(x.shape)
-    ctx.check(lib.zant_hip_quantize_linear_f32_u8(ctx.handle, _p(x), xd, r, _p(s), _p(zp), s.numel(), axis, _p(y)))
+    fn = lib.zant_hip_quantize_linear_f32_i8 if signed else lib.zant_hip_quantize_linear_f32_u8
+    ctx.check(fn(ctx.handle, _p(x), xd, r, _p(s), _p(zp), s.numel(), axis, _p(y)))
     return y
 
 
 def dequantize_linear(x, x_scale, x_zp=None, axis=1):
+    """x: uint8, int8 or int32 codes (the zero point has x's type)."""
     ctx = context()
     s = _scalar_tensor(x_scale, torch.float32, x.device)
-    zp = None if x_zp is None else _scalar_tensor(x_zp, torch.uint8, x.device)
+    zp = None if x_zp is None else _scalar_tensor(x_zp, x.dtype, x.device)
     y = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
     xd, r = dims(x.shape)
-    ctx.check(lib.zant_hip_dequantize_linear_u8_f32(ctx.handle, _p(x), xd, r, _p(s), _p(zp), s.numel(), axis, _p(y)))
+    fn = {torch.uint8: lib.zant_hip_dequantize_linear_u8_f32, torch.int8: lib.zant_hip_dequantize_linear_i8_f32,
+          torch.int32: lib.zant_hip_dequantize_linear_i32_f32}[x.dtype]
+    ctx.check(fn(ctx.handle, _p(x), xd, r, _p(s), _p(zp), s.numel(), axis, _p(y)))
     return y
 
 
