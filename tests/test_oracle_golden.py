@@ -165,3 +165,40 @@ def test_onnx_reader_decodes_the_bundled_mnist8_graph():
     assert shapes["Parameter5"] == (8, 1, 5, 5) and shapes["Parameter87"] == (16, 8, 5, 5)
     assert shapes["Parameter6"] == (8, 1, 1) and shapes["Parameter193"] == (16, 4, 4, 10) and shapes["Parameter194"] == (1, 10)
     assert g["inputs"] == [("Input3", [1, 1, 28, 28])] and g["outputs"] == [("Plus214_Output_0", [1, 10])]
+
+
+def test_onnx_reader_decodes_a_quantised_graph_written_by_the_test_writer(tmp_path):
+    """Round trip through the wire format without a GPU: node list, attributes, typed initialisers, element types."""
+    import importlib.util
+    import os
+    import sys
+    import onnx_writer
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("zant_onnx_front", os.path.join(root, "z-ant_amd", "onnx_front.py"))
+    front = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(front)
+    arch = dict(name="t", input=(3, 8, 8), layers=[
+        dict(op="conv", k=3, stride=2, pad=1, cin=3, cout=8, group=1, act="leaky", alpha=0.1),
+        dict(op="pool"),
+        dict(op="conv", k=1, stride=1, pad=0, cin=8, cout=8, group=1, act="relu6"),
+        dict(op="add", res=1),
+        dict(op="gap")])
+    g = np.random.default_rng(0)
+    params = [dict(w=g.integers(-127, 128, (8, 3, 3, 3), dtype=np.int8), w_scale=g.random(8, dtype=np.float32), bias=g.integers(-9, 9, 8, dtype=np.int32)),
+              None, dict(w=g.integers(-127, 128, (8, 8, 1, 1), dtype=np.int8), w_scale=g.random(8, dtype=np.float32), bias=g.integers(-9, 9, 8, dtype=np.int32)),
+              None, None]
+    quant = {"input": [0.02, 128], "layers": [[0.05, 128, 0.04, 30], None, [0.06, 120, 0.03, 0], [0.07, 100], [0.07, 100]]}
+    data, shape = onnx_writer.int8_network(arch, params, quant, 2)
+    path = tmp_path / "q.onnx"
+    path.write_bytes(data)
+    graph = front.read_graph(str(path))
+    ops = [n["op"] for n in graph["nodes"]]
+    assert ops == ["QLinearConv", "DequantizeLinear", "LeakyRelu", "QuantizeLinear", "MaxPool", "QLinearConv", "DequantizeLinear",
+                   "Clip", "QuantizeLinear", "QLinearAdd", "QLinearGlobalAveragePool"]
+    assert graph["elem_types"]["input"] == 2 and graph["inputs"][0][1] == [2, 3, 8, 8] and tuple(graph["outputs"][0][1]) == shape
+    conv = graph["nodes"][0]
+    assert conv["attrs"]["strides"] == [2, 2] and conv["attrs"]["pads"] == [1, 1, 1, 1] and conv["attrs"]["group"] == 1
+    np.testing.assert_array_equal(graph["initializers"][conv["inputs"][3]], params[0]["w"])
+    np.testing.assert_array_equal(graph["initializers"][conv["inputs"][8]], params[0]["bias"])
+    assert graph["initializers"][conv["inputs"][1]].dtype == np.float32 and graph["initializers"][conv["inputs"][2]].dtype == np.uint8
+    assert abs(graph["nodes"][2]["attrs"]["alpha"] - 0.1) < 1e-7

@@ -3,7 +3,10 @@ package), folds Reshape on initialisers, and builds a ``Model`` (the executor be
 
 The reference parses ONNX in Zig (src/onnx/protobuf.zig:31-203, src/onnx/onnx.zig) and turns each node into one
 ``tensMath.*_lean`` call (src/codeGen/math_handler.zig:31-108); this does the same for Conv, Add, Relu, LeakyRelu,
-MaxPool, Reshape, MatMul, Gemm and Softmax, which covers the bundled mnist-8 network.
+MaxPool, Reshape, MatMul, Gemm and Softmax, which covers the bundled mnist-8 network, and for quantised graphs in
+operator form: QuantizeLinear, DequantizeLinear, QLinearConv, MaxPool on u8, QLinearAdd and
+QLinearGlobalAveragePool (com.microsoft), and the activation idiom DequantizeLinear -> Relu | LeakyRelu | Clip(0, 6)
+-> QuantizeLinear, which becomes one quantised activation node (the executor then folds it into the convolution).
 """
 import struct
 
@@ -125,7 +128,7 @@ def _node(buf):
 
 
 def _value_info(buf):
-    name, dims = "", []
+    name, dims, elem = "", [], 1
     for num, _, val in _fields(buf):
         if num == 1:
             name = bytes(val).decode()
@@ -133,7 +136,9 @@ def _value_info(buf):
             for n2, _, v2 in _fields(val):
                 if n2 == 1:  # tensor_type
                     for n3, _, v3 in _fields(v2):
-                        if n3 == 2:  # shape
+                        if n3 == 1:
+                            elem = int(v3)
+                        elif n3 == 2:  # shape
                             for n4, _, v4 in _fields(v3):
                                 if n4 == 1:  # dim
                                     d = 1
@@ -141,11 +146,12 @@ def _value_info(buf):
                                         if n5 == 1:
                                             d = v5
                                     dims.append(int(d))
-    return name, dims
+    return name, dims, elem
 
 
 def read_graph(path):
-    """-> {"nodes": [...], "initializers": {name: ndarray}, "inputs": [(name, dims)], "outputs": [(name, dims)]}"""
+    """-> {"nodes": [...], "initializers": {name: ndarray}, "inputs": [(name, dims)], "outputs": [(name, dims)],
+    "elem_types": {name: ONNX element type of a graph input / output}}"""
     buf = memoryview(open(path, "rb").read())
     graph = None
     for num, _, val in _fields(buf):
@@ -153,17 +159,17 @@ def read_graph(path):
             graph = val
     if graph is None:
         raise ValueError("no graph in the ONNX file")
-    g = {"nodes": [], "initializers": {}, "inputs": [], "outputs": []}
+    g = {"nodes": [], "initializers": {}, "inputs": [], "outputs": [], "elem_types": {}}
     for num, _, val in _fields(graph):
         if num == 1:
             g["nodes"].append(_node(val))
         elif num == 5:
             name, arr = _tensor(val)
             g["initializers"][name] = arr
-        elif num == 11:
-            g["inputs"].append(_value_info(val))
-        elif num == 12:
-            g["outputs"].append(_value_info(val))
+        elif num in (11, 12):
+            name, dims, elem = _value_info(val)
+            g["inputs" if num == 11 else "outputs"].append((name, dims))
+            g["elem_types"][name] = elem
     g["inputs"] = [(n, d) for n, d in g["inputs"] if n not in g["initializers"]]
     return g
 
@@ -212,17 +218,44 @@ def run_graph(graph, ops, x):
 def build_model(ctx, graph):
     """Turns the graph into a finalized ``Model``: one executor node per ONNX node, initialisers as parameters, Reshape
     of an initialiser folded on the host (as the reference's code generator does for constant inputs)."""
-    from .model import Model
+    from .model import Model, U8
     m = Model(ctx)
     consts = dict(graph["initializers"])
     name, dims = graph["inputs"][0]
-    tens = {name: m.input(tuple(dims))}
+    nodes = graph["nodes"]
+    readers = {}  # tensor name -> indices of the nodes that read it
+    for k, nd in enumerate(nodes):
+        for n in nd["inputs"]:
+            readers.setdefault(n, []).append(k)
+    qparams = {}  # name of a u8 tensor -> (scale, zero point)
+    if graph["elem_types"].get(name, 1) == 2:
+        # a u8 graph input carries no quantisation parameters of its own: they are those its first reader names
+        first = nodes[readers[name][0]]
+        if first["op"] not in ("QLinearConv", "DequantizeLinear", "QLinearAdd", "QLinearGlobalAveragePool"):
+            raise NotImplementedError("a uint8 graph input must feed a quantised operator")
+        sc = float(consts[first["inputs"][1]].reshape(-1)[0])
+        zp = int(consts[first["inputs"][2]].reshape(-1)[0]) if len(first["inputs"]) > 2 and first["inputs"][2] else 0
+        tens = {name: m.input(tuple(dims), U8, sc, zp)}
+        qparams[name] = (sc, zp)
+    else:
+        tens = {name: m.input(tuple(dims))}
 
     def reshape_const(arr, shape):
         shape = [arr.shape[k] if v == 0 else int(v) for k, v in enumerate(shape)]
         return arr.reshape(shape)
 
-    for nd in graph["nodes"]:
+    def scalar(n, default=0):
+        return default if not n else consts[n].reshape(-1)[0]
+
+    def check_q(n, scale_name, zp_name):
+        sc, zp = qparams[n]
+        if np.float32(scalar(scale_name)) != np.float32(sc) or int(scalar(zp_name)) != zp:
+            raise ValueError(f"{n}: quantisation parameters differ from those of its producer")
+
+    skip = set()
+    for k, nd in enumerate(nodes):
+        if k in skip:
+            continue
         ins, a, out = nd["inputs"], nd["attrs"], nd["outputs"][0]
         op = nd["op"]
         if op == "Reshape" and ins[0] in consts:
@@ -249,6 +282,8 @@ def build_model(ctx, graph):
             s, p, d, ap = _pool_or_conv_attrs(a, [1, 1])
             t = m.maxpool(tens[ins[0]], a["kernel_shape"], s, d, p if p is not None else [0, 0, 0, 0], ap,
                           bool(a.get("ceil_mode", 0)))
+            if ins[0] in qparams:
+                qparams[out] = qparams[ins[0]]
         elif op == "Reshape":
             t = m.reshape(tens[ins[0]], [int(v) for v in consts[ins[1]]])
         elif op == "MatMul":
@@ -259,6 +294,64 @@ def build_model(ctx, graph):
                        bool(a.get("transA", 0)), bool(a.get("transB", 0)))
         elif op == "Softmax":
             t = m.softmax(tens[ins[0]])
+        elif op == "QuantizeLinear":
+            sc, zp = float(scalar(ins[1])), int(scalar(ins[2] if len(ins) > 2 else ""))
+            t = m.quantize(tens[ins[0]], sc, zp)
+            qparams[out] = (sc, zp)
+        elif op == "DequantizeLinear":
+            check_q(ins[0], ins[1], ins[2] if len(ins) > 2 else "")
+            # DequantizeLinear -> activation -> QuantizeLinear with single readers in between: one quantised activation
+            fused = False
+            r1 = readers.get(out, [])
+            if len(r1) == 1 and nodes[r1[0]]["op"] in ("Relu", "LeakyRelu", "Clip"):
+                an = nodes[r1[0]]
+                r2 = readers.get(an["outputs"][0], [])
+                if len(r2) == 1 and nodes[r2[0]]["op"] == "QuantizeLinear":
+                    qn = nodes[r2[0]]
+                    act, alpha = None, 0.0
+                    if an["op"] == "Relu":
+                        act = "relu"
+                    elif an["op"] == "LeakyRelu":
+                        act, alpha = "leaky", float(an["attrs"].get("alpha", 0.01))
+                    else:
+                        lo = float(scalar(an["inputs"][1])) if len(an["inputs"]) > 1 else float(an["attrs"].get("min", -np.inf))
+                        hi = float(scalar(an["inputs"][2])) if len(an["inputs"]) > 2 else float(an["attrs"].get("max", np.inf))
+                        if lo == 0.0 and hi == 6.0:
+                            act = "relu6"
+                    if act is not None:
+                        sc, zp = float(scalar(qn["inputs"][1])), int(scalar(qn["inputs"][2] if len(qn["inputs"]) > 2 else ""))
+                        t = m.qlinear_act(tens[ins[0]], act, alpha, sc, zp)
+                        out = qn["outputs"][0]
+                        qparams[out] = (sc, zp)
+                        skip.update((r1[0], r2[0]))
+                        fused = True
+            if not fused:
+                t = m.dequantize(tens[ins[0]])
+        elif op == "QLinearConv":
+            check_q(ins[0], ins[1], ins[2])
+            if ins[5] and np.any(consts[ins[5]] != 0):
+                raise NotImplementedError("QLinearConv with a non-zero weight zero point")
+            s, p, d, ap = _pool_or_conv_attrs(a, [1, 1])
+            if ap != "NOTSET":
+                raise NotImplementedError("QLinearConv with auto_pad")
+            sc, zp = float(scalar(ins[6])), int(scalar(ins[7]))
+            bias = consts[ins[8]] if len(ins) > 8 and ins[8] else None
+            t = m.qlinearconv(tens[ins[0]], consts[ins[3]], consts[ins[4]], bias, sc, zp, s, p if p is not None else [0, 0, 0, 0],
+                              d, a.get("group", 1))
+            qparams[out] = (sc, zp)
+        elif op == "QLinearAdd":
+            check_q(ins[0], ins[1], ins[2])
+            check_q(ins[3], ins[4], ins[5])
+            sc, zp = float(scalar(ins[6])), int(scalar(ins[7]))
+            t = m.qlinear_add(tens[ins[0]], tens[ins[3]], sc, zp)
+            qparams[out] = (sc, zp)
+        elif op == "QLinearGlobalAveragePool":
+            check_q(ins[0], ins[1], ins[2])
+            if a.get("channels_last", 0):
+                raise NotImplementedError("QLinearGlobalAveragePool with channels_last")
+            sc, zp = float(scalar(ins[3])), int(scalar(ins[4]))
+            t = m.qlinear_global_avgpool(tens[ins[0]], sc, zp)
+            qparams[out] = (sc, zp)
         else:
             raise NotImplementedError(f"ONNX operator {op} is outside the hot path")
         tens[out] = t
