@@ -225,7 +225,18 @@ def main():
         hbm("add_f32_same_shape", lambda: tm.sum_tensors_lean(xf, bf, yf), 3 * xf.numel() * 4)
         bc = torch.randn(32, 1, 1, device=dev)
         hbm("add_f32_per_channel_broadcast", lambda: tm.sum_tensors_lean(xf, bc, yf), 2 * xf.numel() * 4)
+        hbm("sigmoid_f32_4096x32x26x26", lambda: tm.sigmoid_lean(xf, yf), 2 * xf.numel() * 4)
         del bf, yp
+        gx = torch.randn(256, 64, 56, 56, device=dev)
+        gy = torch.empty(256, 64, 1, 1, device=dev)
+        hbm("reduce_mean_hw_f32_256x64x56x56", lambda: tm.reduce_mean_lean(gx, gy, [2, 3], True), gx.numel() * 4 + gy.numel() * 4)
+        cy = torch.empty(256, 128, 56, 56, device=dev)
+        hbm("concat_channels_f32_2x256x64x56x56", lambda: tm.lean_concatenate([gx, gx], 1, cy), 2 * cy.numel() * 4)
+        del cy
+        rx = torch.randn(256, 64, 28, 28, device=dev)
+        hbm("resize_nearest_x2_f32_256x64x28x28", lambda: tm.resize(rx, "nearest", [1.0, 1.0, 2.0, 2.0], None, "asymmetric"),
+            5 * rx.numel() * 4)
+        del gx, gy, rx
         sm = torch.randn(1 << 20, 10, device=dev)
         so = torch.empty_like(sm)
         hbm("softmax_f32_1Mx10", lambda: tm.softmax_lean(sm, so), 2 * sm.numel() * 4)

@@ -46,6 +46,12 @@ enum zant_status {
     ZANT_InputArrayWrongSize = -11,         /* TensorError.InputArrayWrongSize */
     ZANT_WrongStride = -12,                 /* TensorMathError.WrongStride */
     ZANT_MemError = -13,                    /* TensorMathError.MemError (host or device allocation) */
+    ZANT_InvalidAxes = -14,                 /* TensorMathError.InvalidAxes */
+    ZANT_AxisOutOfBounds = -15,             /* TensorError.AxisOutOfBounds */
+    ZANT_MismatchedShape = -16,             /* TensorError.MismatchedShape */
+    ZANT_MismatchedRank = -17,              /* TensorError.MismatchedRank */
+    ZANT_EmptyTensorList = -18,             /* TensorMathError.EmptyTensorList */
+    ZANT_UnsupportedMode = -19,             /* TensorError.UnsupportedMode */
     ZANT_HipError = -100,                   /* a HIP runtime call failed; see zant_hip_last_error() */
     ZANT_NullPointer = -101,
     ZANT_ArenaOverflow = -102,
@@ -148,6 +154,8 @@ int zant_hip_maxpool2d_out_shape(const int64_t xdim[4], const int64_t kernel[2],
 int zant_hip_relu_f32(zant_ctx *ctx, const float *x, float *y, int64_t n);
 /* leakyReLU_lean (:68-77): x <= 0 ? slope*x : x. */
 int zant_hip_leaky_relu_f32(zant_ctx *ctx, const float *x, float slope, float *y, int64_t n);
+/* sigmoid_lean (:107-122): 1 / (1 + exp(-x)). */
+int zant_hip_sigmoid_f32(zant_ctx *ctx, const float *x, float *y, int64_t n);
 /* softmax_lean (:154-187): rows = shape[0], cols = shape[1]. */
 int zant_hip_softmax_f32(zant_ctx *ctx, const float *x, float *y, int64_t rows, int64_t cols);
 /* sum_tensors_lean (lib_elementWise_math.zig:70-210): same-size add, else
@@ -158,6 +166,30 @@ int zant_hip_add_f32(zant_ctx *ctx, const float *a, const int64_t *adim, int a_r
 /* add_bias (lib_elementWise_math.zig:22-45), in place over the last axis. */
 int zant_hip_add_bias_f32(zant_ctx *ctx, float *t, const int64_t *tdim, int t_rank, const float *bias,
                           const int64_t *bdim, int b_rank);
+/* reduce_mean / lean_reduce_mean (lib_reduction_math.zig:30-268).  axes NULL or
+ * n_axes 0: a copy when noop_with_empty_axes, else the mean of everything (shape
+ * all ones with keepdims, else [1]).  Negative axes count from the end; an axis
+ * outside the rank, or named twice, is ZANT_InvalidAxes.  The output shape goes
+ * to ydim_out / y_rank_out (room for 8); y == NULL asks for the shape only.
+ * Sums run in f32 like the reference's, in a different order (tree / lanes). */
+int zant_hip_reduce_mean_f32(zant_ctx *ctx, const float *x, const int64_t *xdim, int rank, const int64_t *axes,
+                             int n_axes, int keepdims, int noop_with_empty_axes, float *y, int64_t *ydim_out,
+                             int *y_rank_out);
+/* concatenate / lean_concatenate and get_concatenate_output_shape
+ * (lib_shape_math.zig:307-461, 463-580, 582-630) for elements of 1, 2, 4 or 8
+ * bytes, up to 16 inputs.  Lower-rank inputs get leading ones as in
+ * lean_concatenate (:335-358).  y == NULL asks for the shape only. */
+int zant_hip_concatenate(zant_ctx *ctx, const void *const *xs, const int64_t *const *dims, const int *ranks, int n,
+                         int64_t axis, size_t elem_size, void *y, int64_t *ydim_out, int *y_rank_out);
+/* resize(mode "nearest") and get_resize_output_shape (lib_shape_math.zig:22-160):
+ * exactly one of scales / sizes, each of length rank (else ZANT_InvalidInput);
+ * coord_mode 0 half_pixel, 1 align_corners, anything else asymmetric, as the
+ * reference's string comparison falls through; indices computed in f32 and
+ * rounded half away from zero, as there.  Elements of 1, 2, 4 or 8 bytes.
+ * The "linear" and "cubic" modes are not provided.  y == NULL: shape only. */
+int zant_hip_resize_nearest(zant_ctx *ctx, const void *x, const int64_t *xdim, int rank, size_t elem_size,
+                            const float *scales, const int64_t *sizes, int n_param, int coord_mode, void *y,
+                            int64_t *ydim_out);
 /* reshape_lean (lib_shape_math.zig:1139-1209): resolves 0 / -1 entries into
  * ydim_out and copies the data unless y == x (a view). */
 int zant_hip_reshape(zant_ctx *ctx, const void *x, const int64_t *xdim, int x_rank, size_t elem_size,

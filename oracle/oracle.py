@@ -20,7 +20,8 @@ ERR = {
     0: "OK", -1: "InvalidDimensions", -2: "InvalidPadding", -3: "InputTensorsWrongShape",
     -4: "InputTensorDifferentShape", -5: "InputTensorDimensionMismatch", -6: "IncompatibleBroadcastShapes",
     -7: "InputTensorDifferentSize", -8: "EmptyTensor", -9: "ZeroSizeTensor", -10: "InvalidInput",
-    -11: "InputArrayWrongSize", -12: "WrongStride", -13: "MemError",
+    -11: "InputArrayWrongSize", -12: "WrongStride", -13: "MemError", -14: "InvalidAxes", -15: "AxisOutOfBounds",
+    -16: "MismatchedShape", -17: "MismatchedRank", -18: "EmptyTensorList", -19: "UnsupportedMode",
 }
 PAD = {"NOTSET": 0, "SAME_UPPER": 1, "SAME_LOWER": 2, "VALID": 3}
 ACT = {None: 0, "none": 0, "relu": 1, "leaky": 2, "relu6": 3}
@@ -220,6 +221,74 @@ def softmax(x):
     if x.size == 0:
         raise OracleError(-9)
     return softmax_lean(x, np.zeros(x.shape, np.float32))
+
+
+def sigmoid_lean(x, y):
+    x = _f32(x)
+    _chk(_lib.zo_sigmoid_lean_f32(_ptr(x), _ptr(y), C.c_int64(x.size)))
+    return y
+
+
+def sigmoid(x):
+    if x.size == 0:
+        raise OracleError(-9)
+    return sigmoid_lean(x, np.zeros(x.shape, np.float32))
+
+
+def reduce_mean(x, axes=None, keepdims=True, noop_with_empty_axes=False):
+    x = _f32(x)
+    xd, xr = _dims(x.shape)
+    ax = (C.c_int64 * max(len(axes), 1))(*axes) if axes is not None else None
+    na = len(axes) if axes is not None else 0
+    yd = (C.c_int64 * 8)(); yr = C.c_int()
+    _chk(_lib.zo_reduce_mean_f32(_ptr(x), xd, xr, ax, na, int(keepdims), int(noop_with_empty_axes), None, yd, C.byref(yr)))
+    y = np.zeros(tuple(yd)[:yr.value], np.float32)
+    _chk(_lib.zo_reduce_mean_f32(_ptr(x), xd, xr, ax, na, int(keepdims), int(noop_with_empty_axes), _ptr(y), yd, C.byref(yr)))
+    return y
+
+
+def _tensor_list(tensors):
+    n = len(tensors)
+    keep = [_dims(t.shape) for t in tensors]
+    ptrs = (C.c_void_p * max(n, 1))(*[t.ctypes.data for t in tensors])
+    dims = (C.POINTER(C.c_int64) * max(n, 1))(*[C.cast(d, C.POINTER(C.c_int64)) for d, _ in keep])
+    ranks = (C.c_int * max(n, 1))(*[r for _, r in keep])
+    return ptrs, dims, ranks, keep
+
+
+def concatenate(tensors, axis):
+    tensors = [np.ascontiguousarray(t) for t in tensors]
+    ptrs, dims, ranks, keep = _tensor_list(tensors)
+    es = tensors[0].itemsize if tensors else 4
+    yd = (C.c_int64 * 8)(); yr = C.c_int()
+    _chk(_lib.zo_concatenate(ptrs, dims, ranks, len(tensors), C.c_int64(axis), C.c_size_t(es), None, yd, C.byref(yr)))
+    y = np.zeros(tuple(yd)[:yr.value], tensors[0].dtype)
+    _chk(_lib.zo_concatenate(ptrs, dims, ranks, len(tensors), C.c_int64(axis), C.c_size_t(es), _ptr(y), yd, C.byref(yr)))
+    return y
+
+
+COORD = {"half_pixel": 0, "align_corners": 1, "asymmetric": 2}
+
+
+def resize(x, mode, scales, sizes, coordinate_transformation_mode="half_pixel"):
+    """Only the "nearest" mode is restated; other known modes raise NotImplementedError, unknown ones UnsupportedMode."""
+    x = np.ascontiguousarray(x)
+    if (scales is None) == (sizes is None):
+        raise OracleError(-10)  # before the mode is looked at (lib_shape_math.zig:23-28)
+    if mode in ("linear", "cubic"):
+        raise NotImplementedError(mode)
+    if mode != "nearest":
+        raise OracleError(-19)
+    xd, xr = _dims(x.shape)
+    sc = (C.c_float * max(len(scales), 1))(*scales) if scales is not None else None
+    sz = (C.c_int64 * max(len(sizes), 1))(*sizes) if sizes is not None else None
+    n = len(scales) if scales is not None else len(sizes)
+    cm = COORD.get(coordinate_transformation_mode, 2)
+    yd = (C.c_int64 * 8)()
+    _chk(_lib.zo_resize_nearest(_ptr(x), xd, xr, C.c_size_t(x.itemsize), sc, sz, n, cm, None, yd))
+    y = np.zeros(tuple(yd)[:x.ndim], x.dtype)
+    _chk(_lib.zo_resize_nearest(_ptr(x), xd, xr, C.c_size_t(x.itemsize), sc, sz, n, cm, _ptr(y), yd))
+    return y
 
 
 def sum_tensors_lean(a, b, y=None):

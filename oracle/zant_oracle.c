@@ -8,6 +8,9 @@
  *     pinned by the reference's own known-answer tests (transcribed under
  *     tests/golden/), by a brute-force 7-loop convolution, by numpy/scipy
  *     library routines and by closed forms (tests/test_oracle_*.py).
+ *   Sigmoid / ReduceMean / Concat / Resize(nearest): pinned by the reference's
+ *     known-answer tests (tests/golden/), numpy (mean, concatenate), scipy's
+ *     expit and closed forms (integer upscales repeat elements).
  *   broadcast Add: the reference has no test for the broadcast branch and its
  *     stride computation reads out of bounds for mid-axis broadcasts; restated
  *     to NumPy semantics and pinned by numpy.
@@ -47,6 +50,12 @@ const char *zo_error_name(int code) {
     case ZO_InputArrayWrongSize: return "InputArrayWrongSize";
     case ZO_WrongStride: return "WrongStride";
     case ZO_MemError: return "MemError";
+    case ZO_InvalidAxes: return "InvalidAxes";
+    case ZO_AxisOutOfBounds: return "AxisOutOfBounds";
+    case ZO_MismatchedShape: return "MismatchedShape";
+    case ZO_MismatchedRank: return "MismatchedRank";
+    case ZO_EmptyTensorList: return "EmptyTensorList";
+    case ZO_UnsupportedMode: return "UnsupportedMode";
     default: return "Unknown";
     }
 }
@@ -476,6 +485,136 @@ int zo_relu_lean_f32(const float *x, float *y, int64_t n) {
 
 int zo_leaky_relu_lean_f32(const float *x, float slope, float *y, int64_t n) {
     for (int64_t i = 0; i < n; ++i) y[i] = x[i] <= 0 ? slope * x[i] : x[i]; /* :70-76 */
+    return ZO_OK;
+}
+
+int zo_sigmoid_lean_f32(const float *x, float *y, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) y[i] = 1.0f / (1.0f + expf(-x[i])); /* :116-120 */
+    return ZO_OK;
+}
+
+int zo_reduce_mean_f32(const float *x, const int64_t *xdim, int rank, const int64_t *axes, int n_axes, int keepdims,
+                       int noop_with_empty_axes, float *y, int64_t *ydim_out, int *y_rank_out) {
+    if (rank < 0 || rank > 8) return ZO_InvalidDimensions;
+    int64_t size = 1;
+    for (int i = 0; i < rank; ++i) size *= xdim[i];
+    if (!axes || n_axes == 0) { /* lib_reduction_math.zig:35-46, 111-128 */
+        if (noop_with_empty_axes) {
+            for (int i = 0; i < rank; ++i) ydim_out[i] = xdim[i];
+            *y_rank_out = rank;
+            if (y) memcpy(y, x, (size_t)size * sizeof(float));
+            return ZO_OK;
+        }
+        if (keepdims) { for (int i = 0; i < rank; ++i) ydim_out[i] = 1; *y_rank_out = rank; }
+        else { ydim_out[0] = 1; *y_rank_out = 1; }
+        if (y) {
+            float sum = 0.0f;
+            for (int64_t i = 0; i < size; ++i) sum += x[i];
+            y[0] = sum / (float)size;
+        }
+        return ZO_OK;
+    }
+    int reduced[8] = {0};
+    int64_t ax[8];
+    if (n_axes > 8) return ZO_InvalidAxes;
+    for (int i = 0; i < n_axes; ++i) { /* :131-141 */
+        const int64_t a = axes[i] < 0 ? axes[i] + rank : axes[i];
+        if (a < 0 || a >= rank || reduced[a]) return ZO_InvalidAxes;
+        reduced[a] = 1;
+        ax[i] = a;
+    }
+    int out_rank = 0, n_rem = 0, rem[8];
+    for (int i = 0; i < rank; ++i) { /* :62-76 */
+        if (!reduced[i] || keepdims) ydim_out[out_rank++] = reduced[i] ? 1 : xdim[i];
+        if (!reduced[i]) rem[n_rem++] = i;
+    }
+    *y_rank_out = out_rank;
+    if (!y) return ZO_OK;
+    int64_t istr[8], count = 1, out_size = 1;
+    { int64_t st = 1; for (int i = rank - 1; i >= 0; --i) { istr[i] = st; st *= xdim[i]; } }
+    for (int i = 0; i < n_axes; ++i) count *= xdim[ax[i]];
+    for (int i = 0; i < n_rem; ++i) out_size *= xdim[rem[i]];
+    /* reduced extents innermost first: the last listed axis varies fastest (:236-243) */
+    int64_t rsize[8], rstr[8];
+    for (int i = 0; i < n_axes; ++i) { rsize[n_axes - 1 - i] = xdim[ax[i]]; rstr[n_axes - 1 - i] = istr[ax[i]]; }
+    for (int64_t o = 0; o < out_size; ++o) {
+        int64_t r = o, base = 0;
+        for (int i = n_rem - 1; i >= 0; --i) { base += (r % xdim[rem[i]]) * istr[rem[i]]; r /= xdim[rem[i]]; }
+        float sum = 0.0f;
+        for (int64_t k = 0; k < count; ++k) { /* :246-258 */
+            int64_t t = k, off = base;
+            for (int i = 0; i < n_axes; ++i) { off += (t % rsize[i]) * rstr[i]; t /= rsize[i]; }
+            sum += x[off];
+        }
+        y[o] = sum / (float)count; /* :266 */
+    }
+    return ZO_OK;
+}
+
+int zo_concatenate(const void *const *xs, const int64_t *const *dims, const int *ranks, int n, int64_t axis,
+                   size_t elem_size, void *y, int64_t *ydim_out, int *y_rank_out) {
+    if (n <= 0) return ZO_EmptyTensorList; /* lib_shape_math.zig:308 */
+    int rank = 0;
+    for (int t = 0; t < n; ++t) if (ranks[t] > rank) rank = ranks[t]; /* :314-320 */
+    if (rank > 8) return ZO_InvalidDimensions;
+    if (axis < 0) axis += rank; /* :363-370 */
+    if (axis < 0 || axis >= rank) return ZO_AxisOutOfBounds;
+    int64_t shp[16][8];
+    if (n > 16) return ZO_InvalidDimensions;
+    for (int t = 0; t < n; ++t) { /* leading ones, :335-358 */
+        const int off = rank - ranks[t];
+        for (int d = 0; d < rank; ++d) shp[t][d] = d < off ? 1 : dims[t][d - off];
+    }
+    int64_t total = 0;
+    for (int t = 0; t < n; ++t) { /* :374-380 */
+        for (int d = 0; d < rank; ++d)
+            if (d != axis && shp[t][d] != shp[0][d]) return ZO_MismatchedShape;
+        total += shp[t][axis];
+    }
+    for (int d = 0; d < rank; ++d) ydim_out[d] = d == axis ? total : shp[0][d];
+    *y_rank_out = rank;
+    if (!y) return ZO_OK;
+    int64_t slices = 1, inner = 1;
+    for (int d = 0; d < axis; ++d) slices *= shp[0][d];
+    for (int d = (int)axis + 1; d < rank; ++d) inner *= shp[0][d];
+    char *dst = (char *)y;
+    for (int64_t sl = 0; sl < slices; ++sl) /* :398-424 */
+        for (int t = 0; t < n; ++t) {
+            const size_t bytes = (size_t)(shp[t][axis] * inner) * elem_size;
+            memcpy(dst, (const char *)xs[t] + (size_t)sl * bytes, bytes);
+            dst += bytes;
+        }
+    return ZO_OK;
+}
+
+int zo_resize_nearest(const void *x, const int64_t *xdim, int rank, size_t elem_size, const float *scales,
+                      const int64_t *sizes, int n_param, int coord_mode, void *y, int64_t *ydim_out) {
+    if ((!scales && !sizes) || (scales && sizes)) return ZO_InvalidInput; /* lib_shape_math.zig:23-28 */
+    if (n_param != rank || rank < 1 || rank > 8) return ZO_InvalidInput;  /* :35-37, 43-45 */
+    for (int i = 0; i < rank; ++i)
+        ydim_out[i] = scales ? (int64_t)floorf((float)xdim[i] * scales[i]) : sizes[i]; /* :38-40 */
+    if (!y) return ZO_OK;
+    int64_t istr[8], total = 1;
+    { int64_t st = 1; for (int i = rank - 1; i >= 0; --i) { istr[i] = st; st *= xdim[i]; } }
+    for (int i = 0; i < rank; ++i) total *= ydim_out[i];
+    for (int64_t o = 0; o < total; ++o) {
+        int64_t r = o, in_idx = 0;
+        for (int i = rank - 1; i >= 0; --i) {
+            const int64_t oi = r % ydim_out[i];
+            r /= ydim_out[i];
+            const float scale = (float)ydim_out[i] / (float)xdim[i]; /* :130 */
+            float pos;
+            if (coord_mode == 0) pos = ((float)oi + 0.5f) / scale - 0.5f; /* :133-134 */
+            else if (coord_mode == 1) pos = (float)oi * (float)(xdim[i] - 1) / (float)(ydim_out[i] - 1); /* :136 */
+            else pos = (float)oi / scale; /* :138 */
+            if (!(pos == pos)) pos = 0.0f; /* 0 / 0 of a one-element axis under align_corners */
+            int64_t ii = (int64_t)roundf(pos); /* @round: half away from zero (:141) */
+            if (ii < 0) ii = 0;
+            if (ii > xdim[i] - 1) ii = xdim[i] - 1;
+            in_idx += ii * istr[i];
+        }
+        memcpy((char *)y + (size_t)o * elem_size, (const char *)x + (size_t)in_idx * elem_size, elem_size);
+    }
     return ZO_OK;
 }
 

@@ -46,7 +46,13 @@ enum {
     ZO_InvalidInput = -10,
     ZO_InputArrayWrongSize = -11,
     ZO_WrongStride = -12,
-    ZO_MemError = -13
+    ZO_MemError = -13,
+    ZO_InvalidAxes = -14,       /* TensorMathError.InvalidAxes */
+    ZO_AxisOutOfBounds = -15,   /* TensorError.AxisOutOfBounds */
+    ZO_MismatchedShape = -16,   /* TensorError.MismatchedShape */
+    ZO_MismatchedRank = -17,    /* TensorError.MismatchedRank */
+    ZO_EmptyTensorList = -18,   /* TensorMathError.EmptyTensorList */
+    ZO_UnsupportedMode = -19    /* TensorError.UnsupportedMode */
 };
 
 /* AutoPadType, op_pooling.zig:9-14 (same numbering). */
@@ -101,6 +107,29 @@ int zo_relu_lean_f32(const float *x, float *y, int64_t n);
 int zo_leaky_relu_lean_f32(const float *x, float slope, float *y, int64_t n);
 /* lean_softmax (:154-187): rows = shape[0], cols = shape[1]. */
 int zo_softmax_lean_f32(const float *x, float *y, int64_t rows, int64_t cols);
+/* sigmoid_lean (lib_activation_function_math.zig:107-122): 1 / (1 + exp(-x)). */
+int zo_sigmoid_lean_f32(const float *x, float *y, int64_t n);
+/* reduce_mean + lean_reduce_mean (lib_reduction_math.zig:30-268).  axes NULL or
+ * n_axes 0: identity when noop_with_empty_axes, else the mean of everything
+ * (shape all ones with keepdims, else [1]).  Negative axes count from the end;
+ * an axis outside the rank is InvalidAxes.  A repeated axis is InvalidAxes here
+ * (the reference would square the reduced extent and read out of bounds).
+ * y NULL: shape only. */
+int zo_reduce_mean_f32(const float *x, const int64_t *xdim, int rank, const int64_t *axes, int n_axes, int keepdims,
+                       int noop_with_empty_axes, float *y, int64_t *ydim_out, int *y_rank_out);
+/* concatenate / lean_concatenate + get_concatenate_output_shape
+ * (lib_shape_math.zig:307-461, 463-580, 582-630), any element width.  Lower-rank
+ * inputs are padded with leading ones as lean_concatenate does (:335-358); the
+ * output rank is the largest input rank.  y NULL: shape only. */
+int zo_concatenate(const void *const *xs, const int64_t *const *dims, const int *ranks, int n, int64_t axis,
+                   size_t elem_size, void *y, int64_t *ydim_out, int *y_rank_out);
+/* resize in "nearest" mode + get_resize_output_shape (lib_shape_math.zig:22-160):
+ * exactly one of scales / sizes (each of length rank); coordinate modes
+ * 0 half_pixel, 1 align_corners, 2 asymmetric (anything else in the reference);
+ * index = clamp(round-half-away(pos)), all in f32 as the reference computes it.
+ * y NULL: shape only. */
+int zo_resize_nearest(const void *x, const int64_t *xdim, int rank, size_t elem_size, const float *scales,
+                      const int64_t *sizes, int n_param, int coord_mode, void *y, int64_t *ydim_out);
 /* lean_sum_tensors (lib_elementWise_math.zig:70-210): same-size add, else
  * right-aligned NumPy broadcast up to rank 4.  The reference derives the
  * operand strides from the OUTPUT strides (:160-169), which indexes past the

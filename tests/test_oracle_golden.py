@@ -121,6 +121,64 @@ def test_reshape(c):
         np.testing.assert_array_equal(y.ravel(), x.ravel())
 
 
+@pytest.mark.parametrize("c", cases_for("sigmoid"))
+def test_sigmoid(c):
+    assert np.all(np.abs(zo.sigmoid(T(c["x"])) - T(c["expect"])) < c["atol"])
+
+
+@pytest.mark.parametrize("c", cases_for("reduce_mean"))
+def test_reduce_mean(c):
+    y = zo.reduce_mean(T(c["x"]), c["axes"], c["keepdims"], c["noop"])
+    if "expect" in c:
+        assert list(y.shape) == c["expect"]["shape"]
+        assert np.all(np.abs(y - T(c["expect"])) <= c["atol"])
+    else:
+        assert list(y.shape) == c["expect_shape"]
+        assert np.all(np.abs(y.ravel()[:len(c["expect_first"])] - np.array(c["expect_first"], np.float32)) <= c["atol"])
+
+
+@pytest.mark.parametrize("c", cases_for("concatenate"))
+def test_concatenate(c):
+    ts = [T(t) for t in c["tensors"]]
+    if "error" in c:
+        with pytest.raises(zo.OracleError) as e:
+            zo.concatenate(ts, c["axis"])
+        assert e.value.name == c["error"]
+        return
+    y = zo.concatenate(ts, c["axis"])
+    if "expect" in c:
+        assert list(y.shape) == c["expect"]["shape"]
+        np.testing.assert_array_equal(y, T(c["expect"]))
+    else:
+        assert list(y.shape) == c["expect_shape"]
+
+
+@pytest.mark.parametrize("c", cases_for("concatenate_shape"))
+def test_concatenate_shape(c):
+    ts = [np.zeros(s, np.float32) for s in c["shapes"]]
+    if "error" in c:
+        with pytest.raises(zo.OracleError) as e:
+            zo.concatenate(ts, c["axis"])
+        assert e.value.name == c["error"]
+    else:
+        assert list(zo.concatenate(ts, c["axis"]).shape) == c["expect_shape"]
+
+
+@pytest.mark.parametrize("c", cases_for("resize", "resize_shape"))
+def test_resize(c):
+    x = T(c["x"], np.uint8) if "x" in c else np.zeros(c["shape"], np.uint8)
+    args = (x, c.get("mode", "nearest"), c["scales"], c["sizes"], c.get("coord", "half_pixel"))
+    if "error" in c:
+        with pytest.raises(zo.OracleError) as e:
+            zo.resize(*args)
+        assert e.value.name == c["error"]
+        return
+    y = zo.resize(*args)
+    assert list(y.shape) == c["expect_shape"]
+    if "expect_first" in c:
+        assert list(y.ravel()[:len(c["expect_first"])]) == c["expect_first"]
+
+
 def test_conv_error_paths():
     # group != 1 -> InvalidDimensions (op_convolution.zig:59-65)
     x, w = np.zeros((1, 2, 4, 4), np.float32), np.zeros((2, 1, 3, 3), np.float32)

@@ -187,3 +187,72 @@ def test_broadcast_add_incompatible():
     with pytest.raises(zo.OracleError) as e:
         zo.sum_tensors_lean(np.zeros((2, 3), np.float32), np.zeros((4,), np.float32))
     assert e.value.name == "IncompatibleBroadcastShapes"
+
+
+# ---- Sigmoid / ReduceMean / Concat / Resize(nearest): pinned beyond the reference's vectors by numpy / scipy / closed forms
+
+def test_sigmoid_matches_scipy_expit():
+    from scipy.special import expit
+    x = np.random.default_rng(0).standard_normal(4096).astype(np.float32) * 8
+    np.testing.assert_allclose(zo.sigmoid(x), expit(x.astype(np.float64)), rtol=1e-6, atol=1e-7)
+    assert zo.sigmoid(np.array([-200.0, 200.0], np.float32)).tolist() == [0.0, 1.0]  # exp overflow gives 1/inf, not NaN
+
+
+@pytest.mark.parametrize("shape,axes,keep", [((3, 4, 5), [1], True), ((3, 4, 5), [0, 2], False), ((2, 3, 4, 5), [2, 3], True),
+                                             ((2, 3, 4, 5), [-1, 1], False), ((6,), [0], False), ((2, 3, 4, 5), [3, 0], True)])
+def test_reduce_mean_matches_numpy(shape, axes, keep):
+    x = np.random.default_rng(1).standard_normal(shape).astype(np.float32)
+    y = zo.reduce_mean(x, axes, keep, False)
+    ref = x.astype(np.float64).mean(axis=tuple(axes), keepdims=keep)
+    assert y.shape == ref.shape
+    np.testing.assert_allclose(y, ref, rtol=1e-5, atol=1e-6)
+
+
+def test_reduce_mean_axis_errors():
+    x = np.zeros((2, 3), np.float32)
+    for axes in ([2], [-3], [0, 0]):
+        with pytest.raises(zo.OracleError) as e:
+            zo.reduce_mean(x, axes, True, False)
+        assert e.value.name == "InvalidAxes"
+    assert zo.reduce_mean(x + 2, None, False, False).shape == (1,)
+
+
+@pytest.mark.parametrize("shapes,axis", [([(2, 3, 4), (2, 5, 4), (2, 1, 4)], 1), ([(2, 3), (4, 3)], 0), ([(1, 2, 3, 4), (1, 2, 3, 1)], -1),
+                                         ([(5,), (3,)], 0)])
+def test_concatenate_matches_numpy(shapes, axis):
+    g = np.random.default_rng(2)
+    for dt in (np.float32, np.uint8):
+        ts = [(g.standard_normal(s) * 50).astype(dt) for s in shapes]
+        np.testing.assert_array_equal(zo.concatenate(ts, axis), np.concatenate(ts, axis))
+
+
+def test_concatenate_pads_lower_ranks_with_leading_ones():
+    a, b = np.arange(6, dtype=np.float32).reshape(1, 2, 3), np.arange(3, dtype=np.float32) + 10  # [1,2,3] and [3] -> [1,1,3]
+    np.testing.assert_array_equal(zo.concatenate([a, b], 1), np.concatenate([a, b.reshape(1, 1, 3)], 1))
+
+
+def test_resize_nearest_closed_forms():
+    g = np.random.default_rng(3)
+    x = g.integers(0, 255, (2, 3, 4, 5), dtype=np.uint8)
+    # half_pixel: an integer upscale repeats every element
+    y = zo.resize(x, "nearest", [1.0, 1.0, 2.0, 3.0], None, "half_pixel")
+    np.testing.assert_array_equal(y, x.repeat(2, axis=2).repeat(3, axis=3))
+    # asymmetric x2 takes round-half-away(o / 2), clamped: 0 1 1 2 2 3 3 3 on an axis of 4
+    y = zo.resize(x, "nearest", [1.0, 1.0, 2.0, 1.0], None, "asymmetric")
+    np.testing.assert_array_equal(y, x[:, :, [0, 1, 1, 2, 2, 3, 3, 3], :])
+    np.testing.assert_array_equal(zo.resize(x, "nearest", None, list(x.shape), "half_pixel"), x)  # identity
+    # asymmetric halving keeps round(2 i): every other element
+    np.testing.assert_array_equal(zo.resize(x[..., :4], "nearest", [1, 1, 0.5, 0.5], None, "asymmetric"), x[:, :, ::2, 0:4:2])
+    # align_corners maps the ends onto the ends
+    xf = g.standard_normal((1, 1, 5, 7)).astype(np.float32)
+    y = zo.resize(xf, "nearest", None, [1, 1, 9, 13], "align_corners")
+    assert y[0, 0, 0, 0] == xf[0, 0, 0, 0] and y[0, 0, -1, -1] == xf[0, 0, -1, -1] and y[0, 0, 4, 6] == xf[0, 0, 2, 3]
+    # brute force with the published formula, half_pixel, round half away from zero, clamped
+    y = zo.resize(xf, "nearest", None, [1, 1, 8, 4], "half_pixel")
+    for oh in range(8):
+        for ow in range(4):
+            ph = np.float32(np.float32(oh + 0.5) / np.float32(8 / 5)) - np.float32(0.5)
+            pw = np.float32(np.float32(ow + 0.5) / np.float32(np.float32(4) / np.float32(7))) - np.float32(0.5)
+            ih = int(min(max(np.floor(abs(ph) + 0.5) * np.sign(ph), 0), 4))
+            iw = int(min(max(np.floor(abs(pw) + 0.5) * np.sign(pw), 0), 6))
+            assert y[0, 0, oh, ow] == xf[0, 0, ih, iw]

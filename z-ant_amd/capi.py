@@ -56,6 +56,11 @@ PROTOTYPES = {
     "zant_hip_relu_f32": (i32, [vp, vp, vp, i64]),
     "zant_hip_leaky_relu_f32": (i32, [vp, vp, f32, vp, i64]),
     "zant_hip_softmax_f32": (i32, [vp, vp, vp, i64, i64]),
+    "zant_hip_sigmoid_f32": (i32, [vp, vp, vp, i64]),
+    "zant_hip_reduce_mean_f32": (i32, [vp, vp, c_i64p, i32, c_i64p, i32, i32, i32, vp, c_i64p, C.POINTER(i32)]),
+    "zant_hip_concatenate": (i32, [vp, C.POINTER(vp), C.POINTER(c_i64p), C.POINTER(i32), i32, i64, sz, vp, c_i64p,
+                                   C.POINTER(i32)]),
+    "zant_hip_resize_nearest": (i32, [vp, vp, c_i64p, i32, sz, C.POINTER(f32), c_i64p, i32, i32, vp, c_i64p]),
     "zant_hip_add_f32": (i32, [vp, vp, c_i64p, i32, vp, c_i64p, i32, vp, c_i64p, C.POINTER(i32)]),
     "zant_hip_add_bias_f32": (i32, [vp, vp, c_i64p, i32, vp, c_i64p, i32]),
     "zant_hip_reshape": (i32, [vp, vp, c_i64p, i32, sz, c_i64p, i32, vp, c_i64p]),

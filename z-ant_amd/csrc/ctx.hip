@@ -144,6 +144,12 @@ extern "C" const char *zant_hip_status_name(int s) {
     case ZANT_InputArrayWrongSize: return "InputArrayWrongSize";
     case ZANT_WrongStride: return "WrongStride";
     case ZANT_MemError: return "MemError";
+    case ZANT_InvalidAxes: return "InvalidAxes";
+    case ZANT_AxisOutOfBounds: return "AxisOutOfBounds";
+    case ZANT_MismatchedShape: return "MismatchedShape";
+    case ZANT_MismatchedRank: return "MismatchedRank";
+    case ZANT_EmptyTensorList: return "EmptyTensorList";
+    case ZANT_UnsupportedMode: return "UnsupportedMode";
     case ZANT_HipError: return "HipError";
     case ZANT_NullPointer: return "NullPointer";
     case ZANT_ArenaOverflow: return "ArenaOverflow";

@@ -17,11 +17,12 @@ inline unsigned grid_for(int64_t work_items, int per_block, int num_cus) {
 
 // ---- unary f32 ---------------------------------------------------------------------------------
 
-enum { UN_RELU = 0, UN_LEAKY = 1 };
+enum { UN_RELU = 0, UN_LEAKY = 1, UN_SIGMOID = 2 };
 
 template <int OP>
 __device__ __forceinline__ float unary_op(float v, float slope) {
     if (OP == UN_RELU) return v > 0.0f ? v : 0.0f;  // NaN -> 0, like the reference's `if (x > 0)` on a zeroed output
+    if (OP == UN_SIGMOID) return 1.0f / (1.0f + expf(-v));  // lib_activation_function_math.zig:118
     return v <= 0.0f ? slope * v : v;
 }
 
@@ -466,6 +467,10 @@ extern "C" int zant_hip_relu_f32(zant_ctx *ctx, const float *x, float *y, int64_
 
 extern "C" int zant_hip_leaky_relu_f32(zant_ctx *ctx, const float *x, float slope, float *y, int64_t n) {
     return launch_unary<UN_LEAKY>(ctx, x, y, n, slope);
+}
+
+extern "C" int zant_hip_sigmoid_f32(zant_ctx *ctx, const float *x, float *y, int64_t n) {
+    return launch_unary<UN_SIGMOID>(ctx, x, y, n, 0.0f);
 }
 
 extern "C" int zant_hip_softmax_f32(zant_ctx *ctx, const float *x, float *y, int64_t rows, int64_t cols) {

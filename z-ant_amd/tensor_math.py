@@ -184,6 +184,114 @@ def softmax(x):
     return softmax_lean(x, torch.zeros_like(x))
 
 
+def sigmoid_lean(x, y):
+    """sigmoid_lean (lib_activation_function_math.zig:107)."""
+    ctx = context()
+    ctx.check(lib.zant_hip_sigmoid_f32(ctx.handle, _p(x), _p(y), x.numel()))
+    return y
+
+
+def sigmoid(x):
+    if x.numel() == 0:
+        raise ZantError(-9)
+    return sigmoid_lean(x, torch.zeros_like(x))
+
+
+def get_reduce_mean_output_shape(xshape, axes=None, keepdims=True, noop_with_empty_axes=False):
+    xd, xr = dims(xshape); ad, na = dims(axes)
+    yd = (C.c_int64 * 8)(); yr = C.c_int()
+    rc = lib.zant_hip_reduce_mean_f32(None, None, xd, xr, ad, na, int(keepdims), int(noop_with_empty_axes), None, yd, C.byref(yr))
+    if rc:
+        raise ZantError(rc)
+    return tuple(yd)[:yr.value]
+
+
+def reduce_mean_lean(x, y, axes=None, keepdims=True, noop_with_empty_axes=False):
+    """lean_reduce_mean (lib_reduction_math.zig:87): y is pre-shaped by the caller."""
+    ctx = context()
+    xd, xr = dims(x.shape); ad, na = dims(axes)
+    yd = (C.c_int64 * 8)(); yr = C.c_int()
+    ctx.check(lib.zant_hip_reduce_mean_f32(ctx.handle, _p(x), xd, xr, ad, na, int(keepdims), int(noop_with_empty_axes), _p(y),
+                                           yd, C.byref(yr)))
+    return y
+
+
+def reduce_mean(x, axes=None, keepdims=True, noop_with_empty_axes=False):
+    """reduce_mean (lib_reduction_math.zig:30)."""
+    shape = get_reduce_mean_output_shape(x.shape, axes, keepdims, noop_with_empty_axes)
+    return reduce_mean_lean(x, torch.zeros(shape, dtype=torch.float32, device=x.device), axes, keepdims, noop_with_empty_axes)
+
+
+def _tensor_list(tensors, shapes):
+    n = len(shapes)
+    keep = [dims(s) for s in shapes]
+    ptrs = (C.c_void_p * max(n, 1))(*[t.data_ptr() if t is not None else None for t in tensors])
+    dd = (C.POINTER(C.c_int64) * max(n, 1))(*[C.cast(d, C.POINTER(C.c_int64)) for d, _ in keep])
+    rr = (C.c_int * max(n, 1))(*[r for _, r in keep])
+    return ptrs, dd, rr, keep
+
+
+def get_concatenate_output_shape(shapes, axis):
+    ptrs, dd, rr, keep = _tensor_list([None] * len(shapes), shapes)
+    yd = (C.c_int64 * 8)(); yr = C.c_int()
+    rc = lib.zant_hip_concatenate(None, ptrs, dd, rr, len(shapes), axis, 4, None, yd, C.byref(yr))
+    if rc:
+        raise ZantError(rc)
+    return tuple(yd)[:yr.value]
+
+
+def lean_concatenate(tensors, axis, y):
+    """lean_concatenate (lib_shape_math.zig:307): any element type; all inputs and y of one dtype."""
+    ctx = context()
+    for t in tensors:
+        _p(t)
+    ptrs, dd, rr, keep = _tensor_list(tensors, [t.shape for t in tensors])
+    yd = (C.c_int64 * 8)(); yr = C.c_int()
+    ctx.check(lib.zant_hip_concatenate(ctx.handle, ptrs, dd, rr, len(tensors), axis, y.element_size(), _p(y), yd, C.byref(yr)))
+    return y
+
+
+def concatenate(tensors, axis):
+    """concatenate (lib_shape_math.zig:463)."""
+    shape = get_concatenate_output_shape([t.shape for t in tensors], axis)
+    return lean_concatenate(tensors, axis, torch.zeros(shape, dtype=tensors[0].dtype, device=tensors[0].device))
+
+
+COORD = {"half_pixel": 0, "align_corners": 1, "asymmetric": 2}
+
+
+def get_resize_output_shape(xshape, scales, sizes):
+    xd, xr = dims(xshape)
+    sc = (C.c_float * max(len(scales), 1))(*scales) if scales is not None else None
+    sd, _ = dims(sizes)
+    n = len(scales) if scales is not None else (len(sizes) if sizes is not None else 0)
+    yd = (C.c_int64 * 8)()
+    rc = lib.zant_hip_resize_nearest(None, None, xd, xr, 4, sc, sd, n, 0, None, yd)
+    if rc:
+        raise ZantError(rc)
+    return tuple(yd)[:xr]
+
+
+def resize(x, mode, scales, sizes, coordinate_transformation_mode="half_pixel"):
+    """resize (lib_shape_math.zig:22) in its "nearest" mode; "linear" and "cubic" are not provided, any other mode
+    string is UnsupportedMode as in the reference.  Unknown coordinate modes mean "asymmetric" (the reference's else)."""
+    shape = get_resize_output_shape(x.shape, scales, sizes)  # InvalidInput comes before the mode is looked at (:23-28)
+    if mode in ("linear", "cubic"):
+        raise NotImplementedError(f"resize mode {mode}")
+    if mode != "nearest":
+        raise ZantError(-19)
+    ctx = context()
+    y = torch.zeros(shape, dtype=x.dtype, device=x.device)
+    xd, xr = dims(x.shape)
+    sc = (C.c_float * max(len(scales), 1))(*scales) if scales is not None else None
+    sd, _ = dims(sizes)
+    n = len(scales) if scales is not None else len(sizes)
+    yd = (C.c_int64 * 8)()
+    ctx.check(lib.zant_hip_resize_nearest(ctx.handle, _p(x), xd, xr, x.element_size(), sc, sd, n,
+                                          COORD.get(coordinate_transformation_mode, 2), _p(y), yd))
+    return y
+
+
 def sum_tensors_lean(a, b, y=None):
     ctx = context()
     ad, ar = dims(a.shape); bd, br = dims(b.shape)
