@@ -276,6 +276,14 @@ int zant_model_matmul(zant_model *m, int a, const float *b, const int64_t *bdim,
 int zant_model_add_const(zant_model *m, int x, const float *c, const int64_t *cdim, int c_rank);
 int zant_model_add(zant_model *m, int a, int b);
 int zant_model_softmax(zant_model *m, int x);
+int zant_model_sigmoid(zant_model *m, int x);
+/* ReduceMean over the given axes (GlobalAveragePool is axes {2, 3} with keepdims). */
+int zant_model_reduce_mean(zant_model *m, int x, const int64_t *axes, int n_axes, int keepdims);
+/* Concat of up to 16 tensors of one element type; quantised inputs must share scale and zero point. */
+int zant_model_concat(zant_model *m, const int *xs, int n, int64_t axis);
+/* Resize, "nearest" mode: exactly one of scales / sizes (length = rank), coord_mode as zant_hip_resize_nearest. */
+int zant_model_resize_nearest(zant_model *m, int x, const float *scales, const int64_t *sizes, int n_param,
+                              int coord_mode);
 /* int8 nodes; activation scales / zero points are tracked per tensor. */
 int zant_model_quantize(zant_model *m, int x, float y_scale, int y_zp);
 int zant_model_dequantize(zant_model *m, int x);
@@ -289,6 +297,8 @@ int zant_model_qlinear_global_avgpool(zant_model *m, int x, float y_scale, int y
  * the network output. */
 int zant_model_finalize(zant_model *m);
 int zant_model_output_dims(zant_model *m, int64_t *dims, int *rank, int *dtype);
+/* Shape (room for 8 dims) and element type of any tensor id handed out by the builder calls. */
+int zant_model_tensor_dims(zant_model *m, int tensor, int64_t *dims, int *rank, int *dtype);
 size_t zant_model_arena_bytes(zant_model *m);   /* planned arena size */
 size_t zant_model_unfused_bytes(zant_model *m); /* sum of all node outputs, the reference's static arrays */
 int zant_model_num_launches(zant_model *m);     /* operator calls per run after fusion */

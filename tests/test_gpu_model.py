@@ -250,3 +250,95 @@ def test_cpp_host_mirror_runs_the_reference_tests():
     r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
     assert r.returncode == 0, r.stdout + r.stderr
     assert "all passed" in r.stdout
+
+
+def _neck_graph(tmp_path, N, coord, sizes=False):
+    """A detector-neck shaped f32 graph: two convolutions, Sigmoid, a x2 nearest Resize of the coarse map, Concat with the
+    fine map along the channels, ReduceMean / GlobalAveragePool heads."""
+    import onnx_writer as ow
+    g = np.random.default_rng(4)
+    w1 = (g.standard_normal((8, 3, 3, 3)) * 0.3).astype(np.float32)
+    b1 = g.standard_normal(8).astype(np.float32)
+    w2 = (g.standard_normal((16, 8, 3, 3)) * 0.2).astype(np.float32)
+    b2 = g.standard_normal(16).astype(np.float32)
+    inits = [ow.tensor("w1", w1), ow.tensor("b1", b1), ow.tensor("w2", w2), ow.tensor("b2", b2),
+             ow.tensor("scales", np.array([] if sizes else [1, 1, 2, 2], np.float32)),
+             ow.tensor("sizes", np.array([N, 16, 12, 12] if sizes else [], np.int64)), ow.tensor("axes", np.array([2, 3], np.int64))]
+    nodes = [ow.node("Conv", ["x", "w1", "b1"], ["c1"], pads=[1, 1, 1, 1], kernel_shape=[3, 3]),
+             ow.node("MaxPool", ["c1"], ["p1"], kernel_shape=[2, 2], strides=[2, 2]),
+             ow.node("Conv", ["p1", "w2", "b2"], ["c2"], pads=[1, 1, 1, 1], kernel_shape=[3, 3]),
+             ow.node("Sigmoid", ["c2"], ["s2"]),
+             ow.node("Resize", ["s2", "", "scales", "sizes"], ["r2"], mode="nearest", coordinate_transformation_mode=coord,
+                     nearest_mode="round_prefer_ceil"),
+             ow.node("Concat", ["c1", "r2"], ["cat"], axis=1),
+             ow.node("LeakyRelu", ["cat"], ["act"], alpha=0.1),
+             ow.node("ReduceMean", ["act", "axes"], ["gm"], keepdims=1),
+             ow.node("GlobalAveragePool", ["cat"], ["ga"]),
+             ow.node("Add", ["gm", "ga"], ["y"])]
+    path = tmp_path / "neck.onnx"
+    path.write_bytes(ow.model(nodes, inits, [ow.value_info("x", (N, 3, 12, 12), np.float32)], [ow.value_info("y", (N, 24, 1, 1), np.float32)]))
+    return str(path)
+
+
+@pytest.mark.parametrize("coord,sizes", [("half_pixel", False), ("asymmetric", False), ("align_corners", True)])
+def test_neck_graph_with_sigmoid_resize_concat_reduce_mean_through_the_onnx_front_end(G, tmp_path, coord, sizes):
+    from zant_amd import onnx_front
+    N = 5
+    graph = onnx_front.read_graph(_neck_graph(tmp_path, N, coord, sizes))
+    m = onnx_front.build_model(G.tm.context(), graph)
+    x = np.random.default_rng(8).standard_normal((N, 3, 12, 12)).astype(np.float32)
+    ref = onnx_front.run_graph(graph, zo, x)
+    y = m.predict_host(x)
+    assert y.shape == ref.shape == (N, 24, 1, 1)
+    np.testing.assert_allclose(y, ref, rtol=G.RTOL, atol=G.ATOL)
+    m.close()
+
+
+def test_resize_rounding_convention_is_checked_by_the_front_end(G, tmp_path):
+    """ONNX's default nearest_mode (round_prefer_floor) and the reference's round-half-away differ only on exact ties:
+    half_pixel x2 has none and is accepted, asymmetric x2 has them and is refused rather than silently changed."""
+    import onnx_writer as ow
+    from zant_amd import onnx_front
+
+    def graph(coord):
+        nodes = [ow.node("Resize", ["x", "", "scales"], ["y"], mode="nearest", coordinate_transformation_mode=coord)]
+        p = tmp_path / "r.onnx"
+        p.write_bytes(ow.model(nodes, [ow.tensor("scales", np.array([1, 1, 2, 2], np.float32))], [ow.value_info("x", (1, 2, 4, 4), np.float32)],
+                               [ow.value_info("y", (1, 2, 8, 8), np.float32)]))
+        return onnx_front.read_graph(str(p))
+
+    m = onnx_front.build_model(G.tm.context(), graph("half_pixel"))
+    x = np.arange(32, dtype=np.float32).reshape(1, 2, 4, 4)
+    np.testing.assert_array_equal(m.predict_host(x), x.repeat(2, axis=2).repeat(2, axis=3))
+    m.close()
+    with pytest.raises(NotImplementedError):
+        onnx_front.build_model(G.tm.context(), graph("asymmetric"))
+
+
+def test_quantised_concat_and_resize_nodes_keep_codes_and_parameters(G):
+    """u8 tensors through MaxPool, Resize and Concat: codes move unchanged, scale / zero point ride along; inputs with
+    different parameters are refused."""
+    from zant_amd.model import Model, U8
+    g = np.random.default_rng(6)
+    N = 3
+    x = g.integers(0, 256, (N, 16, 8, 8), dtype=np.uint8)
+    m = Model(G.tm.context())
+    t = m.input(x.shape, U8, 0.05, 120)
+    p = m.maxpool(t, [2, 2], [2, 2])
+    r = m.resize_nearest(p, [1.0, 1.0, 2.0, 2.0], None, "half_pixel")
+    c = m.concat([t, r, t], 1)
+    o = m.qlinear_act(c, "relu", 0.0, 0.04, 3)  # a reader that needs the propagated parameters
+    other = m.qlinear_act(t, "relu", 0.0, 0.07, 0)
+    with pytest.raises(G.ZantError) as e:
+        m.concat([t, other], 1)
+    assert e.value.name == "InvalidInput"
+    m2 = Model(G.tm.context())  # the rejected call must not have left a node behind: build the graph again without it
+    t = m2.input(x.shape, U8, 0.05, 120)
+    c = m2.concat([t, m2.resize_nearest(m2.maxpool(t, [2, 2], [2, 2]), [1.0, 1.0, 2.0, 2.0], None, "half_pixel"), t], 1)
+    m2.qlinear_act(c, "relu", 0.0, 0.04, 3)
+    m2.finalize()
+    pooled = zo.onnx_maxpool(x, [2, 2], [2, 2], [1, 1], [0, 0, 0, 0])
+    cat = np.concatenate([x, pooled.repeat(2, axis=2).repeat(2, axis=3), x], axis=1)
+    ref = zo.qlinear_act(cat, 0.05, 120, "relu", 0.0, 0.04, 3)
+    np.testing.assert_array_equal(m2.predict_host(x), ref)
+    m2.close(); m.close()

@@ -87,6 +87,10 @@ PROTOTYPES = {
     "zant_model_add_const": (i32, [vp, i32, vp, c_i64p, i32]),
     "zant_model_add": (i32, [vp, i32, i32]),
     "zant_model_softmax": (i32, [vp, i32]),
+    "zant_model_sigmoid": (i32, [vp, i32]),
+    "zant_model_reduce_mean": (i32, [vp, i32, c_i64p, i32, i32]),
+    "zant_model_concat": (i32, [vp, C.POINTER(i32), i32, i64]),
+    "zant_model_resize_nearest": (i32, [vp, i32, C.POINTER(f32), c_i64p, i32, i32]),
     "zant_model_quantize": (i32, [vp, i32, f32, i32]),
     "zant_model_dequantize": (i32, [vp, i32]),
     "zant_model_qlinearconv": (i32, [vp, i32, vp, c_i64p, vp, i64, vp, f32, i32, c_i64p, c_i64p, c_i64p, i64]),
@@ -95,6 +99,7 @@ PROTOTYPES = {
     "zant_model_qlinear_global_avgpool": (i32, [vp, i32, f32, i32]),
     "zant_model_finalize": (i32, [vp]),
     "zant_model_output_dims": (i32, [vp, c_i64p, C.POINTER(i32), C.POINTER(i32)]),
+    "zant_model_tensor_dims": (i32, [vp, i32, c_i64p, C.POINTER(i32), C.POINTER(i32)]),
     "zant_model_arena_bytes": (sz, [vp]),
     "zant_model_unfused_bytes": (sz, [vp]),
     "zant_model_num_launches": (i32, [vp]),

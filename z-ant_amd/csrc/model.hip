@@ -23,7 +23,8 @@ namespace {
 
 enum OpKind {
     OP_CONV, OP_RELU, OP_LEAKY, OP_MAXPOOL, OP_RESHAPE, OP_GEMM, OP_MATMUL, OP_ADD_CONST, OP_ADD, OP_SOFTMAX,
-    OP_QUANT, OP_DEQUANT, OP_QCONV, OP_QACT, OP_QADD, OP_QGAP, OP_QBLOCK
+    OP_QUANT, OP_DEQUANT, OP_QCONV, OP_QACT, OP_QADD, OP_QGAP, OP_QBLOCK,
+    OP_SIGMOID, OP_REDUCE_MEAN, OP_CONCAT, OP_RESIZE
 };
 
 struct MTensor {
@@ -76,6 +77,11 @@ struct MNode {
     mutable zant_pack_slot slot;  // packed weights / tables of this node, filled by its first launch
     // OP_QBLOCK (a fused inverted residual block): the expansion, depthwise, projection and residual Add nodes
     int blk_expand = -1, blk_dw = -1, blk_project = -1, blk_add = -1;
+    std::vector<int> more;        // inputs of a Concat beyond the first two
+    std::vector<int64_t> axes;    // ReduceMean axes / Resize sizes
+    std::vector<float> scales;    // Resize scales
+    int64_t axis = 0;             // Concat axis
+    int keepdims = 1, coord_mode = 0;
 };
 
 }  // namespace
@@ -130,7 +136,8 @@ const void *param_ptr(const zant_model *m, int idx) {
 int consumers(const zant_model *m, int tensor, int *only) {
     int cnt = 0;
     for (size_t i = 0; i < m->n.size(); ++i)
-        if (m->n[i].in0 == tensor || m->n[i].in1 == tensor) { ++cnt; *only = int(i); }
+        if (m->n[i].in0 == tensor || m->n[i].in1 == tensor ||
+            std::find(m->n[i].more.begin(), m->n[i].more.end(), tensor) != m->n[i].more.end()) { ++cnt; *only = int(i); }
     return cnt;
 }
 
@@ -232,6 +239,31 @@ int run_node(zant_model *m, const MNode &nd) {
     }
     case OP_SOFTMAX:
         return zant_hip_softmax_f32(ctx, static_cast<const float *>(x), static_cast<float *>(y), ti.dim[0], ti.dim[1]);
+    case OP_SIGMOID:
+        return zant_hip_sigmoid_f32(ctx, static_cast<const float *>(x), static_cast<float *>(y), int64_t(ti.bytes() / 4));
+    case OP_REDUCE_MEAN: {
+        int64_t ydim[8];
+        int yr = 0;
+        return zant_hip_reduce_mean_f32(ctx, static_cast<const float *>(x), ti.dim, ti.rank, nd.axes.data(), int(nd.axes.size()),
+                                        nd.keepdims, 0, static_cast<float *>(y), ydim, &yr);
+    }
+    case OP_CONCAT: {
+        const void *xs[16];
+        const int64_t *dd[16];
+        int rr[16], n = 0;
+        for (int in : {nd.in0, nd.in1})
+            if (in >= 0) { xs[n] = tensor_ptr(m, in); dd[n] = m->t[in].dim; rr[n++] = m->t[in].rank; }
+        for (int in : nd.more) { xs[n] = tensor_ptr(m, in); dd[n] = m->t[in].dim; rr[n++] = m->t[in].rank; }
+        int64_t ydim[8];
+        int yr = 0;
+        return zant_hip_concatenate(ctx, xs, dd, rr, n, nd.axis, ti.dtype == ZANT_F32 ? 4 : 1, y, ydim, &yr);
+    }
+    case OP_RESIZE: {
+        int64_t ydim[8];
+        const bool by_scale = !nd.scales.empty();
+        return zant_hip_resize_nearest(ctx, x, ti.dim, ti.rank, ti.dtype == ZANT_F32 ? 4 : 1, by_scale ? nd.scales.data() : nullptr,
+                                       by_scale ? nullptr : nd.axes.data(), ti.rank, nd.coord_mode, y, ydim);
+    }
     case OP_QUANT:
         return zant_hip_quantize_linear_f32_u8(ctx, static_cast<const float *>(x), ti.dim, ti.rank,
                                                static_cast<const float *>(param_ptr(m, nd.ws)),
@@ -458,6 +490,60 @@ extern "C" int zant_model_softmax(zant_model *m, int x) {
     MNode nd;
     nd.op = OP_SOFTMAX; nd.in0 = x;
     return append(m, nd, ZANT_F32, tx.dim, tx.rank, 1.0f, 0);
+}
+
+extern "C" int zant_model_sigmoid(zant_model *m, int x) { return unary_same_shape(m, x, OP_SIGMOID, 0.0f); }
+
+extern "C" int zant_model_reduce_mean(zant_model *m, int x, const int64_t *axes, int n_axes, int keepdims) {
+    if (!valid_tensor(m, x)) return ZANT_NullPointer;
+    const MTensor tx = m->t[x];
+    if (tx.dtype != ZANT_F32) return ZANT_InvalidInput;
+    int64_t ydim[8];
+    int yr = 0;
+    const int rc = zant_hip_reduce_mean_f32(nullptr, nullptr, tx.dim, tx.rank, axes, n_axes, keepdims, 0, nullptr, ydim, &yr);
+    if (rc != ZANT_OK) return rc;
+    MNode nd;
+    nd.op = OP_REDUCE_MEAN; nd.in0 = x; nd.keepdims = keepdims;
+    if (axes) nd.axes.assign(axes, axes + n_axes);
+    return append(m, nd, ZANT_F32, ydim, yr, 1.0f, 0);
+}
+
+extern "C" int zant_model_concat(zant_model *m, const int *xs, int n, int64_t axis) {
+    if (!m || !xs) return ZANT_NullPointer;
+    if (n <= 0) return ZANT_EmptyTensorList;
+    if (n > 16) return ZANT_InvalidDimensions;
+    const int64_t *dd[16];
+    int rr[16];
+    for (int i = 0; i < n; ++i) {
+        if (!valid_tensor(m, xs[i])) return ZANT_NullPointer;
+        const MTensor &t = m->t[xs[i]], &t0 = m->t[xs[0]];
+        // quantised inputs must already share their parameters: concatenation moves codes, it does not requantise
+        if (t.dtype != t0.dtype || (t.dtype == ZANT_U8 && (t.scale != t0.scale || t.zp != t0.zp))) return ZANT_InvalidInput;
+        dd[i] = t.dim; rr[i] = t.rank;
+    }
+    int64_t ydim[8];
+    int yr = 0;
+    const int rc = zant_hip_concatenate(nullptr, nullptr, dd, rr, n, axis, 1, nullptr, ydim, &yr);
+    if (rc != ZANT_OK) return rc;
+    const MTensor t0 = m->t[xs[0]];
+    MNode nd;
+    nd.op = OP_CONCAT; nd.in0 = xs[0]; nd.in1 = n > 1 ? xs[1] : -1; nd.axis = axis;
+    for (int i = 2; i < n; ++i) nd.more.push_back(xs[i]);
+    return append(m, nd, t0.dtype, ydim, yr, t0.scale, t0.zp);
+}
+
+extern "C" int zant_model_resize_nearest(zant_model *m, int x, const float *scales, const int64_t *sizes, int n_param,
+                                         int coord_mode) {
+    if (!valid_tensor(m, x)) return ZANT_NullPointer;
+    const MTensor tx = m->t[x];
+    int64_t ydim[8];
+    const int rc = zant_hip_resize_nearest(nullptr, nullptr, tx.dim, tx.rank, 1, scales, sizes, n_param, coord_mode, nullptr, ydim);
+    if (rc != ZANT_OK) return rc;
+    MNode nd;
+    nd.op = OP_RESIZE; nd.in0 = x; nd.coord_mode = coord_mode;
+    if (scales) nd.scales.assign(scales, scales + n_param);
+    else nd.axes.assign(sizes, sizes + n_param);
+    return append(m, nd, tx.dtype, ydim, tx.rank, tx.scale, tx.zp);
 }
 
 extern "C" int zant_model_quantize(zant_model *m, int x, float y_scale, int y_zp) {
@@ -700,6 +786,8 @@ extern "C" int zant_model_finalize(zant_model *m) {
                 if (!blocked_op(nd)) {
                     demote(nd.in0, changed);
                     if (nd.in1 >= 0) demote(nd.in1, changed);
+                    for (int in : nd.more) demote(in, changed);
+                    demote(nd.out, changed);
                     continue;
                 }
                 if (nd.op == OP_QCONV) {
@@ -840,6 +928,7 @@ extern "C" int zant_model_finalize(zant_model *m) {
         if (m->t[ro].def < 0) m->t[ro].def = i + 1;
         for (int in : {nd.in0, nd.in1})
             if (in >= 0) { const int r = root_of(m, in); m->t[r].last = std::max(m->t[r].last, i + 1); }
+        for (int in : nd.more) { const int r = root_of(m, in); m->t[r].last = std::max(m->t[r].last, i + 1); }
     }
     m->t[root_of(m, m->output)].last = nn + 1;  // the output outlives the pass
     m->t[root_of(m, m->input)].last = std::max(m->t[root_of(m, m->input)].last, 1);
@@ -926,6 +1015,15 @@ extern "C" int zant_model_output_dims(zant_model *m, int64_t *dims, int *rank, i
     return ZANT_OK;
 }
 
+extern "C" int zant_model_tensor_dims(zant_model *m, int tensor, int64_t *dims, int *rank, int *dtype) {
+    if (!valid_tensor(m, tensor) || !dims || !rank) return ZANT_NullPointer;
+    const MTensor &t = m->t[tensor];
+    *rank = t.rank;
+    for (int i = 0; i < t.rank; ++i) dims[i] = t.dim[i];
+    if (dtype) *dtype = t.dtype;
+    return ZANT_OK;
+}
+
 extern "C" size_t zant_model_arena_bytes(zant_model *m) { return m ? m->arena_bytes : 0; }
 extern "C" size_t zant_model_unfused_bytes(zant_model *m) { return m ? m->unfused_bytes : 0; }
 extern "C" int zant_model_num_launches(zant_model *m) { return m ? m->launches : 0; }
@@ -982,6 +1080,10 @@ const char *op_name(const MNode &nd) {
     case OP_ADD_CONST: return "Add(const)";
     case OP_ADD: return "Add";
     case OP_SOFTMAX: return "Softmax";
+    case OP_SIGMOID: return "Sigmoid";
+    case OP_REDUCE_MEAN: return "ReduceMean";
+    case OP_CONCAT: return "Concat";
+    case OP_RESIZE: return "Resize";
     case OP_QUANT: return "QuantizeLinear";
     case OP_DEQUANT: return "DequantizeLinear";
     case OP_QCONV:
@@ -1001,6 +1103,7 @@ void node_work(const zant_model *m, const MNode &nd, double *ops, double *bytes)
     const MTensor &to = m->t[nd.out];
     double b = double(ti.bytes()) + double(to.bytes());
     if (nd.in1 >= 0) b += double(m->t[nd.in1].bytes());
+    for (int in : nd.more) b += double(m->t[in].bytes());
     double o = 0.0;
     switch (nd.op) {
     case OP_CONV:

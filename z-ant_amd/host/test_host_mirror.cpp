@@ -117,6 +117,50 @@ int main() {
         EXPECT(out.shape == Dims({3, 2}));
         EXPECT(error_of([&] { tensMath::reshape_lean<float>(&t, {-1, -1}, std::nullopt, &out); }) == ZANT_InvalidInput);
     }
+    {   // tests/Model/test_activation_function.zig:210-227 sigmoid; test_lib_reduction_math.zig:45-61, 126-155 reduce_mean
+        float v[3] = {0, 2, -2};
+        auto x = Tensor<float>::fromArray(v, {3});
+        auto s = tensMath::sigmoid(&x).toHost();
+        EXPECT(std::fabs(s[0] - 0.5f) < 1e-6f && std::fabs(s[1] - 0.880797f) < 1e-6f && std::fabs(s[2] - 0.119203f) < 1e-6f);
+        float w[24];
+        for (int i = 0; i < 24; ++i) w[i] = float(i + 1);
+        auto t = Tensor<float>::fromArray(w, {2, 2, 2});
+        Dims axes = {1, 2};
+        auto m = tensMath::reduce_mean(&t, &axes, false, false);
+        auto h = m.toHost();
+        EXPECT(m.shape == Dims({2}) && std::fabs(h[0] - 2.5f) < 1e-4f && std::fabs(h[1] - 6.5f) < 1e-4f);
+        auto t3 = Tensor<float>::fromArray(w, {2, 3, 4});
+        Dims axes02 = {0, 2};
+        auto m3 = tensMath::reduce_mean(&t3, &axes02, true, false);
+        auto h3 = m3.toHost();
+        EXPECT(m3.shape == Dims({1, 3, 1}) && std::fabs(h3[0] - 8.5f) < 1e-4f && std::fabs(h3[2] - 16.5f) < 1e-4f);
+        Dims bad = {3};
+        EXPECT(error_of([&] { tensMath::reduce_mean(&t3, &bad, true, false); }) == ZANT_InvalidAxes);
+    }
+    {   // test_lib_shape_math.zig:139-192 concat along axis 2, :2182-2255 errors; :480-499, 596-627 resize
+        float a[8] = {1, 2, 3, 4, 5, 6, 7, 8}, b[12];
+        for (int i = 0; i < 12; ++i) b[i] = float(9 + i);
+        auto A = Tensor<float>::fromArray(a, {2, 2, 2});
+        auto B = Tensor<float>::fromArray(b, {2, 2, 3});
+        auto Y = tensMath::concatenate<float>({&A, &B}, 2);
+        const float expect[20] = {1, 2, 9, 10, 11, 3, 4, 12, 13, 14, 5, 6, 15, 16, 17, 7, 8, 18, 19, 20};
+        auto h = Y.toHost();
+        EXPECT(Y.shape == Dims({2, 2, 5}));
+        for (int i = 0; i < 20; ++i) EXPECT(h[i] == expect[i]);
+        EXPECT(error_of([&] { tensMath::concatenate<float>({&A, &B}, 0); }) == ZANT_MismatchedShape);
+        EXPECT(error_of([&] { tensMath::concatenate<float>({&A, &A}, 3); }) == ZANT_AxisOutOfBounds);
+        EXPECT(error_of([&] { tensMath::concatenate<float>({}, 0); }) == ZANT_EmptyTensorList);
+        uint8_t u[4] = {1, 2, 3, 4};
+        auto U = Tensor<uint8_t>::fromArray(u, {4});
+        std::vector<float> scales = {2.0f};
+        auto R = tensMath::resize<uint8_t>(&U, "nearest", &scales, nullptr, "half_pixel");
+        auto r = R.toHost();
+        EXPECT(R.size == 8 && r[0] == 1 && r[1] == 1 && r[2] == 2 && r[3] == 2);
+        Dims sizes = {8};
+        EXPECT(error_of([&] { tensMath::resize<uint8_t>(&U, "invalid_mode", &scales, nullptr, "half_pixel"); }) == ZANT_UnsupportedMode);
+        EXPECT(error_of([&] { tensMath::resize<uint8_t>(&U, "nearest", &scales, &sizes, "half_pixel"); }) == ZANT_InvalidInput);
+        EXPECT(error_of([&] { tensMath::resize<uint8_t>(&U, "nearest", nullptr, nullptr, "half_pixel"); }) == ZANT_InvalidInput);
+    }
     check(zant_hip_sync(default_ctx()));
     std::printf(failures ? "host mirror: %d FAILED\n" : "host mirror: all passed\n", failures);
     return failures ? 1 : 0;

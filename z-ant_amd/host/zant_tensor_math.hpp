@@ -219,6 +219,78 @@ inline Tensor<float> softmax(Tensor<float> *in) {
     return out;
 }
 
+// sigmoid_lean / sigmoid (lib_activation_function_math.zig:107, :95)
+inline void sigmoid_lean(Tensor<float> *in, Tensor<float> *out) {
+    check(zant_hip_sigmoid_f32(default_ctx(), in->data, out->data, int64_t(in->size)));
+}
+inline Tensor<float> sigmoid(Tensor<float> *in) {
+    if (in->size == 0) throw Error(ZANT_ZeroSizeTensor);
+    Tensor<float> out = Tensor<float>::fromShape(in->shape);
+    sigmoid_lean(in, &out);
+    return out;
+}
+
+// lean_reduce_mean / reduce_mean (lib_reduction_math.zig:87, :30); axes == nullptr is Zig's null
+inline void reduce_mean_lean(Tensor<float> *in, Tensor<float> *out, const Dims *axes, bool keepdims, bool noop_with_empty_axes) {
+    int64_t ydim[8];
+    int yr = 0;
+    check(zant_hip_reduce_mean_f32(default_ctx(), in->data, in->shape.data(), int(in->shape.size()), axes ? axes->data() : nullptr,
+                                   axes ? int(axes->size()) : 0, keepdims, noop_with_empty_axes, out->data, ydim, &yr));
+}
+inline Tensor<float> reduce_mean(Tensor<float> *in, const Dims *axes, bool keepdims, bool noop_with_empty_axes) {
+    int64_t ydim[8];
+    int yr = 0;
+    check(zant_hip_reduce_mean_f32(nullptr, nullptr, in->shape.data(), int(in->shape.size()), axes ? axes->data() : nullptr,
+                                   axes ? int(axes->size()) : 0, keepdims, noop_with_empty_axes, nullptr, ydim, &yr));
+    Tensor<float> out = Tensor<float>::fromShape(Dims(ydim, ydim + yr));
+    reduce_mean_lean(in, &out, axes, keepdims, noop_with_empty_axes);
+    return out;
+}
+
+// get_concatenate_output_shape / lean_concatenate / concatenate (lib_shape_math.zig:582, :307, :463)
+template <typename T>
+inline Dims concatenate_impl(const std::vector<Tensor<T> *> &tensors, int64_t axis, T *out) {
+    std::vector<const void *> ptrs;
+    std::vector<const int64_t *> shapes;
+    std::vector<int> ranks;
+    for (Tensor<T> *t : tensors) {
+        ptrs.push_back(t->data);
+        shapes.push_back(t->shape.data());
+        ranks.push_back(int(t->shape.size()));
+    }
+    int64_t ydim[8];
+    int yr = 0;
+    check(zant_hip_concatenate(out ? default_ctx() : nullptr, ptrs.data(), shapes.data(), ranks.data(), int(tensors.size()), axis,
+                               sizeof(T), out, ydim, &yr));
+    return Dims(ydim, ydim + yr);
+}
+template <typename T>
+inline void lean_concatenate(const std::vector<Tensor<T> *> &tensors, int64_t axis, Tensor<T> *out) {
+    out->shape = concatenate_impl<T>(tensors, axis, out->data);
+}
+template <typename T>
+inline Tensor<T> concatenate(const std::vector<Tensor<T> *> &tensors, int64_t axis) {
+    Tensor<T> out = Tensor<T>::fromShape(concatenate_impl<T>(tensors, axis, nullptr));
+    lean_concatenate<T>(tensors, axis, &out);
+    return out;
+}
+
+// resize in "nearest" mode (lib_shape_math.zig:22); scales / sizes == nullptr is Zig's null
+template <typename T>
+inline Tensor<T> resize(Tensor<T> *t, const std::string &mode, const std::vector<float> *scales, const Dims *sizes,
+                        const std::string &coordinate_transformation_mode) {
+    int64_t ydim[8];
+    const int n = scales ? int(scales->size()) : sizes ? int(sizes->size()) : 0;
+    const int cm = coordinate_transformation_mode == "half_pixel" ? 0 : coordinate_transformation_mode == "align_corners" ? 1 : 2;
+    check(zant_hip_resize_nearest(nullptr, nullptr, t->shape.data(), int(t->shape.size()), sizeof(T), scales ? scales->data() : nullptr,
+                                  sizes ? sizes->data() : nullptr, n, cm, nullptr, ydim));
+    if (mode != "nearest") throw Error(ZANT_UnsupportedMode);  // "linear" / "cubic" are not provided either
+    Tensor<T> out = Tensor<T>::fromShape(Dims(ydim, ydim + t->shape.size()));
+    check(zant_hip_resize_nearest(default_ctx(), t->data, t->shape.data(), int(t->shape.size()), sizeof(T),
+                                  scales ? scales->data() : nullptr, sizes ? sizes->data() : nullptr, n, cm, out.data, ydim));
+    return out;
+}
+
 // sum_tensors_lean / sum_tensors, add_bias (lib_elementWise_math.zig:70, :52, :22)
 inline void sum_tensors_lean(Tensor<float> *t1, Tensor<float> *t2, Tensor<float> *out) {
     int64_t ydim[8];

@@ -78,6 +78,33 @@ class Model:
     def softmax(self, x):
         return self._id(lib.zant_model_softmax(self.handle, x))
 
+    def sigmoid(self, x):
+        return self._id(lib.zant_model_sigmoid(self.handle, x))
+
+    def reduce_mean(self, x, axes, keepdims=True):
+        ad, na = dims(axes)
+        return self._id(lib.zant_model_reduce_mean(self.handle, x, ad, na, int(keepdims)))
+
+    def global_average_pool(self, x):
+        """ONNX GlobalAveragePool of an NCHW tensor: the mean over H and W, rank kept."""
+        return self.reduce_mean(x, [2, 3], True)
+
+    def concat(self, xs, axis):
+        arr = (C.c_int * max(len(xs), 1))(*xs)
+        return self._id(lib.zant_model_concat(self.handle, arr, len(xs), axis))
+
+    def resize_nearest(self, x, scales=None, sizes=None, coordinate_transformation_mode="half_pixel"):
+        sc = (C.c_float * len(scales))(*scales) if scales is not None else None
+        sd, _ = dims(sizes)
+        n = len(scales) if scales is not None else (len(sizes) if sizes is not None else 0)
+        mode = {"half_pixel": 0, "align_corners": 1}.get(coordinate_transformation_mode, 2)
+        return self._id(lib.zant_model_resize_nearest(self.handle, x, sc, sd, n, mode))
+
+    def tensor_shape(self, x):
+        d = (C.c_int64 * 8)(); r = C.c_int()
+        self._id(lib.zant_model_tensor_dims(self.handle, x, d, C.byref(r), None))
+        return tuple(d)[:r.value]
+
     def quantize(self, x, scale, zp):
         return self._id(lib.zant_model_quantize(self.handle, x, scale, zp))
 

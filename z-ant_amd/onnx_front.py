@@ -209,10 +209,49 @@ def run_graph(graph, ops, x):
             y = ops.mat_mul(i[0], i[1])
         elif nd["op"] == "Softmax":
             y = ops.softmax(i[0])
+        elif nd["op"] == "Sigmoid":
+            y = ops.sigmoid(i[0])
+        elif nd["op"] == "LeakyRelu":
+            y = ops.leakyReLU(i[0], a.get("alpha", 0.01))
+        elif nd["op"] == "GlobalAveragePool":
+            y = ops.reduce_mean(i[0], [2, 3], True, False)
+        elif nd["op"] == "ReduceMean":
+            axes = a.get("axes")
+            if axes is None and len(i) > 1:
+                axes = [int(v) for v in i[1].reshape(-1)]
+            y = ops.reduce_mean(i[0], axes, bool(a.get("keepdims", 1)), False)
+        elif nd["op"] == "Concat":
+            y = ops.concatenate(i, a["axis"])
+        elif nd["op"] == "Resize":
+            names = nd["inputs"] + ["", "", ""]
+            scales = vals[names[2]].reshape(-1) if names[2] and vals[names[2]].size else None
+            sizes = vals[names[3]].reshape(-1) if names[3] and vals[names[3]].size else None
+            coord = a.get("coordinate_transformation_mode", "half_pixel")
+            coord = coord.decode() if isinstance(coord, bytes) else coord
+            y = ops.resize(i[0], "nearest", None if scales is None else [float(v) for v in scales],
+                           None if sizes is None else [int(v) for v in sizes], coord)
         else:
             raise NotImplementedError(nd["op"])
         vals[nd["outputs"][0]] = y
     return vals[graph["outputs"][0][0]]
+
+
+def _resize_has_ties(in_dims, out_dims, coord):
+    """Whether any output coordinate of a nearest-neighbour Resize lands exactly between two input elements, computed in
+    f32 like the reference (lib_shape_math.zig:128-139): only then does the rounding convention matter."""
+    for n_in, n_out in zip(in_dims, out_dims):
+        o = np.arange(n_out, dtype=np.float32)
+        scale = np.float32(n_out) / np.float32(n_in)
+        if coord == "half_pixel":
+            pos = (o + np.float32(0.5)) / scale - np.float32(0.5)
+        elif coord == "align_corners":
+            pos = o * np.float32(n_in - 1) / np.float32(max(n_out - 1, 1))
+        else:
+            pos = o / scale
+        pos = pos[(pos > 0) & (pos < n_in - 1)]  # outside that range the clamp decides
+        if np.any(pos - np.floor(pos) == np.float32(0.5)):
+            return True
+    return False
 
 
 def build_model(ctx, graph):
@@ -294,6 +333,44 @@ def build_model(ctx, graph):
                        bool(a.get("transA", 0)), bool(a.get("transB", 0)))
         elif op == "Softmax":
             t = m.softmax(tens[ins[0]])
+        elif op == "Sigmoid":
+            t = m.sigmoid(tens[ins[0]])
+        elif op == "GlobalAveragePool":
+            t = m.global_average_pool(tens[ins[0]])
+        elif op == "ReduceMean":
+            if a.get("noop_with_empty_axes", 0):
+                raise NotImplementedError("ReduceMean with noop_with_empty_axes")
+            axes = a.get("axes")
+            if axes is None and len(ins) > 1 and ins[1]:
+                axes = [int(v) for v in consts[ins[1]].reshape(-1)]
+            t = m.reduce_mean(tens[ins[0]], axes, bool(a.get("keepdims", 1)))
+        elif op == "Concat":
+            t = m.concat([tens[n] for n in ins], a["axis"])
+            if ins[0] in qparams:
+                qparams[out] = qparams[ins[0]]
+        elif op == "Resize":
+            mode = a.get("mode", b"nearest")
+            mode = mode.decode() if isinstance(mode, bytes) else mode
+            if mode != "nearest":
+                raise NotImplementedError(f"Resize mode {mode}")
+            coord = a.get("coordinate_transformation_mode", b"half_pixel")
+            coord = coord.decode() if isinstance(coord, bytes) else coord
+            if coord not in ("half_pixel", "align_corners", "asymmetric"):
+                raise NotImplementedError(f"Resize coordinate_transformation_mode {coord}")
+            scales = consts[ins[2]].reshape(-1) if len(ins) > 2 and ins[2] and consts[ins[2]].size else None
+            sizes = consts[ins[3]].reshape(-1) if len(ins) > 3 and ins[3] and consts[ins[3]].size else None
+            nearest = a.get("nearest_mode", b"round_prefer_floor")
+            nearest = nearest.decode() if isinstance(nearest, bytes) else nearest
+            in_dims = m.tensor_shape(tens[ins[0]])
+            out_dims = [int(np.floor(np.float32(d) * np.float32(f))) for d, f in zip(in_dims, scales)] if scales is not None \
+                else [int(v) for v in sizes]
+            if nearest != "round_prefer_ceil" and _resize_has_ties(in_dims, out_dims, coord):
+                # the reference rounds half away from zero (lib_shape_math.zig:141), which is round_prefer_ceil here
+                raise NotImplementedError(f"Resize nearest_mode {nearest} differs from the reference's rounding on this shape")
+            t = m.resize_nearest(tens[ins[0]], None if scales is None else [float(v) for v in scales],
+                                 None if sizes is None else out_dims, coord)
+            if ins[0] in qparams:
+                qparams[out] = qparams[ins[0]]
         elif op == "QuantizeLinear":
             sc, zp = float(scalar(ins[1])), int(scalar(ins[2] if len(ins) > 2 else ""))
             t = m.quantize(tens[ins[0]], sc, zp)
