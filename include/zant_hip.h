@@ -80,7 +80,9 @@ const char *zant_hip_version(void);
 /* Replaces setLogFunctionC (src/Core/Tensor/TensorMath/op_convolution.zig:37-41)
  * and the generated library's setLogFunction (src/codeGen/skeleton.zig:93-97). */
 void setLogFunctionC(void (*func)(char *));
+#ifndef ZANT_HIP_NO_PREDICT_DECL
 void setLogFunction(void (*func)(char *));
+#endif
 
 /* The activation arena: ONE device allocation that model-level forward passes
  * carve their tensors from (the reference keeps one static array per node
@@ -327,7 +329,11 @@ int zant_model_read_tensor(zant_model *m, int id, void *dst_host, size_t bytes);
  * (predict.zig:317-335); otherwise *result points at library-owned host storage that stays valid
  * until the next call. */
 int zant_model_bind_predict(zant_model *m);
+/* A generated library defines predict / setLogFunction itself, typed by its network's element types (the reference's
+ * comptime T); it defines ZANT_HIP_NO_PREDICT_DECL before including this file. */
+#ifndef ZANT_HIP_NO_PREDICT_DECL
 void predict(float *input, uint32_t *input_shape, uint32_t shape_len, float **result);
+#endif
 /* predict() for callers that only know the batch: `n` must equal the leading dimension the bound model was built
  * with (the reference compiles the batch into predict's shape check, predict.zig:328-334); otherwise it returns
  * silently with *result untouched, as predict does.  No counterpart in the reference: it exists for the batched

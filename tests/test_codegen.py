@@ -1,0 +1,109 @@
+"""The code generator: ONNX graph -> C source of a stand-alone library over the C ABI (the counterpart of the reference's
+lib_<model>.zig emitter).  Generation and compilation need no GPU; running the generated predict() does."""
+import ctypes as C
+import json
+import os
+
+import numpy as np
+import pytest
+
+import __graft_entry__ as ge
+import onnx_writer
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+MNIST = os.path.join(HERE, "golden", "mnist-8.onnx")
+
+
+@pytest.fixture(scope="module")
+def codegen():
+    ge.load_package()
+    from zant_amd import codegen
+    return codegen
+
+
+def _load(so):
+    lib = C.CDLL(so)
+    lib.predict.restype = None
+    lib.predict.argtypes = [C.c_void_p, C.POINTER(C.c_uint32), C.c_uint32, C.POINTER(C.c_void_p)]
+    return lib
+
+
+def _predict(lib, x, shape=None):
+    shape = x.shape if shape is None else shape
+    arr = (C.c_uint32 * max(len(shape), 1))(*shape)
+    res = C.c_void_p()
+    lib.predict(x.ctypes.data_as(C.c_void_p), arr, len(shape), C.byref(res))
+    return res.value
+
+
+def test_generated_source_replays_the_graph_and_compiles_without_a_gpu(codegen, tmp_path):
+    info = codegen.generate(MNIST, str(tmp_path), "mnist8")
+    text = open(info["c"]).read()
+    # mnist-8: 12 ONNX nodes, one of them a Reshape of an initialiser that is folded at generation time
+    assert info["nodes"] == 11 and info["in_shape"] == (1, 1, 28, 28) and info["out_shape"] == (1, 10)
+    for call in ("zant_model_input(m, 0,", "zant_model_conv(m, 0,", '"SAME_UPPER"', "zant_model_add_const(m, 1,", "zant_model_relu(m, 2)",
+                 "zant_model_maxpool(m, 3,", "zant_model_reshape(m, 8,", "zant_model_matmul(m, 9,", "static float g_result[10];"):
+        assert call in text, call
+    assert os.path.getsize(info["params"]) == info["param_bytes"] >= 4 * (8 * 25 + 8 + 16 * 8 * 25 + 16 + 2560 + 10)
+    so = codegen.compile_library(info)
+    lib = _load(so)
+    for sym in ("predict", "setLogFunction", "mnist8_init", "mnist8_model", "mnist8_shutdown"):
+        assert hasattr(lib, sym)
+    # the reference's predict() returns silently, result untouched, on a wrong rank / shape / empty shape
+    # (tests/CodeGen/test_model.template.zig:60-160); these paths end before any GPU call
+    x = np.zeros((1, 1, 28, 28), np.float32)
+    assert _predict(lib, x, (1, 1, 28)) is None
+    assert _predict(lib, x, (1, 1, 28, 27)) is None
+    assert _predict(lib, x, ()) is None
+
+
+def test_generator_rejects_a_graph_the_executor_would_reject(codegen, tmp_path):
+    nodes = [onnx_writer.node("Conv", ["x", "w"], ["y"], kernel_shape=[3, 3])]
+    p = tmp_path / "bad.onnx"   # 4 input channels against a filter with 3: the dry-run model refuses the node
+    p.write_bytes(onnx_writer.model(nodes, [onnx_writer.tensor("w", np.zeros((2, 3, 3, 3), np.float32))],
+                                    [onnx_writer.value_info("x", (1, 4, 8, 8), np.float32)], [onnx_writer.value_info("y", (1, 2, 6, 6), np.float32)]))
+    from zant_amd import ZantError
+    with pytest.raises(ZantError):
+        codegen.generate(str(p), str(tmp_path), "bad")
+
+
+@pytest.mark.gpu
+def test_generated_mnist8_library_matches_the_oracle(codegen, tmp_path):
+    from oracle import oracle as zo
+    from zant_amd import onnx_front
+    info = codegen.generate(MNIST, str(tmp_path), "mnist8")
+    lib = _load(codegen.compile_library(info))
+    graph = onnx_front.read_graph(MNIST)
+    g = np.random.default_rng(0)
+    logged = []
+    cb = C.CFUNCTYPE(None, C.c_char_p)(lambda s: logged.append(s))
+    lib.setLogFunction(cb)
+    for _ in range(3):
+        x = g.random((1, 1, 28, 28), dtype=np.float32)
+        ptr = _predict(lib, x)
+        assert ptr is not None
+        y = np.ctypeslib.as_array(C.cast(ptr, C.POINTER(C.c_float)), (1, 10)).copy()
+        np.testing.assert_allclose(y, onnx_front.run_graph(graph, zo, x), rtol=1e-4, atol=1e-5)
+    assert b"Starting prediction...\n" in logged and b"Prediction completed.\n" in logged
+    lib.setLogFunction(None)
+    lib.mnist8_shutdown()
+
+
+@pytest.mark.gpu
+def test_generated_int8_detector_library_reproduces_the_golden_bytes(codegen, tmp_path):
+    from zant_amd import networks as nets
+    gold = json.load(open(os.path.join(HERE, "golden", "int8_networks.json")))["tiny_yolo_int8"]
+    arch = nets.tiny_yolo_arch()
+    params = nets.int8_params(arch, seed=gold["param_seed"])
+    data, out_shape = onnx_writer.int8_network(arch, params, gold["quant"], 2)
+    p = tmp_path / "yolo.onnx"
+    p.write_bytes(data)
+    info = codegen.generate(str(p), str(tmp_path), "tiny_yolo")
+    assert info["in_dtype"] == 1 and info["out_dtype"] == 1 and tuple(info["out_shape"]) == tuple(out_shape)
+    lib = _load(codegen.compile_library(info))
+    x = np.random.default_rng(gold["input_seed"]).integers(0, 256, (2,) + tuple(arch["input"]), dtype=np.uint8)
+    ptr = _predict(lib, x)
+    assert ptr is not None
+    y = np.ctypeslib.as_array(C.cast(ptr, C.POINTER(C.c_uint8)), (int(np.prod(out_shape)),)).copy()
+    np.testing.assert_array_equal(y, np.array(gold["expected_u8"], np.uint8))
+    lib.tiny_yolo_shutdown()

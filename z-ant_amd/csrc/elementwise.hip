@@ -493,14 +493,14 @@ extern "C" int zant_hip_softmax_f32(zant_ctx *ctx, const float *x, float *y, int
 
 extern "C" int zant_hip_add_f32(zant_ctx *ctx, const float *a, const int64_t *adim, int a_rank, const float *b,
                                 const int64_t *bdim, int b_rank, float *y, int64_t *ydim_out, int *y_rank_out) {
-    if (!ctx || !adim || !bdim) return ZANT_NullPointer;
+    if (!adim || !bdim) return ZANT_NullPointer;  // ctx is looked at with the data pointers: shape queries pass none
     if (a_rank < 0 || b_rank < 0 || a_rank > 8 || b_rank > 8) return ZANT_InvalidDimensions;
     const int64_t asz = prod_dims(adim, a_rank), bsz = prod_dims(bdim, b_rank);
     if (asz == bsz) {  // lib_elementWise_math.zig:72-110
         if (y_rank_out) *y_rank_out = a_rank;
         if (ydim_out) for (int i = 0; i < a_rank; ++i) ydim_out[i] = adim[i];
         if (asz == 0) return ZANT_OK;
-        if (!a || !b || !y) return ZANT_NullPointer;
+        if (!ctx || !a || !b || !y) return ZANT_NullPointer;
         const int vec = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
         KernelTimer kt(ctx);
         hipLaunchKernelGGL(add_same_f32_kernel, dim3(zant_stream_grid((asz + 3) >> 2)), dim3(kThreads), 0, ctx->stream, a, b,
@@ -528,7 +528,7 @@ extern "C" int zant_hip_add_f32(zant_ctx *ctx, const float *a, const int64_t *ad
     if (y_rank_out) *y_rank_out = g.rank;
     if (ydim_out) for (int i = 0; i < g.rank; ++i) ydim_out[i] = g.out_dim[i];
     if (osz == 0) return ZANT_OK;
-    if (!a || !b || !y) return ZANT_NullPointer;
+    if (!ctx || !a || !b || !y) return ZANT_NullPointer;
     KernelTimer kt(ctx);
     {
         // per-channel fast path: one operand is the whole output, the other varies along exactly one axis
@@ -577,7 +577,7 @@ extern "C" int zant_hip_add_bias_f32(zant_ctx *ctx, float *t, const int64_t *tdi
 
 extern "C" int zant_hip_reshape(zant_ctx *ctx, const void *x, const int64_t *xdim, int x_rank, size_t elem_size,
                                 const int64_t *new_shape, int new_rank, void *y, int64_t *ydim_out) {
-    if (!ctx || !xdim || !new_shape || !ydim_out) return ZANT_NullPointer;
+    if (!xdim || !new_shape || !ydim_out) return ZANT_NullPointer;
     const int64_t in_size = prod_dims(xdim, x_rank);
     int neg = -1;
     int64_t known = 1;
@@ -602,7 +602,7 @@ extern "C" int zant_hip_reshape(zant_ctx *ctx, const void *x, const int64_t *xdi
     }
     if (prod_dims(ydim_out, new_rank) != in_size) return ZANT_InputArrayWrongSize;  // :1197-1199
     if (in_size == 0 || x == y) return ZANT_OK;  // a view inside the arena needs no copy
-    if (!x || !y) return ZANT_NullPointer;
+    if (!ctx || !x || !y) return ZANT_NullPointer;
     ZANT_HIP_TRY(ctx, hipMemcpyAsync(y, x, size_t(in_size) * elem_size, hipMemcpyDeviceToDevice, ctx->stream));
     return ZANT_OK;
 }

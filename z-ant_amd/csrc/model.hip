@@ -315,7 +315,7 @@ int run_node(zant_model *m, const MNode &nd) {
 }  // namespace
 
 extern "C" int zant_model_create(zant_ctx *ctx, zant_model **out) {
-    if (!ctx || !out) return ZANT_NullPointer;
+    if (!out) return ZANT_NullPointer;  // ctx may be NULL: such a model validates nodes and answers shape queries only
     zant_model *m = new (std::nothrow) zant_model();
     if (!m) return ZANT_MemError;
     m->ctx = ctx;
@@ -625,6 +625,7 @@ extern "C" int zant_model_qlinear_global_avgpool(zant_model *m, int x, float y_s
 extern "C" int zant_model_finalize(zant_model *m) {
     if (!m) return ZANT_NullPointer;
     if (m->finalized) return ZANT_OK;
+    if (!m->ctx) return ZANT_NullPointer;  // built without a context: a dry run
     if (m->input < 0 || m->n.empty()) return ZANT_InvalidInput;
     zant_ctx *ctx = m->ctx;
     const int nn = int(m->n.size());
@@ -1202,7 +1203,9 @@ extern "C" int zant_model_bind_predict(zant_model *m) {
     return ZANT_OK;
 }
 
-extern "C" void predict(float *input, uint32_t *input_shape, uint32_t shape_len, float **result) {
+// predict's body; predict_batched calls it directly so that a generated library's own `predict` symbol, which comes
+// first in a process that links both, is never reached from here.
+static void predict_bound(float *input, uint32_t *input_shape, uint32_t shape_len, float **result) {
     zant_log("Starting prediction...\n");
     zant_model *m = g_predict_model;
     if (!m || !input || !input_shape || !result) return;
@@ -1217,6 +1220,10 @@ extern "C" void predict(float *input, uint32_t *input_shape, uint32_t shape_len,
     zant_log("Prediction completed.\n");
 }
 
+extern "C" void predict(float *input, uint32_t *input_shape, uint32_t shape_len, float **result) {
+    predict_bound(input, input_shape, shape_len, result);
+}
+
 extern "C" void predict_batched(float *input, uint32_t n, float **result) {
     zant_model *m = g_predict_model;
     if (!m || !input || !result) return;
@@ -1224,5 +1231,5 @@ extern "C" void predict_batched(float *input, uint32_t n, float **result) {
     if (tin.rank < 1 || int64_t(n) != tin.dim[0]) return;
     uint32_t shape[8];
     for (int i = 0; i < tin.rank; ++i) shape[i] = uint32_t(tin.dim[i]);
-    predict(input, shape, uint32_t(tin.rank), result);
+    predict_bound(input, shape, uint32_t(tin.rank), result);
 }

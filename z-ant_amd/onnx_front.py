@@ -254,11 +254,12 @@ def _resize_has_ties(in_dims, out_dims, coord):
     return False
 
 
-def build_model(ctx, graph):
+def build_model(ctx, graph, model=None):
     """Turns the graph into a finalized ``Model``: one executor node per ONNX node, initialisers as parameters, Reshape
-    of an initialiser folded on the host (as the reference's code generator does for constant inputs)."""
+    of an initialiser folded on the host (as the reference's code generator does for constant inputs).  ``model``: an
+    object with Model's builder methods to drive instead of a new Model (the code generator passes its recorder)."""
     from .model import Model, U8
-    m = Model(ctx)
+    m = model if model is not None else Model(ctx)
     consts = dict(graph["initializers"])
     name, dims = graph["inputs"][0]
     nodes = graph["nodes"]
