@@ -181,42 +181,72 @@ qpack_kernel(const int8_t *__restrict__ w, const float *__restrict__ w_scale, co
 // Bytes of the weight region of a staging buffer: the slab rounded up to one 16-byte unit per thread and round.
 __device__ __host__ __forceinline__ int w_region_bytes(int w_chunk, int nt) { return ((w_chunk / 16 + nt - 1) / nt) * nt * 16; }
 
+// Where this thread's patch slots of one tile come from: byte offset of the first 16-channel half of chunk 0 from the
+// start of the blocked input, per copy round, and which rounds read real data (the others copy the padding vector).
+// Filled once per tile (qconv_describe), so a step's copies cost an address add and a select each.
+constexpr int QR_MAX = 4;  // copy rounds of the patch region: P1s / threads
+struct PatchDesc {
+    unsigned long long off[QR_MAX];
+    unsigned ok;      // bit r: round r reads the input
+    int kb;           // output-channel block of the tile (selects the weight slab)
+};
+
+template <int NT>
+__device__ __forceinline__ void qconv_describe(PatchDesc &d, const int2 *__restrict__ ptab, const ConvGeom &g, const TileGeom &t,
+                                               int CB, int itile) {
+    int n0, oh0, kb;
+    decode_tile(t, itile, n0, oh0, kb);
+    d.kb = kb;
+    d.ok = 0;
+    const int64_t plane = int64_t(g.H) * g.W;
+    const int ih0 = oh0 * g.sh - g.pt;
+    const int imgs_here = min(t.NB, g.N - n0);
+    const int64_t tile_base = int64_t(n0) * CB * plane + int64_t(ih0) * g.W;
+#pragma unroll
+    for (int r = 0; r < QR_MAX; ++r) {
+        d.off[r] = 0;
+        if (r * NT < t.P1s) {
+            const int2 e = ptab[r * NT + int(threadIdx.x)];  // entries past P1 say "padding"
+            const int ih = ih0 + (e.y & 0xffff);
+            const bool ok = e.x >= 0 && ih >= 0 && ih < g.H && (e.y >> 16) < imgs_here;
+            d.off[r] = ok ? (unsigned long long)((tile_base + e.x) * 16) : 0ull;
+            d.ok |= ok ? 1u << r : 0u;
+        }
+    }
+}
+
 // The asynchronous copies of one (tile, chunk) step into the staging buffer `dma`.  Every thread issues the same
 // number of copies whatever the geometry (lanes past the end of the slab repeat its last unit, patch slots past P1
 // -- the patch region is padded to a multiple of the workgroup size -- copy the padding vector), so the number of
 // copies a wave has in flight per step is a constant the ring's waits can count with.
 template <int WM, int WN, int TT>
-__device__ __forceinline__ void qconv_issue(char *__restrict__ dma, const int2 *__restrict__ ptab,
-                                            const int8_t *__restrict__ xb, const int8_t *__restrict__ wp,
-                                            const int8_t *__restrict__ padvec, const ConvGeom &g, const TileGeom &t, int CB,
-                                            int itile, int ichunk) {
+__device__ __forceinline__ void qconv_issue(char *__restrict__ dma, const PatchDesc &d, const int8_t *__restrict__ xb,
+                                            const int8_t *__restrict__ wp, const int8_t *__restrict__ padvec,
+                                            const ConvGeom &g, const TileGeom &t, int CB, int ichunk) {
     constexpr int NT = WM * WN * 64;
     constexpr int K_BLK = WN * 32;
     const int T = TT > 0 ? TT : g.KH * g.KW;
     const int w_chunk = T * QCC * K_BLK;  // bytes
     const int tid = threadIdx.x, wave = tid >> 6;
-    int n0, oh0, kb;
-    decode_tile(t, itile, n0, oh0, kb);
     char *xl = dma + w_region_bytes(w_chunk, NT);
-    const int8_t *wsrc = wp + (int64_t(ichunk) * t.n_kblocks + kb) * w_chunk;
+    const int8_t *wsrc = wp + (int64_t(ichunk) * t.n_kblocks + d.kb) * w_chunk;
     const int units = w_chunk >> 4;
     for (int u0 = 0; u0 < units; u0 += NT) {
         const int u = min(u0 + tid, units - 1);
         __builtin_amdgcn_global_load_lds((gptr_t)(wsrc + u * 16), (lptr_t)(dma + (u0 + wave * 64) * 16), 16, 0, 0);
     }
-    const int64_t plane = int64_t(g.H) * g.W;
-    const int8_t *xg = xb + int64_t(n0) * CB * plane * 16;
-    const int ih0 = oh0 * g.sh - g.pt;
-    const int imgs_here = min(t.NB, g.N - n0);
-    for (int p0 = 0; p0 < t.P1s; p0 += NT) {
-        const int2 e = ptab[p0 + tid];  // entries past P1 say "padding"
-        const int ih = ih0 + (e.y & 0xffff);
-        const bool ok = e.x >= 0 && ih >= 0 && ih < g.H && (e.y >> 16) < imgs_here;
-        const int8_t *src = xg + (int64_t(e.x + ih0 * g.W) + int64_t(ichunk * 2) * plane) * 16;
+    const int64_t plane16 = int64_t(g.H) * g.W * 16;
+    const int8_t *xc = xb + int64_t(ichunk * 2) * plane16;   // first half of this chunk
+    const bool second = ichunk * 2 + 1 < CB;                 // an odd block count leaves the last chunk half empty
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            const int8_t *sp = (ok && ichunk * 2 + half < CB) ? src + half * plane * 16 : padvec;
-            __builtin_amdgcn_global_load_lds((gptr_t)sp, (lptr_t)(xl + (half * t.P1s + p0 + wave * 64) * 16), 16, 0, 0);
+    for (int r = 0; r < QR_MAX; ++r) {
+        if (r * NT < t.P1s) {
+            const bool ok = (d.ok >> r) & 1u;
+            const int8_t *src = xc + d.off[r];
+            const int8_t *s0 = ok ? src : padvec;
+            const int8_t *s1 = (ok && second) ? src + plane16 : padvec;
+            __builtin_amdgcn_global_load_lds((gptr_t)s0, (lptr_t)(xl + (r * NT + wave * 64) * 16), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)s1, (lptr_t)(xl + (t.P1s + r * NT + wave * 64) * 16), 16, 0, 0);
         }
     }
 }
@@ -259,11 +289,10 @@ __device__ __forceinline__ void wait_vmcnt(int n) {
 // matrix cores over this step's operands in `cmp`.  The LDS regions never overlap within a step and
 // are __restrict__ so that the copies stay in flight across this step's LDS reads.
 template <int MT, int WM, int WN, int TT>
-__device__ __forceinline__ void qconv_step(char *__restrict__ dma, const char *__restrict__ cmp,
-                                           const int2 *__restrict__ ptab, const int8_t *__restrict__ xb,
-                                           const int8_t *__restrict__ wp, const int8_t *__restrict__ padvec,
-                                           const ConvGeom &g, const TileGeom &t, int CB, bool do_issue, int itile,
-                                           int ichunk, const int (&lds_off)[MT], i32x16 (&acc)[MT]) {
+__device__ __forceinline__ void qconv_step(char *__restrict__ dma, const char *__restrict__ cmp, const PatchDesc &desc,
+                                           const int8_t *__restrict__ xb, const int8_t *__restrict__ wp,
+                                           const int8_t *__restrict__ padvec, const ConvGeom &g, const TileGeom &t, int CB,
+                                           bool do_issue, int ichunk, const int (&lds_off)[MT], i32x16 (&acc)[MT]) {
     constexpr int NT = WM * WN * 64;
     constexpr int K_BLK = WN * 32;
     const int T = TT > 0 ? TT : g.KH * g.KW;
@@ -272,7 +301,7 @@ __device__ __forceinline__ void qconv_step(char *__restrict__ dma, const char *_
     const int wn = wave / WM;
     const int l32 = lane & 31, lh = lane >> 5;
 
-    if (do_issue) qconv_issue<WM, WN, TT>(dma, ptab, xb, wp, padvec, g, t, CB, itile, ichunk);
+    if (do_issue) qconv_issue<WM, WN, TT>(dma, desc, xb, wp, padvec, g, t, CB, ichunk);
     __builtin_amdgcn_sched_barrier(0);
 
     const char *wl = cmp + (lh * K_BLK + wn * 32 + l32) * 16;
@@ -375,9 +404,11 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
     // copies per thread and step (see qconv_issue)
     const int P = w_region_bytes(w_chunk, NT) / (16 * NT) + 2 * (t.P1s / NT);
     // prologue: the first n_stages - 1 steps' copies, in flight behind the index arithmetic below
-    for (int s0 = 0; s0 < n_stages - 1 && s0 < n_steps; ++s0)
-        qconv_issue<WM, WN, TT>(ring + s0 * buf_bytes, ptab, xb, wp, padvec, g, t, CB,
-                                int(blockIdx.x) + (s0 / t.n_chunks) * int(gridDim.x), s0 % t.n_chunks);
+    PatchDesc desc;
+    for (int s0 = 0; s0 < n_stages - 1 && s0 < n_steps; ++s0) {
+        if (s0 % t.n_chunks == 0) qconv_describe<NT>(desc, ptab, g, t, CB, int(blockIdx.x) + (s0 / t.n_chunks) * int(gridDim.x));
+        qconv_issue<WM, WN, TT>(ring + s0 * buf_bytes, desc, xb, wp, padvec, g, t, CB, s0 % t.n_chunks);
+    }
     __builtin_amdgcn_sched_barrier(0);
 
     // Position slot i of this lane: image, row and column inside the tile.  pos[i] packs them for the epilogue
@@ -423,7 +454,11 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
         // This wave's copies of step s0 have landed once no more than the copies of the later steps are outstanding
         // (loads complete in order); after the barrier everybody's have, and everybody is done with step s0 - 1,
         // whose ring slot is refilled now.  A bare s_barrier: __syncthreads() would drain every outstanding copy.
-        wait_vmcnt(P * min(n_stages - 2, n_steps - 1 - s0));
+        {
+            const int pending = P * min(n_stages - 2, n_steps - 1 - s0);
+            if (pending == 0) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): two-stage rings and the last step
+            else wait_vmcnt(pending);
+        }
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
         if (chunk == 0) {
@@ -439,8 +474,10 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[i][v] = int(craw[v]);
         }
-        qconv_step<MT, WM, WN, TT>(ring + dbuf * buf_bytes, ring + cbuf * buf_bytes, ptab, xb, wp, padvec, g, t, CB,
-                                   s0 + n_stages - 1 < n_steps, itile, ichunk, lds_off, acc);
+        const bool do_issue = s0 + n_stages - 1 < n_steps;
+        if (do_issue && ichunk == 0) qconv_describe<NT>(desc, ptab, g, t, CB, itile);
+        qconv_step<MT, WM, WN, TT>(ring + dbuf * buf_bytes, ring + cbuf * buf_bytes, desc, xb, wp, padvec, g, t, CB, do_issue,
+                                   ichunk, lds_off, acc);
         if (++ichunk == t.n_chunks) { ichunk = 0; itile += int(gridDim.x); }
         cbuf = cbuf + 1 == n_stages ? 0 : cbuf + 1;
         dbuf = dbuf + 1 == n_stages ? 0 : dbuf + 1;
@@ -634,6 +671,7 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
     // tell apart.  The patch region is padded to one slot per thread and round.
     constexpr int NT = 256;
     plan.t.P1s = ((plan.t.P1 + NT - 1) / NT) * NT;
+    if (plan.t.P1s / NT > QR_MAX) return 1;  // more copy rounds than the per-tile descriptors hold
     const size_t buf_bytes = size_t(w_region_bytes(T * QCC * K_BLK, NT)) + size_t(QCC) * plan.t.P1s;
     const size_t fixed_bytes = size_t(plan.t.P1s) * 8 + 512 + size_t(plan.t.n_kblocks) * K_BLK * 8;  // 256: table, 256: its alignment
     const int copies = w_region_bytes(T * QCC * K_BLK, NT) / (16 * NT) + 2 * (plan.t.P1s / NT);
