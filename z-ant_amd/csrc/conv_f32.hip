@@ -482,8 +482,21 @@ conv_f32_smallc_pool_kernel(const float *__restrict__ x, const float *__restrict
                     patch[c][r][q] = ok ? x[((int64_t(n) * C + c) * g.H + ih) * g.W + iw] : 0.0f;
                 }
         float *yp = y + int64_t(n) * g.K * pplane + pos;
+        // The weights of a channel are wave-uniform (scalar loads).  Those of channel k + 1 are requested before the
+        // arithmetic of channel k, so the scalar-load latency hides behind 4 * CKK FMAs instead of stalling every channel.
+        float wcur[CKK], wnext[CKK];
+        const float *bp = bias ? bias : w;  // always loadable: the value is dropped below when there is no bias
+        float bcur = bias ? bp[0] : 0.0f, bnext = 0.0f;
+#pragma unroll
+        for (int e = 0; e < CKK; ++e) wcur[e] = w[e];
         for (int k = 0; k < g.K; ++k) {
-            const float *wk = w + int64_t(k) * CKK;
+            const int kn = k + 1 < g.K ? k + 1 : k;
+            const float *wk = w + int64_t(kn) * CKK;
+#pragma unroll
+            for (int e = 0; e < CKK; ++e) wnext[e] = wk[e];
+            const float bl = bp[kn];
+            __builtin_amdgcn_sched_barrier(0);  // keep the requests ahead of the arithmetic
+            bnext = bias ? bl : 0.0f;
             float a00 = 0.f, a01 = 0.f, a10 = 0.f, a11 = 0.f;
 #pragma unroll
             for (int c = 0; c < C; ++c)
@@ -491,16 +504,19 @@ conv_f32_smallc_pool_kernel(const float *__restrict__ x, const float *__restrict
                 for (int kh = 0; kh < KH; ++kh)
 #pragma unroll
                     for (int kw = 0; kw < KW; ++kw) {
-                        const float wv = wk[(c * KH + kh) * KW + kw];
+                        const float wv = wcur[(c * KH + kh) * KW + kw];
                         a00 = __builtin_fmaf(patch[c][kh][kw], wv, a00);
                         a01 = __builtin_fmaf(patch[c][kh][kw + 1], wv, a01);
                         a10 = __builtin_fmaf(patch[c][kh + 1][kw], wv, a10);
                         a11 = __builtin_fmaf(patch[c][kh + 1][kw + 1], wv, a11);
                     }
-            const float b = bias ? bias[k] : 0.0f;
-            float r = fmaxf(fmaxf(a00 + b, a01 + b), fmaxf(a10 + b, a11 + b));
+            // adding the same bias is monotone and so is its rounding: max(a_i + b) == max(a_i) + b exactly
+            float r = fmaxf(fmaxf(a00, a01), fmaxf(a10, a11)) + bcur;
             if (relu) r = r > 0.0f ? r : 0.0f;  // max and ReLU commute (both monotone)
             yp[int64_t(k) * pplane] = r;
+#pragma unroll
+            for (int e = 0; e < CKK; ++e) wcur[e] = wnext[e];
+            bcur = bnext;
         }
     }
 }
