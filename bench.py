@@ -255,6 +255,27 @@ def main():
         hbm("quantize_linear_f32_u8", lambda: tm.quantize_linear(ff, s1, z1, 1), ff.numel() * 5)
         hbm("dequantize_linear_u8_f32", lambda: tm.dequantize_linear(qa, s1, z1, 1), ff.numel() * 5)
         del qa, qb, qp, ff
+        # depthwise 3x3 between channel-blocked tensors (the layout the executor keeps int8 activations in), timed as a
+        # node of a small model: dense 3x3 -> depthwise 3x3 -> dense 3x3 keeps it out of the fused-block pattern
+        from zant_amd.model import Model, U8
+        gd = np.random.default_rng(3)
+        DN, DC, DH = 1024, 96, 48
+        dm = Model(ctx)
+        dt = dm.input((DN, 16, DH, DH), U8, 0.02, 128)
+        dws = gd.uniform(0.001, 0.01, DC).astype(np.float32)
+        dt = dm.qlinearconv(dt, gd.integers(-127, 128, (DC, 16, 3, 3), dtype=np.int8), dws, gd.integers(-99, 99, DC, dtype=np.int32),
+                            0.05, 128, [1, 1], [1, 1, 1, 1])
+        dt = dm.qlinearconv(dt, gd.integers(-127, 128, (DC, 1, 3, 3), dtype=np.int8), dws, gd.integers(-99, 99, DC, dtype=np.int32),
+                            0.05, 128, [1, 1], [1, 1, 1, 1], [1, 1], DC)
+        dt = dm.qlinearconv(dt, gd.integers(-127, 128, (16, DC, 3, 3), dtype=np.int8), dws[:16], gd.integers(-99, 99, 16, dtype=np.int32),
+                            0.05, 128, [1, 1], [1, 1, 1, 1])
+        dm.finalize()
+        dm.profile()
+        dw_ms = sum(dm.profile()[1][1] for _ in range(5)) / 5
+        dw_bytes = 2 * DN * DC * DH * DH + 9 * DC + 8 * DC
+        operators["qlinearconv_depthwise3x3_u8_blocked_1024x96x48x48"] = {
+            "ms": round(dw_ms, 4), "gbs": round(dw_bytes / dw_ms / 1e6, 1), "frac_hbm_peak": round(dw_bytes / dw_ms / 1e6 / PEAK_HBM_GBS, 4)}
+        dm.close()
 
     # ---- int8 networks (configs 4 and 5): whole-network throughput with the calibrated scales of the golden fixture ----
     nets_out = None

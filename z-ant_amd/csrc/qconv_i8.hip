@@ -1227,9 +1227,10 @@ __global__ void __launch_bounds__(256)
 qdw3x3_mfma_kernel(const uint4 *__restrict__ x, const uint32_t *__restrict__ wm, const float *__restrict__ mult,
                    const int32_t *__restrict__ corr, uint8_t *__restrict__ y, ConvGeom g, QConvArgs q, int CB,
                    int blocks_per_pair) {
-    __shared__ uint8_t lut[256];
+    __shared__ __attribute__((aligned(256))) uint8_t lut[256];
     lut[threadIdx.x] = uint8_t((q.has_act ? qact_apply(uint8_t(threadIdx.x), q.act) : uint8_t(threadIdx.x)) ^ 0x80);
     __syncthreads();
+    const unsigned lut_a = lds_address(lut);  // 256-aligned: a converted byte is the low byte of the entry's address
     const int pair = blockIdx.x / blocks_per_pair, blk = blockIdx.x - pair * blocks_per_pair;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lh = lane >> 5;
     const int cb = 2 * pair + lh;
@@ -1291,23 +1292,44 @@ qdw3x3_mfma_kernel(const uint4 *__restrict__ x, const uint32_t *__restrict__ wm,
         uint4 xv[9];
 #pragma unroll
         for (int t = 0; t < 9; ++t) xv[t] = *reinterpret_cast<const uint4 *>(xbytes + (rowb[t / 3] + colb[t % 3]));
+        // Only tiles that touch an image border (or the tail of the channel blocks) replace taps by the padding vector:
+        // a wave-uniform branch keeps the 36 selects out of the interior tiles.
+        const bool inner = rv[0] && rv[2] && cvd[0] && cvd[2];
+        if (__builtin_amdgcn_ballot_w64(!inner) != 0) {
+#pragma unroll
+            for (int t = 0; t < 9; ++t) {
+                const bool ok = rv[t / 3] && cvd[t % 3];
+                xv[t].x = ok ? xv[t].x : pad4; xv[t].y = ok ? xv[t].y : pad4;
+                xv[t].z = ok ? xv[t].z : pad4; xv[t].w = ok ? xv[t].w : pad4;
+            }
+        }
         i32x16 acc;
 #pragma unroll
         for (int t = 0; t < 9; ++t) {
-            const bool ok = rv[t / 3] && cvd[t % 3];
             i32x4 b;
-            b[0] = int(ok ? xv[t].x : pad4); b[1] = int(ok ? xv[t].y : pad4);
-            b[2] = int(ok ? xv[t].z : pad4); b[3] = int(ok ? xv[t].w : pad4);
+            b[0] = int(xv[t].x); b[1] = int(xv[t].y); b[2] = int(xv[t].z); b[3] = int(xv[t].w);
             acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[t], b, t == 0 ? cvec : acc, 0, 0, 0);
         }
         uint32_t d[4];
+        if (q.has_act) {
 #pragma unroll
-        for (int gq = 0; gq < 4; ++gq) {
-            uint32_t o = 0;
+            for (int gq = 0; gq < 4; ++gq) {
+                uint32_t o = 0;
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-                o |= uint32_t(lut[sat_u8_rne_finite(float(acc[gq * 4 + e]) * mv[gq * 4 + e], zpf)]) << (8 * e);
-            d[gq] = o;
+                for (int e = 0; e < 4; ++e)
+                    o |= requant_lookup(float(acc[gq * 4 + e]) * mv[gq * 4 + e], zpf, lut_a) << (8 * e);
+                d[gq] = o;
+            }
+        } else {
+            // no activation: the saturating conversion packs the four bytes of a dword itself
+#pragma unroll
+            for (int gq = 0; gq < 4; ++gq) {
+                uint32_t w4 = 0;
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    w4 = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(float(acc[gq * 4 + e]) * mv[gq * 4 + e]) + zpf, unsigned(e), w4);
+                d[gq] = w4 ^ 0x80808080u;
+            }
         }
         // lanes p and p + 32 exchange one dword per channel block so that each stores 8 consecutive bytes
 #pragma unroll
