@@ -68,7 +68,15 @@ __global__ void __launch_bounds__(kThreads) reduce_mean_lanes_kernel(const float
             if (vec4) {  // the host checked: base 16-byte aligned, every run start and length a multiple of 4
                 const f4 *p4 = reinterpret_cast<const f4 *>(p);
                 float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
-                for (int64_t j = (lo >> 2) + lane; j < (hi >> 2); j += LANES) {
+                int64_t j = (lo >> 2) + lane;
+                const int64_t j_end = hi >> 2;
+                for (; j + 3 * LANES < j_end; j += 4 * LANES) {  // four loads in flight per lane
+                    const f4 v0 = __builtin_nontemporal_load(p4 + j), v1 = __builtin_nontemporal_load(p4 + j + LANES);
+                    const f4 v2 = __builtin_nontemporal_load(p4 + j + 2 * LANES), v3 = __builtin_nontemporal_load(p4 + j + 3 * LANES);
+                    a0 += (v0.x + v1.x) + (v2.x + v3.x); a1 += (v0.y + v1.y) + (v2.y + v3.y);
+                    a2 += (v0.z + v1.z) + (v2.z + v3.z); a3 += (v0.w + v1.w) + (v2.w + v3.w);
+                }
+                for (; j < j_end; j += LANES) {
                     const f4 v = __builtin_nontemporal_load(p4 + j);
                     a0 += v.x; a1 += v.y; a2 += v.z; a3 += v.w;
                 }
@@ -193,27 +201,37 @@ __global__ void __launch_bounds__(kThreads) resize_gather_kernel(const U *__rest
 }
 
 // VEC consecutive outputs of the innermost axis per thread (one 16-byte store); the outer axes are decoded once per thread.
+// Streaming pattern: a workgroup takes ZANT_STREAM_U x 256 consecutive output vectors and issues all its gathers before its
+// stores.
 template <typename U, int VEC>
 __global__ void __launch_bounds__(kThreads) resize_gather_vec_kernel(const U *__restrict__ x, U *__restrict__ y,
                                                                     const int64_t *__restrict__ tab, ResizeGeom g,
                                                                     unsigned nvec, unsigned ow_vec) {
     typedef U UV __attribute__((ext_vector_type(VEC)));
-    const unsigned step = gridDim.x * kThreads;
     const int64_t *tw = tab + g.tab_off[g.rank - 1];
-    for (unsigned v = blockIdx.x * kThreads + threadIdx.x; v < nvec; v += step) {
-        unsigned r = v / ow_vec;
-        const unsigned cv = v - r * ow_vec;
-        int64_t off = 0;
-        for (int d = g.rank - 2; d >= 0; --d) {
-            const unsigned n = unsigned(g.ydim[d]), q = r / n;
-            off += tab[g.tab_off[d] + (r - q * n)];
-            r = q;
-        }
-        const U *row = x + off;
-        UV out;
+    const unsigned base = blockIdx.x * unsigned(kThreads * ZANT_STREAM_U) + threadIdx.x;
+    UV out[ZANT_STREAM_U];
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) out[k] = row[tw[cv * VEC + k]];
-        __builtin_nontemporal_store(out, reinterpret_cast<UV *>(y) + v);
+    for (int u = 0; u < ZANT_STREAM_U; ++u) {
+        const unsigned v = base + unsigned(u * kThreads);
+        if (v < nvec) {
+            unsigned r = v / ow_vec;
+            const unsigned cv = v - r * ow_vec;
+            int64_t off = 0;
+            for (int d = g.rank - 2; d >= 0; --d) {
+                const unsigned n = unsigned(g.ydim[d]), q = r / n;
+                off += tab[g.tab_off[d] + (r - q * n)];
+                r = q;
+            }
+            const U *row = x + off;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) out[u][k] = row[tw[cv * VEC + k]];
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < ZANT_STREAM_U; ++u) {
+        const unsigned v = base + unsigned(u * kThreads);
+        if (v < nvec) __builtin_nontemporal_store(out[u], reinterpret_cast<UV *>(y) + v);
     }
 }
 
@@ -223,7 +241,7 @@ int launch_resize(zant_ctx *ctx, const void *x, void *y, const int64_t *tab, con
     const int64_t ow = g.ydim[g.rank - 1];
     KernelTimer kt(ctx);
     if (ow % VEC == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0 && g.total / VEC < (int64_t(1) << 31))
-        hipLaunchKernelGGL((resize_gather_vec_kernel<U, VEC>), dim3(grid_for(g.total / VEC, kThreads, ctx->num_cus)), dim3(kThreads),
+        hipLaunchKernelGGL((resize_gather_vec_kernel<U, VEC>), dim3(zant_stream_grid(g.total / VEC)), dim3(kThreads),
                            0, ctx->stream, static_cast<const U *>(x), static_cast<U *>(y), tab, g, unsigned(g.total / VEC),
                            unsigned(ow / VEC));
     else
