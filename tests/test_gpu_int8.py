@@ -22,6 +22,9 @@ QCASES = [
     (2, 3, 96, 96, 16, 3, 3, [2, 2], [1, 1, 1, 1], [1, 1], 1),      # MobileNet stem
     (2, 96, 24, 24, 96, 3, 3, [1, 1], [1, 1, 1, 1], [1, 1], 96),    # depthwise
     (2, 48, 25, 25, 48, 3, 3, [2, 2], [1, 1, 1, 1], [1, 1], 48),    # depthwise stride 2, odd size
+    (3, 40, 9, 11, 40, 3, 3, [1, 1], [1, 1, 1, 1], [1, 1], 40),     # depthwise stride 1, odd output height (row pairs)
+    (2, 32, 7, 5, 32, 3, 3, [1, 1], [0, 0, 0, 0], [1, 1], 32),      # depthwise, no padding, 5 x 3 outputs
+    (1, 16, 3, 9, 16, 3, 3, [1, 1], [0, 1, 0, 1], [1, 1], 16),      # depthwise, a single output row
     (2, 16, 24, 24, 96, 1, 1, [1, 1], [0, 0, 0, 0], [1, 1], 1),     # pointwise expand
     (1, 8, 6, 6, 4, 3, 3, [2, 1], [0, 1, 2, 0], [1, 1], 2),         # grouped, asymmetric pads
     (1, 3, 9, 9, 5, 2, 2, [1, 1], [0, 0, 0, 0], [2, 2], 1),         # dilation

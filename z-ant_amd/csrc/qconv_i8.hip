@@ -1223,6 +1223,9 @@ qdw3x3_blocked_kernel(const uint4 *__restrict__ x, const uint32_t *__restrict__ 
 // channel c in column c), built once per workgroup in registers.  1/32 of the multiplies are useful, yet nine MFMAs
 // replace 144 dot instructions per lane, which is what bounded the VALU version.  The accumulators come out as 16
 // channels of one position per lane, requantised and stored like the dense kernel's blocked epilogue.
+// ROWS = 2 (stride 1): a lane computes two vertically adjacent outputs from a 4 x 3 patch -- twelve loads instead of
+// eighteen, one index decode, and two independent accumulator chains whose MFMAs interleave.
+template <int ROWS>
 __global__ void __launch_bounds__(256)
 qdw3x3_mfma_kernel(const uint4 *__restrict__ x, const uint32_t *__restrict__ wm, const float *__restrict__ mult,
                    const int32_t *__restrict__ corr, uint8_t *__restrict__ y, ConvGeom g, QConvArgs q, int CB,
@@ -1249,98 +1252,110 @@ qdw3x3_mfma_kernel(const uint4 *__restrict__ x, const uint32_t *__restrict__ wm,
         }
     }
     float mv[16];
-    int cv[16];
+    i32x16 cvec;
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
         const int k = pair * 32 + (v >> 2) * 8 + lh * 4 + (v & 3);
         mv[v] = mult[k];
-        cv[v] = corr[k];
+        cvec[v] = corr[k];
     }
-    const unsigned total = unsigned(g.N) * unsigned(g.OH) * unsigned(g.OW);  // < 2^31 (checked by the host)
+    // positions are (image, row group, column): a row group is ROWS output rows
+    const int OHG = (g.OH + ROWS - 1) / ROWS;
+    const unsigned total = unsigned(g.N) * unsigned(OHG) * unsigned(g.OW);  // < 2^31 (checked by the host)
     const unsigned n_ptiles = (total + 31u) / 32u;
-    const unsigned per_img = unsigned(g.OH) * unsigned(g.OW);                // < 2^20 (checked by the host)
+    const unsigned per_img = unsigned(OHG) * unsigned(g.OW);                 // < 2^20 (checked by the host)
     const float inv_per_img = 1.0f / float(per_img), inv_ow = 1.0f / float(g.OW);
     const bool small_total = total < (1u << 20);
     const uint32_t pad4 = uint32_t(q.x_zp ^ 0x80) * 0x01010101u;
     const float zpf = float(q.y_zp);
-    i32x16 cvec;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) cvec[v] = cv[v];
     const char *xbytes = reinterpret_cast<const char *>(x);  // the whole tensor is < 4 GB (checked by the host)
     const unsigned plane = unsigned(g.H) * unsigned(g.W);
+    constexpr int PR = ROWS + 2;  // input rows of the patch (ROWS = 2 implies stride 1)
     for (unsigned pt = unsigned(blk) * 4u + unsigned(wave); pt < n_ptiles; pt += unsigned(blocks_per_pair) * 4u) {
         const unsigned i = pt * 32u + unsigned(l32);
         const bool valid = i < total;
         const unsigned ii = valid ? i : total - 1u;
         const unsigned n = small_total ? unsigned(small_div(int(ii), int(per_img), inv_per_img)) : ii / per_img;
         const int rem = int(ii - n * per_img);
-        const int oh = small_div(rem, g.OW, inv_ow), ow = rem - oh * g.OW;
+        const int ohg = small_div(rem, g.OW, inv_ow), ow = rem - ohg * g.OW;
+        const int oh = ohg * ROWS;
         // Every tap is loaded from an address inside the tensor (a tap outside the image reads its clamped neighbour)
         // and replaced by the padding vector afterwards: no divergent control flow around the loads.
         const int ih0 = oh * g.sh - g.pt, iw0 = ow * g.sw - g.pl;  // top-left tap
         const unsigned base = (n * unsigned(CB) + unsigned(cb_ok ? cb : 0)) * plane * 16u;
-        bool rv[3], cvd[3];
-        unsigned rowb[3], colb[3];
+        bool rv[PR], cvd[3];
+        unsigned rowb[PR], colb[3];
+#pragma unroll
+        for (int k = 0; k < PR; ++k) {
+            const int ih = ih0 + k;
+            rv[k] = cb_ok && ih >= 0 && ih < g.H;
+            rowb[k] = base + unsigned(min(max(ih, 0), g.H - 1)) * unsigned(g.W) * 16u;
+        }
 #pragma unroll
         for (int k = 0; k < 3; ++k) {
-            const int ih = ih0 + k, iw = iw0 + k;
-            rv[k] = cb_ok && ih >= 0 && ih < g.H;
+            const int iw = iw0 + k;
             cvd[k] = iw >= 0 && iw < g.W;
-            rowb[k] = base + unsigned(min(max(ih, 0), g.H - 1)) * unsigned(g.W) * 16u;
             colb[k] = unsigned(min(max(iw, 0), g.W - 1)) * 16u;
         }
-        uint4 xv[9];
+        uint4 xv[PR * 3];
 #pragma unroll
-        for (int t = 0; t < 9; ++t) xv[t] = *reinterpret_cast<const uint4 *>(xbytes + (rowb[t / 3] + colb[t % 3]));
+        for (int t = 0; t < PR * 3; ++t) xv[t] = *reinterpret_cast<const uint4 *>(xbytes + (rowb[t / 3] + colb[t % 3]));
         // Only tiles that touch an image border (or the tail of the channel blocks) replace taps by the padding vector:
-        // a wave-uniform branch keeps the 36 selects out of the interior tiles.
-        const bool inner = rv[0] && rv[2] && cvd[0] && cvd[2];
+        // a wave-uniform branch keeps the selects out of the interior tiles.
+        const bool inner = rv[0] && rv[PR - 1] && cvd[0] && cvd[2];
         if (__builtin_amdgcn_ballot_w64(!inner) != 0) {
 #pragma unroll
-            for (int t = 0; t < 9; ++t) {
+            for (int t = 0; t < PR * 3; ++t) {
                 const bool ok = rv[t / 3] && cvd[t % 3];
                 xv[t].x = ok ? xv[t].x : pad4; xv[t].y = ok ? xv[t].y : pad4;
                 xv[t].z = ok ? xv[t].z : pad4; xv[t].w = ok ? xv[t].w : pad4;
             }
         }
-        i32x16 acc;
+        i32x16 acc[ROWS];
 #pragma unroll
-        for (int t = 0; t < 9; ++t) {
-            i32x4 b;
-            b[0] = int(xv[t].x); b[1] = int(xv[t].y); b[2] = int(xv[t].z); b[3] = int(xv[t].w);
-            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[t], b, t == 0 ? cvec : acc, 0, 0, 0);
-        }
-        uint32_t d[4];
-        if (q.has_act) {
+        for (int t = 0; t < 9; ++t)
 #pragma unroll
-            for (int gq = 0; gq < 4; ++gq) {
-                uint32_t o = 0;
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    o |= requant_lookup(float(acc[gq * 4 + e]) * mv[gq * 4 + e], zpf, lut_a) << (8 * e);
-                d[gq] = o;
+            for (int r = 0; r < ROWS; ++r) {
+                const uint4 &xt = xv[t + 3 * r];  // output row r reads patch rows r .. r + 2
+                i32x4 b;
+                b[0] = int(xt.x); b[1] = int(xt.y); b[2] = int(xt.z); b[3] = int(xt.w);
+                acc[r] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[t], b, t == 0 ? cvec : acc[r], 0, 0, 0);
             }
-        } else {
-            // no activation: the saturating conversion packs the four bytes of a dword itself
 #pragma unroll
-            for (int gq = 0; gq < 4; ++gq) {
-                uint32_t w4 = 0;
+        for (int r = 0; r < ROWS; ++r) {
+            uint32_t d[4];
+            if (q.has_act) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    w4 = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(float(acc[gq * 4 + e]) * mv[gq * 4 + e]) + zpf, unsigned(e), w4);
-                d[gq] = w4 ^ 0x80808080u;
+                for (int gq = 0; gq < 4; ++gq) {
+                    uint32_t o = 0;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        o |= requant_lookup(float(acc[r][gq * 4 + e]) * mv[gq * 4 + e], zpf, lut_a) << (8 * e);
+                    d[gq] = o;
+                }
+            } else {
+                // no activation: the saturating conversion packs the four bytes of a dword itself
+#pragma unroll
+                for (int gq = 0; gq < 4; ++gq) {
+                    uint32_t w4 = 0;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        w4 = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(float(acc[r][gq * 4 + e]) * mv[gq * 4 + e]) + zpf, unsigned(e), w4);
+                    d[gq] = w4 ^ 0x80808080u;
+                }
             }
-        }
-        // lanes p and p + 32 exchange one dword per channel block so that each stores 8 consecutive bytes
+            // lanes p and p + 32 exchange one dword per channel block so that each stores 8 consecutive bytes
+            const bool row_ok = valid && oh + r < g.OH;
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
-            const uint32_t send = lh ? d[2 * b] : d[2 * b + 1];
-            const uint32_t recv = uint32_t(__shfl_xor(int(send), 32, 64));
-            const uint2 out = lh ? make_uint2(recv, d[2 * b + 1]) : make_uint2(d[2 * b], recv);
-            const int cbo = 2 * pair + b;
-            if (valid && cbo < CB) {
-                uint8_t *yp = y + (((int64_t(n) * CB + cbo) * g.OH + oh) * int64_t(g.OW) + ow) * 16 + lh * 8;
-                *reinterpret_cast<uint2 *>(yp) = out;
+            for (int b = 0; b < 2; ++b) {
+                const uint32_t send = lh ? d[2 * b] : d[2 * b + 1];
+                const uint32_t recv = uint32_t(__shfl_xor(int(send), 32, 64));
+                const uint2 out = lh ? make_uint2(recv, d[2 * b + 1]) : make_uint2(d[2 * b], recv);
+                const int cbo = 2 * pair + b;
+                if (row_ok && cbo < CB) {
+                    uint8_t *yp = y + (((int64_t(n) * CB + cbo) * g.OH + oh + r) * int64_t(g.OW) + ow) * 16 + lh * 8;
+                    *reinterpret_cast<uint2 *>(yp) = out;
+                }
             }
         }
     }
@@ -1375,8 +1390,12 @@ int run_qdw_blocked(zant_ctx *ctx, const uint8_t *xb, const int8_t *w, const flo
         int64_t(g.N) * CB * g.H * g.W * 16 < (int64_t(1) << 32)) {
         const int64_t want = std::max<int64_t>(1, (int64_t(ctx->num_cus) * 8 + n_pairs - 1) / n_pairs);
         const int blocks_per_pair = int(std::min<int64_t>(std::max<int64_t>(ceil_div64(per_cb, 128), 1), want));
-        hipLaunchKernelGGL(qdw3x3_mfma_kernel, dim3(unsigned(n_pairs) * blocks_per_pair), dim3(256), 0, ctx->stream,
-                           reinterpret_cast<const uint4 *>(xb), wm, mult, corr, yb, g, q, CB, blocks_per_pair);
+        if (g.sh == 1 && g.sw == 1 && g.OH >= 2)
+            hipLaunchKernelGGL(qdw3x3_mfma_kernel<2>, dim3(unsigned(n_pairs) * blocks_per_pair), dim3(256), 0, ctx->stream,
+                               reinterpret_cast<const uint4 *>(xb), wm, mult, corr, yb, g, q, CB, blocks_per_pair);
+        else
+            hipLaunchKernelGGL(qdw3x3_mfma_kernel<1>, dim3(unsigned(n_pairs) * blocks_per_pair), dim3(256), 0, ctx->stream,
+                               reinterpret_cast<const uint4 *>(xb), wm, mult, corr, yb, g, q, CB, blocks_per_pair);
     } else {
         const int64_t want = std::max<int64_t>(1, (int64_t(ctx->num_cus) * 16 + CB - 1) / CB);
         const int blocks_per_cb = int(std::min<int64_t>(std::max<int64_t>(ceil_div64(per_cb, 256), 1), want));
