@@ -259,6 +259,8 @@ int zant_hip_qlinear_global_avgpool_u8(zant_ctx *ctx, const uint8_t *x, const in
  * Tensor handles are small non-negative ints; a negative return is a zant_status. */
 enum zant_dtype { ZANT_F32 = 0, ZANT_U8 = 1 };
 
+/* ctx == NULL creates a dry-run model: nodes are validated and shapes can be queried (zant_model_tensor_dims,
+ * zant_model_output_dims) without touching a GPU, as a code generator needs; zant_model_finalize refuses it. */
 int zant_model_create(zant_ctx *ctx, zant_model **out);
 void zant_model_destroy(zant_model *m);
 /* The network input (batch compiled in, like the reference).  scale / zp describe a u8 input. */
