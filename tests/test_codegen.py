@@ -90,15 +90,16 @@ def test_generated_mnist8_library_matches_the_oracle(codegen, tmp_path):
 
 
 @pytest.mark.gpu
-def test_generated_int8_detector_library_reproduces_the_golden_bytes(codegen, tmp_path):
+@pytest.mark.parametrize("net", ["tiny_yolo_int8", "mobilenet_v2_035_int8"])
+def test_generated_int8_network_library_reproduces_the_golden_bytes(codegen, tmp_path, net):
     from zant_amd import networks as nets
-    gold = json.load(open(os.path.join(HERE, "golden", "int8_networks.json")))["tiny_yolo_int8"]
-    arch = nets.tiny_yolo_arch()
+    gold = json.load(open(os.path.join(HERE, "golden", "int8_networks.json")))[net]
+    arch = nets.tiny_yolo_arch() if net == "tiny_yolo_int8" else nets.mobilenet_v2_035_arch()
     params = nets.int8_params(arch, seed=gold["param_seed"])
     data, out_shape = onnx_writer.int8_network(arch, params, gold["quant"], 2)
     p = tmp_path / "yolo.onnx"
     p.write_bytes(data)
-    info = codegen.generate(str(p), str(tmp_path), "tiny_yolo")
+    info = codegen.generate(str(p), str(tmp_path), net)
     assert info["in_dtype"] == 1 and info["out_dtype"] == 1 and tuple(info["out_shape"]) == tuple(out_shape)
     lib = _load(codegen.compile_library(info))
     x = np.random.default_rng(gold["input_seed"]).integers(0, 256, (2,) + tuple(arch["input"]), dtype=np.uint8)
@@ -106,4 +107,4 @@ def test_generated_int8_detector_library_reproduces_the_golden_bytes(codegen, tm
     assert ptr is not None
     y = np.ctypeslib.as_array(C.cast(ptr, C.POINTER(C.c_uint8)), (int(np.prod(out_shape)),)).copy()
     np.testing.assert_array_equal(y, np.array(gold["expected_u8"], np.uint8))
-    lib.tiny_yolo_shutdown()
+    getattr(lib, net + "_shutdown")()
