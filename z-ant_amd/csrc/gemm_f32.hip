@@ -324,8 +324,6 @@ __device__ __forceinline__ void gemm_step(float *__restrict__ dma, unsigned cmp_
     constexpr int NW = WM * WN, BM = WM * MT * 32, BN = WN * 32;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave % WM, wn = wave / WM;
-    const int l32 = lane & 31, lh = lane >> 5;
     constexpr int PA = stage_instrs<AM, BM>() / NW, PB = stage_instrs<BMODE, BN>() / NW;
     static_assert(PA + PB <= 4 * MT * (BK / 8), "one copy instruction per MFMA at most");
     // Whole chunk inside K: no masks, addresses are a uniform offset from chunk 0, and the copy instructions are

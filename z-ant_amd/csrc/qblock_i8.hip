@@ -348,7 +348,6 @@ int zant_qblock_blocked(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], 
     // LDS: fixed part, then per patch position the input and expanded bytes and one table entry
     const size_t w1_bytes = size_t(a.Cin32) * a.Ce32 * 1024, w2_bytes = size_t(a.Ce32) * CO32 * 1024;
     const size_t wdw_bytes = size_t(CeP) * 9 * 4, tab_bytes = (size_t(CeP) * 4 + size_t(CO32) * 32 * 2) * 4;
-    const size_t fixed = 512 + w1_bytes + w2_bytes + wdw_bytes + tab_bytes;
     if (CO32 > 4) return 1;
     // Tile = NB whole images, or TH output rows of one image.  Among the shapes that fit -- in half a CU's LDS first, so
     // that two workgroups share a CU -- the one with the fewest wave instructions per image by a model of the kernel's

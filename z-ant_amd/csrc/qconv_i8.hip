@@ -653,13 +653,13 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
     // Both workgroup shapes are tried for more than 32 output channels; plans are ranked by the planner's time estimate
     // over the GPU's 2 x CUs workgroup slots.
     const int target = 2 * ctx->num_cus;
-    int WN = 1, WM = 4;
+    int WN = 1;
     // The footprint counts two staging buffers: larger tiles (more operand reuse per staged byte) beat a deeper ring.
     bool have = zant_plan_conv_tiles(gp, 4, 1, 6, 2, 16, 80 * 1024, &plan, pool, target, 32, 256);
     if (g.K > 32) {
         TilePlan wide;
         if (zant_plan_conv_tiles(gp, 2, 2, 6, 2, 16, 80 * 1024, &wide, pool, target, 32, 256) && (!have || wide.score >= plan.score * 0.98)) {
-            plan = wide; WN = 2; WM = 2; have = true;
+            plan = wide; WN = 2; have = true;
         }
     }
     if (!have || plan.eff < 0.4) return 1;
