@@ -108,3 +108,29 @@ def test_generated_int8_network_library_reproduces_the_golden_bytes(codegen, tmp
     y = np.ctypeslib.as_array(C.cast(ptr, C.POINTER(C.c_uint8)), (int(np.prod(out_shape)),)).copy()
     np.testing.assert_array_equal(y, np.array(gold["expected_u8"], np.uint8))
     getattr(lib, net + "_shutdown")()
+
+
+def test_dry_run_model_validates_and_answers_shapes_without_a_gpu(codegen):
+    """A model built without a context: nodes are checked, shapes are available, nothing can run."""
+    from zant_amd import ZantError
+    from zant_amd.model import Model
+    m = Model(None)
+    x = m.input((2, 3, 16, 16))
+    c = m.conv(x, np.zeros((8, 3, 3, 3), np.float32), np.zeros(8, np.float32), [1, 1], [1, 1, 1, 1], None, 1, "NOTSET")
+    p = m.maxpool(m.relu(c), [2, 2], [2, 2])
+    r = m.resize_nearest(p, [1.0, 1.0, 2.0, 2.0], None, "half_pixel")
+    k = m.concat([c, r], 1)
+    g = m.reduce_mean(m.sigmoid(k), [2, 3], False)
+    assert m.tensor_shape(c) == (2, 8, 16, 16) and m.tensor_shape(p) == (2, 8, 8, 8) and m.tensor_shape(r) == (2, 8, 16, 16)
+    assert m.tensor_shape(k) == (2, 16, 16, 16) and m.tensor_shape(g) == (2, 16)
+    with pytest.raises(ZantError) as e:
+        m.conv(x, np.zeros((8, 4, 3, 3), np.float32), None, [1, 1], None, None, 1, None)  # channel mismatch
+    assert e.value.code < 0
+    with pytest.raises(ZantError) as e:
+        m.concat([c, p], 1)
+    assert e.value.name == "MismatchedShape"
+    with pytest.raises(ZantError) as e:
+        m.finalize()
+    assert e.value.name == "NullPointer"
+    assert m.input_ptr is None
+    m.close()
