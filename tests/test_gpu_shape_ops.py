@@ -171,6 +171,9 @@ def test_resize_known_answers(G, c):
     ((11,), [3.3], None, np.int16),
     ((2, 1, 4, 4), None, [2, 1, 1, 1], np.float32),   # one-element outputs (0 / 0 under align_corners)
     ((2, 2, 3, 3, 3), [1, 1, 2, 2, 2], None, np.float32),
+    ((3000, 2, 8), None, [3000, 3, 16], np.float32),  # the outermost axis' table is too long for LDS: looked up in global memory
+    ((2, 1100), None, [3, 4400], np.float32),          # even the innermost one is
+    ((2100, 4), None, [2100, 8], np.uint8),
 ])
 @pytest.mark.parametrize("coord", ["half_pixel", "align_corners", "asymmetric"])
 def test_resize_matches_oracle(G, shape, scales, sizes, dtype, coord):
@@ -179,7 +182,27 @@ def test_resize_matches_oracle(G, shape, scales, sizes, dtype, coord):
     np.testing.assert_array_equal(y, zo.resize(x, "nearest", scales, sizes, coord))
 
 
-def test_resize_at_full_size_repeats_elements(G):
-    x = torch.randint(0, 255, (512, 128, 6, 6), dtype=torch.uint8, device="cuda")
+@pytest.mark.parametrize("dtype", [np.uint8, np.int16, np.float32, np.float64])
+@pytest.mark.parametrize("shape,sizes", [
+    ((3, 5, 7, 16), [3, 5, 14, 32]),    # rows and columns doubled
+    ((2, 3, 5, 32), [2, 3, 15, 64]),    # rows tripled
+    ((2, 3, 5, 32), [2, 3, 5, 64]),     # rows kept
+    ((9, 48), [36, 96]),                # rank 2, rows x4
+    ((2, 3, 5, 32), [4, 3, 10, 64]),    # a leading axis resized too
+    ((1, 1300, 2, 16), [1, 1300, 4, 32]),  # more rows than one workgroup covers
+])
+@pytest.mark.parametrize("coord", ["half_pixel", "align_corners", "asymmetric"])
+def test_resize_integer_upsampling_matches_oracle(G, shape, sizes, dtype, coord):
+    # under half_pixel an integer factor repeats elements; asymmetric and align_corners round differently at the same sizes
+    x = (np.random.default_rng(11).standard_normal(shape) * 90).astype(dtype)
+    y = G.tm.resize(dev(x), "nearest", None, sizes, coord).cpu().numpy()
+    np.testing.assert_array_equal(y, zo.resize(x, "nearest", None, sizes, coord))
+    if coord == "half_pixel" and tuple(sizes[:-2]) == shape[:-2]:
+        np.testing.assert_array_equal(y, x.repeat(sizes[-2] // shape[-2], axis=-2).repeat(2, axis=-1))
+
+
+@pytest.mark.parametrize("shape", [(512, 128, 6, 6), (256, 64, 28, 32)])
+def test_resize_at_full_size_repeats_elements(G, shape):
+    x = torch.randint(0, 255, shape, dtype=torch.uint8, device="cuda")
     y = G.tm.resize(x, "nearest", [1.0, 1.0, 2.0, 2.0], None, "half_pixel")
     assert torch.equal(y, x.repeat_interleave(2, dim=2).repeat_interleave(2, dim=3))

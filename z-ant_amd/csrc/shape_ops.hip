@@ -2,6 +2,7 @@
 // (lib_reduction_math.zig:30-268, lib_shape_math.zig:22-160, 307-630 in the reference).
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdint>
 
@@ -153,11 +154,14 @@ struct ResizeGeom {
     int64_t tab_off[8];  // where each axis starts in the offset table
     int64_t tab_total, total;
     int coord_mode;
+    FastDiv ydiv[8];  // division by ydim[d] (the vector kernel, whose indices stay below 2^31)
+    FastDiv owdiv;    // ... by the number of vectors in an output row
 };
 
 // Input offset (index * stride) of every output coordinate of every axis, in the reference's f32 arithmetic
 // (lib_shape_math.zig:128-145): scale = out / in; half_pixel (o + 0.5) / scale - 0.5; align_corners o (in-1) / (out-1);
 // otherwise o / scale; round half away from zero; clamp.
+// Written twice: as 64-bit offsets, and (for inputs of fewer than 2^31 elements) as 32-bit ones behind them.
 __global__ void __launch_bounds__(kThreads) resize_table_kernel(int64_t *__restrict__ tab, ResizeGeom g) {
     const int64_t t = int64_t(blockIdx.x) * kThreads + threadIdx.x;
     if (t >= g.tab_total) return;
@@ -174,6 +178,7 @@ __global__ void __launch_bounds__(kThreads) resize_table_kernel(int64_t *__restr
     i = i < 0 ? 0 : i;
     i = i > g.xdim[d] - 1 ? g.xdim[d] - 1 : i;
     tab[t] = i * g.xstride[d];
+    reinterpret_cast<int *>(tab + g.tab_total)[t] = int(i * g.xstride[d]);
 }
 
 template <typename U>
@@ -202,30 +207,52 @@ __global__ void __launch_bounds__(kThreads) resize_gather_kernel(const U *__rest
 
 // VEC consecutive outputs of the innermost axis per thread (one 16-byte store); the outer axes are decoded once per thread.
 // Streaming pattern: a workgroup takes ZANT_STREAM_U x 256 consecutive output vectors and issues all its gathers before its
-// stores.
+// stores.  Stores are what this kernel is built around: whole, aligned, consecutive vectors (a variant that loaded whole
+// input vectors and wrote each to its repeated places was twice as slow on rows that are not multiples of a cache line).
+// What then bounds it is the address unit of the vector memory path, which takes every lane of every load whatever the
+// lanes point at: so the tables of the innermost `lds_axes` axes (kResizeLdsEntries entries at most, 32-bit) are first
+// copied to LDS and looked up there, and only the VEC gathers and the outer axes' 32-bit lookups go through it.
+constexpr int kResizeLdsEntries = 2048;
 template <typename U, int VEC>
 __global__ void __launch_bounds__(kThreads) resize_gather_vec_kernel(const U *__restrict__ x, U *__restrict__ y,
-                                                                    const int64_t *__restrict__ tab, ResizeGeom g,
-                                                                    unsigned nvec, unsigned ow_vec) {
+                                                                    const int *__restrict__ tab, ResizeGeom g,
+                                                                    unsigned nvec, unsigned ow_vec, int lds_axes, unsigned n_chunks) {
     typedef U UV __attribute__((ext_vector_type(VEC)));
-    const int64_t *tw = tab + g.tab_off[g.rank - 1];
-    const unsigned base = blockIdx.x * unsigned(kThreads * ZANT_STREAM_U) + threadIdx.x;
+    __shared__ __attribute__((aligned(16))) int tab_lds[kResizeLdsEntries];
+    const int first = g.rank - lds_axes;  // axes first .. rank-1 are looked up in LDS
+    const int lds_base = first < g.rank ? int(g.tab_off[first]) : int(g.tab_total);
+    for (int c = threadIdx.x; c < int(g.tab_total) - lds_base; c += kThreads) tab_lds[c] = tab[lds_base + c];
+    __syncthreads();
+    const int *tw = tab + g.tab_off[g.rank - 1];
+    const int tw_lds = int(g.tab_off[g.rank - 1]) - lds_base;
+    // a workgroup stays for several chunks so that the table copy above is paid once and its waves drift apart
+    for (unsigned chunk = blockIdx.x; chunk < n_chunks; chunk += gridDim.x) {
+    const unsigned base = chunk * unsigned(kThreads * ZANT_STREAM_U) + threadIdx.x;
     UV out[ZANT_STREAM_U];
 #pragma unroll
     for (int u = 0; u < ZANT_STREAM_U; ++u) {
         const unsigned v = base + unsigned(u * kThreads);
         if (v < nvec) {
-            unsigned r = v / ow_vec;
+            unsigned r = fastdiv(v, g.owdiv);
             const unsigned cv = v - r * ow_vec;
-            int64_t off = 0;
+            int off = 0;  // below 2^31: the input has fewer elements than that
             for (int d = g.rank - 2; d >= 0; --d) {
-                const unsigned n = unsigned(g.ydim[d]), q = r / n;
-                off += tab[g.tab_off[d] + (r - q * n)];
+                const unsigned n = unsigned(g.ydim[d]), q = fastdiv(r, g.ydiv[d]);
+                const int e = int(g.tab_off[d]) + int(r - q * n);
+                off += d >= first ? tab_lds[e - lds_base] : tab[e];
                 r = q;
             }
             const U *row = x + off;
+            if (lds_axes > 0) {
+                int col[VEC];
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) out[u][k] = row[tw[cv * VEC + k]];
+                for (int k = 0; k < VEC; ++k) col[k] = tab_lds[tw_lds + int(cv) * VEC + k];
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) out[u][k] = row[col[k]];
+            } else {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) out[u][k] = row[tw[cv * VEC + k]];
+            }
         }
     }
 #pragma unroll
@@ -233,18 +260,27 @@ __global__ void __launch_bounds__(kThreads) resize_gather_vec_kernel(const U *__
         const unsigned v = base + unsigned(u * kThreads);
         if (v < nvec) __builtin_nontemporal_store(out[u], reinterpret_cast<UV *>(y) + v);
     }
+    }
 }
 
 template <typename U>
-int launch_resize(zant_ctx *ctx, const void *x, void *y, const int64_t *tab, const ResizeGeom &g) {
+int launch_resize(zant_ctx *ctx, const void *x, void *y, const int64_t *tab, ResizeGeom &g) {
     constexpr int VEC = 16 / int(sizeof(U));
     const int64_t ow = g.ydim[g.rank - 1];
+    int64_t in_total = 1;
+    for (int d = 0; d < g.rank; ++d) in_total *= g.xdim[d];
     KernelTimer kt(ctx);
-    if (ow % VEC == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0 && g.total / VEC < (int64_t(1) << 31))
-        hipLaunchKernelGGL((resize_gather_vec_kernel<U, VEC>), dim3(zant_stream_grid(g.total / VEC)), dim3(kThreads),
-                           0, ctx->stream, static_cast<const U *>(x), static_cast<U *>(y), tab, g, unsigned(g.total / VEC),
-                           unsigned(ow / VEC));
-    else
+    if (ow % VEC == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0 && g.total / VEC < (int64_t(1) << 31) &&
+        in_total < (int64_t(1) << 31) && g.tab_total < (int64_t(1) << 31)) {
+        for (int d = 0; d < g.rank; ++d) g.ydiv[d] = make_fastdiv(unsigned(g.ydim[d]));  // ydim[d] <= total / VEC here for d < rank - 1
+        g.owdiv = make_fastdiv(unsigned(ow / VEC));
+        int lds_axes = 0;  // as many innermost axes as fit
+        while (lds_axes < g.rank && g.tab_total - g.tab_off[g.rank - 1 - lds_axes] <= kResizeLdsEntries) ++lds_axes;
+        const unsigned n_chunks = zant_stream_grid(g.total / VEC);
+        hipLaunchKernelGGL((resize_gather_vec_kernel<U, VEC>), dim3(std::min(n_chunks, unsigned(ctx->num_cus) * 8u)), dim3(kThreads), 0,
+                           ctx->stream, static_cast<const U *>(x), static_cast<U *>(y), reinterpret_cast<const int *>(tab + g.tab_total),
+                           g, unsigned(g.total / VEC), unsigned(ow / VEC), lds_axes, n_chunks);
+    } else
         hipLaunchKernelGGL(resize_gather_kernel<U>, dim3(grid_for(g.total, kThreads, ctx->num_cus)), dim3(kThreads), 0, ctx->stream,
                            static_cast<const U *>(x), static_cast<U *>(y), tab, g);
     ZANT_LAUNCH_CHECK(ctx);
@@ -475,7 +511,7 @@ extern "C" int zant_hip_resize_nearest(zant_ctx *ctx, const void *x, const int64
     int64_t st = 1;
     for (int i = rank - 1; i >= 0; --i) { g.xstride[i] = st; st *= xdim[i]; }
     void *ws = nullptr;
-    const int rc = zant_workspace(ctx, size_t(g.tab_total) * sizeof(int64_t), &ws);
+    const int rc = zant_workspace(ctx, size_t(g.tab_total) * (sizeof(int64_t) + sizeof(int)), &ws);
     if (rc != ZANT_OK) return rc;
     int64_t *tab = static_cast<int64_t *>(ws);
     hipLaunchKernelGGL(resize_table_kernel, dim3(unsigned(ceil_div64(g.tab_total, kThreads))), dim3(kThreads), 0, ctx->stream, tab, g);
