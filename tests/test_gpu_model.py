@@ -203,6 +203,36 @@ def test_conv_with_fused_pool_on_the_matrix_cores(G, N, C, H, W, K, k, pad, relu
     m.close()
 
 
+@pytest.mark.parametrize("N,C,H,W,K,k,pad,relu", [
+    (19, 1, 28, 28, 32, 3, 0, True),    # single-channel 3x3 on the matrix cores; the last workgroup holds 3 of 8 images
+    (5, 1, 31, 27, 40, 3, 0, False),    # odd sizes (scalar image copy, dropped last row / column), two channel blocks, no ReLU
+    (4, 1, 64, 64, 8, 3, 0, True),      # two images per workgroup, fewer channels than a block
+    (3, 1, 120, 90, 16, 3, 0, True),    # an image too large for the LDS copy: the direct kernel
+    (6, 1, 28, 28, 32, 3, 1, True),     # padded: the direct kernel
+    (7, 1, 28, 28, 20, 5, 0, True),     # 5x5
+    (4, 3, 30, 30, 24, 3, 0, True),     # three channels
+])
+def test_first_layer_conv_with_fused_pool(G, N, C, H, W, K, k, pad, relu):
+    from zant_amd.model import Model
+    g = np.random.default_rng(N * 100 + K)
+    x = g.standard_normal((N, C, H, W), dtype=np.float32)
+    w = (g.standard_normal((K, C, k, k)) * np.sqrt(2.0 / (C * k * k))).astype(np.float32)
+    b = (g.standard_normal(K) * 0.1).astype(np.float32)
+    m = Model(G.tm.context())
+    t = m.conv(m.input((N, C, H, W)), w, b, [1, 1], [pad] * 4, [1, 1], 1, "NOTSET")
+    if relu:
+        t = m.relu(t)
+    t = m.maxpool(t, [2, 2], [2, 2])
+    m.finalize()
+    assert m.num_launches == 1
+    ref = zo.Conv(x, w, b, [1, 1], [pad] * 4, [1, 1], 1, "NOTSET")
+    if relu:
+        ref = zo.ReLU(ref)
+    ref = zo.onnx_maxpool(ref, [2, 2], [2, 2], [1, 1], [0, 0, 0, 0])
+    np.testing.assert_allclose(m.predict_host(x), ref, rtol=G.RTOL, atol=G.ATOL)
+    m.close()
+
+
 def test_int8_network_fuses_activation_and_is_bit_exact(G):
     """QLinearConv -> Dequant/LeakyReLU/Quant -> MaxPool -> QLinearConv -> ReLU6 -> residual add -> global average pool."""
     from zant_amd.model import Model, U8

@@ -18,6 +18,7 @@
 namespace {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(1))) const void *gptr_t;
 typedef __attribute__((address_space(3))) void *lptr_t;
 
@@ -238,7 +239,7 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
     }
     // With a fused 2x2/2 max pool the lane's tile registers 4j .. 4j+3 are the four members of ONE pooling window
     // (pooled position (wm*MT/4 + j)*32 + l32), so the pool is a register-wise max in the epilogue.
-    const int per_img_p = POOL ? (t.TH / 2) * t.POW : 0;
+    const int per_img_p = POOL ? (t.TH / 2) * t.POW : 1;
     int lds_off[MT];  // float4 index of each of this lane's output positions inside a patch half
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
@@ -521,6 +522,115 @@ conv_f32_smallc_pool_kernel(const float *__restrict__ x, const float *__restrict
     }
 }
 
+// max without the NaN-quieting pass the compiler puts in front of fmaxf (an MFMA result is never a signalling NaN); a NaN
+// operand yields the other one, like fmaxf
+__device__ __forceinline__ float vmax(float a, float b) {
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ float vmax3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+// Single-channel 3x3 first layer + ReLU + MaxPool 2x2/2 on the matrix cores (stride 1, no padding).
+//   D[k, p] = sum_t W[k, t] * X[window(p) + tap t]: output channels are the MFMA rows (32 per workgroup), pooled
+// positions the columns, and the nine taps the reduction axis, two per v_mfma_f32_32x32x2_f32: (0,0)|(0,1), (1,0)|(1,1),
+// (2,0)|(2,1), (0,2)|(1,2), (2,2)|none.  The pairing makes the address of a lane's tap a per-lane base plus an offset
+// that is the same for both halves of the wave; the tenth, absent tap reads a zero word against a zero weight.
+// A workgroup copies `imgs` whole images to LDS and walks their pooled positions 32 at a time per wave; the four members
+// of a pooling window are four accumulator tiles of the same lane, so the pool is a register-wise max (then bias and
+// ReLU, both monotone: equal to pool(relu(conv + bias)) exactly).  20 MFMAs produce 32 positions x 32 channels.
+__global__ void __launch_bounds__(256, 4) conv_f32_c1k3_pool_mfma_kernel(const float *__restrict__ x, const float *__restrict__ w,
+                                                                     const float *__restrict__ bias, float *__restrict__ y,
+                                                                     int N, int H, int W, int K, int POH, int POW, int imgs,
+                                                                     int relu, FastDiv dpp, FastDiv dpw) {
+    extern __shared__ __attribute__((aligned(16))) float img_lds[];  // [imgs][H][W] then four zero words
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int HW = H * W, PP = POH * POW;
+    const int n0 = blockIdx.x * imgs, imgs_here = min(imgs, N - n0);
+    const int kb = blockIdx.y * 32;
+    const int cnt = imgs_here * HW;
+    const float *src = x + int64_t(n0) * HW;
+    if ((HW & 3) == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+        for (int i = tid; i < (cnt >> 2); i += 256)
+            reinterpret_cast<f32x4 *>(img_lds)[i] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(src) + i);
+    } else {
+        for (int i = tid; i < cnt; i += 256) img_lds[i] = src[i];
+    }
+    const int zero_idx = imgs * HW;
+    if (tid < 4) img_lds[zero_idx + tid] = 0.0f;
+
+    // this lane's A operands: channel kb + l32, tap pair member lh
+    float wa[5];
+    {
+        const int ch = kb + l32;
+        const float *wr = w + int64_t(ch < K ? ch : 0) * 9;
+        const bool okc = ch < K;
+        wa[0] = okc ? wr[0 + lh] : 0.0f;
+        wa[1] = okc ? wr[3 + lh] : 0.0f;
+        wa[2] = okc ? wr[6 + lh] : 0.0f;
+        wa[3] = okc ? wr[lh ? 5 : 2] : 0.0f;
+        wa[4] = (okc && !lh) ? wr[8] : 0.0f;
+    }
+    float bv[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const int k = kb + (v >> 2) * 8 + lh * 4 + (v & 3);
+        bv[v] = (bias != nullptr && k < K) ? bias[k] : 0.0f;
+    }
+    __syncthreads();
+
+    const int total = imgs_here * PP;
+    const bool full_k = kb + 32 <= K;
+    float *ybase = y + (int64_t(n0) * K + kb) * PP;
+    for (int p0 = wave * 32; p0 < total; p0 += 4 * 32) {
+        const int p = p0 + l32;
+        const bool valid = p < total;
+        const unsigned pc_ = valid ? unsigned(p) : 0u;
+        const unsigned img = fastdiv(pc_, dpp), pp = pc_ - img * unsigned(PP);
+        const unsigned pr = fastdiv(pp, dpw), pcol = pp - pr * unsigned(POW);
+        const int wb = int(img) * HW + int(2 * pr) * W + int(2 * pcol);  // window origin in LDS
+        const int a012 = wb + lh, a3 = wb + 2 + lh * W;
+        f32x16 acc[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[j][v] = 0.0f;
+        float b[5][4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int to = (j >> 1) * W + (j & 1);  // window member (dy, dx)
+            b[0][j] = img_lds[a012 + to];
+            b[1][j] = img_lds[a012 + to + W];
+            b[2][j] = img_lds[a012 + to + 2 * W];
+            b[3][j] = img_lds[a3 + to];
+            b[4][j] = img_lds[lh ? zero_idx : wb + to + 2 * W + 2];
+        }
+        // tap pairs outermost: consecutive MFMAs go to different accumulators
+#pragma unroll
+        for (int t = 0; t < 5; ++t)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(wa[t], b[t][j], acc[j], 0, 0, 0);
+        if (valid) {
+            // one uniform base and a 32-bit element offset per lane (the host checks that N * K * PP fits)
+            const unsigned lane_off = (unsigned(img) * unsigned(K) + unsigned(lh * 4)) * unsigned(PP) + pp;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int dk = (v >> 2) * 8 + (v & 3);
+                if (full_k || kb + lh * 4 + dk < K) {
+                    float o = vmax(vmax3(acc[0][v], acc[1][v], acc[2][v]), acc[3][v]) + bv[v];
+                    if (relu) o = vmax(o, 0.0f);
+                    ybase[lane_off + unsigned(dk * PP)] = o;
+                }
+            }
+        }
+    }
+}
+
 typedef TilePlan MfmaPlan;
 
 // Tile shape with the best useful-lane fraction whose LDS footprint allows two workgroups per CU.
@@ -791,6 +901,18 @@ int zant_conv2d_f32_fused_pool(zant_ctx *ctx, const float *x, const int64_t xdim
     }
     if (query_only) return ZANT_OK;
     const int POH = int(OH / 2), POW = int(OW / 2);
+    if (k133 && g.pt == 0 && g.pl == 0 && OH == xdim[2] - 2 && OW == xdim[3] - 2 && int64_t(g.H) * g.W * 4 <= 40 * 1024 &&
+        int64_t(POH) * POW < (1 << 20) && int64_t(g.N) * g.K * POH * POW < (int64_t(1) << 31)) {
+        // the matrix-core first layer: four whole images per workgroup (fewer if they do not fit in 40 KB of LDS); with
+        // its 104 registers four workgroups share a CU, which measured better than eight images and two workgroups
+        const int imgs = int(std::min<int64_t>(4, (40 * 1024) / (int64_t(g.H) * g.W * 4)));
+        const dim3 grid(unsigned(ceil_div64(g.N, imgs)), unsigned(ceil_div64(g.K, 32)));
+        KernelTimer kt(ctx);
+        hipLaunchKernelGGL(conv_f32_c1k3_pool_mfma_kernel, grid, dim3(256), size_t(imgs) * g.H * g.W * 4 + 16, ctx->stream, x, w, bias, y,
+                           g.N, g.H, g.W, g.K, POH, POW, imgs, relu, make_fastdiv(unsigned(POH * POW)), make_fastdiv(unsigned(POW)));
+        ZANT_LAUNCH_CHECK(ctx);
+        return ZANT_OK;
+    }
     const int64_t positions = int64_t(g.N) * POH * POW;
     const unsigned pb = unsigned(std::min<int64_t>(ceil_div64(positions, 256), int64_t(ctx->num_cus) * 16));
     KernelTimer kt(ctx);
