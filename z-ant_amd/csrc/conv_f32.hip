@@ -543,10 +543,11 @@ __device__ __forceinline__ float vmax3(float a, float b, float c) {
 // A workgroup copies `imgs` whole images to LDS and walks their pooled positions 32 at a time per wave; the four members
 // of a pooling window are four accumulator tiles of the same lane, so the pool is a register-wise max (then bias and
 // ReLU, both monotone: equal to pool(relu(conv + bias)) exactly).  20 MFMAs produce 32 positions x 32 channels.
+template <bool RELU, bool FULLK>
 __global__ void __launch_bounds__(256, 4) conv_f32_c1k3_pool_mfma_kernel(const float *__restrict__ x, const float *__restrict__ w,
                                                                      const float *__restrict__ bias, float *__restrict__ y,
                                                                      int N, int H, int W, int K, int POH, int POW, int imgs,
-                                                                     int relu, FastDiv dpp, FastDiv dpw) {
+                                                                     FastDiv dpp, FastDiv dpw) {
     extern __shared__ __attribute__((aligned(16))) float img_lds[];  // [imgs][H][W] then four zero words
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, lh = lane >> 5;
@@ -585,7 +586,6 @@ __global__ void __launch_bounds__(256, 4) conv_f32_c1k3_pool_mfma_kernel(const f
     __syncthreads();
 
     const int total = imgs_here * PP;
-    const bool full_k = kb + 32 <= K;
     float *ybase = y + (int64_t(n0) * K + kb) * PP;
     for (int p0 = wave * 32; p0 < total; p0 += 4 * 32) {
         const int p = p0 + l32;
@@ -616,15 +616,16 @@ __global__ void __launch_bounds__(256, 4) conv_f32_c1k3_pool_mfma_kernel(const f
 #pragma unroll
             for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(wa[t], b[t][j], acc[j], 0, 0, 0);
         if (valid) {
-            // one uniform base and a 32-bit element offset per lane (the host checks that N * K * PP fits)
-            const unsigned lane_off = (unsigned(img) * unsigned(K) + unsigned(lh * 4)) * unsigned(PP) + pp;
+            // a uniform base per output channel and one 32-bit byte offset per lane (the host checks that N * K * PP * 4
+            // fits): the stores then need no address arithmetic in the vector unit
+            const unsigned byte_off = ((unsigned(img) * unsigned(K) + unsigned(lh * 4)) * unsigned(PP) + pp) * 4u;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int dk = (v >> 2) * 8 + (v & 3);
-                if (full_k || kb + lh * 4 + dk < K) {
+                if (FULLK || kb + lh * 4 + dk < K) {
                     float o = vmax(vmax3(acc[0][v], acc[1][v], acc[2][v]), acc[3][v]) + bv[v];
-                    if (relu) o = vmax(o, 0.0f);
-                    ybase[lane_off + unsigned(dk * PP)] = o;
+                    if (RELU) o = vmax(o, 0.0f);
+                    *reinterpret_cast<float *>(reinterpret_cast<char *>(ybase + dk * PP) + byte_off) = o;
                 }
             }
         }
@@ -902,14 +903,21 @@ int zant_conv2d_f32_fused_pool(zant_ctx *ctx, const float *x, const int64_t xdim
     if (query_only) return ZANT_OK;
     const int POH = int(OH / 2), POW = int(OW / 2);
     if (k133 && g.pt == 0 && g.pl == 0 && OH == xdim[2] - 2 && OW == xdim[3] - 2 && int64_t(g.H) * g.W * 4 <= 40 * 1024 &&
-        int64_t(POH) * POW < (1 << 20) && int64_t(g.N) * g.K * POH * POW < (int64_t(1) << 31)) {
+        int64_t(POH) * POW < (1 << 20) && int64_t(g.N) * g.K * POH * POW < (int64_t(1) << 30)) {
         // the matrix-core first layer: four whole images per workgroup (fewer if they do not fit in 40 KB of LDS); with
         // its 104 registers four workgroups share a CU, which measured better than eight images and two workgroups
         const int imgs = int(std::min<int64_t>(4, (40 * 1024) / (int64_t(g.H) * g.W * 4)));
         const dim3 grid(unsigned(ceil_div64(g.N, imgs)), unsigned(ceil_div64(g.K, 32)));
         KernelTimer kt(ctx);
-        hipLaunchKernelGGL(conv_f32_c1k3_pool_mfma_kernel, grid, dim3(256), size_t(imgs) * g.H * g.W * 4 + 16, ctx->stream, x, w, bias, y,
-                           g.N, g.H, g.W, g.K, POH, POW, imgs, relu, make_fastdiv(unsigned(POH * POW)), make_fastdiv(unsigned(POW)));
+        const size_t lds = size_t(imgs) * g.H * g.W * 4 + 16;
+        const FastDiv dpp = make_fastdiv(unsigned(POH * POW)), dpw = make_fastdiv(unsigned(POW));
+        const bool fullk = g.K % 32 == 0;
+#define ZANT_C1K3(R, F)                                                                                                      \
+    hipLaunchKernelGGL((conv_f32_c1k3_pool_mfma_kernel<R, F>), grid, dim3(256), lds, ctx->stream, x, w, bias, y, g.N, g.H, g.W, g.K, \
+                       POH, POW, imgs, dpp, dpw)
+        if (relu) { if (fullk) ZANT_C1K3(true, true); else ZANT_C1K3(true, false); }
+        else { if (fullk) ZANT_C1K3(false, true); else ZANT_C1K3(false, false); }
+#undef ZANT_C1K3
         ZANT_LAUNCH_CHECK(ctx);
         return ZANT_OK;
     }
