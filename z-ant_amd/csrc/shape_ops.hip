@@ -247,8 +247,34 @@ __global__ void __launch_bounds__(kThreads) resize_gather_vec_kernel(const U *__
                 int col[VEC];
 #pragma unroll
                 for (int k = 0; k < VEC; ++k) col[k] = tab_lds[tw_lds + int(cv) * VEC + k];
+                bool wide = false;
+                if constexpr (VEC <= 4) {
+                    // up-sampling: the VEC sources lie within VEC consecutive input elements, so one (unaligned) 16-byte
+                    // load and a register select replace VEC gathers -- a 4-byte gather at an 8-byte lane stride makes
+                    // some thirty cache accesses per wave, a contiguous load four
+                    int lo = col[0], hi = col[0];
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) out[u][k] = row[col[k]];
+                    for (int k = 1; k < VEC; ++k) { lo = min(lo, col[k]); hi = max(hi, col[k]); }
+                    const int row_len = int(g.xdim[g.rank - 1]);
+                    if (hi - lo < VEC && row_len >= VEC) {
+                        wide = true;
+                        const int b0 = min(lo, row_len - VEC);  // keep the window inside the row
+                        UV w;
+                        __builtin_memcpy(&w, row + b0, sizeof(UV));
+#pragma unroll
+                        for (int k = 0; k < VEC; ++k) {
+                            const int sel = col[k] - b0;
+                            U e = w[0];
+#pragma unroll
+                            for (int j = 1; j < VEC; ++j) e = sel == j ? w[j] : e;
+                            out[u][k] = e;
+                        }
+                    }
+                }
+                if (!wide) {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) out[u][k] = row[col[k]];
+                }
             } else {
 #pragma unroll
                 for (int k = 0; k < VEC; ++k) out[u][k] = row[tw[cv * VEC + k]];
