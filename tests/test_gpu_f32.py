@@ -158,6 +158,10 @@ CONV_CASES = [
     (2, 3, 20, 20, 16, 3, 3, [1, 1], [1, 1, 1, 1], [1, 1], "NOTSET"),   # 3 input channels (few-channel kernel)
     (2, 3, 17, 17, 16, 3, 3, [2, 2], [1, 1, 1, 1], [1, 1], "NOTSET"),   # ... stride 2 stem
     (2, 1, 12, 12, 8, 5, 5, [1, 1], None, None, "SAME_UPPER"),        # 1 channel, 5x5 (mnist-8 first layer)
+    (600, 16, 3, 3, 32, 3, 3, [1, 1], None, None, None),              # one output per image: hundreds of images per tile
+    (300, 8, 4, 4, 64, 3, 3, [1, 1], [1, 1, 1, 1], [1, 1], "NOTSET"),   # ... padded, ragged last group, a single chunk per tile
+    (5, 8, 6, 300, 32, 3, 3, [1, 1], [1, 1, 1, 1], [1, 1], "NOTSET"),   # wide rows
+    (20000, 8, 4, 4, 32, 3, 3, [1, 1], [1, 1, 1, 1], [1, 1], "NOTSET"),  # single-chunk tiles, more tiles than workgroup slots
 ]
 
 

@@ -52,15 +52,15 @@ __global__ void pack_weights_f32_kernel(const float *__restrict__ w, float *__re
 __device__ __forceinline__ unsigned lds_addr_of(const void *p) {
     return unsigned(reinterpret_cast<uintptr_t>((lptr_t) const_cast<void *>(p)));
 }
-// Starts a 64-bit LDS read without the compiler's knowledge (it inserts no waits of its own for it) ...
-__device__ __forceinline__ int2 lds_read64_async(unsigned addr) {
-    int2 v;
-    asm volatile("ds_read_b64 %0, %1" : "=v"(v) : "v"(addr));
+// Starts a 32-bit LDS read without the compiler's knowledge (it inserts no waits of its own for it) ...
+__device__ __forceinline__ int lds_read32_async(unsigned addr) {
+    int v;
+    asm volatile("ds_read_b32 %0, %1" : "=v"(v) : "v"(addr));
     return v;
 }
 // ... and this waits for every outstanding LDS operation; the values are in/out operands so that their users stay
 // behind the wait.
-__device__ __forceinline__ void lds_wait_all(int2 &a, int2 &b, int2 &c, int2 &d) {
+__device__ __forceinline__ void lds_wait_all(int &a, int &b, int &c, int &d) {
     asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
 }
 
@@ -70,27 +70,27 @@ __device__ float g_zero_words[4] = {0.f, 0.f, 0.f, 0.f};
 // One (tile, chunk) step of the pipeline: start the asynchronous global->LDS copies of the NEXT step
 // into `dma` and run the matrix cores over THIS step's operands in `cmp`.
 //
-// The three LDS regions are passed as __restrict__ pointers on purpose: `dma`, `cmp` and `ptab` never
+// The three LDS regions are passed as __restrict__ pointers on purpose: `dma`, `cmp` and `ttab` never
 // overlap within a step, and saying so is what lets the compiler leave the copies in flight across
 // the LDS reads of this step instead of draining them (vmcnt(0)) before the first one.
 template <int MT, int WM, int WN, int KV, int TT>
 __device__ __forceinline__ void conv_step(float *__restrict__ dma, const float *__restrict__ cmp,
-                                          const int2 *__restrict__ ptab, const float *__restrict__ x,
+                                          const int *__restrict__ ttab, const float *__restrict__ x,
                                           const float *__restrict__ wp, const ConvGeom &g, const TileGeom &t,
-                                          bool do_issue, int itile, int ichunk, const int (&lds_off)[MT],
+                                          bool do_issue, int n0, int kb, int ichunk, const int (&lds_off)[MT],
                                           f32x16 (&acc)[MT]) {
     constexpr int NT = WM * WN * 64;
     constexpr int K_BLK = WN * 32;
     constexpr int PPI = NT / 4;  // patch positions covered by one staging instruction of the workgroup
     const int T = TT > 0 ? TT : g.KH * g.KW;
     const int w_chunk = T * CC * K_BLK;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction; says so to the compiler (LDS
+                                                                // copy destinations then stay in scalar registers)
     const int wn = wave / WM;
     const int l32 = lane & 31, lh = lane >> 5;
 
     if (do_issue) {
-        int n0, oh0, kb;
-        decode_tile(t, itile, n0, oh0, kb);
         float *xl = dma + w_chunk;
         // weight slab: contiguous 16-byte units, lane-consecutive in LDS
         const float *wsrc = wp + (int64_t(ichunk) * t.n_kblocks + kb) * w_chunk;
@@ -100,37 +100,37 @@ __device__ __forceinline__ void conv_step(float *__restrict__ dma, const float *
             if (u < units)
                 __builtin_amdgcn_global_load_lds((gptr_t)(wsrc + u * 4), (lptr_t)(dma + (u0 + wave * 64) * 4), 16, 0, 0);
         }
-        // input patch: lane -> (position, channel j of a half); zero words for padding
+        // input patch: lane -> (position, channel j of a half); zero words for padding.  The tile's table gives each
+        // position's element offset inside the image group (or -1), so a copy costs an add, a compare and the selects:
+        // whatever is decided here per step is paid in matrix-pipe time.
         const int64_t x_plane = int64_t(g.H) * g.W;
-        const float *xb = x + int64_t(n0) * g.C * x_plane;
-        const int ih0 = oh0 * g.sh - g.pt;
-        const int imgs_here = min(t.NB, g.N - n0);
         const int j = tid & 3;
-        // The patch table lives in LDS.  The compiler drains every outstanding asynchronous copy before an LDS read
+        const float *b0 = x + (int64_t(n0) * g.C + ichunk * CC) * x_plane;  // wave-uniform: channel ichunk*CC of image n0
+        const float *b1 = b0 + 4 * x_plane;
+        const bool c_ok0 = ichunk * CC + j < g.C, c_ok1 = ichunk * CC + 4 + j < g.C;
+        const int jplane = j * int(x_plane);  // NB * C * H * W * 4 < 2^31 is checked on the host
+        // The table lives in LDS.  The compiler drains every outstanding asynchronous copy before an LDS read
         // it issues itself in this loop (one round trip to L2 per iteration, which made staging cost ~18 % of a
-        // step), so the table is read with hand-written ds_read_b64, one iteration ahead of its use.
-        const unsigned ptab_addr = lds_addr_of(ptab);
+        // step), so the table is read with hand-written ds_read_b32, one iteration ahead of its use.
+        const unsigned ttab_addr = lds_addr_of(ttab);
         for (int p0 = 0; p0 < t.P1; p0 += 4 * PPI) {
             // four table entries per round; nothing read this way stays in flight across a loop edge (a register
             // copy there would run before the data has landed)
-            int2 e[4];
+            int e[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u)
-                e[u] = lds_read64_async(ptab_addr + unsigned(min(p0 + u * PPI + (tid >> 2), t.P1 - 1)) * 8u);
+                e[u] = lds_read32_async(ttab_addr + unsigned(min(p0 + u * PPI + (tid >> 2), t.P1 - 1)) * 4u);
             lds_wait_all(e[0], e[1], e[2], e[3]);
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 const int pos = p0 + u * PPI + (tid >> 2);
                 if (pos < t.P1) {
-                    const int ih = ih0 + (e[u].y & 0xffff);
-                    const bool ok = e[u].x >= 0 && ih >= 0 && ih < g.H && (e[u].y >> 16) < imgs_here;
-                    const float *src = xb + (e[u].x + ih0 * g.W) + int64_t(ichunk * CC + j) * x_plane;
-#pragma unroll
-                    for (int half = 0; half < 2; ++half) {
-                        const int c = ichunk * CC + half * 4 + j;
-                        const float *sp = (ok && c < g.C) ? src + half * 4 * x_plane : g_zero_words;
-                        __builtin_amdgcn_global_load_lds((gptr_t)sp, (lptr_t)(xl + (half * t.P1s + p0 + u * PPI + wave * 16) * 4), 4, 0, 0);
-                    }
+                    const bool ok = e[u] >= 0;
+                    const unsigned vo = unsigned(e[u] + jplane);
+                    const float *sp0 = (ok && c_ok0) ? b0 + vo : g_zero_words;
+                    const float *sp1 = (ok && c_ok1) ? b1 + vo : g_zero_words;
+                    __builtin_amdgcn_global_load_lds((gptr_t)sp0, (lptr_t)(xl + (p0 + u * PPI + wave * 16) * 4), 4, 0, 0);
+                    __builtin_amdgcn_global_load_lds((gptr_t)sp1, (lptr_t)(xl + (t.P1s + p0 + u * PPI + wave * 16) * 4), 4, 0, 0);
                 }
             }
         }
@@ -217,10 +217,14 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
     const int w_chunk = T * CC * K_BLK;          // floats per (chunk, kblock) weight slab
     const int buf_floats = w_chunk + CC * t.P1s;  // one staging buffer
     float *buf0 = lds, *buf1 = lds + buf_floats;
-    int2 *ptab = reinterpret_cast<int2 *>(lds + 2 * buf_floats);  // [P1]: {offset in image group, img<<16 | ph}
-    int *sched = reinterpret_cast<int *>(ptab + t.P1s);            // [2]: tile ids handed out by thread 0
+    int *ptab = reinterpret_cast<int *>(lds + 2 * buf_floats);     // [P1s]: img << 24 | patch row << 12 | patch column
+    int *ttab0 = ptab + t.P1s;                                     // [2][P1s]: per tile, a position's element offset in
+    int *ttab1 = ttab0 + t.P1s;                                    //   the image group, -1 where the patch is padding
+    int *sched = ttab1 + t.P1s;                                    // [2]: tile ids handed out by thread 0
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction; says so to the compiler (LDS
+                                                                // copy destinations then stay in scalar registers)
     const int wm = wave % WM, wn = wave / WM;
     const int l32 = lane & 31, lh = lane >> 5;
     const int64_t x_img = int64_t(g.C) * g.H * g.W;
@@ -231,11 +235,7 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
     for (int e = tid; e < t.P1; e += NT) {
         const int img = e / patch_hw, rem = e - img * patch_hw;
         const int ph = rem / t.PW, pw = rem - ph * t.PW;
-        const int iw = pw - g.pl;
-        int2 v;
-        v.x = (iw >= 0 && iw < g.W) ? int(img * x_img) + ph * g.W + iw : -1;  // NB*C*H*W < 2^31 is checked on the host
-        v.y = (img << 16) | ph;
-        ptab[e] = v;
+        ptab[e] = (img << 24) | (ph << 12) | pw;  // NB < 256, PH and PW < 4096: the planner's limits
     }
     // With a fused 2x2/2 max pool the lane's tile registers 4j .. 4j+3 are the four members of ONE pooling window
     // (pooled position (wm*MT/4 + j)*32 + l32), so the pool is a register-wise max in the epilogue.
@@ -264,14 +264,31 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
     if (tid == 0 && blockIdx.x == 0) tile_counters[parity ^ 1] = 2 * int(gridDim.x);
     __syncthreads();
 
+    // A tile's table: which patch positions exist for this tile (rows above / below the image and images past the
+    // batch do not) and where they are.  Built once per tile by the whole workgroup, read by every step's copies.
+    auto fill_ttab = [&](int *tt, int n0, int oh0) {
+        const int ih0 = oh0 * g.sh - g.pt;
+        const int imgs_here = min(t.NB, g.N - n0);
+        for (int e = tid; e < t.P1; e += NT) {
+            const int v = ptab[e];
+            const int img = int(unsigned(v) >> 24), ih = ih0 + ((v >> 12) & 0xfff), iw = (v & 0xfff) - g.pl;
+            const bool ok = iw >= 0 && iw < g.W && ih >= 0 && ih < g.H && img < imgs_here;
+            tt[e] = ok ? img * int(x_img) + ih * g.W + iw : -1;  // NB*C*H*W*4 < 2^31 is checked on the host
+        }
+    };
+
     int cur = blockIdx.x;
     if (cur >= t.n_tiles) return;
     f32x16 acc[MT];
+    // Tiles are decoded once, when their id is known, and the id is made wave-uniform first: decoded per step from the
+    // LDS slot (a vector register) the divisions ran in the vector unit, some sixty instructions per step.
+    int cn0, coh0, ckb, nn0 = 0, noh0 = 0, nkb = 0;
+    decode_tile(t, cur, cn0, coh0, ckb);
+    fill_ttab(ttab0, cn0, coh0);
+    __syncthreads();
     // prologue: copies of the first step, with nothing to compute yet
     {
-        int n0, oh0, kb;
-        decode_tile(t, cur, n0, oh0, kb);
-        const float *wsrc = wp + int64_t(kb) * w_chunk;
+        const float *wsrc = wp + int64_t(ckb) * w_chunk;
         const int units = w_chunk >> 2;
         for (int u0 = 0; u0 < units; u0 += NT) {
             const int u = u0 + tid;
@@ -279,22 +296,17 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
                 __builtin_amdgcn_global_load_lds((gptr_t)(wsrc + u * 4), (lptr_t)(buf0 + (u0 + wave * 64) * 4), 16, 0, 0);
         }
         const int64_t x_plane = int64_t(g.H) * g.W;
-        const float *xb = x + int64_t(n0) * x_img;
-        const int ih0 = oh0 * g.sh - g.pt;
-        const int imgs_here = min(t.NB, g.N - n0);
+        const float *xb = x + int64_t(cn0) * x_img;
         const int j = tid & 3;
         float *xl = buf0 + w_chunk;
         for (int p0 = 0; p0 < t.P1; p0 += NT / 4) {
             const int pos = p0 + (tid >> 2);
             if (pos < t.P1) {
-                const int2 e = ptab[pos];
-                const int ih = ih0 + (e.y & 0xffff);
-                const bool ok = e.x >= 0 && ih >= 0 && ih < g.H && (e.y >> 16) < imgs_here;
-                const float *src = xb + (e.x + ih0 * g.W) + int64_t(j) * x_plane;
+                const int e = ttab0[pos];
 #pragma unroll
                 for (int half = 0; half < 2; ++half) {
                     const int c = half * 4 + j;
-                    const float *sp = (ok && c < g.C) ? src + half * 4 * x_plane : g_zero_words;
+                    const float *sp = (e >= 0 && c < g.C) ? xb + e + int64_t(c) * x_plane : g_zero_words;
                     __builtin_amdgcn_global_load_lds((gptr_t)sp, (lptr_t)(xl + (half * t.P1s + p0 + wave * 16) * 4), 4, 0, 0);
                 }
             }
@@ -312,21 +324,29 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
             __builtin_amdgcn_s_waitcnt(0);  // this thread's copies for this step have landed
             __syncthreads();                // ... everyone's have; all waves are done with the other buffer
             if (chunk == 0) {
-                nxt = sched[tile_par];  // written at least one barrier ago
+                nxt = __builtin_amdgcn_readfirstlane(sched[tile_par]);  // written at least one barrier ago
                 if (tid == 0) sched[tile_par ^ 1] = atomicAdd(tile_counters + parity, 1);
+                if (nxt < t.n_tiles) {
+                    decode_tile(t, nxt, nn0, noh0, nkb);
+                    // no copy is in flight here (the wait above), and the slot's last readers were the copies of the
+                    // previous tile; its first readers come a barrier later unless the tile has a single chunk
+                    fill_ttab(tile_par ? ttab0 : ttab1, nn0, noh0);
+                    if (t.n_chunks == 1) __syncthreads();
+                }
             }
             const bool same_tile = chunk + 1 < t.n_chunks;
             const bool do_issue = same_tile || nxt < t.n_tiles;
-            const int itile = same_tile ? cur : nxt, ichunk = same_tile ? chunk + 1 : 0;
+            const int ichunk = same_tile ? chunk + 1 : 0;
             float *dma = (step & 1) ? buf0 : buf1;
             const float *cmp = (step & 1) ? buf1 : buf0;
-            conv_step<MT, WM, WN, KV, TT>(dma, cmp, ptab, x, wp, g, t, do_issue, itile, ichunk, lds_off, acc);
+            const int *ttab = (same_tile ? tile_par == 0 : tile_par != 0) ? ttab0 : ttab1;  // tile k's table is slot k & 1
+            conv_step<MT, WM, WN, KV, TT>(dma, cmp, ttab, x, wp, g, t, do_issue, same_tile ? cn0 : nn0, same_tile ? ckb : nkb,
+                                          ichunk, lds_off, acc);
         }
 
         // ---- epilogue: bias (+ReLU), coalesced NCHW stores; the next tile's first chunk is in flight ----
         {
-            int n0, oh0, kb;
-            decode_tile(t, cur, n0, oh0, kb);
+            const int n0 = cn0, oh0 = coh0, kb = ckb;
             const int rows_here = min(t.TH, g.OH - oh0);
             const int imgs_here = min(t.NB, g.N - n0);
             const int64_t plane = int64_t(g.OH) * g.OW;
@@ -381,6 +401,7 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
             }
         }
         cur = nxt;
+        cn0 = nn0; coh0 = noh0; ckb = nkb;
         tile_par ^= 1;
     }
 }
@@ -549,7 +570,9 @@ __global__ void __launch_bounds__(256, 4) conv_f32_c1k3_pool_mfma_kernel(const f
                                                                      int N, int H, int W, int K, int POH, int POW, int imgs,
                                                                      FastDiv dpp, FastDiv dpw) {
     extern __shared__ __attribute__((aligned(16))) float img_lds[];  // [imgs][H][W] then four zero words
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction; says so to the compiler (LDS
+                                                                // copy destinations then stay in scalar registers)
     const int l32 = lane & 31, lh = lane >> 5;
     const int HW = H * W, PP = POH * POW;
     const int n0 = blockIdx.x * imgs, imgs_here = min(imgs, N - n0);
@@ -636,14 +659,14 @@ typedef TilePlan MfmaPlan;
 
 // Tile shape with the best useful-lane fraction whose LDS footprint allows two workgroups per CU.
 bool plan_mfma(const ConvGeom &g, MfmaPlan *best, bool pool = false) {
-    if (g.K <= 32) return zant_plan_conv_tiles(g, 4, 1, 8, CC, sizeof(float), 80 * 1024, best, pool);
+    if (g.K <= 32) return zant_plan_conv_tiles(g, 4, 1, 8, CC, sizeof(float), 80 * 1024, best, pool, 0, 32, 0, 2, 4, 256, 4096);
     // 64 output channels per workgroup (2 x 2 waves) stage the input patch once per 64 channels; 32 per workgroup
     // (4 x 1 waves) stage it twice but have twice the position slots, which can fit small feature maps much better
     // (e.g. 5 whole 5x5 pooled images in 128 slots instead of 2 in 64).  Take the narrow shape only for a clear win: at
     // 0.98 against 0.78 useful columns the two measured the same time, and the wide one reads the input once.
     MfmaPlan wide, narrow;
-    const bool ok_w = zant_plan_conv_tiles(g, 2, 2, 8, CC, sizeof(float), 80 * 1024, &wide, pool);
-    const bool ok_n = zant_plan_conv_tiles(g, 4, 1, 8, CC, sizeof(float), 80 * 1024, &narrow, pool);
+    const bool ok_w = zant_plan_conv_tiles(g, 2, 2, 8, CC, sizeof(float), 80 * 1024, &wide, pool, 0, 32, 0, 2, 4, 256, 4096);
+    const bool ok_n = zant_plan_conv_tiles(g, 4, 1, 8, CC, sizeof(float), 80 * 1024, &narrow, pool, 0, 32, 0, 2, 4, 256, 4096);
     if (ok_n && (!ok_w || narrow.eff > wide.eff + 0.25)) { *best = narrow; return true; }
     if (ok_w) { *best = wide; return true; }
     return false;

@@ -54,9 +54,12 @@ __device__ __forceinline__ void decode_tile(const TileGeom &t, int tile, int &n0
 // copying thread and round, and keeps 8 bytes of requantisation table per output channel in LDS; the footprint and the
 // staging estimate then count those padded sizes.
 // n_buffers: staging buffers that must fit (2 = double buffering; more for a deeper copy ring).
+// extra_bytes_per_pos: LDS the kernel keeps per patch position beyond the 8 bytes counted here (may be negative).
+// max_nb, max_patch_dim: limits of the kernel's packed patch table (images per tile; patch rows and columns).
 inline bool zant_plan_conv_tiles(const ConvGeom &g, int WM, int WN, int mt_max, int chunk_channels, size_t elem_bytes,
                                  size_t lds_cap, TilePlan *best, bool pool = false, int target_tiles = 0,
-                                 int mfma_cycles_per_tap = 32, int copy_threads = 0, int n_buffers = 2) {
+                                 int mfma_cycles_per_tap = 32, int copy_threads = 0, int n_buffers = 2,
+                                 int extra_bytes_per_pos = 0, int max_nb = 1 << 15, int max_patch_dim = 1 << 16) {
     const int T = g.KH * g.KW;
     const int K_BLK = WN * 32;
     bool found = false;
@@ -83,7 +86,7 @@ inline bool zant_plan_conv_tiles(const ConvGeom &g, int WM, int WN, int mt_max, 
         t.PW = (g.OW - 1) * g.sw + (g.KW - 1) * g.dw + 1;
         t.P1 = t.NB * t.PH * t.PW;
         t.P1s = copy_threads > 0 ? (t.P1 + copy_threads - 1) / copy_threads * copy_threads : (t.P1 + 3) & ~3;
-        if (t.PH >= (1 << 16) || t.NB >= (1 << 15)) continue;  // packed into one int of the patch table
+        if (t.PH >= max_patch_dim || t.PW >= max_patch_dim || t.NB >= max_nb) continue;  // packed into one int of the patch table
         if (int64_t(t.NB) * g.C * g.H * g.W * int64_t(elem_bytes) >= (int64_t(1) << 31)) continue;  // 32-bit offsets per image group
         t.n_chunks = (g.C + chunk_channels - 1) / chunk_channels;
         t.n_kblocks = (g.K + K_BLK - 1) / K_BLK;
@@ -97,6 +100,7 @@ inline bool zant_plan_conv_tiles(const ConvGeom &g, int WM, int WN, int mt_max, 
             w_slab = (w_slab + round - 1) / round * round;
             fixed = size_t(t.P1s) * 8 + 512 + size_t(t.n_kblocks) * K_BLK * 8;
         }
+        fixed = size_t(int64_t(fixed) + int64_t(extra_bytes_per_pos) * t.P1s);  // the kernel's own per-position tables
         const size_t lds = n_buffers * (w_slab + size_t(32) * t.P1s) + fixed;  // the staging buffers
         if (lds > lds_cap) continue;
         const double eff = double(g.N) * rows * cols / (double(t.n_sblocks) * S);
