@@ -74,7 +74,7 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
     int *c3 = reinterpret_cast<int *>(m3 + CO32 * 32);
     int *ptab = reinterpret_cast<int *>(lds + a.o_ptab);   // [P] image << 20 | patch row << 10 | patch column
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, lh = lane >> 5;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l32 = lane & 31, lh = lane >> 5;
     const unsigned lut1_a = lds_address(lut1), lut2_a = lds_address(lut2);
 
     // ---- once per workgroup: tables and weights into LDS ----

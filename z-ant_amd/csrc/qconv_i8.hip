@@ -227,7 +227,7 @@ __device__ __forceinline__ void qconv_issue(char *__restrict__ dma, const PatchD
     constexpr int K_BLK = WN * 32;
     const int T = TT > 0 ? TT : g.KH * g.KW;
     const int w_chunk = T * QCC * K_BLK;  // bytes
-    const int tid = threadIdx.x, wave = tid >> 6;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     char *xl = dma + w_region_bytes(w_chunk, NT);
     const int8_t *wsrc = wp + (int64_t(ichunk) * t.n_kblocks + d.kb) * w_chunk;
     const int units = w_chunk >> 4;
@@ -297,7 +297,7 @@ __device__ __forceinline__ void qconv_step(char *__restrict__ dma, const char *_
     constexpr int K_BLK = WN * 32;
     const int T = TT > 0 ? TT : g.KH * g.KW;
     const int w_chunk = T * QCC * K_BLK;  // bytes
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wn = wave / WM;
     const int l32 = lane & 31, lh = lane >> 5;
 
@@ -372,7 +372,7 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
     float *mult_l = reinterpret_cast<float *>(ptab + t.P1s);    // [kpad] requantisation multipliers ...
     int *corr_l = reinterpret_cast<int *>(mult_l + kpad);       // [kpad] ... and integer corrections, copied once
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave % WM, wn = wave / WM;
     const int l32 = lane & 31, lh = lane >> 5;
     const int64_t plane_in = int64_t(g.H) * g.W;
@@ -1235,7 +1235,7 @@ qdw3x3_mfma_kernel(const uint4 *__restrict__ x, const uint32_t *__restrict__ wm,
     __syncthreads();
     const unsigned lut_a = lds_address(lut);  // 256-aligned: a converted byte is the low byte of the entry's address
     const int pair = blockIdx.x / blocks_per_pair, blk = blockIdx.x - pair * blocks_per_pair;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, lh = lane >> 5;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(int(threadIdx.x >> 6)), l32 = lane & 31, lh = lane >> 5;
     const int cb = 2 * pair + lh;
     const bool cb_ok = cb < CB;
     i32x4 a[9];
