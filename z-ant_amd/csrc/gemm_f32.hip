@@ -313,7 +313,7 @@ __device__ __forceinline__ void read_group(unsigned stage, int gi, const unsigne
 
 // One pipeline step: start the copies of chunk `ichunk` into `dma`, multiply the chunk at LDS address `cmp_addr`,
 // request the first operands of the chunk at `nxt_addr`.
-template <int MT, int WM, int WN, int AM, int BMODE>
+template <int MT, int WM, int WN, int AM, int BMODE, bool FAST>
 __device__ __forceinline__ void gemm_step(float *__restrict__ dma, unsigned cmp_addr, unsigned nxt_addr,
                                           const unsigned (&offa)[BK / 8], const unsigned (&offb)[BK / 8],
                                           f32x4 (&a)[2][MT], f32x4 (&b)[2],
@@ -326,21 +326,20 @@ __device__ __forceinline__ void gemm_step(float *__restrict__ dma, unsigned cmp_
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     constexpr int PA = stage_instrs<AM, BM>() / NW, PB = stage_instrs<BMODE, BN>() / NW;
     static_assert(PA + PB <= 4 * MT * (BK / 8), "one copy instruction per MFMA at most");
-    // Whole chunk inside K: no masks, addresses are a uniform offset from chunk 0, and the copy instructions are
-    // spread between the MFMAs (each is issued while the previous MFMA of the dependent chain executes).  Otherwise
-    // (the K tail and the zero chunks behind it) the masked copies are issued up front.
-    const bool fast = (ichunk + 1) * BK <= g.K;
+    // FAST: the whole chunk lies inside K: no masks, addresses are a uniform offset from chunk 0, and the copy
+    // instructions are spread between the MFMAs (each is issued while the previous MFMA of the dependent chain
+    // executes).  Otherwise (the K tail and the zero chunks behind it) the masked copies are issued up front.  The
+    // caller runs the fast steps and the others in two loops of their own: with both in one loop body the operand
+    // registers of the two paths were reconciled by eight 64-bit register copies per step, paid in matrix-pipe time.
     const int64_t koffa = AM == RC4 ? int64_t(ichunk) * BK * g.lda : int64_t(ichunk) * BK;
     const int64_t koffb = BMODE == RC4 ? int64_t(ichunk) * BK * g.ldb : int64_t(ichunk) * BK;
-    if (!fast) {
+    if (!FAST) {
         stage_panel<AM, BM, NW>(dma, A, g.lda, m0, g.M, ichunk * BK, g.K, wave, lane);
         stage_panel<BMODE, BN, NW>(dma + BM * BK, B, g.ldb, n0, g.N, ichunk * BK, g.K, wave, lane);
     }
     __builtin_amdgcn_sched_barrier(0);
 
     static_assert((BK / 8) % 2 == 0, "group 0 of every chunk uses operand registers 0");
-    auto multiply = [&](auto fast_c) {
-    constexpr bool FAST = decltype(fast_c)::value;
     int q = 0;  // MFMAs issued so far in this step (a constant after unrolling)
 #pragma unroll
     for (int gi = 0; gi < BK / 8; ++gi) {
@@ -367,9 +366,6 @@ __device__ __forceinline__ void gemm_step(float *__restrict__ dma, unsigned cmp_
     // The look-ahead reads were issued a whole burst ago; make sure they have landed before the step ends: a value
     // still in flight across the loop edge would be at the mercy of any register copy the compiler puts there.
     lds_wait<0, MT>(a[0], b[0]);
-    };
-    if (fast) multiply(std::true_type{});
-    else multiply(std::false_type{});
 }
 
 // s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt in bits 3:0 and 15:14).
@@ -428,17 +424,29 @@ gemm_f32_dma_kernel(const float *__restrict__ A, const float *__restrict__ B, co
     f32x4 ra[2][MT], rb[2];
     read_group<MT, AM, BMODE, BM, BN>(lds0, 0, offa, offb, ra[0], rb[0]);
     int cbuf = 0, dbuf = S - 1;
-    for (int c = 0; c < n_chunks; ++c) {
-        // After this barrier: chunk c+1 is complete for everyone (each wave waited for its own copies of it), and
-        // everyone is done with chunk c-1, whose stage is refilled now.  A bare s_barrier: __syncthreads() carries a
-        // fence that drains ALL outstanding copies, which would serialise the ring.  The step multiplies chunk c,
-        // whose first operands were fetched at the end of the previous step, and ends by fetching those of chunk c+1.
+    // After the barrier of a step: chunk c+1 is complete for everyone (each wave waited for its own copies of it), and
+    // everyone is done with chunk c-1, whose stage is refilled now.  A bare s_barrier: __syncthreads() carries a
+    // fence that drains ALL outstanding copies, which would serialise the ring.  The step multiplies chunk c,
+    // whose first operands were fetched at the end of the previous step, and ends by fetching those of chunk c+1.
+    const int n_fast = max(0, min(n_chunks, g.K / BK - (S - 1)));  // steps whose refill chunk c + S - 1 lies inside K
+    int c = 0;
+    for (; c < n_fast; ++c) {
         __builtin_amdgcn_s_waitcnt(vmcnt_imm(P * (S - 3)));
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
         const int nbuf = cbuf + 1 == S ? 0 : cbuf + 1;
-        gemm_step<MT, WM, WN, AM, BMODE>(lds + dbuf * STAGE, lds0 + cbuf * (STAGE * 4), lds0 + nbuf * (STAGE * 4), offa, offb,
-                                         ra, rb, A, B, g, pa, pb, m0, n0, c + S - 1, acc);
+        gemm_step<MT, WM, WN, AM, BMODE, true>(lds + dbuf * STAGE, lds0 + cbuf * (STAGE * 4), lds0 + nbuf * (STAGE * 4), offa,
+                                               offb, ra, rb, A, B, g, pa, pb, m0, n0, c + S - 1, acc);
+        cbuf = nbuf;
+        dbuf = dbuf + 1 == S ? 0 : dbuf + 1;
+    }
+    for (; c < n_chunks; ++c) {
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(P * (S - 3)));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        const int nbuf = cbuf + 1 == S ? 0 : cbuf + 1;
+        gemm_step<MT, WM, WN, AM, BMODE, false>(lds + dbuf * STAGE, lds0 + cbuf * (STAGE * 4), lds0 + nbuf * (STAGE * 4), offa,
+                                                offb, ra, rb, A, B, g, pa, pb, m0, n0, c + S - 1, acc);
         cbuf = nbuf;
         dbuf = dbuf + 1 == S ? 0 : dbuf + 1;
     }
