@@ -162,6 +162,7 @@ CONV_CASES = [
     (300, 8, 4, 4, 64, 3, 3, [1, 1], [1, 1, 1, 1], [1, 1], "NOTSET"),   # ... padded, ragged last group, a single chunk per tile
     (5, 8, 6, 300, 32, 3, 3, [1, 1], [1, 1, 1, 1], [1, 1], "NOTSET"),   # wide rows
     (20000, 8, 4, 4, 32, 3, 3, [1, 1], [1, 1, 1, 1], [1, 1], "NOTSET"),  # single-chunk tiles, more tiles than workgroup slots
+    (1, 8, 3, 4200, 32, 3, 3, [1, 1], [1, 1, 1, 1], [1, 1], "NOTSET"),   # rows wider than the tiled kernel's patch table takes
 ]
 
 
