@@ -123,6 +123,22 @@ int zant_hip_conv2d_out_shape(const int64_t xdim[4], const int64_t wdim[4], cons
                               const int64_t *pads, int n_pads, const int64_t *dil, int n_dil, int64_t group,
                               const char *auto_pad, int64_t ydim[4]);
 
+/* zant_hip_conv2d_f32 for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, checks
+ * and results; the tiled kernel's scratch (packed weights and two tile counters, which zant_hip_conv2d_f32
+ * keeps in a context workspace it grows with hipMalloc) lives in a static device array of
+ * ZANT_HIP_STATIC_SCRATCH_BYTES that every device the library runs on holds until the process ends.  The call
+ * performs no hipMalloc / hipFree.  A convolution whose packed weights (K and C rounded up to the tile, x KH x KW
+ * x 4 bytes, + 256) exceed the array returns ZANT_ArenaOverflow and launches nothing; zant_hip_last_error()
+ * gives both sizes.  Every call on a device shares that device's array: calls on one stream may follow each
+ * other freely (each re-packs the weights and re-arms the counters in stream order), calls that overlap on one
+ * device (several contexts or streams) race. */
+#define ZANT_HIP_STATIC_SCRATCH_BYTES (8u << 20)
+int zant_hip_conv2d_f32_static(zant_ctx *ctx, const float *x, const int64_t xdim[4], const float *w,
+                               const int64_t wdim[4], const float *bias, float *y, const int64_t ydim[4],
+                               const int64_t *stride, int n_stride, const int64_t *pads, int n_pads,
+                               const int64_t *dil, int n_dil, int64_t group, const char *auto_pad, int fuse_act);
+
 /* mat_mul_lean = lean_mat_mul (op_mat_mul.zig:92-172): last two dims only. */
 int zant_hip_matmul_f32(zant_ctx *ctx, const float *a, const int64_t *adim, int a_rank, const float *b,
                         const int64_t *bdim, int b_rank, float *y);

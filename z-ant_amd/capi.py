@@ -45,6 +45,8 @@ PROTOTYPES = {
     "zant_hip_kernel_ms": (i32, [vp, C.POINTER(f32)]),
     "zant_hip_conv2d_f32": (i32, [vp, vp, c_i64p, vp, c_i64p, vp, vp, c_i64p, c_i64p, i32, c_i64p, i32, c_i64p, i32,
                                   i64, C.c_char_p, i32]),
+    "zant_hip_conv2d_f32_static": (i32, [vp, vp, c_i64p, vp, c_i64p, vp, vp, c_i64p, c_i64p, i32, c_i64p, i32, c_i64p,
+                                         i32, i64, C.c_char_p, i32]),
     "zant_hip_conv2d_out_shape": (i32, [c_i64p, c_i64p, c_i64p, i32, c_i64p, i32, c_i64p, i32, i64, C.c_char_p, c_i64p]),
     "zant_hip_matmul_f32": (i32, [vp, vp, c_i64p, i32, vp, c_i64p, i32, vp]),
     "zant_hip_matmul_check": (i32, [c_i64p, i32, c_i64p, i32]),

@@ -65,6 +65,7 @@ struct zant_pack_slot {
     size_t bytes = 0;
     bool ready = false;   // the packed contents are valid
     unsigned runs = 0;    // launches so far; its parity selects the tile counter of a launch
+    bool fixed = false;   // `dev` is memory the slot does not own and must not grow: a request beyond `bytes` fails
 };
 void zant_pack_slot_free(zant_ctx *ctx, zant_pack_slot *slot);
 // Hands out `static_bytes` of weight-derived scratch (the slot's own allocation, or the front of the context
@@ -112,6 +113,11 @@ int zant_conv2d_f32_fused_pool(zant_ctx *ctx, const float *x, const int64_t xdim
                                const float *bias, float *y, const int64_t ydim[4], const int64_t *stride, int n_stride,
                                const int64_t *pads, int n_pads, const int64_t *dil, int n_dil, int64_t group,
                                const char *auto_pad, int relu, bool query_only, zant_pack_slot *slot = nullptr);
+
+// Resolves, once per device, the device address of the static scratch array behind zant_hip_conv2d_f32_static
+// (conv_f32.hip).  Called by zant_hip_ctx_create with the context's device current; a failure is remembered and
+// reported by the entry point.
+void zant_conv_static_scratch_init(int device);
 
 // zant_hip_conv2d_f32 with a pack slot (see above).
 int zant_conv2d_f32_slot(zant_ctx *ctx, const float *x, const int64_t xdim[4], const float *w, const int64_t wdim[4],

@@ -12,6 +12,7 @@
 // register holds 32 consecutive NCHW positions and stores are 128-byte coalesced.
 // A direct kernel (one thread per output element) covers shapes the tiled kernel does not take.
 #include <algorithm>
+#include <mutex>
 
 #include "conv_tile.h"
 
@@ -833,6 +834,58 @@ extern "C" int zant_hip_conv2d_f32(zant_ctx *ctx, const float *x, const int64_t 
                                    const int64_t *dil, int n_dil, int64_t group, const char *auto_pad, int fuse_act) {
     return zant_conv2d_f32_slot(ctx, x, xdim, w, wdim, bias, y, ydim, stride, n_stride, pads, n_pads, dil, n_dil, group, auto_pad,
                                 fuse_act, nullptr);
+}
+
+// ---- zant_hip_conv2d_f32_static: the same convolution for callers that cannot allocate ---------------------------
+//
+// The tiled kernel's scratch (two tile counters and the packed weights) lives in a static device array instead of
+// the context workspace.  `scratch` below is only the host-side handle of that array: every device holds its own
+// copy at its own address, which hipGetSymbolAddress returns and which is what kernels, copies and fills must be
+// given.  The array is shared by every call on a device and keeps the previous call's contents; each call re-packs
+// the weights and re-arms the counters before its convolution kernel, in stream order, so calls on ONE stream are
+// safe back to back, while calls that overlap on one device (two contexts, two streams) race.
+static __device__ __align__(256) unsigned char scratch[ZANT_HIP_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices];        // device address of `scratch` per device, nullptr until resolved
+hipError_t g_scratch_err[kMaxDevices];   // what hipGetSymbolAddress returned on that device
+bool g_scratch_tried[kMaxDevices];
+}  // namespace
+
+void zant_conv_static_scratch_init(int device) {
+    if (device < 0 || device >= kMaxDevices) return;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_tried[device]) return;
+    g_scratch_tried[device] = true;
+    void *ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));  // `device` is current (see the caller)
+    g_scratch_err[device] = e;
+    g_scratch_ptr[device] = e == hipSuccess ? ptr : nullptr;
+}
+
+extern "C" int zant_hip_conv2d_f32_static(zant_ctx *ctx, const float *x, const int64_t xdim[4], const float *w,
+                                          const int64_t wdim[4], const float *bias, float *y, const int64_t ydim[4],
+                                          const int64_t *stride, int n_stride, const int64_t *pads, int n_pads,
+                                          const int64_t *dil, int n_dil, int64_t group, const char *auto_pad,
+                                          int fuse_act) {
+    if (!ctx) return ZANT_NullPointer;
+    if (ctx->device < 0 || ctx->device >= kMaxDevices) return ZANT_InvalidInput;
+    void *ptr;
+    hipError_t e;
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        ptr = g_scratch_ptr[ctx->device];
+        e = g_scratch_err[ctx->device];
+    }
+    if (!ptr) return zant_fail_hip(ctx, e == hipSuccess ? hipErrorNotInitialized : e, "hipGetSymbolAddress(scratch)");
+    zant_pack_slot slot;
+    slot.dev = ptr;
+    slot.bytes = ZANT_HIP_STATIC_SCRATCH_BYTES;
+    slot.fixed = true;
+    return zant_conv2d_f32_slot(ctx, x, xdim, w, wdim, bias, y, ydim, stride, n_stride, pads, n_pads, dil, n_dil, group,
+                                auto_pad, fuse_act, &slot);
 }
 
 int zant_conv2d_f32_slot(zant_ctx *ctx, const float *x, const int64_t xdim[4], const float *w, const int64_t wdim[4],

@@ -39,7 +39,7 @@ int zant_workspace(zant_ctx *ctx, size_t bytes, void **out) {
 }
 
 void zant_pack_slot_free(zant_ctx *ctx, zant_pack_slot *slot) {
-    if (!slot || !slot->dev) return;
+    if (!slot || !slot->dev || slot->fixed) return;
     if (ctx && ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     (void)hipFree(slot->dev);
     slot->dev = nullptr; slot->bytes = 0; slot->ready = false; slot->runs = 0;
@@ -55,6 +55,21 @@ int zant_pack_region(zant_ctx *ctx, zant_pack_slot *slot, size_t static_bytes, s
         *stat = ws;
         *dyn = static_cast<char *>(ws) + sa;
         *need_pack = true;
+        *parity = 0;
+        return ZANT_OK;
+    }
+    if (slot->fixed) {
+        // borrowed memory of a fixed size: nothing is allocated, larger requests are refused
+        if (!slot->dev) return ZANT_NullPointer;
+        if (sa > slot->bytes || dyn_bytes) {
+            ctx->last_error = "static scratch too small: " + std::to_string(sa + dyn_bytes) + " bytes needed, " +
+                              std::to_string(slot->bytes) + " available";
+            zant_log(ctx->last_error.c_str());
+            return ZANT_ArenaOverflow;
+        }
+        *stat = slot->dev;
+        *dyn = nullptr;
+        *need_pack = true;  // the array is shared by every call on the device and the weights may have changed
         *parity = 0;
         return ZANT_OK;
     }
@@ -91,6 +106,7 @@ extern "C" int zant_hip_ctx_create(zant_ctx **out, int device, void *stream) {
         if (e != hipSuccess) { delete ctx; return create_failed(e, "hipStreamCreate"); }
         ctx->owns_stream = true;
     }
+    zant_conv_static_scratch_init(device);
     hipDeviceProp_t prop;
     if (hipGetDeviceProperties(&prop, device) == hipSuccess) ctx->num_cus = prop.multiProcessorCount;
     hipEvent_t *evs[4] = {&ctx->ev_start, &ctx->ev_stop, &ctx->ev_k0, &ctx->ev_k1};

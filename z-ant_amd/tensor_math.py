@@ -71,6 +71,18 @@ def conv_lean(x, w, y, bias, stride, pads=None, dilations=None, group=None, auto
     return y
 
 
+def conv_lean_static(x, w, y, bias, stride, pads=None, dilations=None, group=None, auto_pad=None, fuse_act=None):
+    """conv_lean through the entry point that allocates nothing (scratch in a static device array)."""
+    if x.dim() != 4 or w.dim() != 4:
+        raise ZantError(-1)
+    ctx = context()
+    xd, _ = dims(x.shape); wd, _ = dims(w.shape); yd, _ = dims(y.shape)
+    s, ns = dims(stride); p, npd = dims(pads); d, nd = dims(dilations)
+    ctx.check(lib.zant_hip_conv2d_f32_static(ctx.handle, _p(x), xd, _p(w), wd, _p(bias), _p(y), yd, s, ns, p, npd, d,
+                                             nd, _grp(group), _enc(auto_pad), ACT[fuse_act]))
+    return y
+
+
 def Conv(x, w, bias, stride, pads=None, dilations=None, group=None, auto_pad=None):
     """OnnxConv (op_convolution.zig:647): allocate the expected shape (zero filled), then conv_lean."""
     if x.dim() != 4 or w.dim() != 4:
