@@ -1,0 +1,83 @@
+"""Bit-exact parity of the patch-stationary int8 convolution kernel (3x3, stride 1, at least 32 input and 33 output
+channels) with the CPU oracle: every path of its tiling and of its epilogues."""
+import numpy as np
+import pytest
+
+from oracle import oracle as zo
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def G():
+    import gpu_util
+    return gpu_util
+
+
+def _operands(seed, N, C, H, W, K):
+    g = np.random.default_rng(seed)
+    x = g.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+    w = g.integers(-127, 128, (K, C, 3, 3), dtype=np.int8)
+    ws = (g.uniform(0.5, 1.5, K) * 0.08 / np.sqrt(9 * C)).astype(np.float32)
+    b = g.integers(-1000, 1001, K, dtype=np.int32)
+    return x, w, ws, b
+
+
+PS_CASES = [
+    # N, C, H, W, K, pads                    what the shape exercises
+    (3, 64, 12, 12, 96, [1, 1, 1, 1]),       # several whole images per tile; 96 channels in a pass of 128
+    (2, 32, 9, 13, 40, [0, 1, 0, 1]),        # one channel chunk, a pass of 64 channels, asymmetric padding
+    (1, 160, 6, 6, 256, [1, 1, 1, 1]),       # two output-channel passes, five channel chunks
+    (5, 48, 30, 30, 64, [1, 1, 1, 1]),       # odd number of 16-channel blocks, row tiles with a short last tile
+    (2, 128, 28, 28, 128, [0, 0, 0, 0]),     # no padding
+    (7, 40, 5, 5, 72, [1, 1, 1, 1]),         # channels not a multiple of 16, images not a multiple of the tile
+    (2, 256, 7, 9, 200, [1, 0, 1, 0]),       # eight chunks, ragged output channels
+]
+
+
+@pytest.mark.parametrize("case", PS_CASES, ids=[str(i) for i in range(len(PS_CASES))])
+@pytest.mark.parametrize("act", [None, "leaky"])
+def test_patch_stationary_shapes_bit_exact(G, case, act):
+    N, C, H, W, K, pads = case
+    x, w, ws, b = _operands(11 * N + C + K, N, C, H, W, K)
+    kw = dict(act=act, act_alpha=0.1, act_scale=0.04, act_zp=30) if act else {}
+    ref = zo.qlinearconv(x, 0.02, 128, w, ws, None, 0.05, 128, b, [1, 1], pads, [1, 1], 1, **kw)
+    y = G.tm.qlinearconv(G.dev(x), 0.02, 128, G.dev(w), G.dev(ws), None, 0.05, 128, G.dev(b), [1, 1], pads, [1, 1], 1, **kw)
+    np.testing.assert_array_equal(G.host(y), ref)
+    assert len(np.unique(ref)) > 8
+
+
+@pytest.mark.parametrize("C", [32, 64])
+def test_more_tiles_than_compute_units(G, C):
+    """Every workgroup walks several tiles: with one channel chunk the next tile's patch goes in at once, with two it
+    streams in during the last step of the current tile."""
+    N, H, K = 1100, 14, 64
+    x, w, ws, b = _operands(C, N, C, H, H, K)
+    ref = zo.qlinearconv(x, 0.02, 128, w, ws, None, 0.05, 128, b, [1, 1], [1, 1, 1, 1], [1, 1], 1)
+    y = G.host(G.tm.qlinearconv(G.dev(x), 0.02, 128, G.dev(w), G.dev(ws), None, 0.05, 128, G.dev(b), [1, 1], [1, 1, 1, 1], [1, 1], 1))
+    np.testing.assert_array_equal(y, ref)
+
+
+def test_blocked_in_and_out_inside_a_model(G):
+    """Three convolutions in a row: the middle one reads and writes the channel-blocked layout (once without and once
+    with a fused activation), the first reads NCHW, the last writes it."""
+    from zant_amd.model import Model, U8
+    N, C, H = 6, 64, 20
+    g = np.random.default_rng(5)
+    x = g.integers(0, 256, (N, C, H, H), dtype=np.uint8)
+    layers = [_operands(100 + i, 1, C, 4, 4, C)[1:] for i in range(3)]
+    for act in (None, "relu6"):
+        m = Model(G.tm.context())
+        t = m.input((N, C, H, H), U8, 0.02, 128)
+        ref, s, z = x, 0.02, 128
+        for i, (w, ws, b) in enumerate(layers):
+            t = m.qlinearconv(t, w, ws, b, 0.05, 120 + i, [1, 1], [1, 1, 1, 1])
+            ref = zo.qlinearconv(ref, s, z, w, ws, None, 0.05, 120 + i, b, [1, 1], [1, 1, 1, 1], [1, 1], 1)
+            s, z = 0.05, 120 + i
+            if act and i == 1:
+                t = m.qlinear_act(t, act, 0.0, 0.03, 10)
+                ref = zo.qlinear_act(ref, s, z, act, 0.0, 0.03, 10)
+                s, z = 0.03, 10
+        m.finalize()
+        y = m.predict_host(x)
+        np.testing.assert_array_equal(y, ref)

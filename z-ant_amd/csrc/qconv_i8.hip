@@ -20,15 +20,6 @@
 
 namespace {
 
-struct QConvArgs {
-    float x_scale, y_scale;
-    int x_zp;
-    uint8_t y_zp;
-    int n_wscale;       // 1 or K
-    int has_act;
-    QAct act;
-};
-
 // Requantises one accumulator of output channel k.
 __device__ __forceinline__ uint8_t requant(int acc, float m, const QConvArgs &q) {
     uint8_t r = sat_u8_rne(float(acc) * m, q.y_zp);
@@ -641,6 +632,11 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
                    const ConvGeom &g, const QConvArgs &q, bool x_blocked, bool y_blocked, zant_pack_slot *slot, bool pool = false,
                    bool plan_only = false) {
     if (g.groups != 1 || g.C < 5 || int64_t(g.N) * g.OH * g.OW < 64) return 1;
+    if (!pool) {
+        // 3x3 / stride 1 layers with at least 32 channels on both sides: the patch-stationary kernel
+        const int rc = zant_qconv_ps(ctx, x, w, w_scale, bias, y, g, q, x_blocked, y_blocked, slot, plan_only);
+        if (rc <= 0) return rc;
+    }
     // a fused 2x2/2 max pool needs whole windows and an activation that keeps the order of its inputs
     if (pool && (g.OH < 2 || g.OW < 2 || (q.has_act && !(q.act.alpha >= 0.0f && q.act.in_scale > 0.0f && q.act.out_scale > 0.0f))))
         return 1;

@@ -1,0 +1,671 @@
+// QLinearConv 3x3 / stride 1 on the int8 matrix cores, patch-stationary form.
+//
+// One workgroup of eight wavefronts (two per SIMD) owns a tile of NB whole images x TH output rows x all columns and
+// ALL output channels.  The tile's input patch (with its halo) is brought to LDS once, for every input channel, and
+// stays there; only the weights stream through LDS, one slab of 32 input channels x 9 taps x up to 128 output channels
+// per step, through a two-slab ring that the copies of step s + 1 fill while the matrix cores work on step s.
+// Compared with staging patch chunk and weight slab per (tile, chunk, output-channel block) step this moves each
+// activation into LDS once instead of once per output-channel block, needs one barrier per 9 taps x 32 channels, and
+// lets the tile be chosen to fill the GPU exactly ("128 x 128 x 28 x 28, 128 filters": half an image per workgroup =
+// 256 tiles on 256 CUs).
+//
+// Wave w computes two 32-channel blocks (pair w mod pairs, pairs = output channels per pass / 64) for the position
+// tiles of group w div pairs; the tile's position tiles of 32 are dealt evenly to the groups.  One activation operand
+// feeds two MFMAs, which keeps the LDS read traffic per MFMA low.  Copies go through registers (an ordinary load, an
+// LDS write two taps later), two units per thread and tap, in the shadow of the MFMAs; the two waves of a SIMD cover
+// each other's waits.
+// Arithmetic, operand layout (channel-blocked signed activations, [tap][half][channel][16] weights), zero-point folding
+// and the requantisation epilogue are those of qconv_mfma_kernel (qconv_i8.hip).
+#include <algorithm>
+
+#include "quant_common.h"
+#include "quant_layout.h"
+
+namespace {
+
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(1))) const void *gptr_t;
+typedef __attribute__((address_space(3))) void *lptr_t;
+
+constexpr int PS_WAVES = 8;           // wavefronts per workgroup: two per SIMD
+constexpr int PS_NT = PS_WAVES * 64;  // threads per workgroup
+constexpr int PS_RMAX = 2;            // 16-byte units per thread of one 16-channel block of the patch: P1s / PS_NT
+constexpr int PS_MTMAX = 4;           // position tiles per wave (x 2 channel blocks x 16 accumulator registers)
+constexpr int PS_RING = 36 * 1024;    // bytes of one slab of the weight ring: 9 taps x 4 KB
+
+struct PsGeom {
+    int N, H, W, CB;            // input: images, rows, columns, 16-channel blocks
+    int K, KB, OH, OW, pt, pl;  // output channels and 16-channel blocks, output rows / columns, top / left padding
+    int NB, TH;                 // images and output rows per tile
+    int PH, PW, P1, P1s;        // patch rows / columns / positions; positions rounded up to a multiple of PS_NT
+    int n_row_tiles, n_tiles;
+    int NC;                     // chunks of 32 input channels
+    int NKP, KP;                // output-channel passes and channels per pass (64 or 128)
+    int npt;                    // position tiles of 32 per tile
+    int kpad;                   // NKP * KP
+    int tab_rounds;             // copy rounds of the multiplier and correction tables: ceil(kpad / 2 / PS_NT)
+};
+
+__device__ __forceinline__ unsigned ps_lds_addr(const void *p) {
+    return unsigned(reinterpret_cast<uintptr_t>((lptr_t) const_cast<void *>(p)));
+}
+// LDS reads the compiler does not see, so that it inserts no waits of its own for them.  The waits take the values as
+// in/out operands so their users stay behind them.
+__device__ __forceinline__ uint32_t ps_read_u8(unsigned addr) {
+    uint32_t v;
+    asm volatile("ds_read_u8 %0, %1" : "=v"(v) : "v"(addr));
+    return v;
+}
+__device__ __forceinline__ uint32_t ps_read_b32(unsigned addr) {
+    uint32_t v;
+    asm volatile("ds_read_b32 %0, %1" : "=v"(v) : "v"(addr));
+    return v;
+}
+__device__ __forceinline__ void ps_wait16(uint32_t (&v)[16]) {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]), "+v"(v[8]),
+                   "+v"(v[9]), "+v"(v[10]), "+v"(v[11]), "+v"(v[12]), "+v"(v[13]), "+v"(v[14]), "+v"(v[15]));
+}
+// One 128-bit LDS read at an immediate byte offset from a per-lane address.  ps_operand_ready waits until at most
+// `pending` younger LDS operations are outstanding (they complete in order; operations of other kinds that share the
+// counter only make the wait stricter) and makes the operand visible to its users only behind that wait.
+__device__ __forceinline__ void ps_ds_read128(i32x4 &v, unsigned addr, int imm) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "i"(imm));
+}
+__device__ __forceinline__ void ps_operand_ready(i32x4 &b, int pending) {
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(b) : "i"(pending));
+}
+__device__ __forceinline__ void ps_operands_ready(i32x4 &a0, i32x4 &a1, i32x4 &b, int pending) {
+    asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(a0), "+v"(a1), "+v"(b) : "i"(pending));
+}
+
+// Where this thread's patch units of a tile come from: offset (in 16-byte units) of the unit's position in channel
+// block 0 of the blocked input, per round, and which rounds read real data (the others hold the padding vector).
+struct PsDesc {
+    unsigned off[PS_RMAX];
+    unsigned ok;
+};
+
+__device__ __forceinline__ void ps_describe(PsDesc &d, const PsGeom &p, int tile) {
+    const int ig = tile / p.n_row_tiles;
+    const int n0 = ig * p.NB, oh0 = (tile - ig * p.n_row_tiles) * p.TH;
+    const int patch_hw = p.PH * p.PW;
+    const float inv_patch = 1.0f / float(patch_hw), inv_pw = 1.0f / float(p.PW);
+    d.ok = 0;
+#pragma unroll
+    for (int r = 0; r < PS_RMAX; ++r) {
+        d.off[r] = 0;
+        if (r * PS_NT < p.P1s) {
+            const int e = r * PS_NT + int(threadIdx.x);
+            const int img = small_div(e, patch_hw, inv_patch), rem = e - img * patch_hw;
+            const int ph = small_div(rem, p.PW, inv_pw), pw = rem - ph * p.PW;
+            const int ih = oh0 - p.pt + ph, iw = pw - p.pl, n = n0 + img;
+            const bool ok = e < p.P1 && n < p.N && ih >= 0 && ih < p.H && iw >= 0 && iw < p.W;
+            d.off[r] = ok ? unsigned((n * p.CB * p.H + ih) * p.W + iw) : 0u;
+            d.ok |= ok ? 1u << r : 0u;
+        }
+    }
+}
+
+// One 16-byte unit of the patch: round r, half h of channel chunk c of the tile `d` describes.  Units outside the
+// image, past the patch or of a channel block the tensor does not have hold the padding vector.  Loaded into registers
+// and written to LDS later (ps_patch_store): an ordinary load issues in a few cycles, where a direct global->LDS copy
+// holds the issuing wave for a couple of hundred.
+__device__ __forceinline__ u32x4 ps_patch_load(const PsDesc &d, const int8_t *__restrict__ xb, const int8_t *__restrict__ padvec,
+                                               const PsGeom &p, int c, int r, int h) {
+    const int cb = 2 * c + h;
+    const bool ok = ((d.ok >> r) & 1u) && cb < p.CB;
+    const int8_t *src = ok ? xb + (size_t(d.off[r]) + size_t(cb) * unsigned(p.H * p.W)) * 16 : padvec;
+    return *reinterpret_cast<const u32x4 *>(src);
+}
+__device__ __forceinline__ void ps_patch_store(char *patch, const PsGeom &p, int c, int r, int h, const u32x4 &v) {
+    *reinterpret_cast<u32x4 *>(patch + ((2 * c + h) * p.P1s + r * PS_NT + int(threadIdx.x)) * 16) = v;
+}
+
+// What a thread copies while its wave multiplies: up to 4 units of a patch chunk (of this tile, or chunk 0 of the next)
+// and its share of the NEXT step's weight slab: unit wunit of the taps wtap0, wtap0 + wtaps, ...
+struct PsStream {
+    const int8_t *wsrc;      // this thread's unit in tap 0 of the next step's slab (taps tap_bytes apart)
+    char *wdst;              // the same place in the ring slab the next step reads (taps 4 KB apart)
+    int tap_bytes;
+    int wtap0, wtaps;        // first tap this thread copies, and the stride of its taps
+    int pcur;                // the step copies a patch chunk
+    char *patch;             // patch base
+    int pchunk;              // channel chunk this step's patch copies fill
+};
+
+constexpr int PS_PCMAX = 2 * PS_RMAX;  // patch units per thread and chunk
+constexpr int PS_WUMAX = 5;            // weight units per thread and step: ceil(9 taps / 2 thread groups)
+
+// The matrix-core work of one step: 9 taps x 32 input channels for this wave's MT position tiles x 2 channel blocks.
+// wr: LDS address of this lane's weight operand of tap 0 of the wave's first channel block (the second block 512 bytes
+// on, taps 4 KB apart); xbase[i] + chunk_off: LDS address of position slot i's patch entry for tap (0, 0) in this step's
+// channel chunk and this lane's half; PW16: bytes of a patch row.
+// The activation operand of slot i for the NEXT tap is read into the same registers right behind slot i's two MFMAs of
+// this tap: a rolling pipeline one tap deep in which every read has 2 * MT MFMAs to land and each MFMA pair waits only
+// for its own operand.  Filter columns are immediate offsets, filter rows an address increment.
+// The copies of PsStream ride along: two units loaded behind the first MFMA pair of each of taps 0..4 and written to
+// LDS two taps later.
+// FIRST: the step opens a pass: its first tap starts the accumulators from zero (an inline constant of the MFMA).
+template <int MT, bool FIRST>
+__device__ __forceinline__ void ps_mfma_step(unsigned wr, const unsigned (&xbase)[MT], unsigned chunk_off, unsigned PW16, const PsStream &st,
+                                             const PsDesc &d, const int8_t *__restrict__ xb, const int8_t *__restrict__ padvec,
+                                             const PsGeom &p, i32x16 (&acc)[2][MT]) {
+    i32x4 a[2][2], b[MT];  // a[buffer][channel block]
+    u32x4 stg[3][2];       // units on their way from global memory to LDS, by tap modulo 3
+    unsigned xr[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) xr[i] = xbase[i] + chunk_off;
+    ps_ds_read128(a[0][0], wr, 0);
+    ps_ds_read128(a[0][1], wr, 512);
+#pragma unroll
+    for (int i = 0; i < MT; ++i) ps_ds_read128(b[i], xr[i], 0);
+    // unit j of the thread's copy list: j < PS_PCMAX: patch unit (round j >> 1, half j & 1); else weight unit j - PS_PCMAX
+    auto unit_load = [&](int j, u32x4 &v) {
+        if (j < PS_PCMAX) {
+            if (st.pcur && (j >> 1) * PS_NT < p.P1s) v = ps_patch_load(d, xb, padvec, p, st.pchunk, j >> 1, j & 1);
+        } else if (j < PS_PCMAX + PS_WUMAX) {
+            const int tp = st.wtap0 + (j - PS_PCMAX) * st.wtaps;
+            if (tp < 9) v = *reinterpret_cast<const u32x4 *>(st.wsrc + tp * st.tap_bytes);
+        }
+    };
+    auto unit_store = [&](int j, const u32x4 &v) {
+        if (j < PS_PCMAX) {
+            if (st.pcur && (j >> 1) * PS_NT < p.P1s) ps_patch_store(st.patch, p, st.pchunk, j >> 1, j & 1, v);
+        } else if (j < PS_PCMAX + PS_WUMAX) {
+            const int tp = st.wtap0 + (j - PS_PCMAX) * st.wtaps;
+            if (tp < 9) *reinterpret_cast<u32x4 *>(st.wdst + tp * 4096) = v;
+        }
+    };
+    // which position slot of a tap the loads / stores ride behind: loads early, stores late, so that a unit has more
+    // than two taps to arrive
+    const int i_load = 0, i_store = MT - 1;
+#pragma unroll
+    for (int t = 0; t < 9; ++t) {
+        const int cur = t & 1, nxt = cur ^ 1;
+        const int kw1 = (t + 1) % 3;  // filter column of the next tap
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            // younger than this operand: the rest of this tap's, and what was issued for the next tap so far
+            // (two weight operands and the activation operands of the slots before this one)
+            const int pending = t == 8 ? MT - 1 - i : (i == 0 ? MT - 1 : MT + 1);
+            if (i == 0) ps_operands_ready(a[cur][0], a[cur][1], b[i], pending);
+            else ps_operand_ready(b[i], pending);
+            __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                if (FIRST && t == 0) {
+                    const i32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                    acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[cur][j], b[i], zero, 0, 0, 0);
+                } else {
+                    acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[cur][j], b[i], acc[j][i], 0, 0, 0);
+                }
+            }
+            __builtin_amdgcn_s_setprio(0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (i == 0 && t < 8) {
+                ps_ds_read128(a[nxt][0], wr, (t + 1) * 4096);
+                ps_ds_read128(a[nxt][1], wr, (t + 1) * 4096 + 512);
+            }
+            if (i == i_load && 2 * t < PS_PCMAX + PS_WUMAX) {
+                unit_load(2 * t, stg[t % 3][0]);
+                unit_load(2 * t + 1, stg[t % 3][1]);
+            }
+            if (i == i_store && t >= 2 && 2 * (t - 2) < PS_PCMAX + PS_WUMAX) {
+                unit_store(2 * (t - 2), stg[(t - 2) % 3][0]);
+                unit_store(2 * (t - 2) + 1, stg[(t - 2) % 3][1]);
+            }
+            if (t < 8) {
+                if (kw1 == 0) xr[i] += PW16;  // the next tap starts a filter row
+                ps_ds_read128(b[i], xr[i], kw1 * 16);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+}
+
+// OUT: how the output bytes are formed and stored.
+enum { PS_OUT_NCHW = 0, PS_OUT_BLOCKED_LUT = 1, PS_OUT_BLOCKED = 2 };
+
+// tabs: the per-channel requantisation multipliers (kpad floats) followed by the integer corrections (kpad ints).
+template <int MT, int OUT>
+__global__ void __launch_bounds__(PS_NT)
+qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, const char *__restrict__ tabs,
+                const int8_t *__restrict__ padvec, uint8_t *__restrict__ y, PsGeom p, QConvArgs q) {
+    constexpr bool y_blocked = OUT != PS_OUT_NCHW, use_lut = OUT != PS_OUT_BLOCKED;
+    extern __shared__ __attribute__((aligned(256))) char ps_lds_raw[];
+    // LDS: [256-byte activation table, 256-aligned][multipliers, corrections][weight ring: 2 slabs][slot table]
+    //      [patch: 2*NC blocks x P1s x 16]
+    const unsigned lut_a = (ps_lds_addr(ps_lds_raw) + 255u) & ~255u;
+    char *lds = ps_lds_raw + (lut_a - ps_lds_addr(ps_lds_raw));
+    uint8_t *lut = reinterpret_cast<uint8_t *>(lds);
+    char *tab_l = lds + 256;
+    char *wring = tab_l + p.tab_rounds * PS_NT * 16;
+    int *postab = reinterpret_cast<int *>(wring + 2 * PS_RING);  // [MT][PS_NT]: where each lane's position slots lie
+    char *patch = reinterpret_cast<char *>(postab + MT * PS_NT);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, lh = lane >> 5;
+    // wave -> (pair of channel blocks, group of position tiles): KP = 128: two pairs x four groups; KP = 64: one pair x
+    // eight groups.  Waves w and w + 4 share a SIMD; with two pairs they hold groups g and g + 2 of one pair.
+    const int pairs = p.KP >> 6, NG = PS_WAVES / pairs;
+    const int cp = wave % pairs, grp = wave / pairs;
+    // position tiles of this wave's group: the tile's npt tiles dealt evenly, the first (npt mod NG) groups one more
+    const int base = p.npt / NG, rem = p.npt - base * NG;
+    const int mt = base + (grp < rem ? 1 : 0), pt0 = grp * base + min(grp, rem);
+
+    // The activation table first, the table copies after it: an LDS write behind an asynchronous copy waits for it.
+    if (use_lut && tid < 256) {
+        const uint8_t v = uint8_t(tid);
+        lut[tid] = uint8_t((q.has_act ? qact_apply(v, q.act) : v) ^ (y_blocked ? 0x80 : 0));
+    }
+    const unsigned mult_a = ps_lds_addr(tab_l), corr_a = mult_a + unsigned(p.kpad) * 4u;
+    const unsigned postab_a = ps_lds_addr(postab) + unsigned(tid) * 4u;
+
+    const int NS = p.NKP * p.NC;           // steps per tile: (pass, chunk)
+    const int tap_bytes = 2 * p.KP * 16;   // packed weights of one tap: [half][KP][16]
+    const unsigned PW16 = unsigned(p.PW * 16);
+    // The weight ring: two slabs (the step being multiplied, the step being copied) of 9 taps x 4 KB, each tap laid out
+    // as in the packed weights.  The threads split a slab: unit wunit of every wtaps-th tap from wtap0.
+    const int upt = tap_bytes >> 4;        // 16-byte units per tap: 256 or 128
+    PsStream st;
+    st.tap_bytes = tap_bytes; st.patch = patch;
+    st.wtaps = PS_NT / upt; st.wtap0 = __builtin_amdgcn_readfirstlane(tid / upt);  // wave-uniform: upt is a multiple of 64
+    const int wunit = tid - st.wtap0 * upt;
+    const unsigned wr0 = ps_lds_addr(wring) + unsigned(lh * p.KP + 2 * cp * 32 + l32) * 16u;  // this lane's operand, tap 0
+
+    int tile = int(blockIdx.x);
+    if (tile >= p.n_tiles) return;
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the activation table is written
+    // the two tables: rounds of 16-byte units straight into LDS; lanes past the end repeat the last unit into padding
+    for (int r = 0; r < p.tab_rounds; ++r) {
+        const int u = min(r * PS_NT + tid, p.kpad / 2 - 1);
+        __builtin_amdgcn_global_load_lds((gptr_t)(tabs + u * 16), (lptr_t)(tab_l + (r * PS_NT + wave * 64) * 16), 16, 0, 0);
+    }
+    // The first tile's first patch chunk and the weights of step 0 at once.  Everything later is copied by the steps
+    // themselves, two units per tap, so that the copy stream never stops.
+    PsDesc desc;
+    ps_describe(desc, p, tile);
+    u32x4 pv[PS_RMAX][2], wv[PS_WUMAX];
+#pragma unroll
+    for (int r = 0; r < PS_RMAX; ++r)
+        if (r * PS_NT < p.P1s) {
+            pv[r][0] = ps_patch_load(desc, xb, padvec, p, 0, r, 0);
+            pv[r][1] = ps_patch_load(desc, xb, padvec, p, 0, r, 1);
+        }
+#pragma unroll
+    for (int k = 0; k < PS_WUMAX; ++k) {
+        const int tp = st.wtap0 + k * st.wtaps;
+        if (tp < 9) wv[k] = *reinterpret_cast<const u32x4 *>(wp + wunit * 16 + tp * tap_bytes);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // While those loads are in flight: position slot i of this lane: image, row, column inside the tile
+    // (image << 20 | row << 10 | column, -1 beyond the tile; kept in LDS for the epilogues) and the LDS address of the
+    // slot's patch entry in channel block `lh`.
+    unsigned xbase[MT];
+    {
+        const int per_img = p.TH * p.OW;
+        const float inv_per_img = 1.0f / float(per_img), inv_ow = 1.0f / float(p.OW);
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const int pp = (pt0 + i) * 32 + l32;
+            const int img = small_div(pp, per_img, inv_per_img), r2 = pp - img * per_img;
+            const int r = small_div(r2, p.OW, inv_ow), c = r2 - r * p.OW;
+            const bool in_tile = i < mt && img < p.NB;
+            const int lds_off = in_tile ? (img * p.PH + r) * p.PW + c : 0;
+            xbase[i] = ps_lds_addr(patch) + unsigned(lh * p.P1s + lds_off) * 16u;
+            postab[i * PS_NT + tid] = in_tile ? (img << 20) | (r << 10) | c : -1;
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int r = 0; r < PS_RMAX; ++r)
+        if (r * PS_NT < p.P1s) {
+            ps_patch_store(patch, p, 0, r, 0, pv[r][0]);
+            ps_patch_store(patch, p, 0, r, 1, pv[r][1]);
+        }
+#pragma unroll
+    for (int k = 0; k < PS_WUMAX; ++k) {
+        const int tp = st.wtap0 + k * st.wtaps;
+        if (tp < 9) *reinterpret_cast<u32x4 *>(wring + wunit * 16 + tp * 4096) = wv[k];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    i32x16 acc[2][MT];
+    int gs = 0;  // steps done by this workgroup; its parity selects the ring slab a step reads
+    while (true) {
+        const int next_tile = tile + int(gridDim.x);
+        int s = 0;
+        for (int kp = 0; kp < p.NKP; ++kp) {
+            // One step = (pass kp, chunk c).  At its boundary this thread's copies (LDS writes, and the table copies of
+            // the first tile) are done, and everybody has left the previous step.
+            auto boundary = [&]() {
+                if (gs == 0) __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+                else __builtin_amdgcn_s_waitcnt(0xC07F);           // lgkmcnt(0): output stores may still be on their way
+                __builtin_amdgcn_s_barrier();
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            // what step s copies: the next step's weights (the first step's after the last), and a patch chunk
+            auto plan_copies = [&](int c) {
+                const int s1 = s + 1 == NS ? 0 : s + 1;
+                st.wsrc = wp + size_t(s1) * 9 * tap_bytes + wunit * 16;
+                st.wdst = wring + ((gs + 1) & 1) * PS_RING + wunit * 16;
+                st.pcur = 0;
+                st.pchunk = 0;
+                if (kp == 0 && c + 1 < p.NC) {
+                    st.pcur = 1; st.pchunk = c + 1;
+                } else if (s + 1 == NS && p.NC > 1 && next_tile < p.n_tiles) {
+                    ps_describe(desc, p, next_tile);  // chunk 0 of the next tile: nobody reads that region any more
+                    st.pcur = 1;
+                }
+            };
+            {
+                boundary();
+                plan_copies(0);
+                // slots past this wave's tiles multiply patch entry 0; their results are dropped
+                ps_mfma_step<MT, true>(wr0 + unsigned((gs & 1) * PS_RING), xbase, 0u, PW16, st, desc, xb, padvec, p, acc);
+                ++s; ++gs;
+            }
+            for (int c = 1; c < p.NC; ++c, ++s, ++gs) {
+                boundary();
+                plan_copies(c);
+                ps_mfma_step<MT, false>(wr0 + unsigned((gs & 1) * PS_RING), xbase, unsigned(2 * c * p.P1s * 16), PW16, st, desc,
+                                        xb, padvec, p, acc);
+            }
+
+            // ---- end of pass kp: requantisation (+ fused activation), stores ----
+            if (s == NS && p.NC == 1 && next_tile < p.n_tiles) {
+                // a single channel chunk cannot be refilled while it is read: the next tile's patch goes in at once,
+                // after everybody has left the matrix-core loop, and lands under this epilogue
+                __builtin_amdgcn_s_barrier();
+                __builtin_amdgcn_sched_barrier(0);
+                ps_describe(desc, p, next_tile);
+#pragma unroll
+                for (int r = 0; r < PS_RMAX; ++r)
+                    if (r * PS_NT < p.P1s) {
+                        ps_patch_store(patch, p, 0, r, 0, ps_patch_load(desc, xb, padvec, p, 0, r, 0));
+                        ps_patch_store(patch, p, 0, r, 1, ps_patch_load(desc, xb, padvec, p, 0, r, 1));
+                    }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            {
+                const int ig = tile / p.n_row_tiles;
+                const int n0 = ig * p.NB, oh0 = (tile - ig * p.n_row_tiles) * p.TH;
+                const int rows_here = min(p.TH, p.OH - oh0), imgs_here = min(p.NB, p.N - n0);
+                const int plane = p.OH * p.OW;
+                const float zpf = float(q.y_zp);
+                const unsigned img_stride = unsigned((y_blocked ? p.KB : p.K) * plane);
+                // where this lane's position slots lie
+                uint32_t praw[MT];
+#pragma unroll
+                for (int i = 0; i < MT; ++i) praw[i] = ps_read_b32(postab_a + unsigned(i * PS_NT * 4));
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int kblk = kp * p.KP + (2 * cp + j) * 32;  // first channel of this 32-channel block
+                    const int kbase = kblk + lh * 4;
+                    // multipliers and integer corrections (bias and zero-point term) of this lane's 16 channels
+                    uint32_t mraw[16], craw[16];
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) mraw[v] = ps_read_b32(mult_a + unsigned(kbase + (v >> 2) * 8 + (v & 3)) * 4u);
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) craw[v] = ps_read_b32(corr_a + unsigned(kbase + (v >> 2) * 8 + (v & 3)) * 4u);
+                    ps_wait16(mraw);
+                    ps_wait16(craw);
+                    if (j == 0) {
+#pragma unroll
+                        for (int i = 0; i < MT; ++i) asm volatile("" : "+v"(praw[i]));  // behind the wait above
+                    }
+                    float mv[16];
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) mv[v] = __uint_as_float(mraw[v]);
+                    const int cb0 = kblk >> 4;
+                    // scalar part of the output offset (16-byte units of the blocked tensor / elements of the NCHW one)
+                    const unsigned origin = y_blocked ? unsigned((n0 * p.KB + cb0) * plane + oh0 * p.OW)
+                                                      : unsigned((n0 * p.K + kbase) * plane + oh0 * p.OW);
+#pragma unroll
+                    for (int i = 0; i < MT; ++i) {
+                        __builtin_amdgcn_sched_barrier(0);  // one position tile at a time
+                        const int pos = int(praw[i]);
+                        const int img = pos >> 20, r = (pos >> 10) & 1023, cc = pos & 1023;
+                        const bool ok = pos >= 0 && img < imgs_here && r < rows_here;
+                        const unsigned rel = __umul24(unsigned(img), img_stride) + __umul24(unsigned(r), unsigned(p.OW)) + unsigned(cc);
+                        int av[16];  // this tile's sums with the corrections added
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) av[v] = acc[j][i][v] + int(craw[v]);
+                        if constexpr (y_blocked) {
+                            // [N][KB][OH][OW][16] signed.  A lane holds 4 groups of 4 consecutive channels of one position
+                            uint32_t d[4];
+                            if constexpr (use_lut) {
+                                uint32_t ob[16];
+#pragma unroll
+                                for (int v = 0; v < 16; ++v)
+                                    ob[v] = ps_read_u8(__builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(float(av[v]) * mv[v]) + zpf, 0u, lut_a));
+                                ps_wait16(ob);
+#pragma unroll
+                                for (int gq = 0; gq < 4; ++gq)
+                                    d[gq] = ob[gq * 4] | (ob[gq * 4 + 1] << 8) | (ob[gq * 4 + 2] << 16) | (ob[gq * 4 + 3] << 24);
+                            } else {
+#pragma unroll
+                                for (int gq = 0; gq < 4; ++gq) {
+                                    uint32_t w4 = 0;
+#pragma unroll
+                                    for (int e = 0; e < 4; ++e)
+                                        w4 = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(float(av[gq * 4 + e]) * mv[gq * 4 + e]) + zpf, unsigned(e), w4);
+                                    d[gq] = w4 ^ 0x80808080u;
+                                }
+                            }
+                            // Lanes l and l + 32 hold the two interleaved halves of the wave's two 16-channel blocks: the
+                            // half-wave swap leaves the lower lane with all 16 bytes of the first block and the upper lane
+                            // with those of the second, so each lane stores one whole 16-byte unit and a half wave 512
+                            // contiguous bytes.
+                            const auto s0 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
+                            const auto s1 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
+                            u32x4 out;
+                            out[0] = s0[0]; out[1] = s0[1]; out[2] = s1[0]; out[3] = s1[1];
+                            if (ok && cb0 + lh < p.KB)
+                                __builtin_nontemporal_store(out, reinterpret_cast<u32x4 *>(y) + (origin + rel + unsigned(lh * plane)));
+                        } else {
+                            uint32_t ob[16];
+#pragma unroll
+                            for (int v = 0; v < 16; ++v)
+                                ob[v] = ps_read_u8(__builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(float(av[v]) * mv[v]) + zpf, 0u, lut_a));
+                            ps_wait16(ob);
+                            if (ok) {
+                                uint8_t *yp = y + (origin + rel);
+#pragma unroll
+                                for (int v = 0; v < 16; ++v) {
+                                    const int dk = (v >> 2) * 8 + (v & 3);
+                                    if (kbase + dk < p.K) yp[dk * plane] = uint8_t(ob[v]);
+                                }
+                            }
+                        }
+                    }
+                }
+            }
+        }
+        tile = next_tile;
+        if (tile >= p.n_tiles) break;
+    }
+}
+
+// Packs OIHW int8 weights into [pass][chunk of 32 input channels][tap][half][KP][16] (zero padded): the order in
+// which the kernel's steps consume them, so that the weight stream is one run of addresses.  Also writes the
+// per-channel requantisation multiplier, the integer correction (bias + (128 - x_zp) * sum of weights) and the 16-byte
+// padding vector (x_zp - 128 in every lane).
+__global__ void __launch_bounds__(256)
+ps_pack_kernel(const int8_t *__restrict__ w, const float *__restrict__ w_scale, const int32_t *__restrict__ bias,
+               int8_t *__restrict__ wp, float *__restrict__ mult, int32_t *__restrict__ corr, int8_t *__restrict__ padvec,
+               int K, int C, int NC, int NKP, int KP, float x_scale, float y_scale, int x_zp, int n_wscale) {
+    const int64_t total = int64_t(NKP) * NC * 9 * 32 * KP;
+    const int64_t step = int64_t(gridDim.x) * blockDim.x;
+    const int64_t gid = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (gid < 16) padvec[gid] = int8_t(x_zp - 128);
+    for (int64_t i = gid; i < total; i += step) {
+        int64_t r = i;
+        const int j = int(r & 15); r >>= 4;
+        const int kk = int(r % KP); r /= KP;
+        const int half = int(r & 1); r >>= 1;
+        const int tap = int(r % 9); r /= 9;
+        const int chunk = int(r % NC); r /= NC;
+        const int kp = int(r);
+        const int k = kp * KP + kk, c = chunk * 32 + half * 16 + j;
+        wp[i] = (k < K && c < C) ? w[(int64_t(k) * C + c) * 9 + tap] : int8_t(0);
+    }
+    // per output channel: one wavefront sums the channel's weights
+    const int kpad = NKP * KP;
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = gid >> 6, n_waves = step >> 6;
+    for (int64_t k = wave; k < kpad; k += n_waves) {
+        int sum = 0;
+        if (k < K) {
+            const int8_t *wk = w + k * int64_t(C) * 9;
+            for (int e = lane; e < C * 9; e += 64) sum += int(wk[e]);
+        }
+        for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+        if (lane == 0) {
+            corr[k] = k < K ? (bias ? bias[k] : 0) + (128 - x_zp) * sum : 0;
+            mult[k] = k < K ? (x_scale * w_scale[n_wscale == 1 ? 0 : k]) / y_scale : 0.0f;
+        }
+    }
+}
+
+size_t ps_align256(size_t v) { return (v + 255) & ~size_t(255); }
+
+// Picks the tile (NB images x TH rows) with the smallest estimated time: rounds of tiles over the CUs times the MFMA
+// count of the busiest SIMD of a tile, plus a fixed cost per tile for its fill and epilogue.
+bool ps_plan(const ConvGeom &g, int num_cus, PsGeom *out, size_t *lds_bytes, int *MT) {
+    if (g.groups != 1 || g.KH != 3 || g.KW != 3 || g.sh != 1 || g.sw != 1 || g.dh != 1 || g.dw != 1) return false;
+    if (g.pt > 1 || g.pl > 1 || g.C < 32 || g.K < 33) return false;
+    if (g.OH > 1023 || g.OW > 1023) return false;
+    const int CB = (g.C + 15) / 16;
+    if (int64_t(g.N) * CB * g.H * g.W >= (int64_t(1) << 27)) return false;  // 16-byte units addressed with 32-bit offsets
+    PsGeom p{};
+    p.N = g.N; p.H = g.H; p.W = g.W; p.CB = CB; p.K = g.K; p.KB = (g.K + 15) / 16; p.OH = g.OH; p.OW = g.OW; p.pt = g.pt; p.pl = g.pl;
+    p.NC = (g.C + 31) / 32;
+    p.KP = g.K > 64 ? 128 : 64;
+    p.NKP = (g.K + p.KP - 1) / p.KP;
+    p.kpad = p.NKP * p.KP;
+    p.tab_rounds = (p.kpad / 2 + PS_NT - 1) / PS_NT;
+    const int pairs = p.KP / 64, NG = PS_WAVES / pairs;
+    const int max_pos = NG * PS_MTMAX * 32;
+    // output offsets are formed in 32 bits, per-image strides with 24-bit multiplies
+    const int64_t plane = int64_t(g.OH) * g.OW;
+    if (int64_t(p.KB) * plane >= (1 << 24) || int64_t(g.N) * p.KB * plane >= (int64_t(1) << 28)) return false;
+    if (int64_t(g.K) * plane >= (1 << 24) || int64_t(g.N) * g.K * plane >= (int64_t(1) << 31)) return false;
+    const size_t fixed = 256 + 256 + size_t(p.tab_rounds) * PS_NT * 16 + 2 * size_t(PS_RING);  // + slot table and patch
+    const size_t cap = 160 * 1024;
+    double best = 0;
+    bool found = false;
+    p.PW = g.OW + 2;
+    auto consider = [&](int NB, int TH) {
+        PsGeom t = p;
+        t.NB = NB; t.TH = TH;
+        const int S = NB * TH * g.OW;
+        if (S > max_pos || S < 1) return;
+        t.PH = TH + 2;
+        t.P1 = NB * t.PH * t.PW;
+        t.P1s = (t.P1 + PS_NT - 1) / PS_NT * PS_NT;
+        if (t.P1s / PS_NT > PS_RMAX || NB > 2047) return;
+        t.npt = (S + 31) / 32;
+        const int per_wave = (t.npt + NG - 1) / NG;
+        const size_t lds = fixed + size_t(per_wave) * PS_NT * 4 + size_t(2 * t.NC) * t.P1s * 16;
+        if (lds > cap) return;
+        t.n_row_tiles = (g.OH + TH - 1) / TH;
+        const int64_t nt = int64_t((g.N + NB - 1) / NB) * t.n_row_tiles;
+        if (nt >= (int64_t(1) << 30)) return;
+        t.n_tiles = int(nt);
+        // MFMAs of the busiest SIMD (waves w and w + 4) per tile
+        const int base = t.npt / NG, rem = t.npt % NG;
+        auto tiles_of = [&](int grp) { return base + (grp < rem ? 1 : 0); };
+        int busiest_tiles = 0;
+        for (int w = 0; w < 4; ++w) busiest_tiles = std::max(busiest_tiles, tiles_of(w / pairs) + tiles_of((w + 4) / pairs));
+        const double mfma = 2.0 * busiest_tiles * t.NKP * t.NC * 9 * 32.0;
+        const double rounds = double((t.n_tiles + num_cus - 1) / num_cus);
+        const double tile_cycles = mfma + 4000.0 + double(S) * p.kpad / 256.0 * 7.0;  // + fill, + epilogue VALU
+        const double score = 1.0 / (rounds * tile_cycles);
+        if (!found || score > best * 1.01) {
+            best = score; found = true; *out = t; *lds_bytes = lds; *MT = per_wave;
+        }
+    };
+    const int per_img = g.OH * g.OW;
+    if (per_img <= max_pos)
+        for (int NB = 1; NB <= std::min(g.N, max_pos / per_img); ++NB) consider(NB, g.OH);
+    for (int TH = 1; TH <= g.OH; ++TH) consider(1, TH);
+    return found;
+}
+
+template <int MT, int OUT>
+void ps_launch_out(zant_ctx *ctx, int grid, size_t lds, const int8_t *xb, const int8_t *wp, const char *tabs,
+                   const int8_t *padvec, uint8_t *y, const PsGeom &p, const QConvArgs &q) {
+    static bool attr_set = false;
+    if (!attr_set) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&qconv_ps_kernel<MT, OUT>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((qconv_ps_kernel<MT, OUT>), dim3(grid), dim3(PS_NT), lds, ctx->stream, xb, wp, tabs, padvec, y, p, q);
+}
+
+template <int MT>
+void ps_launch(zant_ctx *ctx, int grid, size_t lds, const int8_t *xb, const int8_t *wp, const char *tabs,
+               const int8_t *padvec, uint8_t *y, const PsGeom &p, const QConvArgs &q, int yb) {
+    if (!yb) ps_launch_out<MT, PS_OUT_NCHW>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
+    else if (q.has_act) ps_launch_out<MT, PS_OUT_BLOCKED_LUT>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
+    else ps_launch_out<MT, PS_OUT_BLOCKED>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
+}
+
+}  // namespace
+
+// The patch-stationary matrix-core path; ZANT_OK when it ran (or, with plan_only, would run), 1 when the shape is left
+// to the other kernels.
+int zant_qconv_ps(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float *w_scale, const int32_t *bias, uint8_t *y,
+                  const ConvGeom &g, const QConvArgs &q, bool x_blocked, bool y_blocked, zant_pack_slot *slot, bool plan_only) {
+    PsGeom p;
+    size_t lds = 0;
+    int MT = 0;
+    if (!ps_plan(g, ctx->num_cus, &p, &lds, &MT)) return 1;
+    if (MT < 1 || MT > PS_MTMAX) return 1;
+    if (plan_only) return ZANT_OK;
+    const size_t wp_bytes = size_t(p.NKP) * p.NC * 9 * 32 * p.KP;
+    const size_t xb_bytes = x_blocked ? 0 : size_t(g.N) * p.CB * g.H * g.W * 16;
+    // [tile counters (unused) | padding vector | multipliers, corrections (one contiguous table) | packed weights]
+    const size_t o_pad = 256, o_mult = 512, o_corr = o_mult + size_t(p.kpad) * 4,
+                 o_wp = o_mult + ps_align256(size_t(p.kpad) * 8), static_bytes = o_wp + ps_align256(wp_bytes);
+    void *ws = nullptr, *dyn = nullptr;
+    bool need_pack = true;
+    int parity = 0;
+    int rc = zant_pack_region(ctx, slot, static_bytes, xb_bytes, &ws, &dyn, &need_pack, &parity);
+    if (rc) return rc;
+    char *base = static_cast<char *>(ws);
+    int8_t *padvec = reinterpret_cast<int8_t *>(base + o_pad);
+    float *mult = reinterpret_cast<float *>(base + o_mult);
+    int32_t *corr = reinterpret_cast<int32_t *>(base + o_corr);
+    int8_t *wp = reinterpret_cast<int8_t *>(base + o_wp);
+    if (need_pack) {
+        const unsigned pb = unsigned(std::min<int64_t>(std::max<int64_t>(ceil_div64(int64_t(wp_bytes), 256), ceil_div64(p.kpad, 4)), 1024));
+        hipLaunchKernelGGL(ps_pack_kernel, dim3(pb), dim3(256), 0, ctx->stream, w, w_scale, bias, wp, mult, corr, padvec, g.K, g.C,
+                           p.NC, p.NKP, p.KP, q.x_scale, q.y_scale, q.x_zp, q.n_wscale);
+        ZANT_LAUNCH_CHECK(ctx);
+    }
+    const int8_t *xb = reinterpret_cast<const int8_t *>(x);
+    if (!x_blocked) {
+        rc = zant_to_blocked(ctx, x, g.N, g.C, int64_t(g.H) * g.W, static_cast<uint8_t *>(dyn));
+        if (rc) return rc;
+        xb = static_cast<const int8_t *>(dyn);
+    }
+    const int grid = std::min(p.n_tiles, ctx->num_cus);
+    KernelTimer kt(ctx);
+    const int yb = y_blocked ? 1 : 0;
+    const char *tabs = base + o_mult;
+    switch (MT) {
+    case 1: ps_launch<1>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q, yb); break;
+    case 2: ps_launch<2>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q, yb); break;
+    case 3: ps_launch<3>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q, yb); break;
+    default: ps_launch<4>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q, yb); break;
+    }
+    ZANT_LAUNCH_CHECK(ctx);
+    return ZANT_OK;
+}

@@ -29,6 +29,16 @@ struct QAct {
     uint8_t out_zp;
 };
 
+// Quantisation parameters of one QLinearConv as its kernels take them.
+struct QConvArgs {
+    float x_scale, y_scale;
+    int x_zp;
+    uint8_t y_zp;
+    int n_wscale;       // 1 or K
+    int has_act;
+    QAct act;
+};
+
 __device__ __forceinline__ float act_f32(float v, int act, float alpha) {
     switch (act) {
     case ZANT_ACT_RELU: return v > 0.0f ? v : 0.0f;
