@@ -148,7 +148,7 @@ int zant_hip_matmul_check(const int64_t *adim, int a_rank, const int64_t *bdim, 
 /* gemm_lean = lean_gemm (op_gemm.zig:91-185): Y = alpha*op(A)*op(B) + beta*C on
  * {1,1,R,C} tensors, C broadcast over rows and/or columns.  Transposes are folded
  * into the loads.  fuse_act as for conv; ZANT_ACT_SOFTMAX (the classifier head Gemm -> Softmax in one kernel,
- * reference op_softmax.zig lean_softmax on the [rows, cols] result) is accepted for cols <= 16 without trans_a
+ * lean_softmax, lib_activation_function_math.zig:154-187, on the [rows, cols] result) is accepted for cols <= 16 without trans_a
  * and returns InvalidInput otherwise. */
 int zant_hip_gemm_f32(zant_ctx *ctx, const float *a, const int64_t adim[4], const float *b, const int64_t bdim[4],
                       const float *c, const int64_t *cdim, int c_rank, float alpha, float beta, int trans_a,
@@ -165,6 +165,23 @@ int zant_hip_maxpool2d_f32(zant_ctx *ctx, const float *x, const int64_t xdim[4],
 int zant_hip_maxpool2d_out_shape(const int64_t xdim[4], const int64_t kernel[2], const int64_t strides[2],
                                  const int64_t dil[2], const int64_t pads[4], int auto_pad, int ceil_mode,
                                  int64_t ydim[4]);
+
+/* Average pooling: pool_forward with PoolingType.Avg (op_pooling.zig:223-260, 373-408): per window the sum of
+ * the taps inside the input, in (row, column) order, divided by their count.  The reference takes no padding;
+ * pads [top, left, bottom, right] (NULL = none, each smaller than the kernel) and count_include_pad extend it to
+ * ONNX AveragePool: with count_include_pad the divisor is the number of taps inside the PADDED input.  The
+ * shape function gives pool_forward's (H - k) / s + 1 over the padded input, with ONNX's ceil_mode (host only). */
+int zant_hip_avgpool2d_f32(zant_ctx *ctx, const float *x, const int64_t xdim[4], float *y, const int64_t ydim[4],
+                           const int64_t kernel[2], const int64_t strides[2], const int64_t pads[4],
+                           int count_include_pad);
+int zant_hip_avgpool2d_out_shape(const int64_t xdim[4], const int64_t kernel[2], const int64_t strides[2],
+                                 const int64_t pads[4], int ceil_mode, int64_t ydim[4]);
+/* BatchNormalization, inference form: BatchNormLayer.forward with is_training false
+ * (src/Model/Layers/batchNormLayer.zig:130-148): y = (x - mean[f]) / sqrt(var[f] + epsilon) * gamma[f] + beta[f]
+ * in that order of operations, f the index on axis 1 (the reference's layer takes [batch, features]; any rank
+ * 2..8 here, as ONNX BatchNormalization on NCHW needs).  gamma, beta, mean, var: device arrays of xdim[1]. */
+int zant_hip_batchnorm_f32(zant_ctx *ctx, const float *x, const int64_t *xdim, int rank, const float *gamma,
+                           const float *beta, const float *mean, const float *var, float epsilon, float *y);
 
 /* ReLU_lean (lib_activation_function_math.zig:22-28).  The reference writes only
  * where x > 0 and relies on a zeroed output; this writes x > 0 ? x : 0 everywhere,
@@ -289,6 +306,14 @@ int zant_model_relu(zant_model *m, int x);
 int zant_model_leaky_relu(zant_model *m, int x, float slope);
 int zant_model_maxpool(zant_model *m, int x, const int64_t kernel[2], const int64_t strides[2],
                        const int64_t dil[2], const int64_t pads[4], int auto_pad, int ceil_mode);
+/* AveragePool (zant_hip_avgpool2d_f32); pads may be NULL. */
+int zant_model_avgpool(zant_model *m, int x, const int64_t kernel[2], const int64_t strides[2], const int64_t pads[4],
+                       int ceil_mode, int count_include_pad);
+/* BatchNormalization, inference form (zant_hip_batchnorm_f32); gamma / beta / mean / var are HOST arrays of
+ * `features` = dims[1] floats.  Behind a convolution that nothing else reads, finalize folds it into the
+ * convolution's weights and bias (w * s, (b - mean) * s + beta with s = gamma / sqrt(var + epsilon)). */
+int zant_model_batchnorm(zant_model *m, int x, const float *gamma, const float *beta, const float *mean,
+                         const float *var, int64_t features, float epsilon);
 int zant_model_reshape(zant_model *m, int x, const int64_t *new_shape, int rank);
 int zant_model_gemm(zant_model *m, int a, const float *b, const int64_t bdim[4], const float *c,
                     const int64_t *cdim, int c_rank, float alpha, float beta, int trans_a, int trans_b);
@@ -324,7 +349,8 @@ size_t zant_model_unfused_bytes(zant_model *m); /* sum of all node outputs, the 
 int zant_model_num_launches(zant_model *m);     /* operator calls per run after fusion */
 /* One forward pass, device in / device out, asynchronous, no allocation.  input_dev == NULL means the
  * caller already wrote the input at zant_model_input_ptr(); output_dev == NULL leaves the result at
- * zant_model_output_ptr() (both inside the arena, valid after finalize). */
+ * zant_model_output_ptr() (both inside the arena, valid after finalize).  A pass does not write to the
+ * input's storage: an input placed at zant_model_input_ptr() once serves any number of passes. */
 int zant_model_run(zant_model *m, const void *input_dev, void *output_dev);
 void *zant_model_input_ptr(zant_model *m);
 void *zant_model_output_ptr(zant_model *m);
@@ -337,7 +363,8 @@ int zant_model_predict_host(zant_model *m, const void *input_host, void *output_
  * "Conv+Relu+MaxPool". */
 int zant_model_profile(zant_model *m, float *ms, double *ops, double *bytes, int capacity);
 const char *zant_model_launch_name(zant_model *m, int i);
-/* Debug: copies tensor `id` (as planned in the arena) to the host after a run.  Tensors that a fusion removed (the
+/* Debug: copies tensor `id` to the host: replays the last pass up to the node that produces it (its storage may have
+ * been planned under a later tensor), then reads it from the arena.  Tensors that a fusion removed (the
  * output of a convolution whose pool, or of a residual block's inner layers, run in the same kernel) are never
  * materialised: ZANT_InvalidInput. */
 int zant_model_read_tensor(zant_model *m, int id, void *dst_host, size_t bytes);

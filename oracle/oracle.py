@@ -187,6 +187,53 @@ def onnx_maxpool(x, kernel, strides, dilations, pads, auto_pad="NOTSET", ceil_mo
     return onnx_maxpool_lean(x, y, kernel, strides, dilations, pads, auto_pad)
 
 
+def avgpool_out_shape(xshape, kernel, strides, pads=(0, 0, 0, 0), ceil_mode=False):
+    """pool_forward's output size (op_pooling.zig:239-240) with ONNX AveragePool's pads and ceil_mode; a last window
+    that would start in the bottom / right padding is dropped, as ONNX and torch do."""
+    out = []
+    for ax in range(2):
+        n = xshape[2 + ax] + pads[ax] + pads[2 + ax] - kernel[ax]
+        if n < 0:
+            raise OracleError(-1)
+        o = (-(-n // strides[ax]) if ceil_mode else n // strides[ax]) + 1
+        if ceil_mode and (o - 1) * strides[ax] >= xshape[2 + ax] + pads[ax]:
+            o -= 1
+        out.append(o)
+    return (xshape[0], xshape[1], out[0], out[1])
+
+
+def avgpool_lean(x, y, kernel, strides, pads=(0, 0, 0, 0), count_include_pad=False):
+    x = _f32(x)
+    xd, _ = _dims(x.shape); yd, _ = _dims(y.shape)
+    k, _ = _dims(kernel); s, _ = _dims(strides); p, _ = _dims(pads)
+    _chk(_lib.zo_avgpool_f32(_ptr(x), xd, _ptr(y), yd, k, s, p, int(count_include_pad)))
+    return y
+
+
+def avgpool(x, kernel, strides, pads=(0, 0, 0, 0), ceil_mode=False, count_include_pad=False):
+    """pool_forward(.Avg) for pads 0 / floor; ONNX AveragePool otherwise."""
+    if x.ndim != 4:
+        raise OracleError(-5)
+    y = np.zeros(avgpool_out_shape(x.shape, kernel, strides, pads, ceil_mode), np.float32)
+    return avgpool_lean(x, y, kernel, strides, pads, count_include_pad)
+
+
+def batchnorm(x, gamma, beta, mean, var, epsilon=1e-5):
+    """Inference BatchNormalization with the features on axis 1."""
+    x = _f32(x)
+    if x.ndim < 2:
+        raise OracleError(-1)
+    g, b, m, v = (_f32(np.asarray(a).reshape(-1)) for a in (gamma, beta, mean, var))
+    F = x.shape[1]
+    if not (g.size == b.size == m.size == v.size == F):
+        raise OracleError(-5)
+    y = np.zeros(x.shape, np.float32)
+    inner = int(np.prod(x.shape[2:])) if x.ndim > 2 else 1
+    _chk(_lib.zo_batchnorm_f32(_ptr(x), C.c_int64(x.shape[0]), C.c_int64(F), C.c_int64(inner), _ptr(g), _ptr(b), _ptr(m),
+                               _ptr(v), C.c_float(epsilon), _ptr(y)))
+    return y
+
+
 def ReLU_lean(x, y):
     x = _f32(x)
     _chk(_lib.zo_relu_lean_f32(_ptr(x), _ptr(y), C.c_int64(x.size)))

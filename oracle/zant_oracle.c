@@ -11,6 +11,12 @@
  *   Sigmoid / ReduceMean / Concat / Resize(nearest): pinned by the reference's
  *     known-answer tests (tests/golden/), numpy (mean, concatenate), scipy's
  *     expit and closed forms (integer upscales repeat elements).
+ *   AveragePool (pool_forward, .Avg) / BatchNormalization (inference form of
+ *     BatchNormLayer.forward): the reference's tests hold no expected values for
+ *     either (test_op_pooling.zig pools with .Max only; test_layers.zig:539-611
+ *     checks shapes only): parity unpinned by the reference; pinned by brute
+ *     force, torch.nn.functional.avg_pool2d / batch_norm on the CPU and the
+ *     closed forms (constant input, identity statistics).
  *   broadcast Add: the reference has no test for the broadcast branch and its
  *     stride computation reads out of bounds for mid-axis broadcasts; restated
  *     to NumPy semantics and pinned by numpy.
@@ -470,6 +476,56 @@ int zo_maxpool_lean_u8(const uint8_t *x, const int64_t xdim[4], uint8_t *y, cons
                 dst[oh * OW + ow] = m;
             }
     }
+    return ZO_OK;
+}
+
+/* Average pooling: pool_forward's .Avg branch (op_pooling.zig:223-260, 373-408): for each window the sum of the taps
+ * that lie inside the input, in kr, kc order, divided by their count.  The reference takes no padding (output
+ * (H - k) / s + 1, so every tap is inside); `pads` [top, left, bottom, right] extends it to ONNX AveragePool:
+ * with count_include_pad the divisor is the number of taps inside the PADDED input (ONNX: pad cells count as
+ * zeros, cells past the padded input -- ceil_mode -- do not), otherwise the in-bounds count as in the reference. */
+int zo_avgpool_f32(const float *x, const int64_t xdim[4], float *y, const int64_t ydim[4], const int64_t kernel[2],
+                   const int64_t strides[2], const int64_t pads[4], int count_include_pad) {
+    const int64_t N = xdim[0], C = xdim[1], H = xdim[2], W = xdim[3], OH = ydim[2], OW = ydim[3];
+    if (kernel[0] <= 0 || kernel[1] <= 0 || strides[0] <= 0 || strides[1] <= 0) return ZO_InvalidDimensions; /* :233-236 */
+    if (ydim[0] != N || ydim[1] != C || OH <= 0 || OW <= 0) return ZO_InvalidDimensions;
+    const int64_t top = pads ? pads[0] : 0, left = pads ? pads[1] : 0;
+    const int64_t bottom = pads ? pads[2] : 0, right = pads ? pads[3] : 0;
+    for (int64_t bc = 0; bc < N * C; ++bc) {
+        const float *src = x + bc * H * W;
+        float *dst = y + bc * OH * OW;
+        for (int64_t oh = 0; oh < OH; ++oh)
+            for (int64_t ow = 0; ow < OW; ++ow) {
+                float sum = 0.0f;
+                int64_t count = 0, padded = 0;
+                for (int64_t kr = 0; kr < kernel[0]; ++kr)
+                    for (int64_t kc = 0; kc < kernel[1]; ++kc) {
+                        const int64_t ih = oh * strides[0] - top + kr, iw = ow * strides[1] - left + kc;
+                        if (ih >= 0 && ih < H && iw >= 0 && iw < W) { sum += src[ih * W + iw]; ++count; } /* :381-387 */
+                        if (ih >= -top && ih < H + bottom && iw >= -left && iw < W + right) ++padded;
+                    }
+                const int64_t div = count_include_pad ? padded : count;
+                dst[oh * OW + ow] = div > 0 ? sum / (float)div : 0.0f; /* :401 */
+            }
+    }
+    return ZO_OK;
+}
+
+/* BatchNormalization, inference form (BatchNormLayer.forward with is_training false, batchNormLayer.zig:130-148):
+ * x_normalized = (x - running_mean[f]) / sqrt(running_var[f] + epsilon); y = x_normalized * gamma[f] + beta[f].
+ * The reference's layer takes [batch, features]; here the feature axis is axis 1 of a tensor of any rank (ONNX
+ * BatchNormalization on NCHW), `inner` = elements per (batch, feature) pair. */
+int zo_batchnorm_f32(const float *x, int64_t outer, int64_t features, int64_t inner, const float *gamma,
+                     const float *beta, const float *mean, const float *var, float epsilon, float *y) {
+    for (int64_t b = 0; b < outer; ++b)
+        for (int64_t f = 0; f < features; ++f) {
+            const float sd = sqrtf(var[f] + epsilon);
+            for (int64_t i = 0; i < inner; ++i) {
+                const int64_t idx = (b * features + f) * inner + i;
+                const float xn = (x[idx] - mean[f]) / sd;
+                y[idx] = xn * gamma[f] + beta[f];
+            }
+        }
     return ZO_OK;
 }
 

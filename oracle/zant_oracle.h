@@ -102,6 +102,12 @@ int zo_maxpool_lean_f32(const float *x, const int64_t xdim[4], float *y, const i
 
 /* lean_ReLU (lib_activation_function_math.zig:22-28): writes only where x > 0;
  * the caller's output keeps its previous content elsewhere. */
+/* pool_forward, .Avg (op_pooling.zig:223-260, 373-408), extended with ONNX AveragePool's pads / count_include_pad. */
+int zo_avgpool_f32(const float *x, const int64_t xdim[4], float *y, const int64_t ydim[4], const int64_t kernel[2],
+                   const int64_t strides[2], const int64_t pads[4], int count_include_pad);
+/* BatchNormLayer.forward, inference branch (batchNormLayer.zig:130-148), features on axis 1. */
+int zo_batchnorm_f32(const float *x, int64_t outer, int64_t features, int64_t inner, const float *gamma,
+                     const float *beta, const float *mean, const float *var, float epsilon, float *y);
 int zo_relu_lean_f32(const float *x, float *y, int64_t n);
 /* lean_leakyReLU (:68-77). */
 int zo_leaky_relu_lean_f32(const float *x, float slope, float *y, int64_t n);

@@ -12,6 +12,7 @@ import onnx_writer
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 MNIST = os.path.join(HERE, "golden", "mnist-8.onnx")
+DEBUG_MODEL = os.path.join(HERE, "golden", "debug_model.onnx")
 
 
 @pytest.fixture(scope="module")
@@ -87,6 +88,50 @@ def test_generated_mnist8_library_matches_the_oracle(codegen, tmp_path):
     assert b"Starting prediction...\n" in logged and b"Prediction completed.\n" in logged
     lib.setLogFunction(None)
     lib.mnist8_shutdown()
+
+
+def test_generator_lifts_onnx_gemm_operands_to_the_lean_form(codegen, tmp_path):
+    """debug_model.onnx (Gemm, Relu, Gemm, Relu, Softmax on a [1, 5] input): each Gemm has a 2-D A and B and a 1-D C in
+    the file and reaches the executor as [1,1,M,K] x [1,1,N,K] + [1,1,1,N] between two reshape views."""
+    info = codegen.generate(DEBUG_MODEL, str(tmp_path), "dbg")
+    text = open(info["c"]).read()
+    assert info["in_shape"] == (1, 5) and info["out_shape"] == (1, 5) and info["nodes"] == 9
+    assert text.count("zant_model_gemm(m,") == 2 and text.count("zant_model_reshape(m,") == 4
+    assert "(const int64_t[]){1, 1, 5, 5}" in text and "(const int64_t[]){1, 1, 1, 5}, 4," in text
+    assert text.count(", 0, 1) != ") == 2          # transA = 0, transB = 1 as the file says
+    assert "zant_model_softmax(m, 8)" in text
+    so = codegen.compile_library(info)
+    assert hasattr(_load(so), "dbg_init")
+
+
+def test_generator_records_pooling_and_normalisation_nodes(codegen, tmp_path):
+    g = np.random.default_rng(0)
+    vec = lambda n: onnx_writer.tensor(n, (g.random(4, dtype=np.float32) + 0.5))
+    nodes = [onnx_writer.node("BatchNormalization", ["x", "gamma", "beta", "mean", "var"], ["b"], epsilon=1e-3),
+             onnx_writer.node("AveragePool", ["b"], ["y"], kernel_shape=[2, 2], strides=[2, 2], count_include_pad=1)]
+    p = tmp_path / "pn.onnx"
+    p.write_bytes(onnx_writer.model(nodes, [vec("gamma"), vec("beta"), vec("mean"), vec("var")],
+                                    [onnx_writer.value_info("x", (2, 4, 8, 8), np.float32)], [onnx_writer.value_info("y", (2, 4, 4, 4), np.float32)]))
+    info = codegen.generate(str(p), str(tmp_path), "pn")
+    text = open(info["c"]).read()
+    assert "zant_model_batchnorm(m, 0," in text and "zant_model_avgpool(m, 1," in text and info["out_shape"] == (2, 4, 4, 4)
+
+
+@pytest.mark.gpu
+def test_generated_debug_model_library_matches_the_oracle(codegen, tmp_path):
+    from oracle import oracle as zo
+    from zant_amd import onnx_front
+    info = codegen.generate(DEBUG_MODEL, str(tmp_path), "dbg")
+    lib = _load(codegen.compile_library(info))
+    graph = onnx_front.read_graph(DEBUG_MODEL)
+    g = np.random.default_rng(3)
+    for _ in range(3):
+        x = (g.random((1, 5), dtype=np.float32) * 4 - 2).astype(np.float32)
+        ptr = _predict(lib, x)
+        assert ptr is not None
+        y = np.ctypeslib.as_array(C.cast(ptr, C.POINTER(C.c_float)), (1, 5)).copy()
+        np.testing.assert_allclose(y, onnx_front.run_graph(graph, zo, x), rtol=1e-4, atol=1e-5)
+    lib.dbg_shutdown()
 
 
 @pytest.mark.gpu

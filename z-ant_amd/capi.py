@@ -55,6 +55,9 @@ PROTOTYPES = {
     "zant_hip_maxpool2d_f32": (i32, [vp, vp, c_i64p, vp, c_i64p, c_i64p, c_i64p, c_i64p, c_i64p, i32, i32]),
     "zant_hip_maxpool2d_u8": (i32, [vp, vp, c_i64p, vp, c_i64p, c_i64p, c_i64p, c_i64p, c_i64p, i32, i32]),
     "zant_hip_maxpool2d_out_shape": (i32, [c_i64p, c_i64p, c_i64p, c_i64p, c_i64p, i32, i32, c_i64p]),
+    "zant_hip_avgpool2d_f32": (i32, [vp, vp, c_i64p, vp, c_i64p, c_i64p, c_i64p, c_i64p, i32]),
+    "zant_hip_avgpool2d_out_shape": (i32, [c_i64p, c_i64p, c_i64p, c_i64p, i32, c_i64p]),
+    "zant_hip_batchnorm_f32": (i32, [vp, vp, c_i64p, i32, vp, vp, vp, vp, f32, vp]),
     "zant_hip_relu_f32": (i32, [vp, vp, vp, i64]),
     "zant_hip_leaky_relu_f32": (i32, [vp, vp, f32, vp, i64]),
     "zant_hip_softmax_f32": (i32, [vp, vp, vp, i64, i64]),
@@ -83,6 +86,8 @@ PROTOTYPES = {
     "zant_model_relu": (i32, [vp, i32]),
     "zant_model_leaky_relu": (i32, [vp, i32, f32]),
     "zant_model_maxpool": (i32, [vp, i32, c_i64p, c_i64p, c_i64p, c_i64p, i32, i32]),
+    "zant_model_avgpool": (i32, [vp, i32, c_i64p, c_i64p, c_i64p, i32, i32]),
+    "zant_model_batchnorm": (i32, [vp, i32, vp, vp, vp, vp, i64, f32]),
     "zant_model_reshape": (i32, [vp, i32, c_i64p, i32]),
     "zant_model_gemm": (i32, [vp, i32, vp, c_i64p, vp, c_i64p, i32, f32, f32, i32, i32]),
     "zant_model_matmul": (i32, [vp, i32, vp, c_i64p, i32]),

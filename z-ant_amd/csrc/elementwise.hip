@@ -457,6 +457,94 @@ int launch_maxpool(zant_ctx *ctx, const T *x, const int64_t xdim[4], T *y, const
     return ZANT_OK;
 }
 
+// ---- average pool (pool_forward, .Avg: op_pooling.zig:373-408) -------------------------------------------------------
+// One thread per output: the sum of the window's taps that lie inside the input, in (row, column) order like the
+// reference, divided by their count -- or, with count_include_pad, by the number of taps inside the padded input.
+struct AvgGeom {
+    int64_t NC;
+    int H, W, OH, OW, kh, kw, sh, sw, pt, pl, pb, pr, include_pad;
+};
+
+__global__ void __launch_bounds__(kThreads) avgpool_f32_kernel(const float *__restrict__ x, float *__restrict__ y, AvgGeom g) {
+    const int64_t total = g.NC * g.OH * g.OW;
+    const int64_t step = int64_t(gridDim.x) * blockDim.x;
+    for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += step) {
+        const int ow = int(i % g.OW);
+        const int oh = int((i / g.OW) % g.OH);
+        const int64_t nc = i / (int64_t(g.OW) * g.OH);
+        const float *src = x + nc * g.H * g.W;
+        const int ih0 = oh * g.sh - g.pt, iw0 = ow * g.sw - g.pl;
+        float sum = 0.0f;
+        for (int kr = 0; kr < g.kh; ++kr) {
+            const int ih = ih0 + kr;
+            if (ih < 0 || ih >= g.H) continue;
+            for (int kc = 0; kc < g.kw; ++kc) {
+                const int iw = iw0 + kc;
+                if (iw >= 0 && iw < g.W) sum += src[ih * g.W + iw];
+            }
+        }
+        // taps inside the input / inside the padded input: products of the row and column overlaps
+        const int rows_in = min(ih0 + g.kh, g.H) - max(ih0, 0), cols_in = min(iw0 + g.kw, g.W) - max(iw0, 0);
+        const int rows_pad = min(ih0 + g.kh, g.H + g.pb) - ih0, cols_pad = min(iw0 + g.kw, g.W + g.pr) - iw0;
+        const int cnt = g.include_pad ? rows_pad * cols_pad : max(rows_in, 0) * max(cols_in, 0);
+        y[i] = cnt > 0 ? sum / float(cnt) : 0.0f;
+    }
+}
+
+// 2x2 / stride 2, no padding: each thread produces two outputs of one row from two 16-byte row segments.
+__global__ void __launch_bounds__(kThreads) avgpool_2x2s2_f32_kernel(const float *__restrict__ x, float *__restrict__ y, AvgGeom g,
+                                                                     int64_t total2) {
+    const int ow2 = g.OW >> 1;
+    const int64_t step = int64_t(gridDim.x) * blockDim.x;
+    for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < total2; i += step) {
+        const int c = int(i % ow2);
+        const int64_t row = i / ow2;            // (nc, oh)
+        const int oh = int(row % g.OH);
+        const int64_t nc = row / g.OH;
+        const float *src = x + (nc * g.H + 2 * oh) * g.W + 4 * c;
+        const float4 a = *reinterpret_cast<const float4 *>(src), b = *reinterpret_cast<const float4 *>(src + g.W);
+        float2 o;
+        o.x = (((a.x + a.y) + b.x) + b.y) / 4.0f;  // the reference's tap order: (0,0), (0,1), (1,0), (1,1)
+        o.y = (((a.z + a.w) + b.z) + b.w) / 4.0f;
+        *reinterpret_cast<float2 *>(y + row * g.OW + 2 * c) = o;
+    }
+}
+
+// ---- BatchNormalization, inference form (BatchNormLayer.forward, batchNormLayer.zig:130-148) -------------------------
+// y = (x - mean[f]) / sqrt(var[f] + eps) * gamma[f] + beta[f] in the reference's order of operations; f = the index on
+// axis 1, `inner` elements per (batch, feature) pair.
+__global__ void __launch_bounds__(kThreads) batchnorm_f32_kernel(const float *__restrict__ x, float *__restrict__ y,
+                                                                 const float *__restrict__ gamma, const float *__restrict__ beta,
+                                                                 const float *__restrict__ mean, const float *__restrict__ var,
+                                                                 float eps, int64_t total, int64_t inner, int features) {
+    const int64_t step = int64_t(gridDim.x) * blockDim.x;
+    for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += step) {
+        const int f = int((i / inner) % features);
+        const float sd = sqrtf(var[f] + eps);
+        const float xn = (x[i] - mean[f]) / sd;
+        y[i] = xn * gamma[f] + beta[f];
+    }
+}
+// inner a multiple of 4 and 16-byte aligned pointers: one feature per vector
+__global__ void __launch_bounds__(kThreads) batchnorm_vec_f32_kernel(const float *__restrict__ x, float *__restrict__ y,
+                                                                     const float *__restrict__ gamma, const float *__restrict__ beta,
+                                                                     const float *__restrict__ mean, const float *__restrict__ var,
+                                                                     float eps, int64_t total4, int64_t inner4, int features) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    const f4 *x4 = reinterpret_cast<const f4 *>(x);
+    f4 *y4 = reinterpret_cast<f4 *>(y);
+    const int64_t step = int64_t(gridDim.x) * blockDim.x;
+    for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < total4; i += step) {
+        const int f = int((i / inner4) % features);
+        const float sd = sqrtf(var[f] + eps), m = mean[f], ga = gamma[f], be = beta[f];
+        const f4 v = __builtin_nontemporal_load(x4 + i);
+        f4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = (v[e] - m) / sd * ga + be;
+        __builtin_nontemporal_store(o, y4 + i);
+    }
+}
+
 }  // namespace
 
 // -------------------------------------------------------------------------------------------------
@@ -651,5 +739,93 @@ extern "C" int zant_hip_maxpool2d_out_shape(const int64_t xdim[4], const int64_t
         ydim[3] = (W + pw - ekw) / strides[1] + 1;
     }
     ydim[0] = xdim[0]; ydim[1] = xdim[1];
+    return ZANT_OK;
+}
+
+// AveragePool: pool_forward with PoolingType.Avg (op_pooling.zig:223-260, 373-408), plus ONNX AveragePool's pads and
+// count_include_pad.
+extern "C" int zant_hip_avgpool2d_f32(zant_ctx *ctx, const float *x, const int64_t xdim[4], float *y, const int64_t ydim[4],
+                                      const int64_t kernel[2], const int64_t strides[2], const int64_t pads[4],
+                                      int count_include_pad) {
+    if (!ctx || !xdim || !ydim || !kernel || !strides) return ZANT_NullPointer;
+    for (int i = 0; i < 4; ++i)
+        if (xdim[i] < 0 || ydim[i] < 0 || xdim[i] > INT32_MAX || ydim[i] > INT32_MAX) return ZANT_InvalidDimensions;
+    if (kernel[0] <= 0 || kernel[1] <= 0 || strides[0] <= 0 || strides[1] <= 0) return ZANT_InvalidDimensions;  // :233-236
+    if (kernel[0] > INT32_MAX / 4 || kernel[1] > INT32_MAX / 4 || strides[0] > INT32_MAX / 4 || strides[1] > INT32_MAX / 4)
+        return ZANT_InvalidDimensions;
+    if (ydim[0] != xdim[0] || ydim[1] != xdim[1]) return ZANT_InvalidDimensions;
+    AvgGeom g;
+    g.pt = g.pl = g.pb = g.pr = 0;
+    if (pads) {
+        for (int i = 0; i < 4; ++i)
+            if (pads[i] < 0 || pads[i] >= (i & 1 ? kernel[1] : kernel[0])) return ZANT_InvalidPadding;
+        g.pt = int(pads[0]); g.pl = int(pads[1]); g.pb = int(pads[2]); g.pr = int(pads[3]);
+    }
+    // every window must start inside the input or its top / left padding
+    if (ydim[2] > 0 && (ydim[2] - 1) * strides[0] - g.pt >= xdim[2]) return ZANT_InvalidDimensions;
+    if (ydim[3] > 0 && (ydim[3] - 1) * strides[1] - g.pl >= xdim[3]) return ZANT_InvalidDimensions;
+    g.NC = xdim[0] * xdim[1];
+    g.H = int(xdim[2]); g.W = int(xdim[3]); g.OH = int(ydim[2]); g.OW = int(ydim[3]);
+    g.kh = int(kernel[0]); g.kw = int(kernel[1]); g.sh = int(strides[0]); g.sw = int(strides[1]);
+    g.include_pad = count_include_pad != 0;
+    const int64_t total = g.NC * g.OH * g.OW;
+    if (total == 0) return ZANT_OK;
+    if (!x || !y) return ZANT_NullPointer;
+    const bool fast = g.kh == 2 && g.kw == 2 && g.sh == 2 && g.sw == 2 && !g.pt && !g.pl && 2 * g.OH <= g.H && 2 * g.OW <= g.W &&
+                      g.OW % 2 == 0 && g.W % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 8 == 0;
+    KernelTimer kt(ctx);
+    if (fast) {
+        const int64_t total2 = total / 2;
+        hipLaunchKernelGGL(avgpool_2x2s2_f32_kernel, dim3(grid_for(total2, kThreads, ctx->num_cus)), dim3(kThreads), 0, ctx->stream, x,
+                           y, g, total2);
+    } else {
+        hipLaunchKernelGGL(avgpool_f32_kernel, dim3(grid_for(total, kThreads, ctx->num_cus)), dim3(kThreads), 0, ctx->stream, x, y, g);
+    }
+    ZANT_LAUNCH_CHECK(ctx);
+    return ZANT_OK;
+}
+
+// Output shape of an average pool: pool_forward's (H - k) / s + 1 (op_pooling.zig:239-240) over the padded input, with
+// ONNX AveragePool's ceil_mode (a last window that would start in the bottom / right padding is dropped).  Host only.
+extern "C" int zant_hip_avgpool2d_out_shape(const int64_t xdim[4], const int64_t kernel[2], const int64_t strides[2],
+                                            const int64_t pads[4], int ceil_mode, int64_t ydim[4]) {
+    if (!xdim || !kernel || !strides || !ydim) return ZANT_NullPointer;
+    if (kernel[0] <= 0 || kernel[1] <= 0 || strides[0] <= 0 || strides[1] <= 0) return ZANT_InvalidDimensions;
+    for (int ax = 0; ax < 2; ++ax) {
+        const int64_t lead = pads ? pads[ax] : 0, trail = pads ? pads[2 + ax] : 0;
+        const int64_t n = xdim[2 + ax] + lead + trail - kernel[ax];
+        if (lead < 0 || trail < 0) return ZANT_InvalidPadding;
+        if (n < 0) return ZANT_InvalidDimensions;  // :243-245
+        int64_t o = (ceil_mode ? (n + strides[ax] - 1) / strides[ax] : n / strides[ax]) + 1;
+        if (ceil_mode && (o - 1) * strides[ax] >= xdim[2 + ax] + lead) --o;
+        ydim[2 + ax] = o;
+    }
+    ydim[0] = xdim[0]; ydim[1] = xdim[1];
+    return ZANT_OK;
+}
+
+// BatchNormalization, inference form: features on axis 1; gamma / beta / mean / var are device arrays of xdim[1] floats.
+extern "C" int zant_hip_batchnorm_f32(zant_ctx *ctx, const float *x, const int64_t *xdim, int rank, const float *gamma,
+                                      const float *beta, const float *mean, const float *var, float epsilon, float *y) {
+    if (!ctx || !xdim) return ZANT_NullPointer;
+    if (rank < 2 || rank > 8) return ZANT_InvalidDimensions;
+    int64_t total = 1, inner = 1;
+    for (int i = 0; i < rank; ++i) {
+        if (xdim[i] < 0) return ZANT_InvalidDimensions;
+        total *= xdim[i];
+        if (i >= 2) inner *= xdim[i];
+    }
+    if (total == 0) return ZANT_OK;
+    if (xdim[1] > INT32_MAX) return ZANT_InvalidDimensions;
+    if (!x || !y || !gamma || !beta || !mean || !var) return ZANT_NullPointer;
+    KernelTimer kt(ctx);
+    if (inner % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0) {
+        hipLaunchKernelGGL(batchnorm_vec_f32_kernel, dim3(grid_for(total / 4, kThreads, ctx->num_cus)), dim3(kThreads), 0, ctx->stream,
+                           x, y, gamma, beta, mean, var, epsilon, total / 4, inner / 4, int(xdim[1]));
+    } else {
+        hipLaunchKernelGGL(batchnorm_f32_kernel, dim3(grid_for(total, kThreads, ctx->num_cus)), dim3(kThreads), 0, ctx->stream, x, y,
+                           gamma, beta, mean, var, epsilon, total, inner, int(xdim[1]));
+    }
+    ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
 }

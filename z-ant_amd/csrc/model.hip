@@ -14,6 +14,7 @@
 // run() then enqueues the operator kernels on arena pointers: no allocation, no memset (every
 // kernel writes its whole output).
 #include <algorithm>
+#include <cmath>
 #include <vector>
 
 #include "common.h"
@@ -24,7 +25,7 @@ namespace {
 enum OpKind {
     OP_CONV, OP_RELU, OP_LEAKY, OP_MAXPOOL, OP_RESHAPE, OP_GEMM, OP_MATMUL, OP_ADD_CONST, OP_ADD, OP_SOFTMAX,
     OP_QUANT, OP_DEQUANT, OP_QCONV, OP_QACT, OP_QADD, OP_QGAP, OP_QBLOCK,
-    OP_SIGMOID, OP_REDUCE_MEAN, OP_CONCAT, OP_RESIZE
+    OP_SIGMOID, OP_REDUCE_MEAN, OP_CONCAT, OP_RESIZE, OP_AVGPOOL, OP_BATCHNORM
 };
 
 struct MTensor {
@@ -220,6 +221,14 @@ int run_node(zant_model *m, const MNode &nd) {
                                          nd.kernel, nd.stride, nd.dil, nd.pads, 4, nd.pool_pad);
         return zant_hip_maxpool2d_f32(ctx, static_cast<const float *>(x), ti.dim, static_cast<float *>(y), to.dim, nd.kernel,
                                       nd.stride, nd.dil, nd.pads, 4, nd.pool_pad);
+    case OP_AVGPOOL:
+        return zant_hip_avgpool2d_f32(ctx, static_cast<const float *>(x), ti.dim, static_cast<float *>(y), to.dim, nd.kernel,
+                                      nd.stride, nd.pads, nd.keepdims /* count_include_pad */);
+    case OP_BATCHNORM:
+        return zant_hip_batchnorm_f32(ctx, static_cast<const float *>(x), ti.dim, ti.rank,
+                                      static_cast<const float *>(param_ptr(m, nd.w)), static_cast<const float *>(param_ptr(m, nd.b)),
+                                      static_cast<const float *>(param_ptr(m, nd.c)), static_cast<const float *>(param_ptr(m, nd.ws)),
+                                      nd.alpha /* epsilon */, static_cast<float *>(y));
     case OP_GEMM:
         return zant_hip_gemm_f32(ctx, static_cast<const float *>(x), ti.dim, static_cast<const float *>(param_ptr(m, nd.w)),
                                  nd.wdim, static_cast<const float *>(param_ptr(m, nd.c)), nd.cdim, nd.c_rank, nd.alpha,
@@ -402,6 +411,43 @@ extern "C" int zant_model_maxpool(zant_model *m, int x, const int64_t kernel[2],
     return append(m, nd, tx.dtype, ydim, 4, tx.scale, tx.zp);
 }
 
+extern "C" int zant_model_avgpool(zant_model *m, int x, const int64_t kernel[2], const int64_t strides[2],
+                                  const int64_t pads[4], int ceil_mode, int count_include_pad) {
+    if (!valid_tensor(m, x) || !kernel || !strides) return ZANT_NullPointer;
+    const MTensor tx = m->t[x];
+    if (tx.rank != 4) return ZANT_InputTensorDimensionMismatch;  // op_pooling.zig:229-231
+    if (tx.dtype != ZANT_F32) return ZANT_InvalidInput;
+    int64_t ydim[4];
+    int rc = zant_hip_avgpool2d_out_shape(tx.dim, kernel, strides, pads, ceil_mode, ydim);
+    if (rc) return rc;
+    if (pads)
+        for (int i = 0; i < 4; ++i)
+            if (pads[i] >= (i & 1 ? kernel[1] : kernel[0])) return ZANT_InvalidPadding;
+    MNode nd;
+    nd.op = OP_AVGPOOL; nd.in0 = x;
+    nd.keepdims = count_include_pad != 0;  // (the field ReduceMean uses for its own flag)
+    for (int i = 0; i < 2; ++i) { nd.kernel[i] = kernel[i]; nd.stride[i] = strides[i]; }
+    for (int i = 0; i < 4; ++i) nd.pads[i] = pads ? pads[i] : 0;
+    return append(m, nd, ZANT_F32, ydim, 4, 1.0f, 0);
+}
+
+extern "C" int zant_model_batchnorm(zant_model *m, int x, const float *gamma, const float *beta, const float *mean,
+                                    const float *var, int64_t features, float epsilon) {
+    if (!valid_tensor(m, x) || !gamma || !beta || !mean || !var) return ZANT_NullPointer;
+    const MTensor tx = m->t[x];
+    if (tx.dtype != ZANT_F32) return ZANT_InvalidInput;
+    if (tx.rank < 2) return ZANT_InvalidDimensions;
+    if (features != tx.dim[1]) return ZANT_InputTensorDimensionMismatch;
+    MNode nd;
+    nd.op = OP_BATCHNORM; nd.in0 = x;
+    nd.alpha = epsilon;  // (the field Gemm uses for its own scalar)
+    nd.w = add_param(m, gamma, size_t(features) * 4);
+    nd.b = add_param(m, beta, size_t(features) * 4);
+    nd.c = add_param(m, mean, size_t(features) * 4);
+    nd.ws = add_param(m, var, size_t(features) * 4);
+    return append(m, nd, ZANT_F32, tx.dim, tx.rank, 1.0f, 0);
+}
+
 extern "C" int zant_model_reshape(zant_model *m, int x, const int64_t *new_shape, int rank) {
     if (!valid_tensor(m, x) || !new_shape) return ZANT_NullPointer;
     if (rank < 1 || rank > 8) return ZANT_InvalidInput;
@@ -423,6 +469,9 @@ extern "C" int zant_model_gemm(zant_model *m, int a, const float *b, const int64
     int64_t ydim[4];
     int rc = zant_hip_gemm_check(ta.dim, ta.rank, bdim, 4, cdim, c_rank, c != nullptr, trans_a, trans_b, ydim);
     if (rc) return rc;
+    // lean_gemm multiplies the first matrix only and leaves the other planes of the (zero filled) result alone
+    // (op_gemm.zig:126-128, op_mat_mul.zig:95-97); the arena is not zero filled per pass, so batched shapes are refused
+    if (ta.dim[0] * ta.dim[1] != 1) return ZANT_InvalidInput;
     MNode nd;
     nd.op = OP_GEMM; nd.in0 = a;
     for (int i = 0; i < 4; ++i) nd.wdim[i] = bdim[i];
@@ -651,18 +700,52 @@ extern "C" int zant_model_finalize(zant_model *m) {
             for (int k = 0; k < ad.c_rank; ++k) cnt *= ad.cdim[k];
             const bool per_channel = cnt == nd.wdim[0] &&
                                      ((ad.c_rank == 3 && ad.cdim[0] == nd.wdim[0]) || (ad.c_rank == 4 && ad.cdim[1] == nd.wdim[0]) ||
-                                      (ad.c_rank == 1 && m->t[nd.out].dim[3] == 1 && m->t[nd.out].dim[2] == 1));
+                                      // {M} broadcasts against the LAST axis: a per-channel bias only for a [1, M, 1, 1]
+                                      // result, where the Add is an equal-size flat add and keeps the shape
+                                      (ad.c_rank == 1 && m->t[nd.out].dim[3] == 1 && m->t[nd.out].dim[2] == 1 &&
+                                       m->t[nd.out].dim[0] == 1 && m->t[ad.out].rank == m->t[nd.out].rank &&
+                                       m->t[ad.out].bytes() == m->t[nd.out].bytes()));
             if (per_channel) {
                 nd.b = ad.c;
                 m->t[ad.out].alias_of = nd.out;
                 ad.skip = true;
             }
         }
+        if (nd.op == OP_CONV) {
+            // Conv (-> folded Add) -> BatchNormalization that nothing else reads the input of: the normalisation is a
+            // per-channel scale and shift, folded into the weights and the bias on the host:
+            //   w'[k] = w[k] * s[k],  b'[k] = (b[k] - mean[k]) * s[k] + beta[k],  s[k] = gamma[k] / sqrt(var[k] + eps)
+            int out = nd.out, c1 = -1;
+            while (consumers(m, out, &c1) == 1 && m->n[c1].skip && m->n[c1].op == OP_ADD_CONST) out = m->n[c1].out;
+            if (consumers(m, out, &only) == 1 && m->n[only].op == OP_BATCHNORM && !m->n[only].skip && m->n[only].in0 == out &&
+                m->t[out].rank == 4 && out != m->output) {
+                MNode &bn = m->n[only];
+                const int64_t K = nd.wdim[0], per_k = nd.wdim[1] * nd.wdim[2] * nd.wdim[3];
+                float *w = reinterpret_cast<float *>(m->p[nd.w].host.data());
+                const float *ga = reinterpret_cast<const float *>(m->p[bn.w].host.data());
+                const float *be = reinterpret_cast<const float *>(m->p[bn.b].host.data());
+                const float *mu = reinterpret_cast<const float *>(m->p[bn.c].host.data());
+                const float *va = reinterpret_cast<const float *>(m->p[bn.ws].host.data());
+                std::vector<float> bias(size_t(K), 0.0f);
+                if (nd.b >= 0) memcpy(bias.data(), m->p[nd.b].host.data(), size_t(K) * 4);
+                for (int64_t k = 0; k < K; ++k) {
+                    const float sc = ga[k] / sqrtf(va[k] + bn.alpha);
+                    for (int64_t e = 0; e < per_k; ++e) w[k * per_k + e] *= sc;
+                    bias[size_t(k)] = (bias[size_t(k)] - mu[k]) * sc + be[k];
+                }
+                nd.b = add_param(m, bias.data(), size_t(K) * 4);  // (a bias shared with another node keeps its own copy)
+                m->t[bn.out].alias_of = out;
+                bn.skip = true;
+            }
+        }
         if ((nd.op == OP_CONV || nd.op == OP_GEMM) && nd.fuse_act == ZANT_ACT_NONE) {
             int out = nd.out;
             // look through an Add that was just folded
             int c1 = -1;
-            while (consumers(m, out, &c1) == 1 && m->n[c1].skip && m->n[c1].op == OP_ADD_CONST) out = m->n[c1].out;
+            // ... or a normalisation, and through Reshape views (ReLU is elementwise: the view's shape does not matter)
+            while (consumers(m, out, &c1) == 1 &&
+                   ((m->n[c1].skip && (m->n[c1].op == OP_ADD_CONST || m->n[c1].op == OP_BATCHNORM)) || m->n[c1].op == OP_RESHAPE))
+                out = m->n[c1].out;
             if (consumers(m, out, &only) == 1 && m->n[only].op == OP_RELU && !m->n[only].skip) {
                 nd.fuse_act = ZANT_ACT_RELU;
                 m->t[m->n[only].out].alias_of = out;
@@ -686,7 +769,8 @@ extern "C" int zant_model_finalize(zant_model *m) {
         if (nd.op == OP_CONV) {
             // Conv (+ReLU) -> MaxPool 2x2/2: one kernel, pooled output only (where the convolution kernels take the shape)
             int out = nd.out, c1 = -1;
-            while (consumers(m, out, &c1) == 1 && m->n[c1].skip && (m->n[c1].op == OP_ADD_CONST || m->n[c1].op == OP_RELU))
+            while (consumers(m, out, &c1) == 1 && m->n[c1].skip &&
+                   (m->n[c1].op == OP_ADD_CONST || m->n[c1].op == OP_RELU || m->n[c1].op == OP_BATCHNORM))
                 out = m->n[c1].out;
             if (consumers(m, out, &only) == 1 && m->n[only].op == OP_MAXPOOL && !m->n[only].skip) {
                 MNode &pn = m->n[only];
@@ -710,7 +794,9 @@ extern "C" int zant_model_finalize(zant_model *m) {
             }
         }
         if (nd.op == OP_QCONV && nd.fuse_act == ZANT_ACT_NONE && consumers(m, nd.out, &only) == 1 &&
-            m->n[only].op == OP_QACT && !m->n[only].skip) {
+            m->n[only].op == OP_QACT && !m->n[only].skip && m->n[only].act != ZANT_ACT_NONE) {
+            // (a plain requantisation node, act == none, stays a node of its own: fused, the kernel would take the
+            // activation's parameters for its first stage and skip the rounding and saturation of the intermediate u8)
             // the activation's output parameters become the kernel's second requantisation stage
             const MNode &an = m->n[only];
             const MTensor &ao = m->t[an.out];
@@ -932,7 +1018,9 @@ extern "C" int zant_model_finalize(zant_model *m) {
         for (int in : nd.more) { const int r = root_of(m, in); m->t[r].last = std::max(m->t[r].last, i + 1); }
     }
     m->t[root_of(m, m->output)].last = nn + 1;  // the output outlives the pass
-    m->t[root_of(m, m->input)].last = std::max(m->t[root_of(m, m->input)].last, 1);
+    // The input keeps its storage for the whole pass: a caller that uploads it once to zant_model_input_ptr() may run
+    // the model any number of times (the reference's predict() copies its input on every call, predict.zig:339-366)
+    m->t[root_of(m, m->input)].last = nn + 1;
     struct Placed { size_t off, size; int def, last; };
     std::vector<Placed> placed;
     size_t arena = 0;
@@ -1085,6 +1173,8 @@ const char *op_name(const MNode &nd) {
     case OP_REDUCE_MEAN: return "ReduceMean";
     case OP_CONCAT: return "Concat";
     case OP_RESIZE: return "Resize";
+    case OP_AVGPOOL: return "AveragePool";
+    case OP_BATCHNORM: return "BatchNormalization";
     case OP_QUANT: return "QuantizeLinear";
     case OP_DEQUANT: return "DequantizeLinear";
     case OP_QCONV:
@@ -1185,6 +1275,19 @@ extern "C" int zant_model_read_tensor(zant_model *m, int id, void *dst_host, siz
     if (bytes > m->t[id].bytes()) return ZANT_InvalidDimensions;
     if (m->t[root_of(m, id)].def < 0) return ZANT_InvalidInput;  // fused away: the tensor is never materialised
     const MTensor &t = m->t[id];
+    // A later node may have been planned over this tensor's storage once its last reader was done, so the pass is
+    // replayed up to the node that produces it (the input still sits in its slot: a pass never writes there).
+    {
+        const int root = root_of(m, id);
+        int last_writer = -1;
+        for (int i = 0; i < int(m->n.size()); ++i)
+            if (!m->n[i].skip && root_of(m, m->n[i].out) == root) last_writer = i;
+        for (int i = 0; i <= last_writer; ++i) {
+            if (m->n[i].skip) continue;
+            const int rc = run_node(m, m->n[i]);
+            if (rc) return rc;
+        }
+    }
     if (m->t[root_of(m, id)].layout == ZANT_LAYOUT_BLOCKED16) {  // hand out NCHW u8 like everywhere outside the executor
         void *ws = nullptr;
         int rc = zant_workspace(m->ctx, t.bytes(), &ws);

@@ -65,12 +65,29 @@ class Model:
         k, _ = dims(kernel); s, _ = dims(strides); d, _ = dims(dilations); p, _ = dims(pads)
         return self._id(self._lib.zant_model_maxpool(self.handle, x, k, s, d, p, PAD[auto_pad], int(ceil_mode)))
 
+    def avgpool(self, x, kernel, strides, pads=None, ceil_mode=False, count_include_pad=False):
+        k, _ = dims(kernel); s, _ = dims(strides); p, _ = dims(pads)
+        return self._id(self._lib.zant_model_avgpool(self.handle, x, k, s, p, int(ceil_mode), int(count_include_pad)))
+
+    def batchnorm(self, x, gamma, beta, mean, var, epsilon=1e-5):
+        g, b, mu, v = (_np(np.asarray(a).reshape(-1), np.float32) for a in (gamma, beta, mean, var))
+        if not (g.size == b.size == mu.size == v.size):
+            raise ZantError(-5)
+        return self._id(self._lib.zant_model_batchnorm(self.handle, x, _hp(g), _hp(b), _hp(mu), _hp(v), g.size, epsilon))
+
     def reshape(self, x, new_shape):
         d, r = dims(new_shape)
         return self._id(self._lib.zant_model_reshape(self.handle, x, d, r))
 
     def gemm(self, a, b, c=None, alpha=1.0, beta=1.0, trans_a=False, trans_b=False):
+        """gemm_lean: A (a rank-4 tensor {1, 1, rows, cols}), B and C in the reference's rank-4 form; B and C of lower
+        rank are given leading ones (the C side reads four B dimensions)."""
         b = _np(b, np.float32); c = _np(c, np.float32)
+        if b.ndim > 4 or (c is not None and c.ndim > 4):
+            raise ZantError(-3)
+        b = b.reshape((1,) * (4 - b.ndim) + b.shape)
+        if c is not None:
+            c = c.reshape((1,) * (4 - c.ndim) + c.shape)
         bd, _ = dims(b.shape); cd, cr = dims(None if c is None else c.shape)
         return self._id(self._lib.zant_model_gemm(self.handle, a, _hp(b), bd, _hp(c), cd, cr, alpha, beta, int(trans_a), int(trans_b)))
 

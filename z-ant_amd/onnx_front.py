@@ -3,7 +3,7 @@ package), folds Reshape on initialisers, and builds a ``Model`` (the executor be
 
 The reference parses ONNX in Zig (src/onnx/protobuf.zig:31-203, src/onnx/onnx.zig) and turns each node into one
 ``tensMath.*_lean`` call (src/codeGen/math_handler.zig:31-108); this does the same for Conv, Add, Relu, LeakyRelu,
-MaxPool, Reshape, MatMul, Gemm and Softmax, which covers the bundled mnist-8 network, and for quantised graphs in
+MaxPool, AveragePool, BatchNormalization, Reshape, MatMul, Gemm and Softmax, which covers the bundled mnist-8 network, and for quantised graphs in
 operator form: QuantizeLinear, DequantizeLinear, QLinearConv, MaxPool on u8, QLinearAdd and
 QLinearGlobalAveragePool (com.microsoft), and the activation idiom DequantizeLinear -> Relu | LeakyRelu | Clip(0, 6)
 -> QuantizeLinear, which becomes one quantised activation node (the executor then folds it into the convolution).
@@ -184,6 +184,11 @@ def _pool_or_conv_attrs(a, rank2_default):
     return strides, pads, dil, auto_pad
 
 
+def _lift4(arr):
+    """An ONNX Gemm operand in the reference's rank-4 form: leading ones."""
+    return arr.reshape((1,) * (4 - arr.ndim) + arr.shape)
+
+
 def run_graph(graph, ops, x):
     """Executes the graph with ``ops`` (an object with the reference-named operators: the CPU oracle module, or any
     other implementation with the same signatures) on the numpy input ``x``.  Used by tests as the checker's driver."""
@@ -203,10 +208,23 @@ def run_graph(graph, ops, x):
         elif nd["op"] == "MaxPool":
             s, p, d, ap = _pool_or_conv_attrs(a, [1, 1])
             y = ops.onnx_maxpool(i[0], a["kernel_shape"], s, d, p if p is not None else [0, 0, 0, 0], ap)
+        elif nd["op"] == "AveragePool":
+            s, p, _, ap = _pool_or_conv_attrs(a, [1, 1])
+            y = ops.avgpool(i[0], a["kernel_shape"], s, p if p is not None else [0, 0, 0, 0], bool(a.get("ceil_mode", 0)),
+                            bool(a.get("count_include_pad", 0)))
+        elif nd["op"] == "BatchNormalization":
+            y = ops.batchnorm(i[0], i[1], i[2], i[3], i[4], a.get("epsilon", 1e-5))
         elif nd["op"] == "Reshape":
             y = ops.reshape_lean(i[0], [int(v) for v in i[1]])
         elif nd["op"] == "MatMul":
             y = ops.mat_mul(i[0], i[1])
+        elif nd["op"] == "Gemm":
+            # the reference's gemm takes {1, 1, rows, cols} tensors (op_gemm.zig:22-27): ONNX's 2-D operands are lifted
+            a4, b4 = _lift4(i[0]), _lift4(i[1])
+            c4 = _lift4(i[2]) if len(i) > 2 else None
+            y = ops.gemm(a4, b4, c4, a.get("alpha", 1.0), a.get("beta", 1.0), bool(a.get("transA", 0)), bool(a.get("transB", 0)))
+            if i[0].ndim == 2:
+                y = y.reshape(y.shape[2], y.shape[3])
         elif nd["op"] == "Softmax":
             y = ops.softmax(i[0])
         elif nd["op"] == "Sigmoid":
@@ -324,14 +342,32 @@ def build_model(ctx, graph, model=None):
                           bool(a.get("ceil_mode", 0)))
             if ins[0] in qparams:
                 qparams[out] = qparams[ins[0]]
+        elif op == "AveragePool":
+            s, p, d, ap = _pool_or_conv_attrs(a, [1, 1])
+            if ap != "NOTSET" or any(v != 1 for v in d):
+                raise NotImplementedError("AveragePool with auto_pad or dilations")
+            t = m.avgpool(tens[ins[0]], a["kernel_shape"], s, p, bool(a.get("ceil_mode", 0)), bool(a.get("count_include_pad", 0)))
+        elif op == "BatchNormalization":
+            if a.get("training_mode", 0) or len(nd["outputs"]) > 1:
+                raise NotImplementedError("BatchNormalization in training mode")
+            t = m.batchnorm(tens[ins[0]], consts[ins[1]], consts[ins[2]], consts[ins[3]], consts[ins[4]], a.get("epsilon", 1e-5))
         elif op == "Reshape":
             t = m.reshape(tens[ins[0]], [int(v) for v in consts[ins[1]]])
         elif op == "MatMul":
             t = m.matmul(tens[ins[0]], consts[ins[1]].astype(np.float32))
         elif op == "Gemm":
+            # gemm_lean works on {1, 1, rows, cols} tensors (op_gemm.zig:22-27, 52-60): a 2-D A is viewed as such, B and
+            # C get leading ones, and the result is viewed back as ONNX's (M, N)
             c = consts[ins[2]].astype(np.float32) if len(ins) > 2 and ins[2] else None
-            t = m.gemm(tens[ins[0]], consts[ins[1]].astype(np.float32), c, a.get("alpha", 1.0), a.get("beta", 1.0),
+            a_id, a_shape = tens[ins[0]], m.tensor_shape(tens[ins[0]])
+            if len(a_shape) > 4 or len(a_shape) < 2:
+                raise NotImplementedError(f"Gemm with a rank-{len(a_shape)} input")
+            if len(a_shape) < 4:
+                a_id = m.reshape(a_id, [1] * (4 - len(a_shape)) + list(a_shape))
+            t = m.gemm(a_id, consts[ins[1]].astype(np.float32), c, a.get("alpha", 1.0), a.get("beta", 1.0),
                        bool(a.get("transA", 0)), bool(a.get("transB", 0)))
+            if len(a_shape) < 4:
+                t = m.reshape(t, list(m.tensor_shape(t))[4 - len(a_shape):])
         elif op == "Softmax":
             t = m.softmax(tens[ins[0]])
         elif op == "Sigmoid":

@@ -158,6 +158,45 @@ def onnx_maxpool(x, kernel, strides, dilations, pads, auto_pad="NOTSET", ceil_mo
     return onnx_maxpool_lean(x, y, kernel, strides, dilations, pads, auto_pad)
 
 
+def get_avgpool_output_shape(xshape, kernel, strides, pads=None, ceil_mode=False):
+    xd, _ = dims(xshape); k, _ = dims(kernel); s, _ = dims(strides); p, _ = dims(pads)
+    out = (C.c_int64 * 4)()
+    rc = lib.zant_hip_avgpool2d_out_shape(xd, k, s, p, int(ceil_mode), out)
+    if rc:
+        raise ZantError(rc)
+    return tuple(out)
+
+
+def avgpool_lean(x, y, kernel, strides, pads=None, count_include_pad=False):
+    """pool_forward with PoolingType.Avg (op_pooling.zig:223-260, 373-408) into a pre-shaped output."""
+    if x.dim() != 4:
+        raise ZantError(-5)
+    ctx = context()
+    xd, _ = dims(x.shape); yd, _ = dims(y.shape); k, _ = dims(kernel); s, _ = dims(strides); p, _ = dims(pads)
+    ctx.check(lib.zant_hip_avgpool2d_f32(ctx.handle, _p(x), xd, _p(y), yd, k, s, p, int(count_include_pad)))
+    return y
+
+
+def avgpool(x, kernel, strides, pads=None, ceil_mode=False, count_include_pad=False):
+    if x.dim() != 4:
+        raise ZantError(-5)
+    y = torch.zeros(get_avgpool_output_shape(x.shape, kernel, strides, pads, ceil_mode), dtype=torch.float32, device=x.device)
+    return avgpool_lean(x, y, kernel, strides, pads, count_include_pad)
+
+
+def batchnorm(x, gamma, beta, mean, var, epsilon=1e-5):
+    """BatchNormLayer.forward, inference branch (batchNormLayer.zig:130-148), features on axis 1."""
+    if x.dim() < 2:
+        raise ZantError(-1)
+    if not (gamma.numel() == beta.numel() == mean.numel() == var.numel() == x.shape[1]):
+        raise ZantError(-5)
+    ctx = context()
+    xd, xr = dims(x.shape)
+    y = torch.zeros_like(x)
+    ctx.check(lib.zant_hip_batchnorm_f32(ctx.handle, _p(x), xd, xr, _p(gamma), _p(beta), _p(mean), _p(var), epsilon, _p(y)))
+    return y
+
+
 # ------------------------------------------------------------------------------------------ activations, add, reshape
 
 def ReLU_lean(x, y):
