@@ -60,3 +60,70 @@ def test_host_only_shape_functions():
                                  ([3, 3], [2, 2], [2, 1], [1, 1, 1, 1], "NOTSET", False)]:
         assert tm.get_onnx_maxpool_output_shape((1, 1, 9, 9), k, s, d, p, ap, ceil) == \
             zo.maxpool_out_shape((1, 1, 9, 9), k, s, d, p, ap, ceil)
+
+
+def _split_params(s):
+    """Top-level comma split of a parameter list (function-pointer parameters carry their own parentheses)."""
+    out, depth, cur = [], 0, ""
+    for ch in s:
+        if ch in "([":
+            depth += 1
+        elif ch in ")]":
+            depth -= 1
+        if ch == "," and depth == 0:
+            out.append(cur.strip())
+            cur = ""
+        else:
+            cur += ch
+    if cur.strip() and cur.strip() != "void":
+        out.append(cur.strip())
+    return out
+
+
+def _header_prototypes():
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    protos = {}
+    for m in re.finditer(r"\b(zant_hip_\w+|zant_model_\w+|setLogFunctionC|setLogFunction|predict_batched|predict)\s*\(((?:[^()]|\([^()]*\))*)\)\s*;", text):
+        protos[m.group(1)] = _split_params(m.group(2))
+    return protos
+
+
+def test_zig_binding_mirrors_the_header():
+    """bindings/zant_hip.zig (no Zig compiler here: a text check): one `extern fn` per function of the header with
+    the same number of parameters in the same order of names, and the reference's lean signatures verbatim."""
+    zig = open(os.path.join(ROOT, "bindings", "zant_hip.zig")).read()
+    externs = {m.group(1): _split_params(m.group(2))
+               for m in re.finditer(r"pub extern fn (\w+)\(((?:[^()]|\([^()]*\))*)\)", zig)}
+    protos = _header_prototypes()
+    assert sorted(protos) == declared_symbols()
+    assert sorted(externs) == sorted(protos)
+    rename = {"var": "variance"}  # `var` is a Zig keyword
+    for name, params in protos.items():
+        assert len(externs[name]) == len(params), name
+        for c_param, z_param in zip(params, externs[name]):
+            if "(*" in c_param:   # a function pointer: void (*func)(char *)
+                c_name = re.search(r"\(\*(\w+)\)", c_param).group(1)
+            else:
+                c_name = re.search(r"(\w+)(\[\d*\])?$", c_param).group(1)
+            assert z_param.split(":")[0].strip() == rename.get(c_name, c_name), (name, c_param, z_param)
+    lean = [  # tensor_math_standard.zig name, then the parameter list as the reference writes it
+        "pub fn conv_lean(comptime T: type, input: *Tensor(T), kernel: *Tensor(T), output: *Tensor(T), bias: ?*const Tensor(T), stride: []const usize, pads: ?[]const usize, dilations: ?[]const usize, group: ?usize, auto_pad: ?[]const u8) !void",
+        "pub fn gemm_lean(comptime T: anytype, A: *Tensor(T), B: *Tensor(T), C: ?*Tensor(T), alpha: T, beta: T, transA: bool, transB: bool, result: *Tensor(T)) !void",
+        "pub fn mat_mul_lean(comptime T: anytype, A: *const Tensor(T), B: *const Tensor(T), Y: *Tensor(T)) !void",
+        "pub fn onnx_maxpool_lean(comptime T: type, input: *Tensor(T), output: *Tensor(T), kernel_shape: []const usize, strides: []const usize, dilations: []const usize, pads: []const usize, auto_pad: AutoPadType) !void",
+        "pub fn ReLU_lean(comptime T: anytype, input_tensor: *Tensor(T), output_tensor: *Tensor(T)) !void",
+        "pub fn leakyReLU_lean(comptime T: anytype, input_tensor: *Tensor(T), slope: T, output_tensor: *Tensor(T)) !void",
+        "pub fn softmax_lean(comptime T: anytype, input: *Tensor(T), output: *Tensor(T)) !void",
+        "pub fn sum_tensors_lean(comptime inputType: anytype, comptime outputType: anytype, t1: *Tensor(inputType), t2: *Tensor(inputType), outputTensor: *Tensor(outputType)) !void",
+        "pub fn reshape_lean(comptime T: anytype, input: *Tensor(T), newShape: []const usize, allowZero: ?bool, output: *Tensor(T)) !void",
+        "pub fn sigmoid_lean(comptime T: anytype, input_tensor: *Tensor(T), output_tensor: *Tensor(T)) !void",
+        "pub fn reduce_mean_lean(comptime T: anytype, input_tensor: *Tensor(T), output_tensor: *Tensor(T), axes: ?[]const i64, _: bool, noop_with_empty_axes: bool) !void",
+        "pub fn lean_concatenate(comptime T: type, allocator: *const std.mem.Allocator, tensors: []const Tensor(T), axis: isize, output: *Tensor(T)) !void",
+    ]
+    for sig in lean:
+        assert sig in zig, sig
+    # every status the header names maps to an error (or to the catch-all for HIP / memory failures)
+    header = open(HEADER).read()
+    for code in re.findall(r"ZANT_\w+ = (-\d+),", header):
+        if int(code) > -100 and int(code) != -13:
+            assert f"        {code} => " in zig, code
