@@ -61,6 +61,7 @@ pub extern fn zant_hip_timer_start(ctx: ?*zant_ctx) c_int;
 pub extern fn zant_hip_timer_stop(ctx: ?*zant_ctx, elapsed_ms: *f32) c_int;
 pub extern fn zant_hip_kernel_timing(ctx: ?*zant_ctx, enable: c_int) c_int;
 pub extern fn zant_hip_kernel_ms(ctx: ?*zant_ctx, elapsed_ms: *f32) c_int;
+pub extern fn zant_hip_kernel_name(ctx: ?*zant_ctx) [*:0]const u8;
 
 // f32 operators
 pub extern fn zant_hip_conv2d_f32(ctx: ?*zant_ctx, x: [*]const f32, xdim: *const [4]i64, w: [*]const f32, wdim: *const [4]i64, bias: ?[*]const f32, y: [*]f32, ydim: *const [4]i64, stride: [*]const i64, n_stride: c_int, pads: ?[*]const i64, n_pads: c_int, dil: ?[*]const i64, n_dil: c_int, group: i64, auto_pad: ?[*:0]const u8, fuse_act: c_int) c_int;
@@ -136,6 +137,7 @@ pub extern fn zant_model_output_ptr(m: ?*zant_model) ?*anyopaque;
 pub extern fn zant_model_predict_host(m: ?*zant_model, input_host: ?*const anyopaque, output_host: ?*anyopaque) c_int;
 pub extern fn zant_model_profile(m: ?*zant_model, ms: [*]f32, ops: [*]f64, bytes: [*]f64, capacity: c_int) c_int;
 pub extern fn zant_model_launch_name(m: ?*zant_model, i: c_int) [*:0]const u8;
+pub extern fn zant_model_launch_kernel(m: ?*zant_model, i: c_int) [*:0]const u8;
 pub extern fn zant_model_read_tensor(m: ?*zant_model, id: c_int, dst_host: ?*anyopaque, bytes: usize) c_int;
 pub extern fn zant_model_bind_predict(m: ?*zant_model) c_int;
 pub extern fn predict(input: [*]f32, input_shape: [*]u32, shape_len: u32, result: *[*]f32) void;

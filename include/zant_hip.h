@@ -105,6 +105,10 @@ int zant_hip_timer_stop(zant_ctx *ctx, float *elapsed_ms);
  * the most recent one and returns its duration.  Off by default (two event records per call). */
 int zant_hip_kernel_timing(zant_ctx *ctx, int enable);
 int zant_hip_kernel_ms(zant_ctx *ctx, float *elapsed_ms);
+/* The device function of the most recent operator's main kernel as a profiler's kernel trace names it, with its
+ * template arguments (e.g. "conv_f32_mfma_kernel<4,2,2,4,9,true>"); "" where the launch site does not say.  The
+ * string lives in the context and changes with the next operator call. */
+const char *zant_hip_kernel_name(zant_ctx *ctx);
 
 /* ---- f32 operators ------------------------------------------------------------ */
 
@@ -363,6 +367,8 @@ int zant_model_predict_host(zant_model *m, const void *input_host, void *output_
  * "Conv+Relu+MaxPool". */
 int zant_model_profile(zant_model *m, float *ms, double *ops, double *bytes, int capacity);
 const char *zant_model_launch_name(zant_model *m, int i);
+/* The device function behind entry i of the last zant_model_profile (see zant_hip_kernel_name); "" before it. */
+const char *zant_model_launch_kernel(zant_model *m, int i);
 /* Debug: copies tensor `id` to the host: replays the last pass up to the node that produces it (its storage may have
  * been planned under a later tensor), then reads it from the arena.  Tensors that a fusion removed (the
  * output of a convolution whose pool, or of a residual block's inner layers, run in the same kernel) are never

@@ -43,6 +43,7 @@ PROTOTYPES = {
     "zant_hip_timer_stop": (i32, [vp, C.POINTER(f32)]),
     "zant_hip_kernel_timing": (i32, [vp, i32]),
     "zant_hip_kernel_ms": (i32, [vp, C.POINTER(f32)]),
+    "zant_hip_kernel_name": (C.c_char_p, [vp]),
     "zant_hip_conv2d_f32": (i32, [vp, vp, c_i64p, vp, c_i64p, vp, vp, c_i64p, c_i64p, i32, c_i64p, i32, c_i64p, i32,
                                   i64, C.c_char_p, i32]),
     "zant_hip_conv2d_f32_static": (i32, [vp, vp, c_i64p, vp, c_i64p, vp, vp, c_i64p, c_i64p, i32, c_i64p, i32, c_i64p,
@@ -116,6 +117,7 @@ PROTOTYPES = {
     "zant_model_predict_host": (i32, [vp, vp, vp]),
     "zant_model_profile": (i32, [vp, C.POINTER(f32), C.POINTER(C.c_double), C.POINTER(C.c_double), i32]),
     "zant_model_launch_name": (C.c_char_p, [vp, i32]),
+    "zant_model_launch_kernel": (C.c_char_p, [vp, i32]),
     "zant_model_read_tensor": (i32, [vp, i32, vp, sz]),
     "zant_model_bind_predict": (i32, [vp]),
     "predict": (None, [vp, C.POINTER(C.c_uint32), C.c_uint32, C.POINTER(vp)]),
@@ -181,6 +183,10 @@ class Context:
         ms = f32()
         self.check(lib.zant_hip_kernel_ms(self.handle, C.byref(ms)))
         return ms.value
+
+    def kernel_name(self):
+        """Device function of the last operator's main kernel ("" where the launch site does not name it)."""
+        return lib.zant_hip_kernel_name(self.handle).decode()
 
     def close(self):
         if self.handle:

@@ -22,6 +22,7 @@ struct zant_ctx {
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
     hipEvent_t ev_k0 = nullptr, ev_k1 = nullptr;  // bracket the last main kernel when kernel_timing is on
     bool kernel_timing = false;
+    char last_kernel[96] = {0};  // device function of the last main kernel, template arguments included where the launch site knows them
     int num_cus = 256;
     std::string last_error;
 };
@@ -43,10 +44,14 @@ int zant_fail_hip(zant_ctx *ctx, hipError_t e, const char *what);
 // Checks the launch that was just enqueued.
 #define ZANT_LAUNCH_CHECK(ctx) ZANT_HIP_TRY(ctx, hipGetLastError())
 
+// Names the main kernel a launch site is about to enqueue (what a profiler's kernel trace shows for it).
+#define ZANT_KERNEL_NAME(ctx, ...) snprintf((ctx)->last_kernel, sizeof((ctx)->last_kernel), __VA_ARGS__)
+
 // Brackets the main kernel of an operator with events when per-kernel timing is enabled.
 struct KernelTimer {
     zant_ctx *ctx;
     explicit KernelTimer(zant_ctx *c) : ctx(c) {
+        ctx->last_kernel[0] = 0;
         if (ctx->kernel_timing) (void)hipEventRecord(ctx->ev_k0, ctx->stream);
     }
     ~KernelTimer() {

@@ -684,6 +684,7 @@ void launch_mfma_tt(zant_ctx *ctx, const float *x, const float *wp, const float 
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         attr_set = true;
     }
+    ZANT_KERNEL_NAME(ctx, "conv_f32_mfma_kernel<%d,%d,%d,%d,%d,%s>", MT, WM, WN, KV, TT, POOL ? "true" : "false");
     hipLaunchKernelGGL((conv_f32_mfma_kernel<MT, WM, WN, KV, TT, POOL>), dim3(grid), dim3(WM * WN * 64), p.lds_bytes,
                        ctx->stream, x, wp, bias, y, g, p.t, relu, counter, parity);
 }
@@ -931,6 +932,7 @@ int zant_conv2d_f32_slot(zant_ctx *ctx, const float *x, const int64_t xdim[4], c
         const int64_t positions = int64_t(g.N) * g.OH * g.OW;
         const unsigned pb = unsigned(std::min<int64_t>(ceil_div64(positions, 256), int64_t(ctx->num_cus) * 16));
         KernelTimer kt(ctx);
+        ZANT_KERNEL_NAME(ctx, "conv_f32_smallc_kernel<%d>", ckk);
         if (ckk == 9) hipLaunchKernelGGL(conv_f32_smallc_kernel<9>, dim3(pb), dim3(256), 0, ctx->stream, x, w, bias, y, g, relu);
         else if (ckk == 25) hipLaunchKernelGGL(conv_f32_smallc_kernel<25>, dim3(pb), dim3(256), 0, ctx->stream, x, w, bias, y, g, relu);
         else hipLaunchKernelGGL(conv_f32_smallc_kernel<27>, dim3(pb), dim3(256), 0, ctx->stream, x, w, bias, y, g, relu);
@@ -942,6 +944,7 @@ int zant_conv2d_f32_slot(zant_ctx *ctx, const float *x, const int64_t xdim[4], c
     int64_t blocks = ceil_div64(total, 256);
     if (blocks > int64_t(ctx->num_cus) * 32) blocks = int64_t(ctx->num_cus) * 32;
     KernelTimer kt(ctx);
+    ZANT_KERNEL_NAME(ctx, "conv_f32_direct_kernel");
     hipLaunchKernelGGL(conv_f32_direct_kernel, dim3(unsigned(blocks)), dim3(256), 0, ctx->stream, x, w, bias, y, g, relu);
     ZANT_LAUNCH_CHECK(ctx);
     zant_log("OnnxConvLean4");
@@ -988,6 +991,7 @@ int zant_conv2d_f32_fused_pool(zant_ctx *ctx, const float *x, const int64_t xdim
         const size_t lds = size_t(imgs) * g.H * g.W * 4 + 16;
         const FastDiv dpp = make_fastdiv(unsigned(POH * POW)), dpw = make_fastdiv(unsigned(POW));
         const bool fullk = g.K % 32 == 0;
+        ZANT_KERNEL_NAME(ctx, "conv_f32_c1k3_pool_mfma_kernel<%s,%s>", relu ? "true" : "false", fullk ? "true" : "false");
 #define ZANT_C1K3(R, F)                                                                                                      \
     hipLaunchKernelGGL((conv_f32_c1k3_pool_mfma_kernel<R, F>), grid, dim3(256), lds, ctx->stream, x, w, bias, y, g.N, g.H, g.W, g.K, \
                        POH, POW, imgs, dpp, dpw)
@@ -1000,6 +1004,7 @@ int zant_conv2d_f32_fused_pool(zant_ctx *ctx, const float *x, const int64_t xdim
     const int64_t positions = int64_t(g.N) * POH * POW;
     const unsigned pb = unsigned(std::min<int64_t>(ceil_div64(positions, 256), int64_t(ctx->num_cus) * 16));
     KernelTimer kt(ctx);
+    ZANT_KERNEL_NAME(ctx, "conv_f32_smallc_pool_kernel<%s>", k133 ? "1,3,3" : k155 ? "1,5,5" : "3,3,3");
     if (k133) hipLaunchKernelGGL((conv_f32_smallc_pool_kernel<1, 3, 3>), dim3(pb), dim3(256), 0, ctx->stream, x, w, bias, y, g, POH, POW, relu);
     else if (k155) hipLaunchKernelGGL((conv_f32_smallc_pool_kernel<1, 5, 5>), dim3(pb), dim3(256), 0, ctx->stream, x, w, bias, y, g, POH, POW, relu);
     else hipLaunchKernelGGL((conv_f32_smallc_pool_kernel<3, 3, 3>), dim3(pb), dim3(256), 0, ctx->stream, x, w, bias, y, g, POH, POW, relu);

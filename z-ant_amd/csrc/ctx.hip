@@ -263,6 +263,8 @@ extern "C" int zant_hip_kernel_timing(zant_ctx *ctx, int enable) {
     return ZANT_OK;
 }
 
+extern "C" const char *zant_hip_kernel_name(zant_ctx *ctx) { return ctx ? ctx->last_kernel : ""; }
+
 extern "C" int zant_hip_kernel_ms(zant_ctx *ctx, float *elapsed_ms) {
     if (!ctx || !elapsed_ms) return ZANT_NullPointer;
     ZANT_HIP_TRY(ctx, hipEventSynchronize(ctx->ev_k1));

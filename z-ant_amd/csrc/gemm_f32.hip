@@ -501,6 +501,7 @@ void launch_gemm_dma(zant_ctx *ctx, const float *A, const float *B, const float 
         attr_set = true;
     }
     const unsigned blocks = unsigned(((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN));
+    ZANT_KERNEL_NAME(ctx, "gemm_f32_dma_kernel<%d,%d,%d,%d,%d,%d>", MT, WM, WN, AM, BMODE, S);
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(WM * WN * 64), lds_bytes, ctx->stream, A, B, C, Y, g);
 }
 
@@ -607,6 +608,7 @@ void launch_gemm(zant_ctx *ctx, const float *A, const float *B, const float *C, 
     constexpr int BM = WM * TM * 32, BN = WN * 32;
     const unsigned blocks = unsigned(((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN));
     const dim3 grid(blocks), block(WM * WN * 64);
+    ZANT_KERNEL_NAME(ctx, "gemm_f32_mfma_kernel<%d,%d,%d,%s,%s>", TM, WM, WN, a_kc ? "true" : "false", b_kc ? "true" : "false");
     if (a_kc && b_kc) hipLaunchKernelGGL((gemm_f32_mfma_kernel<TM, WM, WN, true, true>), grid, block, 0, ctx->stream, A, B, C, Y, g);
     else if (a_kc && !b_kc) hipLaunchKernelGGL((gemm_f32_mfma_kernel<TM, WM, WN, true, false>), grid, block, 0, ctx->stream, A, B, C, Y, g);
     else if (!a_kc && b_kc) hipLaunchKernelGGL((gemm_f32_mfma_kernel<TM, WM, WN, false, true>), grid, block, 0, ctx->stream, A, B, C, Y, g);
@@ -631,6 +633,7 @@ int run_gemm(zant_ctx *ctx, const float *A, const float *B, const float *C, floa
     if (softmax && (trans_a || N > 16)) return ZANT_InvalidInput;
     KernelTimer kt(ctx);
     if (!trans_a && N <= 16) {
+        ZANT_KERNEL_NAME(ctx, "gemm_f32_skinny_kernel");
         hipLaunchKernelGGL(gemm_f32_skinny_kernel, dim3(unsigned((M + 15) / 16)), dim3(256), 0, ctx->stream, A, B, C, Y, g,
                            trans_b ? 1 : g.ldb, trans_b ? g.ldb : 1, softmax);
         ZANT_LAUNCH_CHECK(ctx);

@@ -98,6 +98,7 @@ struct zant_model {
     size_t arena_bytes = 0, unfused_bytes = 0;
     int launches = 0;
     std::vector<char> result_host;  // what predict() hands out
+    std::vector<std::string> launch_kernels;  // device function of each launch's main kernel, filled by zant_model_profile
 };
 
 namespace {
@@ -1248,6 +1249,8 @@ extern "C" int zant_model_profile(zant_model *m, float *ms, double *ops, double 
         if (cnt < capacity) {
             rc = zant_hip_kernel_ms(ctx, &ms[cnt]);
             if (rc) break;
+            if (cnt >= int(m->launch_kernels.size())) m->launch_kernels.resize(cnt + 1);
+            m->launch_kernels[cnt] = ctx->last_kernel;
             double o = 0, b = 0;
             node_work(m, nd, &o, &b);
             if (ops) ops[cnt] = o;
@@ -1267,6 +1270,11 @@ extern "C" const char *zant_model_launch_name(zant_model *m, int i) {
         if (cnt++ == i) return op_name(nd);
     }
     return "";
+}
+
+extern "C" const char *zant_model_launch_kernel(zant_model *m, int i) {
+    if (!m || i < 0 || i >= int(m->launch_kernels.size())) return "";
+    return m->launch_kernels[i].c_str();
 }
 
 extern "C" int zant_model_read_tensor(zant_model *m, int id, void *dst_host, size_t bytes) {

@@ -582,6 +582,7 @@ void launch_qmfma_tt(zant_ctx *ctx, const int8_t *xb, const int8_t *wp, const fl
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         attr_set = true;
     }
+    ZANT_KERNEL_NAME(ctx, "qconv_mfma_kernel<%d,%d,%d,%d,%s>", MT, WM, WN, TT, POOL ? "true" : "false");
     hipLaunchKernelGGL((qconv_mfma_kernel<MT, WM, WN, TT, POOL>), dim3(grid), dim3(WM * WN * 64), p.lds_bytes, ctx->stream, xb,
                        wp, mult, corr, padvec, y, g, p.t, CB, q, n_stages, yb);
 }

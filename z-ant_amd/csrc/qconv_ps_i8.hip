@@ -606,6 +606,7 @@ void ps_launch_out(zant_ctx *ctx, int grid, size_t lds, const int8_t *xb, const 
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         attr_set = true;
     }
+    ZANT_KERNEL_NAME(ctx, "qconv_ps_kernel<%d,%d>", MT, OUT);
     hipLaunchKernelGGL((qconv_ps_kernel<MT, OUT>), dim3(grid), dim3(PS_NT), lds, ctx->stream, xb, wp, tabs, padvec, y, p, q);
 }
 

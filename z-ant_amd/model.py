@@ -202,6 +202,10 @@ class Model:
             raise ZantError(rc)
         return [(self._lib.zant_model_launch_name(self.handle, i).decode(), ms[i], ops[i], by[i]) for i in range(rc)]
 
+    def launch_kernels(self):
+        """Device function of each launch's main kernel as of the last profile() (a profiler's kernel-trace names)."""
+        return [self._lib.zant_model_launch_kernel(self.handle, i).decode() for i in range(self.num_launches)]
+
     def predict_host(self, x):
         x = np.ascontiguousarray(x)
         y = np.zeros(self.out_shape, self.out_dtype)

@@ -25,11 +25,16 @@ def readme_cnn_params(seed=0):
 
 
 def readme_cnn_flops_per_inference():
+    """Multiply-adds x 2 of one inference.  "total" counts the graph as written (conv2 at its 11 x 11 outputs);
+    "executed" counts what the fused pass computes: the 2x2/2 pool behind conv2 drops row and column 10, and the
+    fused kernel does not compute them (10 x 10 outputs)."""
     conv1 = 2 * 32 * 26 * 26 * 9
     conv2 = 2 * 64 * 11 * 11 * 32 * 9
+    conv2_executed = 2 * 64 * 10 * 10 * 32 * 9
     gemm1 = 2 * 1600 * 512
     gemm2 = 2 * 512 * 10
-    return {"conv1": conv1, "conv2": conv2, "gemm1": gemm1, "gemm2": gemm2, "total": conv1 + conv2 + gemm1 + gemm2}
+    return {"conv1": conv1, "conv2": conv2, "conv2_executed": conv2_executed, "gemm1": gemm1, "gemm2": gemm2,
+            "total": conv1 + conv2 + gemm1 + gemm2, "executed": conv1 + conv2_executed + gemm1 + gemm2}
 
 
 def build_readme_cnn_model(ctx, batch, params):
