@@ -32,6 +32,7 @@ typedef int i32x4 __attribute__((ext_vector_type(4)));
 struct QBlockArgs {
     int N, H, W, OH, OW, stride;
     int CBin, Cin32, Ce32, CBo;        // input channel blocks (16) / chunks (32); expanded chunks; output blocks
+    int Co;                            // output channels (the rest of the last block is padding)
     int NB, TH, PH, PW, P, Ppad, Q;    // tile: images, output rows, patch rows / columns / positions, output positions
     int n_row_tiles, n_tiles;
     int o_xl, o_e, o_w1, o_w2, o_wdw, o_tab, o_ptab;  // LDS byte offsets
@@ -46,13 +47,49 @@ struct QBlockArgs {
     int ra_zp, rb_zp, ry_zp;
 };
 
+// LDS reads the compiler does not see, so that it neither serialises them with waits of its own nor reorders them:
+// the kernel issues a batch (the nine taps of a position tile, the sixteen table lookups of a requantisation), keeps
+// computing, and waits with a counted s_waitcnt that hands the values to their users.  LDS operations complete in
+// order; operations the compiler issues in between only make a counted wait stricter.
+__device__ __forceinline__ void qb_read128(i32x4 &v, unsigned addr, int imm) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "i"(imm));
+}
+__device__ __forceinline__ void qb_ready(i32x4 &b, int pending) {
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(b) : "i"(pending));
+}
+__device__ __forceinline__ uint32_t qb_read_u8(unsigned addr) {
+    uint32_t v;
+    asm volatile("ds_read_u8 %0, %1" : "=v"(v) : "v"(addr));
+    return v;
+}
+__device__ __forceinline__ void qb_ready8(uint32_t *v) {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]));
+}
+// Requantises the accumulator values [V0, V0 + 8 * G) of one MFMA tile and looks their bytes up in the activation
+// table at `table` (256-byte aligned): all lookups of the batch are issued before the one wait.  d[g] receives the four
+// bytes of accumulator registers 4g .. 4g + 3.
+template <int G>
+__device__ __forceinline__ void qb_requant_lookup(const i32x16 &acc, const float (&mv)[16], float zp_f, unsigned table,
+                                                  uint32_t (&d)[4]) {
+    uint32_t b[16];
+#pragma unroll
+    for (int v = 0; v < 4 * G; ++v)
+        b[v] = qb_read_u8(__builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(float(acc[v]) * mv[v]) + zp_f, 0u, table));
+    qb_ready8(b);
+    if (G > 2) qb_ready8(b + 8);
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+        d[g] = g < G ? (b[4 * g] | (b[4 * g + 1] << 8) | (b[4 * g + 2] << 16) | (b[4 * g + 3] << 24)) : 0u;
+}
+
 __device__ __forceinline__ i32x4 as_i32x4(const uint4 &v) {
     i32x4 r;
     r[0] = int(v.x); r[1] = int(v.y); r[2] = int(v.z); r[3] = int(v.w);
     return r;
 }
 
-template <int CO32, int MQ>
+template <int CO32, int MQ, bool PF>
 __global__ void __launch_bounds__(256, CO32 <= 2 ? 2 : 1)  // wide projections need the whole CU's LDS anyway
 qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 *__restrict__ w1p,
               const uint4 *__restrict__ w2p, const uint32_t *__restrict__ wm, const float *__restrict__ mult1,
@@ -109,25 +146,75 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
     const uint32_t dm0 = diag_mine && diag_q == 0 ? 0xffffffffu : 0u, dm1 = diag_mine && diag_q == 1 ? 0xffffffffu : 0u,
                    dm2 = diag_mine && diag_q == 2 ? 0xffffffffu : 0u, dm3 = diag_mine && diag_q == 3 ? 0xffffffffu : 0u;
 
+    // ---- A: input patch -> LDS (positions outside the image are left as they are: C overwrites what they yield).  The
+    // first tile's patch is copied before the loop; every later one is loaded into registers before stage B of the tile
+    // in front of it and written to LDS after that stage (the input patch is dead once B is done), so its global
+    // latency passes under B.  Patches of more than QB_PF units per thread are copied in place instead. ----
+    constexpr int QB_PF = 4;
+    const int a_units = a.CBin * a.P;
+    const bool prefetch = PF && a_units <= QB_PF * 256;  // PF is off for the instantiations without registers to spare
+    auto patch_unit = [&](int tile_, int u, int &dst) -> const uint4 * {  // source of unit u of a tile's patch, or null
+        const int ig_ = tile_ / a.n_row_tiles, rt_ = tile_ - ig_ * a.n_row_tiles;
+        const int cb = small_div(u, a.P, inv_p), p = u - cb * a.P;
+        const int e = ptab[p];
+        const int n = ig_ * a.NB + (e >> 20), ih = rt_ * a.TH * a.stride - 1 + ((e >> 10) & 1023), iw = (e & 1023) - 1;
+        dst = cb * a.Ppad + p;
+        if (n < a.N && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W) return x + ((int64_t(n) * a.CBin + cb) * a.H + ih) * int64_t(a.W) + iw;
+        return nullptr;
+    };
+    auto copy_patch = [&](int tile_) {  // four loads in flight per thread, then their four LDS writes
+        for (int u0 = tid; u0 < a_units; u0 += 4 * 256) {
+            i32x4 v[4];  // (a native vector type: arrays of it are kept in registers)
+            int dst[4];
+            bool ok[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int u = min(u0 + r * 256, a_units - 1);
+                const uint4 *src = patch_unit(tile_, u, dst[r]);
+                ok[r] = src != nullptr && u0 + r * 256 < a_units;
+                v[r] = *reinterpret_cast<const i32x4 *>(ok[r] ? src : x);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (ok[r]) *reinterpret_cast<i32x4 *>(XL + dst[r]) = v[r];
+        }
+    };
+    if (int(blockIdx.x) < a.n_tiles) copy_patch(blockIdx.x);
+    __syncthreads();
+
     for (int tile = blockIdx.x; tile < a.n_tiles; tile += gridDim.x) {
         const int ig = tile / a.n_row_tiles, rt = tile - ig * a.n_row_tiles;
         const int n0 = ig * a.NB, oh0 = rt * a.TH, ih0 = oh0 * a.stride - 1;
-
-        // ---- A: input patch -> LDS (positions outside the image are left as they are: C overwrites what they yield) ----
-        for (int u = tid; u < a.CBin * a.P; u += 256) {
-            const int cb = small_div(u, a.P, inv_p), p = u - cb * a.P;
-            const int e = ptab[p];
-            const int n = n0 + (e >> 20), ih = ih0 + ((e >> 10) & 1023), iw = (e & 1023) - 1;
-            if (n < a.N && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W)
-                XL[cb * a.Ppad + p] = x[((int64_t(n) * a.CBin + cb) * a.H + ih) * int64_t(a.W) + iw];
+        const int next_tile = tile + int(gridDim.x);
+        const bool has_next = next_tile < a.n_tiles;
+        i32x4 nxt[QB_PF];
+        int nxt_dst[QB_PF];
+        unsigned nxt_ok = 0;
+        if (PF && prefetch && has_next) {
+#pragma unroll
+            for (int r = 0; r < QB_PF; ++r) {
+                nxt_dst[r] = 0;
+                if (r * 256 < a_units) {
+                    // every lane loads (from the tensor's first unit when it has nothing to fetch): no divergent branch
+                    // around the load, so nothing waits for it before stage C
+                    const int u = min(r * 256 + tid, a_units - 1);
+                    const uint4 *src = patch_unit(next_tile, u, nxt_dst[r]);
+                    const bool ok = src != nullptr && r * 256 + tid < a_units;
+                    nxt[r] = *reinterpret_cast<const i32x4 *>(ok ? src : x);
+                    nxt_ok |= ok ? 1u << r : 0u;
+                }
+            }
         }
-        __syncthreads();
 
         // ---- B: expansion.  A wave keeps one block of 32 expanded channels (its multipliers, corrections and, for one
         // chunk of input channels, its weights) in registers and walks the position tiles with it. ----
         {
             // (channel block, position tile) units in channel-block-major order, split evenly over the four waves
-            const int units = a.Ce32 * n_ptiles, u_begin = (units * wave) >> 2, u_end = (units * (wave + 1)) >> 2;
+            // (a block whose second half is padding costs about 4/5 of a full one: half the requantisation)
+            const int full_units = (a.half_last ? a.Ce32 - 1 : a.Ce32) * n_ptiles, half_units = a.half_last ? n_ptiles : 0;
+            const int cost = full_units * 5 + half_units * 4;
+            auto unit_at = [&](int c) { return c <= full_units * 5 ? c / 5 : full_units + (c - full_units * 5) / 4; };
+            const int u_begin = unit_at((cost * wave) >> 2), u_end = wave == 3 ? full_units + half_units : unit_at((cost * (wave + 1)) >> 2);
             int kb = small_div(u_begin, n_ptiles, inv_nptiles), ptile = u_begin - kb * n_ptiles;
             for (int u = u_begin; u < u_end;) {
                 const int kch = kb * 32 + lh * 4;
@@ -140,42 +227,31 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
                 }
                 const i32x4 wa0 = as_i32x4(W1[kb * 64 + lh * 32 + l32]);
                 const bool half = a.half_last && kb == a.Ce32 - 1;
-                char *erow = reinterpret_cast<char *>(E) + (kb * 2 * a.Ppad + l32) * 16 + lh * 8;
+                // this lane's operand of input chunk 0 and the 16-byte unit it writes: lane (p, 0) the block of expanded
+                // channels 32 kb .. + 15 of its position, lane (p, 1) the block of channels 32 kb + 16 .. + 31
+                const unsigned x_addr = lds_address(XL) + unsigned(lh * a.Ppad + l32) * 16u;
+                const unsigned e_addr = lds_address(E) + unsigned((2 * kb + lh) * a.Ppad + l32) * 16u;
                 for (; ptile < n_ptiles && u < u_end; ++ptile, ++u) {
                     const int p = ptile * 32 + l32;
-                    i32x16 acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wa0, as_i32x4(XL[lh * a.Ppad + p]), cvec, 0, 0, 0);
+                    i32x4 xb;
+                    qb_read128(xb, x_addr + unsigned(ptile) * 512u, 0);
+                    qb_ready(xb, 0);
+                    i32x16 acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wa0, xb, cvec, 0, 0, 0);
                     for (int chunk = 1; chunk < a.Cin32; ++chunk)
                         acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(as_i32x4(W1[(chunk * a.Ce32 + kb) * 64 + lh * 32 + l32]),
                                                                     as_i32x4(XL[(2 * chunk + lh) * a.Ppad + p]), acc, 0, 0, 0);
                     // a last block with at most 16 real channels: accumulator rows 16..31 (values 8..15) are padding
-                    uint32_t d[4] = {0u, 0u, 0u, 0u};
-                    if (half) {
-#pragma unroll
-                        for (int gq = 0; gq < 2; ++gq) {
-                            uint32_t o = 0;
-#pragma unroll
-                            for (int e = 0; e < 4; ++e)
-                                o |= requant_lookup(float(acc[gq * 4 + e]) * mv[gq * 4 + e], a.zp1f, lut1_a) << (8 * e);
-                            d[gq] = o;
-                        }
-                    } else {
-#pragma unroll
-                        for (int gq = 0; gq < 4; ++gq) {
-                            uint32_t o = 0;
-#pragma unroll
-                            for (int e = 0; e < 4; ++e)
-                                o |= requant_lookup(float(acc[gq * 4 + e]) * mv[gq * 4 + e], a.zp1f, lut1_a) << (8 * e);
-                            d[gq] = o;
-                        }
-                    }
-                    // lanes p and p + 32 exchange one dword per 16-channel block so that each writes 8 consecutive bytes
-#pragma unroll
-                    for (int b = 0; b < 2; ++b) {
-                        const uint32_t send = lh ? d[2 * b] : d[2 * b + 1];
-                        const uint32_t recv = uint32_t(__shfl_xor(int(send), 32, 64));
-                        const uint2 out = lh ? make_uint2(recv, d[2 * b + 1]) : make_uint2(d[2 * b], recv);
-                        if (b == 0 || !half) *reinterpret_cast<uint2 *>(erow + (b * a.Ppad + ptile * 32) * 16) = out;
-                    }
+                    uint32_t d[4];
+                    if (half) qb_requant_lookup<2>(acc, mv, a.zp1f, lut1_a, d);
+                    else qb_requant_lookup<4>(acc, mv, a.zp1f, lut1_a, d);
+                    // the half-wave swap leaves the lower lane with the 16 bytes of the first block of 16 channels and the
+                    // upper lane with those of the second: one 16-byte write per lane
+                    const auto s0 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
+                    const auto s1 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
+                    i32x4 out;
+                    out[0] = int(s0[0]); out[1] = int(s0[1]); out[2] = int(s1[0]); out[3] = int(s1[1]);
+                    if (!half || !lh)
+                        *reinterpret_cast<__attribute__((address_space(3))) i32x4 *>(e_addr + unsigned(ptile) * 512u) = out;
                 }
                 ptile = 0;
                 ++kb;
@@ -183,12 +259,21 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
         }
         __syncthreads();
 
-        // ---- C: the depthwise convolution's padding ----
+        // ---- C: the depthwise convolution's padding; the next tile's input patch goes to LDS ----
         for (int p = tid; p < a.P; p += 256) {
             const int e = ptab[p];
             const int ih = ih0 + ((e >> 10) & 1023), pw = e & 1023;
             if (pw == 0 || pw == a.PW - 1 || ih < 0 || ih >= a.H)
                 for (int cb = 0; cb < a.Ce32 * 2; ++cb) E[cb * a.Ppad + p] = pad_e;
+        }
+        if (has_next) {
+            if (PF && prefetch) {
+#pragma unroll
+                for (int r = 0; r < QB_PF; ++r)
+                    if ((nxt_ok >> r) & 1u) *reinterpret_cast<i32x4 *>(XL + nxt_dst[r]) = nxt[r];
+            } else {
+                copy_patch(next_tile);
+            }
         }
         __syncthreads();
 
@@ -238,39 +323,36 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
                 i32x4 w2a[CO32];
 #pragma unroll
                 for (int kb3 = 0; kb3 < CO32; ++kb3) w2a[kb3] = as_i32x4(W2[(ch * CO32 + kb3) * 64 + lh * 32 + l32]);
+                // The nine taps of a position tile are issued as one batch and consumed by the MFMAs as they arrive; the
+                // taps of the next tile are issued before this tile's requantisation, so they travel under its arithmetic.
+                const unsigned e_ch = lds_address(E) + unsigned((2 * ch + lh) * a.Ppad) * 16u;
+                const unsigned row_b = unsigned(a.PW) * 16u;
+                i32x4 tap[9];
+                auto issue_taps = [&](int j) {
+                    const unsigned r0 = e_ch + unsigned(p0[j]) * 16u, r1 = r0 + row_b, r2 = r1 + row_b;
+                    qb_read128(tap[0], r0, 0); qb_read128(tap[1], r0, 16); qb_read128(tap[2], r0, 32);
+                    qb_read128(tap[3], r1, 0); qb_read128(tap[4], r1, 16); qb_read128(tap[5], r1, 32);
+                    qb_read128(tap[6], r2, 0); qb_read128(tap[7], r2, 16); qb_read128(tap[8], r2, 32);
+                };
+                issue_taps(0);
 #pragma unroll
                 for (int j = 0; j < MQ; ++j) {
-                    const uint4 *ep = E + (2 * ch + lh) * a.Ppad + p0[j];
-                    i32x16 acc2 = __builtin_amdgcn_mfma_i32_32x32x32_i8(wa[0], as_i32x4(ep[0]), cvec, 0, 0, 0);
+                    qb_ready(tap[0], 8);
+                    i32x16 acc2 = __builtin_amdgcn_mfma_i32_32x32x32_i8(wa[0], tap[0], cvec, 0, 0, 0);
 #pragma unroll
-                    for (int t = 1; t < 9; ++t)
-                        acc2 = __builtin_amdgcn_mfma_i32_32x32x32_i8(wa[t], as_i32x4(ep[(t / 3) * a.PW + (t % 3)]), acc2, 0, 0, 0);
-                    uint32_t d[4] = {0u, 0u, 0u, 0u};
-                    if (half) {
-#pragma unroll
-                        for (int gq = 0; gq < 2; ++gq) {
-                            uint32_t o = 0;
-#pragma unroll
-                            for (int e = 0; e < 4; ++e)
-                                o |= requant_lookup(float(acc2[gq * 4 + e]) * mv[gq * 4 + e], a.zp2f, lut2_a) << (8 * e);
-                            d[gq] = o;
-                        }
-                    } else {
-#pragma unroll
-                        for (int gq = 0; gq < 4; ++gq) {
-                            uint32_t o = 0;
-#pragma unroll
-                            for (int e = 0; e < 4; ++e)
-                                o |= requant_lookup(float(acc2[gq * 4 + e]) * mv[gq * 4 + e], a.zp2f, lut2_a) << (8 * e);
-                            d[gq] = o;
-                        }
+                    for (int t = 1; t < 9; ++t) {
+                        qb_ready(tap[t], 8 - t);
+                        acc2 = __builtin_amdgcn_mfma_i32_32x32x32_i8(wa[t], tap[t], acc2, 0, 0, 0);
                     }
+                    if (j + 1 < MQ) issue_taps(j + 1);
+                    uint32_t d[4];
+                    if (half) qb_requant_lookup<2>(acc2, mv, a.zp2f, lut2_a, d);
+                    else qb_requant_lookup<4>(acc2, mv, a.zp2f, lut2_a, d);
                     // lane (p, 0) gathers channels 0..15 of the chunk, lane (p, 1) channels 16..31
-                    const uint32_t r0 = uint32_t(__shfl_xor(int(lh ? d[0] : d[2]), 32, 64));
-                    const uint32_t r1 = uint32_t(__shfl_xor(int(lh ? d[1] : d[3]), 32, 64));
+                    const auto s0 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
+                    const auto s1 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
                     i32x4 db;
-                    db[0] = int(lh ? r0 : d[0]); db[1] = int(lh ? d[2] : r0);
-                    db[2] = int(lh ? r1 : d[1]); db[3] = int(lh ? d[3] : r1);
+                    db[0] = int(s0[0]); db[1] = int(s0[1]); db[2] = int(s1[0]); db[3] = int(s1[1]);
 #pragma unroll
                     for (int kb3 = 0; kb3 < CO32; ++kb3)
                         acc3[j][kb3] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w2a[kb3], db, acc3[j][kb3], 0, 0, 0);
@@ -278,34 +360,67 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
             }
             auto store_tiles = [&](auto res_tag, auto fast_tag) {
                 constexpr bool RES = decltype(res_tag)::value, FAST = decltype(fast_tag)::value;
+                // byte offset of this lane's four channels in block 0 of its position (the host checks that the blocked
+                // tensors stay below 2^31 bytes); a block of 16 channels further on is one plane further
+                unsigned ybase[MQ];
+                bool ok[MQ];
+                const unsigned plane16 = unsigned(a.OH * a.OW) * 16u;
 #pragma unroll
                 for (int j = 0; j < MQ; ++j) {
                     const int n = n0 + qimg[j], oh = oh0 + qr[j];
-                    const bool ok = qvalid[j] && n < a.N && oh < a.OH;
+                    ok[j] = qvalid[j] && n < a.N && oh < a.OH;
+                    ybase[j] = ((unsigned(n) * unsigned(a.CBo) * unsigned(a.OH) + unsigned(oh)) * unsigned(a.OW) + unsigned(qc[j])) * 16u + unsigned(lh) * 4u;
+                }
+                // the residual's bytes of every (tile, group) first, as one batch of loads
+                uint32_t xr[MQ][CO32 * 4];
+                if (RES) {
 #pragma unroll
-                    for (int kb3 = 0; kb3 < CO32; ++kb3) {
+                    for (int j = 0; j < MQ; ++j)
 #pragma unroll
-                        for (int gq = 0; gq < 4; ++gq) {
-                            const int cbq = kb3 * 2 + (gq >> 1);
-                            const bool st = ok && cbq < a.CBo;
-                            const int64_t off = (((int64_t(n) * a.CBo + cbq) * a.OH + oh) * int64_t(a.OW) + qc[j]) * 16 + (gq & 1) * 8 + lh * 4;
-                            uint32_t xr = 0;
-                            if (RES && st)
-                                xr = *reinterpret_cast<const uint32_t *>(reinterpret_cast<const char *>(x) + off) ^ 0x80808080u;
+                        for (int g = 0; g < CO32 * 4; ++g) {
+                            xr[j][g] = 0;
+                            if (ok[j] && g * 8 < a.Co)
+                                xr[j][g] = *reinterpret_cast<const uint32_t *>(reinterpret_cast<const char *>(x) + (ybase[j] + unsigned(g >> 1) * plane16 + unsigned(g & 1) * 8u));
+                        }
+                }
+#pragma unroll
+                for (int kb3 = 0; kb3 < CO32; ++kb3) {
+#pragma unroll
+                    for (int gq = 0; gq < 4; ++gq) {
+                        const int cbq = kb3 * 2 + (gq >> 1);
+                        if (cbq >= a.CBo) continue;
+                        const unsigned goff = unsigned(cbq) * plane16 + unsigned(gq & 1) * 8u;
+                        // eight output channels per group: a group past the last real channel is padding of the blocked
+                        // layout (no kernel reads it against a non-zero weight): no arithmetic, zeros stored
+                        if (kb3 * 32 + gq * 8 >= a.Co) {
+#pragma unroll
+                            for (int j = 0; j < MQ; ++j)
+                                if (ok[j]) *reinterpret_cast<uint32_t *>(y + (ybase[j] + goff)) = 0u;
+                            continue;
+                        }
+                        float mq[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) mq[e] = m3[kb3 * 32 + gq * 8 + lh * 4 + e];
+#pragma unroll
+                        for (int j = 0; j < MQ; ++j) {
                             uint32_t o = 0;
 #pragma unroll
                             for (int e = 0; e < 4; ++e) {
-                                uint32_t v = sat_u8_rne_finite(float(acc3[j][kb3][gq * 4 + e]) * m3[kb3 * 32 + gq * 8 + lh * 4 + e], a.zp3f);
+                                const float r = __builtin_rintf(float(acc3[j][kb3][gq * 4 + e]) * mq[e]) + a.zp3f;
                                 if (RES) {
-                                    const float fa = float(int(v) - a.ra_zp) * a.ra_scale;
-                                    const float fb = float(int((xr >> (8 * e)) & 0xffu) - a.rb_zp) * a.rb_scale;
+                                    // the projection's own output byte as a float (the saturation is the clamp), then the
+                                    // quantised add in dequantised space; every step is the stand-alone kernels' arithmetic
+                                    const float va = __builtin_amdgcn_fmed3f(r, 0.0f, 255.0f);
+                                    const float fa = (va - float(a.ra_zp)) * a.ra_scale;
+                                    const float fb = (float(((xr[j][kb3 * 4 + gq] ^ 0x80808080u) >> (8 * e)) & 0xffu) - float(a.rb_zp)) * a.rb_scale;
                                     // finite operands: the saturating conversion replaces the clamp
-                                    v = FAST ? sat_u8_rne_finite(div_by(fa + fb, a.ry_scale, a.ry_rcp, 1), float(a.ry_zp))
-                                             : uint32_t(sat_u8_rne((fa + fb) / a.ry_scale, uint8_t(a.ry_zp)));
+                                    const float qv = FAST ? div_by(fa + fb, a.ry_scale, a.ry_rcp, 1) : (fa + fb) / a.ry_scale;
+                                    o = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(qv) + float(a.ry_zp), e, o);
+                                } else {
+                                    o = __builtin_amdgcn_cvt_pk_u8_f32(r, e, o);
                                 }
-                                o |= v << (8 * e);
                             }
-                            if (st) *reinterpret_cast<uint32_t *>(y + off) = o ^ 0x80808080u;
+                            if (ok[j]) *reinterpret_cast<uint32_t *>(y + (ybase[j] + goff)) = o ^ 0x80808080u;
                         }
                     }
                 }
@@ -342,7 +457,7 @@ int zant_qblock_blocked(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], 
 
     QBlockArgs a;
     a.N = int(N); a.H = int(H); a.W = int(W); a.OH = int(OH); a.OW = int(OW); a.stride = int(dw_stride);
-    a.CBin = int((Cin + 15) / 16); a.Cin32 = int((Cin + 31) / 32); a.Ce32 = int((Ce + 31) / 32); a.CBo = int((Co + 15) / 16);
+    a.CBin = int((Cin + 15) / 16); a.Cin32 = int((Cin + 31) / 32); a.Ce32 = int((Ce + 31) / 32); a.CBo = int((Co + 15) / 16); a.Co = int(Co);
     const int CO32 = int((Co + 31) / 32), CeP = a.Ce32 * 32;
     a.PW = int(W) + 2;
     // LDS: fixed part, then per patch position the input and expanded bytes and one table entry
@@ -482,27 +597,28 @@ int zant_qblock_blocked(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], 
     const int q_per_wave = (nq_tiles + 3) / 4;
     const int rounds = (q_per_wave + mq_cap - 1) / mq_cap;
     const int MQv = std::max(1, (q_per_wave + rounds - 1) / rounds);
-#define ZANT_QBLOCK_LAUNCH(CO, M)                                                                                           \
+#define ZANT_QBLOCK_LAUNCH(CO, M, P)                                                                                          \
     do {                                                                                                                    \
         static bool attr_set = false;                                                                                       \
         if (!attr_set) {                                                                                                    \
-            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&qblock_kernel<CO, M>),                               \
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&qblock_kernel<CO, M, P>),                               \
                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                             \
             attr_set = true;                                                                                                \
         }                                                                                                                   \
-        hipLaunchKernelGGL((qblock_kernel<CO, M>), dim3(grid), dim3(256), cap_used, ctx->stream,                           \
+        ZANT_KERNEL_NAME(ctx, "qblock_kernel<%d,%d,%s>", CO, M, P ? "true" : "false");                                          \
+        hipLaunchKernelGGL((qblock_kernel<CO, M, P>), dim3(grid), dim3(256), cap_used, ctx->stream,                           \
                            reinterpret_cast<const uint4 *>(x), y, reinterpret_cast<const uint4 *>(w1p),                    \
                            reinterpret_cast<const uint4 *>(w2p), wmk, m1, c1, m2, c2, m3, c3, a);                          \
     } while (0)
     switch (CO32 * 10 + MQv) {
-    case 11: ZANT_QBLOCK_LAUNCH(1, 1); break;
-    case 12: ZANT_QBLOCK_LAUNCH(1, 2); break;
-    case 13: ZANT_QBLOCK_LAUNCH(1, 3); break;
-    case 14: ZANT_QBLOCK_LAUNCH(1, 4); break;
-    case 21: ZANT_QBLOCK_LAUNCH(2, 1); break;
-    case 22: ZANT_QBLOCK_LAUNCH(2, 2); break;
-    case 31: ZANT_QBLOCK_LAUNCH(3, 1); break;
-    default: ZANT_QBLOCK_LAUNCH(4, 1); break;
+    case 11: ZANT_QBLOCK_LAUNCH(1, 1, true); break;
+    case 12: ZANT_QBLOCK_LAUNCH(1, 2, true); break;
+    case 13: ZANT_QBLOCK_LAUNCH(1, 3, true); break;
+    case 14: ZANT_QBLOCK_LAUNCH(1, 4, false); break;
+    case 21: ZANT_QBLOCK_LAUNCH(2, 1, true); break;
+    case 22: ZANT_QBLOCK_LAUNCH(2, 2, false); break;
+    case 31: ZANT_QBLOCK_LAUNCH(3, 1, true); break;
+    default: ZANT_QBLOCK_LAUNCH(4, 1, true); break;
     }
 #undef ZANT_QBLOCK_LAUNCH
     ZANT_LAUNCH_CHECK(ctx);
