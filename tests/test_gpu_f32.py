@@ -244,7 +244,16 @@ POOL_CASES = [((4, 32, 26, 26), [2, 2], [2, 2], [1, 1], [0, 0, 0, 0], "NOTSET"),
               ((2, 5, 13, 11), [3, 2], [1, 2], [2, 1], [0, 1, 2, 0], "NOTSET"),
               ((2, 3, 9, 9), [3, 3], [3, 3], [1, 1], [0, 0, 0, 0], "NOTSET"),
               ((1, 3, 9, 10), [2, 2], [1, 1], [1, 1], [0, 0, 0, 0], "SAME_UPPER"),
-              ((1, 3, 9, 10), [2, 2], [1, 1], [1, 1], [0, 0, 0, 0], "SAME_LOWER")]
+              ((1, 3, 9, 10), [2, 2], [1, 1], [1, 1], [0, 0, 0, 0], "SAME_LOWER"),
+              # the plane-staged 2x2/2 kernels: a partial last group of planes, planes that are not a whole number of
+              # vectors (13 x 26), fewer planes than a group, result rows of 24 bytes (u8)
+              ((5, 3, 26, 26), [2, 2], [2, 2], [1, 1], [0, 0, 0, 0], "NOTSET"),
+              ((3, 7, 13, 26), [2, 2], [2, 2], [1, 1], [0, 0, 0, 0], "NOTSET"),
+              ((3, 1, 10, 14), [2, 2], [2, 2], [1, 1], [0, 0, 0, 0], "NOTSET"),
+              ((7, 5, 6, 6), [2, 2], [2, 2], [1, 1], [0, 0, 0, 0], "NOTSET"),
+              ((3, 5, 48, 48), [2, 2], [2, 2], [1, 1], [0, 0, 0, 0], "NOTSET"),
+              ((2, 3, 16, 48), [2, 2], [2, 2], [1, 1], [0, 0, 0, 0], "NOTSET"),
+              ((9, 11, 4, 16), [2, 2], [2, 2], [1, 1], [0, 0, 0, 0], "NOTSET")]
 
 
 @pytest.mark.parametrize("xs,k,s,d,p,ap", POOL_CASES)

@@ -368,27 +368,130 @@ __global__ void __launch_bounds__(kThreads) maxpool_2x2s2_stream_kernel(const T 
                                   fmaxf(__uint_as_float(r1[u][0]), __uint_as_float(r1[u][1])));
             __builtin_nontemporal_store(m, reinterpret_cast<float *>(y) + dst[u]);
         } else {
+            // bytes as 16-bit lanes (even bytes and odd bytes of a dword apart): the vertical maximum is one packed
+            // 16-bit max per half, the horizontal one (bytes 0|1 and 2|3) the packed max of the two halves, and one byte
+            // permute gathers the four window maxima of two input dwords
+            typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+            auto pk = [](uint32_t v) { us2 r; r[0] = (unsigned short)(v & 0xffffu); r[1] = (unsigned short)(v >> 16); return r; };
+            auto window_max = [&](uint32_t a, uint32_t b) -> uint32_t {  // -> max(bytes 0,1) | max(bytes 2,3) << 16
+                const us2 e = __builtin_elementwise_max(pk(a & 0x00ff00ffu), pk(b & 0x00ff00ffu));
+                const us2 od = __builtin_elementwise_max(pk((a >> 8) & 0x00ff00ffu), pk((b >> 8) & 0x00ff00ffu));
+                const us2 h = __builtin_elementwise_max(e, od);
+                return uint32_t(h[0]) | (uint32_t(h[1]) << 16);
+            };
             u2 o;
 #pragma unroll
             for (int d = 0; d < 2; ++d) {
-                uint32_t w = 0;
-#pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    // bytewise max of the two rows, then of horizontal neighbours
-                    const uint32_t a = r0[u][d * 2 + h], b = r1[u][d * 2 + h];
-                    uint32_t m = 0;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const uint32_t ba = (a >> (8 * e)) & 0xffu, bb = (b >> (8 * e)) & 0xffu;
-                        m |= (ba > bb ? ba : bb) << (8 * e);
-                    }
-                    const uint32_t p01 = max(m & 0xffu, (m >> 8) & 0xffu), p23 = max((m >> 16) & 0xffu, m >> 24);
-                    w |= (p01 | (p23 << 8)) << (16 * h);
-                }
-                o[d] = w;
+                const uint32_t lo = window_max(r0[u][d * 2], r1[u][d * 2]), hi = window_max(r0[u][d * 2 + 1], r1[u][d * 2 + 1]);
+                o[d] = __builtin_amdgcn_perm(hi, lo, 0x06040200u);  // bytes 0, 2 of lo then bytes 0, 2 of hi
             }
             __builtin_nontemporal_store(o, reinterpret_cast<u2 *>(reinterpret_cast<uint8_t *>(y) + dst[u]));
         }
+    }
+}
+
+// 2x2 / stride 2 on f32 planes that are not a whole number of vectors wide (26 x 26 -> 13 x 13 ...): a workgroup copies G
+// whole consecutive planes to LDS -- a contiguous run of the input, read as 16-byte vectors whatever the row length --
+// and writes their G * OH * OW results, also a contiguous run, as 16-byte vectors, four results per thread.  The rows of
+// a window are two 8-byte LDS reads (W is even).  G is a multiple of 4, so both runs start on 16-byte boundaries.
+constexpr int kPoolLdsFloats = 4 * 1024;  // 16 KB: eight workgroups (all 32 wave slots) share a CU
+__global__ void __launch_bounds__(kThreads) maxpool_2x2s2_planes_f32_kernel(const float *__restrict__ x, float *__restrict__ y,
+                                                                           int64_t NC, int G, int H, int W, int OH, int OW,
+                                                                           float inv_ohw, float inv_ow) {
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    __shared__ __attribute__((aligned(16))) float pl[kPoolLdsFloats];
+    const int64_t p0 = int64_t(blockIdx.x) * G;
+    const int planes = int(min<int64_t>(G, NC - p0));
+    const int HW = H * W, OHW = OH * OW;
+    const int n_in = planes * HW, n_out = planes * OHW;  // n_in is a multiple of 4 unless this is the tensor's tail
+    const float *src = x + p0 * HW;
+    const int n_in4 = n_in >> 2;
+    constexpr int B = kPoolLdsFloats / 4 / kThreads;  // every vector of a full LDS buffer in flight at once: 12 per thread
+    for (int i0 = 0; i0 < n_in4; i0 += kThreads * B) {
+        f4 v[B];
+#pragma unroll
+        for (int u = 0; u < B; ++u) {
+            const int i = i0 + u * kThreads + int(threadIdx.x);
+            if (i < n_in4) v[u] = __builtin_nontemporal_load(reinterpret_cast<const f4 *>(src) + i);
+        }
+#pragma unroll
+        for (int u = 0; u < B; ++u) {
+            const int i = i0 + u * kThreads + int(threadIdx.x);
+            if (i < n_in4) reinterpret_cast<f4 *>(pl)[i] = v[u];
+        }
+    }
+    for (int i = (n_in4 << 2) + int(threadIdx.x); i < n_in; i += kThreads) pl[i] = src[i];
+    __syncthreads();
+    float *dst = y + p0 * OHW;
+    auto one = [&](int o) {
+        const int pz = small_div_host(o, OHW, inv_ohw), rem = o - pz * OHW;
+        const int oh = small_div_host(rem, OW, inv_ow), ow = rem - oh * OW;
+        const float *r = pl + pz * HW + 2 * oh * W + 2 * ow;
+        const f2 a = *reinterpret_cast<const f2 *>(r), b = *reinterpret_cast<const f2 *>(r + W);
+        return fmaxf(fmaxf(a[0], a[1]), fmaxf(b[0], b[1]));
+    };
+    const int n_out4 = n_out >> 2;
+    for (int i = int(threadIdx.x); i < n_out4; i += kThreads) {
+        f4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = one(4 * i + e);
+        __builtin_nontemporal_store(o, reinterpret_cast<f4 *>(dst) + i);
+    }
+    for (int o = (n_out4 << 2) + int(threadIdx.x); o < n_out; o += kThreads) dst[o] = one(o);
+}
+
+// The same for u8 planes whose rows are whole 16-byte vectors but whose result rows are not (48 x 48 -> 24 x 24 ...): a
+// thread turns two pairs of 16-byte LDS row segments into two groups of eight results (each group lies inside one result
+// row: OW is a multiple of 8) and stores them as one 16-byte vector.  H * W and OH * OW are multiples of 16.
+__global__ void __launch_bounds__(kThreads) maxpool_2x2s2_planes_u8_kernel(const uint8_t *__restrict__ x, uint8_t *__restrict__ y,
+                                                                          int64_t NC, int G, int H, int W, int OH, int OW,
+                                                                          float inv_ohw8, float inv_ow8) {
+    typedef unsigned u4 __attribute__((ext_vector_type(4)));
+    typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+    __shared__ __attribute__((aligned(16))) uint8_t pl[kPoolLdsFloats * 4];
+    const int64_t p0 = int64_t(blockIdx.x) * G;
+    const int planes = int(min<int64_t>(G, NC - p0));
+    const int HW = H * W, OHW = OH * OW;
+    const int n_in16 = planes * HW / 16, n_out16 = planes * OHW / 16;
+    const u4 *src = reinterpret_cast<const u4 *>(x + p0 * HW);
+    constexpr int B = kPoolLdsFloats / 4 / kThreads;
+    for (int i0 = 0; i0 < n_in16; i0 += kThreads * B) {
+        u4 v[B];
+#pragma unroll
+        for (int u = 0; u < B; ++u) {
+            const int i = i0 + u * kThreads + int(threadIdx.x);
+            if (i < n_in16) v[u] = __builtin_nontemporal_load(src + i);
+        }
+#pragma unroll
+        for (int u = 0; u < B; ++u) {
+            const int i = i0 + u * kThreads + int(threadIdx.x);
+            if (i < n_in16) reinterpret_cast<u4 *>(pl)[i] = v[u];
+        }
+    }
+    __syncthreads();
+    auto pk = [](uint32_t v) { us2 r; r[0] = (unsigned short)(v & 0xffffu); r[1] = (unsigned short)(v >> 16); return r; };
+    auto window_max = [&](uint32_t a, uint32_t b) -> uint32_t {  // -> max(bytes 0,1) | max(bytes 2,3) << 16
+        const us2 e = __builtin_elementwise_max(pk(a & 0x00ff00ffu), pk(b & 0x00ff00ffu));
+        const us2 od = __builtin_elementwise_max(pk((a >> 8) & 0x00ff00ffu), pk((b >> 8) & 0x00ff00ffu));
+        const us2 h = __builtin_elementwise_max(e, od);
+        return uint32_t(h[0]) | (uint32_t(h[1]) << 16);
+    };
+    const int ohw8 = OHW / 8, ow8 = OW / 8;
+    u4 *dst = reinterpret_cast<u4 *>(y + p0 * OHW);
+    for (int i = int(threadIdx.x); i < n_out16; i += kThreads) {
+        u4 o;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int g8 = 2 * i + h;  // group of eight results: plane, result row, eight columns
+            const int pz = small_div_host(g8, ohw8, inv_ohw8), rem = g8 - pz * ohw8;
+            const int oh = small_div_host(rem, ow8, inv_ow8), oc = rem - oh * ow8;
+            const uint8_t *r = pl + pz * HW + 2 * oh * W + 16 * oc;
+            const u4 a = *reinterpret_cast<const u4 *>(r), b = *reinterpret_cast<const u4 *>(r + W);
+            o[2 * h] = __builtin_amdgcn_perm(window_max(a[1], b[1]), window_max(a[0], b[0]), 0x06040200u);
+            o[2 * h + 1] = __builtin_amdgcn_perm(window_max(a[3], b[3]), window_max(a[2], b[2]), 0x06040200u);
+        }
+        __builtin_nontemporal_store(o, dst + i);
     }
 }
 
@@ -436,6 +539,33 @@ int launch_maxpool(zant_ctx *ctx, const T *x, const int64_t xdim[4], T *y, const
     const bool stream = fast && g.H >= 2 * g.OH && g.OW % VEC == 0 && g.W % (sizeof(T) == 1 ? 16 : 2) == 0 &&
                         (reinterpret_cast<uintptr_t>(x) % (sizeof(T) == 1 ? 16 : 8)) == 0 &&
                         (reinterpret_cast<uintptr_t>(y) % (sizeof(T) == 1 ? 8 : 4)) == 0 && g.OW / VEC < (1 << 18) && g.OH < (1 << 18);
+    // f32 planes of a few KB whose rows are not whole vectors: the plane-staged kernel reads and writes 16-byte vectors
+    if (sizeof(T) == 4 && fast && g.W % 2 == 0 && g.W % 8 != 0 && int64_t(g.H) * g.W * 4 <= kPoolLdsFloats &&
+        int64_t(g.OH) * g.OW >= 4 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0) {
+        const int G = int(std::min<int64_t>((kPoolLdsFloats / (int64_t(g.H) * g.W)) & ~int64_t(3), 64));
+        if (G >= 4 && ceil_div64(g.NC, G) < (int64_t(1) << 31)) {
+            KernelTimer kt(ctx);
+            ZANT_KERNEL_NAME(ctx, "maxpool_2x2s2_planes_f32_kernel");
+            hipLaunchKernelGGL(maxpool_2x2s2_planes_f32_kernel, dim3(unsigned(ceil_div64(g.NC, G))), dim3(kThreads), 0, ctx->stream,
+                               reinterpret_cast<const float *>(x), reinterpret_cast<float *>(y), g.NC, G, g.H, g.W, g.OH, g.OW,
+                               1.0f / float(g.OH * g.OW), 1.0f / float(g.OW));
+            ZANT_LAUNCH_CHECK(ctx);
+            return ZANT_OK;
+        }
+    }
+    if (sizeof(T) == 1 && fast && g.W % 16 == 0 && g.OW % 8 == 0 && g.OW % 16 != 0 && (int64_t(g.OH) * g.OW) % 16 == 0 &&
+        int64_t(g.H) * g.W <= kPoolLdsFloats * 4 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0) {
+        const int G = int(std::min<int64_t>(kPoolLdsFloats * 4 / (int64_t(g.H) * g.W), 64));
+        if (G >= 1 && ceil_div64(g.NC, G) < (int64_t(1) << 31)) {
+            KernelTimer kt(ctx);
+            ZANT_KERNEL_NAME(ctx, "maxpool_2x2s2_planes_u8_kernel");
+            hipLaunchKernelGGL(maxpool_2x2s2_planes_u8_kernel, dim3(unsigned(ceil_div64(g.NC, G))), dim3(kThreads), 0, ctx->stream,
+                               reinterpret_cast<const uint8_t *>(x), reinterpret_cast<uint8_t *>(y), g.NC, G, g.H, g.W, g.OH, g.OW,
+                               1.0f / float(g.OH * g.OW / 8), 1.0f / float(g.OW / 8));
+            ZANT_LAUNCH_CHECK(ctx);
+            return ZANT_OK;
+        }
+    }
     if (stream) {
         const int ow_vec = g.OW / VEC;
         const int64_t total_vec = g.NC * g.OH * ow_vec;

@@ -1385,6 +1385,7 @@ int run_qdw_blocked(zant_ctx *ctx, const uint8_t *xb, const int8_t *w, const flo
     KernelTimer kt(ctx);
     if (per_cb < (int64_t(1) << 31) - 64 && int64_t(g.OH) * g.OW < (1 << 20) &&
         int64_t(g.N) * CB * g.H * g.W * 16 < (int64_t(1) << 32)) {
+        ZANT_KERNEL_NAME(ctx, "qdw3x3_mfma_kernel<%d>", (g.sh == 1 && g.sw == 1 && g.OH >= 2) ? 2 : 1);
         const int64_t want = std::max<int64_t>(1, (int64_t(ctx->num_cus) * 8 + n_pairs - 1) / n_pairs);
         const int blocks_per_pair = int(std::min<int64_t>(std::max<int64_t>(ceil_div64(per_cb, 128), 1), want));
         if (g.sh == 1 && g.sw == 1 && g.OH >= 2)

@@ -100,3 +100,42 @@ __device__ __forceinline__ uint32_t requant_lookup(float v, float zp_f, unsigned
     return *reinterpret_cast<const __attribute__((address_space(3))) uint8_t *>(addr);
 }
 
+typedef int zq_i32x4 __attribute__((ext_vector_type(4)));
+typedef int zq_i32x16 __attribute__((ext_vector_type(16)));
+
+// LDS reads the compiler does not see, so that it neither serialises them with waits of its own nor reorders them:
+// the kernel issues a batch (the nine taps of a position tile, the sixteen table lookups of a requantisation), keeps
+// computing, and waits with a counted s_waitcnt that hands the values to their users.  LDS operations complete in
+// order; operations the compiler issues in between only make a counted wait stricter.
+__device__ __forceinline__ void qb_read128(zq_i32x4 &v, unsigned addr, int imm) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "i"(imm));
+}
+__device__ __forceinline__ void qb_ready(zq_i32x4 &b, int pending) {
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(b) : "i"(pending));
+}
+__device__ __forceinline__ uint32_t qb_read_u8(unsigned addr) {
+    uint32_t v;
+    asm volatile("ds_read_u8 %0, %1" : "=v"(v) : "v"(addr));
+    return v;
+}
+__device__ __forceinline__ void qb_ready8(uint32_t *v) {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]));
+}
+// Requantises the accumulator values [V0, V0 + 8 * G) of one MFMA tile and looks their bytes up in the activation
+// table at `table` (256-byte aligned): all lookups of the batch are issued before the one wait.  d[g] receives the four
+// bytes of accumulator registers 4g .. 4g + 3.
+template <int G>
+__device__ __forceinline__ void qb_requant_lookup(const zq_i32x16 &acc, const float (&mv)[16], float zp_f, unsigned table,
+                                                  uint32_t (&d)[4]) {
+    uint32_t b[16];
+#pragma unroll
+    for (int v = 0; v < 4 * G; ++v)
+        b[v] = qb_read_u8(__builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(float(acc[v]) * mv[v]) + zp_f, 0u, table));
+    qb_ready8(b);
+    if (G > 2) qb_ready8(b + 8);
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+        d[g] = g < G ? (b[4 * g] | (b[4 * g + 1] << 8) | (b[4 * g + 2] << 16) | (b[4 * g + 3] << 24)) : 0u;
+}
+
