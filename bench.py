@@ -269,6 +269,9 @@ def main():
         yp = torch.empty(4096, 32, 13, 13, device=dev)
         hbm("maxpool2x2_f32_4096x32x26x26", lambda: tm.onnx_maxpool_lean(xf, yp, [2, 2], [2, 2], [1, 1], [0, 0, 0, 0]),
             xf.numel() * 5)
+        hbm("avgpool2x2_f32_4096x32x26x26", lambda: tm.avgpool_lean(xf, yp, [2, 2], [2, 2]), xf.numel() * 5)
+        bn = [torch.rand(32, device=dev) + 0.5 for _ in range(4)]
+        hbm("batchnorm_f32_4096x32x26x26", lambda: tm.batchnorm(xf, bn[0], bn[1], bn[2], bn[3], 1e-5, out=yf), 2 * xf.numel() * 4)
         bf = torch.randn(4096, 32, 26, 26, device=dev)
         hbm("add_f32_same_shape", lambda: tm.sum_tensors_lean(xf, bf, yf), 3 * xf.numel() * 4)
         bc = torch.randn(32, 1, 1, device=dev)

@@ -28,6 +28,9 @@ AVG_CASES = [
     ((2, 3, 9, 11), [3, 3], [2, 2], [1, 1, 1, 1], True, True),
     ((1, 5, 7, 7), [2, 3], [2, 2], [1, 0, 0, 2], True, False),
     ((3, 4, 6, 6), [6, 6], [1, 1], None, False, False),             # one window: the mean of the plane
+    ((5, 3, 26, 26), [2, 2], [2, 2], None, False, False),           # the plane-staged kernel, a partial last group
+    ((3, 7, 13, 26), [2, 2], [2, 2], None, False, False),           # planes that are not a whole number of vectors
+    ((3, 1, 10, 14), [2, 2], [2, 2], None, False, False),
 ]
 
 
@@ -38,6 +41,8 @@ def test_avgpool_vs_oracle(G, shape, k, s, pads, ceil_mode, include_pad):
     y = G.host(G.tm.avgpool(G.dev(x), k, s, pads, ceil_mode, include_pad))
     assert y.shape == ref.shape
     np.testing.assert_allclose(y, ref, rtol=G.RTOL, atol=G.ATOL)
+    if k == [2, 2] and s == [2, 2] and pads is None:  # these kernels add the four taps in the reference's order
+        np.testing.assert_array_equal(y, ref)
 
 
 def test_avgpool_errors(G):

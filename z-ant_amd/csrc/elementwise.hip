@@ -395,7 +395,8 @@ __global__ void __launch_bounds__(kThreads) maxpool_2x2s2_stream_kernel(const T 
 // and writes their G * OH * OW results, also a contiguous run, as 16-byte vectors, four results per thread.  The rows of
 // a window are two 8-byte LDS reads (W is even).  G is a multiple of 4, so both runs start on 16-byte boundaries.
 constexpr int kPoolLdsFloats = 4 * 1024;  // 16 KB: eight workgroups (all 32 wave slots) share a CU
-__global__ void __launch_bounds__(kThreads) maxpool_2x2s2_planes_f32_kernel(const float *__restrict__ x, float *__restrict__ y,
+template <bool AVG>  // AVG: the average in the reference's tap order (op_pooling.zig:373-408) instead of the maximum
+__global__ void __launch_bounds__(kThreads) pool_2x2s2_planes_f32_kernel(const float *__restrict__ x, float *__restrict__ y,
                                                                            int64_t NC, int G, int H, int W, int OH, int OW,
                                                                            float inv_ohw, float inv_ow) {
     typedef float f2 __attribute__((ext_vector_type(2)));
@@ -429,6 +430,7 @@ __global__ void __launch_bounds__(kThreads) maxpool_2x2s2_planes_f32_kernel(cons
         const int oh = small_div_host(rem, OW, inv_ow), ow = rem - oh * OW;
         const float *r = pl + pz * HW + 2 * oh * W + 2 * ow;
         const f2 a = *reinterpret_cast<const f2 *>(r), b = *reinterpret_cast<const f2 *>(r + W);
+        if (AVG) return (((a[0] + a[1]) + b[0]) + b[1]) / 4.0f;  // taps (0,0), (0,1), (1,0), (1,1), divided by their count
         return fmaxf(fmaxf(a[0], a[1]), fmaxf(b[0], b[1]));
     };
     const int n_out4 = n_out >> 2;
@@ -545,8 +547,8 @@ int launch_maxpool(zant_ctx *ctx, const T *x, const int64_t xdim[4], T *y, const
         const int G = int(std::min<int64_t>((kPoolLdsFloats / (int64_t(g.H) * g.W)) & ~int64_t(3), 64));
         if (G >= 4 && ceil_div64(g.NC, G) < (int64_t(1) << 31)) {
             KernelTimer kt(ctx);
-            ZANT_KERNEL_NAME(ctx, "maxpool_2x2s2_planes_f32_kernel");
-            hipLaunchKernelGGL(maxpool_2x2s2_planes_f32_kernel, dim3(unsigned(ceil_div64(g.NC, G))), dim3(kThreads), 0, ctx->stream,
+            ZANT_KERNEL_NAME(ctx, "pool_2x2s2_planes_f32_kernel<false>");
+            hipLaunchKernelGGL(pool_2x2s2_planes_f32_kernel<false>, dim3(unsigned(ceil_div64(g.NC, G))), dim3(kThreads), 0, ctx->stream,
                                reinterpret_cast<const float *>(x), reinterpret_cast<float *>(y), g.NC, G, g.H, g.W, g.OH, g.OW,
                                1.0f / float(g.OH * g.OW), 1.0f / float(g.OW));
             ZANT_LAUNCH_CHECK(ctx);
@@ -659,19 +661,36 @@ __global__ void __launch_bounds__(kThreads) batchnorm_f32_kernel(const float *__
 __global__ void __launch_bounds__(kThreads) batchnorm_vec_f32_kernel(const float *__restrict__ x, float *__restrict__ y,
                                                                      const float *__restrict__ gamma, const float *__restrict__ beta,
                                                                      const float *__restrict__ mean, const float *__restrict__ var,
-                                                                     float eps, int64_t total4, int64_t inner4, int features) {
+                                                                     float eps, int64_t total4, uint32_t inner4, uint32_t features) {
+    // the streaming pattern: a workgroup's ZANT_STREAM_U x 256 vectors are all loaded before any is stored
     typedef float f4 __attribute__((ext_vector_type(4)));
     const f4 *x4 = reinterpret_cast<const f4 *>(x);
     f4 *y4 = reinterpret_cast<f4 *>(y);
-    const int64_t step = int64_t(gridDim.x) * blockDim.x;
-    for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < total4; i += step) {
-        const int f = int((i / inner4) % features);
-        const float sd = sqrtf(var[f] + eps), m = mean[f], ga = gamma[f], be = beta[f];
-        const f4 v = __builtin_nontemporal_load(x4 + i);
-        f4 o;
+    const int64_t base = int64_t(blockIdx.x) * (kThreads * ZANT_STREAM_U) + threadIdx.x;
+    // (batch, feature) pair of the workgroup's first vector; the vectors of a thread are kThreads apart
+    const int64_t pair0 = (int64_t(blockIdx.x) * (kThreads * ZANT_STREAM_U)) / inner4;
+    const uint32_t off0 = uint32_t(int64_t(blockIdx.x) * (kThreads * ZANT_STREAM_U) - pair0 * inner4);
+    const uint32_t f0 = uint32_t(pair0 % features);
+    f4 v[ZANT_STREAM_U];
+    float sd[ZANT_STREAM_U], m[ZANT_STREAM_U], ga[ZANT_STREAM_U], be[ZANT_STREAM_U];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = (v[e] - m) / sd * ga + be;
-        __builtin_nontemporal_store(o, y4 + i);
+    for (int u = 0; u < ZANT_STREAM_U; ++u) {
+        const int64_t j = base + u * kThreads;
+        if (j < total4) {
+            v[u] = __builtin_nontemporal_load(x4 + j);
+            const uint32_t f = (f0 + (off0 + uint32_t(threadIdx.x) + uint32_t(u * kThreads)) / inner4) % features;
+            sd[u] = sqrtf(var[f] + eps); m[u] = mean[f]; ga[u] = gamma[f]; be[u] = beta[f];
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < ZANT_STREAM_U; ++u) {
+        const int64_t j = base + u * kThreads;
+        if (j < total4) {
+            f4 o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = (v[u][e] - m[u]) / sd[u] * ga[u] + be[u];
+            __builtin_nontemporal_store(o, y4 + j);
+        }
     }
 }
 
@@ -903,6 +922,20 @@ extern "C" int zant_hip_avgpool2d_f32(zant_ctx *ctx, const float *x, const int64
     if (!x || !y) return ZANT_NullPointer;
     const bool fast = g.kh == 2 && g.kw == 2 && g.sh == 2 && g.sw == 2 && !g.pt && !g.pl && 2 * g.OH <= g.H && 2 * g.OW <= g.W &&
                       g.OW % 2 == 0 && g.W % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 8 == 0;
+    // small planes, 2x2 / stride 2, no padding: the plane-staged kernel of the max pool
+    if (g.kh == 2 && g.kw == 2 && g.sh == 2 && g.sw == 2 && !g.pt && !g.pl && 2 * g.OH <= g.H && 2 * g.OW <= g.W && g.W % 2 == 0 &&
+        int64_t(g.H) * g.W * 4 <= kPoolLdsFloats && int64_t(g.OH) * g.OW >= 4 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+        reinterpret_cast<uintptr_t>(y) % 16 == 0) {
+        const int G = int(std::min<int64_t>((kPoolLdsFloats / (int64_t(g.H) * g.W)) & ~int64_t(3), 64));
+        if (G >= 4 && ceil_div64(g.NC, G) < (int64_t(1) << 31)) {
+            KernelTimer kt(ctx);
+            ZANT_KERNEL_NAME(ctx, "pool_2x2s2_planes_f32_kernel<true>");
+            hipLaunchKernelGGL(pool_2x2s2_planes_f32_kernel<true>, dim3(unsigned(ceil_div64(g.NC, G))), dim3(kThreads), 0, ctx->stream, x, y,
+                               g.NC, G, g.H, g.W, g.OH, g.OW, 1.0f / float(g.OH * g.OW), 1.0f / float(g.OW));
+            ZANT_LAUNCH_CHECK(ctx);
+            return ZANT_OK;
+        }
+    }
     KernelTimer kt(ctx);
     if (fast) {
         const int64_t total2 = total / 2;
@@ -949,9 +982,9 @@ extern "C" int zant_hip_batchnorm_f32(zant_ctx *ctx, const float *x, const int64
     if (xdim[1] > INT32_MAX) return ZANT_InvalidDimensions;
     if (!x || !y || !gamma || !beta || !mean || !var) return ZANT_NullPointer;
     KernelTimer kt(ctx);
-    if (inner % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0) {
-        hipLaunchKernelGGL(batchnorm_vec_f32_kernel, dim3(grid_for(total / 4, kThreads, ctx->num_cus)), dim3(kThreads), 0, ctx->stream,
-                           x, y, gamma, beta, mean, var, epsilon, total / 4, inner / 4, int(xdim[1]));
+    if (inner % 4 == 0 && inner / 4 < (int64_t(1) << 31) && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0) {
+        hipLaunchKernelGGL(batchnorm_vec_f32_kernel, dim3(zant_stream_grid(total / 4)), dim3(kThreads), 0, ctx->stream,
+                           x, y, gamma, beta, mean, var, epsilon, total / 4, uint32_t(inner / 4), uint32_t(xdim[1]));
     } else {
         hipLaunchKernelGGL(batchnorm_f32_kernel, dim3(grid_for(total, kThreads, ctx->num_cus)), dim3(kThreads), 0, ctx->stream, x, y,
                            gamma, beta, mean, var, epsilon, total, inner, int(xdim[1]));

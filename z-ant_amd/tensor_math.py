@@ -184,7 +184,7 @@ def avgpool(x, kernel, strides, pads=None, ceil_mode=False, count_include_pad=Fa
     return avgpool_lean(x, y, kernel, strides, pads, count_include_pad)
 
 
-def batchnorm(x, gamma, beta, mean, var, epsilon=1e-5):
+def batchnorm(x, gamma, beta, mean, var, epsilon=1e-5, out=None):
     """BatchNormLayer.forward, inference branch (batchNormLayer.zig:130-148), features on axis 1."""
     if x.dim() < 2:
         raise ZantError(-1)
@@ -192,7 +192,7 @@ def batchnorm(x, gamma, beta, mean, var, epsilon=1e-5):
         raise ZantError(-5)
     ctx = context()
     xd, xr = dims(x.shape)
-    y = torch.zeros_like(x)
+    y = torch.zeros_like(x) if out is None else out
     ctx.check(lib.zant_hip_batchnorm_f32(ctx.handle, _p(x), xd, xr, _p(gamma), _p(beta), _p(mean), _p(var), epsilon, _p(y)))
     return y
 
