@@ -4,6 +4,7 @@ Usage: python z-ant_amd/build.py            (from the repository root)
 """
 import glob
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -31,6 +32,9 @@ def sources():
 HOST_TEST = os.path.join(HERE, "host", "test_host_mirror")
 
 
+# sources whose kernels hide LDS reads from the compiler (checked for spills at build time, see build())
+NO_SPILL_SOURCES = {"qconv_ps_i8.hip", "qblock_i8.hip", "qconv_i8.hip", "conv_f32.hip", "gemm_f32.hip"}
+
 OBJ = os.path.join(HERE, "_obj")  # per-source objects (not tracked); every build recompiles all of them
 
 
@@ -44,7 +48,26 @@ def build(verbose=True):
     def run(job):
         if verbose:
             print(" ".join(job[1]), flush=True)
-        subprocess.check_call(job[1])
+        if os.path.basename(job[1][-3]) not in NO_SPILL_SOURCES:
+            subprocess.check_call(job[1])
+            return job[0]
+        # These sources issue LDS reads the compiler does not see and wait for them by hand.  A register that is in
+        # flight between such a read and its wait must not be copied: a spill to scratch taken in that window saves
+        # garbage.  So a kernel of these files that spills fails the build.
+        res = subprocess.run(job[1] + ["-Rpass-analysis=kernel-resource-usage"], stderr=subprocess.PIPE, text=True)
+        if res.returncode:
+            sys.stderr.write(res.stderr)
+            raise subprocess.CalledProcessError(res.returncode, job[1])
+        name, bad = None, []
+        for line in res.stderr.splitlines():
+            m = re.search(r"remark: Function Name: (\S+)", line)
+            if m:
+                name = m.group(1)
+            m = re.search(r"remark:\s+(VGPRs Spill): (\d+)", line)
+            if m and name and int(m.group(2)) > 0 and "_kernel" in name:
+                bad.append(f"{name}: {m.group(1)} = {m.group(2)}")
+        if bad:
+            raise RuntimeError("kernels with hand-scheduled LDS reads must not spill:\n  " + "\n  ".join(bad))
         return job[0]
 
     with ThreadPoolExecutor(max_workers=min(8, len(jobs))) as pool:  # one translation unit per core

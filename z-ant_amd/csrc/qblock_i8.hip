@@ -36,6 +36,8 @@ struct QBlockArgs {
     int NB, TH, PH, PW, P, Ppad, Q;    // tile: images, output rows, patch rows / columns / positions, output positions
     int n_row_tiles, n_tiles;
     int o_xl, o_e, o_w1, o_w2, o_wdw, o_tab, o_ptab;  // LDS byte offsets
+    int packed_units;                  // 16-byte units of weights and tables: the LDS bytes from o_w1 to o_ptab
+    int split;                         // stage D deals (position tile, channel chunk) units to the waves (few position tiles)
     float zp1f, zp2f, zp3f;            // zero points of the three convolutions' own outputs
     QAct act1, act2;
     int has_act1, has_act2;
@@ -53,12 +55,10 @@ __device__ __forceinline__ i32x4 as_i32x4(const uint4 &v) {
     return r;
 }
 
-template <int CO32, int MQ, bool PF>
-__global__ void __launch_bounds__(256, CO32 <= 2 ? 2 : 1)  // wide projections need the whole CU's LDS anyway
-qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 *__restrict__ w1p,
-              const uint4 *__restrict__ w2p, const uint32_t *__restrict__ wm, const float *__restrict__ mult1,
-              const int32_t *__restrict__ corr1, const float *__restrict__ mult2, const int32_t *__restrict__ corr2,
-              const float *__restrict__ mult3, const int32_t *__restrict__ corr3, QBlockArgs a) {
+template <int CO32, int MQ, bool PF, bool SPLIT>
+__global__ void __launch_bounds__(256, 2)  // 256 registers per lane for every instantiation: over that, values would be
+                                           // parked in accumulator registers, which the hand-issued LDS reads do not survive
+qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 *__restrict__ packed, QBlockArgs a) {
     extern __shared__ __attribute__((aligned(256))) char lds[];  // the activation tables need 256-byte alignment
     uint8_t *lut1 = reinterpret_cast<uint8_t *>(lds), *lut2 = lut1 + 256;
     uint4 *XL = reinterpret_cast<uint4 *>(lds + a.o_xl);   // [Cin32*2][Ppad] units of 16 channels
@@ -84,11 +84,13 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
         lut1[tid] = uint8_t((a.has_act1 ? qact_apply(b, a.act1) : b) ^ 0x80);
         lut2[tid] = uint8_t((a.has_act2 ? qact_apply(b, a.act2) : b) ^ 0x80);
     }
-    for (int i = tid; i < a.Cin32 * a.Ce32 * 64; i += 256) W1[i] = w1p[i];
-    for (int i = tid; i < a.Ce32 * CO32 * 64; i += 256) W2[i] = w2p[i];
-    for (int i = tid; i < Ce * 9; i += 256) WDW[i] = wm[i];
-    for (int k = tid; k < Ce; k += 256) { m1[k] = mult1[k]; c1[k] = corr1[k]; m2[k] = mult2[k]; c2[k] = corr2[k]; }
-    for (int k = tid; k < CO32 * 32; k += 256) { m3[k] = mult3[k]; c3[k] = corr3[k]; }
+    // weights and requantisation tables: `packed` holds them in the order and spacing of their LDS region, so they are
+    // one copy, eight 16-byte units per thread in flight at a time.  The first eight are loaded here and written to LDS
+    // behind the first tile's input patch, whose loads thereby travel with them.
+    i32x4 *wdst = reinterpret_cast<i32x4 *>(lds + a.o_w1);
+    i32x4 w0[8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) w0[r] = *reinterpret_cast<const i32x4 *>(packed + min(r * 256 + tid, a.packed_units - 1));
     {
         const int patch = a.PH * a.PW;
         const float inv_patch = 1.0f / float(patch), inv_pw = 1.0f / float(a.PW);
@@ -98,7 +100,6 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
             ptab[p] = (img << 20) | (ph << 10) | pw;
         }
     }
-    __syncthreads();
 
     const float inv_p = 1.0f / float(a.P), inv_nptiles = 1.0f / float(a.Ppad >> 5);
     const float inv_tile_img = 1.0f / float(a.TH * a.OW), inv_ow = 1.0f / float(a.OW);
@@ -115,13 +116,16 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
     // in front of it and written to LDS after that stage (the input patch is dead once B is done), so its global
     // latency passes under B.  Patches of more than QB_PF units per thread are copied in place instead. ----
     constexpr int QB_PF = 4;
+    const int patch_hw = a.PH * a.PW;
+    const float inv_patch_hw = 1.0f / float(patch_hw), inv_pw_ = 1.0f / float(a.PW);
     const int a_units = a.CBin * a.P;
     const bool prefetch = PF && a_units <= QB_PF * 256;  // PF is off for the instantiations without registers to spare
     auto patch_unit = [&](int tile_, int u, int &dst) -> const uint4 * {  // source of unit u of a tile's patch, or null
         const int ig_ = tile_ / a.n_row_tiles, rt_ = tile_ - ig_ * a.n_row_tiles;
         const int cb = small_div(u, a.P, inv_p), p = u - cb * a.P;
-        const int e = ptab[p];
-        const int n = ig_ * a.NB + (e >> 20), ih = rt_ * a.TH * a.stride - 1 + ((e >> 10) & 1023), iw = (e & 1023) - 1;
+        const int img = small_div(p, patch_hw, inv_patch_hw), rem = p - img * patch_hw;   // (not from the position table: the
+        const int ph = small_div(rem, a.PW, inv_pw_), pw = rem - ph * a.PW;               // first patch is fetched before it exists)
+        const int n = ig_ * a.NB + img, ih = rt_ * a.TH * a.stride - 1 + ph, iw = pw - 1;
         dst = cb * a.Ppad + p;
         if (n < a.N && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W) return x + ((int64_t(n) * a.CBin + cb) * a.H + ih) * int64_t(a.W) + iw;
         return nullptr;
@@ -144,6 +148,17 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
         }
     };
     if (int(blockIdx.x) < a.n_tiles) copy_patch(blockIdx.x);
+#pragma unroll
+    for (int r = 0; r < 8; ++r)
+        if (r * 256 + tid < a.packed_units) wdst[r * 256 + tid] = w0[r];
+    for (int i0 = 8 * 256; i0 < a.packed_units; i0 += 8 * 256) {
+        i32x4 v[8];
+#pragma unroll
+        for (int r = 0; r < 8; ++r) v[r] = *reinterpret_cast<const i32x4 *>(packed + min(i0 + r * 256 + tid, a.packed_units - 1));
+#pragma unroll
+        for (int r = 0; r < 8; ++r)
+            if (i0 + r * 256 + tid < a.packed_units) wdst[i0 + r * 256 + tid] = v[r];
+    }
     __syncthreads();
 
     for (int tile = blockIdx.x; tile < a.n_tiles; tile += gridDim.x) {
@@ -243,8 +258,14 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
 
         // ---- D: depthwise 3x3 + projection.  A wave takes MQ tiles of 32 output positions at a time; per chunk of 32
         // expanded channels the nine diagonal operands and the requantisation tables are set up once for all of them. ----
-        const int q_per_wave = (nq_tiles + 3) >> 2, q_end = min(nq_tiles, (wave + 1) * q_per_wave);
-        for (int q0 = wave * q_per_wave; q0 < q_end; q0 += MQ) {
+        // With few position tiles per workgroup tile (late, small feature maps) that split leaves waves idle while others
+        // walk every chunk: then (SPLIT) every wave holds all MQ = nq_tiles position tiles, the (position tile, chunk)
+        // units are dealt evenly to the four waves in position-tile-major order, and the waves' partial projection sums
+        // are added up in LDS (integer addition: the order does not matter) before wave j requantises position tile j.
+        const int q_per_wave = SPLIT ? nq_tiles : (nq_tiles + 3) >> 2;
+        const int q_end = SPLIT ? nq_tiles : min(nq_tiles, (wave + 1) * q_per_wave);
+        const int n_units = nq_tiles * a.Ce32, u_begin = (n_units * wave) >> 2, u_end = (n_units * (wave + 1)) >> 2;
+        for (int q0 = SPLIT ? 0 : wave * q_per_wave; q0 < q_end; q0 += MQ) {
             int p0[MQ], qimg[MQ], qr[MQ], qc[MQ];
             bool qvalid[MQ];
 #pragma unroll
@@ -263,11 +284,17 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
             for (int kb3 = 0; kb3 < CO32; ++kb3)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
-                    const int cv = c3[kb3 * 32 + lh * 4 + (v >> 2) * 8 + (v & 3)];
+                    const int cv = SPLIT ? 0 : c3[kb3 * 32 + lh * 4 + (v >> 2) * 8 + (v & 3)];  // split: added after the sum
 #pragma unroll
                     for (int j = 0; j < MQ; ++j) acc3[j][kb3][v] = cv;
                 }
             for (int ch = 0; ch < a.Ce32; ++ch) {
+                if (SPLIT) {  // does any position tile's unit of this chunk belong to this wave?
+                    bool any = false;
+#pragma unroll
+                    for (int j = 0; j < MQ; ++j) any |= j * a.Ce32 + ch >= u_begin && j * a.Ce32 + ch < u_end;
+                    if (!any) continue;
+                }
                 const int kch = ch * 32 + lh * 4;
                 const bool half = a.half_last && ch == a.Ce32 - 1;
                 i32x16 cvec;
@@ -298,9 +325,13 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
                     qb_read128(tap[3], r1, 0); qb_read128(tap[4], r1, 16); qb_read128(tap[5], r1, 32);
                     qb_read128(tap[6], r2, 0); qb_read128(tap[7], r2, 16); qb_read128(tap[8], r2, 32);
                 };
-                issue_taps(0);
+                if (!SPLIT) issue_taps(0);
 #pragma unroll
                 for (int j = 0; j < MQ; ++j) {
+                    if (SPLIT) {
+                        if (j * a.Ce32 + ch < u_begin || j * a.Ce32 + ch >= u_end) continue;
+                        issue_taps(j);
+                    }
                     qb_ready(tap[0], 8);
                     i32x16 acc2 = __builtin_amdgcn_mfma_i32_32x32x32_i8(wa[0], tap[0], cvec, 0, 0, 0);
 #pragma unroll
@@ -308,7 +339,7 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
                         qb_ready(tap[t], 8 - t);
                         acc2 = __builtin_amdgcn_mfma_i32_32x32x32_i8(wa[t], tap[t], acc2, 0, 0, 0);
                     }
-                    if (j + 1 < MQ) issue_taps(j + 1);
+                    if (j + 1 < MQ && !SPLIT) issue_taps(j + 1);
                     uint32_t d[4];
                     if (half) qb_requant_lookup<2>(acc2, mv, a.zp2f, lut2_a, d);
                     else qb_requant_lookup<4>(acc2, mv, a.zp2f, lut2_a, d);
@@ -322,6 +353,32 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
                         acc3[j][kb3] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w2a[kb3], db, acc3[j][kb3], 0, 0, 0);
                 }
             }
+            if (SPLIT) {
+                // the expanded patch is dead once every wave has left the chunk loop: its first bytes hold the sums,
+                // [position tile][output block][accumulator register][lane]
+                int *R = reinterpret_cast<int *>(E);
+                __syncthreads();
+                for (int i = tid; i < MQ * CO32 * 16 * 64; i += 256) R[i] = 0;
+                __syncthreads();
+#pragma unroll
+                for (int j = 0; j < MQ; ++j) {
+                    if (u_begin >= (j + 1) * a.Ce32 || u_end <= j * a.Ce32 || u_begin >= u_end) continue;  // no unit of tile j
+#pragma unroll
+                    for (int kb3 = 0; kb3 < CO32; ++kb3)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) atomicAdd(R + ((j * CO32 + kb3) * 16 + v) * 64 + lane, acc3[j][kb3][v]);
+                }
+                __syncthreads();
+#pragma unroll
+                for (int j = 0; j < MQ; ++j) {
+                    if (j != wave) continue;
+#pragma unroll
+                    for (int kb3 = 0; kb3 < CO32; ++kb3)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v)
+                            acc3[j][kb3][v] = R[((j * CO32 + kb3) * 16 + v) * 64 + lane] + c3[kb3 * 32 + lh * 4 + (v >> 2) * 8 + (v & 3)];
+                }
+            }
             auto store_tiles = [&](auto res_tag, auto fast_tag) {
                 constexpr bool RES = decltype(res_tag)::value, FAST = decltype(fast_tag)::value;
                 // byte offset of this lane's four channels in block 0 of its position (the host checks that the blocked
@@ -332,7 +389,7 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
 #pragma unroll
                 for (int j = 0; j < MQ; ++j) {
                     const int n = n0 + qimg[j], oh = oh0 + qr[j];
-                    ok[j] = qvalid[j] && n < a.N && oh < a.OH;
+                    ok[j] = qvalid[j] && n < a.N && oh < a.OH && (!SPLIT || j == wave);
                     ybase[j] = ((unsigned(n) * unsigned(a.CBo) * unsigned(a.OH) + unsigned(oh)) * unsigned(a.OW) + unsigned(qc[j])) * 16u + unsigned(lh) * 4u;
                 }
                 // the residual's bytes of every (tile, group) first, as one batch of loads
@@ -509,9 +566,13 @@ int zant_qblock_blocked(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], 
 
     // packed weights and tables of the three convolutions
     const size_t kp1 = size_t(CeP), kp3 = size_t(CO32) * 32;
-    const size_t o_w1p = 256, o_m1 = o_w1p + align256(w1_bytes), o_c1 = o_m1 + align256(kp1 * 4), o_w2p = o_c1 + align256(kp1 * 4),
-                 o_m3 = o_w2p + align256(w2_bytes), o_c3 = o_m3 + align256(kp3 * 4), o_wm = o_c3 + align256(kp3 * 4),
-                 o_m2 = o_wm + align256(wdw_bytes), o_c2 = o_m2 + align256(kp1 * 4), static_bytes = o_c2 + align256(kp1 * 4);
+    // in the order and spacing of the kernel's LDS region [o_w1, o_ptab): weights of the expansion, of the projection, of
+    // the depthwise convolution, then the tables m1 c1 m2 c2 (CeP entries each) m3 c3 (kp3 entries each)
+    const size_t o_w1p = 256, o_w2p = o_w1p + w1_bytes, o_wm = o_w2p + w2_bytes, o_m1 = o_wm + wdw_bytes, o_c1 = o_m1 + kp1 * 4,
+                 o_m2 = o_c1 + kp1 * 4, o_c2 = o_m2 + kp1 * 4, o_m3 = o_c2 + kp1 * 4, o_c3 = o_m3 + kp3 * 4,
+                 static_bytes = align256(o_c3 + kp3 * 4);
+    if (o_c3 + kp3 * 4 - o_w1p != w1_bytes + w2_bytes + wdw_bytes + tab_bytes || size_t(a.o_ptab - a.o_w1) != o_c3 + kp3 * 4 - o_w1p)
+        return ZANT_InvalidInput;  // the two layouts must stay in step
     void *ws = nullptr, *dyn = nullptr;
     bool need_pack = true;
     int parity = 0;
@@ -553,6 +614,7 @@ int zant_qblock_blocked(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], 
     a.fast_div = residual && zant_fast_div_ok(a.ra_scale, a.rb_scale, add_scale);
     a.ry_rcp = a.fast_div ? zant_refined_rcp(add_scale) : 0.0f;
 
+    a.packed_units = int((a.o_ptab - a.o_w1) / 16);
     const int per_cu = cap_used <= 76 * 1024 ? 2 : 1;
     const int grid = int(std::min<int64_t>(a.n_tiles, int64_t(ctx->num_cus) * per_cu));
     KernelTimer kt(ctx);
@@ -560,29 +622,36 @@ int zant_qblock_blocked(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], 
     const int nq_tiles = (a.Q + 31) / 32;
     const int q_per_wave = (nq_tiles + 3) / 4;
     const int rounds = (q_per_wave + mq_cap - 1) / mq_cap;
-    const int MQv = std::max(1, (q_per_wave + rounds - 1) / rounds);
-#define ZANT_QBLOCK_LAUNCH(CO, M, P)                                                                                          \
+    // fewer position tiles than waves: the waves share them chunk by chunk (their sums meet in the expanded patch's LDS)
+    a.split = CO32 <= 2 && nq_tiles < 4 && nq_tiles <= mq_cap && a.Ce32 >= 2 &&
+              size_t(nq_tiles) * CO32 * 4096 <= size_t(a.Ce32) * 2 * a.Ppad * 16;
+    const int MQv = a.split ? nq_tiles : std::max(1, (q_per_wave + rounds - 1) / rounds);
+#define ZANT_QBLOCK_LAUNCH(CO, M, P, S)                                                                                          \
     do {                                                                                                                    \
         static bool attr_set = false;                                                                                       \
         if (!attr_set) {                                                                                                    \
-            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&qblock_kernel<CO, M, P>),                               \
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&qblock_kernel<CO, M, P, S>),                               \
                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                             \
             attr_set = true;                                                                                                \
         }                                                                                                                   \
-        ZANT_KERNEL_NAME(ctx, "qblock_kernel<%d,%d,%s>", CO, M, P ? "true" : "false");                                          \
-        hipLaunchKernelGGL((qblock_kernel<CO, M, P>), dim3(grid), dim3(256), cap_used, ctx->stream,                           \
-                           reinterpret_cast<const uint4 *>(x), y, reinterpret_cast<const uint4 *>(w1p),                    \
-                           reinterpret_cast<const uint4 *>(w2p), wmk, m1, c1, m2, c2, m3, c3, a);                          \
+        ZANT_KERNEL_NAME(ctx, "qblock_kernel<%d,%d,%s,%s>", CO, M, P ? "true" : "false", S ? "true" : "false");                                          \
+        hipLaunchKernelGGL((qblock_kernel<CO, M, P, S>), dim3(grid), dim3(256), cap_used, ctx->stream,                           \
+                           reinterpret_cast<const uint4 *>(x), y, reinterpret_cast<const uint4 *>(base + o_w1p), a);       \
     } while (0)
-    switch (CO32 * 10 + MQv) {
-    case 11: ZANT_QBLOCK_LAUNCH(1, 1, true); break;
-    case 12: ZANT_QBLOCK_LAUNCH(1, 2, true); break;
-    case 13: ZANT_QBLOCK_LAUNCH(1, 3, true); break;
-    case 14: ZANT_QBLOCK_LAUNCH(1, 4, false); break;
-    case 21: ZANT_QBLOCK_LAUNCH(2, 1, true); break;
-    case 22: ZANT_QBLOCK_LAUNCH(2, 2, false); break;
-    case 31: ZANT_QBLOCK_LAUNCH(3, 1, true); break;
-    default: ZANT_QBLOCK_LAUNCH(4, 1, true); break;
+    switch ((a.split ? 100 : 0) + CO32 * 10 + MQv) {
+    case 11: ZANT_QBLOCK_LAUNCH(1, 1, true, false); break;
+    case 12: ZANT_QBLOCK_LAUNCH(1, 2, true, false); break;
+    case 13: ZANT_QBLOCK_LAUNCH(1, 3, false, false); break;
+    case 14: ZANT_QBLOCK_LAUNCH(1, 4, false, false); break;
+    case 21: ZANT_QBLOCK_LAUNCH(2, 1, true, false); break;
+    case 22: ZANT_QBLOCK_LAUNCH(2, 2, false, false); break;
+    case 31: ZANT_QBLOCK_LAUNCH(3, 1, true, false); break;
+    case 111: ZANT_QBLOCK_LAUNCH(1, 1, true, true); break;
+    case 112: ZANT_QBLOCK_LAUNCH(1, 2, true, true); break;
+    case 113: ZANT_QBLOCK_LAUNCH(1, 3, false, true); break;
+    case 121: ZANT_QBLOCK_LAUNCH(2, 1, true, true); break;
+    case 122: ZANT_QBLOCK_LAUNCH(2, 2, false, true); break;
+    default: ZANT_QBLOCK_LAUNCH(4, 1, true, false); break;
     }
 #undef ZANT_QBLOCK_LAUNCH
     ZANT_LAUNCH_CHECK(ctx);

@@ -570,7 +570,9 @@ bool ps_plan(const ConvGeom &g, int num_cus, PsGeom *out, size_t *lds_bytes, int
         t.P1s = (t.P1 + PS_NT - 1) / PS_NT * PS_NT;
         if (t.P1s / PS_NT > PS_RMAX || NB > 2047) return;
         t.npt = (S + 31) / 32;
-        const int per_wave = (t.npt + NG - 1) / NG;
+        // (two position slots per wave at least: the one-slot instantiation needs more registers than it has, and a
+        // kernel whose LDS reads are hidden from the compiler must not spill)
+        const int per_wave = std::max(2, (t.npt + NG - 1) / NG);
         const size_t lds = fixed + size_t(per_wave) * PS_NT * 4 + size_t(2 * t.NC) * t.P1s * 16;
         if (lds > cap) return;
         t.n_row_tiles = (g.OH + TH - 1) / TH;
@@ -628,7 +630,7 @@ int zant_qconv_ps(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float 
     size_t lds = 0;
     int MT = 0;
     if (!ps_plan(g, ctx->num_cus, &p, &lds, &MT)) return 1;
-    if (MT < 1 || MT > PS_MTMAX) return 1;
+    if (MT < 2 || MT > PS_MTMAX) return 1;
     if (plan_only) return ZANT_OK;
     const size_t wp_bytes = size_t(p.NKP) * p.NC * 9 * 32 * p.KP;
     const size_t xb_bytes = x_blocked ? 0 : size_t(g.N) * p.CB * g.H * g.W * 16;
@@ -662,7 +664,6 @@ int zant_qconv_ps(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float 
     const int yb = y_blocked ? 1 : 0;
     const char *tabs = base + o_mult;
     switch (MT) {
-    case 1: ps_launch<1>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q, yb); break;
     case 2: ps_launch<2>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q, yb); break;
     case 3: ps_launch<3>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q, yb); break;
     default: ps_launch<4>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q, yb); break;
