@@ -108,7 +108,7 @@ inline bool zant_plan_conv_tiles(const ConvGeom &g, int WM, int WN, int mt_max, 
         if (target_tiles > 0) {
             const double rounds = double((t.n_tiles + target_tiles - 1) / target_tiles);
             const double mfma = rounds * 2.0 * t.n_chunks * mt * T * mfma_cycles_per_tap;                 // cycles
-            const double stage = double(t.n_tiles) * t.n_chunks * (double(w_slab) + 32.0 * t.P1s) / 2500.0;  // cycles at 6 TB/s
+            const double stage = double(t.n_tiles) * t.n_chunks * (double(w_slab) + 32.0 * t.P1s) / 7000.0;  // cycles at the measured L2 -> LDS copy rate (17 TB/s and up)
             score = 1.0e6 / (mfma > stage ? mfma : stage);
         }
         if (!found || score > best->score * 1.02) {  // larger tiles win ties: fewer tiles, more operand reuse
