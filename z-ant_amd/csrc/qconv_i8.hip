@@ -890,6 +890,7 @@ int launch_smallc(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float 
         ZANT_LAUNCH_CHECK(ctx);
     }
     const int64_t positions = int64_t(g.N) * (pool ? g.OH / 2 : g.OH) * (pool ? g.OW / 2 : g.OW);
+    if (positions * ((g.K + 15) / 16) >= (int64_t(1) << 31)) return 1;  // blocked output units are addressed in 32 bits
     const unsigned blocks = unsigned(std::min<int64_t>(std::max<int64_t>(ceil_div64(positions, 256), 1), int64_t(ctx->num_cus) * 32));
     KernelTimer kt(ctx);
     const int yb = y_blocked ? 1 : 0;
@@ -944,9 +945,10 @@ qfirst_mfma_kernel(const uint8_t *__restrict__ x, const uint4 *__restrict__ wpk,
                    const int32_t *__restrict__ corr, uint8_t *__restrict__ y, ConvGeom g, QConvArgs q, int y_blocked, int kb32) {
     constexpr int RW = C * 3, NCH = (RW + 7) / 8;
     constexpr int PR = POOL ? 4 : 3, NWIN = POOL ? 4 : 1;
-    __shared__ uint8_t lut[256];  // the fused activation as a byte table, in the byte values the output stores
+    __shared__ __attribute__((aligned(256))) uint8_t lut[256];  // the fused activation as a byte table, in the byte values the output stores
     lut[threadIdx.x] = uint8_t((q.has_act ? qact_apply(uint8_t(threadIdx.x), q.act) : uint8_t(threadIdx.x)) ^ (y_blocked ? 0x80 : 0));
     __syncthreads();
+    const unsigned lut_a = lds_address(lut);  // 256-byte aligned: a converted byte is the low byte of the entry's address
     const int lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
     const int OHo = POOL ? g.OH / 2 : g.OH, OWo = POOL ? g.OW / 2 : g.OW;
     const int KB16 = (g.K + 15) >> 4;
@@ -960,8 +962,8 @@ qfirst_mfma_kernel(const uint8_t *__restrict__ x, const uint4 *__restrict__ wpk,
     const unsigned wave_id = (blockIdx.x * blockDim.x + threadIdx.x) >> 6, n_waves = (gridDim.x * blockDim.x) >> 6;
     i32x16 cvec;
     float mv[16];
-    i32x4 wa_all[NCH];
-    bool tables_loaded = false;
+    i32x4 wa_all[NCH], wa_dx1[NCH];
+    bool tables_loaded = false, any_negative = false;
     // The row loads of the NEXT tile are issued before this tile's arithmetic: with two wavefronts per SIMD the load
     // latency would otherwise sit on the critical path of every tile.
     struct TileMeta { unsigned n; int oho, owo, ih0, sh; bool valid; };
@@ -1017,60 +1019,76 @@ qfirst_mfma_kernel(const uint8_t *__restrict__ x, const uint4 *__restrict__ wpk,
                     mv[v] = mult[kch + (v >> 2) * 8 + (v & 3)];
                 }
 #pragma unroll
-                for (int ch = 0; ch < NCH; ++ch) wa_all[ch] = as_i32x4_q(wpk[((kb * NCH + ch) * 2 + lh) * 32 + l32]);
+                for (int ch = 0; ch < NCH; ++ch) {
+                    wa_all[ch] = as_i32x4_q(wpk[((kb * NCH + ch) * 2 + lh) * 32 + l32]);
+                    // the window member one column to the right reads the same four input columns against the filter
+                    // row moved up one byte (columns 1..3 instead of 0..2): the shift is in the weights, once per table
+                    // load, instead of in every activation operand
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) wa_dx1[ch][e] = int(uint32_t(wa_all[ch][e]) << 8);
+                }
+                any_negative = false;
+#pragma unroll
+                for (int v = 0; v < NV; ++v) any_negative |= mv[v] < 0.0f;
+                any_negative = __builtin_amdgcn_ballot_w64(any_negative) != 0;
                 tables_loaded = true;
             }
             i32x16 acc[NWIN];
 #pragma unroll
             for (int ch = 0; ch < NCH; ++ch) {
-                const i32x4 wa = wa_all[ch];
 #pragma unroll
-                for (int wd = 0; wd < NWIN; ++wd) {
-                    const int dy = wd >> 1, dx = wd & 1;
+                for (int dy = 0; dy < (POOL ? 2 : 1); ++dy) {
                     i32x4 b;
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         // reduction rows ch*8 + j (lanes (p, 0)) and ch*8 + 4 + j (lanes (p, 1)): (channel, filter row)
                         const int ra = ch * 8 + j, rb = ch * 8 + 4 + j;
-                        const uint32_t va = ra < RW ? row[ra / 3][ra % 3 + dy] >> (8 * dx) : 0u;
-                        const uint32_t vb = rb < RW ? row[rb / 3][rb % 3 + dy] >> (8 * dx) : 0u;
+                        const uint32_t va = ra < RW ? row[ra / 3][ra % 3 + dy] : 0u;
+                        const uint32_t vb = rb < RW ? row[rb / 3][rb % 3 + dy] : 0u;
                         b[j] = int(lh ? vb : va);
                     }
-                    acc[wd] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wa, b, ch == 0 ? cvec : acc[wd], 0, 0, 0);
+#pragma unroll
+                    for (int dx = 0; dx < (POOL ? 2 : 1); ++dx) {
+                        const int wd = dy * 2 + dx;
+                        acc[wd] = __builtin_amdgcn_mfma_i32_32x32x32_i8(dx ? wa_dx1[ch] : wa_all[ch], b, ch == 0 ? cvec : acc[wd], 0, 0, 0);
+                    }
                 }
             }
             if (POOL) {
-                // requantisation and the activation keep (multiplier >= 0) or reverse (< 0) the order of the accumulators
+                // requantisation and the activation keep (multiplier >= 0) or reverse (< 0) the order of the accumulators;
+                // scales are positive in practice, and then the minima are never computed
+                if (!any_negative) {
 #pragma unroll
-                for (int v = 0; v < NV; ++v) {
-                    const int a0 = acc[0][v], a1 = acc[NWIN > 1 ? 1 : 0][v], a2 = acc[NWIN > 2 ? 2 : 0][v], a3 = acc[NWIN > 3 ? 3 : 0][v];
-                    const int mx = max(max(a0, a1), max(a2, a3)), mn = min(min(a0, a1), min(a2, a3));
-                    acc[0][v] = mv[v] >= 0.0f ? mx : mn;
+                    for (int v = 0; v < NV; ++v) acc[0][v] = max(max(acc[0][v], acc[1][v]), max(acc[2][v], acc[3][v]));
+                } else {
+#pragma unroll
+                    for (int v = 0; v < NV; ++v) {
+                        const int a0 = acc[0][v], a1 = acc[1][v], a2 = acc[2][v], a3 = acc[3][v];
+                        const int mx = max(max(a0, a1), max(a2, a3)), mn = min(min(a0, a1), min(a2, a3));
+                        acc[0][v] = mv[v] >= 0.0f ? mx : mn;
+                    }
                 }
             }
-            uint32_t ob[16];
-#pragma unroll
-            for (int v = 0; v < 16; ++v) ob[v] = v < NV ? uint32_t(lut[sat_u8_rne_finite(float(acc[0][v]) * mv[v], zpf)]) : 0u;
+            // the table lookups of the tile as one batch behind one wait
+            uint32_t d[4];
+            qb_requant_lookup<NV / 4>(acc[0], mv, zpf, lut_a, d);
             if (y_blocked) {
-                uint32_t d[4];
-#pragma unroll
-                for (int gq = 0; gq < 4; ++gq) d[gq] = ob[gq * 4] | (ob[gq * 4 + 1] << 8) | (ob[gq * 4 + 2] << 16) | (ob[gq * 4 + 3] << 24);
-#pragma unroll
-                for (int b = 0; b < 2; ++b) {
-                    const uint32_t send = lh ? d[2 * b] : d[2 * b + 1];
-                    const uint32_t recv = uint32_t(__shfl_xor(int(send), 32, 64));
-                    const uint2 out = lh ? make_uint2(recv, d[2 * b + 1]) : make_uint2(d[2 * b], recv);
-                    const int cbq = kb * 2 + b;
-                    if (valid && cbq < KB16) {
-                        uint8_t *yp = y + (((int64_t(n) * KB16 + cbq) * OHo + oho) * int64_t(OWo) + owo) * 16 + lh * 8;
-                        *reinterpret_cast<uint2 *>(yp) = out;
-                    }
+                // the half-wave swap leaves lane (p, 0) with the 16 bytes of the first block of 16 channels of its
+                // position and lane (p, 1) with those of the second: one 16-byte store per lane
+                const auto s0 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
+                const auto s1 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
+                i32x4 out;
+                out[0] = int(s0[0]); out[1] = int(s0[1]); out[2] = int(s1[0]); out[3] = int(s1[1]);
+                const int cbq = kb * 2 + lh;
+                if (valid && cbq < KB16) {
+                    const unsigned off = ((n * unsigned(KB16) + unsigned(cbq)) * unsigned(OHo) + unsigned(oho)) * unsigned(OWo) + unsigned(owo);
+                    *reinterpret_cast<i32x4 *>(y + size_t(off) * 16) = out;
                 }
             } else if (valid) {
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     const int k = kch + (v >> 2) * 8 + (v & 3);
-                    if (k < g.K) y[((int64_t(n) * g.K + k) * OHo + oho) * int64_t(OWo) + owo] = uint8_t(ob[v]);
+                    if (k < g.K) y[((int64_t(n) * g.K + k) * OHo + oho) * int64_t(OWo) + owo] = uint8_t(d[v >> 2] >> (8 * (v & 3)));
                 }
             }
         }
@@ -1108,6 +1126,7 @@ int launch_qfirst(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float 
         ZANT_LAUNCH_CHECK(ctx);
     }
     const int64_t positions = int64_t(g.N) * (pool ? g.OH / 2 : g.OH) * (pool ? g.OW / 2 : g.OW);
+    if (positions * ((g.K + 15) / 16) >= (int64_t(1) << 31)) return 1;  // blocked output units are addressed in 32 bits
     const unsigned blocks = unsigned(std::min<int64_t>(std::max<int64_t>(ceil_div64(positions, 128), 1), int64_t(ctx->num_cus) * 16));
     KernelTimer kt(ctx);
     const int yb = y_blocked ? 1 : 0;
