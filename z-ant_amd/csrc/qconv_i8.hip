@@ -1127,22 +1127,31 @@ int launch_qfirst(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float 
     }
     const int64_t positions = int64_t(g.N) * (pool ? g.OH / 2 : g.OH) * (pool ? g.OW / 2 : g.OW);
     if (positions * ((g.K + 15) / 16) >= (int64_t(1) << 31)) return 1;  // blocked output units are addressed in 32 bits
-    const unsigned blocks = unsigned(std::min<int64_t>(std::max<int64_t>(ceil_div64(positions, 128), 1), int64_t(ctx->num_cus) * 16));
-    KernelTimer kt(ctx);
+    // One resident generation of workgroups walks all the tiles: a workgroup's set-up (the activation table, the
+    // weights and tables of its channel block) is paid once per wave slot, not once per two tiles.
     const int yb = y_blocked ? 1 : 0;
+    KernelTimer kt(ctx);
+#define ZANT_QFIRST_NV(SV, PV, NVV)                                                                                         \
+    do {                                                                                                                    \
+        static int per_cu = 0;                                                                                              \
+        if (!per_cu && hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, qfirst_mfma_kernel<C, SV, PV, NVV>, 256, 0) != hipSuccess) \
+            per_cu = 2;                                                                                                     \
+        const unsigned blocks = unsigned(std::min<int64_t>(std::max<int64_t>(ceil_div64(positions, 128), 1),              \
+                                                           int64_t(ctx->num_cus) * std::max(per_cu, 1)));                   \
+        ZANT_KERNEL_NAME(ctx, "qfirst_mfma_kernel<%d,%d,%s,%d>", C, SV, PV ? "true" : "false", NVV);                        \
+        hipLaunchKernelGGL((qfirst_mfma_kernel<C, SV, PV, NVV>), dim3(blocks), dim3(256), 0, ctx->stream, x,               \
+                           reinterpret_cast<const uint4 *>(wpk), mult, corr, y, g, q, yb, kb32);                           \
+    } while (0)
 #define ZANT_QFIRST(SV, PV)                                                                                                 \
     do {                                                                                                                    \
-        if (g.K <= 16)                                                                                                      \
-            hipLaunchKernelGGL((qfirst_mfma_kernel<C, SV, PV, 8>), dim3(blocks), dim3(256), 0, ctx->stream, x,             \
-                               reinterpret_cast<const uint4 *>(wpk), mult, corr, y, g, q, yb, kb32);                       \
-        else                                                                                                                \
-            hipLaunchKernelGGL((qfirst_mfma_kernel<C, SV, PV, 16>), dim3(blocks), dim3(256), 0, ctx->stream, x,            \
-                               reinterpret_cast<const uint4 *>(wpk), mult, corr, y, g, q, yb, kb32);                       \
+        if (g.K <= 16) ZANT_QFIRST_NV(SV, PV, 8);                                                                           \
+        else ZANT_QFIRST_NV(SV, PV, 16);                                                                                    \
     } while (0)
     if (pool) ZANT_QFIRST(1, true);
     else if (g.sh == 1) ZANT_QFIRST(1, false);
     else ZANT_QFIRST(2, false);
 #undef ZANT_QFIRST
+#undef ZANT_QFIRST_NV
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
 }
