@@ -1414,7 +1414,16 @@ int run_qdw_blocked(zant_ctx *ctx, const uint8_t *xb, const int8_t *w, const flo
     if (per_cb < (int64_t(1) << 31) - 64 && int64_t(g.OH) * g.OW < (1 << 20) &&
         int64_t(g.N) * CB * g.H * g.W * 16 < (int64_t(1) << 32)) {
         ZANT_KERNEL_NAME(ctx, "qdw3x3_mfma_kernel<%d>", (g.sh == 1 && g.sw == 1 && g.OH >= 2) ? 2 : 1);
-        const int64_t want = std::max<int64_t>(1, (int64_t(ctx->num_cus) * 8 + n_pairs - 1) / n_pairs);
+        // one resident generation of workgroups (three share a CU at this kernel's register count): a workgroup's
+        // set-up -- the activation table, the nine diagonal operands, the tables -- is paid once per wave slot
+        static int per_cu[2] = {0, 0};
+        const int rows2 = (g.sh == 1 && g.sw == 1 && g.OH >= 2) ? 1 : 0;
+        if (!per_cu[rows2]) {
+            const hipError_t e = rows2 ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu[1], qdw3x3_mfma_kernel<2>, 256, 0)
+                                       : hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu[0], qdw3x3_mfma_kernel<1>, 256, 0);
+            if (e != hipSuccess || per_cu[rows2] < 1) per_cu[rows2] = 2;
+        }
+        const int64_t want = std::max<int64_t>(1, (int64_t(ctx->num_cus) * per_cu[rows2] + n_pairs - 1) / n_pairs);
         const int blocks_per_pair = int(std::min<int64_t>(std::max<int64_t>(ceil_div64(per_cb, 128), 1), want));
         if (g.sh == 1 && g.sw == 1 && g.OH >= 2)
             hipLaunchKernelGGL(qdw3x3_mfma_kernel<2>, dim3(unsigned(n_pairs) * blocks_per_pair), dim3(256), 0, ctx->stream,
