@@ -29,6 +29,12 @@ QCASES = [
     (1, 8, 6, 6, 4, 3, 3, [2, 1], [0, 1, 2, 0], [1, 1], 2),         # grouped, asymmetric pads
     (1, 3, 9, 9, 5, 2, 2, [1, 1], [0, 0, 0, 0], [2, 2], 1),         # dilation
     (4, 1280, 1, 1, 1000, 1, 1, [1, 1], [0, 0, 0, 0], [1, 1], 1),   # final Gemm as a 1x1 conv
+    # the same on the matrix cores (64 images and up), where 16-channel blocks are regrouped 8, 4 or 2 at a time:
+    (96, 1280, 1, 1, 1000, 1, 1, [1, 1], [0, 0, 0, 0], [1, 1], 1),  # 80 blocks: groups of 8
+    (64, 192, 1, 1, 33, 1, 1, [1, 1], [0, 0, 0, 0], [1, 1], 1),     # 12 blocks: groups of 4
+    (65, 90, 1, 1, 70, 1, 1, [1, 1], [0, 0, 0, 0], [1, 1], 1),      # 6 blocks, the last one partly filled: groups of 2
+    (128, 64, 1, 1, 64, 1, 1, [2, 2], [0, 0, 0, 0], [1, 1], 1),     # 4 blocks: groups of 2 (a stride changes nothing)
+    (70, 200, 1, 1, 40, 1, 1, [1, 1], [0, 0, 0, 0], [1, 1], 1),     # 13 blocks: not regrouped
 ]
 
 

@@ -123,14 +123,15 @@ __global__ void __launch_bounds__(256) to_blocked_s8_kernel(const uint8_t *__res
     }
 }
 
-// Packs OIHW int8 weights into [chunk][kblock][tap][half][K_BLK][16] (zero padded), and writes the
+// Packs OIHW int8 weights into [chunk][kblock][tap][half][K_BLK][16] (zero padded; fc_g > 0: the weights of a 1x1
+// layer with c_orig channels, read as a 1 x fc_g filter over C = 16 * ceil(c_orig / 16) / fc_g channels), and writes the
 // per-channel requantisation multiplier, the integer correction (bias + (128 - x_zp) * sum w), the
 // 16-byte padding vector (x_zp - 128 in every lane).
 __global__ void __launch_bounds__(256)
 qpack_kernel(const int8_t *__restrict__ w, const float *__restrict__ w_scale, const int32_t *__restrict__ bias,
              int8_t *__restrict__ wp, float *__restrict__ mult, int32_t *__restrict__ corr, int8_t *__restrict__ padvec,
              int K, int C, int T, int n_chunks, int n_kblocks, int k_blk,
-             float x_scale, float y_scale, int x_zp, int n_wscale) {
+             float x_scale, float y_scale, int x_zp, int n_wscale, int fc_g, int c_orig) {
     const int64_t total = int64_t(n_chunks) * n_kblocks * T * QCC * k_blk;
     const int64_t step = int64_t(gridDim.x) * blockDim.x;
     const int64_t gid = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -144,7 +145,13 @@ qpack_kernel(const int8_t *__restrict__ w, const float *__restrict__ w_scale, co
         const int kb = int(r % n_kblocks); r /= n_kblocks;
         const int chunk = int(r);
         const int k = kb * k_blk + kk, c = chunk * QCC + half * 16 + j;
-        wp[i] = (k < K && c < C) ? w[(int64_t(k) * C + c) * T + tap] : int8_t(0);
+        if (fc_g) {
+            // regrouped 1x1 layer: "tap" t of 16-channel block b is channel block b * fc_g + t of the c_orig real channels
+            const int oc = ((c >> 4) * fc_g + tap) * 16 + j;
+            wp[i] = (k < K && oc < c_orig) ? w[int64_t(k) * c_orig + oc] : int8_t(0);
+        } else {
+            wp[i] = (k < K && c < C) ? w[(int64_t(k) * C + c) * T + tap] : int8_t(0);
+        }
     }
     // per output channel: one wavefront sums the channel's weights
     const int kpad = n_kblocks * k_blk;
@@ -153,8 +160,9 @@ qpack_kernel(const int8_t *__restrict__ w, const float *__restrict__ w_scale, co
     for (int64_t k = wave; k < kpad; k += n_waves) {
         int sum = 0;
         if (k < K) {
-            const int8_t *wk = w + k * int64_t(C) * T;
-            for (int e = lane; e < C * T; e += 64) sum += int(wk[e]);
+            const int row = fc_g ? c_orig : C * T;
+            const int8_t *wk = w + k * int64_t(row);
+            for (int e = lane; e < row; e += 64) sum += int(wk[e]);
         }
         for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
         if (lane == 0) {
@@ -630,13 +638,31 @@ unsigned to_blocked_grid(zant_ctx *ctx, int64_t N, int64_t CB, int64_t hw) {
 // The matrix-core path; returns ZANT_OK when it ran, 1 when the shape is left to the other kernels.
 // x_blocked / y_blocked: x, y are already / are to be written in the blocked signed layout.
 int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float *w_scale, const int32_t *bias, uint8_t *y,
-                   const ConvGeom &g, const QConvArgs &q, bool x_blocked, bool y_blocked, zant_pack_slot *slot, bool pool = false,
+                   const ConvGeom &g0, const QConvArgs &q, bool x_blocked, bool y_blocked, zant_pack_slot *slot, bool pool = false,
                    bool plan_only = false) {
-    if (g.groups != 1 || g.C < 5 || int64_t(g.N) * g.OH * g.OW < 64) return 1;
+    if (g0.groups != 1 || g0.C < 5 || int64_t(g0.N) * g0.OH * g0.OW < 64) return 1;
     if (!pool) {
         // 3x3 / stride 1 layers with at least 32 channels on both sides: the patch-stationary kernel
-        const int rc = zant_qconv_ps(ctx, x, w, w_scale, bias, y, g, q, x_blocked, y_blocked, slot, plan_only);
+        const int rc = zant_qconv_ps(ctx, x, w, w_scale, bias, y, g0, q, x_blocked, y_blocked, slot, plan_only);
         if (rc <= 0) return rc;
+    }
+    // A 1x1 layer over 1x1 feature maps (a classifier head behind a global pool) is a matrix product whose rows, the
+    // images, are ceil(C / 16) * 16 contiguous bytes each.  Staged 32 channels at a time it runs C / 32 short steps of
+    // 32-byte copies, one cache line each.  Read instead as a 1 x G filter over a 1 x G "image" of C / G channels -- G
+    // consecutive 16-channel blocks taken as G columns: the same bytes, the same sums -- it runs G times fewer steps,
+    // each copying G times longer contiguous runs.  Only the weight packing knows the difference.
+    ConvGeom g = g0;
+    int fc_g = 0;
+    if (!pool && g0.H == 1 && g0.W == 1 && g0.KH == 1 && g0.KW == 1 && g0.OH == 1 && g0.OW == 1 && g0.pt == 0 && g0.pl == 0) {
+        const int cb = (g0.C + 15) / 16;
+        for (int cand = 8; cand >= 2 && !fc_g; cand >>= 1)
+            if (cb % cand == 0 && cb / cand >= 2) fc_g = cand;
+        if (fc_g) {
+            g.C = cb / fc_g * 16;
+            g.CG = g.C;
+            g.W = g.KW = fc_g;
+            g.sh = g.sw = g.dh = g.dw = 1;
+        }
     }
     // a fused 2x2/2 max pool needs whole windows and an activation that keeps the order of its inputs
     if (pool && (g.OH < 2 || g.OW < 2 || (q.has_act && !(q.act.alpha >= 0.0f && q.act.in_scale > 0.0f && q.act.out_scale > 0.0f))))
@@ -682,7 +708,8 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
     plan.lds_bytes = n_stages * buf_bytes + fixed_bytes;
     const size_t wp_bytes = size_t(plan.t.n_chunks) * plan.t.n_kblocks * T * QCC * K_BLK;
     const size_t kpad = size_t(plan.t.n_kblocks) * K_BLK;
-    const size_t xb_bytes = x_blocked ? 0 : size_t(g.N) * CB * g.H * g.W * 16;
+    const int CB0 = (g0.C + 15) / 16;
+    const size_t xb_bytes = x_blocked ? 0 : size_t(g0.N) * CB0 * g0.H * g0.W * 16;
     const size_t o_pad = 256, o_mult = 512, o_corr = o_mult + align256(kpad * 4), o_wp = o_corr + align256(kpad * 4),
                  static_bytes = o_wp + align256(wp_bytes);
     void *ws = nullptr, *dyn = nullptr;
@@ -701,14 +728,14 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
     if (need_pack) {
         hipLaunchKernelGGL(qpack_kernel, dim3(pb), dim3(256), 0, ctx->stream, w, w_scale, bias, wp, mult, corr, padvec,
                            g.K, g.C, T, plan.t.n_chunks, plan.t.n_kblocks, K_BLK, q.x_scale, q.y_scale, q.x_zp,
-                           q.n_wscale);
+                           q.n_wscale, fc_g, g0.C);
         ZANT_LAUNCH_CHECK(ctx);
     }
     if (!x_blocked) {
-        const int64_t hw = int64_t(g.H) * g.W;
+        const int64_t hw = int64_t(g0.H) * g0.W;
         const int vec_ok = (hw % 4 == 0) && (reinterpret_cast<uintptr_t>(x) % 4 == 0);
-        hipLaunchKernelGGL(to_blocked_s8_kernel, dim3(to_blocked_grid(ctx, g.N, CB, hw)), dim3(256), 0, ctx->stream, x,
-                           static_cast<uint4 *>(dyn), g.N, g.C, CB, hw, vec_ok);
+        hipLaunchKernelGGL(to_blocked_s8_kernel, dim3(to_blocked_grid(ctx, g0.N, CB0, hw)), dim3(256), 0, ctx->stream, x,
+                           static_cast<uint4 *>(dyn), g0.N, g0.C, CB0, hw, vec_ok);
         ZANT_LAUNCH_CHECK(ctx);
     }
     KernelTimer kt(ctx);
@@ -1451,7 +1478,7 @@ int zant_qpack_dense(zant_ctx *ctx, const int8_t *w, const float *w_scale, int64
     const int64_t wp_bytes = int64_t(n_chunks) * n_kblocks * T * QCC * k_blk, kpad = int64_t(n_kblocks) * k_blk;
     const unsigned pb = unsigned(std::min<int64_t>(std::max<int64_t>(ceil_div64(wp_bytes, 256), ceil_div64(kpad, 4)), 1024));
     hipLaunchKernelGGL(qpack_kernel, dim3(pb), dim3(256), 0, ctx->stream, w, w_scale, bias, wp, mult, corr, padvec,
-                       K, C, T, n_chunks, n_kblocks, k_blk, x_scale, y_scale, x_zp, int(n_wscale));
+                       K, C, T, n_chunks, n_kblocks, k_blk, x_scale, y_scale, x_zp, int(n_wscale), 0, C);
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
 }
