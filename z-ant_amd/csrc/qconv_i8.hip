@@ -384,7 +384,6 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
         const uint8_t b = uint8_t(tid & 255);
         lut[tid & 255] = uint8_t((q.has_act ? qact_apply(b, q.act) : b) ^ (y_blocked ? 0x80 : 0));  // NT == 256
     }
-    for (int k = tid; k < kpad; k += NT) { mult_l[k] = mult[k]; corr_l[k] = corr[k]; }
     {
         const float inv_patch = 1.0f / float(patch_hw), inv_pw = 1.0f / float(t.PW);
         for (int e = tid; e < t.P1s; e += NT) {
@@ -400,6 +399,14 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
     if (int(blockIdx.x) >= t.n_tiles) return;
     const int my_tiles = (t.n_tiles - int(blockIdx.x) + int(gridDim.x) - 1) / int(gridDim.x);
     const int n_steps = my_tiles * t.n_chunks;
+    // The requantisation tables go to LDS as asynchronous copies at the head of the copy stream: copies land in order,
+    // so they are there when the first step's operands are, and nobody waits for a global load before the first
+    // operand copy is on its way.
+    for (int k0 = 0; k0 < kpad; k0 += NT)
+        if (k0 + tid < kpad) {
+            __builtin_amdgcn_global_load_lds((gptr_t)(mult + k0 + tid), (lptr_t)(mult_l + k0 + wave * 64), 4, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(corr + k0 + tid), (lptr_t)(corr_l + k0 + wave * 64), 4, 0, 0);
+        }
     // copies per thread and step (see qconv_issue)
     const int P = w_region_bytes(w_chunk, NT) / (16 * NT) + 2 * (t.P1s / NT);
     // prologue: the first n_stages - 1 steps' copies, in flight behind the index arithmetic below
@@ -507,6 +514,7 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
             const int KB = (g.K + 15) >> 4;
             const int cb0 = (kb * K_BLK + wn * 32) >> 4;
             const bool use_lut = q.has_act || !y_blocked;
+            const bool y_dwords = !POOL && plane == 1 && (g.K & 3) == 0 && (reinterpret_cast<uintptr_t>(y) & 3) == 0;
             if (POOL) {
                 // Requantisation and the activation are monotone (non-decreasing for a positive multiplier, non-increasing
                 // for a negative one), so the window's maximum output comes from its largest or smallest accumulator.
@@ -567,10 +575,19 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
                     lds_wait16(ob);
                     if (ok) {
                         uint8_t *yp = y + (int64_t(n0 + img) * g.K + kbase) * plane + int64_t(oh0 + r) * OWo + c;
+                        if (y_dwords) {
+                            // one output position per image: a lane's four consecutive channels are four consecutive bytes
 #pragma unroll
-                        for (int v = 0; v < 16; ++v) {
-                            const int dk = (v >> 2) * 8 + (v & 3);
-                            if (kbase + dk < g.K) yp[dk * plane] = uint8_t(ob[v]);
+                            for (int gq = 0; gq < 4; ++gq)
+                                if (kbase + gq * 8 < g.K)
+                                    *reinterpret_cast<uint32_t *>(yp + gq * 8) =
+                                        ob[gq * 4] | (ob[gq * 4 + 1] << 8) | (ob[gq * 4 + 2] << 16) | (ob[gq * 4 + 3] << 24);
+                        } else {
+#pragma unroll
+                            for (int v = 0; v < 16; ++v) {
+                                const int dk = (v >> 2) * 8 + (v & 3);
+                                if (kbase + dk < g.K) yp[dk * plane] = uint8_t(ob[v]);
+                            }
                         }
                     }
                 }
