@@ -245,7 +245,9 @@ __device__ __forceinline__ void qconv_issue(char *__restrict__ dma, const PatchD
             const int8_t *s0 = ok ? src : padvec;
             const int8_t *s1 = (ok && second) ? src + plane16 : padvec;
             __builtin_amdgcn_global_load_lds((gptr_t)s0, (lptr_t)(xl + (r * NT + wave * 64) * 16), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((gptr_t)s1, (lptr_t)(xl + (t.P1s + r * NT + wave * 64) * 16), 16, 0, 0);
+            // A layer of at most 16 input channels has no second half anywhere: its slots stay as they are -- whatever
+            // integers they hold meet zero weights.
+            if (CB > 1) __builtin_amdgcn_global_load_lds((gptr_t)s1, (lptr_t)(xl + (t.P1s + r * NT + wave * 64) * 16), 16, 0, 0);
         }
     }
 }
@@ -408,7 +410,7 @@ qconv_mfma_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, 
             __builtin_amdgcn_global_load_lds((gptr_t)(corr + k0 + tid), (lptr_t)(corr_l + k0 + wave * 64), 4, 0, 0);
         }
     // copies per thread and step (see qconv_issue)
-    const int P = w_region_bytes(w_chunk, NT) / (16 * NT) + 2 * (t.P1s / NT);
+    const int P = w_region_bytes(w_chunk, NT) / (16 * NT) + (CB > 1 ? 2 : 1) * (t.P1s / NT);
     // prologue: the first n_stages - 1 steps' copies, in flight behind the index arithmetic below
     PatchDesc desc;
     for (int s0 = 0; s0 < n_stages - 1 && s0 < n_steps; ++s0) {
@@ -714,7 +716,7 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
     if (plan.t.P1s / NT > QR_MAX) return 1;  // more copy rounds than the per-tile descriptors hold
     const size_t buf_bytes = size_t(w_region_bytes(T * QCC * K_BLK, NT)) + size_t(QCC) * plan.t.P1s;
     const size_t fixed_bytes = size_t(plan.t.P1s) * 8 + 512 + size_t(plan.t.n_kblocks) * K_BLK * 8;  // 256: table, 256: its alignment
-    const int copies = w_region_bytes(T * QCC * K_BLK, NT) / (16 * NT) + 2 * (plan.t.P1s / NT);
+    const int copies = w_region_bytes(T * QCC * K_BLK, NT) / (16 * NT) + (CB > 1 ? 2 : 1) * (plan.t.P1s / NT);
     const bool sparse = plan.t.n_tiles <= ctx->num_cus;
     const size_t lds_cap = sparse ? 160 * 1024 : 80 * 1024;
     int n_stages = sparse ? 8 : 4;
