@@ -207,6 +207,8 @@ def test_conv_with_fused_pool_on_the_matrix_cores(G, N, C, H, W, K, k, pad, relu
     (19, 1, 28, 28, 32, 3, 0, True),    # single-channel 3x3 on the matrix cores; the last workgroup holds 3 of 8 images
     (5, 1, 31, 27, 40, 3, 0, False),    # odd sizes (scalar image copy, dropped last row / column), two channel blocks, no ReLU
     (4, 1, 64, 64, 8, 3, 0, True),      # two images per workgroup, fewer channels than a block
+    (9, 1, 12, 14, 32, 3, 0, True),     # 30 pooled positions per image: several image wraps per 128-position step
+    (6, 1, 20, 34, 32, 3, 0, True),     # 16 pooled columns: a step of 128 positions is a whole number of rows
     (3, 1, 120, 90, 16, 3, 0, True),    # an image too large for the LDS copy: the direct kernel
     (6, 1, 28, 28, 32, 3, 1, True),     # padded: the direct kernel
     (7, 1, 28, 28, 20, 5, 0, True),     # 5x5

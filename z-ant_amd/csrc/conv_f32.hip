@@ -561,16 +561,19 @@ __device__ __forceinline__ float vmax3(float a, float b, float c) {
 //   D[k, p] = sum_t W[k, t] * X[window(p) + tap t]: output channels are the MFMA rows (32 per workgroup), pooled
 // positions the columns, and the nine taps the reduction axis, two per v_mfma_f32_32x32x2_f32: (0,0)|(0,1), (1,0)|(1,1),
 // (2,0)|(2,1), (0,2)|(1,2), (2,2)|none.  The pairing makes the address of a lane's tap a per-lane base plus an offset
-// that is the same for both halves of the wave; the tenth, absent tap reads a zero word against a zero weight.
+// that is the same for both halves of the wave; the tenth, absent tap reads a word holding 1.0 against the channel's bias
+// as its weight, so the matrix cores add the bias too.
 // A workgroup copies `imgs` whole images to LDS and walks their pooled positions 32 at a time per wave; the four members
-// of a pooling window are four accumulator tiles of the same lane, so the pool is a register-wise max (then bias and
-// ReLU, both monotone: equal to pool(relu(conv + bias)) exactly).  20 MFMAs produce 32 positions x 32 channels.
+// of a pooling window are four accumulator tiles of the same lane, so the pool is a register-wise max (then ReLU, which
+// commutes with it).  20 MFMAs produce 32 positions x 32 channels.  Vector instructions of a SIMD's other waves do not
+// hide behind its matrix instructions here (a tile's wall time measured as the sum of both), so everything around the
+// MFMAs is kept to a minimum: two instructions per output value and a store without address arithmetic.
 template <bool RELU, bool FULLK>
 __global__ void __launch_bounds__(256, 4) conv_f32_c1k3_pool_mfma_kernel(const float *__restrict__ x, const float *__restrict__ w,
                                                                      const float *__restrict__ bias, float *__restrict__ y,
                                                                      int N, int H, int W, int K, int POH, int POW, int imgs,
                                                                      FastDiv dpp, FastDiv dpw) {
-    extern __shared__ __attribute__((aligned(16))) float img_lds[];  // [imgs][H][W] then four zero words
+    extern __shared__ __attribute__((aligned(16))) float img_lds[];  // [imgs][H][W], four words (1, 0, 0, 0), weights, bias
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction; says so to the compiler (LDS
                                                                 // copy destinations then stay in scalar registers)
@@ -586,32 +589,57 @@ __global__ void __launch_bounds__(256, 4) conv_f32_c1k3_pool_mfma_kernel(const f
     } else {
         for (int i = tid; i < cnt; i += 256) img_lds[i] = src[i];
     }
-    const int zero_idx = imgs * HW;
-    if (tid < 4) img_lds[zero_idx + tid] = 0.0f;
-
-    // this lane's A operands: channel kb + l32, tap pair member lh
-    float wa[5];
-    {
-        const int ch = kb + l32;
-        const float *wr = w + int64_t(ch < K ? ch : 0) * 9;
-        const bool okc = ch < K;
-        wa[0] = okc ? wr[0 + lh] : 0.0f;
-        wa[1] = okc ? wr[3 + lh] : 0.0f;
-        wa[2] = okc ? wr[6 + lh] : 0.0f;
-        wa[3] = okc ? wr[lh ? 5 : 2] : 0.0f;
-        wa[4] = (okc && !lh) ? wr[8] : 0.0f;
-    }
-    float bv[16];
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        const int k = kb + (v >> 2) * 8 + lh * 4 + (v & 3);
-        bv[v] = (bias != nullptr && k < K) ? bias[k] : 0.0f;
+    // [0]: the word the absent tenth tap of the upper half-wave reads -- 1.0, against the channel's bias as its weight, so
+    // the last MFMA adds the bias; [1..3]: zero
+    const int one_idx = imgs * HW;
+    if (tid < 4) img_lds[one_idx + tid] = tid == 0 ? 1.0f : 0.0f;
+    // Weights and bias of the workgroup's 32 channels go through LDS: one coalesced read per workgroup, where per-lane
+    // reads would be 21 scattered loads per wave, queued in front of the other workgroups' image loads on the CU.
+    float *wl = img_lds + one_idx + 4;  // [32][9] weights, then [32] bias
+    for (int i = tid; i < 32 * 9 + 32; i += 256) {
+        float v = 0.0f;
+        if (i < 32 * 9) {
+            if (kb + i / 9 < K) v = w[int64_t(kb) * 9 + i];
+        } else if (bias != nullptr && kb + i - 32 * 9 < K) {
+            v = bias[kb + i - 32 * 9];
+        }
+        wl[i] = v;
     }
     __syncthreads();
 
+    // this lane's A operands: channel kb + l32, tap pair member lh; the tenth "tap" is the bias
+    float wa[5];
+    {
+        const float *wr = wl + l32 * 9;
+        wa[0] = wr[0 + lh];
+        wa[1] = wr[3 + lh];
+        wa[2] = wr[6 + lh];
+        wa[3] = wr[lh ? 5 : 2];
+        wa[4] = lh ? wl[32 * 9 + l32] : wr[8];
+    }
+
     const int total = imgs_here * PP;
-    float *ybase = y + (int64_t(n0) * K + kb) * PP;
+    // store bases of this lane group's 16 output channels: workgroup-uniform, pinned to scalar registers
+    unsigned long long ybase[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const unsigned long long a = reinterpret_cast<unsigned long long>(y + (int64_t(n0) * K + kb + (v >> 2) * 8 + (v & 3)) * PP);
+        // (the builtin returns int: without the casts the low word would be sign-extended over the high one)
+        const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(unsigned(a))));
+        const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(unsigned(a >> 32))));
+        ybase[v] = (static_cast<unsigned long long>(hi) << 32) | static_cast<unsigned long long>(lo);
+    }
     for (int p0 = wave * 32; p0 < total; p0 += 4 * 32) {
+        // Waves with more steps left go first.  Left alone the SIMD serves its oldest waves first: the youngest workgroup on
+        // a CU then runs most of its steps after the others are gone, one wave per SIMD, which keeps the matrix pipe half
+        // busy; with the laggards in front the four waves of a SIMD finish together.
+        {
+            const int left = (total - p0 + 127) >> 7;
+            if (left >= 5) __builtin_amdgcn_s_setprio(3);
+            else if (left >= 3) __builtin_amdgcn_s_setprio(2);
+            else if (left == 2) __builtin_amdgcn_s_setprio(1);
+            else __builtin_amdgcn_s_setprio(0);
+        }
         const int p = p0 + l32;
         const bool valid = p < total;
         const unsigned pc_ = valid ? unsigned(p) : 0u;
@@ -632,7 +660,7 @@ __global__ void __launch_bounds__(256, 4) conv_f32_c1k3_pool_mfma_kernel(const f
             b[1][j] = img_lds[a012 + to + W];
             b[2][j] = img_lds[a012 + to + 2 * W];
             b[3][j] = img_lds[a3 + to];
-            b[4][j] = img_lds[lh ? zero_idx : wb + to + 2 * W + 2];
+            b[4][j] = img_lds[lh ? one_idx : wb + to + 2 * W + 2];
         }
         // tap pairs outermost: consecutive MFMAs go to different accumulators
 #pragma unroll
@@ -640,16 +668,23 @@ __global__ void __launch_bounds__(256, 4) conv_f32_c1k3_pool_mfma_kernel(const f
 #pragma unroll
             for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(wa[t], b[t][j], acc[j], 0, 0, 0);
         if (valid) {
-            // a uniform base per output channel and one 32-bit byte offset per lane (the host checks that N * K * PP * 4
-            // fits): the stores then need no address arithmetic in the vector unit
+            // One 32-bit byte offset per lane and a uniform base per output channel, kept in scalar registers (the host
+            // checks that N * K * PP * 4 fits in 32 bits): the stores need no address arithmetic in the vector unit, which
+            // this kernel's matrix instructions leave little room for.  The bias came in through the tenth tap; adding the
+            // same bias to the four window members is monotone, so the maximum below is pool(conv + bias) exactly.
             const unsigned byte_off = ((unsigned(img) * unsigned(K) + unsigned(lh * 4)) * unsigned(PP) + pp) * 4u;
+            // The first three window members first, for all 16 values: the fourth accumulator tile is the one the last
+            // MFMA is still writing, and these 16 instructions are the distance its readers must keep from it.
+            float m3[16];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) m3[v] = vmax3(acc[0][v], acc[1][v], acc[2][v]);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int dk = (v >> 2) * 8 + (v & 3);
                 if (FULLK || kb + lh * 4 + dk < K) {
-                    float o = vmax(vmax3(acc[0][v], acc[1][v], acc[2][v]), acc[3][v]) + bv[v];
-                    if (RELU) o = vmax(o, 0.0f);
-                    *reinterpret_cast<float *>(reinterpret_cast<char *>(ybase + dk * PP) + byte_off) = o;
+                    const float o = RELU ? vmax3(m3[v], acc[3][v], 0.0f) : vmax(m3[v], acc[3][v]);
+                    asm volatile("global_store_dword %0, %1, %2" : : "v"(byte_off), "v"(o), "s"(ybase[v]) : "memory");
                 }
             }
         }
@@ -988,7 +1023,7 @@ int zant_conv2d_f32_fused_pool(zant_ctx *ctx, const float *x, const int64_t xdim
         const int imgs = int(std::min<int64_t>(4, (40 * 1024) / (int64_t(g.H) * g.W * 4)));
         const dim3 grid(unsigned(ceil_div64(g.N, imgs)), unsigned(ceil_div64(g.K, 32)));
         KernelTimer kt(ctx);
-        const size_t lds = size_t(imgs) * g.H * g.W * 4 + 16;
+        const size_t lds = size_t(imgs) * g.H * g.W * 4 + 16 + (32 * 9 + 32) * 4;
         const FastDiv dpp = make_fastdiv(unsigned(POH * POW)), dpw = make_fastdiv(unsigned(POW));
         const bool fullk = g.K % 32 == 0;
         ZANT_KERNEL_NAME(ctx, "conv_f32_c1k3_pool_mfma_kernel<%s,%s>", relu ? "true" : "false", fullk ? "true" : "false");
