@@ -518,11 +518,12 @@ void dispatch_gemm_dma(zant_ctx *ctx, const float *A, const float *B, const floa
 // ------------------------------------------------------------------------------------------------------------
 // Skinny Gemm (N <= 16, A row-major): the classifier head.  HBM-bound on A: every wave owns 4 rows, its lanes split
 // K, B sits in LDS, and the 4 x 16 partial sums per lane are reduced across the wave by recursive halving (63
-// exchanges instead of 64 x 6), which leaves result (row r, column n) in lane r*16 + n -- where bias, ReLU or the
-// row softmax (16-lane groups) are applied before one coalesced store.
+// exchanges instead of 64 x 6, 48 of them register swaps), which leaves result (row r, column n) in lane r*16 + n --
+// where bias, ReLU or the row softmax (16-lane groups) are applied before one coalesced store.
 // ------------------------------------------------------------------------------------------------------------
 constexpr int SK_KC = 512;  // k per LDS stage of B
 
+template <int NU>  // column units of 4 that hold data: ceil(N / 4); the others stay zero and cost no arithmetic
 __global__ void __launch_bounds__(256)
 gemm_f32_skinny_kernel(const float *__restrict__ A, const float *__restrict__ B, const float *__restrict__ C,
                        float *__restrict__ Y, GemmArgs g, int ldb_k, int ldb_n, int softmax) {
@@ -563,19 +564,31 @@ gemm_f32_skinny_kernel(const float *__restrict__ A, const float *__restrict__ B,
             const int kq = it * 64 + lane;
             if (it * 64 < kend) {
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
+                for (int u = 0; u < NU; ++u) {
                     const f32x4 b = bs[kq * 4 + (u ^ ((kq >> 2) & 3))];
 #pragma unroll
                     for (int r = 0; r < 4; ++r)
 #pragma unroll
-                        for (int c = 0; c < 4; ++c) v[r * 16 + u * 4 + c] += a[it][r] * b[c];
+                        for (int c = 0; c < 4; ++c) v[r * 16 + u * 4 + c] = __builtin_fmaf(a[it][r], b[c], v[r * 16 + u * 4 + c]);
                 }
             }
         }
     }
-    // recursive halving: after the step with distance s a lane keeps the half of its values selected by (lane & s)
+    // recursive halving: after the step with distance s a lane keeps the half of its values selected by (lane & s).
+    // Distances 32 and 16 are one half-wave / row swap of the two registers and an add: after the swap the lower lanes
+    // (even rows) hold both lanes' parts of value i, the upper lanes (odd rows) those of value i + s.
 #pragma unroll
-    for (int s = 32; s >= 1; s >>= 1) {
+    for (int i = 0; i < 32; ++i) {
+        const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[i]), __float_as_uint(v[i + 32]), false, false);
+        v[i] = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(v[i]), __float_as_uint(v[i + 16]), false, false);
+        v[i] = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+    }
+#pragma unroll
+    for (int s = 8; s >= 1; s >>= 1) {
         const bool up = (lane & s) != 0;
 #pragma unroll
         for (int i = 0; i < s; ++i) {
@@ -633,9 +646,13 @@ int run_gemm(zant_ctx *ctx, const float *A, const float *B, const float *C, floa
     if (softmax && (trans_a || N > 16)) return ZANT_InvalidInput;
     KernelTimer kt(ctx);
     if (!trans_a && N <= 16) {
-        ZANT_KERNEL_NAME(ctx, "gemm_f32_skinny_kernel");
-        hipLaunchKernelGGL(gemm_f32_skinny_kernel, dim3(unsigned((M + 15) / 16)), dim3(256), 0, ctx->stream, A, B, C, Y, g,
-                           trans_b ? 1 : g.ldb, trans_b ? g.ldb : 1, softmax);
+        const int nu = int((N + 3) / 4);
+        ZANT_KERNEL_NAME(ctx, "gemm_f32_skinny_kernel<%d>", nu);
+#define ZANT_SKINNY(NU)                                                                                                     \
+    hipLaunchKernelGGL(gemm_f32_skinny_kernel<NU>, dim3(unsigned((M + 15) / 16)), dim3(256), 0, ctx->stream, A, B, C, Y, g, \
+                       trans_b ? 1 : g.ldb, trans_b ? g.ldb : 1, softmax)
+        if (nu == 1) ZANT_SKINNY(1); else if (nu == 2) ZANT_SKINNY(2); else if (nu == 3) ZANT_SKINNY(3); else ZANT_SKINNY(4);
+#undef ZANT_SKINNY
         ZANT_LAUNCH_CHECK(ctx);
         return ZANT_OK;
     }
