@@ -35,6 +35,10 @@ HOST_TEST = os.path.join(HERE, "host", "test_host_mirror")
 # sources whose kernels hide LDS reads from the compiler (checked for spills at build time, see build())
 NO_SPILL_SOURCES = {"qconv_ps_i8.hip", "qblock_i8.hip", "qconv_i8.hip", "conv_f32.hip", "gemm_f32.hip"}
 
+# kernels whose hand-written stores take their bases from scalar registers: a scalar spill reloaded (v_readlane) right
+# in front of such a store would need wait states the compiler cannot count through inline asm
+NO_SGPR_SPILL_KERNELS = ("conv_f32_c1k3_pool_mfma_kernel",)
+
 OBJ = os.path.join(HERE, "_obj")  # per-source objects (not tracked); every build recompiles all of them
 
 
@@ -66,8 +70,11 @@ def build(verbose=True):
             m = re.search(r"remark:\s+(VGPRs Spill): (\d+)", line)
             if m and name and int(m.group(2)) > 0 and "_kernel" in name:
                 bad.append(f"{name}: {m.group(1)} = {m.group(2)}")
+            m = re.search(r"remark:\s+(SGPRs Spill): (\d+)", line)
+            if m and name and int(m.group(2)) > 0 and any(k in name for k in NO_SGPR_SPILL_KERNELS):
+                bad.append(f"{name}: {m.group(1)} = {m.group(2)}")
         if bad:
-            raise RuntimeError("kernels with hand-scheduled LDS reads must not spill:\n  " + "\n  ".join(bad))
+            raise RuntimeError("kernels with hand-scheduled LDS reads or stores must not spill:\n  " + "\n  ".join(bad))
         return job[0]
 
     with ThreadPoolExecutor(max_workers=min(8, len(jobs))) as pool:  # one translation unit per core
