@@ -55,7 +55,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=50)  # the shader clock settles after ~15 ms of work: fewer warm-up passes time the ramp
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-operators", action="store_true", help="skip the standalone operator figures (configs 2a, 2b, 3)")
     ap.add_argument("--no-networks", action="store_true", help="skip the int8 network figures (configs 4, 5)")

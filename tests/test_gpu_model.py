@@ -374,3 +374,46 @@ def test_quantised_concat_and_resize_nodes_keep_codes_and_parameters(G):
     ref = zo.qlinear_act(cat, 0.05, 120, "relu", 0.0, 0.04, 3)
     np.testing.assert_array_equal(m2.predict_host(x), ref)
     m2.close(); m.close()
+
+
+@pytest.mark.parametrize("N,H,W,K1,K2,pool2,relu", [
+    (6, 28, 28, 32, 64, True, True),    # the README CNN's head: first-layer kernel -> pooled matrix-core convolution
+    (5, 30, 26, 20, 40, True, False),   # 20 channels: five quads, channel blocks and chunk halves partly filled; no ReLU
+    (4, 28, 28, 32, 48, False, True),   # the second convolution without a pool
+    (3, 28, 28, 30, 32, True, True),    # 30 channels are not whole quads: the tensor stays NCHW
+])
+def test_f32_activation_between_two_convolutions(G, N, H, W, K1, K2, pool2, relu):
+    """Conv(1 -> K1, 3x3)+[ReLU]+MaxPool -> Conv(K1 -> K2, 3x3)+[ReLU][+MaxPool]: the tensor between the two nodes is kept
+    in the 16-byte channel-quad layout when K1 is a multiple of 4; results and the read-back of that tensor (handed out
+    as NCHW) must not depend on it."""
+    from zant_amd.model import Model
+    g = np.random.default_rng(N * 1000 + K1)
+    x = g.standard_normal((N, 1, H, W), dtype=np.float32)
+    w1 = (g.standard_normal((K1, 1, 3, 3)) * np.sqrt(2.0 / 9)).astype(np.float32)
+    b1 = (g.standard_normal(K1) * 0.1).astype(np.float32)
+    w2 = (g.standard_normal((K2, K1, 3, 3)) * np.sqrt(2.0 / (K1 * 9))).astype(np.float32)
+    b2 = (g.standard_normal(K2) * 0.1).astype(np.float32)
+    m = Model(G.tm.context())
+    t = m.conv(m.input((N, 1, H, W)), w1, b1, [1, 1], [0, 0, 0, 0], [1, 1], 1, "NOTSET")
+    if relu:
+        t = m.relu(t)
+    mid = m.maxpool(t, [2, 2], [2, 2])
+    t = m.conv(mid, w2, b2, [1, 1], [0, 0, 0, 0], [1, 1], 1, "NOTSET")
+    if relu:
+        t = m.relu(t)
+    if pool2:
+        t = m.maxpool(t, [2, 2], [2, 2])
+    m.finalize()
+    assert m.num_launches == 2
+    r1 = zo.Conv(x, w1, b1, [1, 1], [0, 0, 0, 0], [1, 1], 1, "NOTSET")
+    if relu:
+        r1 = zo.ReLU(r1)
+    r1 = zo.onnx_maxpool(r1, [2, 2], [2, 2], [1, 1], [0, 0, 0, 0])
+    r2 = zo.Conv(r1, w2, b2, [1, 1], [0, 0, 0, 0], [1, 1], 1, "NOTSET")
+    if relu:
+        r2 = zo.ReLU(r2)
+    if pool2:
+        r2 = zo.onnx_maxpool(r2, [2, 2], [2, 2], [1, 1], [0, 0, 0, 0])
+    np.testing.assert_allclose(m.predict_host(x), r2, rtol=G.RTOL, atol=G.ATOL)
+    np.testing.assert_allclose(m.read_tensor(mid, r1.shape, np.float32), r1, rtol=G.RTOL, atol=G.ATOL)
+    m.close()

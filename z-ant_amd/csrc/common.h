@@ -117,7 +117,17 @@ int zant_conv_resolve(const int64_t xdim[4], const int64_t wdim[4], const int64_
 int zant_conv2d_f32_fused_pool(zant_ctx *ctx, const float *x, const int64_t xdim[4], const float *w, const int64_t wdim[4],
                                const float *bias, float *y, const int64_t ydim[4], const int64_t *stride, int n_stride,
                                const int64_t *pads, int n_pads, const int64_t *dil, int n_dil, int64_t group,
-                               const char *auto_pad, int relu, bool query_only, zant_pack_slot *slot = nullptr);
+                               const char *auto_pad, int relu, bool query_only, zant_pack_slot *slot = nullptr,
+                               int x_c4 = 0, int y_c4 = 0);
+
+// Which of a convolution node's tensors may be kept in the quad-blocked f32 layout ([N][C/4][H][W][4], quant_layout.h):
+// *in_ok when the kernel that will run the node (with the fused pool or without) reads it, *out_ok when it writes it.
+void zant_conv2d_f32_c4_caps(const int64_t xdim[4], const int64_t wdim[4], const int64_t ydim[4], const int64_t *stride,
+                             int n_stride, const int64_t *pads, int n_pads, const int64_t *dil, int n_dil, int64_t group,
+                             const char *auto_pad, bool fuse_pool, int *in_ok, int *out_ok);
+
+// [N][C/4][HW][4] f32 -> NCHW f32 (for handing a quad-blocked tensor out of the executor).
+int zant_from_c4_f32(zant_ctx *ctx, const float *x, int64_t N, int64_t C, int64_t HW, float *y);
 
 // Resolves, once per device, the device address of the static scratch array behind zant_hip_conv2d_f32_static
 // (conv_f32.hip).  Called by zant_hip_ctx_create with the context's device current; a failure is remembered and
@@ -128,4 +138,4 @@ void zant_conv_static_scratch_init(int device);
 int zant_conv2d_f32_slot(zant_ctx *ctx, const float *x, const int64_t xdim[4], const float *w, const int64_t wdim[4],
                          const float *bias, float *y, const int64_t ydim[4], const int64_t *stride, int n_stride,
                          const int64_t *pads, int n_pads, const int64_t *dil, int n_dil, int64_t group, const char *auto_pad,
-                         int fuse_act, zant_pack_slot *slot);
+                         int fuse_act, zant_pack_slot *slot, int x_c4 = 0);

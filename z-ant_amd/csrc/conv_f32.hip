@@ -66,7 +66,7 @@ __device__ __forceinline__ void lds_wait_all(int &a, int &b, int &c, int &d) {
 }
 
 // A few zero words that padding lanes of the asynchronous global->LDS copies read from.
-__device__ float g_zero_words[4] = {0.f, 0.f, 0.f, 0.f};
+__device__ __align__(16) float g_zero_words[4] = {0.f, 0.f, 0.f, 0.f};
 
 // One (tile, chunk) step of the pipeline: start the asynchronous global->LDS copies of the NEXT step
 // into `dma` and run the matrix cores over THIS step's operands in `cmp`.
@@ -105,6 +105,31 @@ __device__ __forceinline__ void conv_step(float *__restrict__ dma, const float *
         // position's element offset inside the image group (or -1), so a copy costs an add, a compare and the selects:
         // whatever is decided here per step is paid in matrix-pipe time.
         const int64_t x_plane = int64_t(g.H) * g.W;
+        const unsigned ttab_addr = lds_addr_of(ttab);
+        if (t.x_c4) {
+            // Quad-blocked input ([N][C/4][H][W][4]): the four channels of a chunk half at one position are 16 contiguous
+            // bytes, which is also how the patch sits in LDS -- one copy per position and half, a quarter of the copy
+            // instructions of the NCHW form below (a wave pays ~130 cycles for each, whatever its size).
+            const float *q0 = x + int64_t(n0) * g.C * x_plane + int64_t(ichunk * (CC / 4)) * x_plane * 4;
+            const float *q1 = q0 + x_plane * 4;
+            const bool h_ok1 = ichunk * CC + 4 < g.C;
+            for (int p0 = 0; p0 < t.P1; p0 += 2 * NT) {
+                int e[2], pad0 = 0, pad1 = 0;
+#pragma unroll
+                for (int u = 0; u < 2; ++u) e[u] = lds_read32_async(ttab_addr + unsigned(min(p0 + u * NT + tid, t.P1 - 1)) * 4u);
+                lds_wait_all(e[0], e[1], pad0, pad1);
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    if (p0 + u * NT + tid < t.P1) {
+                        const bool ok = e[u] >= 0;
+                        const float *sp0 = ok ? q0 + unsigned(e[u]) : g_zero_words;
+                        const float *sp1 = (ok && h_ok1) ? q1 + unsigned(e[u]) : g_zero_words;
+                        __builtin_amdgcn_global_load_lds((gptr_t)sp0, (lptr_t)(xl + (p0 + u * NT + wave * 64) * 4), 16, 0, 0);
+                        __builtin_amdgcn_global_load_lds((gptr_t)sp1, (lptr_t)(xl + (t.P1s + p0 + u * NT + wave * 64) * 4), 16, 0, 0);
+                    }
+                }
+            }
+        } else {
         const int j = tid & 3;
         const float *b0 = x + (int64_t(n0) * g.C + ichunk * CC) * x_plane;  // wave-uniform: channel ichunk*CC of image n0
         const float *b1 = b0 + 4 * x_plane;
@@ -113,7 +138,6 @@ __device__ __forceinline__ void conv_step(float *__restrict__ dma, const float *
         // The table lives in LDS.  The compiler drains every outstanding asynchronous copy before an LDS read
         // it issues itself in this loop (one round trip to L2 per iteration, which made staging cost ~18 % of a
         // step), so the table is read with hand-written ds_read_b32, one iteration ahead of its use.
-        const unsigned ttab_addr = lds_addr_of(ttab);
         for (int p0 = 0; p0 < t.P1; p0 += 4 * PPI) {
             // four table entries per round; nothing read this way stays in flight across a loop edge (a register
             // copy there would run before the data has landed)
@@ -134,6 +158,7 @@ __device__ __forceinline__ void conv_step(float *__restrict__ dma, const float *
                     __builtin_amdgcn_global_load_lds((gptr_t)sp1, (lptr_t)(xl + (t.P1s + p0 + u * PPI + wave * 16) * 4), 4, 0, 0);
                 }
             }
+        }
         }
     }
 
@@ -274,7 +299,8 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
             const int v = ptab[e];
             const int img = int(unsigned(v) >> 24), ih = ih0 + ((v >> 12) & 0xfff), iw = (v & 0xfff) - g.pl;
             const bool ok = iw >= 0 && iw < g.W && ih >= 0 && ih < g.H && img < imgs_here;
-            tt[e] = ok ? img * int(x_img) + ih * g.W + iw : -1;  // NB*C*H*W*4 < 2^31 is checked on the host
+            // (quad-blocked input: four floats per position inside a quad's plane)
+            tt[e] = ok ? img * int(x_img) + (ih * g.W + iw) * (t.x_c4 ? 4 : 1) : -1;  // NB*C*H*W*4 < 2^31 is checked on the host
         }
     };
 
@@ -300,6 +326,19 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
         const float *xb = x + int64_t(cn0) * x_img;
         const int j = tid & 3;
         float *xl = buf0 + w_chunk;
+        if (t.x_c4) {
+            for (int p0 = 0; p0 < t.P1; p0 += NT) {
+                const int pos = p0 + tid;
+                if (pos < t.P1) {
+                    const int e = ttab0[pos];
+#pragma unroll
+                    for (int half = 0; half < 2; ++half) {
+                        const float *sp = (e >= 0 && half * 4 < g.C) ? xb + e + int64_t(half) * x_plane * 4 : g_zero_words;
+                        __builtin_amdgcn_global_load_lds((gptr_t)sp, (lptr_t)(xl + (half * t.P1s + p0 + wave * 64) * 4), 16, 0, 0);
+                    }
+                }
+            }
+        } else
         for (int p0 = 0; p0 < t.P1; p0 += NT / 4) {
             const int pos = p0 + (tid >> 2);
             if (pos < t.P1) {
@@ -572,7 +611,7 @@ template <bool RELU, bool FULLK>
 __global__ void __launch_bounds__(256, 4) conv_f32_c1k3_pool_mfma_kernel(const float *__restrict__ x, const float *__restrict__ w,
                                                                      const float *__restrict__ bias, float *__restrict__ y,
                                                                      int N, int H, int W, int K, int POH, int POW, int imgs,
-                                                                     FastDiv dpp, FastDiv dpw) {
+                                                                     FastDiv dpp, FastDiv dpw, int y_c4) {
     extern __shared__ __attribute__((aligned(16))) float img_lds[];  // [imgs][H][W], four words (1, 0, 0, 0), weights, bias
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction; says so to the compiler (LDS
@@ -629,6 +668,16 @@ __global__ void __launch_bounds__(256, 4) conv_f32_c1k3_pool_mfma_kernel(const f
         const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(unsigned(a >> 32))));
         ybase[v] = (static_cast<unsigned long long>(hi) << 32) | static_cast<unsigned long long>(lo);
     }
+    // quad-blocked output ([N][K/4][PP][4]): this lane's four groups of four consecutive channels are four 16-byte units,
+    // 2 * PP units apart; their bases (group offset included) likewise sit in scalar registers
+    unsigned long long ybase4[4];
+#pragma unroll
+    for (int gq = 0; gq < 4; ++gq) {
+        const unsigned long long a = reinterpret_cast<unsigned long long>(y + (int64_t(n0) * K + kb + gq * 8) * PP);
+        const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(unsigned(a))));
+        const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(unsigned(a >> 32))));
+        ybase4[gq] = (static_cast<unsigned long long>(hi) << 32) | static_cast<unsigned long long>(lo);
+    }
     for (int p0 = wave * 32; p0 < total; p0 += 4 * 32) {
         // Waves with more steps left go first.  Left alone the SIMD serves its oldest waves first: the youngest workgroup on
         // a CU then runs most of its steps after the others are gone, one wave per SIMD, which keeps the matrix pipe half
@@ -679,6 +728,23 @@ __global__ void __launch_bounds__(256, 4) conv_f32_c1k3_pool_mfma_kernel(const f
 #pragma unroll
             for (int v = 0; v < 16; ++v) m3[v] = vmax3(acc[0][v], acc[1][v], acc[2][v]);
             __builtin_amdgcn_sched_barrier(0);
+            if (y_c4) {
+                // quad (kb + gq*8 + lh*4) / 4 of image n0 + img: unit ((img * K/4 + lh) * PP + pp) past the group's base
+                const unsigned off16 = ((unsigned(img) * unsigned(K >> 2) + unsigned(lh)) * unsigned(PP) + pp) * 16u;
+#pragma unroll
+                for (int gq = 0; gq < 4; ++gq) {
+                    if (FULLK || kb + gq * 8 + lh * 4 < K) {  // K is a multiple of 4 here: a quad is whole or absent
+                        f32x4 o4;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            o4[e] = RELU ? vmax3(m3[gq * 4 + e], acc[3][gq * 4 + e], 0.0f) : vmax(m3[gq * 4 + e], acc[3][gq * 4 + e]);
+                        // (a store of more than 8 bytes reads its data over the next cycles: the two wait states keep the
+                        // next vector write to these registers -- which the compiler cannot tell apart through the
+                        // statement -- behind it)
+                        asm volatile("global_store_dwordx4 %0, %1, %2\n\ts_nop 1" : : "v"(off16), "v"(o4), "s"(ybase4[gq]) : "memory");
+                    }
+                }
+            } else {
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int dk = (v >> 2) * 8 + (v & 3);
@@ -686,6 +752,7 @@ __global__ void __launch_bounds__(256, 4) conv_f32_c1k3_pool_mfma_kernel(const f
                     const float o = RELU ? vmax3(m3[v], acc[3][v], 0.0f) : vmax(m3[v], acc[3][v]);
                     asm volatile("global_store_dword %0, %1, %2" : : "v"(byte_off), "v"(o), "s"(ybase[v]) : "memory");
                 }
+            }
             }
         }
     }
@@ -766,7 +833,10 @@ bool mfma_eligible(const ConvGeom &g, bool pool, MfmaPlan *plan) {
 
 // Packs the weights, resets the tile counter and launches the persistent implicit-GEMM kernel.
 int run_conv_mfma(zant_ctx *ctx, const float *x, const float *w, const float *bias, float *y, const ConvGeom &g,
-                  const MfmaPlan &plan, int relu, bool pool, zant_pack_slot *slot) {
+                  const MfmaPlan &plan_in, int relu, bool pool, zant_pack_slot *slot, int x_c4 = 0) {
+    if (x_c4 && (g.C & 3)) return ZANT_InvalidInput;
+    MfmaPlan plan = plan_in;
+    plan.t.x_c4 = x_c4 ? 1 : 0;
     const int T = g.KH * g.KW, K_BLK = plan.WN * 32;
     const size_t wp_floats = size_t(plan.t.n_chunks) * plan.t.n_kblocks * T * CC * K_BLK;
     void *ws = nullptr, *dyn = nullptr;
@@ -927,7 +997,7 @@ extern "C" int zant_hip_conv2d_f32_static(zant_ctx *ctx, const float *x, const i
 int zant_conv2d_f32_slot(zant_ctx *ctx, const float *x, const int64_t xdim[4], const float *w, const int64_t wdim[4],
                          const float *bias, float *y, const int64_t ydim[4], const int64_t *stride, int n_stride,
                          const int64_t *pads, int n_pads, const int64_t *dil, int n_dil, int64_t group, const char *auto_pad,
-                         int fuse_act, zant_pack_slot *slot) {
+                         int fuse_act, zant_pack_slot *slot, int x_c4) {
     if (!ctx || !xdim || !wdim || !ydim) return ZANT_NullPointer;
     zant_log("OnnxConvLean1");
     int64_t s[2], d[2], p[4];
@@ -956,12 +1026,13 @@ int zant_conv2d_f32_slot(zant_ctx *ctx, const float *x, const int64_t xdim[4], c
 
     MfmaPlan plan;
     if (mfma_eligible(g, false, &plan)) {
-        rc = run_conv_mfma(ctx, x, w, bias, y, g, plan, relu, false, slot);
+        rc = run_conv_mfma(ctx, x, w, bias, y, g, plan, relu, false, slot, x_c4);
         if (rc <= 0) {
             if (rc == ZANT_OK) zant_log("OnnxConvLean4");
             return rc;
         }
     }
+    if (x_c4) return ZANT_InvalidInput;  // only the matrix-core kernel reads the quad-blocked layout (see zant_conv2d_f32_c4_caps)
     const int ckk = g.C * g.KH * g.KW;
     if (ckk == 9 || ckk == 25 || ckk == 27) {
         const int64_t positions = int64_t(g.N) * g.OH * g.OW;
@@ -992,7 +1063,7 @@ int zant_conv2d_f32_slot(zant_ctx *ctx, const float *x, const int64_t xdim[4], c
 int zant_conv2d_f32_fused_pool(zant_ctx *ctx, const float *x, const int64_t xdim[4], const float *w, const int64_t wdim[4],
                                const float *bias, float *y, const int64_t ydim[4], const int64_t *stride, int n_stride,
                                const int64_t *pads, int n_pads, const int64_t *dil, int n_dil, int64_t group,
-                               const char *auto_pad, int relu, bool query_only, zant_pack_slot *slot) {
+                               const char *auto_pad, int relu, bool query_only, zant_pack_slot *slot, int x_c4, int y_c4) {
     int64_t s[2], d[2], p[4];
     if (zant_conv_resolve(xdim, wdim, stride, n_stride, pads, n_pads, dil, n_dil, group, auto_pad, s, d, p)) return 1;
     if (s[0] != 1 || s[1] != 1 || d[0] != 1 || d[1] != 1 || xdim[1] != wdim[1]) return 1;
@@ -1012,9 +1083,11 @@ int zant_conv2d_f32_fused_pool(zant_ctx *ctx, const float *x, const int64_t xdim
         MfmaPlan plan;
         if (!mfma_eligible(g, true, &plan) || (plan.MT != 4 && plan.MT != 8)) return 1;
         if (query_only) return ZANT_OK;
-        return run_conv_mfma(ctx, x, w, bias, y, g, plan, relu, true, slot);
+        if (y_c4) return ZANT_InvalidInput;  // (zant_conv2d_f32_c4_caps says which kernel writes that layout)
+        return run_conv_mfma(ctx, x, w, bias, y, g, plan, relu, true, slot, x_c4);
     }
     if (query_only) return ZANT_OK;
+    if (x_c4) return ZANT_InvalidInput;
     const int POH = int(OH / 2), POW = int(OW / 2);
     if (k133 && g.pt == 0 && g.pl == 0 && OH == xdim[2] - 2 && OW == xdim[3] - 2 && int64_t(g.H) * g.W * 4 <= 40 * 1024 &&
         int64_t(POH) * POW < (1 << 20) && int64_t(g.N) * g.K * POH * POW < (int64_t(1) << 30)) {
@@ -1029,13 +1102,15 @@ int zant_conv2d_f32_fused_pool(zant_ctx *ctx, const float *x, const int64_t xdim
         ZANT_KERNEL_NAME(ctx, "conv_f32_c1k3_pool_mfma_kernel<%s,%s>", relu ? "true" : "false", fullk ? "true" : "false");
 #define ZANT_C1K3(R, F)                                                                                                      \
     hipLaunchKernelGGL((conv_f32_c1k3_pool_mfma_kernel<R, F>), grid, dim3(256), lds, ctx->stream, x, w, bias, y, g.N, g.H, g.W, g.K, \
-                       POH, POW, imgs, dpp, dpw)
+                       POH, POW, imgs, dpp, dpw, (y_c4 && g.K % 4 == 0) ? 1 : 0)
+        if (y_c4 && g.K % 4 != 0) return ZANT_InvalidInput;
         if (relu) { if (fullk) ZANT_C1K3(true, true); else ZANT_C1K3(true, false); }
         else { if (fullk) ZANT_C1K3(false, true); else ZANT_C1K3(false, false); }
 #undef ZANT_C1K3
         ZANT_LAUNCH_CHECK(ctx);
         return ZANT_OK;
     }
+    if (y_c4) return ZANT_InvalidInput;
     const int64_t positions = int64_t(g.N) * POH * POW;
     const unsigned pb = unsigned(std::min<int64_t>(ceil_div64(positions, 256), int64_t(ctx->num_cus) * 16));
     KernelTimer kt(ctx);
@@ -1043,6 +1118,71 @@ int zant_conv2d_f32_fused_pool(zant_ctx *ctx, const float *x, const int64_t xdim
     if (k133) hipLaunchKernelGGL((conv_f32_smallc_pool_kernel<1, 3, 3>), dim3(pb), dim3(256), 0, ctx->stream, x, w, bias, y, g, POH, POW, relu);
     else if (k155) hipLaunchKernelGGL((conv_f32_smallc_pool_kernel<1, 5, 5>), dim3(pb), dim3(256), 0, ctx->stream, x, w, bias, y, g, POH, POW, relu);
     else hipLaunchKernelGGL((conv_f32_smallc_pool_kernel<3, 3, 3>), dim3(pb), dim3(256), 0, ctx->stream, x, w, bias, y, g, POH, POW, relu);
+    ZANT_LAUNCH_CHECK(ctx);
+    return ZANT_OK;
+}
+
+// Which kernel will run a convolution node decides which of its tensors may be quad-blocked: the implicit-GEMM kernel
+// reads that layout (with the fused pool or without), the single-channel 3x3 first-layer kernel with the fused pool
+// writes it.  The conditions repeat those of zant_conv2d_f32_slot / zant_conv2d_f32_fused_pool above.
+void zant_conv2d_f32_c4_caps(const int64_t xdim[4], const int64_t wdim[4], const int64_t ydim[4], const int64_t *stride,
+                             int n_stride, const int64_t *pads, int n_pads, const int64_t *dil, int n_dil, int64_t group,
+                             const char *auto_pad, bool fuse_pool, int *in_ok, int *out_ok) {
+    *in_ok = *out_ok = 0;
+    int64_t s[2], d[2], p[4];
+    if (zant_conv_resolve(xdim, wdim, stride, n_stride, pads, n_pads, dil, n_dil, group, auto_pad, s, d, p)) return;
+    for (int i = 0; i < 4; ++i)
+        if (xdim[i] <= 0 || wdim[i] <= 0 || xdim[i] > INT32_MAX || wdim[i] > INT32_MAX) return;
+    if (xdim[1] != wdim[1]) return;
+    const int64_t PH = xdim[2] + p[0] + p[2], PW = xdim[3] + p[1] + p[3];
+    const int64_t dkh = (wdim[2] - 1) * d[0] + 1, dkw = (wdim[3] - 1) * d[1] + 1;
+    if (PH < dkh || PW < dkw) return;
+    const int64_t OH = (PH - dkh) / s[0] + 1, OW = (PW - dkw) / s[1] + 1;
+    if (OH > INT32_MAX || OW > INT32_MAX) return;
+    ConvGeom g;
+    g.N = int(xdim[0]); g.C = int(xdim[1]); g.H = int(xdim[2]); g.W = int(xdim[3]);
+    g.K = int(wdim[0]); g.CG = int(wdim[1]); g.KH = int(wdim[2]); g.KW = int(wdim[3]);
+    g.OH = int(OH); g.OW = int(OW);
+    g.sh = int(s[0]); g.sw = int(s[1]); g.dh = int(d[0]); g.dw = int(d[1]);
+    g.pt = int(p[0]); g.pl = int(p[1]); g.groups = 1;
+    MfmaPlan plan;
+    if (!fuse_pool) {
+        *in_ok = (g.C % 4 == 0) && mfma_eligible(g, false, &plan);
+        return;
+    }
+    if (s[0] != 1 || s[1] != 1 || d[0] != 1 || d[1] != 1) return;
+    const bool k133 = g.C == 1 && g.KH == 3 && g.KW == 3, k155 = g.C == 1 && g.KH == 5 && g.KW == 5,
+               k333 = g.C == 3 && g.KH == 3 && g.KW == 3;
+    if (!k133 && !k155 && !k333) {
+        *in_ok = (g.C % 4 == 0) && mfma_eligible(g, true, &plan) && (plan.MT == 4 || plan.MT == 8);
+        return;
+    }
+    const int POH = int(OH / 2), POW = int(OW / 2);
+    *out_ok = k133 && g.K % 4 == 0 && g.pt == 0 && g.pl == 0 && OH == xdim[2] - 2 && OW == xdim[3] - 2 &&
+              int64_t(g.H) * g.W * 4 <= 40 * 1024 && int64_t(POH) * POW < (1 << 20) &&
+              int64_t(g.N) * g.K * POH * POW < (int64_t(1) << 30) && ydim[2] == POH && ydim[3] == POW;
+}
+
+namespace {
+__global__ void __launch_bounds__(256) from_c4_f32_kernel(const f32x4 *__restrict__ x, float *__restrict__ y, int64_t units,
+                                                          int64_t HW) {
+    const int64_t step = int64_t(gridDim.x) * blockDim.x;
+    for (int64_t u = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; u < units; u += step) {
+        const int64_t q = u / HW, pos = u - q * HW;  // q = n * C/4 + quad: NCHW plane 4q + e
+        const f32x4 v = x[u];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) y[(q * 4 + e) * HW + pos] = v[e];
+    }
+}
+}  // namespace
+
+int zant_from_c4_f32(zant_ctx *ctx, const float *x, int64_t N, int64_t C, int64_t HW, float *y) {
+    if (!ctx || !x || !y) return ZANT_NullPointer;
+    if (C % 4 != 0) return ZANT_InvalidInput;
+    const int64_t units = N * (C / 4) * HW;
+    if (units == 0) return ZANT_OK;
+    const unsigned blocks = unsigned(std::min<int64_t>(ceil_div64(units, 256), int64_t(ctx->num_cus) * 16));
+    hipLaunchKernelGGL(from_c4_f32_kernel, dim3(blocks), dim3(256), 0, ctx->stream, reinterpret_cast<const f32x4 *>(x), y, units, HW);
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
 }

@@ -17,6 +17,7 @@ struct TileGeom {
     int n_sblocks;       // spatial tiles
     int n_tiles;         // n_sblocks * n_kblocks
     int POW;             // fused 2x2/2 max pool: pooled columns (OW / 2); 0 = no pooling
+    int x_c4;            // f32 kernel: the input is stored [N][C/4][H][W][4] (set by the launcher, not the planner)
 };
 
 struct TilePlan {
@@ -70,6 +71,7 @@ inline bool zant_plan_conv_tiles(const ConvGeom &g, int WM, int WN, int mt_max, 
         if (rows < 1 || cols < 1) continue;
         const int per_img = rows * cols;
         TileGeom t;
+        t.x_c4 = 0;
         t.POW = pool ? cols : 0;
         int th;  // rows (pooled rows) per tile
         if (per_img <= S) {

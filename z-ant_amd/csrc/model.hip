@@ -203,12 +203,14 @@ int run_node(zant_model *m, const MNode &nd) {
                                               static_cast<const float *>(param_ptr(m, nd.b)), static_cast<float *>(y), to.dim,
                                               nd.stride, nd.n_stride, nd.has_pads ? nd.pads : nullptr, nd.n_pads,
                                               nd.has_dil ? nd.dil : nullptr, nd.n_dil, nd.group,
-                                              nd.has_auto_pad ? nd.auto_pad.c_str() : nullptr, nd.fuse_act == ZANT_ACT_RELU, false, &nd.slot);
+                                              nd.has_auto_pad ? nd.auto_pad.c_str() : nullptr, nd.fuse_act == ZANT_ACT_RELU, false, &nd.slot,
+                                              lin == ZANT_LAYOUT_C4, lout == ZANT_LAYOUT_C4);
+        if (lout == ZANT_LAYOUT_C4) return ZANT_InvalidInput;  // no unpooled kernel writes that layout (finalize never asks)
         return zant_conv2d_f32_slot(ctx, static_cast<const float *>(x), ti.dim, static_cast<const float *>(param_ptr(m, nd.w)),
                                     nd.wdim, static_cast<const float *>(param_ptr(m, nd.b)), static_cast<float *>(y), to.dim,
                                     nd.stride, nd.n_stride, nd.has_pads ? nd.pads : nullptr, nd.n_pads,
                                     nd.has_dil ? nd.dil : nullptr, nd.n_dil, nd.group,
-                                    nd.has_auto_pad ? nd.auto_pad.c_str() : nullptr, nd.fuse_act, &nd.slot);
+                                    nd.has_auto_pad ? nd.auto_pad.c_str() : nullptr, nd.fuse_act, &nd.slot, lin == ZANT_LAYOUT_C4);
     case OP_RELU:
         return zant_hip_relu_f32(ctx, static_cast<const float *>(x), static_cast<float *>(y), int64_t(ti.bytes() / 4));
     case OP_LEAKY:
@@ -903,6 +905,41 @@ extern "C" int zant_model_finalize(zant_model *m) {
         (void)ntl;
     }
 
+    // ---- layouts: an f32 activation between convolution nodes stays quad-blocked ([N][C/4][H][W][4]) where the kernel
+    // that writes it and every kernel that reads it take that layout: 16-byte stores on one side, a quarter of the
+    // patch copies on the other.  Same bytes as NCHW, so the arena plan does not change. ----
+    {
+        auto caps = [&](const MNode &nd, int *in_ok, int *out_ok) {
+            zant_conv2d_f32_c4_caps(m->t[nd.in0].dim, nd.wdim, m->t[nd.out].dim, nd.stride, nd.n_stride,
+                                    nd.has_pads ? nd.pads : nullptr, nd.n_pads, nd.has_dil ? nd.dil : nullptr, nd.n_dil, nd.group,
+                                    nd.has_auto_pad ? nd.auto_pad.c_str() : nullptr, nd.fuse_pool, in_ok, out_ok);
+        };
+        const int in_root = root_of(m, m->input), out_root = root_of(m, m->output);
+        for (const MNode &nd : m->n) {
+            if (nd.skip || nd.op != OP_CONV) continue;
+            const int root = root_of(m, nd.out);
+            MTensor &ro = m->t[root];
+            if (ro.dtype != ZANT_F32 || ro.rank != 4 || root == in_root || root == out_root || ro.layout != ZANT_LAYOUT_NCHW) continue;
+            int in_ok = 0, out_ok = 0;
+            caps(nd, &in_ok, &out_ok);
+            if (!out_ok) continue;
+            bool all = true;
+            int readers = 0;
+            for (const MNode &c : m->n) {
+                if (c.skip && c.op != OP_RESHAPE) continue;  // fused away; a view, though, would need NCHW
+                bool reads = root_of(m, c.in0) == root || (c.in1 >= 0 && root_of(m, c.in1) == root);
+                for (int in : c.more) reads = reads || root_of(m, in) == root;
+                if (!reads) continue;
+                ++readers;
+                if (c.skip || c.op != OP_CONV || root_of(m, c.in0) != root) { all = false; break; }
+                int cin = 0, cout = 0;
+                caps(c, &cin, &cout);
+                if (!cin) { all = false; break; }
+            }
+            if (all && readers > 0) ro.layout = ZANT_LAYOUT_C4;
+        }
+    }
+
     // ---- QLinearConv (+activation) -> MaxPool 2x2/2 between blocked tensors: the pool rides in the matrix-core kernel ----
     for (int i = 0; i < nn; ++i) {
         MNode &nd = m->n[i];
@@ -1302,6 +1339,15 @@ extern "C" int zant_model_read_tensor(zant_model *m, int id, void *dst_host, siz
         if (rc) return rc;
         rc = zant_from_blocked(m->ctx, static_cast<const uint8_t *>(tensor_ptr(m, id)), t.dim[0], t.dim[1], t.dim[2] * t.dim[3],
                                static_cast<uint8_t *>(ws));
+        if (rc) return rc;
+        return zant_hip_download(m->ctx, dst_host, ws, bytes);
+    }
+    if (m->t[root_of(m, id)].layout == ZANT_LAYOUT_C4) {  // likewise NCHW f32
+        void *ws = nullptr;
+        int rc = zant_workspace(m->ctx, t.bytes(), &ws);
+        if (rc) return rc;
+        rc = zant_from_c4_f32(m->ctx, static_cast<const float *>(tensor_ptr(m, id)), t.dim[0], t.dim[1], t.dim[2] * t.dim[3],
+                              static_cast<float *>(ws));
         if (rc) return rc;
         return zant_hip_download(m->ctx, dst_host, ws, bytes);
     }
