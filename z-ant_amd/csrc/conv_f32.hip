@@ -247,6 +247,7 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
     int *ttab0 = ptab + t.P1s;                                     // [2][P1s]: per tile, a position's element offset in
     int *ttab1 = ttab0 + t.P1s;                                    //   the image group, -1 where the patch is padding
     int *sched = ttab1 + t.P1s;                                    // [2]: tile ids handed out by thread 0
+    float *bias_l = reinterpret_cast<float *>(sched + 2);          // [n_kblocks * K_BLK]: the bias, zero past K
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction; says so to the compiler (LDS
@@ -284,6 +285,9 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
         }
         lds_off[i] = (img < t.NB && r < t.TH) ? (img * t.PH + r * g.sh) * t.PW + c * g.sw : 0;
     }
+    // The bias goes to LDS once: read per tile from global memory, its 16 scattered loads sat in every epilogue with
+    // their full latency exposed (the accumulators are done, nothing else is left to do).
+    for (int k = tid; k < t.n_kblocks * K_BLK; k += NT) bias_l[k] = (bias != nullptr && k < g.K) ? bias[k] : 0.0f;
     if (tid == 0) sched[0] = blockIdx.x + gridDim.x;  // the second tile is static, later ones come from the counter
     // Two counters take turns: this launch draws from tile_counters[parity] and re-arms the other one for the next
     // launch of the same operator, so that packed weights and counters can be kept across calls without a reset pass.
@@ -392,11 +396,18 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
             const int64_t plane = int64_t(g.OH) * g.OW;
             const int kbase = kb * K_BLK + wn * 32 + lh * 4;
             const bool full_k = (kb + 1) * K_BLK <= g.K;
+            // (hand-issued LDS reads: the next tile's first copies are in flight, and a read the compiler sees would
+            // wait for them)
             float bv[16];
+            {
+                const unsigned ba = lds_addr_of(bias_l) + unsigned(kbase) * 4u;
+                int raw[16];
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int k = kbase + (v >> 2) * 8 + (v & 3);
-                bv[v] = (bias != nullptr && k < g.K) ? bias[k] : 0.0f;
+                for (int v = 0; v < 16; ++v) raw[v] = lds_read32_async(ba + unsigned((v >> 2) * 8 + (v & 3)) * 4u);
+#pragma unroll
+                for (int q4 = 0; q4 < 4; ++q4) lds_wait_all(raw[q4 * 4], raw[q4 * 4 + 1], raw[q4 * 4 + 2], raw[q4 * 4 + 3]);
+#pragma unroll
+                for (int v = 0; v < 16; ++v) bv[v] = __int_as_float(raw[v]);
             }
             if constexpr (POOL) {
                 // max over the window, then bias and ReLU: both are monotone, so this equals pool(relu(conv + bias))
@@ -761,15 +772,19 @@ __global__ void __launch_bounds__(256, 4) conv_f32_c1k3_pool_mfma_kernel(const f
 typedef TilePlan MfmaPlan;
 
 // Tile shape with the best useful-lane fraction whose LDS footprint allows two workgroups per CU.
+// LDS the kernel keeps beyond the planner's count: the bias of every output channel (padded to whole channel blocks)
+inline size_t bias_lds_bytes(const ConvGeom &g) { return size_t((g.K + 63) / 64) * 64 * sizeof(float); }
+
 bool plan_mfma(const ConvGeom &g, MfmaPlan *best, bool pool = false) {
-    if (g.K <= 32) return zant_plan_conv_tiles(g, 4, 1, 8, CC, sizeof(float), 80 * 1024, best, pool, 0, 32, 0, 2, 4, 256, 4096);
+    const size_t cap = 80 * 1024 - bias_lds_bytes(g);
+    if (g.K <= 32) return zant_plan_conv_tiles(g, 4, 1, 8, CC, sizeof(float), cap, best, pool, 0, 32, 0, 2, 4, 256, 4096);
     // 64 output channels per workgroup (2 x 2 waves) stage the input patch once per 64 channels; 32 per workgroup
     // (4 x 1 waves) stage it twice but have twice the position slots, which can fit small feature maps much better
     // (e.g. 5 whole 5x5 pooled images in 128 slots instead of 2 in 64).  Take the narrow shape only for a clear win: at
     // 0.98 against 0.78 useful columns the two measured the same time, and the wide one reads the input once.
     MfmaPlan wide, narrow;
-    const bool ok_w = zant_plan_conv_tiles(g, 2, 2, 8, CC, sizeof(float), 80 * 1024, &wide, pool, 0, 32, 0, 2, 4, 256, 4096);
-    const bool ok_n = zant_plan_conv_tiles(g, 4, 1, 8, CC, sizeof(float), 80 * 1024, &narrow, pool, 0, 32, 0, 2, 4, 256, 4096);
+    const bool ok_w = zant_plan_conv_tiles(g, 2, 2, 8, CC, sizeof(float), cap, &wide, pool, 0, 32, 0, 2, 4, 256, 4096);
+    const bool ok_n = zant_plan_conv_tiles(g, 4, 1, 8, CC, sizeof(float), cap, &narrow, pool, 0, 32, 0, 2, 4, 256, 4096);
     if (ok_n && (!ok_w || narrow.eff > wide.eff + 0.25)) { *best = narrow; return true; }
     if (ok_w) { *best = wide; return true; }
     return false;
@@ -787,7 +802,7 @@ void launch_mfma_tt(zant_ctx *ctx, const float *x, const float *wp, const float 
         attr_set = true;
     }
     ZANT_KERNEL_NAME(ctx, "conv_f32_mfma_kernel<%d,%d,%d,%d,%d,%s>", MT, WM, WN, KV, TT, POOL ? "true" : "false");
-    hipLaunchKernelGGL((conv_f32_mfma_kernel<MT, WM, WN, KV, TT, POOL>), dim3(grid), dim3(WM * WN * 64), p.lds_bytes,
+    hipLaunchKernelGGL((conv_f32_mfma_kernel<MT, WM, WN, KV, TT, POOL>), dim3(grid), dim3(WM * WN * 64), p.lds_bytes + bias_lds_bytes(g),
                        ctx->stream, x, wp, bias, y, g, p.t, relu, counter, parity);
 }
 
