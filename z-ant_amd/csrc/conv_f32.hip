@@ -65,6 +65,19 @@ __device__ __forceinline__ void lds_wait_all(int &a, int &b, int &c, int &d) {
     asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
 }
 
+// max without the NaN-quieting pass the compiler puts in front of fmaxf (an MFMA result is never a signalling NaN); a NaN
+// operand yields the other one, like fmaxf
+__device__ __forceinline__ float vmax(float a, float b) {
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ float vmax3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
 // A few zero words that padding lanes of the asynchronous global->LDS copies read from.
 __device__ __align__(16) float g_zero_words[4] = {0.f, 0.f, 0.f, 0.f};
 
@@ -288,6 +301,33 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
     // The bias goes to LDS once: read per tile from global memory, its 16 scattered loads sat in every epilogue with
     // their full latency exposed (the accumulators are done, nothing else is left to do).
     for (int k = tid; k < t.n_kblocks * K_BLK; k += NT) bias_l[k] = (bias != nullptr && k < g.K) ? bias[k] : 0.0f;
+    // pooled position slot j of this lane inside a tile: image << 20 | pooled row << 10 | pooled column
+    int pool_pos[POOL ? MT / 4 : 1];
+    if constexpr (POOL) {
+#pragma unroll
+        for (int j = 0; j < MT / 4; ++j) {
+            const int pp = (wm * (MT / 4) + j) * 32 + l32;
+            const int img = pp / per_img_p, rem = pp - img * per_img_p;
+            const int pr = rem / t.POW, pc = rem - pr * t.POW;
+            pool_pos[j] = (min(img, 1023) << 20) | (min(pr, 1023) << 10) | min(pc, 1023);
+        }
+    } else {
+        pool_pos[0] = 0;
+    }
+    // likewise the unpooled position slots: image << 24 | row << 12 | column (NB < 256, rows and columns < 4096: the
+    // planner's limits)
+    int out_pos[POOL ? 1 : MT];
+    if constexpr (!POOL) {
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const int p = (wm * MT + i) * 32 + l32;
+            const int img = p / per_img, rem = p - img * per_img;
+            const int r = rem / g.OW, c = rem - r * g.OW;
+            out_pos[i] = (min(img, 255) << 24) | (min(r, 4095) << 12) | min(c, 4095);
+        }
+    } else {
+        out_pos[0] = 0;
+    }
     if (tid == 0) sched[0] = blockIdx.x + gridDim.x;  // the second tile is static, later ones come from the counter
     // Two counters take turns: this launch draws from tile_counters[parity] and re-arms the other one for the next
     // launch of the same operator, so that packed weights and counters can be kept across calls without a reset pass.
@@ -410,23 +450,22 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
                 for (int v = 0; v < 16; ++v) bv[v] = __int_as_float(raw[v]);
             }
             if constexpr (POOL) {
-                // max over the window, then bias and ReLU: both are monotone, so this equals pool(relu(conv + bias))
+                // max over the window, then bias and ReLU: both are monotone, so this equals pool(relu(conv + bias)).
+                // The lane's pooled position inside the tile (image, row, column) never changes: it was divided out once,
+                // before the tile loop (pool_pos).
                 const int prows_here = min(t.TH / 2, g.OH / 2 - oh0 / 2);
                 const int64_t pplane = int64_t(g.OH / 2) * t.POW;
 #pragma unroll
                 for (int j = 0; j < MT / 4; ++j) {
-                    const int pp = (wm * (MT / 4) + j) * 32 + l32;
-                    const int img = pp / per_img_p, rem = pp - img * per_img_p;
-                    const int pr = rem / t.POW, pc = rem - pr * t.POW;
+                    const int img = pool_pos[j] >> 20, pr = (pool_pos[j] >> 10) & 1023, pc = pool_pos[j] & 1023;
                     if (img < imgs_here && pr < prows_here) {
                         float *yp = y + (int64_t(n0 + img) * g.K + kbase) * pplane + int64_t(oh0 / 2 + pr) * t.POW + pc;
 #pragma unroll
                         for (int v = 0; v < 16; ++v) {
                             const int dk = (v >> 2) * 8 + (v & 3);
                             if (full_k || kbase + dk < g.K) {
-                                float o = fmaxf(fmaxf(acc[4 * j][v], acc[4 * j + 1][v]), fmaxf(acc[4 * j + 2][v], acc[4 * j + 3][v])) + bv[v];
-                                if (relu) o = o > 0.0f ? o : 0.0f;
-                                yp[dk * pplane] = o;
+                                const float o = vmax(vmax3(acc[4 * j][v], acc[4 * j + 1][v], acc[4 * j + 2][v]), acc[4 * j + 3][v]) + bv[v];
+                                yp[dk * pplane] = relu ? vmax(o, 0.0f) : o;
                             }
                         }
                     }
@@ -434,19 +473,15 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
             } else
 #pragma unroll
             for (int i = 0; i < MT; ++i) {
-                const int p = (wm * MT + i) * 32 + l32;
-                const int img = p / per_img, rem = p - img * per_img;
-                const int r = rem / g.OW, c = rem - r * g.OW;
+                // (image, row, column) of the lane's position slot i inside the tile: divided out once (out_pos)
+                const int img = int(unsigned(out_pos[i]) >> 24), r = (out_pos[i] >> 12) & 0xfff, c = out_pos[i] & 0xfff;
                 if (img < imgs_here && r < rows_here) {
                     float *yp = y + (int64_t(n0 + img) * g.K + kbase) * plane + int64_t(oh0 + r) * g.OW + c;
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
                         const int dk = (v >> 2) * 8 + (v & 3);
-                        if (full_k || kbase + dk < g.K) {
-                            float o = acc[i][v] + bv[v];
-                            if (relu) o = o > 0.0f ? o : 0.0f;
-                            yp[dk * plane] = o;
-                        }
+                        const float o = acc[i][v] + bv[v];
+                        if (full_k || kbase + dk < g.K) yp[dk * plane] = relu ? vmax(o, 0.0f) : o;  // (a NaN passes where there is no ReLU)
                     }
                 }
             }
@@ -592,19 +627,6 @@ conv_f32_smallc_pool_kernel(const float *__restrict__ x, const float *__restrict
             bcur = bnext;
         }
     }
-}
-
-// max without the NaN-quieting pass the compiler puts in front of fmaxf (an MFMA result is never a signalling NaN); a NaN
-// operand yields the other one, like fmaxf
-__device__ __forceinline__ float vmax(float a, float b) {
-    float r;
-    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
-    return r;
-}
-__device__ __forceinline__ float vmax3(float a, float b, float c) {
-    float r;
-    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-    return r;
 }
 
 // Single-channel 3x3 first layer + ReLU + MaxPool 2x2/2 on the matrix cores (stride 1, no padding).
