@@ -391,6 +391,13 @@ gemm_f32_dma_kernel(const float *__restrict__ A, const float *__restrict__ B, co
     if ((gridDim.x & 7) != 0) sb = blockIdx.x;
     const int bm = sb / n_tiles, bn = sb - bm * n_tiles;
     const int m0 = bm * BM, n0 = bn * BN;
+    // A C that is broadcast along the rows (a bias vector) is one value per lane: fetched now, it is there when the
+    // epilogue wants it instead of costing a memory round trip after the last MFMA.
+    float c_row = 0.0f;
+    {
+        const int nc = n0 + wn * 32 + l32;
+        if (g.c_mode && g.c_ld_r == 0 && nc < g.N) c_row = C[int64_t(nc) * g.c_ld_c];
+    }
 
     f32x16 acc[MT];
 #pragma unroll
@@ -459,7 +466,7 @@ gemm_f32_dma_kernel(const float *__restrict__ A, const float *__restrict__ B, co
         float cv[MT][16];
         if (g.c_mode) {
             if (g.c_ld_r == 0) {
-                const float c0 = C[int64_t(n) * g.c_ld_c];
+                const float c0 = c_row;
 #pragma unroll
                 for (int i = 0; i < MT; ++i)
 #pragma unroll
