@@ -257,11 +257,35 @@ def main():
 
     # ---- HBM-bound operators (pool / activation / requantisation / residual add): algorithmic bytes / kernel time ----
     if operators is not None:
+        # What the machine gives a plain device-to-device copy moving the same number of bytes (half read, half
+        # written), measured here with HIP events: the practical ceiling of a streaming kernel of that size, beside the
+        # fraction of the 8 TB/s peak.
+        copy_cache = {}
+
+        def copy_gbs(nbytes):
+            half = max(int(nbytes) // 2 // 256 * 256, 256)
+            if half not in copy_cache:
+                src = torch.empty(half, dtype=torch.uint8, device=dev).fill_(1)
+                dst = torch.empty_like(src)
+                for _ in range(3):
+                    dst.copy_(src)
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                torch.cuda.synchronize()
+                e0.record()
+                for _ in range(10):
+                    dst.copy_(src)
+                e1.record()
+                torch.cuda.synchronize()
+                copy_cache[half] = 2 * half / (e0.elapsed_time(e1) / 10) / 1e6
+                del src, dst
+            return copy_cache[half]
+
         def hbm(name, fn, nbytes):
             fn()
             ms = kernel_avg_ms(ctx, fn, 5)
             operators[name] = {"ms": round(ms, 4), "gbs": round(nbytes / ms / 1e6, 1),
-                               "frac_hbm_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
+                               "frac_hbm_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4),
+                               "plain_copy_same_bytes_gbs": round(copy_gbs(nbytes), 1)}
 
         xf = torch.randn(4096, 32, 26, 26, device=dev)
         yf = torch.empty_like(xf)
