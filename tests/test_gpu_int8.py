@@ -35,6 +35,12 @@ QCASES = [
     (65, 90, 1, 1, 70, 1, 1, [1, 1], [0, 0, 0, 0], [1, 1], 1),      # 6 blocks, the last one partly filled: groups of 2
     (128, 64, 1, 1, 64, 1, 1, [2, 2], [0, 0, 0, 0], [1, 1], 1),     # 4 blocks: groups of 2 (a stride changes nothing)
     (70, 200, 1, 1, 40, 1, 1, [1, 1], [0, 0, 0, 0], [1, 1], 1),     # 13 blocks: not regrouped
+    # 3x3 stride-1 layers of 32 channels and up whose NCHW output leaves in dwords of four positions (rows of whole
+    # quads), with a channel count that ends inside a group of four and inside a block of 32:
+    (3, 32, 10, 12, 42, 3, 3, [1, 1], [1, 1, 1, 1], [1, 1], 1),     # 12-wide rows, 42 channels
+    (2, 48, 14, 18, 75, 3, 3, [1, 1], [0, 0, 0, 0], [1, 1], 1),     # no padding, 16-wide rows, 75 channels
+    (5, 64, 37, 8, 66, 3, 3, [1, 1], [1, 1, 1, 1], [1, 1], 1),      # 37 rows of 8: a last tile of fewer rows
+    (2, 40, 9, 9, 50, 3, 3, [1, 1], [1, 1, 1, 1], [1, 1], 1),       # rows that are not whole quads: byte stores
 ]
 
 
@@ -53,6 +59,25 @@ def test_qlinearconv_bit_exact(G, case, act):
     y = G.tm.qlinearconv(G.dev(x), 0.02, 128, G.dev(w), G.dev(ws), None, 0.05, 128, G.dev(b), s, p, d, grp, **kw)
     np.testing.assert_array_equal(G.host(y), ref)
     assert len(np.unique(ref)) > 8  # the case really exercises requantisation
+
+
+@pytest.mark.parametrize("shift", [1, 2, 4])
+def test_qlinearconv_output_at_an_odd_address(G, shift):
+    """An NCHW output that does not start on a 4-byte boundary takes the byte-store epilogue; nothing around it is written."""
+    import torch
+    N, C, H, W, K = 2, 32, 6, 8, 36
+    g = np.random.default_rng(40 + shift)
+    x = g.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+    w = g.integers(-127, 128, (K, C, 3, 3), dtype=np.int8)
+    ws = (g.uniform(0.5, 1.5, K) * 0.08 / np.sqrt(C * 9)).astype(np.float32)
+    b = g.integers(-1000, 1001, K, dtype=np.int32)
+    ref = zo.qlinearconv(x, 0.02, 128, w, ws, None, 0.05, 128, b, [1, 1], [1, 1, 1, 1], [1, 1], 1)
+    buf = torch.full((ref.size + 64,), 7, dtype=torch.uint8, device="cuda:0")
+    y = buf[shift:shift + ref.size].view(N, K, H, W)
+    G.tm.qlinearconv_lean(G.dev(x), 0.02, 128, G.dev(w), G.dev(ws), None, 0.05, 128, G.dev(b), y, [1, 1], [1, 1, 1, 1], [1, 1])
+    out = buf.cpu().numpy()
+    np.testing.assert_array_equal(out[shift:shift + ref.size].reshape(ref.shape), ref)
+    assert (out[:shift] == 7).all() and (out[shift + ref.size:] == 7).all()
 
 
 def test_qlinearconv_per_tensor_scale_weight_zero_point_no_bias(G):

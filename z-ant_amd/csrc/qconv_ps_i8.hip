@@ -398,6 +398,8 @@ qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, co
                 const int plane = p.OH * p.OW;
                 const float zpf = float(q.y_zp);
                 const unsigned img_stride = unsigned((y_blocked ? p.KB : p.K) * plane);
+                // NCHW output in dwords of four positions: rows, planes and tile rows of whole quads, an aligned base
+                const bool quad_rows = !y_blocked && (p.OW & 3) == 0 && (reinterpret_cast<uintptr_t>(y) & 3) == 0;
                 // where this lane's position slots lie
                 uint32_t praw[MT];
 #pragma unroll
@@ -473,7 +475,36 @@ qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, co
                             for (int v = 0; v < 16; ++v)
                                 ob[v] = ps_read_u8(__builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(float(av[v]) * mv[v]) + zpf, 0u, lut_a));
                             ps_wait16(ob);
-                            if (ok) {
+                            if (quad_rows) {
+                                // Four lanes of a quad hold four consecutive positions of one row; a 4 x 4 byte transpose
+                                // across them (two lane exchanges and two byte permutes per group of four channels) leaves
+                                // lane q of the quad with channel q's four position bytes: a dword store per group where
+                                // there were four byte stores.  (Plain stores: the cache gathers the 32-byte pieces of a
+                                // line that successive position tiles write; non-temporal ones were slower.)
+                                // Everything derived from the lane number is made here, per tile, behind an opaque copy:
+                                // held across the main loop it would not fit this kernel's registers.
+                                uint32_t lq = uint32_t(lane);
+                                asm volatile("" : "+v"(lq));
+                                // sel1 = lane & 1 ? 0x03070105 : 0x06020400, sel2 = lane & 2 ? 0x03020706 : 0x05040100, without a
+                                // register per constant
+                                uint32_t sel1, sel2;
+                                asm volatile("v_bfe_i32 %0, %2, 0, 1\n\tv_bfe_i32 %1, %2, 1, 1\n\t"
+                                             "v_and_b32 %0, 0x05050505, %0\n\tv_and_b32 %1, 0x06060606, %1\n\t"
+                                             "v_xor_b32 %0, 0x06020400, %0\n\tv_xor_b32 %1, 0x05040100, %1"
+                                             : "=&v"(sel1), "=&v"(sel2) : "v"(lq));
+                                const unsigned lq3 = lq & 3;
+#pragma unroll
+                                for (int gq = 0; gq < 4; ++gq) {
+                                    const uint32_t d0 = ob[gq * 4] | (ob[gq * 4 + 1] << 8) | (ob[gq * 4 + 2] << 16) | (ob[gq * 4 + 3] << 24);
+                                    const uint32_t x1 = uint32_t(__builtin_amdgcn_update_dpp(0, int(d0), 0xB1, 0xf, 0xf, false));  // lane ^ 1
+                                    const uint32_t t1 = __builtin_amdgcn_perm(x1, d0, sel1);
+                                    const uint32_t x2 = uint32_t(__builtin_amdgcn_update_dpp(0, int(t1), 0x4E, 0xf, 0xf, false));  // lane ^ 2
+                                    const uint32_t o4 = __builtin_amdgcn_perm(x2, t1, sel2);
+                                    const int dk = gq * 8 + int(lq3);
+                                    if (ok && kbase + dk < p.K)
+                                        *reinterpret_cast<uint32_t *>(y + (origin + rel - lq3 + unsigned(dk * plane))) = o4;
+                                }
+                            } else if (ok) {
                                 uint8_t *yp = y + (origin + rel);
 #pragma unroll
                                 for (int v = 0; v < 16; ++v) {
