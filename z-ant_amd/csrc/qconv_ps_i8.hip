@@ -227,14 +227,14 @@ __device__ __forceinline__ void ps_mfma_step(unsigned wr, const unsigned (&xbase
 }
 
 // OUT: how the output bytes are formed and stored.
-enum { PS_OUT_NCHW = 0, PS_OUT_BLOCKED_LUT = 1, PS_OUT_BLOCKED = 2 };
+enum { PS_OUT_NCHW_LUT = 0, PS_OUT_BLOCKED_LUT = 1, PS_OUT_BLOCKED = 2, PS_OUT_NCHW = 3 };
 
 // tabs: the per-channel requantisation multipliers (kpad floats) followed by the integer corrections (kpad ints).
 template <int MT, int OUT>
 __global__ void __launch_bounds__(PS_NT)
 qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, const char *__restrict__ tabs,
                 const int8_t *__restrict__ padvec, uint8_t *__restrict__ y, PsGeom p, QConvArgs q) {
-    constexpr bool y_blocked = OUT != PS_OUT_NCHW, use_lut = OUT != PS_OUT_BLOCKED;
+    constexpr bool y_blocked = OUT == PS_OUT_BLOCKED_LUT || OUT == PS_OUT_BLOCKED, use_lut = OUT == PS_OUT_BLOCKED_LUT || OUT == PS_OUT_NCHW_LUT;
     extern __shared__ __attribute__((aligned(256))) char ps_lds_raw[];
     // LDS: [256-byte activation table, 256-aligned][multipliers, corrections][weight ring: 2 slabs][slot table]
     //      [patch: 2*NC blocks x P1s x 16]
@@ -437,28 +437,29 @@ qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, co
                         int av[16];  // this tile's sums with the corrections added
 #pragma unroll
                         for (int v = 0; v < 16; ++v) av[v] = acc[j][i][v] + int(craw[v]);
-                        if constexpr (y_blocked) {
-                            // [N][KB][OH][OW][16] signed.  A lane holds 4 groups of 4 consecutive channels of one position
-                            uint32_t d[4];
-                            if constexpr (use_lut) {
-                                uint32_t ob[16];
+                        // four dwords of four consecutive channels each, of one position (signed bytes for the blocked layout)
+                        uint32_t d[4];
+                        if constexpr (use_lut) {
+                            uint32_t ob[16];
 #pragma unroll
-                                for (int v = 0; v < 16; ++v)
-                                    ob[v] = ps_read_u8(__builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(float(av[v]) * mv[v]) + zpf, 0u, lut_a));
-                                ps_wait16(ob);
+                            for (int v = 0; v < 16; ++v)
+                                ob[v] = ps_read_u8(__builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(float(av[v]) * mv[v]) + zpf, 0u, lut_a));
+                            ps_wait16(ob);
 #pragma unroll
-                                for (int gq = 0; gq < 4; ++gq)
-                                    d[gq] = ob[gq * 4] | (ob[gq * 4 + 1] << 8) | (ob[gq * 4 + 2] << 16) | (ob[gq * 4 + 3] << 24);
-                            } else {
+                            for (int gq = 0; gq < 4; ++gq)
+                                d[gq] = ob[gq * 4] | (ob[gq * 4 + 1] << 8) | (ob[gq * 4 + 2] << 16) | (ob[gq * 4 + 3] << 24);
+                        } else {
 #pragma unroll
-                                for (int gq = 0; gq < 4; ++gq) {
-                                    uint32_t w4 = 0;
+                            for (int gq = 0; gq < 4; ++gq) {
+                                uint32_t w4 = 0;
 #pragma unroll
-                                    for (int e = 0; e < 4; ++e)
-                                        w4 = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(float(av[gq * 4 + e]) * mv[gq * 4 + e]) + zpf, unsigned(e), w4);
-                                    d[gq] = w4 ^ 0x80808080u;
-                                }
+                                for (int e = 0; e < 4; ++e)
+                                    w4 = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(float(av[gq * 4 + e]) * mv[gq * 4 + e]) + zpf, unsigned(e), w4);
+                                d[gq] = y_blocked ? w4 ^ 0x80808080u : w4;
                             }
+                        }
+                        if constexpr (y_blocked) {
+                            // [N][KB][OH][OW][16] signed.  A lane holds 4 groups of 4 consecutive channels of one position.
                             // Lanes l and l + 32 hold the two interleaved halves of the wave's two 16-channel blocks: the
                             // half-wave swap leaves the lower lane with all 16 bytes of the first block and the upper lane
                             // with those of the second, so each lane stores one whole 16-byte unit and a half wave 512
@@ -470,17 +471,13 @@ qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, co
                             if (ok && cb0 + lh < p.KB)
                                 __builtin_nontemporal_store(out, reinterpret_cast<u32x4 *>(y) + (origin + rel + unsigned(lh * plane)));
                         } else {
-                            uint32_t ob[16];
-#pragma unroll
-                            for (int v = 0; v < 16; ++v)
-                                ob[v] = ps_read_u8(__builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(float(av[v]) * mv[v]) + zpf, 0u, lut_a));
-                            ps_wait16(ob);
                             if (quad_rows) {
                                 // Four lanes of a quad hold four consecutive positions of one row; a 4 x 4 byte transpose
                                 // across them (two lane exchanges and two byte permutes per group of four channels) leaves
                                 // lane q of the quad with channel q's four position bytes: a dword store per group where
                                 // there were four byte stores.  (Plain stores: the cache gathers the 32-byte pieces of a
-                                // line that successive position tiles write; non-temporal ones were slower.)
+                                // line that successive position tiles write; non-temporal ones were slower, and a further transpose to
+                                // one 16-byte store per lane gained nothing.)
                                 // Everything derived from the lane number is made here, per tile, behind an opaque copy:
                                 // held across the main loop it would not fit this kernel's registers.
                                 uint32_t lq = uint32_t(lane);
@@ -495,7 +492,7 @@ qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, co
                                 const unsigned lq3 = lq & 3;
 #pragma unroll
                                 for (int gq = 0; gq < 4; ++gq) {
-                                    const uint32_t d0 = ob[gq * 4] | (ob[gq * 4 + 1] << 8) | (ob[gq * 4 + 2] << 16) | (ob[gq * 4 + 3] << 24);
+                                    const uint32_t d0 = d[gq];
                                     const uint32_t x1 = uint32_t(__builtin_amdgcn_update_dpp(0, int(d0), 0xB1, 0xf, 0xf, false));  // lane ^ 1
                                     const uint32_t t1 = __builtin_amdgcn_perm(x1, d0, sel1);
                                     const uint32_t x2 = uint32_t(__builtin_amdgcn_update_dpp(0, int(t1), 0x4E, 0xf, 0xf, false));  // lane ^ 2
@@ -509,7 +506,7 @@ qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, co
 #pragma unroll
                                 for (int v = 0; v < 16; ++v) {
                                     const int dk = (v >> 2) * 8 + (v & 3);
-                                    if (kbase + dk < p.K) yp[dk * plane] = uint8_t(ob[v]);
+                                    if (kbase + dk < p.K) yp[dk * plane] = uint8_t(d[v >> 2] >> ((v & 3) * 8));
                                 }
                             }
                         }
@@ -646,7 +643,8 @@ void ps_launch_out(zant_ctx *ctx, int grid, size_t lds, const int8_t *xb, const 
 template <int MT>
 void ps_launch(zant_ctx *ctx, int grid, size_t lds, const int8_t *xb, const int8_t *wp, const char *tabs,
                const int8_t *padvec, uint8_t *y, const PsGeom &p, const QConvArgs &q, int yb) {
-    if (!yb) ps_launch_out<MT, PS_OUT_NCHW>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
+    if (!yb && q.has_act) ps_launch_out<MT, PS_OUT_NCHW_LUT>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
+    else if (!yb) ps_launch_out<MT, PS_OUT_NCHW>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
     else if (q.has_act) ps_launch_out<MT, PS_OUT_BLOCKED_LUT>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
     else ps_launch_out<MT, PS_OUT_BLOCKED>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
 }
