@@ -1000,62 +1000,81 @@ qfirst_mfma_kernel(const uint8_t *__restrict__ x, const uint4 *__restrict__ wpk,
     const int KB16 = (g.K + 15) >> 4;
     const unsigned per_img = unsigned(OHo) * unsigned(OWo), total = unsigned(g.N) * per_img;  // < 2^31 (host)
     const unsigned n_ptiles = (total + 31u) / 32u;
-    const float inv_per_img = 1.0f / float(per_img), inv_owo = 1.0f / float(OWo);
-    const bool small_total = total < (1u << 20);
     const uint32_t padb = uint32_t(q.x_zp ^ 0x80) & 0xffu, pad4 = padb * 0x01010101u;
     const float zpf = float(q.y_zp);
-    const int64_t plane_in = int64_t(g.H) * g.W;
-    const unsigned wave_id = (blockIdx.x * blockDim.x + threadIdx.x) >> 6, n_waves = (gridDim.x * blockDim.x) >> 6;
+    const unsigned plane_in = unsigned(g.H) * unsigned(g.W), img_in = unsigned(C) * plane_in;  // the input is < 2^32 bytes (host)
+    const unsigned wave_id = unsigned(__builtin_amdgcn_readfirstlane(int((blockIdx.x * blockDim.x + threadIdx.x) >> 6)));
+    const unsigned n_waves = (gridDim.x * blockDim.x) >> 6;
     i32x16 cvec;
     float mv[16];
     i32x4 wa_all[NCH], wa_dx1[NCH];
     bool tables_loaded = false, any_negative = false;
+    // This lane's position in the next tile to load, as (image, row, column) of the (pooled) output.  Successive tiles
+    // of a wavefront lie n_waves * 32 positions apart: the triple advances by that step's own (images, rows, columns)
+    // with two carries, and is divided out only once.
+    unsigned wn;
+    int woho, wowo;
+    {
+        const unsigned i = wave_id * 32u + unsigned(l32);
+        wn = i / per_img;
+        const unsigned rem = i - wn * per_img;
+        woho = int(rem / unsigned(OWo));
+        wowo = int(rem - unsigned(woho) * unsigned(OWo));
+    }
+    const unsigned step = n_waves * 32u;
+    const unsigned d_n = step / per_img, step_r = step - d_n * per_img;
+    const int d_oho = int(step_r / unsigned(OWo)), d_owo = int(step_r - unsigned(d_oho) * unsigned(OWo));
     // The row loads of the NEXT tile are issued before this tile's arithmetic: with two wavefronts per SIMD the load
     // latency would otherwise sit on the critical path of every tile.
     struct TileMeta { unsigned n; int oho, owo, ih0, sh; bool valid; };
     uint32_t raw[C][PR];
     TileMeta nxt;
-    auto issue = [&](unsigned pt, TileMeta &m) {
-        const unsigned i = pt * 32u + unsigned(l32);
-        m.valid = i < total;
-        const unsigned ii = m.valid ? i : total - 1u;
-        m.n = small_total ? unsigned(small_div(int(ii), int(per_img), inv_per_img)) : ii / per_img;
-        const int rem = int(ii - m.n * per_img);
-        m.oho = small_div(rem, OWo, inv_owo);
-        m.owo = rem - m.oho * OWo;
-        m.ih0 = (POOL ? 2 * m.oho : m.oho) * S - g.pt;
-        const int iw0 = (POOL ? 2 * m.owo : m.owo) * S - g.pl;
+    auto issue = [&](TileMeta &m) {
+        m.valid = wn < unsigned(g.N);           // (only the last tile has lanes past the end: they read image N - 1)
+        m.n = min(wn, unsigned(g.N) - 1u);
+        m.oho = woho;
+        m.owo = wowo;
+        m.ih0 = (POOL ? 2 * woho : woho) * S - g.pt;
+        const int iw0 = (POOL ? 2 * wowo : wowo) * S - g.pl;
         // one dword per (channel, patch row): columns iw0 .. iw0+3, read from a start clamped into the row
         const int iw0c = min(max(iw0, 0), g.W - 4);
         m.sh = iw0 - iw0c;
-        const uint8_t *xn = x + int64_t(m.n) * C * plane_in + iw0c;
+        const unsigned base = m.n * img_in + unsigned(iw0c);
+        unsigned rowoff[PR];
+#pragma unroll
+        for (int r = 0; r < PR; ++r) rowoff[r] = __umul24(unsigned(min(max(m.ih0 + r, 0), g.H - 1)), unsigned(g.W));  // H, W < 2^24 (host)
 #pragma unroll
         for (int c = 0; c < C; ++c)
 #pragma unroll
-            for (int r = 0; r < PR; ++r) {
-                const int ih = m.ih0 + r;
-                raw[c][r] = *reinterpret_cast<const u32_unaligned *>(xn + c * plane_in + int64_t(min(max(ih, 0), g.H - 1)) * g.W);
-            }
+            for (int r = 0; r < PR; ++r)
+                raw[c][r] = *reinterpret_cast<const u32_unaligned *>(x + (base + rowoff[r] + unsigned(c) * plane_in));
+        wowo += d_owo;
+        const int c1 = wowo >= OWo ? 1 : 0;
+        wowo -= c1 ? OWo : 0;
+        woho += d_oho + c1;
+        const int c2 = woho >= OHo ? 1 : 0;
+        woho -= c2 ? OHo : 0;
+        wn += d_n + unsigned(c2);
     };
-    if (wave_id < n_ptiles) issue(wave_id, nxt);
+    if (wave_id < n_ptiles) issue(nxt);
     for (unsigned pt = wave_id; pt < n_ptiles; pt += n_waves) {
         const TileMeta cur = nxt;
         const unsigned n = cur.n;
         const int oho = cur.oho, owo = cur.owo, ih0 = cur.ih0, sh = cur.sh;
         const bool valid = cur.valid;
-        // shifted into place; columns outside the image (and rows outside it) take the padding byte
+        // Shifted into place with one byte permute per dword: selector byte b picks data byte b + sh (4 + b + sh in the
+        // permute's numbering) or, where that falls outside the dword, a padding byte (0).  A start clamped at the left
+        // edge (sh = -1) shifts the row up behind one padding byte, one clamped at the right edge (sh > 0) shifts it down
+        // with padding bytes following; a row outside the image is padding altogether.
+        const uint32_t sel = sh < 0 ? 0x06050403u : 0x07060504u >> (8 * sh);
         uint32_t row[C][PR];
 #pragma unroll
-        for (int c = 0; c < C; ++c)
+        for (int r = 0; r < PR; ++r) {
+            const uint32_t sel_r = unsigned(ih0 + r) < unsigned(g.H) ? sel : 0u;
 #pragma unroll
-            for (int r = 0; r < PR; ++r) {
-                const int ih = ih0 + r;
-                const uint32_t d = (ih >= 0 && ih < g.H) ? raw[c][r] ^ 0x80808080u : pad4;
-                // bytes of (hi:lo) >> 8 * s: a start clamped at the left edge shifts the row up behind one padding byte,
-                // one clamped at the right edge shifts it down with padding bytes following
-                row[c][r] = __builtin_amdgcn_alignbyte(sh < 0 ? d : pad4, sh < 0 ? pad4 : d, sh < 0 ? 3u : unsigned(sh));
-            }
-        if (pt + n_waves < n_ptiles) issue(pt + n_waves, nxt);
+            for (int c = 0; c < C; ++c) row[c][r] = __builtin_amdgcn_perm(raw[c][r] ^ 0x80808080u, pad4, sel_r);
+        }
+        if (pt + n_waves < n_ptiles) issue(nxt);
         for (int kb = 0; kb < kb32; ++kb) {
             const int kch = kb * 32 + lh * 4;
             if (kb32 > 1 || !tables_loaded) {  // one block of output channels: the tables stay in registers across tiles
@@ -1148,6 +1167,8 @@ bool qfirst_eligible(const ConvGeom &g, bool pool) {
     const int last = ((pool ? (g.OW / 2) * 2 : g.OW) - 1) * S - g.pl;
     if (last + 3 - (g.W - 1) > 3) return false;
     const int64_t OHo = pool ? g.OH / 2 : g.OH, OWo = pool ? g.OW / 2 : g.OW;
+    // input offsets are formed in 32 bits, row offsets with a 24-bit multiply
+    if (int64_t(g.N) * g.C * g.H * g.W >= (int64_t(1) << 32) - 64 || g.H >= (1 << 24) || g.W >= (1 << 24)) return false;
     return OHo >= 1 && OWo >= 1 && int64_t(g.N) * OHo * OWo < (int64_t(1) << 31) - 64 && OHo * OWo < (1 << 20);
 }
 
