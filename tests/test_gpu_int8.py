@@ -41,6 +41,10 @@ QCASES = [
     (2, 48, 14, 18, 75, 3, 3, [1, 1], [0, 0, 0, 0], [1, 1], 1),     # no padding, 16-wide rows, 75 channels
     (5, 64, 37, 8, 66, 3, 3, [1, 1], [1, 1, 1, 1], [1, 1], 1),      # 37 rows of 8: a last tile of fewer rows
     (2, 40, 9, 9, 50, 3, 3, [1, 1], [1, 1, 1, 1], [1, 1], 1),       # rows that are not whole quads: byte stores
+    # NCHW input of whole-dword planes on its way to the 16-channel blocked layout, the last block holding 2 and 13 channels
+    (2, 50, 8, 12, 40, 3, 3, [1, 1], [1, 1, 1, 1], [1, 1], 1),
+    (3, 45, 6, 6, 35, 3, 3, [1, 1], [0, 0, 0, 0], [1, 1], 1),
+    (70, 77, 2, 2, 40, 1, 1, [1, 1], [0, 0, 0, 0], [1, 1], 1),      # pointwise layer on 2 x 2 planes: one quad per plane
 ]
 
 

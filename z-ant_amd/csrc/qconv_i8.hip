@@ -123,6 +123,48 @@ __global__ void __launch_bounds__(256) to_blocked_s8_kernel(const uint8_t *__res
     }
 }
 
+// The same for planes of whole dwords (HW a multiple of 4, an aligned base) and fewer than 2^31 units.  A workgroup
+// turns 64 quads of positions (counted through the whole tensor: rows of (image, channel block) follow each other in
+// the output) x 16 channels.  Wavefront g loads the dwords of channels 4g .. 4g+3, a quad per lane (256 contiguous bytes
+// per load), transposes its 4 x 4 bytes with byte permutes (dword b: position b, channels 4g .. 4g+3) and writes the
+// four dwords to LDS row g; then thread u gathers unit u's four dwords (one per row, consecutive lanes on consecutive
+// banks) and stores its 16 bytes: a workgroup's stores are one run of 4 KB.
+// (One tile per workgroup: with two, all eight loads of a thread in flight together, the kernel was slower.)
+__global__ void __launch_bounds__(256) to_blocked_s8_quads_kernel(const uint8_t *__restrict__ x, uint4 *__restrict__ xb,
+                                                                 unsigned n_quads, int C, unsigned CB, unsigned HW4) {
+    __shared__ __attribute__((aligned(16))) uint32_t stage[4][256];
+    const unsigned g = threadIdx.x >> 6, lane = threadIdx.x & 63u;
+    const unsigned qi = blockIdx.x * 64u + lane;
+    uint32_t r[4] = {0u, 0u, 0u, 0u};  // r[j] = 4 consecutive positions of channel c0 + j
+    if (qi < n_quads) {
+        const unsigned row = qi / HW4, q = qi - row * HW4;  // row = image * CB + channel block
+        const unsigned n = row / CB, cb = row - n * CB;
+        const int c0 = int(cb) * 16 + int(g) * 4;
+        const uint32_t *src = reinterpret_cast<const uint32_t *>(x) + (int64_t(n) * C * HW4 + q);
+        // The four loads leave together: a channel past C reads channel C - 1 instead of branching around its load
+        // (with a branch per load the compiler waited for each one before the next), and is zeroed afterwards.
+        uint32_t v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = __builtin_nontemporal_load(src + int64_t(min(c0 + j, C - 1)) * HW4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) r[j] = c0 + j < C ? v[j] ^ 0x80808080u : 0u;
+    }
+    const uint32_t lo01 = __builtin_amdgcn_perm(r[1], r[0], 0x05010400u);  // r0.0 r1.0 r0.1 r1.1
+    const uint32_t hi01 = __builtin_amdgcn_perm(r[1], r[0], 0x07030602u);  // r0.2 r1.2 r0.3 r1.3
+    const uint32_t lo23 = __builtin_amdgcn_perm(r[3], r[2], 0x05010400u);
+    const uint32_t hi23 = __builtin_amdgcn_perm(r[3], r[2], 0x07030602u);
+    uint4 o;  // dword b: position b, channels c0 .. c0+3
+    o.x = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);
+    o.y = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+    o.z = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
+    o.w = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
+    *reinterpret_cast<uint4 *>(&stage[g][lane * 4]) = o;
+    __syncthreads();
+    const unsigned u = threadIdx.x;
+    if (blockIdx.x * 64u + (u >> 2) < n_quads)
+        xb[int64_t(blockIdx.x) * 256 + u] = make_uint4(stage[0][u], stage[1][u], stage[2][u], stage[3][u]);
+}
+
 // Packs OIHW int8 weights into [chunk][kblock][tap][half][K_BLK][16] (zero padded; fc_g > 0: the weights of a 1x1
 // layer with c_orig channels, read as a 1 x fc_g filter over C = 16 * ceil(c_orig / 16) / fc_g channels), and writes the
 // per-channel requantisation multiplier, the integer correction (bias + (128 - x_zp) * sum w), the
@@ -751,11 +793,8 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
         ZANT_LAUNCH_CHECK(ctx);
     }
     if (!x_blocked) {
-        const int64_t hw = int64_t(g0.H) * g0.W;
-        const int vec_ok = (hw % 4 == 0) && (reinterpret_cast<uintptr_t>(x) % 4 == 0);
-        hipLaunchKernelGGL(to_blocked_s8_kernel, dim3(to_blocked_grid(ctx, g0.N, CB0, hw)), dim3(256), 0, ctx->stream, x,
-                           static_cast<uint4 *>(dyn), g0.N, g0.C, CB0, hw, vec_ok);
-        ZANT_LAUNCH_CHECK(ctx);
+        const int rc2 = zant_to_blocked(ctx, x, g0.N, g0.C, int64_t(g0.H) * g0.W, static_cast<uint8_t *>(dyn));
+        if (rc2) return rc2;
     }
     KernelTimer kt(ctx);
     const int yb = y_blocked ? 1 : 0;
@@ -1538,8 +1577,13 @@ int zant_to_blocked(zant_ctx *ctx, const uint8_t *x, int64_t N, int64_t C, int64
     const int64_t CB = (C + 15) / 16;
     const int vec_ok = (HW % 4 == 0) && (reinterpret_cast<uintptr_t>(x) % 4 == 0);
     KernelTimer kt(ctx);
-    hipLaunchKernelGGL(to_blocked_s8_kernel, dim3(to_blocked_grid(ctx, N, CB, HW)), dim3(256), 0, ctx->stream, x,
-                       reinterpret_cast<uint4 *>(xb), int(N), int(C), int(CB), HW, vec_ok);
+    const int64_t quads = N * CB * (HW / 4);  // (16-byte units of the blocked tensor, four at a time)
+    if (vec_ok && quads < (int64_t(1) << 29))
+        hipLaunchKernelGGL(to_blocked_s8_quads_kernel, dim3(unsigned((quads + 63) / 64)), dim3(256), 0, ctx->stream, x,
+                           reinterpret_cast<uint4 *>(xb), unsigned(quads), int(C), unsigned(CB), unsigned(HW / 4));
+    else
+        hipLaunchKernelGGL(to_blocked_s8_kernel, dim3(to_blocked_grid(ctx, N, CB, HW)), dim3(256), 0, ctx->stream, x,
+                           reinterpret_cast<uint4 *>(xb), int(N), int(C), int(CB), HW, vec_ok);
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
 }

@@ -527,35 +527,56 @@ __global__ void __launch_bounds__(256)
 ps_pack_kernel(const int8_t *__restrict__ w, const float *__restrict__ w_scale, const int32_t *__restrict__ bias,
                int8_t *__restrict__ wp, float *__restrict__ mult, int32_t *__restrict__ corr, int8_t *__restrict__ padvec,
                int K, int C, int NC, int NKP, int KP, float x_scale, float y_scale, int x_zp, int n_wscale) {
-    const int64_t total = int64_t(NKP) * NC * 9 * 32 * KP;
-    const int64_t step = int64_t(gridDim.x) * blockDim.x;
-    const int64_t gid = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    // (fewer than 2^31 packed bytes: the host checks; KP is 64 or 128)
+    const unsigned total = unsigned(NKP) * unsigned(NC) * 9u * 32u * unsigned(KP);
+    const unsigned step = gridDim.x * blockDim.x;
+    const unsigned gid = blockIdx.x * blockDim.x + threadIdx.x;
+    const int kp_shift = KP == 128 ? 7 : 6;
     if (gid < 16) padvec[gid] = int8_t(x_zp - 128);
-    for (int64_t i = gid; i < total; i += step) {
-        int64_t r = i;
-        const int j = int(r & 15); r >>= 4;
-        const int kk = int(r % KP); r /= KP;
-        const int half = int(r & 1); r >>= 1;
-        const int tap = int(r % 9); r /= 9;
-        const int chunk = int(r % NC); r /= NC;
-        const int kp = int(r);
-        const int k = kp * KP + kk, c = chunk * 32 + half * 16 + j;
+    for (unsigned i = gid; i < total; i += step) {
+        unsigned r = i;
+        const int j = int(r & 15u); r >>= 4;
+        const int kk = int(r & unsigned(KP - 1)); r >>= kp_shift;
+        const int half = int(r & 1u); r >>= 1;
+        const unsigned r9 = r / 9u;
+        const int tap = int(r - r9 * 9u);
+        const unsigned kp = r9 / unsigned(NC);
+        const int chunk = int(r9 - kp * unsigned(NC));
+        const int k = int(kp) * KP + kk, c = chunk * 32 + half * 16 + j;
         wp[i] = (k < K && c < C) ? w[(int64_t(k) * C + c) * 9 + tap] : int8_t(0);
     }
-    // per output channel: one wavefront sums the channel's weights
+    // per output channel: one wavefront sums the channel's weights, as dwords where the rows are whole aligned dwords
+    // (four signed bytes summed by one dot product with ones), every load of a round issued before the first add
     const int kpad = NKP * KP;
     const int lane = threadIdx.x & 63;
-    const int64_t wave = gid >> 6, n_waves = step >> 6;
-    for (int64_t k = wave; k < kpad; k += n_waves) {
+    const unsigned wave = gid >> 6, n_waves = step >> 6;
+    const int row = C * 9;
+    const bool dwords = (row & 3) == 0 && (reinterpret_cast<uintptr_t>(w) & 3) == 0;
+    for (unsigned k = wave; k < unsigned(kpad); k += n_waves) {
         int sum = 0;
-        if (k < K) {
-            const int8_t *wk = w + k * int64_t(C) * 9;
-            for (int e = lane; e < C * 9; e += 64) sum += int(wk[e]);
+        if (k < unsigned(K)) {
+            const int8_t *wk = w + int64_t(k) * row;
+            if (dwords) {
+                const int *wk4 = reinterpret_cast<const int *>(wk);
+                const int n4 = row >> 2;
+                for (int e0 = 0; e0 < n4; e0 += 8 * 64) {
+                    int v[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) {
+                        const int e = e0 + u * 64 + lane;
+                        v[u] = e < n4 ? wk4[e] : 0;
+                    }
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) sum = __builtin_amdgcn_sdot4(v[u], 0x01010101, sum, false);
+                }
+            } else {
+                for (int e = lane; e < row; e += 64) sum += int(wk[e]);
+            }
         }
         for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
         if (lane == 0) {
-            corr[k] = k < K ? (bias ? bias[k] : 0) + (128 - x_zp) * sum : 0;
-            mult[k] = k < K ? (x_scale * w_scale[n_wscale == 1 ? 0 : k]) / y_scale : 0.0f;
+            corr[k] = k < unsigned(K) ? (bias ? bias[k] : 0) + (128 - x_zp) * sum : 0;
+            mult[k] = k < unsigned(K) ? (x_scale * w_scale[n_wscale == 1 ? 0 : k]) / y_scale : 0.0f;
         }
     }
 }
@@ -660,6 +681,7 @@ int zant_qconv_ps(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float 
     int MT = 0;
     if (!ps_plan(g, ctx->num_cus, &p, &lds, &MT)) return 1;
     if (MT < 2 || MT > PS_MTMAX) return 1;
+    if (size_t(p.NKP) * p.NC * 9 * 32 * p.KP >= (size_t(1) << 31)) return 1;  // the packing kernel indexes in 32 bits
     if (plan_only) return ZANT_OK;
     const size_t wp_bytes = size_t(p.NKP) * p.NC * 9 * 32 * p.KP;
     const size_t xb_bytes = x_blocked ? 0 : size_t(g.N) * p.CB * g.H * g.W * 16;
