@@ -184,7 +184,10 @@ def test_conv_vs_oracle(G, case, relu):
 
 
 GEMM_CASES = [(64, 96, 48), (130, 70, 33), (1, 256, 10), (257, 1600, 512), (33, 5, 7), (128, 512, 10), (67, 1100, 16),
-              (19, 513, 1), (200, 64, 17)]
+              (19, 513, 1), (200, 64, 17),
+              # B stored [K][N] with N a multiple of 4 above 32 (copied in 16-byte pieces of four columns): column tiles that
+              # end inside the matrix, a K tail
+              (130, 70, 36), (96, 45, 100), (40, 160, 68)]
 
 
 @pytest.mark.parametrize("M,K,N", GEMM_CASES)

@@ -14,6 +14,7 @@ namespace {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 constexpr int BK = 32;
 
 struct GemmArgs {
@@ -189,14 +190,17 @@ __device__ __attribute__((aligned(16))) const float g_gemm_zero[4] = {0.f, 0.f, 
 //   KC layout  unit(row, u) at row*8 + (u ^ swz(row))     (XOR swizzle: a 128-byte global row segment lands in one
 //              128-byte LDS row, and lanes that read 32 different rows at the same u still hit 8 different columns)
 //   RC layout  unit(row, u) at u*ROWS + row
-enum { KC16 = 0, KC4 = 1, RC4 = 2 };
+// RC16 (the B operand only, 64 rows): stored like RC4, copied as it lies -- 16 bytes are four consecutive rows at one
+// k, a quarter of RC4's copy instructions and 256 contiguous bytes per k row -- into a [k][row] panel; a lane then
+// gathers its four consecutive k with two ds_read2_b32 (row stride 64 dwords) instead of one 128-bit read.
+enum { KC16 = 0, KC4 = 1, RC4 = 2, RC16 = 3 };
 
 // The LDS serves 128-bit reads 16 lanes at a time from 64 four-byte banks: 16 consecutive rows (two 128-byte rows
 // per 256-byte bank line) must land on 16 different 16-byte columns, so the XOR term steps every second row.
 __device__ __forceinline__ constexpr int swz(int row) { return (row >> 1) & 7; }
 
 template <int MODE, int ROWS>
-constexpr int stage_instrs() { return MODE == KC16 ? ROWS / 8 : ROWS / 2; }
+constexpr int stage_instrs() { return (MODE == KC16 || MODE == RC16) ? ROWS / 8 : ROWS / 2; }
 
 // The copies of one operand panel for chunk k0.  Every wave issues the same number of instructions whatever the
 // masks are (masked lanes fetch zeros), so the number of copies in flight per wave is known at compile time.
@@ -219,6 +223,11 @@ __device__ __forceinline__ void stage_panel(float *dst, const float *__restrict_
             const int k = k0 + ((slot ^ swz(row)) << 2) + j;
             sp = (r0 + row < R && k < K) ? src + int64_t(r0 + row) * ld + k : g_gemm_zero;
             __builtin_amdgcn_global_load_lds((gptr_t)sp, (lptr_t)(dst + i * 64), 4, 0, 0);
+        } else if (MODE == RC16) {
+            const int U = i * 64 + lane, kk = U / (ROWS / 4), row = (U % (ROWS / 4)) << 2;
+            const int k = k0 + kk;
+            sp = (r0 + row < R && k < K) ? src + int64_t(k) * ld + r0 + row : g_gemm_zero;  // (R is a multiple of 4)
+            __builtin_amdgcn_global_load_lds((gptr_t)sp, (lptr_t)(dst + i * 256), 16, 0, 0);
         } else {
             const int F = i * 64 + lane, j = F & 3, row = (F >> 2) % ROWS, u = F / (4 * ROWS);
             const int k = k0 + (u << 2) + j;
@@ -242,6 +251,9 @@ __device__ __forceinline__ void stage_ptrs(const float *(&p)[stage_instrs<MODE, 
         } else if (MODE == KC4) {
             const int F = i * 64 + lane, row = F >> 5, slot = (F >> 2) & 7, j = F & 3;
             p[ii] = src + int64_t(min(r0 + row, R - 1)) * ld + ((slot ^ swz(row)) << 2) + j;
+        } else if (MODE == RC16) {
+            const int U = i * 64 + lane, kk = U / (ROWS / 4), row = (U % (ROWS / 4)) << 2;
+            p[ii] = src + int64_t(kk) * ld + min(r0 + row, R - 4);
         } else {
             const int F = i * 64 + lane, j = F & 3, row = (F >> 2) % ROWS, u = F / (4 * ROWS);
             p[ii] = src + int64_t((u << 2) + j) * ld + min(r0 + row, R - 1);
@@ -256,7 +268,7 @@ __device__ __forceinline__ void stage_fast(float *dst, const float *const (&p)[s
 #pragma unroll
     for (int ii = 0; ii < stage_instrs<MODE, ROWS>() / NW; ++ii) {
         const int i = ii * NW + wave;
-        if (MODE == KC16) __builtin_amdgcn_global_load_lds((gptr_t)(p[ii] + koff), (lptr_t)(dst + i * 256), 16, 0, 0);
+        if (MODE == KC16 || MODE == RC16) __builtin_amdgcn_global_load_lds((gptr_t)(p[ii] + koff), (lptr_t)(dst + i * 256), 16, 0, 0);
         else __builtin_amdgcn_global_load_lds((gptr_t)(p[ii] + koff), (lptr_t)(dst + i * 64), 4, 0, 0);
     }
 }
@@ -265,14 +277,14 @@ __device__ __forceinline__ void stage_fast(float *dst, const float *const (&p)[s
 template <int MODE, int NW>
 __device__ __forceinline__ void stage_fast_one(float *dst, const float *p, int64_t koff, int wave, int ii) {
     const int i = ii * NW + wave;
-    if (MODE == KC16) __builtin_amdgcn_global_load_lds((gptr_t)(p + koff), (lptr_t)(dst + i * 256), 16, 0, 0);
+    if (MODE == KC16 || MODE == RC16) __builtin_amdgcn_global_load_lds((gptr_t)(p + koff), (lptr_t)(dst + i * 256), 16, 0, 0);
     else __builtin_amdgcn_global_load_lds((gptr_t)(p + koff), (lptr_t)(dst + i * 64), 4, 0, 0);
 }
 
 // LDS float offset of unit (row, u) of a panel.
 template <int MODE, int ROWS>
 __device__ __forceinline__ int unit_off(int row, int u) {
-    return MODE == RC4 ? (u * ROWS + row) * 4 : (row * 8 + (u ^ swz(row))) * 4;
+    return MODE == RC16 ? u * 4 * ROWS + row : MODE == RC4 ? (u * ROWS + row) * 4 : (row * 8 + (u ^ swz(row))) * 4;
 }
 
 // Operand reads and their waits are written by hand.  The compiler cannot count LDS reads that are still in flight
@@ -285,21 +297,46 @@ template <int OFF>
 __device__ __forceinline__ void lds_read128(f32x4 &v, unsigned addr) {
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
 }
+template <int OFF0, int OFF1>
+__device__ __forceinline__ void lds_read2x32(f32x2 &v, unsigned addr) {
+    asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(v) : "v"(addr), "n"(OFF0), "n"(OFF1));
+}
+// A lane's B operand of one group (four consecutive k): one 128-bit register tuple, or for RC16 the two pairs its
+// two reads fill (kept apart so that no register copy is needed to put them side by side while they are in flight).
+template <int BMODE>
+struct BOperand {
+    f32x4 v;
+    __device__ __forceinline__ float at(int j) const { return v[j]; }
+};
+template <>
+struct BOperand<RC16> {
+    f32x2 lo, hi;
+    __device__ __forceinline__ float at(int j) const { return j < 2 ? lo[j] : hi[j - 2]; }
+};
+template <int BMODE>
+constexpr int b_reads() { return BMODE == RC16 ? 2 : 1; }  // LDS reads per group for the B operand
+
 // Waits until at most N LDS reads are outstanding.  The operand registers are in/out operands so that nothing
 // that consumes them can be scheduled above the wait.
-template <int N, int MT>
-__device__ __forceinline__ void lds_wait(f32x4 (&a)[MT], f32x4 &b) {
+template <int N, int MT, int BMODE>
+__device__ __forceinline__ void lds_wait(f32x4 (&a)[MT], BOperand<BMODE> &b) {
     static_assert(MT == 1 || MT == 2 || MT == 4, "unsupported tile count");
-    if constexpr (MT == 1) asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a[0]), "+v"(b) : "n"(N));
-    else if constexpr (MT == 2) asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(a[0]), "+v"(a[1]), "+v"(b) : "n"(N));
-    else asm volatile("s_waitcnt lgkmcnt(%5)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b) : "n"(N));
+    if constexpr (BMODE == RC16) {
+        if constexpr (MT == 1) asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(a[0]), "+v"(b.lo), "+v"(b.hi) : "n"(N));
+        else if constexpr (MT == 2) asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(a[0]), "+v"(a[1]), "+v"(b.lo), "+v"(b.hi) : "n"(N));
+        else asm volatile("s_waitcnt lgkmcnt(%6)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b.lo), "+v"(b.hi) : "n"(N));
+    } else {
+        if constexpr (MT == 1) asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a[0]), "+v"(b.v) : "n"(N));
+        else if constexpr (MT == 2) asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(a[0]), "+v"(a[1]), "+v"(b.v) : "n"(N));
+        else asm volatile("s_waitcnt lgkmcnt(%5)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b.v) : "n"(N));
+    }
 }
 
 // The reads of group gi of the chunk at LDS byte address `stage`: MT units of A and one of B per lane.
 //   offa / offb: this lane's byte offsets of its group-0..3 units inside a stage (tile i of A adds i * 32 rows).
 template <int MT, int AM, int BMODE, int BM, int BN>
 __device__ __forceinline__ void read_group(unsigned stage, int gi, const unsigned (&offa)[BK / 8],
-                                           const unsigned (&offb)[BK / 8], f32x4 (&av)[MT], f32x4 &bv) {
+                                           const unsigned (&offb)[BK / 8], f32x4 (&av)[MT], BOperand<BMODE> &bv) {
     constexpr int A_TILE = (AM == RC4 ? 32 * 16 : 32 * 128);  // bytes between rows r and r + 32 of a panel
     const unsigned pa = stage + offa[gi], pb = stage + BM * BK * 4 + offb[gi];
     lds_read128<0>(av[0], pa);
@@ -308,7 +345,13 @@ __device__ __forceinline__ void read_group(unsigned stage, int gi, const unsigne
         lds_read128<2 * A_TILE>(av[2], pa);
         lds_read128<3 * A_TILE>(av[3], pa);
     }
-    lds_read128<0>(bv, pb);
+    if constexpr (BMODE == RC16) {
+        static_assert(BN * 3 < 256, "ds_read2_b32 offsets are 8-bit dword counts");
+        lds_read2x32<0, BN>(bv.lo, pb);
+        lds_read2x32<2 * BN, 3 * BN>(bv.hi, pb);
+    } else {
+        lds_read128<0>(bv.v, pb);
+    }
 }
 
 // One pipeline step: start the copies of chunk `ichunk` into `dma`, multiply the chunk at LDS address `cmp_addr`,
@@ -316,7 +359,7 @@ __device__ __forceinline__ void read_group(unsigned stage, int gi, const unsigne
 template <int MT, int WM, int WN, int AM, int BMODE, bool FAST>
 __device__ __forceinline__ void gemm_step(float *__restrict__ dma, unsigned cmp_addr, unsigned nxt_addr,
                                           const unsigned (&offa)[BK / 8], const unsigned (&offb)[BK / 8],
-                                          f32x4 (&a)[2][MT], f32x4 (&b)[2],
+                                          f32x4 (&a)[2][MT], BOperand<BMODE> (&b)[2],
                                           const float *__restrict__ A, const float *__restrict__ B, const GemmArgs &g,
                                           const float *const (&pa)[stage_instrs<AM, WM * MT * 32>() / (WM * WN)],
                                           const float *const (&pb)[stage_instrs<BMODE, WN * 32>() / (WM * WN)],
@@ -332,7 +375,7 @@ __device__ __forceinline__ void gemm_step(float *__restrict__ dma, unsigned cmp_
     // caller runs the fast steps and the others in two loops of their own: with both in one loop body the operand
     // registers of the two paths were reconciled by eight 64-bit register copies per step, paid in matrix-pipe time.
     const int64_t koffa = AM == RC4 ? int64_t(ichunk) * BK * g.lda : int64_t(ichunk) * BK;
-    const int64_t koffb = BMODE == RC4 ? int64_t(ichunk) * BK * g.ldb : int64_t(ichunk) * BK;
+    const int64_t koffb = (BMODE == RC4 || BMODE == RC16) ? int64_t(ichunk) * BK * g.ldb : int64_t(ichunk) * BK;
     if (!FAST) {
         stage_panel<AM, BM, NW>(dma, A, g.lda, m0, g.M, ichunk * BK, g.K, wave, lane);
         stage_panel<BMODE, BN, NW>(dma + BM * BK, B, g.ldb, n0, g.N, ichunk * BK, g.K, wave, lane);
@@ -349,12 +392,12 @@ __device__ __forceinline__ void gemm_step(float *__restrict__ dma, unsigned cmp_
         // next step starts with its operands in registers (or on their way).
         if (gi + 1 < BK / 8) read_group<MT, AM, BMODE, BM, BN>(cmp_addr, gi + 1, offa, offb, a[cur ^ 1], b[cur ^ 1]);
         else read_group<MT, AM, BMODE, BM, BN>(nxt_addr, 0, offa, offb, a[0], b[0]);
-        lds_wait<MT + 1, MT>(a[cur], b[cur]);  // everything but the MT + 1 reads just issued has landed
+        lds_wait<MT + b_reads<BMODE>(), MT>(a[cur], b[cur]);  // everything but the reads just issued has landed
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int i = 0; i < MT; ++i) {
-                acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][i][j], b[cur][j], acc[i], 0, 0, 0);
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][i][j], b[cur].at(j), acc[i], 0, 0, 0);
                 if (FAST) {
                     if (q < PA) stage_fast_one<AM, NW>(dma, pa[q < PA ? q : 0], koffa, wave, q);
                     else if (q < PA + PB) stage_fast_one<BMODE, NW>(dma + BM * BK, pb[q >= PA && q < PA + PB ? q - PA : 0], koffb, wave, q - PA);
@@ -428,7 +471,8 @@ gemm_f32_dma_kernel(const float *__restrict__ A, const float *__restrict__ B, co
         offb[gi] = unsigned(unit_off<BMODE, BN>(wn * 32 + l32, gi * 2 + lh)) * 4u;
     }
     const unsigned lds0 = lds_addr(lds);
-    f32x4 ra[2][MT], rb[2];
+    f32x4 ra[2][MT];
+    BOperand<BMODE> rb[2];
     read_group<MT, AM, BMODE, BM, BN>(lds0, 0, offa, offb, ra[0], rb[0]);
     int cbuf = 0, dbuf = S - 1;
     // After the barrier of a step: chunk c+1 is complete for everyone (each wave waited for its own copies of it), and
@@ -519,6 +563,7 @@ void dispatch_gemm_dma(zant_ctx *ctx, const float *A, const float *B, const floa
     ZANT_GEMM_CASE(KC16, KC16) ZANT_GEMM_CASE(KC16, KC4) ZANT_GEMM_CASE(KC16, RC4)
     ZANT_GEMM_CASE(KC4, KC16) ZANT_GEMM_CASE(KC4, KC4) ZANT_GEMM_CASE(KC4, RC4)
     ZANT_GEMM_CASE(RC4, KC16) ZANT_GEMM_CASE(RC4, KC4) ZANT_GEMM_CASE(RC4, RC4)
+    ZANT_GEMM_CASE(KC16, RC16) ZANT_GEMM_CASE(KC4, RC16) ZANT_GEMM_CASE(RC4, RC16)
 #undef ZANT_GEMM_CASE
 }
 
@@ -664,7 +709,7 @@ int run_gemm(zant_ctx *ctx, const float *A, const float *B, const float *C, floa
         return ZANT_OK;
     }
     const int am = a_kc ? (g.a_vec ? KC16 : KC4) : RC4;
-    const int bmode = b_kc ? (g.b_vec ? KC16 : KC4) : RC4;
+    const int bmode = b_kc ? (g.b_vec ? KC16 : KC4) : (g.b_vec ? RC16 : RC4);  // (b_vec with B stored [K][N]: N is a multiple of 4)
     if (N > 32) dispatch_gemm_dma<1, 4, 2>(ctx, A, B, C, Y, g, am, bmode);  // 128 x 64 tile, 8 waves, 5 stages
     else launch_gemm<1, 4, 1>(ctx, A, B, C, Y, g, a_kc, b_kc);              // 128 x 32 tile
     ZANT_LAUNCH_CHECK(ctx);
