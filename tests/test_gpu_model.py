@@ -271,6 +271,23 @@ def test_int8_network_fuses_activation_and_is_bit_exact(G):
     assert len(np.unique(r8)) > 4
 
 
+@pytest.mark.parametrize("H,W", [(5, 5), (7, 3), (1, 1), (6, 11)])
+def test_global_average_pool_of_a_blocked_tensor_whose_plane_is_not_a_multiple_of_eight_positions(G, H, W):
+    from zant_amd.model import Model, U8
+    g = np.random.default_rng(H * 16 + W)
+    N, C, K = 3, 16, 20
+    x = g.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+    w = g.integers(-127, 128, (K, C, 3, 3), dtype=np.int8); ws = g.uniform(0.0005, 0.001, K).astype(np.float32)
+    m = Model(G.tm.context())
+    t0 = m.input((N, C, H, W), U8, 0.02, 128)
+    t1 = m.qlinearconv(t0, w, ws, None, 0.05, 120, [1, 1], [1, 1, 1, 1])
+    t2 = m.qlinear_global_avgpool(t1, 0.04, 100)
+    m.finalize()
+    y = m.predict_host(x)
+    r1 = zo.qlinearconv(x, 0.02, 128, w, ws, None, 0.05, 120, None, [1, 1], [1, 1, 1, 1], [1, 1])
+    np.testing.assert_array_equal(y, zo.qlinear_global_avgpool(r1, 0.05, 120, 0.04, 100))
+
+
 def test_cpp_host_mirror_runs_the_reference_tests():
     """z-ant_amd/host/test_host_mirror.cpp restates the reference's operator tests against the C++ mirror of its
     interface; the binary is built by z-ant_amd/build.py (g++ over the C ABI)."""
