@@ -476,8 +476,8 @@ qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, co
                                 // across them (two lane exchanges and two byte permutes per group of four channels) leaves
                                 // lane q of the quad with channel q's four position bytes: a dword store per group where
                                 // there were four byte stores.  (Plain stores: the cache gathers the 32-byte pieces of a
-                                // line that successive position tiles write; non-temporal ones were slower, and a further transpose to
-                                // one 16-byte store per lane gained nothing.)
+                                // line that successive position tiles write; non-temporal ones were slower, and a further
+                                // transpose to one 16-byte store per lane gained nothing.)
                                 // Everything derived from the lane number is made here, per tile, behind an opaque copy:
                                 // held across the main loop it would not fit this kernel's registers.
                                 uint32_t lq = uint32_t(lane);
