@@ -1395,37 +1395,66 @@ qdw3x3_mfma_kernel(const uint4 *__restrict__ x, const uint32_t *__restrict__ wm,
     const unsigned total = unsigned(g.N) * unsigned(OHG) * unsigned(g.OW);  // < 2^31 (checked by the host)
     const unsigned n_ptiles = (total + 31u) / 32u;
     const unsigned per_img = unsigned(OHG) * unsigned(g.OW);                 // < 2^20 (checked by the host)
-    const float inv_per_img = 1.0f / float(per_img), inv_ow = 1.0f / float(g.OW);
-    const bool small_total = total < (1u << 20);
     const uint32_t pad4 = uint32_t(q.x_zp ^ 0x80) * 0x01010101u;
     const float zpf = float(q.y_zp);
     const char *xbytes = reinterpret_cast<const char *>(x);  // the whole tensor is < 4 GB (checked by the host)
     const unsigned plane = unsigned(g.H) * unsigned(g.W);
     constexpr int PR = ROWS + 2;  // input rows of the patch (ROWS = 2 implies stride 1)
-    for (unsigned pt = unsigned(blk) * 4u + unsigned(wave); pt < n_ptiles; pt += unsigned(blocks_per_pair) * 4u) {
-        const unsigned i = pt * 32u + unsigned(l32);
-        const bool valid = i < total;
-        const unsigned ii = valid ? i : total - 1u;
-        const unsigned n = small_total ? unsigned(small_div(int(ii), int(per_img), inv_per_img)) : ii / per_img;
-        const int rem = int(ii - n * per_img);
-        const int ohg = small_div(rem, g.OW, inv_ow), ow = rem - ohg * g.OW;
+    // This lane's position in the wave's next tile as (image, row group, column).  A wave's tiles lie a fixed number
+    // of positions apart, so the triple advances by that step's own triple with two carries; it is divided out once.
+    const unsigned pt_first = unsigned(blk) * 4u + unsigned(wave), pt_step = unsigned(blocks_per_pair) * 4u;
+    // The image is carried as its first 16-byte unit in the input and in the output (both tensors are < 4 GB: the host
+    // checks), so that no multiplication by the image number is left in the loop.
+    const unsigned in_img = unsigned(CB) * plane, out_img = unsigned(CB) * unsigned(g.OH) * unsigned(g.OW);
+    const unsigned in_last = unsigned(g.N - 1) * in_img, out_last = unsigned(g.N - 1) * out_img;
+    unsigned w_in, w_out;  // (past the batch for lanes past the end of the last tile: clamped where they are used)
+    int wohg, wow;
+    {
+        const unsigned i = pt_first * 32u + unsigned(l32);
+        const unsigned wn = i / per_img;
+        const unsigned rem = i - wn * per_img;
+        wohg = int(rem / unsigned(g.OW));
+        wow = int(rem - unsigned(wohg) * unsigned(g.OW));
+        w_in = wn * in_img;
+        w_out = wn * out_img;
+    }
+    const unsigned step = pt_step * 32u;
+    const unsigned d_n = step / per_img, step_r = step - d_n * per_img;
+    const int d_ohg = int(step_r / unsigned(g.OW)), d_ow = int(step_r - unsigned(d_ohg) * unsigned(g.OW));
+    const unsigned d_in = d_n * in_img, d_out = d_n * out_img;
+    const unsigned cb_in = unsigned(cb_ok ? cb : 0) * plane;                      // this lane's channel block inside an image
+    const unsigned out_plane = unsigned(g.OH) * unsigned(g.OW);
+    for (unsigned pt = pt_first; pt < n_ptiles; pt += pt_step) {
+        const bool valid = w_in <= in_last;  // (only the last tile has lanes past the end: they compute image N - 1 again)
+        const unsigned n_in = min(w_in, in_last), n_out = min(w_out, out_last);
+        const int ohg = wohg, ow = wow;
+        {
+            wow += d_ow;
+            const int c1 = wow >= g.OW ? 1 : 0;
+            wow -= c1 ? g.OW : 0;
+            wohg += d_ohg + c1;
+            const bool c2 = wohg >= OHG;
+            wohg -= c2 ? OHG : 0;
+            w_in += d_in + (c2 ? in_img : 0u);
+            w_out += d_out + (c2 ? out_img : 0u);
+        }
         const int oh = ohg * ROWS;
         // Every tap is loaded from an address inside the tensor (a tap outside the image reads its clamped neighbour)
         // and replaced by the padding vector afterwards: no divergent control flow around the loads.
         const int ih0 = oh * g.sh - g.pt, iw0 = ow * g.sw - g.pl;  // top-left tap
-        const unsigned base = (n * unsigned(CB) + unsigned(cb_ok ? cb : 0)) * plane * 16u;
+        const unsigned base = (n_in + cb_in) * 16u;
         bool rv[PR], cvd[3];
         unsigned rowb[PR], colb[3];
 #pragma unroll
         for (int k = 0; k < PR; ++k) {
             const int ih = ih0 + k;
-            rv[k] = cb_ok && ih >= 0 && ih < g.H;
-            rowb[k] = base + unsigned(min(max(ih, 0), g.H - 1)) * unsigned(g.W) * 16u;
+            rv[k] = cb_ok && unsigned(ih) < unsigned(g.H);
+            rowb[k] = base + __umul24(unsigned(min(max(ih, 0), g.H - 1)), unsigned(g.W) * 16u);  // H, W * 16 < 2^24 (host)
         }
 #pragma unroll
         for (int k = 0; k < 3; ++k) {
             const int iw = iw0 + k;
-            cvd[k] = iw >= 0 && iw < g.W;
+            cvd[k] = unsigned(iw) < unsigned(g.W);
             colb[k] = unsigned(min(max(iw, 0), g.W - 1)) * 16u;
         }
         uint4 xv[PR * 3];
@@ -1476,17 +1505,15 @@ qdw3x3_mfma_kernel(const uint4 *__restrict__ x, const uint32_t *__restrict__ wm,
                 }
             }
             // lanes p and p + 32 exchange one dword per channel block so that each stores 8 consecutive bytes
+            // (the half-wave swap: the lower lane ends up with dword 2b of both lanes, the upper lane with dword 2b + 1)
             const bool row_ok = valid && oh + r < g.OH;
+            const unsigned pos = n_out + __umul24(unsigned(oh + r), unsigned(g.OW)) + unsigned(ow);  // unit inside channel block 0
 #pragma unroll
             for (int b = 0; b < 2; ++b) {
-                const uint32_t send = lh ? d[2 * b] : d[2 * b + 1];
-                const uint32_t recv = uint32_t(__shfl_xor(int(send), 32, 64));
-                const uint2 out = lh ? make_uint2(recv, d[2 * b + 1]) : make_uint2(d[2 * b], recv);
+                const auto sw = __builtin_amdgcn_permlane32_swap(d[2 * b], d[2 * b + 1], false, false);
                 const int cbo = 2 * pair + b;
-                if (row_ok && cbo < CB) {
-                    uint8_t *yp = y + (((int64_t(n) * CB + cbo) * g.OH + oh + r) * int64_t(g.OW) + ow) * 16 + lh * 8;
-                    *reinterpret_cast<uint2 *>(yp) = out;
-                }
+                if (row_ok && cbo < CB)
+                    *reinterpret_cast<uint2 *>(y + ((pos + unsigned(cbo) * out_plane) * 16u + unsigned(lh) * 8u)) = make_uint2(sw[0], sw[1]);
             }
         }
     }
@@ -1518,7 +1545,8 @@ int run_qdw_blocked(zant_ctx *ctx, const uint8_t *xb, const int8_t *w, const flo
     const int64_t per_cb = int64_t(g.N) * g.OH * g.OW;
     KernelTimer kt(ctx);
     if (per_cb < (int64_t(1) << 31) - 64 && int64_t(g.OH) * g.OW < (1 << 20) &&
-        int64_t(g.N) * CB * g.H * g.W * 16 < (int64_t(1) << 32)) {
+        int64_t(g.N) * CB * g.H * g.W * 16 < (int64_t(1) << 32) && int64_t(g.N) * CB * g.OH * g.OW * 16 < (int64_t(1) << 32) &&
+        g.H < (1 << 24) && g.W < (1 << 20) && g.OH < (1 << 24) && g.OW < (1 << 24)) {
         ZANT_KERNEL_NAME(ctx, "qdw3x3_mfma_kernel<%d>", (g.sh == 1 && g.sw == 1 && g.OH >= 2) ? 2 : 1);
         // one resident generation of workgroups (three share a CU at this kernel's register count): a workgroup's
         // set-up -- the activation table, the nine diagonal operands, the tables -- is paid once per wave slot
