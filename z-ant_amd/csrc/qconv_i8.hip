@@ -1051,26 +1051,34 @@ qfirst_mfma_kernel(const uint8_t *__restrict__ x, const uint4 *__restrict__ wpk,
     // This lane's position in the next tile to load, as (image, row, column) of the (pooled) output.  Successive tiles
     // of a wavefront lie n_waves * 32 positions apart: the triple advances by that step's own (images, rows, columns)
     // with two carries, and is divided out only once.
-    unsigned wn;
+    // The image is carried as the offset of its first byte in the input and of its first element (blocked: 16-byte
+    // unit) in the output, so that no multiplication by the image number is left in the loop (both tensors are below
+    // 2^32 bytes: the host checks).
+    const unsigned out_img = (y_blocked ? unsigned(KB16) : unsigned(g.K)) * per_img;
+    const unsigned in_last = unsigned(g.N - 1) * img_in, out_last = unsigned(g.N - 1) * out_img;
+    unsigned w_in, w_out;  // (past the batch for lanes past the end of the last tile: clamped where they are used)
     int woho, wowo;
     {
         const unsigned i = wave_id * 32u + unsigned(l32);
-        wn = i / per_img;
+        const unsigned wn = i / per_img;
         const unsigned rem = i - wn * per_img;
         woho = int(rem / unsigned(OWo));
         wowo = int(rem - unsigned(woho) * unsigned(OWo));
+        w_in = wn * img_in;
+        w_out = wn * out_img;
     }
     const unsigned step = n_waves * 32u;
     const unsigned d_n = step / per_img, step_r = step - d_n * per_img;
     const int d_oho = int(step_r / unsigned(OWo)), d_owo = int(step_r - unsigned(d_oho) * unsigned(OWo));
+    const unsigned d_in = d_n * img_in, d_out = d_n * out_img;
     // The row loads of the NEXT tile are issued before this tile's arithmetic: with two wavefronts per SIMD the load
     // latency would otherwise sit on the critical path of every tile.
-    struct TileMeta { unsigned n; int oho, owo, ih0, sh; bool valid; };
+    struct TileMeta { unsigned out0; int oho, owo, ih0, sh; bool valid; };  // out0: the image's first output element
     uint32_t raw[C][PR];
     TileMeta nxt;
     auto issue = [&](TileMeta &m) {
-        m.valid = wn < unsigned(g.N);           // (only the last tile has lanes past the end: they read image N - 1)
-        m.n = min(wn, unsigned(g.N) - 1u);
+        m.valid = w_in <= in_last;              // (only the last tile has lanes past the end: they read image N - 1)
+        m.out0 = min(w_out, out_last);
         m.oho = woho;
         m.owo = wowo;
         m.ih0 = (POOL ? 2 * woho : woho) * S - g.pt;
@@ -1078,7 +1086,7 @@ qfirst_mfma_kernel(const uint8_t *__restrict__ x, const uint4 *__restrict__ wpk,
         // one dword per (channel, patch row): columns iw0 .. iw0+3, read from a start clamped into the row
         const int iw0c = min(max(iw0, 0), g.W - 4);
         m.sh = iw0 - iw0c;
-        const unsigned base = m.n * img_in + unsigned(iw0c);
+        const unsigned base = min(w_in, in_last) + unsigned(iw0c);
         unsigned rowoff[PR];
 #pragma unroll
         for (int r = 0; r < PR; ++r) rowoff[r] = __umul24(unsigned(min(max(m.ih0 + r, 0), g.H - 1)), unsigned(g.W));  // H, W < 2^24 (host)
@@ -1091,14 +1099,15 @@ qfirst_mfma_kernel(const uint8_t *__restrict__ x, const uint4 *__restrict__ wpk,
         const int c1 = wowo >= OWo ? 1 : 0;
         wowo -= c1 ? OWo : 0;
         woho += d_oho + c1;
-        const int c2 = woho >= OHo ? 1 : 0;
+        const bool c2 = woho >= OHo;
         woho -= c2 ? OHo : 0;
-        wn += d_n + unsigned(c2);
+        w_in += d_in + (c2 ? img_in : 0u);
+        w_out += d_out + (c2 ? out_img : 0u);
     };
     if (wave_id < n_ptiles) issue(nxt);
     for (unsigned pt = wave_id; pt < n_ptiles; pt += n_waves) {
         const TileMeta cur = nxt;
-        const unsigned n = cur.n;
+        const unsigned out0 = cur.out0;
         const int oho = cur.oho, owo = cur.owo, ih0 = cur.ih0, sh = cur.sh;
         const bool valid = cur.valid;
         // Shifted into place with one byte permute per dword: selector byte b picks data byte b + sh (4 + b + sh in the
@@ -1185,14 +1194,16 @@ qfirst_mfma_kernel(const uint8_t *__restrict__ x, const uint4 *__restrict__ wpk,
                 out[0] = int(s0[0]); out[1] = int(s0[1]); out[2] = int(s1[0]); out[3] = int(s1[1]);
                 const int cbq = kb * 2 + lh;
                 if (valid && cbq < KB16) {
-                    const unsigned off = ((n * unsigned(KB16) + unsigned(cbq)) * unsigned(OHo) + unsigned(oho)) * unsigned(OWo) + unsigned(owo);
+                    const unsigned off = out0 + unsigned(cbq) * per_img + __umul24(unsigned(oho), unsigned(OWo)) + unsigned(owo);
                     *reinterpret_cast<i32x4 *>(y + size_t(off) * 16) = out;
                 }
             } else if (valid) {
+                // channel kch of the position; the lane's other channels are whole planes further on
+                const unsigned pos = out0 + __umul24(unsigned(oho), unsigned(OWo)) + unsigned(owo) + unsigned(kch) * per_img;
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
-                    const int k = kch + (v >> 2) * 8 + (v & 3);
-                    if (k < g.K) y[((int64_t(n) * g.K + k) * OHo + oho) * int64_t(OWo) + owo] = uint8_t(d[v >> 2] >> (8 * (v & 3)));
+                    const int dk = (v >> 2) * 8 + (v & 3);
+                    if (kch + dk < g.K) y[pos + unsigned(dk) * per_img] = uint8_t(d[v >> 2] >> (8 * (v & 3)));
                 }
             }
         }
@@ -1208,6 +1219,8 @@ bool qfirst_eligible(const ConvGeom &g, bool pool) {
     const int64_t OHo = pool ? g.OH / 2 : g.OH, OWo = pool ? g.OW / 2 : g.OW;
     // input offsets are formed in 32 bits, row offsets with a 24-bit multiply
     if (int64_t(g.N) * g.C * g.H * g.W >= (int64_t(1) << 32) - 64 || g.H >= (1 << 24) || g.W >= (1 << 24)) return false;
+    // ... and so are output offsets (NCHW: bytes; blocked: 16-byte units of 16-channel blocks)
+    if (int64_t(g.N) * (int64_t(g.K + 15) / 16 * 16) * g.OH * g.OW >= (int64_t(1) << 32)) return false;
     return OHo >= 1 && OWo >= 1 && int64_t(g.N) * OHo * OWo < (int64_t(1) << 31) - 64 && OHo * OWo < (1 << 20);
 }
 
