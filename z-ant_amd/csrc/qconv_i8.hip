@@ -1056,11 +1056,13 @@ qfirst_mfma_kernel(const uint8_t *__restrict__ x, const uint4 *__restrict__ wpk,
     // 2^32 bytes: the host checks).
     const unsigned out_img = (y_blocked ? unsigned(KB16) : unsigned(g.K)) * per_img;
     const unsigned in_last = unsigned(g.N - 1) * img_in, out_last = unsigned(g.N - 1) * out_img;
-    unsigned w_in, w_out;  // (past the batch for lanes past the end of the last tile: clamped where they are used)
+    // (lanes past the end of the last tile are told by the image count itself -- the offsets may wrap there -- and take
+    // the last image's)
+    unsigned wn, w_in, w_out;
     int woho, wowo;
     {
         const unsigned i = wave_id * 32u + unsigned(l32);
-        const unsigned wn = i / per_img;
+        wn = i / per_img;
         const unsigned rem = i - wn * per_img;
         woho = int(rem / unsigned(OWo));
         wowo = int(rem - unsigned(woho) * unsigned(OWo));
@@ -1077,8 +1079,8 @@ qfirst_mfma_kernel(const uint8_t *__restrict__ x, const uint4 *__restrict__ wpk,
     uint32_t raw[C][PR];
     TileMeta nxt;
     auto issue = [&](TileMeta &m) {
-        m.valid = w_in <= in_last;              // (only the last tile has lanes past the end: they read image N - 1)
-        m.out0 = min(w_out, out_last);
+        m.valid = wn < unsigned(g.N);           // (only the last tile has lanes past the end: they read image N - 1)
+        m.out0 = m.valid ? w_out : out_last;
         m.oho = woho;
         m.owo = wowo;
         m.ih0 = (POOL ? 2 * woho : woho) * S - g.pt;
@@ -1086,7 +1088,7 @@ qfirst_mfma_kernel(const uint8_t *__restrict__ x, const uint4 *__restrict__ wpk,
         // one dword per (channel, patch row): columns iw0 .. iw0+3, read from a start clamped into the row
         const int iw0c = min(max(iw0, 0), g.W - 4);
         m.sh = iw0 - iw0c;
-        const unsigned base = min(w_in, in_last) + unsigned(iw0c);
+        const unsigned base = (m.valid ? w_in : in_last) + unsigned(iw0c);
         unsigned rowoff[PR];
 #pragma unroll
         for (int r = 0; r < PR; ++r) rowoff[r] = __umul24(unsigned(min(max(m.ih0 + r, 0), g.H - 1)), unsigned(g.W));  // H, W < 2^24 (host)
@@ -1101,6 +1103,7 @@ qfirst_mfma_kernel(const uint8_t *__restrict__ x, const uint4 *__restrict__ wpk,
         woho += d_oho + c1;
         const bool c2 = woho >= OHo;
         woho -= c2 ? OHo : 0;
+        wn += d_n + (c2 ? 1u : 0u);
         w_in += d_in + (c2 ? img_in : 0u);
         w_out += d_out + (c2 ? out_img : 0u);
     };
@@ -1420,11 +1423,13 @@ qdw3x3_mfma_kernel(const uint4 *__restrict__ x, const uint32_t *__restrict__ wm,
     // checks), so that no multiplication by the image number is left in the loop.
     const unsigned in_img = unsigned(CB) * plane, out_img = unsigned(CB) * unsigned(g.OH) * unsigned(g.OW);
     const unsigned in_last = unsigned(g.N - 1) * in_img, out_last = unsigned(g.N - 1) * out_img;
-    unsigned w_in, w_out;  // (past the batch for lanes past the end of the last tile: clamped where they are used)
+    // (lanes past the end of the last tile are told by the image count itself -- the offsets may wrap there -- and take
+    // the last image's)
+    unsigned wn, w_in, w_out;
     int wohg, wow;
     {
         const unsigned i = pt_first * 32u + unsigned(l32);
-        const unsigned wn = i / per_img;
+        wn = i / per_img;
         const unsigned rem = i - wn * per_img;
         wohg = int(rem / unsigned(g.OW));
         wow = int(rem - unsigned(wohg) * unsigned(g.OW));
@@ -1438,8 +1443,8 @@ qdw3x3_mfma_kernel(const uint4 *__restrict__ x, const uint32_t *__restrict__ wm,
     const unsigned cb_in = unsigned(cb_ok ? cb : 0) * plane;                      // this lane's channel block inside an image
     const unsigned out_plane = unsigned(g.OH) * unsigned(g.OW);
     for (unsigned pt = pt_first; pt < n_ptiles; pt += pt_step) {
-        const bool valid = w_in <= in_last;  // (only the last tile has lanes past the end: they compute image N - 1 again)
-        const unsigned n_in = min(w_in, in_last), n_out = min(w_out, out_last);
+        const bool valid = wn < unsigned(g.N);  // (only the last tile has lanes past the end: they compute image N - 1 again)
+        const unsigned n_in = valid ? w_in : in_last, n_out = valid ? w_out : out_last;
         const int ohg = wohg, ow = wow;
         {
             wow += d_ow;
@@ -1448,6 +1453,7 @@ qdw3x3_mfma_kernel(const uint4 *__restrict__ x, const uint32_t *__restrict__ wm,
             wohg += d_ohg + c1;
             const bool c2 = wohg >= OHG;
             wohg -= c2 ? OHG : 0;
+            wn += d_n + (c2 ? 1u : 0u);
             w_in += d_in + (c2 ? in_img : 0u);
             w_out += d_out + (c2 ? out_img : 0u);
         }
