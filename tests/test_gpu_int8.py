@@ -45,6 +45,10 @@ QCASES = [
     (2, 50, 8, 12, 40, 3, 3, [1, 1], [1, 1, 1, 1], [1, 1], 1),
     (3, 45, 6, 6, 35, 3, 3, [1, 1], [0, 0, 0, 0], [1, 1], 1),
     (70, 77, 2, 2, 40, 1, 1, [1, 1], [0, 0, 0, 0], [1, 1], 1),      # pointwise layer on 2 x 2 planes: one quad per plane
+    # two outputs per image and a last position tile that is mostly past the end of the batch (the lanes there would be
+    # images 37 .. 47): first-layer kernel, depthwise kernel
+    (37, 3, 3, 4, 16, 3, 3, [1, 1], [0, 0, 0, 0], [1, 1], 1),
+    (37, 16, 3, 4, 16, 3, 3, [1, 1], [0, 0, 0, 0], [1, 1], 16),
 ]
 
 
