@@ -142,7 +142,9 @@ constexpr int PS_WUMAX = 5;            // weight units per thread and step: ceil
 // The matrix-core work of one step: 9 taps x 32 input channels for this wave's MT position tiles x 2 channel blocks.
 // wr: LDS address of this lane's weight operand of tap 0 of the wave's first channel block (the second block 512 bytes
 // on, taps 4 KB apart); xbase[i] + chunk_off: LDS address of position slot i's patch entry for tap (0, 0) in this step's
-// channel chunk and this lane's half; PW16: bytes of a patch row.
+// channel chunk and this lane's half; PW16: bytes of a patch row.  last_slot: position slot MT - 1 holds a tile of
+// the wave's group (tiles are dealt evenly, so a wave is normally at most one short; slots below the last are always
+// multiplied: an empty one reads a valid address and its sums are dropped).
 // The activation operand of slot i for the NEXT tap is read into the same registers right behind slot i's two MFMAs of
 // this tap: a rolling pipeline one tap deep in which every read has 2 * MT MFMAs to land and each MFMA pair waits only
 // for its own operand.  Filter columns are immediate offsets, filter rows an address increment.
@@ -152,7 +154,7 @@ constexpr int PS_WUMAX = 5;            // weight units per thread and step: ceil
 template <int MT, bool FIRST>
 __device__ __forceinline__ void ps_mfma_step(unsigned wr, const unsigned (&xbase)[MT], unsigned chunk_off, unsigned PW16, const PsStream &st,
                                              const PsDesc &d, const int8_t *__restrict__ xb, const int8_t *__restrict__ padvec,
-                                             const PsGeom &p, i32x16 (&acc)[2][MT]) {
+                                             const PsGeom &p, i32x16 (&acc)[2][MT], bool last_slot) {
     i32x4 a[2][2], b[MT];  // a[buffer][channel block]
     u32x4 stg[3][2];       // units on their way from global memory to LDS, by tap modulo 3
     unsigned xr[MT];
@@ -194,6 +196,8 @@ __device__ __forceinline__ void ps_mfma_step(unsigned wr, const unsigned (&xbase
             if (i == 0) ps_operands_ready(a[cur][0], a[cur][1], b[i], pending);
             else ps_operand_ready(b[i], pending);
             __builtin_amdgcn_s_setprio(1);
+            // (a wave whose last position slot holds no tile of its group skips that slot's MFMAs: wave-uniform)
+            if (i < MT - 1 || last_slot)
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 if (FIRST && t == 0) {
@@ -335,6 +339,7 @@ qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, co
     __builtin_amdgcn_sched_barrier(0);
 
     i32x16 acc[2][MT];
+    const bool last_slot = mt == MT;  // wave-uniform: the wave's last position slot holds a tile of its group
     int gs = 0;  // steps done by this workgroup; its parity selects the ring slab a step reads
     while (true) {
         const int next_tile = tile + int(gridDim.x);
@@ -366,14 +371,14 @@ qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, co
                 boundary();
                 plan_copies(0);
                 // slots past this wave's tiles multiply patch entry 0; their results are dropped
-                ps_mfma_step<MT, true>(wr0 + unsigned((gs & 1) * PS_RING), xbase, 0u, PW16, st, desc, xb, padvec, p, acc);
+                ps_mfma_step<MT, true>(wr0 + unsigned((gs & 1) * PS_RING), xbase, 0u, PW16, st, desc, xb, padvec, p, acc, last_slot);
                 ++s; ++gs;
             }
             for (int c = 1; c < p.NC; ++c, ++s, ++gs) {
                 boundary();
                 plan_copies(c);
                 ps_mfma_step<MT, false>(wr0 + unsigned((gs & 1) * PS_RING), xbase, unsigned(2 * c * p.P1s * 16), PW16, st, desc,
-                                        xb, padvec, p, acc);
+                                        xb, padvec, p, acc, last_slot);
             }
 
             // ---- end of pass kp: requantisation (+ fused activation), stores ----
@@ -430,6 +435,7 @@ qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, co
 #pragma unroll
                     for (int i = 0; i < MT; ++i) {
                         __builtin_amdgcn_sched_barrier(0);  // one position tile at a time
+                        if (i == MT - 1 && !last_slot) continue;  // no tile in the wave's last slot (wave-uniform)
                         const int pos = int(praw[i]);
                         const int img = pos >> 20, r = (pos >> 10) & 1023, cc = pos & 1023;
                         const bool ok = pos >= 0 && img < imgs_here && r < rows_here;
