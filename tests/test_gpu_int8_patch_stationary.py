@@ -81,3 +81,30 @@ def test_blocked_in_and_out_inside_a_model(G):
         m.finalize()
         y = m.predict_host(x)
         np.testing.assert_array_equal(y, ref)
+
+
+# NCHW output whose plane runs are made of aligned 4- or 8-byte units is staged through LDS and written out as whole
+# runs: a staging region of its own, or -- one tile per workgroup, one pass -- the one laid over the dead ring and patch.
+STAGED_CASES = [
+    # N, C, H, W, K, pads
+    (4, 32, 8, 8, 64, [1, 1, 1, 1]),         # 8-byte units, a staging region of its own
+    (300, 32, 8, 8, 64, [1, 1, 1, 1]),       # the same with several tiles per workgroup: staging rows are rewritten
+    (2, 64, 12, 12, 200, [1, 1, 1, 1]),      # two output-channel passes, ragged channels
+    (3, 32, 9, 12, 40, [1, 1, 1, 1]),        # planes of 108 bytes: 4-byte units
+    (2, 128, 28, 28, 128, [1, 1, 1, 1]),     # too large for a region of its own: laid over ring, slot table and patch
+    (5, 48, 14, 28, 96, [1, 1, 1, 1]),       # row tiles that do not divide the rows (short last tile), whole-unit rows
+]
+
+
+@pytest.mark.parametrize("case", STAGED_CASES, ids=[str(i) for i in range(len(STAGED_CASES))])
+@pytest.mark.parametrize("act", [None, "relu6"])
+def test_staged_nchw_write_out_bit_exact(G, case, act):
+    N, C, H, W, K, pads = case
+    x, w, ws, b = _operands(7 * N + C + K, N, C, H, W, K)
+    kw = dict(act=act, act_alpha=0.0, act_scale=0.03, act_zp=0) if act else {}
+    y = G.tm.qlinearconv(G.dev(x), 0.02, 128, G.dev(w), G.dev(ws), None, 0.05, 128, G.dev(b), [1, 1], pads, [1, 1], 1, **kw)
+    assert G.tm.context().kernel_name().startswith("qconv_ps_kernel<"), G.tm.context().kernel_name()
+    assert G.tm.context().kernel_name().rstrip(">").split(",")[1] in ("4", "5"), "the staged write-out did not run"
+    pick = list(range(N)) if N <= 8 else [0, 1, N // 2, N - 2, N - 1]
+    ref = zo.qlinearconv(x[pick], 0.02, 128, w, ws, None, 0.05, 128, b, [1, 1], pads, [1, 1], 1, **kw)
+    np.testing.assert_array_equal(G.host(y)[pick], ref)

@@ -46,6 +46,12 @@ struct PsGeom {
     int npt;                    // position tiles of 32 per tile
     int kpad;                   // NKP * KP
     int tab_rounds;             // copy rounds of the multiplier and correction tables: ceil(kpad / 2 / PS_NT)
+    // NCHW output staged through LDS (PS_OUT_NCHW_ST*): the tile's bytes as [channel of the pass][S_pad] rows, then
+    // written out as whole runs of a plane.
+    int S_pad;                  // bytes of a staging row: a tile's position tiles x 32, rounded up to 8 x an odd number
+    int stage_off;              // staging region, in bytes from the weight ring's start
+    int stage_alias;            // it lies over the ring, the slot table and the patch (one tile per workgroup, one pass)
+    int out_unit;               // bytes per copy of the write-out: 8 or 4
 };
 
 __device__ __forceinline__ unsigned ps_lds_addr(const void *p) {
@@ -151,7 +157,9 @@ constexpr int PS_WUMAX = 5;            // weight units per thread and step: ceil
 // The copies of PsStream ride along: two units loaded behind the first MFMA pair of each of taps 0..4 and written to
 // LDS two taps later.
 // FIRST: the step opens a pass: its first tap starts the accumulators from zero (an inline constant of the MFMA).
-template <int MT, bool FIRST>
+// SWAP: positions are the MFMA's rows and channels its columns (a lane then holds 16 positions of ONE channel) instead of
+// the other way round (16 channels of one position).
+template <int MT, bool FIRST, bool SWAP>
 __device__ __forceinline__ void ps_mfma_step(unsigned wr, const unsigned (&xbase)[MT], unsigned chunk_off, unsigned PW16, const PsStream &st,
                                              const PsDesc &d, const int8_t *__restrict__ xb, const int8_t *__restrict__ padvec,
                                              const PsGeom &p, i32x16 (&acc)[2][MT], bool last_slot) {
@@ -202,9 +210,11 @@ __device__ __forceinline__ void ps_mfma_step(unsigned wr, const unsigned (&xbase
             for (int j = 0; j < 2; ++j) {
                 if (FIRST && t == 0) {
                     const i32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                    acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[cur][j], b[i], zero, 0, 0, 0);
+                    acc[j][i] = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(b[i], a[cur][j], zero, 0, 0, 0)
+                                     : __builtin_amdgcn_mfma_i32_32x32x32_i8(a[cur][j], b[i], zero, 0, 0, 0);
                 } else {
-                    acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[cur][j], b[i], acc[j][i], 0, 0, 0);
+                    acc[j][i] = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(b[i], a[cur][j], acc[j][i], 0, 0, 0)
+                                     : __builtin_amdgcn_mfma_i32_32x32x32_i8(a[cur][j], b[i], acc[j][i], 0, 0, 0);
                 }
             }
             __builtin_amdgcn_s_setprio(0);
@@ -231,14 +241,37 @@ __device__ __forceinline__ void ps_mfma_step(unsigned wr, const unsigned (&xbase
 }
 
 // OUT: how the output bytes are formed and stored.
-enum { PS_OUT_NCHW_LUT = 0, PS_OUT_BLOCKED_LUT = 1, PS_OUT_BLOCKED = 2, PS_OUT_NCHW = 3 };
+enum { PS_OUT_NCHW_LUT = 0, PS_OUT_BLOCKED_LUT = 1, PS_OUT_BLOCKED = 2, PS_OUT_NCHW = 3, PS_OUT_NCHW_ST = 4, PS_OUT_NCHW_ST_LUT = 5 };
+
+// Write-out of a staged NCHW tile: rows of the staging region (one per image and channel, `row_bytes` real bytes each)
+// go to their runs of the output planes in units of U bytes, consecutive threads on consecutive units.
+template <typename U>
+__device__ __forceinline__ void ps_write_out(const char *stage, uint8_t *__restrict__ y, const PsGeom &p, int kh, int imgs_here,
+                                             int row_bytes, unsigned g_origin, int plane) {
+    const int upr = row_bytes / int(sizeof(U)), n_rows = imgs_here * kh, n_units = n_rows * upr;
+    const float inv_upr = 1.0f / float(upr), inv_kh = 1.0f / float(kh);
+    const int per_img = p.TH * p.OW;
+#pragma unroll 4
+    for (int u = int(threadIdx.x); u < n_units; u += PS_NT) {
+        const int row = small_div(u, upr, inv_upr), off = u - row * upr;
+        int img = 0, kk = row;
+        if (p.NB > 1) {
+            img = small_div(row, kh, inv_kh);
+            kk = row - img * kh;
+        }
+        const U v = *reinterpret_cast<const U *>(stage + kk * p.S_pad + img * per_img + off * int(sizeof(U)));
+        *reinterpret_cast<U *>(y + (g_origin + unsigned(img * p.K + kk) * unsigned(plane) + unsigned(off * int(sizeof(U))))) = v;
+    }
+}
 
 // tabs: the per-channel requantisation multipliers (kpad floats) followed by the integer corrections (kpad ints).
 template <int MT, int OUT>
 __global__ void __launch_bounds__(PS_NT)
 qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, const char *__restrict__ tabs,
                 const int8_t *__restrict__ padvec, uint8_t *__restrict__ y, PsGeom p, QConvArgs q) {
-    constexpr bool y_blocked = OUT == PS_OUT_BLOCKED_LUT || OUT == PS_OUT_BLOCKED, use_lut = OUT == PS_OUT_BLOCKED_LUT || OUT == PS_OUT_NCHW_LUT;
+    constexpr bool y_blocked = OUT == PS_OUT_BLOCKED_LUT || OUT == PS_OUT_BLOCKED;
+    constexpr bool use_lut = OUT == PS_OUT_BLOCKED_LUT || OUT == PS_OUT_NCHW_LUT || OUT == PS_OUT_NCHW_ST_LUT;
+    constexpr bool staged = OUT == PS_OUT_NCHW_ST || OUT == PS_OUT_NCHW_ST_LUT;
     extern __shared__ __attribute__((aligned(256))) char ps_lds_raw[];
     // LDS: [256-byte activation table, 256-aligned][multipliers, corrections][weight ring: 2 slabs][slot table]
     //      [patch: 2*NC blocks x P1s x 16]
@@ -371,13 +404,13 @@ qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, co
                 boundary();
                 plan_copies(0);
                 // slots past this wave's tiles multiply patch entry 0; their results are dropped
-                ps_mfma_step<MT, true>(wr0 + unsigned((gs & 1) * PS_RING), xbase, 0u, PW16, st, desc, xb, padvec, p, acc, last_slot);
+                ps_mfma_step<MT, true, staged>(wr0 + unsigned((gs & 1) * PS_RING), xbase, 0u, PW16, st, desc, xb, padvec, p, acc, last_slot);
                 ++s; ++gs;
             }
             for (int c = 1; c < p.NC; ++c, ++s, ++gs) {
                 boundary();
                 plan_copies(c);
-                ps_mfma_step<MT, false>(wr0 + unsigned((gs & 1) * PS_RING), xbase, unsigned(2 * c * p.P1s * 16), PW16, st, desc,
+                ps_mfma_step<MT, false, staged>(wr0 + unsigned((gs & 1) * PS_RING), xbase, unsigned(2 * c * p.P1s * 16), PW16, st, desc,
                                         xb, padvec, p, acc, last_slot);
             }
 
@@ -396,7 +429,67 @@ qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, co
                     }
                 __builtin_amdgcn_sched_barrier(0);
             }
-            {
+            if constexpr (staged) {
+                // A lane holds 16 positions of ONE channel per accumulator tuple (registers 4g..4g+3: four consecutive
+                // positions of the tile's flattened (image, row, column) order): one multiplier and one correction per
+                // lane, a dword of four positions per group with no exchange between lanes.  The dwords go to the
+                // staging rows [channel][position]; the workgroup then writes each row's bytes to its plane as one run.
+                const int ig = tile / p.n_row_tiles;
+                const int n0 = ig * p.NB, oh0 = (tile - ig * p.n_row_tiles) * p.TH;
+                const int rows_here = min(p.TH, p.OH - oh0), imgs_here = min(p.NB, p.N - n0);
+                const int plane = p.OH * p.OW;
+                const float zpf = float(q.y_zp);
+                char *stage = wring + p.stage_off;
+                if (p.stage_alias) {  // everybody has left the matrix-core loop: ring, slot table and patch are free
+                    __builtin_amdgcn_s_waitcnt(0xC07F);
+                    __builtin_amdgcn_s_barrier();
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int kk = (2 * cp + j) * 32 + l32;  // this lane's channel inside the pass
+                    uint32_t mr = ps_read_b32(mult_a + unsigned(kp * p.KP + kk) * 4u), cr = ps_read_b32(corr_a + unsigned(kp * p.KP + kk) * 4u);
+                    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(mr), "+v"(cr));
+                    const float mv = __uint_as_float(mr);
+                    const int cv = int(cr);
+                    char *row = stage + kk * p.S_pad + (pt0 * 32 + lh * 4);
+#pragma unroll
+                    for (int i = 0; i < MT; ++i) {
+                        __builtin_amdgcn_sched_barrier(0);  // one position tile at a time
+                        if (i >= mt) continue;              // (wave-uniform) an empty slot's positions belong to another wave
+#pragma unroll
+                        for (int gq = 0; gq < 4; ++gq) {
+                            uint32_t w4 = 0;
+                            if constexpr (use_lut) {
+                                uint32_t ob[4];
+#pragma unroll
+                                for (int e = 0; e < 4; ++e)
+                                    ob[e] = ps_read_u8(__builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(float(acc[j][i][gq * 4 + e] + cv) * mv) + zpf, 0u, lut_a));
+                                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(ob[0]), "+v"(ob[1]), "+v"(ob[2]), "+v"(ob[3]));
+                                w4 = ob[0] | (ob[1] << 8) | (ob[2] << 16) | (ob[3] << 24);
+                            } else {
+#pragma unroll
+                                for (int e = 0; e < 4; ++e)
+                                    w4 = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(float(acc[j][i][gq * 4 + e] + cv) * mv) + zpf, unsigned(e), w4);
+                            }
+                            *reinterpret_cast<uint32_t *>(row + i * 32 + gq * 8) = w4;
+                        }
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                __builtin_amdgcn_s_waitcnt(0xC07F);
+                __builtin_amdgcn_s_barrier();
+                __builtin_amdgcn_sched_barrier(0);
+                const int kh = min(p.KP, p.K - kp * p.KP);
+                const unsigned g_origin = unsigned((n0 * p.K + kp * p.KP) * plane + oh0 * p.OW);
+                if (p.out_unit == 8) ps_write_out<uint2>(stage, y, p, kh, imgs_here, rows_here * p.OW, g_origin, plane);
+                else ps_write_out<uint32_t>(stage, y, p, kh, imgs_here, rows_here * p.OW, g_origin, plane);
+                if (!p.stage_alias) {  // the next pass or tile writes these rows again: not before everybody has read them
+                    __builtin_amdgcn_s_waitcnt(0xC07F);
+                    __builtin_amdgcn_s_barrier();
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
                 const int ig = tile / p.n_row_tiles;
                 const int n0 = ig * p.NB, oh0 = (tile - ig * p.n_row_tiles) * p.TH;
                 const int rows_here = min(p.TH, p.OH - oh0), imgs_here = min(p.NB, p.N - n0);
@@ -670,7 +763,9 @@ void ps_launch_out(zant_ctx *ctx, int grid, size_t lds, const int8_t *xb, const 
 template <int MT>
 void ps_launch(zant_ctx *ctx, int grid, size_t lds, const int8_t *xb, const int8_t *wp, const char *tabs,
                const int8_t *padvec, uint8_t *y, const PsGeom &p, const QConvArgs &q, int yb) {
-    if (!yb && q.has_act) ps_launch_out<MT, PS_OUT_NCHW_LUT>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
+    if (!yb && p.out_unit && q.has_act) ps_launch_out<MT, PS_OUT_NCHW_ST_LUT>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
+    else if (!yb && p.out_unit) ps_launch_out<MT, PS_OUT_NCHW_ST>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
+    else if (!yb && q.has_act) ps_launch_out<MT, PS_OUT_NCHW_LUT>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
     else if (!yb) ps_launch_out<MT, PS_OUT_NCHW>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
     else if (q.has_act) ps_launch_out<MT, PS_OUT_BLOCKED_LUT>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
     else ps_launch_out<MT, PS_OUT_BLOCKED>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
@@ -717,6 +812,26 @@ int zant_qconv_ps(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float 
         xb = static_cast<const int8_t *>(dyn);
     }
     const int grid = std::min(p.n_tiles, ctx->num_cus);
+    // NCHW output: staged through LDS and written as whole runs of a plane when the runs are made of aligned 8- or
+    // 4-byte units and the tile's bytes have room: a region of their own behind the patch, or -- one tile per workgroup,
+    // one pass -- the ring, slot table and patch, which are dead by then.
+    p.out_unit = 0; p.stage_off = 0; p.stage_alias = 0; p.S_pad = 0;
+    if (!y_blocked) {
+        const int per_img = p.TH * p.OW, plane = p.OH * p.OW;
+        auto unit_ok = [&](int u) {
+            return per_img % u == 0 && plane % u == 0 && (p.OH % p.TH == 0 || p.OW % u == 0) && reinterpret_cast<uintptr_t>(y) % u == 0;
+        };
+        const int unit = unit_ok(8) ? 8 : unit_ok(4) ? 4 : 0;
+        // a staging row holds the tile's positions rounded up to whole position tiles (the last one is written whole);
+        // 8 x an odd number of bytes: the 32 channels of a store then fall on 32 different even banks
+        const int spad = ((p.npt * 32 / 8) | 1) * 8;
+        const size_t need = size_t(spad) * p.KP, behind_ring = size_t(MT) * PS_NT * 4 + size_t(2 * p.NC) * p.P1s * 16;
+        if (unit && lds + need <= size_t(160) * 1024) {
+            p.out_unit = unit; p.S_pad = spad; p.stage_off = int(2 * PS_RING + behind_ring); lds += need;
+        } else if (unit && p.n_tiles <= grid && p.NKP == 1 && need <= 2 * PS_RING + behind_ring) {
+            p.out_unit = unit; p.S_pad = spad; p.stage_alias = 1;
+        }
+    }
     KernelTimer kt(ctx);
     const int yb = y_blocked ? 1 : 0;
     const char *tabs = base + o_mult;
