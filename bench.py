@@ -186,6 +186,17 @@ def main():
     lean_path = {"ms_per_step": round(lean_ms, 4), "inferences_per_s": round(BATCH / lean_ms * 1e3, 1), "calls_per_step": 8,
                  "what": "conv_lean(+relu) / onnx_maxpool_lean / conv_lean(+relu) / onnx_maxpool_lean / gemm_lean(+relu) / "
                          "gemm_lean / softmax_lean through the C ABI on preallocated tensors"}
+    # the same eight calls with prepared-weights handles for the two convolutions (zant_hip_conv2d_f32_prepack): what a
+    # binding that keeps its weights pays once they are packed
+    lean.prepare()
+    np.testing.assert_allclose(lean.forward(xt)[[0, 1, 2, BATCH - 1]].cpu().numpy(), ref, rtol=1e-4, atol=1e-5)
+    for _ in range(3):
+        lean.forward(xt)
+    ctx.sync()
+    ctx.timer_start()
+    for _ in range(kit):
+        lean.forward(xt)
+    lean_path["ms_per_step_prepared_weights"] = round(ctx.timer_stop() / kit, 4)
     del lean, xt, lean_out
 
     # ---- standalone operator figures (the "conv TOPS" half of the metric): configs 2a, 2b, 3 ----
@@ -250,6 +261,30 @@ def main():
         operators["qlinearconv_u8i8_N128_C128_28x28_K128_3x3"] = {"ms": round(ms, 4), "tops": round(op / ms / 1e9, 2),
                                                                   "frac_i8_mfma_peak": round(op / ms / 1e9 / PEAK_I8_MFMA_TOPS, 5),
                                                                   "kernel": q_kernel, "whole_call_ms": round(call_ms, 4)}
+        # with a prepared-weights handle (zant_hip_qlinearconv_prepack): NCHW tensors (the layout conversion stays), and
+        # channel-blocked tensors on both sides (the call is the kernel)
+        qop = operators["qlinearconv_u8i8_N128_C128_28x28_K128_3x3"]
+        plan = tm.QConvPlan(xq.shape, 0.02, 128, wq, ws, None, 0.05, 128, bq, [1, 1], [1, 1, 1, 1], [1, 1])
+        yq2 = torch.zeros_like(yq)
+        plan(xq, yq2)
+        assert torch.equal(yq2, yq), "config 3: the prepared call differs from the plain one"
+        ctx.sync(); ctx.timer_start()
+        for _ in range(kit):
+            plan(xq, yq2)
+        qop["prepared_call_ms"] = round(ctx.timer_stop() / kit, 4)
+        plan.close()
+        planb = tm.QConvPlan(xq.shape, 0.02, 128, wq, ws, None, 0.05, 128, bq, [1, 1], [1, 1, 1, 1], [1, 1],
+                             x_layout=tm.BLOCKED16, y_layout=tm.BLOCKED16)
+        xb = tm.to_blocked16(xq)
+        yb = planb(xb)
+        assert torch.equal(tm.from_blocked16(yb, yq.shape), yq), "config 3: the blocked prepared call differs from the plain one"
+        ctx.sync(); ctx.timer_start()
+        for _ in range(kit):
+            planb(xb, yb)
+        qop["prepared_blocked_call_ms"] = round(ctx.timer_stop() / kit, 4)
+        qop["prepared_blocked_kernel_ms"] = round(kernel_avg_ms(ctx, lambda: planb(xb, yb), kit), 4)
+        planb.close()
+        del xb, yb, yq2
         pick = [0, 127]
         t0 = time.perf_counter()
         ref_q = zo.qlinearconv(xq[pick].cpu().numpy(), 0.02, 128, wq.cpu().numpy(), ws.cpu().numpy(), None, 0.05, 128,
@@ -260,6 +295,20 @@ def main():
         if not args.no_cpu_baseline:
             operators["qlinearconv_u8i8_N128_C128_28x28_K128_3x3"]["cpu_oracle_1core"] = {
                 "gops": round(op * 2 / 128 / dt / 1e9, 2), "sample": f"2 of 128 images, {dt:.1f} s"}
+        # the same layer at batch 1024: eight tiles per compute unit instead of one, which shows the rate of the
+        # kernel's tile pipeline apart from launch, first fill and the last epilogue
+        del xq, yq
+        xq8 = torch.randint(0, 256, (1024, 128, 28, 28), dtype=torch.uint8, device=dev)
+        yq8 = torch.zeros(1024, 128, 28, 28, dtype=torch.uint8, device=dev)
+        fn8 = lambda: tm.qlinearconv_lean(xq8, 0.02, 128, wq, ws, None, 0.05, 128, bq, yq8, [1, 1], [1, 1, 1, 1], [1, 1])
+        fn8(); ms8 = kernel_avg_ms(ctx, fn8, kit)
+        ref8 = zo.qlinearconv(xq8[[0, 1023]].cpu().numpy(), 0.02, 128, wq.cpu().numpy(), ws.cpu().numpy(), None, 0.05, 128,
+                              bq.cpu().numpy(), [1, 1], [1, 1, 1, 1], [1, 1])
+        assert np.array_equal(yq8[[0, 1023]].cpu().numpy(), ref8), "config 3 at batch 1024: timed output differs from the oracle"
+        operators["qlinearconv_u8i8_N1024_C128_28x28_K128_3x3"] = {
+            "ms": round(ms8, 4), "tops": round(8 * op / ms8 / 1e9, 2), "frac_i8_mfma_peak": round(8 * op / ms8 / 1e9 / PEAK_I8_MFMA_TOPS, 5),
+            "kernel": ctx.kernel_name(), "parity_gate": "images 0 and 1023 of the timed output against the oracle, bit-exact"}
+        del xq8, yq8
 
     # ---- HBM-bound operators (pool / activation / requantisation / residual add): algorithmic bytes / kernel time ----
     if operators is not None:
@@ -382,9 +431,15 @@ def main():
                 qm.run()
             ms = ctx.timer_stop() / kit
             macs = gold[name]["macs_per_inference"]
+            # the two floors of the pass: its integer operations at the int8 matrix-core peak, and the algorithmic
+            # bytes of its launches (inputs + parameters + output of each, once) at the HBM peak
+            prof = qm.profile()
             nets_out[name] = {"batch": nb, "ms_per_step": round(ms, 4), "inferences_per_s": round(nb / ms * 1e3, 1),
                               "tops": round(2.0 * macs * nb / ms / 1e9, 2), "launches_per_step": qm.num_launches,
-                              "arena_bytes": qm.arena_bytes}
+                              "arena_bytes": qm.arena_bytes,
+                              "mfma_floor_ms": round(2.0 * macs * nb / (PEAK_I8_MFMA_TOPS * 1e12) * 1e3, 4),
+                              "hbm_floor_ms": round(sum(pb for _, _, _, pb in prof) / (PEAK_HBM_GBS * 1e9) * 1e3, 4),
+                              "kernel_ms": [round(pm, 4) for _, pm, _, _ in prof]}
             qm.close()
 
     # ---- CPU baseline: the oracle on one host core, one image at a time, over a bounded sample ----

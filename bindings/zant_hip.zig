@@ -21,6 +21,8 @@ pub const AutoPadType = @import("op_pooling.zig").AutoPadType; // NOTSET, SAME_U
 
 pub const zant_ctx = opaque {};
 pub const zant_model = opaque {};
+pub const zant_conv_plan = opaque {};
+pub const zant_qconv_plan = opaque {};
 pub const LogFn = ?*const fn ([*c]u8) callconv(.C) void;
 
 pub const ZANT_OK: c_int = 0;
@@ -34,6 +36,9 @@ pub const ZANT_ACT_RELU: c_int = 1;
 pub const ZANT_ACT_LEAKY: c_int = 2;
 pub const ZANT_ACT_RELU6: c_int = 3;
 pub const ZANT_ACT_SOFTMAX: c_int = 4;
+
+pub const ZANT_LAYOUT_NCHW: c_int = 0;
+pub const ZANT_LAYOUT_BLOCKED16: c_int = 1;
 
 pub const ZANT_F32: c_int = 0;
 pub const ZANT_U8: c_int = 1;
@@ -67,6 +72,9 @@ pub extern fn zant_hip_kernel_name(ctx: ?*zant_ctx) [*:0]const u8;
 pub extern fn zant_hip_conv2d_f32(ctx: ?*zant_ctx, x: [*]const f32, xdim: *const [4]i64, w: [*]const f32, wdim: *const [4]i64, bias: ?[*]const f32, y: [*]f32, ydim: *const [4]i64, stride: [*]const i64, n_stride: c_int, pads: ?[*]const i64, n_pads: c_int, dil: ?[*]const i64, n_dil: c_int, group: i64, auto_pad: ?[*:0]const u8, fuse_act: c_int) c_int;
 pub extern fn zant_hip_conv2d_out_shape(xdim: *const [4]i64, wdim: *const [4]i64, stride: [*]const i64, n_stride: c_int, pads: ?[*]const i64, n_pads: c_int, dil: ?[*]const i64, n_dil: c_int, group: i64, auto_pad: ?[*:0]const u8, ydim: *[4]i64) c_int;
 pub extern fn zant_hip_conv2d_f32_static(ctx: ?*zant_ctx, x: [*]const f32, xdim: *const [4]i64, w: [*]const f32, wdim: *const [4]i64, bias: ?[*]const f32, y: [*]f32, ydim: *const [4]i64, stride: [*]const i64, n_stride: c_int, pads: ?[*]const i64, n_pads: c_int, dil: ?[*]const i64, n_dil: c_int, group: i64, auto_pad: ?[*:0]const u8, fuse_act: c_int) c_int;
+pub extern fn zant_hip_conv2d_f32_prepack(ctx: ?*zant_ctx, xdim: *const [4]i64, w: [*]const f32, wdim: *const [4]i64, bias: ?[*]const f32, ydim: *const [4]i64, stride: [*]const i64, n_stride: c_int, pads: ?[*]const i64, n_pads: c_int, dil: ?[*]const i64, n_dil: c_int, group: i64, auto_pad: ?[*:0]const u8, fuse_act: c_int, out: *?*zant_conv_plan) c_int;
+pub extern fn zant_hip_conv2d_f32_packed(ctx: ?*zant_ctx, plan: ?*zant_conv_plan, x: [*]const f32, y: [*]f32) c_int;
+pub extern fn zant_hip_conv2d_plan_destroy(ctx: ?*zant_ctx, plan: ?*zant_conv_plan) void;
 pub extern fn zant_hip_matmul_f32(ctx: ?*zant_ctx, a: [*]const f32, adim: [*]const i64, a_rank: c_int, b: [*]const f32, bdim: [*]const i64, b_rank: c_int, y: [*]f32) c_int;
 pub extern fn zant_hip_matmul_check(adim: [*]const i64, a_rank: c_int, bdim: [*]const i64, b_rank: c_int) c_int;
 pub extern fn zant_hip_gemm_f32(ctx: ?*zant_ctx, a: [*]const f32, adim: *const [4]i64, b: [*]const f32, bdim: *const [4]i64, c: ?[*]const f32, cdim: ?[*]const i64, c_rank: c_int, alpha: f32, beta: f32, trans_a: c_int, trans_b: c_int, y: [*]f32, ydim: *const [4]i64, fuse_act: c_int) c_int;
@@ -94,6 +102,12 @@ pub extern fn zant_hip_quantize_linear_f32_i8(ctx: ?*zant_ctx, x: [*]const f32, 
 pub extern fn zant_hip_dequantize_linear_i8_f32(ctx: ?*zant_ctx, x: [*]const i8, xdim: [*]const i64, rank: c_int, x_scale: [*]const f32, x_zp: ?[*]const i8, n_scale: i64, axis: c_int, y: [*]f32) c_int;
 pub extern fn zant_hip_dequantize_linear_i32_f32(ctx: ?*zant_ctx, x: [*]const i32, xdim: [*]const i64, rank: c_int, x_scale: [*]const f32, x_zp: ?[*]const i32, n_scale: i64, axis: c_int, y: [*]f32) c_int;
 pub extern fn zant_hip_qlinearconv_u8i8(ctx: ?*zant_ctx, x: [*]const u8, xdim: *const [4]i64, x_scale: f32, x_zp: u8, w: [*]const i8, wdim: *const [4]i64, w_scale: [*]const f32, n_wscale: i64, w_zp: ?[*]const i8, y_scale: f32, y_zp: u8, bias: ?[*]const i32, y: [*]u8, ydim: *const [4]i64, stride: *const [2]i64, pads: *const [4]i64, dil: *const [2]i64, group: i64, act: c_int, act_alpha: f32, act_scale: f32, act_zp: u8) c_int;
+pub extern fn zant_hip_blocked16_bytes(dim: *const [4]i64) usize;
+pub extern fn zant_hip_to_blocked16_u8(ctx: ?*zant_ctx, x: [*]const u8, dim: *const [4]i64, x_blocked: [*]u8) c_int;
+pub extern fn zant_hip_from_blocked16_u8(ctx: ?*zant_ctx, x_blocked: [*]const u8, dim: *const [4]i64, y: [*]u8) c_int;
+pub extern fn zant_hip_qlinearconv_prepack(ctx: ?*zant_ctx, xdim: *const [4]i64, x_scale: f32, x_zp: u8, w: [*]const i8, wdim: *const [4]i64, w_scale: [*]const f32, n_wscale: i64, w_zp: ?[*]const i8, y_scale: f32, y_zp: u8, bias: ?[*]const i32, ydim: *const [4]i64, stride: *const [2]i64, pads: *const [4]i64, dil: *const [2]i64, group: i64, act: c_int, act_alpha: f32, act_scale: f32, act_zp: u8, x_layout: c_int, y_layout: c_int, out: *?*zant_qconv_plan) c_int;
+pub extern fn zant_hip_qlinearconv_u8i8_packed(ctx: ?*zant_ctx, plan: ?*zant_qconv_plan, x: [*]const u8, y: [*]u8) c_int;
+pub extern fn zant_hip_qlinearconv_plan_destroy(ctx: ?*zant_ctx, plan: ?*zant_qconv_plan) void;
 pub extern fn zant_hip_qlinear_act_u8(ctx: ?*zant_ctx, x: [*]const u8, n: i64, x_scale: f32, x_zp: u8, act: c_int, alpha: f32, y_scale: f32, y_zp: u8, y: [*]u8) c_int;
 pub extern fn zant_hip_qlinear_add_u8(ctx: ?*zant_ctx, a: [*]const u8, a_scale: f32, a_zp: u8, b: [*]const u8, b_scale: f32, b_zp: u8, y_scale: f32, y_zp: u8, y: [*]u8, n: i64) c_int;
 pub extern fn zant_hip_maxpool2d_u8(ctx: ?*zant_ctx, x: [*]const u8, xdim: *const [4]i64, y: [*]u8, ydim: *const [4]i64, kernel: *const [2]i64, strides: *const [2]i64, dil: *const [2]i64, pads: ?[*]const i64, n_pads: c_int, auto_pad: c_int) c_int;
@@ -207,7 +221,7 @@ fn toI64(comptime n: usize, s: []const usize) [n]i64 {
 }
 
 fn onlyF32(comptime T: type) void {
-    if (T != f32) @compileError("the HIP backend's lean operators are f32; quantised graphs use the zant_model_q* calls");
+    if (T != f32) @compileError("this lean operator of the HIP backend is f32 only; the quantised family is qlinearconv_lean / quantize_linear_lean / dequantize_linear_lean / onnx_maxpool_lean(u8)");
 }
 
 /// conv_lean = OnnxConvLean (op_convolution.zig:42).
@@ -254,14 +268,18 @@ pub const lean_matmul = mat_mul_lean; // both names exist in tensor_math_standar
 
 /// onnx_maxpool_lean = lean_onnx_maxpool (op_pooling.zig:570-579).
 pub fn onnx_maxpool_lean(comptime T: type, input: *Tensor(T), output: *Tensor(T), kernel_shape: []const usize, strides: []const usize, dilations: []const usize, pads: []const usize, auto_pad: AutoPadType) !void {
-    comptime onlyF32(T);
+    if (T != f32 and T != u8) @compileError("onnx_maxpool_lean of the HIP backend takes f32 or u8 (quantised values: max-pooling commutes with the monotone quantisation)");
     const xd = try dims4(input.shape);
     const yd = try dims4(output.shape);
     const k = toI64(2, kernel_shape);
     const s = toI64(2, strides);
     const d = toI64(2, dilations);
     const p = toI64(4, pads);
-    try toErr(zant_hip_maxpool2d_f32(ctx, input.data.ptr, &xd, output.data.ptr, &yd, &k, &s, &d, &p, @intCast(pads.len), @intFromEnum(auto_pad)));
+    if (T == u8) {
+        try toErr(zant_hip_maxpool2d_u8(ctx, input.data.ptr, &xd, output.data.ptr, &yd, &k, &s, &d, &p, @intCast(pads.len), @intFromEnum(auto_pad)));
+    } else {
+        try toErr(zant_hip_maxpool2d_f32(ctx, input.data.ptr, &xd, output.data.ptr, &yd, &k, &s, &d, &p, @intCast(pads.len), @intFromEnum(auto_pad)));
+    }
 }
 
 /// get_onnx_maxpool_output_shape (op_pooling.zig:477-485); the caller frees the result, as there.
@@ -485,6 +503,129 @@ pub fn batchnorm_lean(comptime T: type, input: *Tensor(T), gamma: *Tensor(T), be
     const xd = try dimsN(input.shape);
     try toErr(zant_hip_batchnorm_f32(ctx, input.data.ptr, &xd, @intCast(input.shape.len), gamma.data.ptr, beta.data.ptr, running_mean.data.ptr, running_var.data.ptr, epsilon, output.data.ptr));
 }
+
+// ---- the quantised family (ONNX QuantizeLinear / DequantizeLinear / QLinearConv) ---------------------------
+// The reference has no such operators (src/Core/Quantization/quantization.zig is empty); these follow its house
+// style -- comptime element types, pre-shaped output, `!void` -- and the ONNX input order.  Scales and zero points
+// are tensors, as ONNX passes them: per tensor (one element) or per `axis`.
+
+/// quantize_linear_lean: y = saturate(round_half_even(x / y_scale) + y_zero_point).  T_out: u8 or i8.
+/// y_scale / y_zero_point hold one element, or input.shape[axis] elements (per-axis); they are DEVICE tensors.
+pub fn quantize_linear_lean(comptime T_in: type, comptime T_out: type, x: *Tensor(T_in), y_scale: *Tensor(T_in), y_zero_point: ?*Tensor(T_out), axis: i64, y: *Tensor(T_out)) !void {
+    comptime onlyF32(T_in);
+    if (T_out != u8 and T_out != i8) @compileError("quantize_linear_lean: T_out is u8 or i8");
+    const xd = try dimsN(x.shape);
+    const rank: i64 = @intCast(x.shape.len);
+    const ax: c_int = @intCast(if (axis < 0) axis + rank else axis);
+    if (T_out == u8) {
+        try toErr(zant_hip_quantize_linear_f32_u8(ctx, x.data.ptr, &xd, @intCast(x.shape.len), y_scale.data.ptr, if (y_zero_point) |z| z.data.ptr else null, @intCast(y_scale.size), ax, y.data.ptr));
+    } else {
+        try toErr(zant_hip_quantize_linear_f32_i8(ctx, x.data.ptr, &xd, @intCast(x.shape.len), y_scale.data.ptr, if (y_zero_point) |z| z.data.ptr else null, @intCast(y_scale.size), ax, y.data.ptr));
+    }
+}
+
+/// dequantize_linear_lean: y = (x - x_zero_point) * x_scale.  T_in: u8, i8 or i32 (accumulators, biases).
+pub fn dequantize_linear_lean(comptime T_in: type, comptime T_out: type, x: *Tensor(T_in), x_scale: *Tensor(T_out), x_zero_point: ?*Tensor(T_in), axis: i64, y: *Tensor(T_out)) !void {
+    comptime onlyF32(T_out);
+    if (T_in != u8 and T_in != i8 and T_in != i32) @compileError("dequantize_linear_lean: T_in is u8, i8 or i32");
+    const xd = try dimsN(x.shape);
+    const rank: i64 = @intCast(x.shape.len);
+    const ax: c_int = @intCast(if (axis < 0) axis + rank else axis);
+    const zp = if (x_zero_point) |z| z.data.ptr else null;
+    const n: i64 = @intCast(x_scale.size);
+    const r: c_int = @intCast(x.shape.len);
+    switch (T_in) {
+        u8 => try toErr(zant_hip_dequantize_linear_u8_f32(ctx, x.data.ptr, &xd, r, x_scale.data.ptr, zp, n, ax, y.data.ptr)),
+        i8 => try toErr(zant_hip_dequantize_linear_i8_f32(ctx, x.data.ptr, &xd, r, x_scale.data.ptr, zp, n, ax, y.data.ptr)),
+        else => try toErr(zant_hip_dequantize_linear_i32_f32(ctx, x.data.ptr, &xd, r, x_scale.data.ptr, zp, n, ax, y.data.ptr)),
+    }
+}
+
+/// qlinearconv_lean: ONNX QLinearConv in the input order of the operator (x, x_scale, x_zero_point, w, w_scale,
+/// w_zero_point, y_scale, y_zero_point, B) followed by conv_lean's attributes (op_convolution.zig:42).  x_scale,
+/// x_zero_point, y_scale and y_zero_point are per-tensor HOST scalars (ONNX requires them to be scalars); w_scale
+/// (one element or one per output channel), w_zero_point (null: 0) and bias are DEVICE tensors.  pads are
+/// [top, left, bottom, right]; null pads / dilations mean 0 / 1; group null means 1 (group == channels: depthwise).
+pub fn qlinearconv_lean(x: *Tensor(u8), x_scale: f32, x_zero_point: u8, w: *Tensor(i8), w_scale: *Tensor(f32), w_zero_point: ?*Tensor(i8), y_scale: f32, y_zero_point: u8, bias: ?*const Tensor(i32), y: *Tensor(u8), stride: []const usize, pads: ?[]const usize, dilations: ?[]const usize, group: ?usize) !void {
+    const xd = try dims4(x.shape);
+    const wd = try dims4(w.shape);
+    const yd = try dims4(y.shape);
+    if (stride.len < 1) return TensorMathError.WrongStride;
+    var s = toI64(2, stride);
+    if (stride.len == 1) s[1] = s[0]; // as conv_lean: stride[1] falls back to stride[0] (op_convolution.zig:68-69)
+    var p = [_]i64{0} ** 4;
+    var d = [_]i64{1} ** 2;
+    if (pads) |pp| {
+        if (pp.len < 4) return TensorMathError.InvalidPadding;
+        p = toI64(4, pp);
+    }
+    if (dilations) |dd| {
+        d = toI64(2, dd);
+        if (dd.len == 1) d[1] = d[0];
+    }
+    try toErr(zant_hip_qlinearconv_u8i8(ctx, x.data.ptr, &xd, x_scale, x_zero_point, w.data.ptr, &wd, w_scale.data.ptr, @intCast(w_scale.size), if (w_zero_point) |z| z.data.ptr else null, y_scale, y_zero_point, if (bias) |b| b.data.ptr else null, y.data.ptr, &yd, &s, &p, &d, if (group) |g| @intCast(g) else 1, ZANT_ACT_NONE, 0.0, 1.0, 0));
+}
+
+/// Prepared weights for qlinearconv_lean: the weight-dependent tables are derived once, at the first `run`.
+pub const QLinearConvPlan = struct {
+    handle: ?*zant_qconv_plan = null,
+
+    pub fn init(xshape: []const usize, x_scale: f32, x_zero_point: u8, w: *Tensor(i8), w_scale: *Tensor(f32), w_zero_point: ?*Tensor(i8), y_scale: f32, y_zero_point: u8, bias: ?*const Tensor(i32), yshape: []const usize, stride: [2]usize, pads: [4]usize, dilations: [2]usize, group: usize, x_layout: c_int, y_layout: c_int) !QLinearConvPlan {
+        const xd = try dims4(xshape);
+        const wd = try dims4(w.shape);
+        const yd = try dims4(yshape);
+        const s = toI64(2, &stride);
+        const p = toI64(4, &pads);
+        const d = toI64(2, &dilations);
+        var self = QLinearConvPlan{};
+        try toErr(zant_hip_qlinearconv_prepack(ctx, &xd, x_scale, x_zero_point, w.data.ptr, &wd, w_scale.data.ptr, @intCast(w_scale.size), if (w_zero_point) |z| z.data.ptr else null, y_scale, y_zero_point, if (bias) |b| b.data.ptr else null, &yd, &s, &p, &d, @intCast(group), ZANT_ACT_NONE, 0.0, 1.0, 0, x_layout, y_layout, &self.handle));
+        return self;
+    }
+
+    pub fn run(self: *QLinearConvPlan, x: [*]const u8, y: [*]u8) !void {
+        try toErr(zant_hip_qlinearconv_u8i8_packed(ctx, self.handle, x, y));
+    }
+
+    pub fn deinit(self: *QLinearConvPlan) void {
+        zant_hip_qlinearconv_plan_destroy(ctx, self.handle);
+        self.handle = null;
+    }
+};
+
+/// Prepared weights for conv_lean (same attributes); `run` is conv_lean without the per-call weight packing.
+pub const ConvPlan = struct {
+    handle: ?*zant_conv_plan = null,
+
+    pub fn init(xshape: []const usize, kernel: *Tensor(f32), bias: ?*const Tensor(f32), yshape: []const usize, stride: []const usize, pads: ?[]const usize, dilations: ?[]const usize, group: ?usize, auto_pad: ?[]const u8, fuse_act: c_int) !ConvPlan {
+        const xd = try dims4(xshape);
+        const wd = try dims4(kernel.shape);
+        const yd = try dims4(yshape);
+        const s = toI64(2, stride);
+        var p = [_]i64{0} ** 4;
+        var d = [_]i64{1} ** 2;
+        if (pads) |pp| p = toI64(4, pp);
+        if (dilations) |dd| d = toI64(2, dd);
+        var ap_buf: [16:0]u8 = undefined;
+        const ap: ?[*:0]const u8 = if (auto_pad) |a| blk: {
+            if (a.len > 15) return TensorMathError.InvalidPadding;
+            @memcpy(ap_buf[0..a.len], a);
+            ap_buf[a.len] = 0;
+            break :blk &ap_buf;
+        } else null;
+        var self = ConvPlan{};
+        try toErr(zant_hip_conv2d_f32_prepack(ctx, &xd, kernel.data.ptr, &wd, if (bias) |b| b.data.ptr else null, &yd, &s, @intCast(stride.len), if (pads != null) &p else null, if (pads) |pp| @intCast(pp.len) else 0, if (dilations != null) &d else null, if (dilations) |dd| @intCast(dd.len) else 0, if (group) |g| @intCast(g) else -1, ap, fuse_act, &self.handle));
+        return self;
+    }
+
+    pub fn run(self: *ConvPlan, x: [*]const f32, y: [*]f32) !void {
+        try toErr(zant_hip_conv2d_f32_packed(ctx, self.handle, x, y));
+    }
+
+    pub fn deinit(self: *ConvPlan) void {
+        zant_hip_conv2d_plan_destroy(ctx, self.handle);
+        self.handle = null;
+    }
+};
 
 // ---- device tensors ---------------------------------------------------------------------------------------
 

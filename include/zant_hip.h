@@ -143,6 +143,20 @@ int zant_hip_conv2d_f32_static(zant_ctx *ctx, const float *x, const int64_t xdim
                                const int64_t *stride, int n_stride, const int64_t *pads, int n_pads,
                                const int64_t *dil, int n_dil, int64_t group, const char *auto_pad, int fuse_act);
 
+/* Prepared weights for zant_hip_conv2d_f32.  The reference's conv_lean takes the weights on every call
+ * (op_convolution.zig:42), so zant_hip_conv2d_f32 has to assume they changed and re-packs them for the
+ * matrix-core kernel each time.  A plan fixes shapes, attributes (same meaning and checks as zant_hip_conv2d_f32,
+ * made here) and the weight / bias tensors once: the first zant_hip_conv2d_f32_packed packs into memory the plan
+ * owns, later calls launch the convolution kernel only.  w and bias are DEVICE pointers that must stay valid and
+ * unchanged while the plan lives.  Destroy the plan before its context. */
+typedef struct zant_conv_plan zant_conv_plan;
+int zant_hip_conv2d_f32_prepack(zant_ctx *ctx, const int64_t xdim[4], const float *w, const int64_t wdim[4],
+                                const float *bias, const int64_t ydim[4], const int64_t *stride, int n_stride,
+                                const int64_t *pads, int n_pads, const int64_t *dil, int n_dil, int64_t group,
+                                const char *auto_pad, int fuse_act, zant_conv_plan **out);
+int zant_hip_conv2d_f32_packed(zant_ctx *ctx, zant_conv_plan *plan, const float *x, float *y);
+void zant_hip_conv2d_plan_destroy(zant_ctx *ctx, zant_conv_plan *plan);
+
 /* mat_mul_lean = lean_mat_mul (op_mat_mul.zig:92-172): last two dims only. */
 int zant_hip_matmul_f32(zant_ctx *ctx, const float *a, const int64_t *adim, int a_rank, const float *b,
                         const int64_t *bdim, int b_rank, float *y);
@@ -269,6 +283,31 @@ int zant_hip_qlinearconv_u8i8(zant_ctx *ctx, const uint8_t *x, const int64_t xdi
                               const int32_t *bias, uint8_t *y, const int64_t ydim[4], const int64_t stride[2],
                               const int64_t pads[4], const int64_t dil[2], int64_t group, int act,
                               float act_alpha, float act_scale, uint8_t act_zp);
+/* Layouts of a u8 activation tensor [N, C, H, W].  ZANT_LAYOUT_NCHW is the reference's row-major layout, the only one
+ * the lean operators above take.  ZANT_LAYOUT_BLOCKED16 is what the int8 matrix-core kernels read and write natively:
+ * [N][ceil(C/16)][H][W][16] bytes, each holding value ^ 0x80 (zant_hip_blocked16_bytes() bytes in all; bytes of
+ * channels >= C are unspecified).  A caller that chains prepared convolutions keeps its activations blocked and
+ * converts only at the ends. */
+enum zant_layout { ZANT_LAYOUT_NCHW = 0, ZANT_LAYOUT_BLOCKED16 = 1 };
+size_t zant_hip_blocked16_bytes(const int64_t dim[4]);
+int zant_hip_to_blocked16_u8(zant_ctx *ctx, const uint8_t *x, const int64_t dim[4], uint8_t *x_blocked);
+int zant_hip_from_blocked16_u8(zant_ctx *ctx, const uint8_t *x_blocked, const int64_t dim[4], uint8_t *y);
+/* Prepared weights for zant_hip_qlinearconv_u8i8 (no counterpart in the reference, whose operators take the weights on
+ * every call).  Arguments, checks and results are those of zant_hip_qlinearconv_u8i8, made once here; x_layout /
+ * y_layout say how the activations handed to zant_hip_qlinearconv_u8i8_packed are laid out.  The first packed call
+ * derives everything weight-dependent (packed weights, requantisation multipliers and corrections) into memory the
+ * plan owns; later calls launch the convolution kernel only, and with blocked activations no layout conversion
+ * either.  w, w_scale, w_zp and bias are DEVICE pointers that must stay valid and unchanged while the plan lives.
+ * Destroy the plan before its context. */
+typedef struct zant_qconv_plan zant_qconv_plan;
+int zant_hip_qlinearconv_prepack(zant_ctx *ctx, const int64_t xdim[4], float x_scale, uint8_t x_zp, const int8_t *w,
+                                 const int64_t wdim[4], const float *w_scale, int64_t n_wscale, const int8_t *w_zp,
+                                 float y_scale, uint8_t y_zp, const int32_t *bias, const int64_t ydim[4],
+                                 const int64_t stride[2], const int64_t pads[4], const int64_t dil[2], int64_t group,
+                                 int act, float act_alpha, float act_scale, uint8_t act_zp, int x_layout, int y_layout,
+                                 zant_qconv_plan **out);
+int zant_hip_qlinearconv_u8i8_packed(zant_ctx *ctx, zant_qconv_plan *plan, const uint8_t *x, uint8_t *y);
+void zant_hip_qlinearconv_plan_destroy(zant_ctx *ctx, zant_qconv_plan *plan);
 /* DequantizeLinear -> {none, ReLU, LeakyReLU(alpha), ReLU6} -> QuantizeLinear. */
 int zant_hip_qlinear_act_u8(zant_ctx *ctx, const uint8_t *x, int64_t n, float x_scale, uint8_t x_zp, int act,
                             float alpha, float y_scale, uint8_t y_zp, uint8_t *y);

@@ -119,7 +119,18 @@ def test_zig_binding_mirrors_the_header():
         "pub fn sigmoid_lean(comptime T: anytype, input_tensor: *Tensor(T), output_tensor: *Tensor(T)) !void",
         "pub fn reduce_mean_lean(comptime T: anytype, input_tensor: *Tensor(T), output_tensor: *Tensor(T), axes: ?[]const i64, _: bool, noop_with_empty_axes: bool) !void",
         "pub fn lean_concatenate(comptime T: type, allocator: *const std.mem.Allocator, tensors: []const Tensor(T), axis: isize, output: *Tensor(T)) !void",
+        # the quantised family (not in the reference): house style -- comptime element types, pre-shaped output, !void --
+        # and the ONNX input order
+        "pub fn quantize_linear_lean(comptime T_in: type, comptime T_out: type, x: *Tensor(T_in), y_scale: *Tensor(T_in), y_zero_point: ?*Tensor(T_out), axis: i64, y: *Tensor(T_out)) !void",
+        "pub fn dequantize_linear_lean(comptime T_in: type, comptime T_out: type, x: *Tensor(T_in), x_scale: *Tensor(T_out), x_zero_point: ?*Tensor(T_in), axis: i64, y: *Tensor(T_out)) !void",
+        "pub fn qlinearconv_lean(x: *Tensor(u8), x_scale: f32, x_zero_point: u8, w: *Tensor(i8), w_scale: *Tensor(f32), w_zero_point: ?*Tensor(i8), y_scale: f32, y_zero_point: u8, bias: ?*const Tensor(i32), y: *Tensor(u8), stride: []const usize, pads: ?[]const usize, dilations: ?[]const usize, group: ?usize) !void",
     ]
+    # the façade calls the u8 pooling entry and every quantised entry it wraps
+    for used in ("zant_hip_maxpool2d_u8(ctx", "zant_hip_quantize_linear_f32_u8(ctx", "zant_hip_quantize_linear_f32_i8(ctx",
+                 "zant_hip_dequantize_linear_u8_f32(ctx", "zant_hip_dequantize_linear_i8_f32(ctx",
+                 "zant_hip_dequantize_linear_i32_f32(ctx", "zant_hip_qlinearconv_u8i8(ctx", "zant_hip_qlinearconv_prepack(ctx",
+                 "zant_hip_qlinearconv_u8i8_packed(ctx", "zant_hip_conv2d_f32_prepack(ctx", "zant_hip_conv2d_f32_packed(ctx"):
+        assert used in zig, used
     for sig in lean:
         assert sig in zig, sig
     # every status the header names maps to an error (or to the catch-all for HIP / memory failures)

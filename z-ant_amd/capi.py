@@ -48,6 +48,10 @@ PROTOTYPES = {
                                   i64, C.c_char_p, i32]),
     "zant_hip_conv2d_f32_static": (i32, [vp, vp, c_i64p, vp, c_i64p, vp, vp, c_i64p, c_i64p, i32, c_i64p, i32, c_i64p,
                                          i32, i64, C.c_char_p, i32]),
+    "zant_hip_conv2d_f32_prepack": (i32, [vp, c_i64p, vp, c_i64p, vp, c_i64p, c_i64p, i32, c_i64p, i32, c_i64p, i32, i64,
+                                          C.c_char_p, i32, C.POINTER(vp)]),
+    "zant_hip_conv2d_f32_packed": (i32, [vp, vp, vp, vp]),
+    "zant_hip_conv2d_plan_destroy": (None, [vp, vp]),
     "zant_hip_conv2d_out_shape": (i32, [c_i64p, c_i64p, c_i64p, i32, c_i64p, i32, c_i64p, i32, i64, C.c_char_p, c_i64p]),
     "zant_hip_matmul_f32": (i32, [vp, vp, c_i64p, i32, vp, c_i64p, i32, vp]),
     "zant_hip_matmul_check": (i32, [c_i64p, i32, c_i64p, i32]),
@@ -77,6 +81,13 @@ PROTOTYPES = {
     "zant_hip_dequantize_linear_i32_f32": (i32, [vp, vp, c_i64p, i32, vp, vp, i64, i32, vp]),
     "zant_hip_qlinearconv_u8i8": (i32, [vp, vp, c_i64p, f32, u8, vp, c_i64p, vp, i64, vp, f32, u8, vp, vp, c_i64p,
                                         c_i64p, c_i64p, c_i64p, i64, i32, f32, f32, u8]),
+    "zant_hip_blocked16_bytes": (sz, [c_i64p]),
+    "zant_hip_to_blocked16_u8": (i32, [vp, vp, c_i64p, vp]),
+    "zant_hip_from_blocked16_u8": (i32, [vp, vp, c_i64p, vp]),
+    "zant_hip_qlinearconv_prepack": (i32, [vp, c_i64p, f32, u8, vp, c_i64p, vp, i64, vp, f32, u8, vp, c_i64p, c_i64p,
+                                           c_i64p, c_i64p, i64, i32, f32, f32, u8, i32, i32, C.POINTER(vp)]),
+    "zant_hip_qlinearconv_u8i8_packed": (i32, [vp, vp, vp, vp]),
+    "zant_hip_qlinearconv_plan_destroy": (None, [vp, vp]),
     "zant_hip_qlinear_act_u8": (i32, [vp, vp, i64, f32, u8, i32, f32, f32, u8, vp]),
     "zant_hip_qlinear_add_u8": (i32, [vp, vp, f32, u8, vp, f32, u8, f32, u8, vp, i64]),
     "zant_hip_qlinear_global_avgpool_u8": (i32, [vp, vp, c_i64p, f32, u8, f32, u8, vp]),

@@ -12,7 +12,8 @@
 // of a quad at one position are one 16-byte unit -- one global->LDS copy of the f32 matrix-core convolution (which keeps
 // its patch as [position][4 channels] in LDS and otherwise copies 4 bytes at a time) and one vector store of the kernel
 // that writes it.  Same size as NCHW.  Only between two convolution nodes of a model; never seen outside the executor.
-enum zant_layout { ZANT_LAYOUT_NCHW = 0, ZANT_LAYOUT_BLOCKED16 = 1, ZANT_LAYOUT_C4 = 2 };
+// (ZANT_LAYOUT_NCHW = 0 and ZANT_LAYOUT_BLOCKED16 = 1 are public: include/zant_hip.h)
+constexpr int ZANT_LAYOUT_C4 = 2;
 
 static inline size_t zant_blocked_bytes(const int64_t dim[4]) {
     return size_t(dim[0]) * size_t((dim[1] + 15) / 16) * size_t(dim[2]) * size_t(dim[3]) * 16;

@@ -161,6 +161,102 @@ int main() {
         EXPECT(error_of([&] { tensMath::resize<uint8_t>(&U, "nearest", &scales, &sizes, "half_pixel"); }) == ZANT_InvalidInput);
         EXPECT(error_of([&] { tensMath::resize<uint8_t>(&U, "nearest", nullptr, nullptr, "half_pixel"); }) == ZANT_InvalidInput);
     }
+    {   // QuantizeLinear / DequantizeLinear (ONNX; the reference holds no test): ties round to even, results saturate
+        float v[8] = {0.5f, 1.5f, 2.5f, -0.5f, 300.0f, -300.0f, 3.49f, 126.5f}, one[1] = {1.0f};
+        uint8_t zp0[1] = {0}, zp128[1] = {128};
+        auto x = Tensor<float>::fromArray(v, {8});
+        auto sc = Tensor<float>::fromArray(one, {1});
+        auto z0 = Tensor<uint8_t>::fromArray(zp0, {1});
+        auto z128 = Tensor<uint8_t>::fromArray(zp128, {1});
+        auto q = tensMath::quantize_linear<uint8_t>(&x, &sc, &z0, 0).toHost();
+        const uint8_t e0[8] = {0, 2, 2, 0, 255, 0, 3, 126};
+        for (int i = 0; i < 8; ++i) EXPECT(q[i] == e0[i]);
+        auto q128 = tensMath::quantize_linear<uint8_t>(&x, &sc, &z128, 0).toHost();
+        const uint8_t e128[8] = {128, 130, 130, 128, 255, 0, 131, 254};
+        for (int i = 0; i < 8; ++i) EXPECT(q128[i] == e128[i]);
+        auto qs = tensMath::quantize_linear<int8_t>(&x, &sc, nullptr, 0).toHost();
+        const int8_t es[8] = {0, 2, 2, 0, 127, -128, 3, 126};
+        for (int i = 0; i < 8; ++i) EXPECT(qs[i] == es[i]);
+        // per-axis scales: rows of a [2, 3] tensor quantised with scales {0.5, 2}; then dequantised with the same
+        float m[6] = {1, 2, 3, 4, 5, 6}, sc2[2] = {0.5f, 2.0f};
+        auto xm = Tensor<float>::fromArray(m, {2, 3});
+        auto s2 = Tensor<float>::fromArray(sc2, {2});
+        auto qm = tensMath::quantize_linear<uint8_t>(&xm, &s2, nullptr, 0);
+        auto hm = qm.toHost();
+        const uint8_t em[6] = {2, 4, 6, 2, 2, 3};  // 4/2 = 2, 5/2 = 2.5 -> 2, 6/2 = 3
+        for (int i = 0; i < 6; ++i) EXPECT(hm[i] == em[i]);
+        auto dm = tensMath::dequantize_linear<uint8_t>(&qm, &s2, nullptr, -2).toHost();  // axis -2 = 0
+        const float ed[6] = {1, 2, 3, 4, 4, 6};
+        for (int i = 0; i < 6; ++i) EXPECT(dm[i] == ed[i]);
+        int32_t acc[3] = {-4, 0, 1000};
+        int32_t azp[1] = {-2};
+        auto a = Tensor<int32_t>::fromArray(acc, {3});
+        auto az = Tensor<int32_t>::fromArray(azp, {1});
+        float half[1] = {0.5f};
+        auto sh = Tensor<float>::fromArray(half, {1});
+        auto da = tensMath::dequantize_linear<int32_t>(&a, &sh, &az, 0).toHost();
+        EXPECT(da[0] == -1.0f && da[1] == 1.0f && da[2] == 501.0f);
+    }
+    {   // QLinearConv (ONNX): with unit scales and zero zero-points it is the integer convolution: ones * ones counts
+        // the taps inside the image (the f32 known answer of test_op_convolution.zig:711-812 on integer codes); with
+        // x_zero_point 128 a padding pixel holds the zero point and contributes nothing
+        std::vector<uint8_t> ones(25, 1), x130(25, 130);
+        std::vector<int8_t> k(9, 1);
+        float one[1] = {1.0f};
+        auto w = Tensor<int8_t>::fromArray(k.data(), {1, 1, 3, 3});
+        auto ws = Tensor<float>::fromArray(one, {1});
+        Dims pads{1, 1, 1, 1};
+        const uint8_t expect[25] = {4, 6, 6, 6, 4, 6, 9, 9, 9, 6, 6, 9, 9, 9, 6, 6, 9, 9, 9, 6, 4, 6, 6, 6, 4};
+        auto x = Tensor<uint8_t>::fromArray(ones.data(), {1, 1, 5, 5});
+        auto y = tensMath::qlinearconv(&x, 1.0f, 0, &w, &ws, nullptr, 1.0f, 0, nullptr, {1}, &pads, nullptr, std::nullopt);
+        EXPECT(y.shape == Dims({1, 1, 5, 5}));
+        auto h = y.toHost();
+        for (int i = 0; i < 25; ++i) EXPECT(h[i] == expect[i]);
+        auto x2 = Tensor<uint8_t>::fromArray(x130.data(), {1, 1, 5, 5});  // every pixel is +2 after the zero point
+        int32_t bv[1] = {-3};
+        auto b = Tensor<int32_t>::fromArray(bv, {1});
+        auto y2 = tensMath::qlinearconv(&x2, 1.0f, 128, &w, &ws, nullptr, 1.0f, 10, &b, {1, 1}, &pads, nullptr, 1).toHost();
+        for (int i = 0; i < 25; ++i) EXPECT(y2[i] == 2 * expect[i] - 3 + 10);
+        // the same through a plan, twice (the second run reuses what the first packed)
+        tensMath::QLinearConvPlan plan({1, 1, 5, 5}, 1.0f, 128, &w, &ws, nullptr, 1.0f, 10, &b, {1, 1, 5, 5}, {1, 1}, &pads, nullptr, 1);
+        auto yp = Tensor<uint8_t>::fromShape({1, 1, 5, 5});
+        for (int rep = 0; rep < 2; ++rep) {
+            plan.run(x2.data, yp.data);
+            auto hp = yp.toHost();
+            for (int i = 0; i < 25; ++i) EXPECT(hp[i] == 2 * expect[i] - 3 + 10);
+        }
+        // depthwise: group == channels, each channel with its own filter (1s and 2s)
+        std::vector<uint8_t> two_ch(50, 1);
+        std::vector<int8_t> kd(18, 1);
+        for (int i = 9; i < 18; ++i) kd[size_t(i)] = 2;
+        auto xd = Tensor<uint8_t>::fromArray(two_ch.data(), {1, 2, 5, 5});
+        auto wd = Tensor<int8_t>::fromArray(kd.data(), {2, 1, 3, 3});
+        auto yd = tensMath::qlinearconv(&xd, 1.0f, 0, &wd, &ws, nullptr, 1.0f, 0, nullptr, {1, 1}, &pads, nullptr, 2).toHost();
+        for (int i = 0; i < 25; ++i) EXPECT(yd[i] == expect[i] && yd[25 + i] == 2 * expect[i]);
+        // errors: a group that does not divide the channels, negative padding through the plan
+        EXPECT(error_of([&] { tensMath::qlinearconv(&xd, 1.0f, 0, &wd, &ws, nullptr, 1.0f, 0, nullptr, {1, 1}, &pads, nullptr, 3); }) == ZANT_InvalidDimensions);
+        Dims neg{-1, 0, 0, 0};
+        EXPECT(error_of([&] { tensMath::QLinearConvPlan bad({1, 1, 5, 5}, 1.0f, 0, &w, &ws, nullptr, 1.0f, 0, nullptr, {1, 1, 5, 5}, {1, 1}, &neg, nullptr, 1); }) == ZANT_InvalidPadding);
+        // MaxPool on quantised values (test_op_pooling.zig:156-202 on integer codes)
+        uint8_t pv[16];
+        for (int i = 0; i < 16; ++i) pv[i] = uint8_t(i + 1);
+        auto px = Tensor<uint8_t>::fromArray(pv, {1, 1, 4, 4});
+        auto py = tensMath::onnx_maxpool<uint8_t>(&px, {2, 2}, {2, 2}, {1, 1}, {0, 0, 0, 0}, AutoPadType::NOTSET, false).toHost();
+        EXPECT(py[0] == 6 && py[1] == 8 && py[2] == 14 && py[3] == 16);
+    }
+    {   // conv_lean through a plan (test_op_convolution.zig:654-709 twice)
+        std::vector<float> ones(25, 1.0f), k(9, 1.0f);
+        auto x = Tensor<float>::fromArray(ones.data(), {1, 1, 5, 5});
+        auto w = Tensor<float>::fromArray(k.data(), {1, 1, 3, 3});
+        auto y = Tensor<float>::fromShape({1, 1, 3, 3});
+        Dims pads{0, 0, 0, 0};
+        tensMath::ConvPlan plan({1, 1, 5, 5}, &w, nullptr, {1, 1, 3, 3}, {1}, &pads, nullptr, std::nullopt, nullptr);
+        for (int rep = 0; rep < 2; ++rep) {
+            plan.run(x.data, y.data);
+            for (float v : y.toHost()) EXPECT(v == 9.0f);
+        }
+        EXPECT(error_of([&] { tensMath::ConvPlan bad({1, 1, 5, 5}, &w, nullptr, {1, 1, 4, 4}, {1}, &pads, nullptr, std::nullopt, nullptr); }) == ZANT_InvalidDimensions);
+    }
     check(zant_hip_sync(default_ctx()));
     std::printf(failures ? "host mirror: %d FAILED\n" : "host mirror: all passed\n", failures);
     return failures ? 1 : 0;

@@ -320,5 +320,148 @@ inline void reshape_lean(Tensor<T> *in, const Dims &newShape, std::optional<bool
     out->size = in->size;
 }
 
+// ---- the quantised family: ONNX QuantizeLinear / DequantizeLinear / QLinearConv ---------------------------
+// The reference has no such operators (src/Core/Quantization/quantization.zig is empty); these keep its two forms
+// (lean: pre-shaped output; standard: allocates) and the ONNX input order.  Scale and zero-point tensors live on the
+// device and hold one element (per tensor) or shape[axis] elements (per axis).
+
+// quantize_linear_lean: y = saturate(round_half_even(x / y_scale) + y_zero_point); T_out: uint8_t or int8_t
+template <typename T_out>
+inline void quantize_linear_lean(Tensor<float> *x, Tensor<float> *y_scale, Tensor<T_out> *y_zero_point, int64_t axis,
+                                 Tensor<T_out> *y);
+template <>
+inline void quantize_linear_lean<uint8_t>(Tensor<float> *x, Tensor<float> *y_scale, Tensor<uint8_t> *y_zero_point,
+                                          int64_t axis, Tensor<uint8_t> *y) {
+    if (axis < 0) axis += int64_t(x->shape.size());
+    check(zant_hip_quantize_linear_f32_u8(default_ctx(), x->data, x->shape.data(), int(x->shape.size()), y_scale->data,
+                                          y_zero_point ? y_zero_point->data : nullptr, int64_t(y_scale->size), int(axis), y->data));
+}
+template <>
+inline void quantize_linear_lean<int8_t>(Tensor<float> *x, Tensor<float> *y_scale, Tensor<int8_t> *y_zero_point,
+                                         int64_t axis, Tensor<int8_t> *y) {
+    if (axis < 0) axis += int64_t(x->shape.size());
+    check(zant_hip_quantize_linear_f32_i8(default_ctx(), x->data, x->shape.data(), int(x->shape.size()), y_scale->data,
+                                          y_zero_point ? y_zero_point->data : nullptr, int64_t(y_scale->size), int(axis), y->data));
+}
+template <typename T_out>
+inline Tensor<T_out> quantize_linear(Tensor<float> *x, Tensor<float> *y_scale, Tensor<T_out> *y_zero_point, int64_t axis) {
+    Tensor<T_out> y = Tensor<T_out>::fromShape(x->shape);
+    quantize_linear_lean<T_out>(x, y_scale, y_zero_point, axis, &y);
+    return y;
+}
+
+// dequantize_linear_lean: y = (x - x_zero_point) * x_scale; T_in: uint8_t, int8_t or int32_t
+template <typename T_in>
+inline void dequantize_linear_lean(Tensor<T_in> *x, Tensor<float> *x_scale, Tensor<T_in> *x_zero_point, int64_t axis,
+                                   Tensor<float> *y);
+#define ZANT_DEQUANT_LEAN(T_in, fn)                                                                                       \
+    template <>                                                                                                           \
+    inline void dequantize_linear_lean<T_in>(Tensor<T_in> * x, Tensor<float> * x_scale, Tensor<T_in> * x_zero_point,      \
+                                             int64_t axis, Tensor<float> *y) {                                            \
+        if (axis < 0) axis += int64_t(x->shape.size());                                                                   \
+        check(fn(default_ctx(), x->data, x->shape.data(), int(x->shape.size()), x_scale->data,                            \
+                 x_zero_point ? x_zero_point->data : nullptr, int64_t(x_scale->size), int(axis), y->data));               \
+    }
+ZANT_DEQUANT_LEAN(uint8_t, zant_hip_dequantize_linear_u8_f32)
+ZANT_DEQUANT_LEAN(int8_t, zant_hip_dequantize_linear_i8_f32)
+ZANT_DEQUANT_LEAN(int32_t, zant_hip_dequantize_linear_i32_f32)
+#undef ZANT_DEQUANT_LEAN
+template <typename T_in>
+inline Tensor<float> dequantize_linear(Tensor<T_in> *x, Tensor<float> *x_scale, Tensor<T_in> *x_zero_point, int64_t axis) {
+    Tensor<float> y = Tensor<float>::fromShape(x->shape);
+    dequantize_linear_lean<T_in>(x, x_scale, x_zero_point, axis, &y);
+    return y;
+}
+
+namespace detail {
+inline void qconv_attrs(const Dims &stride, const Dims *pads, const Dims *dilations, int64_t s[2], int64_t p[4], int64_t d[2]) {
+    if (stride.empty()) throw Error(ZANT_WrongStride);
+    s[0] = stride[0]; s[1] = stride.size() > 1 ? stride[1] : stride[0];  // as conv_lean, op_convolution.zig:68-69
+    for (int i = 0; i < 4; ++i) p[i] = 0;
+    if (pads) {
+        if (pads->size() < 4) throw Error(ZANT_InvalidPadding);
+        for (int i = 0; i < 4; ++i) p[i] = (*pads)[size_t(i)];
+    }
+    d[0] = d[1] = 1;
+    if (dilations && !dilations->empty()) { d[0] = (*dilations)[0]; d[1] = dilations->size() > 1 ? (*dilations)[1] : d[0]; }
+}
+}  // namespace detail
+
+// qlinearconv_lean: ONNX input order (x, x_scale, x_zero_point, w, w_scale, w_zero_point, y_scale, y_zero_point, B), then
+// conv_lean's attributes.  The activation scales / zero points are per-tensor scalars (host values); w_scale holds one
+// element or one per output channel; pads are [top, left, bottom, right]; group == channels is a depthwise convolution.
+inline void qlinearconv_lean(Tensor<uint8_t> *x, float x_scale, uint8_t x_zero_point, Tensor<int8_t> *w,
+                             Tensor<float> *w_scale, Tensor<int8_t> *w_zero_point, float y_scale, uint8_t y_zero_point,
+                             const Tensor<int32_t> *bias, Tensor<uint8_t> *y, const Dims &stride, const Dims *pads,
+                             const Dims *dilations, std::optional<int64_t> group) {
+    if (x->shape.size() != 4 || w->shape.size() != 4 || y->shape.size() != 4) throw Error(ZANT_InvalidDimensions);
+    int64_t s[2], p[4], d[2];
+    detail::qconv_attrs(stride, pads, dilations, s, p, d);
+    check(zant_hip_qlinearconv_u8i8(default_ctx(), x->data, x->shape.data(), x_scale, x_zero_point, w->data, w->shape.data(),
+                                    w_scale->data, int64_t(w_scale->size), w_zero_point ? w_zero_point->data : nullptr, y_scale,
+                                    y_zero_point, bias ? bias->data : nullptr, y->data, y->shape.data(), s, p, d,
+                                    group ? *group : 1, ZANT_ACT_NONE, 0.0f, 1.0f, 0));
+}
+inline Tensor<uint8_t> qlinearconv(Tensor<uint8_t> *x, float x_scale, uint8_t x_zero_point, Tensor<int8_t> *w,
+                                   Tensor<float> *w_scale, Tensor<int8_t> *w_zero_point, float y_scale, uint8_t y_zero_point,
+                                   const Tensor<int32_t> *bias, const Dims &stride, const Dims *pads, const Dims *dilations,
+                                   std::optional<int64_t> group) {
+    if (x->shape.size() != 4 || w->shape.size() != 4) throw Error(ZANT_InvalidDimensions);
+    int64_t s[2], p[4], d[2];
+    detail::qconv_attrs(stride, pads, dilations, s, p, d);
+    if (s[0] <= 0 || s[1] <= 0) throw Error(ZANT_WrongStride);
+    const int64_t dkh = (w->shape[2] - 1) * d[0] + 1, dkw = (w->shape[3] - 1) * d[1] + 1;
+    Tensor<uint8_t> y = Tensor<uint8_t>::fromShape({x->shape[0], w->shape[0], (x->shape[2] + p[0] + p[2] - dkh) / s[0] + 1,
+                                                    (x->shape[3] + p[1] + p[3] - dkw) / s[1] + 1});
+    qlinearconv_lean(x, x_scale, x_zero_point, w, w_scale, w_zero_point, y_scale, y_zero_point, bias, &y, stride, pads, dilations, group);
+    return y;
+}
+
+// Prepared weights for qlinearconv_lean (zant_hip_qlinearconv_prepack): everything weight-dependent is derived at the
+// first run and kept; activations are NCHW or, between two prepared convolutions, channel-blocked.
+class QLinearConvPlan {
+  public:
+    QLinearConvPlan(const Dims &xshape, float x_scale, uint8_t x_zero_point, Tensor<int8_t> *w, Tensor<float> *w_scale,
+                    Tensor<int8_t> *w_zero_point, float y_scale, uint8_t y_zero_point, const Tensor<int32_t> *bias,
+                    const Dims &yshape, const Dims &stride, const Dims *pads, const Dims *dilations, std::optional<int64_t> group,
+                    int x_layout = ZANT_LAYOUT_NCHW, int y_layout = ZANT_LAYOUT_NCHW) {
+        if (xshape.size() != 4 || w->shape.size() != 4 || yshape.size() != 4) throw Error(ZANT_InvalidDimensions);
+        int64_t s[2], p[4], d[2];
+        detail::qconv_attrs(stride, pads, dilations, s, p, d);
+        check(zant_hip_qlinearconv_prepack(default_ctx(), xshape.data(), x_scale, x_zero_point, w->data, w->shape.data(),
+                                           w_scale->data, int64_t(w_scale->size), w_zero_point ? w_zero_point->data : nullptr,
+                                           y_scale, y_zero_point, bias ? bias->data : nullptr, yshape.data(), s, p, d,
+                                           group ? *group : 1, ZANT_ACT_NONE, 0.0f, 1.0f, 0, x_layout, y_layout, &plan_));
+    }
+    QLinearConvPlan(const QLinearConvPlan &) = delete;
+    QLinearConvPlan &operator=(const QLinearConvPlan &) = delete;
+    ~QLinearConvPlan() { zant_hip_qlinearconv_plan_destroy(default_ctx(), plan_); }
+    void run(const uint8_t *x, uint8_t *y) { check(zant_hip_qlinearconv_u8i8_packed(default_ctx(), plan_, x, y)); }
+
+  private:
+    zant_qconv_plan *plan_ = nullptr;
+};
+
+// Prepared weights for conv_lean (zant_hip_conv2d_f32_prepack), same attributes.
+class ConvPlan {
+  public:
+    ConvPlan(const Dims &xshape, Tensor<float> *kernel, const Tensor<float> *bias, const Dims &yshape, const Dims &stride,
+             const Dims *pads, const Dims *dilations, std::optional<int64_t> group, const char *auto_pad) {
+        if (xshape.size() != 4 || kernel->shape.size() != 4 || yshape.size() != 4) throw Error(ZANT_InvalidDimensions);
+        check(zant_hip_conv2d_f32_prepack(default_ctx(), xshape.data(), kernel->data, kernel->shape.data(),
+                                          bias ? bias->data : nullptr, yshape.data(), stride.data(), int(stride.size()),
+                                          pads ? pads->data() : nullptr, pads ? int(pads->size()) : 0,
+                                          dilations ? dilations->data() : nullptr, dilations ? int(dilations->size()) : 0,
+                                          group ? *group : -1, auto_pad, ZANT_ACT_NONE, &plan_));
+    }
+    ConvPlan(const ConvPlan &) = delete;
+    ConvPlan &operator=(const ConvPlan &) = delete;
+    ~ConvPlan() { zant_hip_conv2d_plan_destroy(default_ctx(), plan_); }
+    void run(const float *x, float *y) { check(zant_hip_conv2d_f32_packed(default_ctx(), plan_, x, y)); }
+
+  private:
+    zant_conv_plan *plan_ = nullptr;
+};
+
 }  // namespace tensMath
 }  // namespace zant

@@ -83,6 +83,36 @@ def conv_lean_static(x, w, y, bias, stride, pads=None, dilations=None, group=Non
     return y
 
 
+class ConvPlan:
+    """Prepared weights for conv_lean (zant_hip_conv2d_f32_prepack): shapes, attributes and the weight tensors are fixed
+    once; the first call packs the weights into memory the plan owns, later calls launch the convolution only."""
+
+    def __init__(self, xshape, w, bias, yshape, stride, pads=None, dilations=None, group=None, auto_pad=None, fuse_act=None):
+        self.ctx = context()
+        self.w, self.bias, self.yshape = w, bias, tuple(yshape)  # the plan borrows the device tensors: keep them alive
+        xd, _ = dims(xshape); wd, _ = dims(w.shape); yd, _ = dims(yshape)
+        s, ns = dims(stride); p, npd = dims(pads); d, nd = dims(dilations)
+        h = C.c_void_p()
+        self.ctx.check(lib.zant_hip_conv2d_f32_prepack(self.ctx.handle, xd, _p(w), wd, _p(bias), yd, s, ns, p, npd, d, nd,
+                                                       _grp(group), _enc(auto_pad), ACT[fuse_act], C.byref(h)))
+        self.handle = h
+
+    def __call__(self, x, y):
+        self.ctx.check(lib.zant_hip_conv2d_f32_packed(self.ctx.handle, self.handle, _p(x), _p(y)))
+        return y
+
+    def close(self):
+        if self.handle and self.ctx.handle:
+            lib.zant_hip_conv2d_plan_destroy(self.ctx.handle, self.handle)
+        self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 def Conv(x, w, bias, stride, pads=None, dilations=None, group=None, auto_pad=None):
     """OnnxConv (op_convolution.zig:647): allocate the expected shape (zero filled), then conv_lean."""
     if x.dim() != 4 or w.dim() != 4:
@@ -442,6 +472,68 @@ def qlinearconv(x, x_scale, x_zp, w, w_scale, w_zp, y_scale, y_zp, bias, stride,
     y = torch.zeros(qconv_out_shape(x.shape, w.shape, stride, pads, dilations), dtype=torch.uint8, device=x.device)
     return qlinearconv_lean(x, x_scale, x_zp, w, w_scale, w_zp, y_scale, y_zp, bias, y, stride, pads, dilations, group,
                             act, act_alpha, act_scale, act_zp)
+
+
+NCHW, BLOCKED16 = 0, 1  # enum zant_layout
+
+
+def blocked16_bytes(shape):
+    d, _ = dims(shape)
+    return int(lib.zant_hip_blocked16_bytes(d))
+
+
+def to_blocked16(x):
+    """NCHW u8 -> the channel-blocked layout of the int8 matrix-core kernels (a flat byte tensor)."""
+    ctx = context()
+    d, _ = dims(x.shape)
+    xb = torch.empty(blocked16_bytes(x.shape), dtype=torch.uint8, device=x.device)
+    ctx.check(lib.zant_hip_to_blocked16_u8(ctx.handle, _p(x), d, _p(xb)))
+    return xb
+
+
+def from_blocked16(xb, shape):
+    ctx = context()
+    d, _ = dims(shape)
+    y = torch.empty(tuple(shape), dtype=torch.uint8, device=xb.device)
+    ctx.check(lib.zant_hip_from_blocked16_u8(ctx.handle, _p(xb), d, _p(y)))
+    return y
+
+
+class QConvPlan:
+    """Prepared weights for qlinearconv_lean (zant_hip_qlinearconv_prepack).  x_layout / y_layout: NCHW or BLOCKED16."""
+
+    def __init__(self, xshape, x_scale, x_zp, w, w_scale, w_zp, y_scale, y_zp, bias, stride, pads, dilations, group=1,
+                 act=None, act_alpha=0.0, act_scale=1.0, act_zp=0, x_layout=NCHW, y_layout=NCHW):
+        self.ctx = context()
+        self.keep = (w, w_scale, w_zp, bias)  # the plan borrows the device tensors: keep them alive
+        self.yshape = qconv_out_shape(xshape, w.shape, stride, pads, dilations)
+        xd, _ = dims(xshape); wd, _ = dims(w.shape); yd, _ = dims(self.yshape)
+        s, _ = dims(stride); p, _ = dims(pads); d, _ = dims(dilations)
+        h = C.c_void_p()
+        self.ctx.check(lib.zant_hip_qlinearconv_prepack(self.ctx.handle, xd, x_scale, x_zp, _p(w), wd, _p(w_scale),
+                                                        w_scale.numel(), _p(w_zp), y_scale, y_zp, _p(bias), yd, s, p, d,
+                                                        group, ACT[act], act_alpha, act_scale, act_zp, x_layout, y_layout,
+                                                        C.byref(h)))
+        self.handle = h
+        self.y_layout = y_layout
+
+    def __call__(self, x, y=None):
+        if y is None:
+            y = (torch.empty(blocked16_bytes(self.yshape), dtype=torch.uint8, device=x.device) if self.y_layout == BLOCKED16
+                 else torch.zeros(self.yshape, dtype=torch.uint8, device=x.device))
+        self.ctx.check(lib.zant_hip_qlinearconv_u8i8_packed(self.ctx.handle, self.handle, _p(x), _p(y)))
+        return y
+
+    def close(self):
+        if self.handle and self.ctx.handle:
+            lib.zant_hip_qlinearconv_plan_destroy(self.ctx.handle, self.handle)
+        self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 def qlinear_act(x, x_scale, x_zp, act, alpha, y_scale, y_zp):
