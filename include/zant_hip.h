@@ -409,7 +409,9 @@ const char *zant_model_launch_name(zant_model *m, int i);
 /* The device function behind entry i of the last zant_model_profile (see zant_hip_kernel_name); "" before it. */
 const char *zant_model_launch_kernel(zant_model *m, int i);
 /* Debug: copies tensor `id` to the host: replays the last pass up to the node that produces it (its storage may have
- * been planned under a later tensor), then reads it from the arena.  Tensors that a fusion removed (the
+ * been planned under a later tensor), reads it from the arena, then replays the rest of the pass, so that afterwards
+ * the arena -- zant_model_output_ptr() included -- holds the last pass's result again.  It costs a whole pass and, like
+ * a pass, overwrites the per-kernel figures of an earlier zant_model_profile.  Tensors that a fusion removed (the
  * output of a convolution whose pool, or of a residual block's inner layers, run in the same kernel) are never
  * materialised: ZANT_InvalidInput. */
 int zant_model_read_tensor(zant_model *m, int id, void *dst_host, size_t bytes);

@@ -208,3 +208,52 @@ def test_input_survives_repeated_passes(G):
     for n in (0, 31, 63):
         np.testing.assert_allclose(outs[2][n], oracle_readme_cnn(x[n:n + 1], params).ravel(), rtol=G.RTOL, atol=G.ATOL)
     m.close()
+
+
+def _conv_bn_model(G, N, C, K, H, gamma, beta, mean, var, eps, seed=0):
+    from zant_amd.model import Model
+    g = np.random.default_rng(seed)
+    x = g.standard_normal((N, C, H, H)).astype(np.float32)
+    w = (g.standard_normal((K, C, 3, 3)) * np.sqrt(2 / (9 * C))).astype(np.float32)
+    b = (g.standard_normal(K) * 0.1).astype(np.float32)
+    m = Model(G.tm.context())
+    t = m.conv(m.input((N, C, H, H)), w, b, [1, 1], [1, 1, 1, 1], [1, 1], 1, "NOTSET")
+    m.batchnorm(t, gamma, beta, mean, var, eps)
+    m.finalize()
+    ref = zo.batchnorm(zo.Conv(x, w, b, [1, 1], [1, 1, 1, 1], [1, 1], 1, "NOTSET"), gamma, beta, mean, var, eps)
+    return m, x, ref
+
+
+def test_conv_batchnorm_fold_is_bounded_against_the_oracle(G):
+    """Moderate scales are folded into the convolution (one launch); the folded result stays inside the tolerance of the
+    path against the oracle's order of operations, also with a small variance and a large gamma."""
+    K = 16
+    g = np.random.default_rng(1)
+    gamma = g.uniform(0.5, 40.0, K).astype(np.float32)
+    var = g.uniform(2e-3, 1.0, K).astype(np.float32)       # s up to 40 / sqrt(2e-3) ~ 900
+    beta, mean = g.standard_normal(K).astype(np.float32), g.standard_normal(K).astype(np.float32)
+    m, x, ref = _conv_bn_model(G, 3, 8, K, 10, gamma, beta, mean, var, 1e-5)
+    assert m.num_launches == 1
+    np.testing.assert_allclose(m.predict_host(x), ref, rtol=G.RTOL, atol=G.ATOL * float(np.abs(ref).max()))
+    m.close()
+
+
+def test_conv_batchnorm_is_not_folded_for_extreme_or_non_finite_scales(G):
+    K = 8
+    ones, zeros = np.ones(K, np.float32), np.zeros(K, np.float32)
+    # gamma / sqrt(var + eps) = 1e6: beyond the bound, the normalisation stays its own kernel and matches the oracle
+    var = np.full(K, 1e-12, np.float32)
+    m, x, ref = _conv_bn_model(G, 2, 4, K, 8, ones, zeros, zeros, var, 0.0)
+    assert m.num_launches == 2
+    np.testing.assert_allclose(m.predict_host(x), ref, rtol=G.RTOL, atol=G.ATOL * float(np.abs(ref).max()))
+    m.close()
+    # var + eps < 0 in one channel: sqrt gives NaN there -- in that channel's outputs only, as the operator defines it
+    var = np.ones(K, np.float32)
+    var[3] = -1.0
+    m, x, ref = _conv_bn_model(G, 2, 4, K, 8, ones, zeros, zeros, var, 1e-5)
+    assert m.num_launches == 2
+    y = m.predict_host(x)
+    assert np.isnan(y[:, 3]).all() and np.isnan(ref[:, 3]).all()
+    keep = [k for k in range(K) if k != 3]
+    np.testing.assert_allclose(y[:, keep], ref[:, keep], rtol=G.RTOL, atol=G.ATOL)
+    m.close()

@@ -37,6 +37,37 @@ def _both(x, wt, b, act):
     return host(y_ws), host(y_st)
 
 
+def _static_on_a_fresh_context(x, wt, b, act):
+    """The static entry point as the FIRST operator call of a new context: its workspace is still empty, so a path
+    that took its scratch from the workspace (or allocated anything else) would have to call hipMalloc here, and the
+    device's free memory would drop."""
+    from zant_amd.capi import Context, dims
+    X, W, B = dev(x), dev(wt), dev(b)
+    shape = tm.get_convolution_output_shape(x.shape, wt.shape, [1, 1], [1, 1, 1, 1], [1, 1], "NOTSET")
+    y = torch.full(shape, float("nan"), dtype=torch.float32, device="cuda:0")
+    ctx = Context()
+    xd, _ = dims(x.shape); wd, _ = dims(wt.shape); yd, _ = dims(shape)
+    s, ns = dims([1, 1]); p, npd = dims([1, 1, 1, 1]); d, nd = dims([1, 1])
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    ctx.check(za.lib.zant_hip_conv2d_f32_static(ctx.handle, X.data_ptr(), xd, W.data_ptr(), wd, B.data_ptr(), y.data_ptr(), yd,
+                                                s, ns, p, npd, d, nd, 1, b"NOTSET", tm.ACT[act]))
+    ctx.sync()
+    free1 = torch.cuda.mem_get_info()[0]
+    ctx.close()
+    assert free1 == free0, "the static entry point allocated device memory on a context that had none"
+    return host(y)
+
+
+def test_static_entry_point_allocates_nothing_on_a_fresh_context():
+    # the largest shape of this file first, before any allocating convolution has grown a workspace for it
+    x, wt, b, act = _case(1, 16, 64, 28, 28, 64, True)
+    y_fresh = _static_on_a_fresh_context(x, wt, b, act)
+    y_ws, y_st = _both(x, wt, b, act)
+    np.testing.assert_array_equal(y_fresh, y_ws)
+    np.testing.assert_array_equal(y_st, y_ws)
+
+
 def test_static_entry_point_two_calls_in_a_row_second_one_smaller():
     # first a large convolution (tiled kernel, many tiles, packed weights of 64 x 64 x 9), then a smaller one that
     # leaves most of the scratch array holding the first call's contents

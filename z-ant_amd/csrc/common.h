@@ -44,6 +44,12 @@ int zant_fail_hip(zant_ctx *ctx, hipError_t e, const char *what);
 // Checks the launch that was just enqueued.
 #define ZANT_LAUNCH_CHECK(ctx) ZANT_HIP_TRY(ctx, hipGetLastError())
 
+// Opts `kernel` into `bytes` of dynamic LDS (more than 64 KB has to be asked for) on the context's device.  Done once per
+// (kernel, device) under a lock; a failure is not cached, is recorded on the context and leaves the HIP runtime's last
+// error set, so the launch site's ZANT_LAUNCH_CHECK reports it.  Returns false when the limit is not in place: the
+// caller then does not launch.
+bool zant_raise_lds_limit(zant_ctx *ctx, const void *kernel, int bytes);
+
 // Names the main kernel a launch site is about to enqueue (what a profiler's kernel trace shows for it).
 #define ZANT_KERNEL_NAME(ctx, ...) snprintf((ctx)->last_kernel, sizeof((ctx)->last_kernel), __VA_ARGS__)
 

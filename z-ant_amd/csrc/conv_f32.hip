@@ -817,12 +817,7 @@ void launch_mfma_tt(zant_ctx *ctx, const float *x, const float *wp, const float 
                     const MfmaPlan &p, int relu, int *counter, int grid, int parity) {
     constexpr int KV = MT >= 8 ? 2 : 4;  // 64-bit operand reads keep 8 accumulator tiles inside 256 VGPRs
     // more than 64 KB of dynamic LDS has to be opted into once per kernel
-    static bool attr_set = false;
-    if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&conv_f32_mfma_kernel<MT, WM, WN, KV, TT, POOL>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        attr_set = true;
-    }
+    if (!zant_raise_lds_limit(ctx, reinterpret_cast<const void *>(&conv_f32_mfma_kernel<MT, WM, WN, KV, TT, POOL>), 160 * 1024)) return;
     ZANT_KERNEL_NAME(ctx, "conv_f32_mfma_kernel<%d,%d,%d,%d,%d,%s>", MT, WM, WN, KV, TT, POOL ? "true" : "false");
     hipLaunchKernelGGL((conv_f32_mfma_kernel<MT, WM, WN, KV, TT, POOL>), dim3(grid), dim3(WM * WN * 64), p.lds_bytes + bias_lds_bytes(g),
                        ctx->stream, x, wp, bias, y, g, p.t, relu, counter, parity);

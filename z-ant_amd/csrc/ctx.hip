@@ -1,4 +1,8 @@
 // Context, arena, transfers, timing and status names of libzant_hip.so.
+#include <map>
+#include <mutex>
+#include <utility>
+
 #include "common.h"
 
 void (*g_zant_log)(char *) = nullptr;
@@ -21,6 +25,21 @@ int zant_fail_hip(zant_ctx *ctx, hipError_t e, const char *what) {
         zant_log(ctx->last_error.c_str());
     }
     return ZANT_HipError;
+}
+
+bool zant_raise_lds_limit(zant_ctx *ctx, const void *kernel, int bytes) {
+    static std::mutex lock;
+    static std::map<std::pair<const void *, int>, int> raised;  // (kernel, device) -> bytes granted so far
+    std::lock_guard<std::mutex> guard(lock);
+    int &have = raised[{kernel, ctx->device}];
+    if (have >= bytes) return true;
+    const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) {
+        (void)zant_fail_hip(ctx, e, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+        return false;
+    }
+    have = bytes;
+    return true;
 }
 
 int zant_workspace(zant_ctx *ctx, size_t bytes, void **out) {

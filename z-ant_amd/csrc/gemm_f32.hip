@@ -546,11 +546,7 @@ void launch_gemm_dma(zant_ctx *ctx, const float *A, const float *B, const float 
     constexpr int BM = WM * MT * 32, BN = WN * 32;
     constexpr size_t lds_bytes = size_t(S) * (BM + BN) * BK * sizeof(float);
     auto kern = &gemm_f32_dma_kernel<MT, WM, WN, AM, BMODE, S>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
-        attr_set = true;
-    }
+    if (!zant_raise_lds_limit(ctx, reinterpret_cast<const void *>(kern), int(lds_bytes))) return;
     const unsigned blocks = unsigned(((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN));
     ZANT_KERNEL_NAME(ctx, "gemm_f32_dma_kernel<%d,%d,%d,%d,%d,%d>", MT, WM, WN, AM, BMODE, S);
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(WM * WN * 64), lds_bytes, ctx->stream, A, B, C, Y, g);

@@ -729,16 +729,30 @@ extern "C" int zant_model_finalize(zant_model *m) {
                 const float *be = reinterpret_cast<const float *>(m->p[bn.b].host.data());
                 const float *mu = reinterpret_cast<const float *>(m->p[bn.c].host.data());
                 const float *va = reinterpret_cast<const float *>(m->p[bn.ws].host.data());
-                std::vector<float> bias(size_t(K), 0.0f);
-                if (nd.b >= 0) memcpy(bias.data(), m->p[nd.b].host.data(), size_t(K) * 4);
+                // The fold replaces the reference's order of operations ((x - mean) / sqrt(var + eps) * gamma + beta,
+                // batchNormLayer.zig:143-145) by one scale folded into the weights: the two differ by rounding errors that
+                // grow with |s|, and a non-finite s (var + eps <= 0, overflow) would poison every weight of the channel
+                // where the operator itself yields NaN / inf only where the reference does.  So the fold is taken only when
+                // every channel's scale is finite and moderate; otherwise the normalisation stays a node of its own.
+                std::vector<float> scale(static_cast<size_t>(K));
+                bool foldable = true;
                 for (int64_t k = 0; k < K; ++k) {
                     const float sc = ga[k] / sqrtf(va[k] + bn.alpha);
-                    for (int64_t e = 0; e < per_k; ++e) w[k * per_k + e] *= sc;
-                    bias[size_t(k)] = (bias[size_t(k)] - mu[k]) * sc + be[k];
+                    scale[size_t(k)] = sc;
+                    if (!std::isfinite(sc) || fabsf(sc) > 1024.0f || (sc != 0.0f && fabsf(sc) < 1.0f / 1024.0f)) foldable = false;
                 }
-                nd.b = add_param(m, bias.data(), size_t(K) * 4);  // (a bias shared with another node keeps its own copy)
-                m->t[bn.out].alias_of = out;
-                bn.skip = true;
+                if (foldable) {
+                    std::vector<float> bias(size_t(K), 0.0f);
+                    if (nd.b >= 0) memcpy(bias.data(), m->p[nd.b].host.data(), size_t(K) * 4);
+                    for (int64_t k = 0; k < K; ++k) {
+                        const float sc = scale[size_t(k)];
+                        for (int64_t e = 0; e < per_k; ++e) w[k * per_k + e] *= sc;
+                        bias[size_t(k)] = (bias[size_t(k)] - mu[k]) * sc + be[k];
+                    }
+                    nd.b = add_param(m, bias.data(), size_t(K) * 4);  // (a bias shared with another node keeps its own copy)
+                    m->t[bn.out].alias_of = out;
+                    bn.skip = true;
+                }
             }
         }
         if ((nd.op == OP_CONV || nd.op == OP_GEMM) && nd.fuse_act == ZANT_ACT_NONE) {
@@ -1321,37 +1335,45 @@ extern "C" int zant_model_read_tensor(zant_model *m, int id, void *dst_host, siz
     if (m->t[root_of(m, id)].def < 0) return ZANT_InvalidInput;  // fused away: the tensor is never materialised
     const MTensor &t = m->t[id];
     // A later node may have been planned over this tensor's storage once its last reader was done, so the pass is
-    // replayed up to the node that produces it (the input still sits in its slot: a pass never writes there).
-    {
-        const int root = root_of(m, id);
-        int last_writer = -1;
-        for (int i = 0; i < int(m->n.size()); ++i)
-            if (!m->n[i].skip && root_of(m, m->n[i].out) == root) last_writer = i;
-        for (int i = 0; i <= last_writer; ++i) {
-            if (m->n[i].skip) continue;
-            const int rc = run_node(m, m->n[i]);
-            if (rc) return rc;
-        }
+    // replayed up to the node that produces it (the input still sits in its slot: a pass never writes there), the tensor
+    // is copied out, and the rest of the pass is replayed so that the arena -- the output at zant_model_output_ptr()
+    // included -- again holds what the last zant_model_run left.
+    const int root = root_of(m, id);
+    int last_writer = -1;
+    for (int i = 0; i < int(m->n.size()); ++i)
+        if (!m->n[i].skip && root_of(m, m->n[i].out) == root) last_writer = i;
+    for (int i = 0; i <= last_writer; ++i) {
+        if (m->n[i].skip) continue;
+        const int rc = run_node(m, m->n[i]);
+        if (rc) return rc;
     }
-    if (m->t[root_of(m, id)].layout == ZANT_LAYOUT_BLOCKED16) {  // hand out NCHW u8 like everywhere outside the executor
+    int rc;
+    if (m->t[root].layout == ZANT_LAYOUT_BLOCKED16) {  // hand out NCHW u8 like everywhere outside the executor
         void *ws = nullptr;
-        int rc = zant_workspace(m->ctx, t.bytes(), &ws);
+        rc = zant_workspace(m->ctx, t.bytes(), &ws);
         if (rc) return rc;
         rc = zant_from_blocked(m->ctx, static_cast<const uint8_t *>(tensor_ptr(m, id)), t.dim[0], t.dim[1], t.dim[2] * t.dim[3],
                                static_cast<uint8_t *>(ws));
         if (rc) return rc;
-        return zant_hip_download(m->ctx, dst_host, ws, bytes);
-    }
-    if (m->t[root_of(m, id)].layout == ZANT_LAYOUT_C4) {  // likewise NCHW f32
+        rc = zant_hip_download(m->ctx, dst_host, ws, bytes);
+    } else if (m->t[root].layout == ZANT_LAYOUT_C4) {  // likewise NCHW f32
         void *ws = nullptr;
-        int rc = zant_workspace(m->ctx, t.bytes(), &ws);
+        rc = zant_workspace(m->ctx, t.bytes(), &ws);
         if (rc) return rc;
         rc = zant_from_c4_f32(m->ctx, static_cast<const float *>(tensor_ptr(m, id)), t.dim[0], t.dim[1], t.dim[2] * t.dim[3],
                               static_cast<float *>(ws));
         if (rc) return rc;
-        return zant_hip_download(m->ctx, dst_host, ws, bytes);
+        rc = zant_hip_download(m->ctx, dst_host, ws, bytes);
+    } else {
+        rc = zant_hip_download(m->ctx, dst_host, tensor_ptr(m, id), bytes);
     }
-    return zant_hip_download(m->ctx, dst_host, tensor_ptr(m, id), bytes);
+    if (rc) return rc;
+    for (int i = last_writer + 1; i < int(m->n.size()); ++i) {
+        if (m->n[i].skip) continue;
+        rc = run_node(m, m->n[i]);
+        if (rc) return rc;
+    }
+    return ZANT_OK;
 }
 
 extern "C" int zant_model_bind_predict(zant_model *m) {

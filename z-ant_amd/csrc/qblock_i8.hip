@@ -628,12 +628,7 @@ int zant_qblock_blocked(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], 
     const int MQv = a.split ? nq_tiles : std::max(1, (q_per_wave + rounds - 1) / rounds);
 #define ZANT_QBLOCK_LAUNCH(CO, M, P, S)                                                                                          \
     do {                                                                                                                    \
-        static bool attr_set = false;                                                                                       \
-        if (!attr_set) {                                                                                                    \
-            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&qblock_kernel<CO, M, P, S>),                               \
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                             \
-            attr_set = true;                                                                                                \
-        }                                                                                                                   \
+        if (!zant_raise_lds_limit(ctx, reinterpret_cast<const void *>(&qblock_kernel<CO, M, P, S>), 160 * 1024)) break;         \
         ZANT_KERNEL_NAME(ctx, "qblock_kernel<%d,%d,%s,%s>", CO, M, P ? "true" : "false", S ? "true" : "false");                                          \
         hipLaunchKernelGGL((qblock_kernel<CO, M, P, S>), dim3(grid), dim3(256), cap_used, ctx->stream,                           \
                            reinterpret_cast<const uint4 *>(x), y, reinterpret_cast<const uint4 *>(base + o_w1p), a);       \

@@ -645,12 +645,7 @@ template <int MT, int WM, int WN, int TT, bool POOL = false>
 void launch_qmfma_tt(zant_ctx *ctx, const int8_t *xb, const int8_t *wp, const float *mult, const int32_t *corr,
                      const int8_t *padvec, uint8_t *y, const ConvGeom &g, const TilePlan &p, int CB, const QConvArgs &q,
                      int grid, int yb, int n_stages) {
-    static bool attr_set = false;
-    if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&qconv_mfma_kernel<MT, WM, WN, TT, POOL>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        attr_set = true;
-    }
+    if (!zant_raise_lds_limit(ctx, reinterpret_cast<const void *>(&qconv_mfma_kernel<MT, WM, WN, TT, POOL>), 160 * 1024)) return;
     ZANT_KERNEL_NAME(ctx, "qconv_mfma_kernel<%d,%d,%d,%d,%s>", MT, WM, WN, TT, POOL ? "true" : "false");
     hipLaunchKernelGGL((qconv_mfma_kernel<MT, WM, WN, TT, POOL>), dim3(grid), dim3(WM * WN * 64), p.lds_bytes, ctx->stream, xb,
                        wp, mult, corr, padvec, y, g, p.t, CB, q, n_stages, yb);

@@ -750,12 +750,8 @@ bool ps_plan(const ConvGeom &g, int num_cus, PsGeom *out, size_t *lds_bytes, int
 template <int MT, int OUT>
 void ps_launch_out(zant_ctx *ctx, int grid, size_t lds, const int8_t *xb, const int8_t *wp, const char *tabs,
                    const int8_t *padvec, uint8_t *y, const PsGeom &p, const QConvArgs &q) {
-    static bool attr_set = false;
-    if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&qconv_ps_kernel<MT, OUT>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        attr_set = true;
-    }
+    // (the kernel has no static LDS: the whole 160 KB of a compute unit may be asked for as dynamic LDS)
+    if (!zant_raise_lds_limit(ctx, reinterpret_cast<const void *>(&qconv_ps_kernel<MT, OUT>), 160 * 1024)) return;
     ZANT_KERNEL_NAME(ctx, "qconv_ps_kernel<%d,%d>", MT, OUT);
     hipLaunchKernelGGL((qconv_ps_kernel<MT, OUT>), dim3(grid), dim3(PS_NT), lds, ctx->stream, xb, wp, tabs, padvec, y, p, q);
 }
