@@ -326,3 +326,46 @@ def test_full_size_conv_properties(G):
     xs = x[100:102].contiguous()
     ref = zo.Conv(G.host(xs), G.host(w1), None, *args)
     np.testing.assert_allclose(G.host(y1[100:102]), ref, rtol=G.RTOL, atol=G.ATOL)
+
+
+# The staged Gemm kernel has one instantiation per (A copy mode, B copy mode); which one runs follows from the
+# transposition flags, the row lengths and the alignment of the operands.  Modes: 0 = k-contiguous 16-byte copies,
+# 1 = k-contiguous 4-byte copies, 2 = 4-byte copies of the other orientation, 3 (B only) = B stored [K][N] with N a multiple
+# of 4 copied as it lies, the lane gathering its four k with two hand-issued LDS reads.  Every instantiation that takes that
+# last mode is run here with K tails (K not a multiple of the 32-k chunk, K below one chunk), ragged M and N tiles, and
+# the fall-back to 4-byte copies when B is not 16-byte aligned.
+GEMM_MODE_CASES = [
+    # M, K, N, transA, misalign A, misalign B -> expected (A mode, B mode)
+    (300, 100, 64, 0, 0, 0, (0, 3)),     # aligned row-major A, K tail of 4
+    (300, 37, 36, 0, 0, 0, (1, 3)),      # K = 37: A rows are not whole 16-byte units; ragged N tile
+    (129, 1600, 512, 0, 0, 0, (0, 3)),   # the README CNN's first Gemm with a ragged M tile
+    (64, 24, 40, 0, 0, 0, (0, 3)),       # K below one chunk
+    (200, 96, 48, 1, 0, 0, (2, 3)),      # transposed A
+    (70, 33, 68, 1, 0, 0, (2, 3)),       # transposed A, K tail of 1
+    (300, 100, 64, 0, 0, 1, (0, 2)),     # B off the 16-byte grid: falls back to 4-byte copies
+    (300, 100, 64, 0, 1, 0, (1, 3)),     # A off the grid
+    (90, 64, 50, 0, 0, 0, (0, 2)),       # N not a multiple of 4
+]
+
+
+@pytest.mark.parametrize("M,K,N,ta,mis_a,mis_b,modes", GEMM_MODE_CASES)
+def test_gemm_copy_modes_vs_oracle(G, M, K, N, ta, mis_a, mis_b, modes):
+    import torch
+    g = np.random.default_rng(M + 3 * K + 5 * N + ta)
+    a = g.standard_normal((1, 1, K, M) if ta else (1, 1, M, K), dtype=np.float32)
+    b = (g.standard_normal((1, 1, K, N)) * np.sqrt(2.0 / K)).astype(np.float32)
+    c = (g.standard_normal((1, 1, 1, N)) * 0.1).astype(np.float32)
+
+    def place(arr, misalign):  # a device copy that starts 4 bytes past a 16-byte boundary when asked
+        flat = torch.zeros(arr.size + 4, dtype=torch.float32, device="cuda:0")
+        view = flat[1:1 + arr.size] if misalign else flat[:arr.size]
+        view.copy_(torch.from_numpy(arr.ravel()))
+        return view.view(arr.shape)
+
+    A, B = place(a, mis_a), place(b, mis_b)
+    assert (A.data_ptr() % 16 != 0) == bool(mis_a) and (B.data_ptr() % 16 != 0) == bool(mis_b)
+    y = torch.full((1, 1, M, N), -7.0, device="cuda:0")
+    G.tm.gemm_lean(A, B, G.dev(c), 1.0, 1.0, bool(ta), False, y, "relu")
+    assert G.tm.context().kernel_name() == "gemm_f32_dma_kernel<1,4,2,%d,%d,5>" % modes
+    ref = zo.ReLU(zo.gemm(a, b, c, 1.0, 1.0, bool(ta), False))
+    np.testing.assert_allclose(G.host(y), ref, rtol=G.RTOL, atol=G.ATOL)
