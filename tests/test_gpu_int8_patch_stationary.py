@@ -108,3 +108,47 @@ def test_staged_nchw_write_out_bit_exact(G, case, act):
     pick = list(range(N)) if N <= 8 else [0, 1, N // 2, N - 2, N - 1]
     ref = zo.qlinearconv(x[pick], 0.02, 128, w, ws, None, 0.05, 128, b, [1, 1], pads, [1, 1], 1, **kw)
     np.testing.assert_array_equal(G.host(y)[pick], ref)
+
+
+# The fused 2x2/2 max pool (blocked tensors on both sides, inside a model): the pool is taken on the accumulators, one
+# value in four is requantised, and the pooled bytes are staged and written out as whole 16-byte units.
+POOL_CASES = [
+    # N, C, H, W, K                what the shape exercises
+    (6, 32, 24, 24, 64),           # one image per tile, a pass of 64 channels, several tiles per workgroup at larger N
+    (5, 64, 12, 12, 128),          # several images per tile, two channel chunks, a pass of 128 channels
+    (3, 48, 20, 28, 72),           # row tiles (TH < OH), ragged channels on both sides
+    (700, 32, 8, 8, 40),           # many tiles per workgroup: the staging rows are rewritten tile after tile
+]
+
+
+@pytest.mark.parametrize("case", POOL_CASES, ids=[str(i) for i in range(len(POOL_CASES))])
+@pytest.mark.parametrize("act", ["leaky", None])
+def test_fused_pool_bit_exact_inside_a_model(G, case, act):
+    from zant_amd.model import Model, U8
+    N, C, H, W, K = case
+    x, w, ws, b = _operands(3 * N + C + K, N, C, H, W, K)
+    g = np.random.default_rng(N)
+    w0 = g.integers(-127, 128, (C, 3, 3, 3), dtype=np.int8)   # a first layer brings the input into the blocked layout
+    ws0 = (g.uniform(0.5, 1.5, C) * 0.08 / np.sqrt(27)).astype(np.float32)
+    x0 = g.integers(0, 256, (N, 3, H, W), dtype=np.uint8)
+    m = Model(G.tm.context())
+    t = m.input((N, 3, H, W), U8, 0.02, 128)
+    t = m.qlinearconv(t, w0, ws0, None, 0.05, 128, [1, 1], [1, 1, 1, 1])
+    t = m.qlinearconv(t, w, ws, b, 0.05, 128, [1, 1], [1, 1, 1, 1])
+    if act:
+        t = m.qlinear_act(t, act, 0.1, 0.04, 30)
+    t = m.maxpool(t, [2, 2], [2, 2])
+    t = m.qlinearconv(t, np.ones((16, K, 1, 1), np.int8), np.full(16, 0.01, np.float32), None, 0.5, 0, [1, 1], [0, 0, 0, 0])
+    m.finalize()
+    m.profile()
+    assert any(k.startswith("qconv_ps_kernel<") and k.endswith(",6>") for k in m.launch_kernels()), m.launch_kernels()
+    pick = list(range(N)) if N <= 8 else [0, 1, N // 2, N - 1]
+    r = zo.qlinearconv(x0[pick], 0.02, 128, w0, ws0, None, 0.05, 128, None, [1, 1], [1, 1, 1, 1], [1, 1], 1)
+    kw = dict(act=act, act_alpha=0.1, act_scale=0.04, act_zp=30) if act else {}
+    r = zo.qlinearconv(r, 0.05, 128, w, ws, None, 0.05, 128, b, [1, 1], [1, 1, 1, 1], [1, 1], 1, **kw)
+    r = zo.onnx_maxpool(r, [2, 2], [2, 2], [1, 1], [0, 0, 0, 0])
+    s_in, zp_in = (0.04, 30) if act else (0.05, 128)
+    r = zo.qlinearconv(r, s_in, zp_in, np.ones((16, K, 1, 1), np.int8), np.full(16, 0.01, np.float32), None, 0.5, 0, None,
+                       [1, 1], [0, 0, 0, 0], [1, 1], 1)
+    np.testing.assert_array_equal(m.predict_host(x0)[pick], r)
+    m.close()

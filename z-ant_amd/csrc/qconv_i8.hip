@@ -697,9 +697,9 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
                    const ConvGeom &g0, const QConvArgs &q, bool x_blocked, bool y_blocked, zant_pack_slot *slot, bool pool = false,
                    bool plan_only = false) {
     if (g0.groups != 1 || g0.C < 5 || int64_t(g0.N) * g0.OH * g0.OW < 64) return 1;
-    if (!pool) {
+    {
         // 3x3 / stride 1 layers with at least 32 channels on both sides: the patch-stationary kernel
-        const int rc = zant_qconv_ps(ctx, x, w, w_scale, bias, y, g0, q, x_blocked, y_blocked, slot, plan_only);
+        const int rc = zant_qconv_ps(ctx, x, w, w_scale, bias, y, g0, q, x_blocked, y_blocked, slot, plan_only, pool);
         if (rc <= 0) return rc;
     }
     // A 1x1 layer over 1x1 feature maps (a classifier head behind a global pool) is a matrix product whose rows, the

@@ -52,6 +52,10 @@ struct PsGeom {
     int stage_off;              // staging region, in bytes from the weight ring's start
     int stage_alias;            // it lies over the ring, the slot table and the patch (one tile per workgroup, one pass)
     int out_unit;               // bytes per copy of the write-out: 8 or 4
+    // Fused 2x2/2 max pool (PS_OUT_POOL): a tile's positions are numbered window by window (4 consecutive positions =
+    // the members of one window), the windows in (image, pooled row, pooled column) order; OH, OW, TH are even.
+    int pool;
+    int W_pad;                  // windows of a staging row: a tile's position tiles x 8, rounded to an odd multiple of 8
 };
 
 __device__ __forceinline__ unsigned ps_lds_addr(const void *p) {
@@ -241,7 +245,8 @@ __device__ __forceinline__ void ps_mfma_step(unsigned wr, const unsigned (&xbase
 }
 
 // OUT: how the output bytes are formed and stored.
-enum { PS_OUT_NCHW_LUT = 0, PS_OUT_BLOCKED_LUT = 1, PS_OUT_BLOCKED = 2, PS_OUT_NCHW = 3, PS_OUT_NCHW_ST = 4, PS_OUT_NCHW_ST_LUT = 5 };
+enum { PS_OUT_NCHW_LUT = 0, PS_OUT_BLOCKED_LUT = 1, PS_OUT_BLOCKED = 2, PS_OUT_NCHW = 3, PS_OUT_NCHW_ST = 4, PS_OUT_NCHW_ST_LUT = 5,
+       PS_OUT_POOL = 6 };
 
 // Write-out of a staged NCHW tile: rows of the staging region (one per image and channel, `row_bytes` real bytes each)
 // go to their runs of the output planes in units of U bytes, consecutive threads on consecutive units.
@@ -269,9 +274,11 @@ template <int MT, int OUT>
 __global__ void __launch_bounds__(PS_NT)
 qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, const char *__restrict__ tabs,
                 const int8_t *__restrict__ padvec, uint8_t *__restrict__ y, PsGeom p, QConvArgs q) {
-    constexpr bool y_blocked = OUT == PS_OUT_BLOCKED_LUT || OUT == PS_OUT_BLOCKED;
-    constexpr bool use_lut = OUT == PS_OUT_BLOCKED_LUT || OUT == PS_OUT_NCHW_LUT || OUT == PS_OUT_NCHW_ST_LUT;
+    constexpr bool pooled = OUT == PS_OUT_POOL;  // blocked output of the 2x2/2 max-pooled result, through the byte table
+    constexpr bool y_blocked = OUT == PS_OUT_BLOCKED_LUT || OUT == PS_OUT_BLOCKED || pooled;
+    constexpr bool use_lut = OUT == PS_OUT_BLOCKED_LUT || OUT == PS_OUT_NCHW_LUT || OUT == PS_OUT_NCHW_ST_LUT || pooled;
     constexpr bool staged = OUT == PS_OUT_NCHW_ST || OUT == PS_OUT_NCHW_ST_LUT;
+    constexpr bool swapped = staged || pooled;  // positions are the accumulators' rows (registers), channels their lanes
     extern __shared__ __attribute__((aligned(256))) char ps_lds_raw[];
     // LDS: [256-byte activation table, 256-aligned][multipliers, corrections][weight ring: 2 slabs][slot table]
     //      [patch: 2*NC blocks x P1s x 16]
@@ -349,8 +356,21 @@ qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, co
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
             const int pp = (pt0 + i) * 32 + l32;
-            const int img = small_div(pp, per_img, inv_per_img), r2 = pp - img * per_img;
-            const int r = small_div(r2, p.OW, inv_ow), c = r2 - r * p.OW;
+            int img, r, c;
+            if constexpr (pooled) {
+                // window pp / 4 in (image, pooled row, pooled column) order, member pp % 4 = (row, column) inside it
+                const int wi = pp >> 2, per_img_w = per_img >> 2, ow2 = p.OW >> 1;
+                img = small_div(wi, per_img_w, 4.0f * inv_per_img);
+                const int r2 = wi - img * per_img_w;
+                const int wr = small_div(r2, ow2, 2.0f * inv_ow);
+                r = 2 * wr + ((pp >> 1) & 1);
+                c = 2 * (r2 - wr * ow2) + (pp & 1);
+            } else {
+                img = small_div(pp, per_img, inv_per_img);
+                const int r2 = pp - img * per_img;
+                r = small_div(r2, p.OW, inv_ow);
+                c = r2 - r * p.OW;
+            }
             const bool in_tile = i < mt && img < p.NB;
             const int lds_off = in_tile ? (img * p.PH + r) * p.PW + c : 0;
             xbase[i] = ps_lds_addr(patch) + unsigned(lh * p.P1s + lds_off) * 16u;
@@ -404,13 +424,13 @@ qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, co
                 boundary();
                 plan_copies(0);
                 // slots past this wave's tiles multiply patch entry 0; their results are dropped
-                ps_mfma_step<MT, true, staged>(wr0 + unsigned((gs & 1) * PS_RING), xbase, 0u, PW16, st, desc, xb, padvec, p, acc, last_slot);
+                ps_mfma_step<MT, true, swapped>(wr0 + unsigned((gs & 1) * PS_RING), xbase, 0u, PW16, st, desc, xb, padvec, p, acc, last_slot);
                 ++s; ++gs;
             }
             for (int c = 1; c < p.NC; ++c, ++s, ++gs) {
                 boundary();
                 plan_copies(c);
-                ps_mfma_step<MT, false, staged>(wr0 + unsigned((gs & 1) * PS_RING), xbase, unsigned(2 * c * p.P1s * 16), PW16, st, desc,
+                ps_mfma_step<MT, false, swapped>(wr0 + unsigned((gs & 1) * PS_RING), xbase, unsigned(2 * c * p.P1s * 16), PW16, st, desc,
                                         xb, padvec, p, acc, last_slot);
             }
 
@@ -429,7 +449,87 @@ qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, co
                     }
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if constexpr (staged) {
+            if constexpr (pooled) {
+                // A lane holds 16 positions of ONE channel per accumulator tuple, and registers 4g..4g+3 are the four
+                // members of one pooling window.  Requantisation and the activation are monotone in the accumulator
+                // (non-decreasing for a multiplier >= 0, non-increasing below), so the pooled byte is the requantised
+                // maximum (minimum) of the four sums: one value in four goes through the float sequence.  A 4 x 4 byte
+                // transpose across each quad of lanes (= four channels) turns a lane's four window bytes into four
+                // channel bytes of one window: a dword of the staging rows [16-channel block][window][16 bytes], which
+                // the workgroup then writes out as whole 16-byte units of the pooled blocked tensor.
+                const int ig = tile / p.n_row_tiles;
+                const int n0 = ig * p.NB, oh0 = (tile - ig * p.n_row_tiles) * p.TH;
+                const int rows_here = min(p.TH, p.OH - oh0), imgs_here = min(p.NB, p.N - n0);
+                const float zpf = float(q.y_zp);
+                char *stage = wring + p.stage_off;
+                uint32_t lq = uint32_t(lane);
+                asm volatile("" : "+v"(lq));
+                uint32_t sel1, sel2;  // sel1 = lane & 1 ? 0x03070105 : 0x06020400, sel2 = lane & 2 ? 0x03020706 : 0x05040100
+                asm volatile("v_bfe_i32 %0, %2, 0, 1\n\tv_bfe_i32 %1, %2, 1, 1\n\t"
+                             "v_and_b32 %0, 0x05050505, %0\n\tv_and_b32 %1, 0x06060606, %1\n\t"
+                             "v_xor_b32 %0, 0x06020400, %0\n\tv_xor_b32 %1, 0x05040100, %1"
+                             : "=&v"(sel1), "=&v"(sel2) : "v"(lq));
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int kk = (2 * cp + j) * 32 + l32;  // this lane's channel inside the pass
+                    uint32_t mr = ps_read_b32(mult_a + unsigned(kp * p.KP + kk) * 4u), cr = ps_read_b32(corr_a + unsigned(kp * p.KP + kk) * 4u);
+                    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(mr), "+v"(cr));
+                    const float mv = __uint_as_float(mr);
+                    const int cv = int(cr);
+                    const bool up = mv >= 0.0f;
+                    // after the transpose this lane holds window (lane & 3) of each group of four windows... of ITS quad's
+                    // four channels: the dword at [block kk / 16][window][channel (kk & 12)]
+                    char *row = stage + (((kk >> 4) * p.W_pad + pt0 * 8 + int(lq & 3) * 2 + lh) * 16 + (l32 & 12));
+#pragma unroll
+                    for (int i = 0; i < MT; ++i) {
+                        __builtin_amdgcn_sched_barrier(0);  // one position tile at a time
+                        if (i >= mt) continue;              // (wave-uniform) an empty slot's windows belong to another wave
+                        uint32_t ob[4];
+#pragma unroll
+                        for (int gq = 0; gq < 4; ++gq) {
+                            const int a0 = acc[j][i][gq * 4], a1 = acc[j][i][gq * 4 + 1], a2 = acc[j][i][gq * 4 + 2], a3 = acc[j][i][gq * 4 + 3];
+                            const int hi = max(max(a0, a1), max(a2, a3)), lo = min(min(a0, a1), min(a2, a3));
+                            const int sum = (up ? hi : lo) + cv;
+                            ob[gq] = ps_read_u8(__builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(float(sum) * mv) + zpf, 0u, lut_a));
+                        }
+                        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(ob[0]), "+v"(ob[1]), "+v"(ob[2]), "+v"(ob[3]));
+                        const uint32_t d0 = ob[0] | (ob[1] << 8) | (ob[2] << 16) | (ob[3] << 24);  // byte g: window 2g + lh... of the tile
+                        const uint32_t x1 = uint32_t(__builtin_amdgcn_update_dpp(0, int(d0), 0xB1, 0xf, 0xf, false));  // lane ^ 1
+                        const uint32_t t1 = __builtin_amdgcn_perm(x1, d0, sel1);
+                        const uint32_t x2 = uint32_t(__builtin_amdgcn_update_dpp(0, int(t1), 0x4E, 0xf, 0xf, false));  // lane ^ 2
+                        const uint32_t o4 = __builtin_amdgcn_perm(x2, t1, sel2);
+                        *reinterpret_cast<uint32_t *>(row + i * 128) = o4;
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                __builtin_amdgcn_s_waitcnt(0xC07F);
+                __builtin_amdgcn_s_barrier();
+                __builtin_amdgcn_sched_barrier(0);
+                {
+                    // write-out: 16-byte units, rows = (image, 16-channel block), a row's windows one run of the pooled plane
+                    const int ow2 = p.OW >> 1, per_img_w = (p.TH >> 1) * ow2, here_w = (rows_here >> 1) * ow2;
+                    const int kb0 = kp * (p.KP >> 4), kbh = min(p.KP >> 4, p.KB - kb0);
+                    const int n_rows = imgs_here * kbh, n_units = n_rows * here_w;
+                    const int plane_p = (p.OH >> 1) * ow2;
+                    const float inv_w = 1.0f / float(here_w), inv_kbh = 1.0f / float(kbh);
+                    const unsigned g_origin = unsigned((n0 * p.KB + kb0) * plane_p + (oh0 >> 1) * ow2);
+#pragma unroll 2
+                    for (int u = tid; u < n_units; u += PS_NT) {
+                        const int rw = small_div(u, here_w, inv_w), off = u - rw * here_w;
+                        int img = 0, kbl = rw;
+                        if (p.NB > 1) {
+                            img = small_div(rw, kbh, inv_kbh);
+                            kbl = rw - img * kbh;
+                        }
+                        const u32x4 v = *reinterpret_cast<const u32x4 *>(stage + (kbl * p.W_pad + img * per_img_w + off) * 16);
+                        __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(y) + (g_origin + unsigned((img * p.KB + kbl) * plane_p + off)));
+                    }
+                }
+                // the next pass or tile writes these rows again: not before everybody has read them
+                __builtin_amdgcn_s_waitcnt(0xC07F);
+                __builtin_amdgcn_s_barrier();
+                __builtin_amdgcn_sched_barrier(0);
+            } else if constexpr (staged) {
                 // A lane holds 16 positions of ONE channel per accumulator tuple (registers 4g..4g+3: four consecutive
                 // positions of the tile's flattened (image, row, column) order): one multiplier and one correction per
                 // lane, a dword of four positions per group with no exchange between lanes.  The dwords go to the
@@ -684,13 +784,20 @@ size_t ps_align256(size_t v) { return (v + 255) & ~size_t(255); }
 
 // Picks the tile (NB images x TH rows) with the smallest estimated time: rounds of tiles over the CUs times the MFMA
 // count of the busiest SIMD of a tile, plus a fixed cost per tile for its fill and epilogue.
-bool ps_plan(const ConvGeom &g, int num_cus, PsGeom *out, size_t *lds_bytes, int *MT) {
+bool ps_plan(const ConvGeom &g, int num_cus, bool pool, PsGeom *out, size_t *lds_bytes, int *MT) {
     if (g.groups != 1 || g.KH != 3 || g.KW != 3 || g.sh != 1 || g.sw != 1 || g.dh != 1 || g.dw != 1) return false;
-    if (g.pt > 1 || g.pl > 1 || g.C < 32 || g.K < 33) return false;
+    if (g.pt > 1 || g.pl > 1) return false;
+    if (g.C < 32 || g.K < 33) return false;
+    // with the fused pool: whole windows only, and one output-channel pass (measured against the tiled kernel on
+    // 512 x 128 x 6 x 6 -> 256 channels, two passes over 36-position images: 25.7 us here, 23.5 us there; from 16 -> 32
+    // channels at 48 x 48, half of every MFMA multiplying padding: 39 against 26; 32 -> 64 at 24 x 24 and 64 -> 128 at
+    // 12 x 12: 17.8 against 19.5 and 14.0 against 18.1)
+    if (pool && ((g.OH & 1) || (g.OW & 1) || g.K > 128)) return false;
     if (g.OH > 1023 || g.OW > 1023) return false;
     const int CB = (g.C + 15) / 16;
     if (int64_t(g.N) * CB * g.H * g.W >= (int64_t(1) << 27)) return false;  // 16-byte units addressed with 32-bit offsets
     PsGeom p{};
+    p.pool = pool ? 1 : 0;
     p.N = g.N; p.H = g.H; p.W = g.W; p.CB = CB; p.K = g.K; p.KB = (g.K + 15) / 16; p.OH = g.OH; p.OW = g.OW; p.pt = g.pt; p.pl = g.pl;
     p.NC = (g.C + 31) / 32;
     p.KP = g.K > 64 ? 128 : 64;
@@ -709,6 +816,7 @@ bool ps_plan(const ConvGeom &g, int num_cus, PsGeom *out, size_t *lds_bytes, int
     bool found = false;
     p.PW = g.OW + 2;
     auto consider = [&](int NB, int TH) {
+        if (pool && (TH & 1)) return;
         PsGeom t = p;
         t.NB = NB; t.TH = TH;
         const int S = NB * TH * g.OW;
@@ -721,7 +829,12 @@ bool ps_plan(const ConvGeom &g, int num_cus, PsGeom *out, size_t *lds_bytes, int
         // (two position slots per wave at least: the one-slot instantiation needs more registers than it has, and a
         // kernel whose LDS reads are hidden from the compiler must not spill)
         const int per_wave = std::max(2, (t.npt + NG - 1) / NG);
-        const size_t lds = fixed + size_t(per_wave) * PS_NT * 4 + size_t(2 * t.NC) * t.P1s * 16;
+        size_t lds = fixed + size_t(per_wave) * PS_NT * 4 + size_t(2 * t.NC) * t.P1s * 16;
+        if (pool) {  // the staging rows of the pooled bytes: [16-channel block of a pass][window][16], behind the patch
+            t.W_pad = (t.npt | 1) * 8;  // an odd number of position tiles: the two blocks of a store fall on different banks
+            t.stage_off = int(2 * PS_RING + size_t(per_wave) * PS_NT * 4 + size_t(2 * t.NC) * t.P1s * 16);
+            lds += size_t(t.W_pad) * t.KP;
+        }
         if (lds > cap) return;
         t.n_row_tiles = (g.OH + TH - 1) / TH;
         const int64_t nt = int64_t((g.N + NB - 1) / NB) * t.n_row_tiles;
@@ -734,7 +847,7 @@ bool ps_plan(const ConvGeom &g, int num_cus, PsGeom *out, size_t *lds_bytes, int
         for (int w = 0; w < 4; ++w) busiest_tiles = std::max(busiest_tiles, tiles_of(w / pairs) + tiles_of((w + 4) / pairs));
         const double mfma = 2.0 * busiest_tiles * t.NKP * t.NC * 9 * 32.0;
         const double rounds = double((t.n_tiles + num_cus - 1) / num_cus);
-        const double tile_cycles = mfma + 4000.0 + double(S) * p.kpad / 256.0 * 7.0;  // + fill, + epilogue VALU
+        const double tile_cycles = mfma + 4000.0 + double(S) * p.kpad / 256.0 * (pool ? 3.0 : 7.0);  // + fill, + epilogue VALU
         const double score = 1.0 / (rounds * tile_cycles);
         if (!found || score > best * 1.01) {
             best = score; found = true; *out = t; *lds_bytes = lds; *MT = per_wave;
@@ -763,6 +876,7 @@ void ps_launch(zant_ctx *ctx, int grid, size_t lds, const int8_t *xb, const int8
     else if (!yb && p.out_unit) ps_launch_out<MT, PS_OUT_NCHW_ST>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
     else if (!yb && q.has_act) ps_launch_out<MT, PS_OUT_NCHW_LUT>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
     else if (!yb) ps_launch_out<MT, PS_OUT_NCHW>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
+    else if (p.pool) ps_launch_out<MT, PS_OUT_POOL>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
     else if (q.has_act) ps_launch_out<MT, PS_OUT_BLOCKED_LUT>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
     else ps_launch_out<MT, PS_OUT_BLOCKED>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
 }
@@ -772,11 +886,15 @@ void ps_launch(zant_ctx *ctx, int grid, size_t lds, const int8_t *xb, const int8
 // The patch-stationary matrix-core path; ZANT_OK when it ran (or, with plan_only, would run), 1 when the shape is left
 // to the other kernels.
 int zant_qconv_ps(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float *w_scale, const int32_t *bias, uint8_t *y,
-                  const ConvGeom &g, const QConvArgs &q, bool x_blocked, bool y_blocked, zant_pack_slot *slot, bool plan_only) {
+                  const ConvGeom &g, const QConvArgs &q, bool x_blocked, bool y_blocked, zant_pack_slot *slot, bool plan_only,
+                  bool pool) {
     PsGeom p;
     size_t lds = 0;
     int MT = 0;
-    if (!ps_plan(g, ctx->num_cus, &p, &lds, &MT)) return 1;
+    // a fused 2x2/2 max pool: blocked output, and an activation that keeps the order of its inputs (the pool is taken on
+    // the accumulators)
+    if (pool && (!y_blocked || (q.has_act && !(q.act.alpha >= 0.0f && q.act.in_scale > 0.0f && q.act.out_scale > 0.0f)))) return 1;
+    if (!ps_plan(g, ctx->num_cus, pool, &p, &lds, &MT)) return 1;
     if (MT < 2 || MT > PS_MTMAX) return 1;
     if (size_t(p.NKP) * p.NC * 9 * 32 * p.KP >= (size_t(1) << 31)) return 1;  // the packing kernel indexes in 32 bits
     if (plan_only) return ZANT_OK;
@@ -811,7 +929,8 @@ int zant_qconv_ps(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float 
     // NCHW output: staged through LDS and written as whole runs of a plane when the runs are made of aligned 8- or
     // 4-byte units and the tile's bytes have room: a region of their own behind the patch, or -- one tile per workgroup,
     // one pass -- the ring, slot table and patch, which are dead by then.
-    p.out_unit = 0; p.stage_off = 0; p.stage_alias = 0; p.S_pad = 0;
+    p.out_unit = 0; p.stage_alias = 0; p.S_pad = 0;
+    if (!pool) p.stage_off = 0;
     if (!y_blocked) {
         const int per_img = p.TH * p.OW, plane = p.OH * p.OW;
         auto unit_ok = [&](int u) {

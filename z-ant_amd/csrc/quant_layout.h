@@ -33,11 +33,13 @@ int zant_qlinearconv_layout_pool(zant_ctx *ctx, const uint8_t *x, const int64_t 
                                  int y_layout, int fuse_pool, bool query_only, zant_pack_slot *slot);
 
 // The patch-stationary int8 matrix-core convolution (qconv_ps_i8.hip): 3x3, stride 1, pads <= 1, group 1, at least 32
-// channels on both sides.  x / y are NCHW u8 or blocked as said; ZANT_OK when it ran (with plan_only: would run), 1 when
+// channels on both sides; with `pool` (a fused 2x2/2 max pool of even-sized planes into a blocked y: g.OH / g.OW stay the
+// convolution's, y has half of each) up to 128 output channels.  x / y are NCHW u8 or blocked as said; ZANT_OK when it ran (with plan_only: would run), 1 when
 // the shape is left to the other kernels, a negative status on failure.
 struct QConvArgs;
 int zant_qconv_ps(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float *w_scale, const int32_t *bias, uint8_t *y,
-                  const ConvGeom &g, const QConvArgs &q, bool x_blocked, bool y_blocked, zant_pack_slot *slot, bool plan_only);
+                  const ConvGeom &g, const QConvArgs &q, bool x_blocked, bool y_blocked, zant_pack_slot *slot, bool plan_only,
+                  bool pool = false);
 
 // Layout conversions (HW = H * W).
 int zant_to_blocked(zant_ctx *ctx, const uint8_t *x, int64_t N, int64_t C, int64_t HW, uint8_t *xb);
