@@ -126,46 +126,79 @@ __global__ void __launch_bounds__(kThreads) softmax_f32_kernel(const float *__re
 }
 
 // Rows of at most 16 values: one thread per row, the row in registers (a wavefront per row would leave most lanes
-// idle).  A workgroup's 256 rows are one contiguous span: it crosses HBM as whole 16-byte vectors into LDS and back,
-// and each thread picks its row out of LDS.  Sequential max / sum over the row, in column order like the reference.
+// idle).  A workgroup walks chunks of 256 rows; a chunk is one contiguous span that crosses HBM as whole 16-byte
+// vectors into LDS and back, and each thread picks its row out of LDS.  The loop is software-pipelined: the loads of
+// chunk i + 1 are in flight (in registers) while chunk i is computed and written out, and the two LDS buffers take
+// turns, so a workgroup always has a chunk's bytes on their way -- one chunk per workgroup, load -> compute -> store in
+// sequence, left the memory system idle for most of a workgroup's life.  Sequential max / sum over the row, in column
+// order like the reference.
+constexpr int kSoftmaxVecs = 4;  // 16-byte vectors per thread and chunk: 256 rows x 16 columns x 4 bytes / 256 threads / 16
+
 __global__ void __launch_bounds__(kThreads) softmax_small_f32_kernel(const float *__restrict__ x, float *__restrict__ y,
                                                                     int64_t rows, int cols, int vec) {
     typedef float f4 __attribute__((ext_vector_type(4)));
-    __shared__ __attribute__((aligned(16))) float buf[kThreads * 16];
-    const int64_t row0 = int64_t(blockIdx.x) * kThreads;
-    const int nrows = int(min(int64_t(kThreads), rows - row0)), nel = nrows * cols;
-    const float *xb = x + row0 * cols;
-    float *yb = y + row0 * cols;
-    const int nvec = vec ? nel >> 2 : 0;
-    for (int i = threadIdx.x; i < nvec; i += kThreads) reinterpret_cast<f4 *>(buf)[i] = __builtin_nontemporal_load(reinterpret_cast<const f4 *>(xb) + i);
-    for (int i = (nvec << 2) + threadIdx.x; i < nel; i += kThreads) buf[i] = xb[i];
-    __syncthreads();
-    if (int(threadIdx.x) < nrows) {
-        float *row = buf + threadIdx.x * cols;
-        float v[16];
-        float m = -INFINITY;
+    __shared__ __attribute__((aligned(16))) float buf[2][kThreads * 16];
+    const int64_t n_chunks = (rows + kThreads - 1) / kThreads;
+    f4 pre[kSoftmaxVecs];
+    // a chunk's vectors into registers (vec: spans start on 16-byte boundaries; otherwise the scalar path below)
+    auto fetch = [&](int64_t chunk) {
+        const int64_t row0 = chunk * kThreads;
+        const int nel = int(min(int64_t(kThreads), rows - row0)) * cols, nvec = nel >> 2;
+        const f4 *xb = reinterpret_cast<const f4 *>(x + row0 * cols);
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
-            v[j] = j < cols ? row[j] : -INFINITY;
-            m = fmaxf(m, v[j]);
+        for (int u = 0; u < kSoftmaxVecs; ++u) {
+            const int i = u * kThreads + int(threadIdx.x);
+            if (i < nvec) pre[u] = __builtin_nontemporal_load(xb + i);
         }
-        // exp through the hardware's base-2 exponential (arguments are <= 0, results in (0, 1]: relative error a few
-        // 1e-7, far inside the operator's tolerance) and one division per row: ten full-precision exponentials and ten
-        // divisions per row were more vector work than the row's 80 bytes of traffic take to move
-        float sum = 0.0f;
+    };
+    int64_t chunk = blockIdx.x;
+    if (vec && chunk < n_chunks) fetch(chunk);
+    for (int par = 0; chunk < n_chunks; chunk += gridDim.x, par ^= 1) {
+        float *b = buf[par];
+        const int64_t row0 = chunk * kThreads;
+        const int nrows = int(min(int64_t(kThreads), rows - row0)), nel = nrows * cols;
+        const float *xb = x + row0 * cols;
+        float *yb = y + row0 * cols;
+        const int nvec = vec ? nel >> 2 : 0;
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
-            v[j] = j < cols ? __builtin_amdgcn_exp2f((v[j] - m) * 1.44269504088896340736f) : 0.0f;
-            sum += v[j];
+        for (int u = 0; u < kSoftmaxVecs; ++u) {
+            const int i = u * kThreads + int(threadIdx.x);
+            if (i < nvec) reinterpret_cast<f4 *>(b)[i] = pre[u];
         }
-        const float inv = 1.0f / sum;
+        for (int i = (nvec << 2) + threadIdx.x; i < nel; i += kThreads) b[i] = xb[i];
+        __syncthreads();  // (also: everybody has left the previous chunk's write-out of the other buffer)
+        if (vec && chunk + gridDim.x < n_chunks) fetch(chunk + gridDim.x);
+        if (int(threadIdx.x) < nrows) {
+            float *row = b + threadIdx.x * cols;
+            float v[16];
+            float m = -INFINITY;
 #pragma unroll
-        for (int j = 0; j < 16; ++j)
-            if (j < cols) row[j] = v[j] * inv;
+            for (int j = 0; j < 16; ++j) {
+                v[j] = j < cols ? row[j] : -INFINITY;
+                m = fmaxf(m, v[j]);
+            }
+            // exp through the hardware's base-2 exponential (arguments are <= 0, results in (0, 1]: relative error a few
+            // 1e-7, far inside the operator's tolerance) and one division per row: ten full-precision exponentials and
+            // ten divisions per row were more vector work than the row's 80 bytes of traffic take to move
+            float sum = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                v[j] = j < cols ? __builtin_amdgcn_exp2f((v[j] - m) * 1.44269504088896340736f) : 0.0f;
+                sum += v[j];
+            }
+            const float inv = 1.0f / sum;
+#pragma unroll
+            for (int j = 0; j < 16; ++j)
+                if (j < cols) row[j] = v[j] * inv;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < kSoftmaxVecs; ++u) {
+            const int i = u * kThreads + int(threadIdx.x);
+            if (i < nvec) __builtin_nontemporal_store(reinterpret_cast<const f4 *>(b)[i], reinterpret_cast<f4 *>(yb) + i);
+        }
+        for (int i = (nvec << 2) + threadIdx.x; i < nel; i += kThreads) yb[i] = b[i];
     }
-    __syncthreads();
-    for (int i = threadIdx.x; i < nvec; i += kThreads) __builtin_nontemporal_store(reinterpret_cast<const f4 *>(buf)[i], reinterpret_cast<f4 *>(yb) + i);
-    for (int i = (nvec << 2) + threadIdx.x; i < nel; i += kThreads) yb[i] = buf[i];
 }
 
 // ---- add ----------------------------------------------------------------------------------------
@@ -721,7 +754,9 @@ extern "C" int zant_hip_softmax_f32(zant_ctx *ctx, const float *x, float *y, int
     if (!x || !y) return ZANT_NullPointer;
     KernelTimer kt(ctx);
     if (cols <= 16)
-        hipLaunchKernelGGL(softmax_small_f32_kernel, dim3(unsigned((rows + kThreads - 1) / kThreads)), dim3(kThreads), 0,
+        // four workgroups (32 KB of LDS each) per compute unit walk the chunks of 256 rows
+        hipLaunchKernelGGL(softmax_small_f32_kernel,
+                           dim3(unsigned(std::min<int64_t>((rows + kThreads - 1) / kThreads, int64_t(ctx->num_cus) * 4))), dim3(kThreads), 0,
                            ctx->stream, x, y, rows, int(cols),
                            // every workgroup's span starts on a 16-byte boundary when 256 * cols floats do
                            ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0 ? 1 : 0);

@@ -353,7 +353,7 @@ def get_resize_output_shape(xshape, scales, sizes):
     return tuple(yd)[:xr]
 
 
-def resize(x, mode, scales, sizes, coordinate_transformation_mode="half_pixel"):
+def resize(x, mode, scales, sizes, coordinate_transformation_mode="half_pixel", out=None):
     """resize (lib_shape_math.zig:22) in its "nearest" mode; "linear" and "cubic" are not provided, any other mode
     string is UnsupportedMode as in the reference.  Unknown coordinate modes mean "asymmetric" (the reference's else)."""
     shape = get_resize_output_shape(x.shape, scales, sizes)  # InvalidInput comes before the mode is looked at (:23-28)
@@ -362,7 +362,7 @@ def resize(x, mode, scales, sizes, coordinate_transformation_mode="half_pixel"):
     if mode != "nearest":
         raise ZantError(-19)
     ctx = context()
-    y = torch.zeros(shape, dtype=x.dtype, device=x.device)
+    y = out if out is not None else torch.zeros(shape, dtype=x.dtype, device=x.device)
     xd, xr = dims(x.shape)
     sc = (C.c_float * max(len(scales), 1))(*scales) if scales is not None else None
     sd, _ = dims(sizes)
@@ -422,26 +422,26 @@ def _scalar_tensor(v, dtype, device):
     return torch.as_tensor(v, dtype=dtype, device=device).reshape(-1).contiguous()
 
 
-def quantize_linear(x, y_scale, y_zp=None, axis=1, signed=False):
+def quantize_linear(x, y_scale, y_zp=None, axis=1, signed=False, out=None):
     """signed (or an int8 zero point tensor): int8 codes saturating to [-128, 127]; otherwise uint8."""
     ctx = context()
     signed = signed or (torch.is_tensor(y_zp) and y_zp.dtype == torch.int8)
     dt = torch.int8 if signed else torch.uint8
     s = _scalar_tensor(y_scale, torch.float32, x.device)
     zp = None if y_zp is None else _scalar_tensor(y_zp, dt, x.device)
-    y = torch.zeros(x.shape, dtype=dt, device=x.device)
+    y = out if out is not None else torch.zeros(x.shape, dtype=dt, device=x.device)
     xd, r = dims(x.shape)
     fn = lib.zant_hip_quantize_linear_f32_i8 if signed else lib.zant_hip_quantize_linear_f32_u8
     ctx.check(fn(ctx.handle, _p(x), xd, r, _p(s), _p(zp), s.numel(), axis, _p(y)))
     return y
 
 
-def dequantize_linear(x, x_scale, x_zp=None, axis=1):
+def dequantize_linear(x, x_scale, x_zp=None, axis=1, out=None):
     """x: uint8, int8 or int32 codes (the zero point has x's type)."""
     ctx = context()
     s = _scalar_tensor(x_scale, torch.float32, x.device)
     zp = None if x_zp is None else _scalar_tensor(x_zp, x.dtype, x.device)
-    y = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
+    y = out if out is not None else torch.zeros(x.shape, dtype=torch.float32, device=x.device)
     xd, r = dims(x.shape)
     fn = {torch.uint8: lib.zant_hip_dequantize_linear_u8_f32, torch.int8: lib.zant_hip_dequantize_linear_i8_f32,
           torch.int32: lib.zant_hip_dequantize_linear_i32_f32}[x.dtype]
@@ -536,27 +536,27 @@ class QConvPlan:
             pass
 
 
-def qlinear_act(x, x_scale, x_zp, act, alpha, y_scale, y_zp):
+def qlinear_act(x, x_scale, x_zp, act, alpha, y_scale, y_zp, out=None):
     ctx = context()
-    y = torch.zeros_like(x)
+    y = out if out is not None else torch.zeros_like(x)
     ctx.check(lib.zant_hip_qlinear_act_u8(ctx.handle, _p(x), x.numel(), x_scale, x_zp, ACT[act], alpha, y_scale, y_zp,
                                           _p(y)))
     return y
 
 
-def qlinear_add(a, a_scale, a_zp, b, b_scale, b_zp, y_scale, y_zp):
+def qlinear_add(a, a_scale, a_zp, b, b_scale, b_zp, y_scale, y_zp, out=None):
     if a.shape != b.shape:
         raise ZantError(-7)
     ctx = context()
-    y = torch.zeros_like(a)
+    y = out if out is not None else torch.zeros_like(a)
     ctx.check(lib.zant_hip_qlinear_add_u8(ctx.handle, _p(a), a_scale, a_zp, _p(b), b_scale, b_zp, y_scale, y_zp, _p(y),
                                           a.numel()))
     return y
 
 
-def qlinear_global_avgpool(x, x_scale, x_zp, y_scale, y_zp):
+def qlinear_global_avgpool(x, x_scale, x_zp, y_scale, y_zp, out=None):
     ctx = context()
-    y = torch.zeros((x.shape[0], x.shape[1], 1, 1), dtype=torch.uint8, device=x.device)
+    y = out if out is not None else torch.zeros((x.shape[0], x.shape[1], 1, 1), dtype=torch.uint8, device=x.device)
     xd, _ = dims(x.shape)
     ctx.check(lib.zant_hip_qlinear_global_avgpool_u8(ctx.handle, _p(x), xd, x_scale, x_zp, y_scale, y_zp, _p(y)))
     return y
