@@ -197,6 +197,17 @@ def main():
     for _ in range(kit):
         lean.forward(xt)
     lean_path["ms_per_step_prepared_weights"] = round(ctx.timer_stop() / kit, 4)
+    # ... and with the two Conv -> ReLU -> MaxPool chains as one prepared call each (fuse_pool), which is what a code
+    # generator that peephole-fuses the chain emits: six calls, the pooled activations the only ones that exist
+    lean.prepare(fuse_pool=True)
+    np.testing.assert_allclose(lean.forward(xt)[[0, 1, 2, BATCH - 1]].cpu().numpy(), ref, rtol=1e-4, atol=1e-5)
+    for _ in range(3):
+        lean.forward(xt)
+    ctx.sync()
+    ctx.timer_start()
+    for _ in range(kit):
+        lean.forward(xt)
+    lean_path["ms_per_step_prepared_fused_pools"] = round(ctx.timer_stop() / kit, 4)
     del lean, xt, lean_out
 
     # ---- standalone operator figures (the "conv TOPS" half of the metric): configs 2a, 2b, 3 ----

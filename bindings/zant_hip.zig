@@ -72,7 +72,7 @@ pub extern fn zant_hip_kernel_name(ctx: ?*zant_ctx) [*:0]const u8;
 pub extern fn zant_hip_conv2d_f32(ctx: ?*zant_ctx, x: [*]const f32, xdim: *const [4]i64, w: [*]const f32, wdim: *const [4]i64, bias: ?[*]const f32, y: [*]f32, ydim: *const [4]i64, stride: [*]const i64, n_stride: c_int, pads: ?[*]const i64, n_pads: c_int, dil: ?[*]const i64, n_dil: c_int, group: i64, auto_pad: ?[*:0]const u8, fuse_act: c_int) c_int;
 pub extern fn zant_hip_conv2d_out_shape(xdim: *const [4]i64, wdim: *const [4]i64, stride: [*]const i64, n_stride: c_int, pads: ?[*]const i64, n_pads: c_int, dil: ?[*]const i64, n_dil: c_int, group: i64, auto_pad: ?[*:0]const u8, ydim: *[4]i64) c_int;
 pub extern fn zant_hip_conv2d_f32_static(ctx: ?*zant_ctx, x: [*]const f32, xdim: *const [4]i64, w: [*]const f32, wdim: *const [4]i64, bias: ?[*]const f32, y: [*]f32, ydim: *const [4]i64, stride: [*]const i64, n_stride: c_int, pads: ?[*]const i64, n_pads: c_int, dil: ?[*]const i64, n_dil: c_int, group: i64, auto_pad: ?[*:0]const u8, fuse_act: c_int) c_int;
-pub extern fn zant_hip_conv2d_f32_prepack(ctx: ?*zant_ctx, xdim: *const [4]i64, w: [*]const f32, wdim: *const [4]i64, bias: ?[*]const f32, ydim: *const [4]i64, stride: [*]const i64, n_stride: c_int, pads: ?[*]const i64, n_pads: c_int, dil: ?[*]const i64, n_dil: c_int, group: i64, auto_pad: ?[*:0]const u8, fuse_act: c_int, out: *?*zant_conv_plan) c_int;
+pub extern fn zant_hip_conv2d_f32_prepack(ctx: ?*zant_ctx, xdim: *const [4]i64, w: [*]const f32, wdim: *const [4]i64, bias: ?[*]const f32, ydim: *const [4]i64, stride: [*]const i64, n_stride: c_int, pads: ?[*]const i64, n_pads: c_int, dil: ?[*]const i64, n_dil: c_int, group: i64, auto_pad: ?[*:0]const u8, fuse_act: c_int, fuse_pool: c_int, out: *?*zant_conv_plan) c_int;
 pub extern fn zant_hip_conv2d_f32_packed(ctx: ?*zant_ctx, plan: ?*zant_conv_plan, x: [*]const f32, y: [*]f32) c_int;
 pub extern fn zant_hip_conv2d_plan_destroy(ctx: ?*zant_ctx, plan: ?*zant_conv_plan) void;
 pub extern fn zant_hip_matmul_f32(ctx: ?*zant_ctx, a: [*]const f32, adim: [*]const i64, a_rank: c_int, b: [*]const f32, bdim: [*]const i64, b_rank: c_int, y: [*]f32) c_int;
@@ -593,10 +593,11 @@ pub const QLinearConvPlan = struct {
 };
 
 /// Prepared weights for conv_lean (same attributes); `run` is conv_lean without the per-call weight packing.
+/// fuse_pool: Conv (-> ReLU) -> onnx_maxpool_lean 2x2 / stride 2 in one kernel; yshape is then the pooled shape.
 pub const ConvPlan = struct {
     handle: ?*zant_conv_plan = null,
 
-    pub fn init(xshape: []const usize, kernel: *Tensor(f32), bias: ?*const Tensor(f32), yshape: []const usize, stride: []const usize, pads: ?[]const usize, dilations: ?[]const usize, group: ?usize, auto_pad: ?[]const u8, fuse_act: c_int) !ConvPlan {
+    pub fn init(xshape: []const usize, kernel: *Tensor(f32), bias: ?*const Tensor(f32), yshape: []const usize, stride: []const usize, pads: ?[]const usize, dilations: ?[]const usize, group: ?usize, auto_pad: ?[]const u8, fuse_act: c_int, fuse_pool: bool) !ConvPlan {
         const xd = try dims4(xshape);
         const wd = try dims4(kernel.shape);
         const yd = try dims4(yshape);
@@ -613,7 +614,7 @@ pub const ConvPlan = struct {
             break :blk &ap_buf;
         } else null;
         var self = ConvPlan{};
-        try toErr(zant_hip_conv2d_f32_prepack(ctx, &xd, kernel.data.ptr, &wd, if (bias) |b| b.data.ptr else null, &yd, &s, @intCast(stride.len), if (pads != null) &p else null, if (pads) |pp| @intCast(pp.len) else 0, if (dilations != null) &d else null, if (dilations) |dd| @intCast(dd.len) else 0, if (group) |g| @intCast(g) else -1, ap, fuse_act, &self.handle));
+        try toErr(zant_hip_conv2d_f32_prepack(ctx, &xd, kernel.data.ptr, &wd, if (bias) |b| b.data.ptr else null, &yd, &s, @intCast(stride.len), if (pads != null) &p else null, if (pads) |pp| @intCast(pp.len) else 0, if (dilations != null) &d else null, if (dilations) |dd| @intCast(dd.len) else 0, if (group) |g| @intCast(g) else -1, ap, fuse_act, @intFromBool(fuse_pool), &self.handle));
         return self;
     }
 

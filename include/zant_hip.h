@@ -148,12 +148,17 @@ int zant_hip_conv2d_f32_static(zant_ctx *ctx, const float *x, const int64_t xdim
  * matrix-core kernel each time.  A plan fixes shapes, attributes (same meaning and checks as zant_hip_conv2d_f32,
  * made here) and the weight / bias tensors once: the first zant_hip_conv2d_f32_packed packs into memory the plan
  * owns, later calls launch the convolution kernel only.  w and bias are DEVICE pointers that must stay valid and
- * unchanged while the plan lives.  Destroy the plan before its context. */
+ * unchanged while the plan lives.  Destroy the plan before its context.
+ * fuse_pool != 0: the plan is Conv (-> ReLU with fuse_act) -> onnx_maxpool_lean with a 2 x 2 kernel, stride 2, no padding,
+ * floor mode (op_pooling.zig:570-659) in ONE kernel -- what a code generator that peephole-fuses the chain emits
+ * (hardcoded_mnist8.zig:186-268 is such a chain); ydim is then the pooled shape.  Taken for stride 1, dilation 1 and
+ * the shapes whose convolution kernel has the pooled epilogue (8 or more input channels, or a 1- / 3-channel 3x3 or a
+ * 1-channel 5x5 first layer); other shapes return ZANT_InvalidInput and the caller issues the two operators. */
 typedef struct zant_conv_plan zant_conv_plan;
 int zant_hip_conv2d_f32_prepack(zant_ctx *ctx, const int64_t xdim[4], const float *w, const int64_t wdim[4],
                                 const float *bias, const int64_t ydim[4], const int64_t *stride, int n_stride,
                                 const int64_t *pads, int n_pads, const int64_t *dil, int n_dil, int64_t group,
-                                const char *auto_pad, int fuse_act, zant_conv_plan **out);
+                                const char *auto_pad, int fuse_act, int fuse_pool, zant_conv_plan **out);
 int zant_hip_conv2d_f32_packed(zant_ctx *ctx, zant_conv_plan *plan, const float *x, float *y);
 void zant_hip_conv2d_plan_destroy(zant_ctx *ctx, zant_conv_plan *plan);
 

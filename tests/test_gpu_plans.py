@@ -117,3 +117,31 @@ def test_conv_plan_matches_oracle_on_every_call(G, case, relu):
     with pytest.raises(G.ZantError) as e:  # the output shape is checked when the plan is made
         tm.ConvPlan((N, C, H, W), W_, B_, (N, K, 1, 1), stride, pads, None, 1, auto_pad)
     assert e.value.name == "InvalidDimensions"
+
+
+@pytest.mark.parametrize("N,C,H,K,k", [(6, 1, 28, 32, 3), (5, 32, 13, 64, 3), (3, 3, 20, 16, 3), (4, 16, 12, 24, 3)])
+def test_conv_plan_with_the_pool_fused_matches_conv_relu_maxpool(G, N, C, H, K, k):
+    """Conv -> ReLU -> MaxPool 2x2/2 as ONE prepared call against the three oracle operators."""
+    g = np.random.default_rng(N + C + K)
+    w = (g.standard_normal((K, C, k, k)) * np.sqrt(2 / (C * k * k))).astype(np.float32)
+    b = (g.standard_normal(K) * 0.1).astype(np.float32)
+    x = g.standard_normal((N, C, H, H)).astype(np.float32)
+    tm = G.tm
+    W_, B_ = G.dev(w), G.dev(b)
+    ref = zo.onnx_maxpool(zo.ReLU(zo.Conv(x, w, b, [1, 1], None, None, 1, None)), [2, 2], [2, 2], [1, 1], [0, 0, 0, 0])
+    plan = tm.ConvPlan(x.shape, W_, B_, ref.shape, [1, 1], None, None, 1, None, "relu", True)
+    for _ in range(2):
+        y = G.dev(np.full(ref.shape, np.nan, np.float32))
+        np.testing.assert_allclose(G.host(plan(G.dev(x), y)), ref, rtol=G.RTOL, atol=G.ATOL)
+    plan.close()
+
+
+def test_conv_plan_refuses_a_fused_pool_its_kernels_do_not_have(G):
+    tm = G.tm
+    w = G.dev(np.zeros((8, 16, 3, 3), np.float32))
+    with pytest.raises(G.ZantError) as e:  # a strided convolution has no pooled epilogue
+        tm.ConvPlan((2, 16, 20, 20), w, None, (2, 8, 4, 4), [2, 2], None, None, 1, None, "relu", True)
+    assert e.value.name == "InvalidInput"
+    with pytest.raises(G.ZantError) as e:  # the pooled shape is checked
+        tm.ConvPlan((2, 16, 20, 20), w, None, (2, 8, 18, 18), [1, 1], None, None, 1, None, "relu", True)
+    assert e.value.name == "InvalidDimensions"

@@ -49,7 +49,7 @@ PROTOTYPES = {
     "zant_hip_conv2d_f32_static": (i32, [vp, vp, c_i64p, vp, c_i64p, vp, vp, c_i64p, c_i64p, i32, c_i64p, i32, c_i64p,
                                          i32, i64, C.c_char_p, i32]),
     "zant_hip_conv2d_f32_prepack": (i32, [vp, c_i64p, vp, c_i64p, vp, c_i64p, c_i64p, i32, c_i64p, i32, c_i64p, i32, i64,
-                                          C.c_char_p, i32, C.POINTER(vp)]),
+                                          C.c_char_p, i32, i32, C.POINTER(vp)]),
     "zant_hip_conv2d_f32_packed": (i32, [vp, vp, vp, vp]),
     "zant_hip_conv2d_plan_destroy": (None, [vp, vp]),
     "zant_hip_conv2d_out_shape": (i32, [c_i64p, c_i64p, c_i64p, i32, c_i64p, i32, c_i64p, i32, i64, C.c_char_p, c_i64p]),

@@ -23,7 +23,7 @@ struct zant_qconv_plan {
 
 struct zant_conv_plan {
     int64_t xdim[4], wdim[4], ydim[4], stride[2], pads[4], dil[2], group;
-    int n_stride, n_pads, n_dil, has_group, fuse_act;
+    int n_stride, n_pads, n_dil, has_group, fuse_act, fuse_pool;
     char auto_pad[16];
     bool has_auto_pad;
     const float *w, *bias;
@@ -92,7 +92,7 @@ extern "C" void zant_hip_qlinearconv_plan_destroy(zant_ctx *ctx, zant_qconv_plan
 extern "C" int zant_hip_conv2d_f32_prepack(zant_ctx *ctx, const int64_t xdim[4], const float *w, const int64_t wdim[4],
                                            const float *bias, const int64_t ydim[4], const int64_t *stride, int n_stride,
                                            const int64_t *pads, int n_pads, const int64_t *dil, int n_dil, int64_t group,
-                                           const char *auto_pad, int fuse_act, zant_conv_plan **out) {
+                                           const char *auto_pad, int fuse_act, int fuse_pool, zant_conv_plan **out) {
     if (!out) return ZANT_NullPointer;
     *out = nullptr;
     if (!ctx || !xdim || !wdim || !ydim || !w) return ZANT_NullPointer;
@@ -110,7 +110,16 @@ extern "C" int zant_hip_conv2d_f32_prepack(zant_ctx *ctx, const int64_t xdim[4],
     if (PH < dkh || PW < dkw) return ZANT_InvalidDimensions;
     if (xdim[1] != wdim[1]) return ZANT_InputTensorsWrongShape;
     const int64_t OH = (PH - dkh) / s[0] + 1, OW = (PW - dkw) / s[1] + 1;
-    if (ydim[0] != xdim[0] || ydim[1] != wdim[0] || ydim[2] != OH || ydim[3] != OW) return ZANT_InvalidDimensions;
+    const int64_t OHo = fuse_pool ? OH / 2 : OH, OWo = fuse_pool ? OW / 2 : OW;
+    if (ydim[0] != xdim[0] || ydim[1] != wdim[0] || ydim[2] != OHo || ydim[3] != OWo) return ZANT_InvalidDimensions;
+    if (fuse_pool) {
+        // only the shapes whose convolution kernel takes the pool in its epilogue (stride and dilation 1: the matrix-core
+        // kernel from 8 input channels on, the few-channel first-layer kernels): others are refused here, not run unfused
+        const int rc2 = zant_conv2d_f32_fused_pool(ctx, nullptr, xdim, w, wdim, bias, nullptr, ydim, stride, n_stride, pads, n_pads, dil,
+                                                   n_dil, group, auto_pad, fuse_act == ZANT_ACT_RELU, true, nullptr, 0, 0);
+        if (rc2 < 0) return rc2;
+        if (rc2 > 0) return ZANT_InvalidInput;
+    }
     zant_conv_plan *p = new (std::nothrow) zant_conv_plan();
     if (!p) return ZANT_MemError;
     for (int i = 0; i < 4; ++i) { p->xdim[i] = xdim[i]; p->wdim[i] = wdim[i]; p->ydim[i] = ydim[i]; }
@@ -118,7 +127,7 @@ extern "C" int zant_hip_conv2d_f32_prepack(zant_ctx *ctx, const int64_t xdim[4],
     for (int i = 0; i < n_pads; ++i) p->pads[i] = pads[i];
     for (int i = 0; i < n_dil; ++i) p->dil[i] = dil[i];
     p->n_stride = n_stride; p->n_pads = pads ? n_pads : -1; p->n_dil = dil ? n_dil : -1;
-    p->group = group; p->fuse_act = fuse_act;
+    p->group = group; p->fuse_act = fuse_act; p->fuse_pool = fuse_pool ? 1 : 0;
     p->has_auto_pad = auto_pad != nullptr;
     if (auto_pad) {
         size_t n = 0;
@@ -132,6 +141,11 @@ extern "C" int zant_hip_conv2d_f32_prepack(zant_ctx *ctx, const int64_t xdim[4],
 
 extern "C" int zant_hip_conv2d_f32_packed(zant_ctx *ctx, zant_conv_plan *p, const float *x, float *y) {
     if (!ctx || !p || !x || !y) return ZANT_NullPointer;
+    if (p->fuse_pool)
+        return zant_conv2d_f32_fused_pool(ctx, x, p->xdim, p->w, p->wdim, p->bias, y, p->ydim, p->stride, p->n_stride,
+                                          p->n_pads < 0 ? nullptr : p->pads, p->n_pads < 0 ? 0 : p->n_pads,
+                                          p->n_dil < 0 ? nullptr : p->dil, p->n_dil < 0 ? 0 : p->n_dil, p->group,
+                                          p->has_auto_pad ? p->auto_pad : nullptr, p->fuse_act == ZANT_ACT_RELU, false, &p->slot, 0, 0);
     return zant_conv2d_f32_slot(ctx, x, p->xdim, p->w, p->wdim, p->bias, y, p->ydim, p->stride, p->n_stride,
                                 p->n_pads < 0 ? nullptr : p->pads, p->n_pads < 0 ? 0 : p->n_pads,
                                 p->n_dil < 0 ? nullptr : p->dil, p->n_dil < 0 ? 0 : p->n_dil, p->group,

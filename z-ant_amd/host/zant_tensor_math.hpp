@@ -442,17 +442,19 @@ class QLinearConvPlan {
     zant_qconv_plan *plan_ = nullptr;
 };
 
-// Prepared weights for conv_lean (zant_hip_conv2d_f32_prepack), same attributes.
+// Prepared weights for conv_lean (zant_hip_conv2d_f32_prepack), same attributes; fuse_act / fuse_pool: ReLU and a
+// 2 x 2 / stride 2 max pool in the same kernel (yshape is then the pooled shape).
 class ConvPlan {
   public:
     ConvPlan(const Dims &xshape, Tensor<float> *kernel, const Tensor<float> *bias, const Dims &yshape, const Dims &stride,
-             const Dims *pads, const Dims *dilations, std::optional<int64_t> group, const char *auto_pad) {
+             const Dims *pads, const Dims *dilations, std::optional<int64_t> group, const char *auto_pad,
+             int fuse_act = ZANT_ACT_NONE, bool fuse_pool = false) {
         if (xshape.size() != 4 || kernel->shape.size() != 4 || yshape.size() != 4) throw Error(ZANT_InvalidDimensions);
         check(zant_hip_conv2d_f32_prepack(default_ctx(), xshape.data(), kernel->data, kernel->shape.data(),
                                           bias ? bias->data : nullptr, yshape.data(), stride.data(), int(stride.size()),
                                           pads ? pads->data() : nullptr, pads ? int(pads->size()) : 0,
                                           dilations ? dilations->data() : nullptr, dilations ? int(dilations->size()) : 0,
-                                          group ? *group : -1, auto_pad, ZANT_ACT_NONE, &plan_));
+                                          group ? *group : -1, auto_pad, fuse_act, fuse_pool ? 1 : 0, &plan_));
     }
     ConvPlan(const ConvPlan &) = delete;
     ConvPlan &operator=(const ConvPlan &) = delete;

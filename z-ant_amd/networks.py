@@ -73,27 +73,38 @@ class ReadmeCNN:
         self.out = torch.zeros((batch, 10), **f)
 
         self.plans = None
+        self.fused = False
 
-    def prepare(self):
+    def prepare(self, fuse_pool=False):
         """Prepared-weights handles for the two convolutions: forward() then calls conv2d_f32_packed (the weights are
-        packed at the first call, later calls launch the convolution kernels only)."""
+        packed at the first call, later calls launch the convolution kernels only).  fuse_pool: each handle is the chain
+        Conv -> ReLU -> MaxPool 2x2/2 in one kernel, as a code generator that peephole-fuses the chain would emit it."""
         p = self.p
-        self.plans = (tm.ConvPlan((self.n, 1, 28, 28), p["w1"], p["b1"], self.a1.shape, [1, 1], None, None, 1, None, "relu"),
-                      tm.ConvPlan(self.p1.shape, p["w2"], p["b2"], self.a2.shape, [1, 1], None, None, 1, None, "relu"))
+        if fuse_pool:
+            self.plans = (tm.ConvPlan((self.n, 1, 28, 28), p["w1"], p["b1"], self.p1.shape, [1, 1], None, None, 1, None, "relu", True),
+                          tm.ConvPlan(self.p1.shape, p["w2"], p["b2"], self.p2.shape, [1, 1], None, None, 1, None, "relu", True))
+        else:
+            self.plans = (tm.ConvPlan((self.n, 1, 28, 28), p["w1"], p["b1"], self.a1.shape, [1, 1], None, None, 1, None, "relu"),
+                          tm.ConvPlan(self.p1.shape, p["w2"], p["b2"], self.a2.shape, [1, 1], None, None, 1, None, "relu"))
+        self.fused = bool(fuse_pool)
         return self
 
     def forward(self, x):
         p = self.p
-        if self.plans:
-            self.plans[0](x, self.a1)
+        if self.plans and self.fused:
+            self.plans[0](x, self.p1)
+            self.plans[1](self.p1, self.p2)
         else:
-            tm.conv_lean(x, p["w1"], self.a1, p["b1"], [1, 1], None, None, 1, None, "relu")
-        tm.onnx_maxpool_lean(self.a1, self.p1, [2, 2], [2, 2], [1, 1], [0, 0, 0, 0])
-        if self.plans:
-            self.plans[1](self.p1, self.a2)
-        else:
-            tm.conv_lean(self.p1, p["w2"], self.a2, p["b2"], [1, 1], None, None, 1, None, "relu")
-        tm.onnx_maxpool_lean(self.a2, self.p2, [2, 2], [2, 2], [1, 1], [0, 0, 0, 0])
+            if self.plans:
+                self.plans[0](x, self.a1)
+            else:
+                tm.conv_lean(x, p["w1"], self.a1, p["b1"], [1, 1], None, None, 1, None, "relu")
+            tm.onnx_maxpool_lean(self.a1, self.p1, [2, 2], [2, 2], [1, 1], [0, 0, 0, 0])
+            if self.plans:
+                self.plans[1](self.p1, self.a2)
+            else:
+                tm.conv_lean(self.p1, p["w2"], self.a2, p["b2"], [1, 1], None, None, 1, None, "relu")
+            tm.onnx_maxpool_lean(self.a2, self.p2, [2, 2], [2, 2], [1, 1], [0, 0, 0, 0])
         flat = self.p2.view(1, 1, self.n, 1600)  # reshape_lean as a view
         tm.gemm_lean(flat, p["g1"], p["c1"], 1.0, 1.0, False, False, self.h1, "relu")
         tm.gemm_lean(self.h1, p["g2"], p["c2"], 1.0, 1.0, False, False, self.h2)

@@ -87,14 +87,17 @@ class ConvPlan:
     """Prepared weights for conv_lean (zant_hip_conv2d_f32_prepack): shapes, attributes and the weight tensors are fixed
     once; the first call packs the weights into memory the plan owns, later calls launch the convolution only."""
 
-    def __init__(self, xshape, w, bias, yshape, stride, pads=None, dilations=None, group=None, auto_pad=None, fuse_act=None):
+    def __init__(self, xshape, w, bias, yshape, stride, pads=None, dilations=None, group=None, auto_pad=None, fuse_act=None,
+                 fuse_pool=False):
+        """fuse_pool: Conv (-> ReLU) -> MaxPool 2x2 / stride 2 in one kernel; yshape is then the pooled shape."""
         self.ctx = context()
         self.w, self.bias, self.yshape = w, bias, tuple(yshape)  # the plan borrows the device tensors: keep them alive
         xd, _ = dims(xshape); wd, _ = dims(w.shape); yd, _ = dims(yshape)
         s, ns = dims(stride); p, npd = dims(pads); d, nd = dims(dilations)
         h = C.c_void_p()
         self.ctx.check(lib.zant_hip_conv2d_f32_prepack(self.ctx.handle, xd, _p(w), wd, _p(bias), yd, s, ns, p, npd, d, nd,
-                                                       _grp(group), _enc(auto_pad), ACT[fuse_act], C.byref(h)))
+                                                       _grp(group), _enc(auto_pad), ACT[fuse_act], int(bool(fuse_pool)),
+                                                       C.byref(h)))
         self.handle = h
 
     def __call__(self, x, y):
