@@ -9,8 +9,8 @@
 // A workgroup (4 wavefronts) walks tiles of NB images x TH output rows.  Per tile:
 //   A  the input patch ((TH-1)*stride+3 rows, W+2 columns, halo included) is copied into LDS, channel-blocked;
 //   B  expansion: wave w takes (32 patch positions) x (32 expanded channels) pairs, one v_mfma_i32_32x32x32_i8 per 32
-//      input channels, requantises and writes the bytes (value ^ 0x80) to the expanded patch in LDS;
-//   C  patch positions outside the image are overwritten with the depthwise zero point (they are its padding);
+//      input channels, requantises and writes the bytes (value ^ 0x80) to the expanded patch in LDS; patch positions
+//      outside the image receive the depthwise zero point instead (they are its padding);
 //   D  depthwise + projection: wave w takes 32 output positions; per 32 expanded channels nine MFMAs with DIAGONAL
 //      weight matrices (row c = tap weight of channel c in column c) compute the depthwise sums of 32 positions x 32
 //      channels, the requantised bytes are exchanged between lanes p and p+32 so that each lane holds 16 consecutive
@@ -73,7 +73,7 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
     int *c2 = reinterpret_cast<int *>(m2 + Ce);
     float *m3 = reinterpret_cast<float *>(c2 + Ce);
     int *c3 = reinterpret_cast<int *>(m3 + CO32 * 32);
-    int *ptab = reinterpret_cast<int *>(lds + a.o_ptab);   // [P] image << 20 | patch row << 10 | patch column
+    int *ptab = reinterpret_cast<int *>(lds + a.o_ptab);   // [Ppad] patch row; bit 31: a halo column or past the patch
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), l32 = lane & 31, lh = lane >> 5;
     const unsigned lut1_a = lds_address(lut1), lut2_a = lds_address(lut2);
@@ -94,17 +94,17 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
     {
         const int patch = a.PH * a.PW;
         const float inv_patch = 1.0f / float(patch), inv_pw = 1.0f / float(a.PW);
-        for (int p = tid; p < a.P; p += 256) {
-            const int img = small_div(p, patch, inv_patch), rem = p - img * patch;
+        for (int p = tid; p < a.Ppad; p += 256) {
+            const int pp = min(p, a.P - 1);
+            const int img = small_div(pp, patch, inv_patch), rem = pp - img * patch;
             const int ph = small_div(rem, a.PW, inv_pw), pw = rem - ph * a.PW;
-            ptab[p] = (img << 20) | (ph << 10) | pw;
+            ptab[p] = ph | ((p >= a.P || pw == 0 || pw == a.PW - 1) ? int(0x80000000u) : 0);
         }
     }
 
     const float inv_p = 1.0f / float(a.P), inv_nptiles = 1.0f / float(a.Ppad >> 5);
     const float inv_tile_img = 1.0f / float(a.TH * a.OW), inv_ow = 1.0f / float(a.OW);
     const int n_ptiles = a.Ppad >> 5, nq_tiles = (a.Q + 31) >> 5;
-    const uint4 pad_e = make_uint4(a.pad_e4, a.pad_e4, a.pad_e4, a.pad_e4);
     // the diagonal element of row l32 lies in this lane's half of the columns; which dword of the 16-byte operand
     const bool diag_mine = (l32 >> 4) == lh;
     const int diag_q = (l32 >> 2) & 3;
@@ -175,7 +175,7 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
                 nxt_dst[r] = 0;
                 if (r * 256 < a_units) {
                     // every lane loads (from the tensor's first unit when it has nothing to fetch): no divergent branch
-                    // around the load, so nothing waits for it before stage C
+                    // around the load, so nothing waits for it before the values are written to LDS
                     const int u = min(r * 256 + tid, a_units - 1);
                     const uint4 *src = patch_unit(next_tile, u, nxt_dst[r]);
                     const bool ok = src != nullptr && r * 256 + tid < a_units;
@@ -210,41 +210,61 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
                 // channels 32 kb .. + 15 of its position, lane (p, 1) the block of channels 32 kb + 16 .. + 31
                 const unsigned x_addr = lds_address(XL) + unsigned(lh * a.Ppad + l32) * 16u;
                 const unsigned e_addr = lds_address(E) + unsigned((2 * kb + lh) * a.Ppad + l32) * 16u;
-                for (; ptile < n_ptiles && u < u_end; ++ptile, ++u) {
-                    const int p = ptile * 32 + l32;
-                    i32x4 xb;
-                    qb_read128(xb, x_addr + unsigned(ptile) * 512u, 0);
-                    qb_ready(xb, 0);
-                    i32x16 acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wa0, xb, cvec, 0, 0, 0);
-                    for (int chunk = 1; chunk < a.Cin32; ++chunk)
-                        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(as_i32x4(W1[(chunk * a.Ce32 + kb) * 64 + lh * 32 + l32]),
-                                                                    as_i32x4(XL[(2 * chunk + lh) * a.Ppad + p]), acc, 0, 0, 0);
+                // Two position tiles at a time (then a single one): the second tile's operand read, MFMA and table lookups
+                // travel under the first one's arithmetic.  A position of the depthwise convolution's padding -- a halo
+                // column, a row outside the image -- receives that convolution's zero point instead of its expansion.
+                auto units = [&](auto nu_tag) {
+                    constexpr int NU = decltype(nu_tag)::value;
+                    bool padp[NU];
+#pragma unroll
+                    for (int j = 0; j < NU; ++j) {
+                        const int e = ptab[(ptile + j) * 32 + l32];
+                        padp[j] = e < 0 || unsigned(ih0 + (e & 0xffff)) >= unsigned(a.H);
+                    }
+                    i32x4 xb[NU];
+#pragma unroll
+                    for (int j = 0; j < NU; ++j) qb_read128(xb[j], x_addr + unsigned(ptile + j) * 512u, 0);
+                    i32x16 acc[NU];
+#pragma unroll
+                    for (int j = 0; j < NU; ++j) {
+                        qb_ready(xb[j], NU - 1 - j);
+                        acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wa0, xb[j], cvec, 0, 0, 0);
+                    }
+                    for (int chunk = 1; chunk < a.Cin32; ++chunk) {
+                        const i32x4 wc = as_i32x4(W1[(chunk * a.Ce32 + kb) * 64 + lh * 32 + l32]);
+#pragma unroll
+                        for (int j = 0; j < NU; ++j)
+                            acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wc, as_i32x4(XL[(2 * chunk + lh) * a.Ppad + (ptile + j) * 32 + l32]),
+                                                                           acc[j], 0, 0, 0);
+                    }
                     // a last block with at most 16 real channels: accumulator rows 16..31 (values 8..15) are padding
-                    uint32_t d[4];
-                    if (half) qb_requant_lookup<2>(acc, mv, a.zp1f, lut1_a, d);
-                    else qb_requant_lookup<4>(acc, mv, a.zp1f, lut1_a, d);
-                    // the half-wave swap leaves the lower lane with the 16 bytes of the first block of 16 channels and the
-                    // upper lane with those of the second: one 16-byte write per lane
-                    const auto s0 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
-                    const auto s1 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
-                    i32x4 out;
-                    out[0] = int(s0[0]); out[1] = int(s0[1]); out[2] = int(s1[0]); out[3] = int(s1[1]);
-                    if (!half || !lh)
-                        *reinterpret_cast<__attribute__((address_space(3))) i32x4 *>(e_addr + unsigned(ptile) * 512u) = out;
-                }
+                    uint32_t d[NU][4];
+                    if (half) qb_requant_lookup_n<2, NU>(acc, mv, a.zp1f, lut1_a, d);
+                    else qb_requant_lookup_n<4, NU>(acc, mv, a.zp1f, lut1_a, d);
+#pragma unroll
+                    for (int j = 0; j < NU; ++j) {
+                        // the half-wave swap leaves the lower lane with the 16 bytes of the first block of 16 channels and
+                        // the upper lane with those of the second: one 16-byte write per lane
+                        const auto s0 = __builtin_amdgcn_permlane32_swap(d[j][0], d[j][2], false, false);
+                        const auto s1 = __builtin_amdgcn_permlane32_swap(d[j][1], d[j][3], false, false);
+                        i32x4 out;
+                        out[0] = padp[j] ? int(a.pad_e4) : int(s0[0]); out[1] = padp[j] ? int(a.pad_e4) : int(s0[1]);
+                        out[2] = padp[j] ? int(a.pad_e4) : int(s1[0]); out[3] = padp[j] ? int(a.pad_e4) : int(s1[1]);
+                        if (!half || !lh)
+                            *reinterpret_cast<__attribute__((address_space(3))) i32x4 *>(e_addr + unsigned(ptile + j) * 512u) = out;
+                    }
+                    ptile += NU;
+                    u += NU;
+                };
+                while (ptile + 1 < n_ptiles && u + 1 < u_end) units(std::integral_constant<int, 2>());
+                if (ptile < n_ptiles && u < u_end) units(std::integral_constant<int, 1>());
                 ptile = 0;
                 ++kb;
             }
         }
         __syncthreads();
 
-        // ---- C: the depthwise convolution's padding; the next tile's input patch goes to LDS ----
-        for (int p = tid; p < a.P; p += 256) {
-            const int e = ptab[p];
-            const int ih = ih0 + ((e >> 10) & 1023), pw = e & 1023;
-            if (pw == 0 || pw == a.PW - 1 || ih < 0 || ih >= a.H)
-                for (int cb = 0; cb < a.Ce32 * 2; ++cb) E[cb * a.Ppad + p] = pad_e;
-        }
+        // ---- the next tile's input patch goes to LDS (the current one is dead; stage D reads the expanded patch only) ----
         if (has_next) {
             if (PF && prefetch) {
 #pragma unroll
@@ -254,7 +274,6 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
                 copy_patch(next_tile);
             }
         }
-        __syncthreads();
 
         // ---- D: depthwise 3x3 + projection.  A wave takes MQ tiles of 32 output positions at a time; per chunk of 32
         // expanded channels the nine diagonal operands and the requantisation tables are set up once for all of them. ----
@@ -494,7 +513,7 @@ int zant_qblock_blocked(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], 
     auto lds_for = [&](int64_t P) {
         const int64_t Ppad = (P + 31) & ~int64_t(31);
         return size_t(512) + size_t(a.Cin32 * 2 + a.Ce32 * 2) * size_t(Ppad) * 16 + w1_bytes + w2_bytes + wdw_bytes + tab_bytes +
-               align16(size_t(P) * 4);
+               size_t(Ppad) * 4;
     };
     auto tile_cost = [&](int64_t P, int64_t Q) {
         const int64_t b_units = int64_t(a.Ce32) * ((P + 31) / 32), nq = (Q + 31) / 32, qpw = (nq + 3) / 4;
@@ -552,7 +571,7 @@ int zant_qblock_blocked(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], 
         t.o_w2 = int(o); o += w2_bytes;
         t.o_wdw = int(o); o += wdw_bytes;
         t.o_tab = int(o); o += tab_bytes;
-        t.o_ptab = int(o); o += align16(size_t(t.P) * 4);
+        t.o_ptab = int(o); o += size_t(t.Ppad) * 4;
         if (o > cap) continue;
         a = t;
         cap_used = o;

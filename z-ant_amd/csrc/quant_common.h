@@ -139,3 +139,23 @@ __device__ __forceinline__ void qb_requant_lookup(const zq_i32x16 &acc, const fl
         d[g] = g < G ? (b[4 * g] | (b[4 * g + 1] << 8) | (b[4 * g + 2] << 16) | (b[4 * g + 3] << 24)) : 0u;
 }
 
+// The same for NU accumulator tiles at once: every lookup of every tile is issued before the one wait, so the later
+// tiles' lookups travel under the first tile's packing.
+template <int G, int NU>
+__device__ __forceinline__ void qb_requant_lookup_n(const zq_i32x16 (&acc)[NU], const float (&mv)[16], float zp_f, unsigned table,
+                                                    uint32_t (&d)[NU][4]) {
+    uint32_t b[NU][16];
+#pragma unroll
+    for (int j = 0; j < NU; ++j)
+#pragma unroll
+        for (int v = 0; v < 4 * G; ++v)
+            b[j][v] = qb_read_u8(__builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(float(acc[j][v]) * mv[v]) + zp_f, 0u, table));
+#pragma unroll
+    for (int j = 0; j < NU; ++j) {
+        qb_ready8(b[j]);
+        if (G > 2) qb_ready8(b[j] + 8);
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+            d[j][g] = g < G ? (b[j][4 * g] | (b[j][4 * g + 1] << 8) | (b[j][4 * g + 2] << 16) | (b[j][4 * g + 3] << 24)) : 0u;
+    }
+}
