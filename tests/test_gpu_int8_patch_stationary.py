@@ -83,6 +83,52 @@ def test_blocked_in_and_out_inside_a_model(G):
         np.testing.assert_array_equal(y, ref)
 
 
+# An NCHW input with whole 16-channel blocks and rows of whole, aligned dwords is regrouped by the kernel itself (no
+# blocked copy is written first): a tile's whole patch goes to LDS before the tile's first step.
+DIRECT_CASES = [
+    # N, C, H, W, K, pads, x_zp
+    (3, 64, 12, 12, 96, [1, 1, 1, 1], 128),    # several whole images per tile, two channel chunks
+    (2, 128, 28, 28, 128, [0, 0, 0, 0], 128),  # no padding: the patch has no halo columns
+    (5, 48, 14, 28, 96, [1, 1, 1, 1], 3),      # odd number of 16-channel blocks (the last half chunk is padding), row tiles
+    (600, 64, 8, 8, 64, [1, 1, 1, 1], 200),    # several tiles per workgroup: the patch is refilled tile after tile
+    (7, 32, 8, 16, 40, [1, 0, 1, 0], 77),      # one chunk, padding on the top / left only, images not a multiple of the tile
+    (2, 96, 12, 12, 200, [1, 1, 1, 1], 0),     # two output-channel passes over one patch, three chunks
+]
+
+
+@pytest.mark.parametrize("case", DIRECT_CASES, ids=[str(i) for i in range(len(DIRECT_CASES))])
+def test_nchw_input_read_directly_bit_exact(G, case):
+    N, C, H, W, K, pads, x_zp = case
+    x, w, ws, b = _operands(13 * N + C + K, N, C, H, W, K)
+    y = G.tm.qlinearconv(G.dev(x), 0.02, x_zp, G.dev(w), G.dev(ws), None, 0.05, 128, G.dev(b), [1, 1], pads, [1, 1], 1)
+    name = G.tm.context().kernel_name()
+    assert name.startswith("qconv_ps_kernel<") and name.endswith(",true>"), name
+    pick = list(range(N)) if N <= 8 else [0, 1, N // 2, N - 2, N - 1]
+    ref = zo.qlinearconv(x[pick], 0.02, x_zp, w, ws, None, 0.05, 128, b, [1, 1], pads, [1, 1], 1)
+    np.testing.assert_array_equal(G.host(y)[pick], ref)
+
+
+def test_nchw_input_that_needs_the_blocked_copy(G):
+    """Rows that are not whole dwords, or an input that is not 4-byte aligned, take the blocked copy as before."""
+    import torch
+    N, C, H, W, K = 3, 64, 10, 14, 64
+    x, w, ws, b = _operands(5, N, C, H, W, K)
+    ref = zo.qlinearconv(x, 0.02, 128, w, ws, None, 0.05, 128, b, [1, 1], [1, 1, 1, 1], [1, 1], 1)
+    y = G.tm.qlinearconv(G.dev(x), 0.02, 128, G.dev(w), G.dev(ws), None, 0.05, 128, G.dev(b), [1, 1], [1, 1, 1, 1], [1, 1], 1)
+    assert G.tm.context().kernel_name().endswith(",false>"), G.tm.context().kernel_name()
+    np.testing.assert_array_equal(G.host(y), ref)
+    # the same tensor of 16-column rows, one byte off alignment
+    N, C, H, W, K = 2, 32, 8, 16, 64
+    x, w, ws, b = _operands(6, N, C, H, W, K)
+    ref = zo.qlinearconv(x, 0.02, 128, w, ws, None, 0.05, 128, b, [1, 1], [1, 1, 1, 1], [1, 1], 1)
+    buf = torch.zeros(x.size + 1, dtype=torch.uint8, device="cuda:0")
+    xo = buf[1:].view(N, C, H, W)
+    xo.copy_(G.dev(x))
+    y = G.tm.qlinearconv(xo, 0.02, 128, G.dev(w), G.dev(ws), None, 0.05, 128, G.dev(b), [1, 1], [1, 1, 1, 1], [1, 1], 1)
+    assert G.tm.context().kernel_name().endswith(",false>"), G.tm.context().kernel_name()
+    np.testing.assert_array_equal(G.host(y), ref)
+
+
 # NCHW output whose plane runs are made of aligned 4- or 8-byte units is staged through LDS and written out as whole
 # runs: a staging region of its own, or -- one tile per workgroup, one pass -- the one laid over the dead ring and patch.
 STAGED_CASES = [
@@ -141,7 +187,7 @@ def test_fused_pool_bit_exact_inside_a_model(G, case, act):
     t = m.qlinearconv(t, np.ones((16, K, 1, 1), np.int8), np.full(16, 0.01, np.float32), None, 0.5, 0, [1, 1], [0, 0, 0, 0])
     m.finalize()
     m.profile()
-    assert any(k.startswith("qconv_ps_kernel<") and k.endswith(",6>") for k in m.launch_kernels()), m.launch_kernels()
+    assert any(k.startswith("qconv_ps_kernel<") and ",6," in k for k in m.launch_kernels()), m.launch_kernels()
     pick = list(range(N)) if N <= 8 else [0, 1, N // 2, N - 1]
     r = zo.qlinearconv(x0[pick], 0.02, 128, w0, ws0, None, 0.05, 128, None, [1, 1], [1, 1, 1, 1], [1, 1], 1)
     kw = dict(act=act, act_alpha=0.1, act_scale=0.04, act_zp=30) if act else {}

@@ -134,6 +134,60 @@ __device__ __forceinline__ void ps_patch_store(char *patch, const PsGeom &p, int
     *reinterpret_cast<u32x4 *>(patch + ((2 * c + h) * p.P1s + r * PS_NT + int(threadIdx.x)) * 16) = v;
 }
 
+// The whole patch of one tile straight from an NCHW u8 tensor whose channel count is a multiple of 16 and whose rows are
+// whole, aligned dwords (the host checks).  An item is 4 consecutive columns of one input row in
+// one block of 16 channels: 16 dword loads (one per channel plane; a wave's 64 items are consecutive dwords of a plane,
+// so every load instruction fetches 256 contiguous bytes), a 4 x 4 byte transpose per group of four channels, value ^
+// 0x80, and four 16-byte units written to their patch positions.  Positions outside the image (halo columns, rows above
+// or below, images past the batch) receive the padding vector in every channel block, as do blocks past the last one.
+__device__ __forceinline__ void ps_patch_from_nchw(const int8_t *__restrict__ xn, const int8_t *__restrict__ padvec, char *patch,
+                                                   const PsGeom &p, int tile) {
+    const int ig = tile / p.n_row_tiles;
+    const int n0 = ig * p.NB, oh0 = (tile - ig * p.n_row_tiles) * p.TH;
+    const u32x4 pad = *reinterpret_cast<const u32x4 *>(padvec);
+    const int CBp = 2 * p.NC, patch_hw = p.PH * p.PW;
+    const float inv_patch = 1.0f / float(patch_hw), inv_pw = 1.0f / float(p.PW);
+    for (int e = int(threadIdx.x); e < p.P1; e += PS_NT) {
+        const int img = small_div(e, patch_hw, inv_patch), rem = e - img * patch_hw;
+        const int ph = small_div(rem, p.PW, inv_pw), pw = rem - ph * p.PW;
+        const int ih = oh0 - p.pt + ph, iw = pw - p.pl;
+        if (n0 + img >= p.N || ih < 0 || ih >= p.H || iw < 0 || iw >= p.W)
+            for (int cb = 0; cb < CBp; ++cb) *reinterpret_cast<u32x4 *>(patch + (cb * p.P1s + e) * 16) = pad;
+    }
+    const int WQ = p.W >> 2, row_items = p.PH * WQ, n_items = p.NB * CBp * row_items;
+    const float inv_row_items = 1.0f / float(row_items), inv_wq = 1.0f / float(WQ), inv_cbp = 1.0f / float(CBp);
+    const unsigned plane = unsigned(p.H * p.W);
+    for (int it = int(threadIdx.x); it < n_items; it += PS_NT) {
+        const int ic = small_div(it, row_items, inv_row_items), r2 = it - ic * row_items;  // (image, channel block), (row, quad)
+        const int img = small_div(ic, CBp, inv_cbp), cb = ic - img * CBp;
+        const int ph = small_div(r2, WQ, inv_wq), k = r2 - ph * WQ;
+        const int ih = oh0 - p.pt + ph, n = n0 + img;
+        if (n >= p.N || ih < 0 || ih >= p.H) continue;
+        char *dst = patch + (cb * p.P1s + (img * p.PH + ph) * p.PW + 4 * k + p.pl) * 16;
+        if (cb >= p.CB) {
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd) *reinterpret_cast<u32x4 *>(dst + qd * 16) = pad;
+            continue;
+        }
+        const int8_t *src = xn + (size_t(unsigned((n * p.CB + cb) * 16)) * plane + unsigned(ih * p.W + 4 * k));
+        uint32_t d[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) d[j] = *reinterpret_cast<const uint32_t *>(src + size_t(j) * plane);
+        u32x4 o[4];
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {  // channels 4 g4 .. 4 g4 + 3 -> dword g4 of the four units
+            const uint32_t lo01 = __builtin_amdgcn_perm(d[4 * g4 + 1], d[4 * g4], 0x05010400u), hi01 = __builtin_amdgcn_perm(d[4 * g4 + 1], d[4 * g4], 0x07030602u);
+            const uint32_t lo23 = __builtin_amdgcn_perm(d[4 * g4 + 3], d[4 * g4 + 2], 0x05010400u), hi23 = __builtin_amdgcn_perm(d[4 * g4 + 3], d[4 * g4 + 2], 0x07030602u);
+            o[0][g4] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u) ^ 0x80808080u;
+            o[1][g4] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u) ^ 0x80808080u;
+            o[2][g4] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u) ^ 0x80808080u;
+            o[3][g4] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u) ^ 0x80808080u;
+        }
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) *reinterpret_cast<u32x4 *>(dst + qd * 16) = o[qd];
+    }
+}
+
 // What a thread copies while its wave multiplies: up to 4 units of a patch chunk (of this tile, or chunk 0 of the next)
 // and its share of the NEXT step's weight slab: unit wunit of the taps wtap0, wtap0 + wtaps, ...
 struct PsStream {
@@ -270,7 +324,10 @@ __device__ __forceinline__ void ps_write_out(const char *stage, uint8_t *__restr
 }
 
 // tabs: the per-channel requantisation multipliers (kpad floats) followed by the integer corrections (kpad ints).
-template <int MT, int OUT>
+// XN: the input is the caller's NCHW u8 tensor: a tile's whole patch is read and regrouped into 16-channel units by the
+// workgroup itself before the tile's first step (ps_patch_from_nchw), instead of streaming chunk by chunk out of a
+// blocked copy that a kernel of its own would have to write first.
+template <int MT, int OUT, bool XN>
 __global__ void __launch_bounds__(PS_NT)
 qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, const char *__restrict__ tabs,
                 const int8_t *__restrict__ padvec, uint8_t *__restrict__ y, PsGeom p, QConvArgs q) {
@@ -331,14 +388,22 @@ qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, co
     // The first tile's first patch chunk and the weights of step 0 at once.  Everything later is copied by the steps
     // themselves, two units per tap, so that the copy stream never stops.
     PsDesc desc;
-    ps_describe(desc, p, tile);
-    u32x4 pv[PS_RMAX][2], wv[PS_WUMAX];
+    if constexpr (XN) {
+        desc.ok = 0;
 #pragma unroll
-    for (int r = 0; r < PS_RMAX; ++r)
-        if (r * PS_NT < p.P1s) {
-            pv[r][0] = ps_patch_load(desc, xb, padvec, p, 0, r, 0);
-            pv[r][1] = ps_patch_load(desc, xb, padvec, p, 0, r, 1);
-        }
+        for (int r = 0; r < PS_RMAX; ++r) desc.off[r] = 0;
+    } else {
+        ps_describe(desc, p, tile);
+    }
+    u32x4 pv[PS_RMAX][2], wv[PS_WUMAX];
+    if constexpr (!XN) {
+#pragma unroll
+        for (int r = 0; r < PS_RMAX; ++r)
+            if (r * PS_NT < p.P1s) {
+                pv[r][0] = ps_patch_load(desc, xb, padvec, p, 0, r, 0);
+                pv[r][1] = ps_patch_load(desc, xb, padvec, p, 0, r, 1);
+            }
+    }
 #pragma unroll
     for (int k = 0; k < PS_WUMAX; ++k) {
         const int tp = st.wtap0 + k * st.wtaps;
@@ -378,12 +443,16 @@ qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, co
         }
     }
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (!XN) {
 #pragma unroll
-    for (int r = 0; r < PS_RMAX; ++r)
-        if (r * PS_NT < p.P1s) {
-            ps_patch_store(patch, p, 0, r, 0, pv[r][0]);
-            ps_patch_store(patch, p, 0, r, 1, pv[r][1]);
-        }
+        for (int r = 0; r < PS_RMAX; ++r)
+            if (r * PS_NT < p.P1s) {
+                ps_patch_store(patch, p, 0, r, 0, pv[r][0]);
+                ps_patch_store(patch, p, 0, r, 1, pv[r][1]);
+            }
+    } else {
+        ps_patch_from_nchw(xb, padvec, patch, p, tile);
+    }
 #pragma unroll
     for (int k = 0; k < PS_WUMAX; ++k) {
         const int tp = st.wtap0 + k * st.wtaps;
@@ -413,7 +482,9 @@ qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, co
                 st.wdst = wring + ((gs + 1) & 1) * PS_RING + wunit * 16;
                 st.pcur = 0;
                 st.pchunk = 0;
-                if (kp == 0 && c + 1 < p.NC) {
+                if constexpr (XN) {
+                    // the whole patch is in place before the tile's first step
+                } else if (kp == 0 && c + 1 < p.NC) {
                     st.pcur = 1; st.pchunk = c + 1;
                 } else if (s + 1 == NS && p.NC > 1 && next_tile < p.n_tiles) {
                     ps_describe(desc, p, next_tile);  // chunk 0 of the next tile: nobody reads that region any more
@@ -435,7 +506,7 @@ qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, co
             }
 
             // ---- end of pass kp: requantisation (+ fused activation), stores ----
-            if (s == NS && p.NC == 1 && next_tile < p.n_tiles) {
+            if (!XN && s == NS && p.NC == 1 && next_tile < p.n_tiles) {
                 // a single channel chunk cannot be refilled while it is read: the next tile's patch goes in at once,
                 // after everybody has left the matrix-core loop, and lands under this epilogue
                 __builtin_amdgcn_s_barrier();
@@ -715,6 +786,14 @@ qconv_ps_kernel(const int8_t *__restrict__ xb, const int8_t *__restrict__ wp, co
         }
         tile = next_tile;
         if (tile >= p.n_tiles) break;
+        if constexpr (XN) {
+            // everybody has left the patch (and a staging region behind it): the next tile's goes in; the step boundary
+            // that follows waits for these writes
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+            ps_patch_from_nchw(xb, padvec, patch, p, tile);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
 }
 
@@ -860,25 +939,36 @@ bool ps_plan(const ConvGeom &g, int num_cus, bool pool, PsGeom *out, size_t *lds
     return found;
 }
 
-template <int MT, int OUT>
-void ps_launch_out(zant_ctx *ctx, int grid, size_t lds, const int8_t *xb, const int8_t *wp, const char *tabs,
+template <int MT, int OUT, bool XN>
+void ps_launch_one(zant_ctx *ctx, int grid, size_t lds, const int8_t *xb, const int8_t *wp, const char *tabs,
                    const int8_t *padvec, uint8_t *y, const PsGeom &p, const QConvArgs &q) {
     // (the kernel has no static LDS: the whole 160 KB of a compute unit may be asked for as dynamic LDS)
-    if (!zant_raise_lds_limit(ctx, reinterpret_cast<const void *>(&qconv_ps_kernel<MT, OUT>), 160 * 1024)) return;
-    ZANT_KERNEL_NAME(ctx, "qconv_ps_kernel<%d,%d>", MT, OUT);
-    hipLaunchKernelGGL((qconv_ps_kernel<MT, OUT>), dim3(grid), dim3(PS_NT), lds, ctx->stream, xb, wp, tabs, padvec, y, p, q);
+    if (!zant_raise_lds_limit(ctx, reinterpret_cast<const void *>(&qconv_ps_kernel<MT, OUT, XN>), 160 * 1024)) return;
+    ZANT_KERNEL_NAME(ctx, "qconv_ps_kernel<%d,%d,%s>", MT, OUT, XN ? "true" : "false");
+    hipLaunchKernelGGL((qconv_ps_kernel<MT, OUT, XN>), dim3(grid), dim3(PS_NT), lds, ctx->stream, xb, wp, tabs, padvec, y, p, q);
+}
+
+template <int MT, int OUT>
+void ps_launch_out(zant_ctx *ctx, int grid, size_t lds, const int8_t *xb, const int8_t *wp, const char *tabs,
+                   const int8_t *padvec, uint8_t *y, const PsGeom &p, const QConvArgs &q, bool x_nchw) {
+    // an NCHW input comes from a caller of the C ABI, whose output is NCHW too
+    constexpr bool nchw_out = OUT == PS_OUT_NCHW_LUT || OUT == PS_OUT_NCHW || OUT == PS_OUT_NCHW_ST || OUT == PS_OUT_NCHW_ST_LUT;
+    if constexpr (nchw_out) {
+        if (x_nchw) return ps_launch_one<MT, OUT, true>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
+    }
+    ps_launch_one<MT, OUT, false>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
 }
 
 template <int MT>
 void ps_launch(zant_ctx *ctx, int grid, size_t lds, const int8_t *xb, const int8_t *wp, const char *tabs,
-               const int8_t *padvec, uint8_t *y, const PsGeom &p, const QConvArgs &q, int yb) {
-    if (!yb && p.out_unit && q.has_act) ps_launch_out<MT, PS_OUT_NCHW_ST_LUT>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
-    else if (!yb && p.out_unit) ps_launch_out<MT, PS_OUT_NCHW_ST>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
-    else if (!yb && q.has_act) ps_launch_out<MT, PS_OUT_NCHW_LUT>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
-    else if (!yb) ps_launch_out<MT, PS_OUT_NCHW>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
-    else if (p.pool) ps_launch_out<MT, PS_OUT_POOL>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
-    else if (q.has_act) ps_launch_out<MT, PS_OUT_BLOCKED_LUT>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
-    else ps_launch_out<MT, PS_OUT_BLOCKED>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q);
+               const int8_t *padvec, uint8_t *y, const PsGeom &p, const QConvArgs &q, int yb, bool x_nchw) {
+    if (!yb && p.out_unit && q.has_act) ps_launch_out<MT, PS_OUT_NCHW_ST_LUT>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q, x_nchw);
+    else if (!yb && p.out_unit) ps_launch_out<MT, PS_OUT_NCHW_ST>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q, x_nchw);
+    else if (!yb && q.has_act) ps_launch_out<MT, PS_OUT_NCHW_LUT>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q, x_nchw);
+    else if (!yb) ps_launch_out<MT, PS_OUT_NCHW>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q, x_nchw);
+    else if (p.pool) ps_launch_out<MT, PS_OUT_POOL>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q, x_nchw);
+    else if (q.has_act) ps_launch_out<MT, PS_OUT_BLOCKED_LUT>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q, x_nchw);
+    else ps_launch_out<MT, PS_OUT_BLOCKED>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q, x_nchw);
 }
 
 }  // namespace
@@ -899,7 +989,10 @@ int zant_qconv_ps(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float 
     if (size_t(p.NKP) * p.NC * 9 * 32 * p.KP >= (size_t(1) << 31)) return 1;  // the packing kernel indexes in 32 bits
     if (plan_only) return ZANT_OK;
     const size_t wp_bytes = size_t(p.NKP) * p.NC * 9 * 32 * p.KP;
-    const size_t xb_bytes = x_blocked ? 0 : size_t(g.N) * p.CB * g.H * g.W * 16;
+    // an NCHW input the kernel can regroup by itself needs no blocked copy
+    const bool x_direct = !x_blocked && !y_blocked && g.C % 16 == 0 && g.W % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 4 == 0 &&
+                          int64_t(g.N) * g.C * g.H * g.W < (int64_t(1) << 31);
+    const size_t xb_bytes = x_blocked || x_direct ? 0 : size_t(g.N) * p.CB * g.H * g.W * 16;
     // [tile counters (unused) | padding vector | multipliers, corrections (one contiguous table) | packed weights]
     const size_t o_pad = 256, o_mult = 512, o_corr = o_mult + size_t(p.kpad) * 4,
                  o_wp = o_mult + ps_align256(size_t(p.kpad) * 8), static_bytes = o_wp + ps_align256(wp_bytes);
@@ -920,7 +1013,7 @@ int zant_qconv_ps(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float 
         ZANT_LAUNCH_CHECK(ctx);
     }
     const int8_t *xb = reinterpret_cast<const int8_t *>(x);
-    if (!x_blocked) {
+    if (!x_blocked && !x_direct) {
         rc = zant_to_blocked(ctx, x, g.N, g.C, int64_t(g.H) * g.W, static_cast<uint8_t *>(dyn));
         if (rc) return rc;
         xb = static_cast<const int8_t *>(dyn);
@@ -951,9 +1044,9 @@ int zant_qconv_ps(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float 
     const int yb = y_blocked ? 1 : 0;
     const char *tabs = base + o_mult;
     switch (MT) {
-    case 2: ps_launch<2>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q, yb); break;
-    case 3: ps_launch<3>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q, yb); break;
-    default: ps_launch<4>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q, yb); break;
+    case 2: ps_launch<2>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q, yb, x_direct); break;
+    case 3: ps_launch<3>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q, yb, x_direct); break;
+    default: ps_launch<4>(ctx, grid, lds, xb, wp, tabs, padvec, y, p, q, yb, x_direct); break;
     }
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
