@@ -78,6 +78,9 @@ struct MNode {
     mutable zant_pack_slot slot;  // packed weights / tables of this node, filled by its first launch
     // OP_QBLOCK (a fused inverted residual block): the expansion, depthwise, projection and residual Add nodes
     int blk_expand = -1, blk_dw = -1, blk_project = -1, blk_add = -1;
+    // consecutive blocks run as one launch (zant_qblock_chain): the first one lists the others, which are skipped
+    std::vector<int> chain;
+    int chain_head = -1;
     std::vector<int> more;        // inputs of a Concat beyond the first two
     std::vector<int64_t> axes;    // ReduceMean axes / Resize sizes
     std::vector<float> scales;    // Resize scales
@@ -99,6 +102,7 @@ struct zant_model {
     int launches = 0;
     std::vector<char> result_host;  // what predict() hands out
     std::vector<std::string> launch_kernels;  // device function of each launch's main kernel, filled by zant_model_profile
+    bool no_chain = false;  // run chained blocks one by one (zant_model_read_tensor: a chain overwrites its own intermediates)
 };
 
 namespace {
@@ -186,6 +190,33 @@ void fill_block_descs(const zant_model *m, const MNode &nd, zant_qconv_desc d[3]
         *add_scale = ao.scale;
         *add_zp = ao.zp;
     }
+}
+
+// The block `head` and the blocks `more` after it (head.chain when null) as one launch; query_only: would they?
+int run_block_chain(zant_model *m, const MNode &head, bool query_only, const std::vector<int> *more = nullptr) {
+    const std::vector<int> &rest = more ? *more : head.chain;
+    constexpr int kMax = 16;
+    const int n = 1 + int(rest.size());
+    if (n > kMax) return 1;
+    zant_qconv_desc d[kMax][3];
+    zant_qblock_call calls[kMax];
+    for (int b = 0; b < n; ++b) {
+        const MNode &nd = b == 0 ? head : m->n[rest[b - 1]];
+        float add_scale = 1.0f;
+        int add_zp = 0;
+        fill_block_descs(m, nd, d[b], &add_scale, &add_zp);
+        zant_qblock_call &c = calls[b];
+        c.x = query_only ? nullptr : static_cast<const uint8_t *>(tensor_ptr(m, nd.in0));
+        c.xdim = m->t[nd.in0].dim;
+        c.expand = &d[b][0]; c.dw = &d[b][1]; c.project = &d[b][2];
+        c.dw_stride = m->n[nd.blk_dw].stride[0];
+        c.residual = nd.blk_add >= 0;
+        c.add_scale = add_scale; c.add_zp = add_zp;
+        c.y = query_only ? nullptr : static_cast<uint8_t *>(tensor_ptr(m, nd.out));
+        c.ydim = m->t[nd.out].dim;
+        c.slot = query_only ? nullptr : &nd.slot;
+    }
+    return zant_qblock_chain(m->ctx, n, calls, query_only);
 }
 
 int run_node(zant_model *m, const MNode &nd) {
@@ -309,9 +340,21 @@ int run_node(zant_model *m, const MNode &nd) {
         zant_qconv_desc d[3];
         float add_scale = 1.0f;
         int add_zp = 0;
+        const bool chained = !nd.chain.empty() && !m->no_chain;
+        if (chained) {
+            const int rc = run_block_chain(m, nd, false);
+            if (rc != 1) return rc;  // (1: not a chain after all: the blocks one by one, this one first)
+        }
         fill_block_descs(m, nd, d, &add_scale, &add_zp);
-        return zant_qblock_blocked(ctx, static_cast<const uint8_t *>(x), ti.dim, &d[0], &d[1], m->n[nd.blk_dw].stride[0], &d[2],
-                                   nd.blk_add >= 0, add_scale, add_zp, static_cast<uint8_t *>(y), to.dim, false, &nd.slot);
+        int rc = zant_qblock_blocked(ctx, static_cast<const uint8_t *>(x), ti.dim, &d[0], &d[1], m->n[nd.blk_dw].stride[0], &d[2],
+                                     nd.blk_add >= 0, add_scale, add_zp, static_cast<uint8_t *>(y), to.dim, false, &nd.slot);
+        if (chained)
+            for (size_t f = 0; f < nd.chain.size() && !rc; ++f) {
+                m->no_chain = true;
+                rc = run_node(m, m->n[nd.chain[f]]);
+                m->no_chain = false;
+            }
+        return rc;
     }
     case OP_QGAP:
         if (lin == ZANT_LAYOUT_BLOCKED16)
@@ -1054,6 +1097,35 @@ extern "C" int zant_model_finalize(zant_model *m) {
         }
     }
 
+    // ---- chains of inverted residual blocks: blocks that follow each other directly, each reading the one before's output,
+    // become one launch where the kernel can keep a workgroup on the same images through all of them.  A chain stores
+    // every block's output as before, but its workgroups are at different blocks at the same time: the tensors it reads
+    // and writes are all planned as alive at the chain's launch, so none of them shares storage with another.
+    {
+        std::vector<int> live;
+        for (int i = 0; i < nn; ++i)
+            if (!m->n[i].skip) live.push_back(i);
+        for (size_t k = 0; k < live.size();) {
+            MNode &head = m->n[live[k]];
+            size_t j = k + 1;
+            if (head.op == OP_QBLOCK) {
+                std::vector<int> rest;
+                while (j < live.size()) {
+                    const MNode &cand = m->n[live[j]], &prev = m->n[live[j - 1]];
+                    if (cand.op != OP_QBLOCK || root_of(m, cand.in0) != root_of(m, prev.out)) break;
+                    rest.push_back(live[j]);
+                    if (run_block_chain(m, head, true, &rest) != ZANT_OK) { rest.pop_back(); break; }
+                    ++j;
+                }
+                if (!rest.empty()) {
+                    head.chain = rest;
+                    for (int f : rest) m->n[f].chain_head = live[k];
+                }
+            }
+            k = std::max(j, k + 1);
+        }
+    }
+
     // ---- liveness and first-fit arena planning --------------------------------------------------
     const int nt = int(m->t.size());
     for (int i = 0; i < nt; ++i) { m->t[i].def = -1; m->t[i].last = -1; }
@@ -1062,13 +1134,17 @@ extern "C" int zant_model_finalize(zant_model *m) {
     for (int i = 0; i < nn; ++i) {
         const MNode &nd = m->n[i];
         if (nd.skip) continue;  // fused away: its tensors are views of live ones or are never materialised
-        ++m->launches;
+        if (nd.chain_head < 0) ++m->launches;
+        const int when = (nd.chain_head >= 0 ? nd.chain_head : i) + 1;  // a chain's blocks all run at its first block's launch
         const int ro = root_of(m, nd.out);
-        if (m->t[ro].def < 0) m->t[ro].def = i + 1;
+        if (m->t[ro].def < 0) m->t[ro].def = when;
+        m->t[ro].last = std::max(m->t[ro].last, when);
         for (int in : {nd.in0, nd.in1})
-            if (in >= 0) { const int r = root_of(m, in); m->t[r].last = std::max(m->t[r].last, i + 1); }
-        for (int in : nd.more) { const int r = root_of(m, in); m->t[r].last = std::max(m->t[r].last, i + 1); }
+            if (in >= 0) { const int r = root_of(m, in); m->t[r].last = std::max(m->t[r].last, when); }
+        for (int in : nd.more) { const int r = root_of(m, in); m->t[r].last = std::max(m->t[r].last, when); }
     }
+    for (int i = 0; i < nn; ++i)
+        if (m->n[i].chain_head >= 0) m->n[i].skip = true;  // from here on the chain's first block stands for them
     m->t[root_of(m, m->output)].last = nn + 1;  // the output outlives the pass
     // The input keeps its storage for the whole pass: a caller that uploads it once to zant_model_input_ptr() may run
     // the model any number of times (the reference's predict() copies its input on every call, predict.zig:339-366)
@@ -1236,7 +1312,9 @@ const char *op_name(const MNode &nd) {
     case OP_QACT: return "QLinearAct";
     case OP_QADD: return "QLinearAdd";
     case OP_QGAP: return "QLinearGlobalAveragePool";
-    case OP_QBLOCK: return nd.blk_add >= 0 ? "InvertedResidual(1x1+dw3x3+1x1+Add)" : "InvertedResidual(1x1+dw3x3+1x1)";
+    case OP_QBLOCK:
+        if (!nd.chain.empty()) return "InvertedResidualChain";
+        return nd.blk_add >= 0 ? "InvertedResidual(1x1+dw3x3+1x1+Add)" : "InvertedResidual(1x1+dw3x3+1x1)";
     default: return "?";
     }
 }
@@ -1279,6 +1357,12 @@ void node_work(const zant_model *m, const MNode &nd, double *ops, double *bytes)
         break;
     }
     default: break;
+    }
+    for (int f : nd.chain) {  // a chain's launch does the work of all its blocks
+        double fo = 0, fb = 0;
+        node_work(m, m->n[f], &fo, &fb);
+        o += fo;
+        b += fb;
     }
     *ops = o;
     *bytes = b;
@@ -1338,12 +1422,19 @@ extern "C" int zant_model_read_tensor(zant_model *m, int id, void *dst_host, siz
     // replayed up to the node that produces it (the input still sits in its slot: a pass never writes there), the tensor
     // is copied out, and the rest of the pass is replayed so that the arena -- the output at zant_model_output_ptr()
     // included -- again holds what the last zant_model_run left.
+    // (chained blocks run one by one here: a chain may be planned over its own intermediate tensors)
     const int root = root_of(m, id);
+    auto runs = [&](int i) { return !m->n[i].skip || m->n[i].chain_head >= 0; };
+    struct Unchain {
+        zant_model *m;
+        explicit Unchain(zant_model *mm) : m(mm) { m->no_chain = true; }
+        ~Unchain() { m->no_chain = false; }
+    } unchain(m);
     int last_writer = -1;
     for (int i = 0; i < int(m->n.size()); ++i)
-        if (!m->n[i].skip && root_of(m, m->n[i].out) == root) last_writer = i;
+        if (runs(i) && root_of(m, m->n[i].out) == root) last_writer = i;
     for (int i = 0; i <= last_writer; ++i) {
-        if (m->n[i].skip) continue;
+        if (!runs(i)) continue;
         const int rc = run_node(m, m->n[i]);
         if (rc) return rc;
     }
@@ -1369,7 +1460,7 @@ extern "C" int zant_model_read_tensor(zant_model *m, int id, void *dst_host, siz
     }
     if (rc) return rc;
     for (int i = last_writer + 1; i < int(m->n.size()); ++i) {
-        if (m->n[i].skip) continue;
+        if (!runs(i)) continue;
         rc = run_node(m, m->n[i]);
         if (rc) return rc;
     }

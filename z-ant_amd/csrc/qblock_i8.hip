@@ -55,11 +55,11 @@ __device__ __forceinline__ i32x4 as_i32x4(const uint4 &v) {
     return r;
 }
 
+// One block for the tiles of this workgroup; `lds` is the workgroup's dynamic LDS (256-byte aligned: the activation
+// tables need it).
 template <int CO32, int MQ, bool PF, bool SPLIT>
-__global__ void __launch_bounds__(256, 2)  // 256 registers per lane for every instantiation: over that, values would be
-                                           // parked in accumulator registers, which the hand-issued LDS reads do not survive
-qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 *__restrict__ packed, QBlockArgs a) {
-    extern __shared__ __attribute__((aligned(256))) char lds[];  // the activation tables need 256-byte alignment
+__device__ __forceinline__ void qblock_body(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 *__restrict__ packed,
+                                            const QBlockArgs &a, char *lds) {
     uint8_t *lut1 = reinterpret_cast<uint8_t *>(lds), *lut2 = lut1 + 256;
     uint4 *XL = reinterpret_cast<uint4 *>(lds + a.o_xl);   // [Cin32*2][Ppad] units of 16 channels
     uint4 *E = reinterpret_cast<uint4 *>(lds + a.o_e);     // [Ce32*2][Ppad]
@@ -473,16 +473,65 @@ qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 
     }
 }
 
+template <int CO32, int MQ, bool PF, bool SPLIT>
+__global__ void __launch_bounds__(256, 2)  // 256 registers per lane for every instantiation: over that, values would be
+                                           // parked in accumulator registers, which the hand-issued LDS reads do not survive
+qblock_kernel(const uint4 *__restrict__ x, uint8_t *__restrict__ y, const uint4 *__restrict__ packed, QBlockArgs a) {
+    extern __shared__ __attribute__((aligned(256))) char lds[];
+    qblock_body<CO32, MQ, PF, SPLIT>(x, y, packed, a, lds);
+}
+
+// Several blocks in a row as ONE launch.  Every block of a chain works on tiles of the same NB whole images, one tile
+// per workgroup, so the images a workgroup reads in block b + 1 are exactly those it wrote in block b: no workgroup ever
+// waits for another one, and a barrier of the workgroup (whose release waits for its stores; the vector L1 is shared by
+// the wavefronts of a compute unit) orders its own writes before its own reads.  What a chain saves is the launch,
+// the drain and the cold start of every block but the first; the arithmetic is that of the single blocks.
+// Workgroups run through the chain at their own pace, so one may be writing block b + 1's output while another still reads
+// block b's input: the caller must give every tensor of a chain storage of its own (a planner that lets a later tensor
+// reuse an earlier one's memory, as is right for separate launches, would let images overwrite each other here).
+constexpr int QB_CHAIN_MAX = 10;
+struct QBlockLink {
+    const uint4 *x;
+    uint8_t *y;
+    const uint4 *packed;
+    QBlockArgs a;
+};
+struct QBlockChain {
+    int n;
+    QBlockLink link[QB_CHAIN_MAX];
+};
+
+template <int CO32, int MQ>
+__global__ void __launch_bounds__(256, 2)
+qblock_chain_kernel(QBlockChain c) {
+    extern __shared__ __attribute__((aligned(256))) char lds[];
+    for (int b = 0; b < c.n; ++b) {
+        const QBlockLink &l = c.link[b];
+        if (l.a.split) qblock_body<CO32, MQ, false, true>(l.x, l.y, l.packed, l.a, lds);
+        else qblock_body<CO32, MQ, false, false>(l.x, l.y, l.packed, l.a, lds);
+        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0): this wave's stores of the block's output have arrived
+        __syncthreads();
+    }
+}
+
 size_t align256(size_t v) { return (v + 255) & ~size_t(255); }
 size_t align16(size_t v) { return (v + 15) & ~size_t(15); }
 
 bool conv1x1(const zant_qconv_desc *d) { return d && d->K > 0 && d->C > 0 && (d->n_wscale == 1 || d->n_wscale == d->K); }
 
-}  // namespace
+// What a launch needs of one block: its kernel arguments, LDS bytes, instantiation and packed weights.
+struct QBlockPrep {
+    QBlockArgs a;
+    size_t lds_bytes;
+    int CO32, MQv;
+    const uint4 *packed;
+};
 
-int zant_qblock_blocked(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], const zant_qconv_desc *expand,
-                        const zant_qconv_desc *dw, int64_t dw_stride, const zant_qconv_desc *project, int residual,
-                        float add_scale, int add_zp, uint8_t *y, const int64_t ydim[4], bool query_only, zant_pack_slot *slot) {
+// Plans a block's tile, (re)packs its weights and tables into `slot` (or the context workspace) and fills the kernel
+// arguments.  force_nb > 0: tiles of exactly that many whole images, or 1.  plan_only: no packing, no pointers needed.
+int qblock_prepare(zant_ctx *ctx, const int64_t xdim[4], const zant_qconv_desc *expand, const zant_qconv_desc *dw, int64_t dw_stride,
+                   const zant_qconv_desc *project, int residual, float add_scale, int add_zp, const int64_t ydim[4], bool plan_only,
+                   zant_pack_slot *slot, int force_nb, QBlockPrep *out) {
     if (!ctx || !xdim || !ydim || !expand || !dw || !project) return ZANT_NullPointer;
     if (!conv1x1(expand) || !conv1x1(dw) || !conv1x1(project)) return 1;
     const int64_t N = xdim[0], Cin = xdim[1], H = xdim[2], W = xdim[3];
@@ -535,11 +584,12 @@ int zant_qblock_blocked(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], 
         int bNB = 0, bTH = 0;
         if (lds_for(p_img) <= cap) {
             for (int64_t nb = 1; nb <= std::min<int64_t>(N, 2047) && lds_for(nb * p_img) <= cap; ++nb) {
+                if (force_nb > 0 && nb != force_nb) continue;
                 const int64_t tiles = (N + nb - 1) / nb, waves = (tiles + slots - 1) / slots;
                 const double c = tile_cost(nb * p_img, nb * OH * OW) * double(waves);  // time of the busiest workgroup slot
                 if (!bNB || c < best * 0.98) { best = c; bNB = int(nb); bTH = int(OH); }
             }
-        } else {
+        } else if (force_nb <= 0) {
             for (int64_t th = 1; th <= OH; ++th) {
                 const int64_t P = ((th - 1) * dw_stride + 3) * a.PW;
                 if (lds_for(P) > cap) break;
@@ -579,8 +629,24 @@ int zant_qblock_blocked(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], 
         found = true;
     }
     if (!found) return 1;
-    if (query_only) return ZANT_OK;
-    if (!x || !y || !expand->w || !expand->w_scale || !dw->w || !dw->w_scale || !project->w || !project->w_scale)
+    // position tiles a wave handles together in stage D: what its share of the tile needs, within the register budget
+    {
+        const int nq_tiles = (a.Q + 31) / 32;
+        const int q_per_wave = (nq_tiles + 3) / 4;
+        const int rounds = (q_per_wave + mq_cap - 1) / mq_cap;
+        // fewer position tiles than waves: the waves share them chunk by chunk (their sums meet in the expanded patch's LDS)
+        a.split = CO32 <= 2 && nq_tiles < 4 && nq_tiles <= mq_cap && a.Ce32 >= 2 &&
+                  size_t(nq_tiles) * CO32 * 4096 <= size_t(a.Ce32) * 2 * a.Ppad * 16;
+        out->MQv = a.split ? nq_tiles : std::max(1, (q_per_wave + rounds - 1) / rounds);
+        out->CO32 = CO32;
+        out->lds_bytes = cap_used;
+    }
+    if (plan_only) {
+        out->a = a;
+        out->packed = nullptr;
+        return ZANT_OK;
+    }
+    if (!expand->w || !expand->w_scale || !dw->w || !dw->w_scale || !project->w || !project->w_scale)
         return ZANT_NullPointer;
 
     // packed weights and tables of the three convolutions
@@ -634,23 +700,33 @@ int zant_qblock_blocked(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], 
     a.ry_rcp = a.fast_div ? zant_refined_rcp(add_scale) : 0.0f;
 
     a.packed_units = int((a.o_ptab - a.o_w1) / 16);
+    out->a = a;
+    out->packed = reinterpret_cast<const uint4 *>(base + o_w1p);
+    return ZANT_OK;
+}
+
+}  // namespace
+
+int zant_qblock_blocked(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], const zant_qconv_desc *expand,
+                        const zant_qconv_desc *dw, int64_t dw_stride, const zant_qconv_desc *project, int residual,
+                        float add_scale, int add_zp, uint8_t *y, const int64_t ydim[4], bool query_only, zant_pack_slot *slot) {
+    QBlockPrep prep;
+    if (!query_only && (!x || !y)) return ZANT_NullPointer;
+    const int rc = qblock_prepare(ctx, xdim, expand, dw, dw_stride, project, residual, add_scale, add_zp, ydim, query_only, slot, 0, &prep);
+    if (rc || query_only) return rc;
+    const QBlockArgs &a = prep.a;
+    const size_t cap_used = prep.lds_bytes;
+    const int CO32 = prep.CO32, MQv = prep.MQv;
+    const uint4 *packed = prep.packed;
     const int per_cu = cap_used <= 76 * 1024 ? 2 : 1;
     const int grid = int(std::min<int64_t>(a.n_tiles, int64_t(ctx->num_cus) * per_cu));
     KernelTimer kt(ctx);
-    // position tiles a wave handles together in stage D: what its share of the tile needs, within the register budget
-    const int nq_tiles = (a.Q + 31) / 32;
-    const int q_per_wave = (nq_tiles + 3) / 4;
-    const int rounds = (q_per_wave + mq_cap - 1) / mq_cap;
-    // fewer position tiles than waves: the waves share them chunk by chunk (their sums meet in the expanded patch's LDS)
-    a.split = CO32 <= 2 && nq_tiles < 4 && nq_tiles <= mq_cap && a.Ce32 >= 2 &&
-              size_t(nq_tiles) * CO32 * 4096 <= size_t(a.Ce32) * 2 * a.Ppad * 16;
-    const int MQv = a.split ? nq_tiles : std::max(1, (q_per_wave + rounds - 1) / rounds);
 #define ZANT_QBLOCK_LAUNCH(CO, M, P, S)                                                                                          \
     do {                                                                                                                    \
         if (!zant_raise_lds_limit(ctx, reinterpret_cast<const void *>(&qblock_kernel<CO, M, P, S>), 160 * 1024)) break;         \
         ZANT_KERNEL_NAME(ctx, "qblock_kernel<%d,%d,%s,%s>", CO, M, P ? "true" : "false", S ? "true" : "false");                                          \
         hipLaunchKernelGGL((qblock_kernel<CO, M, P, S>), dim3(grid), dim3(256), cap_used, ctx->stream,                           \
-                           reinterpret_cast<const uint4 *>(x), y, reinterpret_cast<const uint4 *>(base + o_w1p), a);       \
+                           reinterpret_cast<const uint4 *>(x), y, packed, a);       \
     } while (0)
     switch ((a.split ? 100 : 0) + CO32 * 10 + MQv) {
     case 11: ZANT_QBLOCK_LAUNCH(1, 1, true, false); break;
@@ -668,6 +744,57 @@ int zant_qblock_blocked(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], 
     default: ZANT_QBLOCK_LAUNCH(4, 1, true, false); break;
     }
 #undef ZANT_QBLOCK_LAUNCH
+    ZANT_LAUNCH_CHECK(ctx);
+    return ZANT_OK;
+}
+
+// Blocks calls[0 .. n) as one launch (qblock_chain_kernel): ZANT_OK when they ran (with query_only: would run), 1 when
+// they do not form a chain -- the caller then runs them one by one.  A chain needs whole-image tiles of one size, one
+// tile per workgroup, one instantiation of the stage D register tiling for all its blocks, and each block's input to be
+// the block before's output.
+int zant_qblock_chain(zant_ctx *ctx, int n, const zant_qblock_call *calls, bool query_only) {
+    if (!ctx || !calls) return ZANT_NullPointer;
+    if (n < 2 || n > QB_CHAIN_MAX) return 1;
+    QBlockChain chain;
+    chain.n = n;
+    size_t lds = 0;
+    int CO32 = 0, MQv = 0, NB = 0, n_tiles = 0;
+    for (int b = 0; b < n; ++b) {
+        const zant_qblock_call &c = calls[b];
+        if (!query_only && (!c.x || !c.y || (b > 0 && c.x != calls[b - 1].y))) return b > 0 && c.x && c.y ? 1 : ZANT_NullPointer;
+        QBlockPrep prep;
+        const int rc = qblock_prepare(ctx, c.xdim, c.expand, c.dw, c.dw_stride, c.project, c.residual, c.add_scale, c.add_zp, c.ydim,
+                                      query_only, c.slot, NB, &prep);
+        if (rc) return rc;
+        if (prep.a.n_row_tiles != 1) return 1;
+        if (b == 0) { CO32 = prep.CO32; MQv = prep.MQv; NB = prep.a.NB; n_tiles = prep.a.n_tiles; }
+        else if (prep.CO32 != CO32 || prep.MQv != MQv || prep.a.NB != NB || prep.a.n_tiles != n_tiles) return 1;
+        lds = std::max(lds, prep.lds_bytes);
+        chain.link[b].x = reinterpret_cast<const uint4 *>(c.x);
+        chain.link[b].y = c.y;
+        chain.link[b].packed = prep.packed;
+        chain.link[b].a = prep.a;
+    }
+    const int per_cu = lds <= 76 * 1024 ? 2 : 1;
+    if (n_tiles > ctx->num_cus * per_cu) return 1;  // one tile per workgroup, all of them resident
+    const int key = CO32 * 10 + MQv;
+    if (key != 11 && key != 12 && key != 13 && key != 21 && key != 22) return 1;
+    if (query_only) return ZANT_OK;
+    KernelTimer kt(ctx);
+#define ZANT_QCHAIN_LAUNCH(CO, M)                                                                                      \
+    do {                                                                                                               \
+        if (!zant_raise_lds_limit(ctx, reinterpret_cast<const void *>(&qblock_chain_kernel<CO, M>), 160 * 1024)) break; \
+        ZANT_KERNEL_NAME(ctx, "qblock_chain_kernel<%d,%d> x %d", CO, M, n);                                            \
+        hipLaunchKernelGGL((qblock_chain_kernel<CO, M>), dim3(n_tiles), dim3(256), lds, ctx->stream, chain);          \
+    } while (0)
+    switch (key) {
+    case 11: ZANT_QCHAIN_LAUNCH(1, 1); break;
+    case 12: ZANT_QCHAIN_LAUNCH(1, 2); break;
+    case 13: ZANT_QCHAIN_LAUNCH(1, 3); break;
+    case 21: ZANT_QCHAIN_LAUNCH(2, 1); break;
+    default: ZANT_QCHAIN_LAUNCH(2, 2); break;
+    }
+#undef ZANT_QCHAIN_LAUNCH
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
 }

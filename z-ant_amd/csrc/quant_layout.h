@@ -90,3 +90,20 @@ struct zant_qconv_desc {
 int zant_qblock_blocked(zant_ctx *ctx, const uint8_t *x, const int64_t xdim[4], const zant_qconv_desc *expand,
                         const zant_qconv_desc *dw, int64_t dw_stride, const zant_qconv_desc *project, int residual,
                         float add_scale, int add_zp, uint8_t *y, const int64_t ydim[4], bool query_only, zant_pack_slot *slot);
+
+// One block of a chain: the arguments of zant_qblock_blocked.
+struct zant_qblock_call {
+    const uint8_t *x;
+    const int64_t *xdim;
+    const zant_qconv_desc *expand, *dw;
+    int64_t dw_stride;
+    const zant_qconv_desc *project;
+    int residual;
+    float add_scale;
+    int add_zp;
+    uint8_t *y;
+    const int64_t *ydim;
+    zant_pack_slot *slot;
+};
+// Consecutive blocks (each one's input is the one before's output) as one launch; 1 when they do not form a chain.
+int zant_qblock_chain(zant_ctx *ctx, int n, const zant_qblock_call *calls, bool query_only);
