@@ -47,7 +47,7 @@ CASES = [
     ((5, 5), 56, [(72, 112, 1, "relu6", "relu6", 1)], 9, 3),                     # four output chunks, whole CU's LDS
     ((40, 40), 8, [(48, 8, 1, "relu6", "relu6", 1)], 2, 3),                      # row tiles with halo, residual
     ((41, 37), 8, [(48, 16, 2, "relu6", "relu6", 1)], 2, 3),                     # row tiles, stride 2, odd sizes
-    ((12, 12), 16, [(96, 16, 1, "relu6", "relu6", 1), (96, 24, 2, "relu6", "relu6", 1)], 6, 4),  # two blocks in a row
+    ((12, 12), 16, [(96, 16, 1, "relu6", "relu6", 1), (96, 24, 2, "relu6", "relu6", 1)], 6, 3),  # two blocks in a row: one launch
     ((9, 9), 8, [(48, 8, 1, "relu6", "relu6", 0)], 3, 5),                        # pad-0 depthwise: not the pattern, unfused
     ((1, 1), 8, [(16, 8, 1, "relu6", "relu6", 1)], 7, 3),                        # one pixel, one half-filled expanded chunk
     ((2, 3), 5, [(30, 128, 2, "relu6", "relu6", 1)], 1, 3),                      # batch 1, ragged input channels, 128 outputs
