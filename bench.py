@@ -263,7 +263,8 @@ def main():
         fn = lambda: tm.qlinearconv_lean(xq, 0.02, 128, wq, ws, None, 0.05, 128, bq, yq, [1, 1], [1, 1, 1, 1], [1, 1])
         fn(); ms = kernel_avg_ms(ctx, fn, kit)
         q_kernel = ctx.kernel_name()
-        # the whole lean call as a per-operator binding pays it: NCHW -> blocked conversion and weight packing included
+        # the whole lean call as a per-operator binding pays it: weight packing included (the kernel regroups the NCHW
+        # input into 16-channel units itself; its time above includes that)
         ctx.sync(); ctx.timer_start()
         for _ in range(kit):
             fn()
@@ -272,8 +273,8 @@ def main():
         operators["qlinearconv_u8i8_N128_C128_28x28_K128_3x3"] = {"ms": round(ms, 4), "tops": round(op / ms / 1e9, 2),
                                                                   "frac_i8_mfma_peak": round(op / ms / 1e9 / PEAK_I8_MFMA_TOPS, 5),
                                                                   "kernel": q_kernel, "whole_call_ms": round(call_ms, 4)}
-        # with a prepared-weights handle (zant_hip_qlinearconv_prepack): NCHW tensors (the layout conversion stays), and
-        # channel-blocked tensors on both sides (the call is the kernel)
+        # with a prepared-weights handle (zant_hip_qlinearconv_prepack): NCHW tensors, and channel-blocked tensors on both
+        # sides (no regrouping of the input, no staging of the output: what a chain of convolutions pays per layer)
         qop = operators["qlinearconv_u8i8_N128_C128_28x28_K128_3x3"]
         plan = tm.QConvPlan(xq.shape, 0.02, 128, wq, ws, None, 0.05, 128, bq, [1, 1], [1, 1, 1, 1], [1, 1])
         yq2 = torch.zeros_like(yq)
@@ -313,12 +314,31 @@ def main():
         yq8 = torch.zeros(1024, 128, 28, 28, dtype=torch.uint8, device=dev)
         fn8 = lambda: tm.qlinearconv_lean(xq8, 0.02, 128, wq, ws, None, 0.05, 128, bq, yq8, [1, 1], [1, 1, 1, 1], [1, 1])
         fn8(); ms8 = kernel_avg_ms(ctx, fn8, kit)
+        k8 = ctx.kernel_name()
+        ctx.sync(); ctx.timer_start()
+        for _ in range(kit):
+            fn8()
+        call8 = ctx.timer_stop() / kit
+        planb8 = tm.QConvPlan(xq8.shape, 0.02, 128, wq, ws, None, 0.05, 128, bq, [1, 1], [1, 1, 1, 1], [1, 1],
+                              x_layout=tm.BLOCKED16, y_layout=tm.BLOCKED16)
+        xb8 = tm.to_blocked16(xq8)
+        yb8 = planb8(xb8)
+        assert torch.equal(tm.from_blocked16(yb8, yq8.shape), yq8), "config 3 at batch 1024: the blocked prepared call differs from the plain one"
+        for _ in range(5):
+            planb8(xb8, yb8)
+        ctx.sync(); ctx.timer_start()
+        for _ in range(kit):
+            planb8(xb8, yb8)
+        blocked8 = ctx.timer_stop() / kit
+        planb8.close()
+        del xb8, yb8
         ref8 = zo.qlinearconv(xq8[[0, 1023]].cpu().numpy(), 0.02, 128, wq.cpu().numpy(), ws.cpu().numpy(), None, 0.05, 128,
                               bq.cpu().numpy(), [1, 1], [1, 1, 1, 1], [1, 1])
         assert np.array_equal(yq8[[0, 1023]].cpu().numpy(), ref8), "config 3 at batch 1024: timed output differs from the oracle"
         operators["qlinearconv_u8i8_N1024_C128_28x28_K128_3x3"] = {
             "ms": round(ms8, 4), "tops": round(8 * op / ms8 / 1e9, 2), "frac_i8_mfma_peak": round(8 * op / ms8 / 1e9 / PEAK_I8_MFMA_TOPS, 5),
-            "kernel": ctx.kernel_name(), "parity_gate": "images 0 and 1023 of the timed output against the oracle, bit-exact"}
+            "kernel": k8, "whole_call_ms": round(call8, 4), "prepared_blocked_call_ms": round(blocked8, 4),
+            "prepared_blocked_frac_i8_mfma_peak": round(8 * op / blocked8 / 1e9 / PEAK_I8_MFMA_TOPS, 5), "parity_gate": "images 0 and 1023 of the timed output against the oracle, bit-exact"}
         del xq8, yq8
 
     # ---- HBM-bound operators (pool / activation / requantisation / residual add): algorithmic bytes / kernel time ----
