@@ -1381,7 +1381,7 @@ qdw3x3_mfma_kernel(const uint4 *__restrict__ x, const uint32_t *__restrict__ wm,
     // Consecutive workgroup ids run on different XCDs, each with an L2 of its own, while consecutive tiles share input rows
     // (a tile's patch overlaps the row group above and below it).  With a multiple of 8 workgroups per pair, XCD j takes
     // the j-th eighth of the workgroup order, so that neighbouring tiles meet in one L2: on 1024 x 96 x 48 x 48 the kernel
-    // fetched 330 MB for its 226 MB input with the round-robin order and fetches 236 MB with this one.
+    // fetched 322 MB for its 226 MB input with the round-robin order and fetches 230 MB with this one.
     if ((blocks_per_pair & 7) == 0) blk = (blk & 7) * (blocks_per_pair >> 3) + (blk >> 3);
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(int(threadIdx.x >> 6)), l32 = lane & 31, lh = lane >> 5;
     const int cb = 2 * pair + lh;
