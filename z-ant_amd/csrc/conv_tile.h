@@ -121,3 +121,47 @@ inline bool zant_plan_conv_tiles(const ConvGeom &g, int WM, int WN, int mt_max, 
     }
     return found;
 }
+
+// LDS bank conflicts of the operand reads of a tile plan, as a function of the patch row pitch.  A lane reads the
+// 16-byte unit of its position slot; the LDS serves 16 such units per cycle when they lie in 16 different groups of four
+// banks (unit index mod 16), and takes one more cycle for every further distinct unit of a group.  Consecutive lanes
+// take consecutive positions of the (pooled) output, so the units a pass touches are spaced by the stride, by two
+// columns with a fused pool, by a patch row at a row change and by a patch image at an image change: on small maps a
+// pitch of 8 or 16 units puts whole columns of the tile into the same banks.  Returns the average number of cycles per
+// 16-lane pass (1 = conflict-free) for patch rows of `pw` units.
+inline double zant_patch_read_cycles(const TilePlan &p, const ConvGeom &g, bool pool, int pw) {
+    const TileGeom &t = p.t;
+    const int per_img = t.TH * g.OW, per_img_p = pool ? (t.TH / 2) * t.POW : 1;
+    long total = 0, passes = 0;
+    for (int wm = 0; wm < p.WM; ++wm)
+        for (int i = 0; i < p.MT; ++i)
+            for (int half = 0; half < 2; ++half) {
+                int unit[16], n_unit = 0, load[16] = {0};
+                for (int l = half * 16; l < half * 16 + 16; ++l) {
+                    int img, r, c;
+                    if (pool) {
+                        const int pp = (wm * (p.MT / 4) + i / 4) * 32 + l;
+                        img = pp / per_img_p;
+                        const int rem = pp - img * per_img_p, pr = rem / t.POW;
+                        r = 2 * pr + ((i & 3) >> 1);
+                        c = 2 * (rem - pr * t.POW) + (i & 1);
+                    } else {
+                        const int q = (wm * p.MT + i) * 32 + l;
+                        img = q / per_img;
+                        const int rem = q - img * per_img;
+                        r = rem / g.OW;
+                        c = rem - r * g.OW;
+                    }
+                    const int u = (img < t.NB && r < t.TH) ? (img * t.PH + r * g.sh) * pw + c * g.sw : 0;
+                    bool seen = false;
+                    for (int k = 0; k < n_unit; ++k) seen |= unit[k] == u;
+                    if (!seen) { unit[n_unit++] = u; ++load[u & 15]; }
+                }
+                int worst = 1;
+                for (int b = 0; b < 16; ++b) worst = load[b] > worst ? load[b] : worst;
+                total += worst;
+                ++passes;
+            }
+    return double(total) / double(passes);
+}
+

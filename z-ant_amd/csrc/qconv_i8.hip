@@ -749,6 +749,24 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
     // per-tile sequences, where a deeper ring hides more of the copy latency) -- and as the 6-bit vmcnt counter can
     // tell apart.  The patch region is padded to one slot per thread and round.
     constexpr int NT = 256;
+    // The patch row pitch: a few columns of padding where they take bank conflicts out of the operand reads (the extra
+    // columns are copied as padding and never read), as long as two staging buffers still fit.
+    {
+        const size_t cap2 = plan.t.n_tiles <= ctx->num_cus ? 160 * 1024 : 80 * 1024;
+        const int pw0 = plan.t.PW;
+        double best_c = zant_patch_read_cycles(plan, g, pool, pw0);
+        int best_pw = pw0;
+        for (int pw = pw0 + 1; pw <= pw0 + 9 && best_c > 1.0; ++pw) {
+            const int p1 = plan.t.NB * plan.t.PH * pw, p1s = ((p1 + NT - 1) / NT) * NT;
+            const size_t need = 2 * (size_t(w_region_bytes(T * QCC * K_BLK, NT)) + size_t(QCC) * p1s) + size_t(p1s) * 8 + 512 +
+                                size_t(plan.t.n_kblocks) * K_BLK * 8;
+            if (p1s / NT > QR_MAX || need > cap2) break;
+            const double c = zant_patch_read_cycles(plan, g, pool, pw);
+            if (c < best_c * 0.9) { best_c = c; best_pw = pw; }
+        }
+        plan.t.PW = best_pw;
+        plan.t.P1 = plan.t.NB * plan.t.PH * best_pw;
+    }
     plan.t.P1s = ((plan.t.P1 + NT - 1) / NT) * NT;
     if (plan.t.P1s / NT > QR_MAX) return 1;  // more copy rounds than the per-tile descriptors hold
     const size_t buf_bytes = size_t(w_region_bytes(T * QCC * K_BLK, NT)) + size_t(QCC) * plan.t.P1s;
