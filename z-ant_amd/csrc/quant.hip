@@ -194,12 +194,11 @@ __global__ void __launch_bounds__(kThreads) qlinear_add_kernel(const uint8_t *__
         }
         return;
     }
-    // the dequantised value of every stored byte, once per workgroup: two table reads replace two subtract-convert-
-    // multiply chains per output byte
-    __shared__ float ta[256], tb[256];
-    ta[threadIdx.x] = float(int(uint8_t(threadIdx.x) ^ f) - q.a_zp) * q.a_scale;
-    tb[threadIdx.x] = float(int(uint8_t(threadIdx.x) ^ f) - q.b_zp) * q.b_scale;
-    __syncthreads();
+    // Every byte is dequantised with arithmetic (byte -> float conversion, subtract, multiply: the conversion picks its
+    // byte out of the dword itself).  Two 256-entry float tables in LDS, which cost one vector instruction less per
+    // byte, made the kernel LDS-bound: random table indices of a wave collide in the banks (the LDS pipe was busy 75 % of
+    // the kernel's time, two thirds of that in bank conflicts).
+    const float za = float(q.a_zp), zb = float(q.b_zp);
     const int64_t n16 = n >> 4;
     const int64_t base = int64_t(blockIdx.x) * (kThreads * ZANT_STREAM_U) + threadIdx.x;
     const u4 *a16 = reinterpret_cast<const u4 *>(a);
@@ -212,28 +211,38 @@ __global__ void __launch_bounds__(kThreads) qlinear_add_kernel(const uint8_t *__
         if (j < n16) { va[u] = __builtin_nontemporal_load(a16 + j); vb[u] = __builtin_nontemporal_load(b16 + j); }
     }
     const float zpf = float(q.y_zp);
+    // The choice of division sequence is made once, outside the element loops: taken per element it split the sixteen
+    // bytes of a vector into sixteen basic blocks, whose dependent chains then ran one after another instead of
+    // interleaved.
+    auto requantise = [&](auto fast_tag) {
+        constexpr bool FAST = decltype(fast_tag)::value;
 #pragma unroll
-    for (int u = 0; u < ZANT_STREAM_U; ++u) {
-        const int64_t j = base + u * kThreads;
-        if (j < n16) {
-            u4 r;
+        for (int u = 0; u < ZANT_STREAM_U; ++u) {
+            const int64_t j = base + u * kThreads;
+            if (j < n16) {
+                u4 r;
 #pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                const uint32_t wa = va[u][w], wb = vb[u][w];
-                uint32_t o = 0;
+                for (int w = 0; w < 4; ++w) {
+                    const uint32_t wa = va[u][w] ^ flip4, wb = vb[u][w] ^ flip4;
+                    uint32_t o = 0;
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const float sum = ta[(wa >> (8 * k)) & 0xffu] + tb[(wb >> (8 * k)) & 0xffu];
-                    if (q.fast_div)  // finite: the saturating conversion clamps and packs
-                        o = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(div_by(sum, q.y_scale, q.y_rcp, 1)) + zpf, unsigned(k), o);
-                    else
-                        o |= uint32_t(sat_u8_rne(sum / q.y_scale, q.y_zp)) << (8 * k);
+                    for (int k = 0; k < 4; ++k) {
+                        const float ca = float((wa >> (8 * k)) & 0xffu), cb = float((wb >> (8 * k)) & 0xffu);  // v_cvt_f32_ubyte<k>
+                        // (the integer difference byte - zero point, exact as a float difference, times the scale)
+                        const float sum = (ca - za) * q.a_scale + (cb - zb) * q.b_scale;
+                        if (FAST)  // finite: the saturating conversion clamps and packs
+                            o = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_rintf(div_by(sum, q.y_scale, q.y_rcp, 1)) + zpf, unsigned(k), o);
+                        else
+                            o |= uint32_t(sat_u8_rne(sum / q.y_scale, q.y_zp)) << (8 * k);
+                    }
+                    r[w] = o ^ flip4;
                 }
-                r[w] = o ^ flip4;
+                __builtin_nontemporal_store(r, y16 + j);
             }
-            __builtin_nontemporal_store(r, y16 + j);
         }
-    }
+    };
+    if (q.fast_div) requantise(std::true_type());
+    else requantise(std::false_type());
     if (blockIdx.x == 0) {
         const int64_t j = (n16 << 4) + threadIdx.x;
         if (j < n) y[j] = uint8_t(qadd_one(a[j] ^ f, b[j] ^ f, q) ^ f);
