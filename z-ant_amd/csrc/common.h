@@ -6,6 +6,8 @@
 #include <cstdio>
 #include <cstring>
 #include <string>
+#include <type_traits>
+#include <vector>
 
 #include "zant_hip.h"
 
@@ -77,7 +79,26 @@ struct zant_pack_slot {
     bool ready = false;   // the packed contents are valid
     unsigned runs = 0;    // launches so far; its parity selects the tile counter of a launch
     bool fixed = false;   // `dev` is memory the slot does not own and must not grow: a request beyond `bytes` fails
+    // What the launcher that last used this slot derived from the call's geometry (tile shape, LDS layout, kernel
+    // choice), and the geometry it derived it from: a model node or a prepared plan calls with the same geometry every
+    // time, and the search for a tile shape costs the host 10-40 us, as much as a small layer takes on the GPU.
+    std::vector<unsigned char> plan_key, plan_val;
 };
+// The cached plan of `slot` when it was made for the geometry `key` (byte-wise equal; fill keys over a zeroed struct).
+template <class K, class V>
+inline bool zant_plan_cached(const zant_pack_slot *slot, const K &key, V *val) {
+    static_assert(std::is_trivially_copyable<K>::value && std::is_trivially_copyable<V>::value, "plain data only");
+    if (!slot || slot->fixed || slot->plan_key.size() != sizeof(K) || slot->plan_val.size() != sizeof(V)) return false;
+    if (std::memcmp(slot->plan_key.data(), &key, sizeof(K)) != 0) return false;
+    std::memcpy(val, slot->plan_val.data(), sizeof(V));
+    return true;
+}
+template <class K, class V>
+inline void zant_plan_remember(zant_pack_slot *slot, const K &key, const V &val) {
+    if (!slot || slot->fixed) return;
+    slot->plan_key.assign(reinterpret_cast<const unsigned char *>(&key), reinterpret_cast<const unsigned char *>(&key) + sizeof(K));
+    slot->plan_val.assign(reinterpret_cast<const unsigned char *>(&val), reinterpret_cast<const unsigned char *>(&val) + sizeof(V));
+}
 void zant_pack_slot_free(zant_ctx *ctx, zant_pack_slot *slot);
 // Hands out `static_bytes` of weight-derived scratch (the slot's own allocation, or the front of the context
 // workspace when slot == nullptr) and `dyn_bytes` of per-call scratch (always workspace).  *need_pack says whether

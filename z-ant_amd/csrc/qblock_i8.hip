@@ -18,6 +18,7 @@
 //      expanded channels in registers.  The result is requantised (and added to the block input) and stored.
 #include <algorithm>
 #include <cmath>
+#include <cstring>
 #include <initializer_list>
 #include <type_traits>
 
@@ -574,10 +575,20 @@ int qblock_prepare(zant_ctx *ctx, const int64_t xdim[4], const zant_qconv_desc *
     bool found = false;
     size_t cap_used = 0;
     double best_time = 0.0;
+    // the tile search below depends on the shapes only: a node or plan that calls again with the same ones reuses it
+    struct PlanKey { int64_t x[4], y[4], Ce, stride; int residual, force_nb, cus, kind; } pkey;
+    struct PlanVal { QBlockArgs a; size_t cap_used; } pval;
+    std::memset(&pkey, 0, sizeof(pkey));
+    for (int i = 0; i < 4; ++i) { pkey.x[i] = xdim[i]; pkey.y[i] = ydim[i]; }
+    pkey.Ce = Ce; pkey.stride = dw_stride; pkey.residual = residual ? 1 : 0; pkey.force_nb = force_nb; pkey.cus = ctx->num_cus;
+    pkey.kind = 0x51424c4b;  // "QBLK"
+    const bool cached = zant_plan_cached(slot, pkey, &pval);
+    if (cached) { a = pval.a; cap_used = pval.cap_used; found = true; }
     // 76 KB: what two workgroups per CU leave each other after the allocation granularity.  Both sizes are planned and
     // the cheaper taken: two workgroups on a CU run at half speed each but overlap each other's barriers and latencies,
     // which the estimate credits with a factor 1.5 against the single large workgroup.
     for (size_t cap : {size_t(76 * 1024), size_t(160 * 1024)}) {
+        if (cached) break;
         const bool two = cap <= 80 * 1024;
         const int64_t slots = int64_t(ctx->num_cus) * (two ? 2 : 1);
         double best = 0.0;
@@ -629,6 +640,12 @@ int qblock_prepare(zant_ctx *ctx, const int64_t xdim[4], const zant_qconv_desc *
         found = true;
     }
     if (!found) return 1;
+    if (!cached) {
+        std::memset(&pval, 0, sizeof(pval));
+        pval.a = a;
+        pval.cap_used = cap_used;
+        zant_plan_remember(slot, pkey, pval);
+    }
     // position tiles a wave handles together in stage D: what its share of the tile needs, within the register budget
     {
         const int nq_tiles = (a.Q + 31) / 32;

@@ -697,18 +697,32 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
                    const ConvGeom &g0, const QConvArgs &q, bool x_blocked, bool y_blocked, zant_pack_slot *slot, bool pool = false,
                    bool plan_only = false) {
     if (g0.groups != 1 || g0.C < 5 || int64_t(g0.N) * g0.OH * g0.OW < 64) return 1;
-    {
+    // What the planning below decides depends on the geometry only: a node or plan that calls again with the same one
+    // reuses it (the searches for a tile shape cost the host as much time as a small layer takes on the GPU).
+    struct PlanKey { ConvGeom g; int x_blocked, y_blocked, pool, cus, act_ok, kind; } pkey;
+    struct PlanVal { ConvGeom g; TilePlan plan; int WN, n_stages, fc_g; } pval;
+    std::memset(&pkey, 0, sizeof(pkey));
+    pkey.g = g0; pkey.x_blocked = x_blocked; pkey.y_blocked = y_blocked; pkey.pool = pool; pkey.cus = ctx->num_cus;
+    pkey.act_ok = !q.has_act || (q.act.alpha >= 0.0f && q.act.in_scale > 0.0f && q.act.out_scale > 0.0f);
+    pkey.kind = 0x54494c45;  // "TILE"
+    const bool cached = !plan_only && zant_plan_cached(slot, pkey, &pval);
+    if (!cached) {
         // 3x3 / stride 1 layers with at least 32 channels on both sides: the patch-stationary kernel
         const int rc = zant_qconv_ps(ctx, x, w, w_scale, bias, y, g0, q, x_blocked, y_blocked, slot, plan_only, pool);
         if (rc <= 0) return rc;
     }
+    ConvGeom g = g0;
+    int fc_g = 0, WN = 1, n_stages = 2;
+    TilePlan plan;
+    constexpr int NT = 256;
+    if (cached) {
+        g = pval.g; plan = pval.plan; WN = pval.WN; n_stages = pval.n_stages; fc_g = pval.fc_g;
+    } else {
     // A 1x1 layer over 1x1 feature maps (a classifier head behind a global pool) is a matrix product whose rows, the
     // images, are ceil(C / 16) * 16 contiguous bytes each.  Staged 32 channels at a time it runs C / 32 short steps of
     // 32-byte copies, one cache line each.  Read instead as a 1 x G filter over a 1 x G "image" of C / G channels -- G
     // consecutive 16-channel blocks taken as G columns: the same bytes, the same sums -- it runs G times fewer steps,
     // each copying G times longer contiguous runs.  Only the weight packing knows the difference.
-    ConvGeom g = g0;
-    int fc_g = 0;
     if (!pool && g0.H == 1 && g0.W == 1 && g0.KH == 1 && g0.KW == 1 && g0.OH == 1 && g0.OW == 1 && g0.pt == 0 && g0.pl == 0) {
         const int cb = (g0.C + 15) / 16;
         for (int cand = 8; cand >= 2 && !fc_g; cand >>= 1)
@@ -725,14 +739,12 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
         return 1;
     const int CB = (g.C + 15) / 16;
     if (int64_t(g.N) * CB * g.H * g.W >= (int64_t(1) << 27)) return 1;  // 16-byte units addressed with 32-bit offsets
-    TilePlan plan;
     ConvGeom gp = g;
     gp.C = CB;  // the planner's 32-bit offset check works in 16-byte units here
     // at most 6 position tiles per wave: with 7 the epilogue spills, and a scratch reload drains the copy ring.
     // Both workgroup shapes are tried for more than 32 output channels; plans are ranked by the planner's time estimate
     // over the GPU's 2 x CUs workgroup slots.
     const int target = 2 * ctx->num_cus;
-    int WN = 1;
     // The footprint counts two staging buffers: larger tiles (more operand reuse per staged byte) beat a deeper ring.
     bool have = zant_plan_conv_tiles(gp, 4, 1, 6, 2, 16, 80 * 1024, &plan, pool, target, 32, 256);
     if (g.K > 32) {
@@ -748,7 +760,6 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
     // 160 KB when two workgroups share a CU, all of it when the layer has no more tiles than the GPU has CUs (short
     // per-tile sequences, where a deeper ring hides more of the copy latency) -- and as the 6-bit vmcnt counter can
     // tell apart.  The patch region is padded to one slot per thread and round.
-    constexpr int NT = 256;
     // The patch row pitch: a few columns of padding where they take bank conflicts out of the operand reads (the extra
     // columns are copied as padding and never read), as long as two staging buffers still fit.
     {
@@ -774,10 +785,20 @@ int run_qconv_mfma(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float
     const int copies = w_region_bytes(T * QCC * K_BLK, NT) / (16 * NT) + (CB > 1 ? 2 : 1) * (plan.t.P1s / NT);
     const bool sparse = plan.t.n_tiles <= ctx->num_cus;
     const size_t lds_cap = sparse ? 160 * 1024 : 80 * 1024;
-    int n_stages = sparse ? 8 : 4;
+    n_stages = sparse ? 8 : 4;
     if (n_stages > plan.t.n_chunks + 1) n_stages = std::max(plan.t.n_chunks + 1, 2);
     while (n_stages > 2 && (n_stages * buf_bytes + fixed_bytes > lds_cap || copies * (n_stages - 2) > 63)) --n_stages;
     if (n_stages * buf_bytes + fixed_bytes > lds_cap) return 1;
+        if (!plan_only) {
+            std::memset(&pval, 0, sizeof(pval));
+            pval.g = g; pval.plan = plan; pval.WN = WN; pval.n_stages = n_stages; pval.fc_g = fc_g;
+            zant_plan_remember(slot, pkey, pval);
+        }
+    }
+    const int CB = (g.C + 15) / 16;
+    const int T = g.KH * g.KW, K_BLK = WN * 32;
+    const size_t buf_bytes = size_t(w_region_bytes(T * QCC * K_BLK, NT)) + size_t(QCC) * plan.t.P1s;
+    const size_t fixed_bytes = size_t(plan.t.P1s) * 8 + 512 + size_t(plan.t.n_kblocks) * K_BLK * 8;  // 256: table, 256: its alignment
     if (plan_only) return ZANT_OK;
     plan.lds_bytes = n_stages * buf_bytes + fixed_bytes;
     const size_t wp_bytes = size_t(plan.t.n_chunks) * plan.t.n_kblocks * T * QCC * K_BLK;

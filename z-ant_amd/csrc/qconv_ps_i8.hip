@@ -17,6 +17,7 @@
 // Arithmetic, operand layout (channel-blocked signed activations, [tap][half][channel][16] weights), zero-point folding
 // and the requantisation epilogue are those of qconv_mfma_kernel (qconv_i8.hip).
 #include <algorithm>
+#include <cstring>
 
 #include "quant_common.h"
 #include "quant_layout.h"
@@ -984,7 +985,21 @@ int zant_qconv_ps(zant_ctx *ctx, const uint8_t *x, const int8_t *w, const float 
     // a fused 2x2/2 max pool: blocked output, and an activation that keeps the order of its inputs (the pool is taken on
     // the accumulators)
     if (pool && (!y_blocked || (q.has_act && !(q.act.alpha >= 0.0f && q.act.in_scale > 0.0f && q.act.out_scale > 0.0f)))) return 1;
-    if (!ps_plan(g, ctx->num_cus, pool, &p, &lds, &MT)) return 1;
+    // the tile search depends on the geometry only: a node or plan that calls again with the same one reuses its result
+    struct PlanKey { ConvGeom g; int pool, cus, kind; } pkey;
+    struct PlanVal { PsGeom p; size_t lds; int MT; } pval;
+    std::memset(&pkey, 0, sizeof(pkey));
+    pkey.g = g; pkey.pool = pool; pkey.cus = ctx->num_cus; pkey.kind = 0x50535f50;  // "PS_P"
+    if (!plan_only && zant_plan_cached(slot, pkey, &pval)) {
+        p = pval.p; lds = pval.lds; MT = pval.MT;
+    } else {
+        if (!ps_plan(g, ctx->num_cus, pool, &p, &lds, &MT)) return 1;
+        if (!plan_only && MT >= 2 && MT <= PS_MTMAX) {
+            std::memset(&pval, 0, sizeof(pval));
+            pval.p = p; pval.lds = lds; pval.MT = MT;
+            zant_plan_remember(slot, pkey, pval);
+        }
+    }
     if (MT < 2 || MT > PS_MTMAX) return 1;
     if (size_t(p.NKP) * p.NC * 9 * 32 * p.KP >= (size_t(1) << 31)) return 1;  // the packing kernel indexes in 32 bits
     if (plan_only) return ZANT_OK;
