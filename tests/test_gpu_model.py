@@ -182,6 +182,23 @@ def test_predict_entry_point_follows_the_reference_abi(G):
     (5, 12, 20, 20, 32, (2, 3), 1, True),  # 2x3 filter (generic tap loop), 32-channel workgroups
 ])
 def test_conv_with_fused_pool_on_the_matrix_cores(G, N, C, H, W, K, k, pad, relu):
+    _fused_pool_case(G, N, C, H, W, K, k, pad, relu, None)
+
+
+@pytest.mark.parametrize("N,C,H,W,K,k,pad,relu", [
+    (9, 32, 12, 12, 64, 3, 0, True),      # 25 windows per image: tiles start anywhere inside an image; the last is part empty
+    (7, 16, 12, 12, 64, 3, 0, True),      # the last tile touches fewer images than its patch holds
+    (23, 16, 12, 12, 64, 3, 0, False),
+    (11, 8, 12, 12, 96, 3, 0, True),      # a single channel chunk, two blocks of output channels (the second half empty)
+    (7, 24, 13, 9, 72, 3, 1, True),       # odd conv rows (the pool drops the last), padding, K not a multiple of 32
+    (13, 12, 11, 12, 64, (2, 3), 1, True),  # generic tap loop
+    (700, 8, 12, 12, 256, 3, 0, True),    # 1096 tiles on 512 workgroups: the last, partial round is dealt out by number
+])
+def test_conv_with_fused_pool_on_window_packed_tiles(G, N, C, H, W, K, k, pad, relu):
+    _fused_pool_case(G, N, C, H, W, K, k, pad, relu, ",true,true>")
+
+
+def _fused_pool_case(G, N, C, H, W, K, k, pad, relu, kernel_suffix):
     from zant_amd.model import Model
     g = np.random.default_rng(N * 1000 + C)
     x = g.standard_normal((N, C, H, W), dtype=np.float32)
@@ -199,7 +216,11 @@ def test_conv_with_fused_pool_on_the_matrix_cores(G, N, C, H, W, K, k, pad, relu
     if relu:
         ref = zo.ReLU(ref)
     ref = zo.onnx_maxpool(ref, [2, 2], [2, 2], [1, 1], [0, 0, 0, 0])
-    np.testing.assert_allclose(m.predict_host(x), ref, rtol=G.RTOL, atol=G.ATOL)
+    for _ in range(2):  # (the second pass draws its tiles from the counter the first one re-armed)
+        np.testing.assert_allclose(m.predict_host(x), ref, rtol=G.RTOL, atol=G.ATOL)
+    if kernel_suffix is not None:
+        m.profile()
+        assert m.launch_kernels()[0].endswith(kernel_suffix), m.launch_kernels()
     m.close()
 
 

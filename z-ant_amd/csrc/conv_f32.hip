@@ -78,6 +78,10 @@ __device__ __forceinline__ float vmax3(float a, float b, float c) {
     return r;
 }
 
+// Window-packed tiles of the pooled kernel: window slots per tile; the tiles from `tail_start` on (tail_n of them, the
+// last partial round) are handed out one per workgroup, to workgroups 0 .. tail_n-1.
+struct PackGeom { int S, tail_start, tail_n; };
+
 // A few zero words that padding lanes of the asynchronous global->LDS copies read from.
 __device__ __align__(16) float g_zero_words[4] = {0.f, 0.f, 0.f, 0.f};
 
@@ -91,7 +95,7 @@ template <int MT, int WM, int WN, int KV, int TT>
 __device__ __forceinline__ void conv_step(float *__restrict__ dma, const float *__restrict__ cmp,
                                           const int *__restrict__ ttab, const float *__restrict__ x,
                                           const float *__restrict__ wp, const ConvGeom &g, const TileGeom &t,
-                                          bool do_issue, int n0, int kb, int ichunk, const int (&lds_off)[MT],
+                                          bool do_issue, int n0, int kb, int ichunk, int p1, const int (&lds_off)[MT],
                                           f32x16 (&acc)[MT]) {
     constexpr int NT = WM * WN * 64;
     constexpr int K_BLK = WN * 32;
@@ -126,14 +130,14 @@ __device__ __forceinline__ void conv_step(float *__restrict__ dma, const float *
             const float *q0 = x + int64_t(n0) * g.C * x_plane + int64_t(ichunk * (CC / 4)) * x_plane * 4;
             const float *q1 = q0 + x_plane * 4;
             const bool h_ok1 = ichunk * CC + 4 < g.C;
-            for (int p0 = 0; p0 < t.P1; p0 += 2 * NT) {
+            for (int p0 = 0; p0 < p1; p0 += 2 * NT) {
                 int e[2], pad0 = 0, pad1 = 0;
 #pragma unroll
-                for (int u = 0; u < 2; ++u) e[u] = lds_read32_async(ttab_addr + unsigned(min(p0 + u * NT + tid, t.P1 - 1)) * 4u);
+                for (int u = 0; u < 2; ++u) e[u] = lds_read32_async(ttab_addr + unsigned(min(p0 + u * NT + tid, p1 - 1)) * 4u);
                 lds_wait_all(e[0], e[1], pad0, pad1);
 #pragma unroll
                 for (int u = 0; u < 2; ++u) {
-                    if (p0 + u * NT + tid < t.P1) {
+                    if (p0 + u * NT + tid < p1) {
                         const bool ok = e[u] >= 0;
                         const float *sp0 = ok ? q0 + unsigned(e[u]) : g_zero_words;
                         const float *sp1 = (ok && h_ok1) ? q1 + unsigned(e[u]) : g_zero_words;
@@ -151,18 +155,18 @@ __device__ __forceinline__ void conv_step(float *__restrict__ dma, const float *
         // The table lives in LDS.  The compiler drains every outstanding asynchronous copy before an LDS read
         // it issues itself in this loop (one round trip to L2 per iteration, which made staging cost ~18 % of a
         // step), so the table is read with hand-written ds_read_b32, one iteration ahead of its use.
-        for (int p0 = 0; p0 < t.P1; p0 += 4 * PPI) {
+        for (int p0 = 0; p0 < p1; p0 += 4 * PPI) {
             // four table entries per round; nothing read this way stays in flight across a loop edge (a register
             // copy there would run before the data has landed)
             int e[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u)
-                e[u] = lds_read32_async(ttab_addr + unsigned(min(p0 + u * PPI + (tid >> 2), t.P1 - 1)) * 4u);
+                e[u] = lds_read32_async(ttab_addr + unsigned(min(p0 + u * PPI + (tid >> 2), p1 - 1)) * 4u);
             lds_wait_all(e[0], e[1], e[2], e[3]);
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 const int pos = p0 + u * PPI + (tid >> 2);
-                if (pos < t.P1) {
+                if (pos < p1) {
                     const bool ok = e[u] >= 0;
                     const unsigned vo = unsigned(e[u] + jplane);
                     const float *sp0 = (ok && c_ok0) ? b0 + vo : g_zero_words;
@@ -245,10 +249,18 @@ __device__ __forceinline__ void conv_step(float *__restrict__ dma, const float *
 // asynchronous (global_load_lds, no VGPR round trip) and run one (tile, chunk) step ahead of the
 // matrix cores, across tile boundaries as well: while a tile's bias/ReLU epilogue stores drain, the
 // first chunk of the workgroup's next tile is already landing.  Tiles are drawn from an atomic counter.
-template <int MT, int WM, int WN, int KV, int TT, bool POOL = false>
+//
+// PACK (with POOL, whole pooled images smaller than a tile's window slots): a tile is not a group of whole images but S
+// consecutive pooling windows of the batch's flat window sequence, wherever in an image they start, so no slot is empty
+// (25 windows per image fill 50 of 64 slots otherwise).  The patch holds every image the run of windows touches (t.NB =
+// the most that can be); a lane's window, its patch offset and its output position change from tile to tile and come
+// from a per-workgroup table indexed by the window's number inside the staged images.
+template <int MT, int WM, int WN, int KV, int TT, bool POOL = false, bool PACK = false>
 __global__ void __launch_bounds__(WM *WN * 64, 2)
 conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, const float *__restrict__ bias,
-                     float *__restrict__ y, ConvGeom g, TileGeom t, int relu, int *__restrict__ tile_counters, int parity) {
+                     float *__restrict__ y, ConvGeom g, TileGeom t, int relu, int *__restrict__ tile_counters, int parity,
+                     PackGeom pk) {
+    static_assert(!PACK || POOL, "window packing belongs to the fused pool");
     constexpr int NT = WM * WN * 64;
     constexpr int K_BLK = WN * 32;
     extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -257,10 +269,11 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
     const int buf_floats = w_chunk + CC * t.P1s;  // one staging buffer
     float *buf0 = lds, *buf1 = lds + buf_floats;
     int *ptab = reinterpret_cast<int *>(lds + 2 * buf_floats);     // [P1s]: img << 24 | patch row << 12 | patch column
-    int *ttab0 = ptab + t.P1s;                                     // [2][P1s]: per tile, a position's element offset in
+    int *ttab0 = ptab + (PACK ? 0 : t.P1s);                        // [2][P1s]: per tile, a position's element offset in
     int *ttab1 = ttab0 + t.P1s;                                    //   the image group, -1 where the patch is padding
     int *sched = ttab1 + t.P1s;                                    // [2]: tile ids handed out by thread 0
     float *bias_l = reinterpret_cast<float *>(sched + 2);          // [n_kblocks * K_BLK]: the bias, zero past K
+    int *wtab = reinterpret_cast<int *>(bias_l + t.n_kblocks * K_BLK);  // PACK: [NB * windows per image][2]
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction; says so to the compiler (LDS
@@ -272,6 +285,8 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
     const int patch_hw = t.PH * t.PW;
 
     // ---- once per workgroup: the tile-independent part of the patch geometry ----
+    // (PACK keeps no such table: its larger patches need the room, and a tile's table costs two divisions per entry)
+    if constexpr (!PACK)
     for (int e = tid; e < t.P1; e += NT) {
         const int img = e / patch_hw, rem = e - img * patch_hw;
         const int ph = rem / t.PW, pw = rem - ph * t.PW;
@@ -281,10 +296,21 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
     // (pooled position (wm*MT/4 + j)*32 + l32), so the pool is a register-wise max in the epilogue.
     const int per_img_p = POOL ? (t.TH / 2) * t.POW : 1;
     int lds_off[MT];  // float4 index of each of this lane's output positions inside a patch half
+    if constexpr (PACK) {
+        // window w of the staged images -> { patch unit of its first member, image << 20 | pooled row << 10 | column }
+        for (int w = tid; w < t.NB * per_img_p; w += NT) {
+            const int img = w / per_img_p, rem = w - img * per_img_p;
+            const int pr = rem / t.POW, pc = rem - pr * t.POW;
+            wtab[2 * w] = (img * t.PH + 2 * pr * g.sh) * t.PW + 2 * pc * g.sw;
+            wtab[2 * w + 1] = (img << 20) | (pr << 10) | pc;
+        }
+    }
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
         int img, r, c;
-        if (POOL) {
+        if (PACK) {
+            img = r = c = 0;  // set per tile
+        } else if (POOL) {
             const int pp = (wm * (MT / 4) + i / 4) * 32 + l32;
             img = pp / per_img_p;
             const int rem = pp - img * per_img_p, pr = rem / t.POW;
@@ -303,7 +329,10 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
     for (int k = tid; k < t.n_kblocks * K_BLK; k += NT) bias_l[k] = (bias != nullptr && k < g.K) ? bias[k] : 0.0f;
     // pooled position slot j of this lane inside a tile: image << 20 | pooled row << 10 | pooled column
     int pool_pos[POOL ? MT / 4 : 1];
-    if constexpr (POOL) {
+    if constexpr (PACK) {
+#pragma unroll
+        for (int j = 0; j < MT / 4; ++j) pool_pos[j] = 0;  // set per tile
+    } else if constexpr (POOL) {
 #pragma unroll
         for (int j = 0; j < MT / 4; ++j) {
             const int pp = (wm * (MT / 4) + j) * 32 + l32;
@@ -336,12 +365,20 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
 
     // A tile's table: which patch positions exist for this tile (rows above / below the image and images past the
     // batch do not) and where they are.  Built once per tile by the whole workgroup, read by every step's copies.
-    auto fill_ttab = [&](int *tt, int n0, int oh0) {
+    auto fill_ttab = [&](int *tt, int n0, int oh0, int p1) {
         const int ih0 = oh0 * g.sh - g.pt;
         const int imgs_here = min(t.NB, g.N - n0);
-        for (int e = tid; e < t.P1; e += NT) {
-            const int v = ptab[e];
-            const int img = int(unsigned(v) >> 24), ih = ih0 + ((v >> 12) & 0xfff), iw = (v & 0xfff) - g.pl;
+        for (int e = tid; e < p1; e += NT) {
+            int img, ih, iw;
+            if constexpr (PACK) {
+                img = e / patch_hw;
+                const int rem = e - img * patch_hw, ph = rem / t.PW;
+                ih = ih0 + ph;
+                iw = rem - ph * t.PW - g.pl;
+            } else {
+                const int v = ptab[e];
+                img = int(unsigned(v) >> 24); ih = ih0 + ((v >> 12) & 0xfff); iw = (v & 0xfff) - g.pl;
+            }
             const bool ok = iw >= 0 && iw < g.W && ih >= 0 && ih < g.H && img < imgs_here;
             // (quad-blocked input: four floats per position inside a quad's plane)
             tt[e] = ok ? img * int(x_img) + (ih * g.W + iw) * (t.x_c4 ? 4 : 1) : -1;  // NB*C*H*W*4 < 2^31 is checked on the host
@@ -354,8 +391,44 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
     // Tiles are decoded once, when their id is known, and the id is made wave-uniform first: decoded per step from the
     // LDS slot (a vector register) the divisions ran in the vector unit, some sixty instructions per step.
     int cn0, coh0, ckb, nn0 = 0, noh0 = 0, nkb = 0;
-    decode_tile(t, cur, cn0, coh0, ckb);
-    fill_ttab(ttab0, cn0, coh0);
+    int cp1 = t.P1, np1 = t.P1;  // patch positions staged for the tile (PACK: only the images its windows touch)
+    int noff = 0;                // PACK: the tile's first window inside its first image
+    auto decode = [&](int tile, int &n0, int &oh0, int &kb, int &off, int &p1) {
+        if constexpr (PACK) {
+            kb = tile % t.n_kblocks;
+            int sb = tile / t.n_kblocks;
+            if ((t.n_sblocks & 7) == 0) sb = (sb & 7) * (t.n_sblocks >> 3) + (sb >> 3);  // a contiguous run per XCD
+            const int w0 = sb * pk.S;  // N * windows per image + S < 2^31 is checked on the host
+            n0 = w0 / per_img_p;
+            off = w0 - n0 * per_img_p;
+            oh0 = 0;
+            p1 = min((off + pk.S - 1) / per_img_p + 1, g.N - n0) * patch_hw;
+        } else {
+            decode_tile(t, tile, n0, oh0, kb);
+            off = 0;
+            p1 = t.P1;
+        }
+    };
+    // PACK: the lane's window slots of a tile starting `off` windows into its first image
+    auto set_slots = [&](int off) {
+        if constexpr (PACK) {
+#pragma unroll
+            for (int j = 0; j < MT / 4; ++j) {
+                const int wl = off + (wm * (MT / 4) + j) * 32 + l32;  // < NB * per_img_p: NB is the longest run's span
+                const int base = wtab[2 * wl];
+                pool_pos[j] = wtab[2 * wl + 1];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) lds_off[4 * j + i] = base + (i >> 1) * g.sh * t.PW + (i & 1) * g.sw;
+            }
+        }
+    };
+    bool tail_taken = false;  // (thread 0) this workgroup has had its tile of the last, partial round
+    {
+        int coff;
+        decode(cur, cn0, coh0, ckb, coff, cp1);
+        set_slots(coff);
+    }
+    fill_ttab(ttab0, cn0, coh0, cp1);
     __syncthreads();
     // prologue: copies of the first step, with nothing to compute yet
     {
@@ -371,9 +444,9 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
         const int j = tid & 3;
         float *xl = buf0 + w_chunk;
         if (t.x_c4) {
-            for (int p0 = 0; p0 < t.P1; p0 += NT) {
+            for (int p0 = 0; p0 < cp1; p0 += NT) {
                 const int pos = p0 + tid;
-                if (pos < t.P1) {
+                if (pos < cp1) {
                     const int e = ttab0[pos];
 #pragma unroll
                     for (int half = 0; half < 2; ++half) {
@@ -383,9 +456,9 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
                 }
             }
         } else
-        for (int p0 = 0; p0 < t.P1; p0 += NT / 4) {
+        for (int p0 = 0; p0 < cp1; p0 += NT / 4) {
             const int pos = p0 + (tid >> 2);
-            if (pos < t.P1) {
+            if (pos < cp1) {
                 const int e = ttab0[pos];
 #pragma unroll
                 for (int half = 0; half < 2; ++half) {
@@ -409,12 +482,24 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
             __syncthreads();                // ... everyone's have; all waves are done with the other buffer
             if (chunk == 0) {
                 nxt = __builtin_amdgcn_readfirstlane(sched[tile_par]);  // written at least one barrier ago
-                if (tid == 0) sched[tile_par ^ 1] = atomicAdd(tile_counters + parity, 1);
+                if (tid == 0) {
+                    int drawn = atomicAdd(tile_counters + parity, 1);
+                    if constexpr (PACK) {
+                        // The tiles of the last, partial round belong to the first workgroups by number, one each (they
+                        // sit on different CUs): drawn freely, two of them can land on one CU and run at half speed
+                        // while other CUs idle, which is a whole round again.
+                        if (drawn >= pk.tail_start) {
+                            drawn = (!tail_taken && int(blockIdx.x) < pk.tail_n) ? pk.tail_start + int(blockIdx.x) : t.n_tiles;
+                            tail_taken = true;
+                        }
+                    }
+                    sched[tile_par ^ 1] = drawn;
+                }
                 if (nxt < t.n_tiles) {
-                    decode_tile(t, nxt, nn0, noh0, nkb);
+                    decode(nxt, nn0, noh0, nkb, noff, np1);
                     // no copy is in flight here (the wait above), and the slot's last readers were the copies of the
                     // previous tile; its first readers come a barrier later unless the tile has a single chunk
-                    fill_ttab(tile_par ? ttab0 : ttab1, nn0, noh0);
+                    fill_ttab(tile_par ? ttab0 : ttab1, nn0, noh0, np1);
                     if (t.n_chunks == 1) __syncthreads();
                 }
             }
@@ -425,7 +510,7 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
             const float *cmp = (step & 1) ? buf1 : buf0;
             const int *ttab = (same_tile ? tile_par == 0 : tile_par != 0) ? ttab0 : ttab1;  // tile k's table is slot k & 1
             conv_step<MT, WM, WN, KV, TT>(dma, cmp, ttab, x, wp, g, t, do_issue, same_tile ? cn0 : nn0, same_tile ? ckb : nkb,
-                                          ichunk, lds_off, acc);
+                                          ichunk, same_tile ? cp1 : np1, lds_off, acc);
         }
 
         // ---- epilogue: bias (+ReLU), coalesced NCHW stores; the next tile's first chunk is in flight ----
@@ -487,7 +572,8 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
             }
         }
         cur = nxt;
-        cn0 = nn0; coh0 = noh0; ckb = nkb;
+        cn0 = nn0; coh0 = noh0; ckb = nkb; cp1 = np1;
+        set_slots(noff);  // (the table reads wait for the copies in flight; so does the top of the next step)
         tile_par ^= 1;
     }
 }
@@ -791,11 +877,50 @@ __global__ void __launch_bounds__(256, 4) conv_f32_c1k3_pool_mfma_kernel(const f
     }
 }
 
-typedef TilePlan MfmaPlan;
+struct MfmaPlan : TilePlan {
+    int pack_S = 0;  // > 0: window-packed pooled tiles of this many window slots
+};
 
 // Tile shape with the best useful-lane fraction whose LDS footprint allows two workgroups per CU.
 // LDS the kernel keeps beyond the planner's count: the bias of every output channel (padded to whole channel blocks)
 inline size_t bias_lds_bytes(const ConvGeom &g) { return size_t((g.K + 63) / 64) * 64 * sizeof(float); }
+
+// Window-packed plan for the pooled kernel (MT = 4: one group of 32 window slots per wave): tiles of S = WM*32 pooling
+// windows cut from the batch's flat window sequence.  The patch stages every image a run of S windows can touch.
+bool plan_packed(const ConvGeom &g, int WM, int WN, size_t cap, MfmaPlan *out) {
+    const int rows = g.OH / 2, cols = g.OW / 2, S = WM * 32, K_BLK = WN * 32, T = g.KH * g.KW;
+    if (rows < 1 || cols < 1) return false;
+    const int per = rows * cols;
+    if (per >= S) return false;  // whole pooled images only
+    TileGeom t;
+    t.x_c4 = 0;
+    t.POW = cols;
+    t.NB = (per - 1 + S - 1) / per + 1;
+    t.TH = 2 * rows;
+    t.n_row_tiles = 1;
+    t.PH = (t.TH - 1) * g.sh + (g.KH - 1) * g.dh + 1;
+    t.PW = (2 * cols - 1) * g.sw + (g.KW - 1) * g.dw + 1;  // (the column an odd OW ends with is never pooled)
+    t.P1 = t.NB * t.PH * t.PW;
+    t.P1s = (t.P1 + 3) & ~3;
+    if (t.PH >= 4096 || t.PW >= 4096 || t.NB >= 256 || rows >= 1024 || cols >= 1024) return false;  // the packed table fields
+    if (int64_t(t.NB) * g.C * g.H * g.W * 4 >= (int64_t(1) << 31)) return false;
+    const int64_t windows = int64_t(g.N) * per;
+    if (windows + S >= (int64_t(1) << 31)) return false;
+    t.n_chunks = (g.C + CC - 1) / CC;
+    t.n_kblocks = (g.K + K_BLK - 1) / K_BLK;
+    t.n_sblocks = int((windows + S - 1) / S);
+    const int64_t n_tiles = int64_t(t.n_sblocks) * t.n_kblocks;
+    if (n_tiles >= (int64_t(1) << 30)) return false;
+    t.n_tiles = int(n_tiles);
+    // two staging buffers, two tile tables, scheduler slots, window table
+    const size_t lds = 2 * (size_t(T) * 32 * K_BLK + size_t(32) * t.P1s) + size_t(t.P1s) * 8 + 8 + size_t(t.NB) * per * 8;
+    if (lds > cap) return false;
+    out->MT = 4; out->WM = WM; out->WN = WN; out->t = t; out->lds_bytes = lds;
+    out->eff = double(windows) / (double(t.n_sblocks) * S);
+    out->score = out->eff;
+    out->pack_S = S;
+    return true;
+}
 
 bool plan_mfma(const ConvGeom &g, MfmaPlan *best, bool pool = false) {
     const size_t cap = 80 * 1024 - bias_lds_bytes(g);
@@ -807,20 +932,36 @@ bool plan_mfma(const ConvGeom &g, MfmaPlan *best, bool pool = false) {
     MfmaPlan wide, narrow;
     const bool ok_w = zant_plan_conv_tiles(g, 2, 2, 8, CC, sizeof(float), cap, &wide, pool, 0, 32, 0, 2, 4, 256, 4096);
     const bool ok_n = zant_plan_conv_tiles(g, 4, 1, 8, CC, sizeof(float), cap, &narrow, pool, 0, 32, 0, 2, 4, 256, 4096);
-    if (ok_n && (!ok_w || narrow.eff > wide.eff + 0.25)) { *best = narrow; return true; }
-    if (ok_w) { *best = wide; return true; }
-    return false;
+    bool ok = false;
+    if (ok_n && (!ok_w || narrow.eff > wide.eff + 0.25)) { *best = narrow; ok = true; }
+    else if (ok_w) { *best = wide; ok = true; }
+    if (pool) {
+        // small pooled images leave window slots empty (25 windows in 32): cut the tiles from the flat window sequence
+        MfmaPlan packed;
+        if (plan_packed(g, 2, 2, cap, &packed) && (!ok || packed.eff > best->eff + 0.1)) { *best = packed; ok = true; }
+    }
+    return ok;
 }
 
-template <int MT, int WM, int WN, int TT, bool POOL>
+template <int MT, int WM, int WN, int TT, bool POOL, bool PACK = false>
 void launch_mfma_tt(zant_ctx *ctx, const float *x, const float *wp, const float *bias, float *y, const ConvGeom &g,
                     const MfmaPlan &p, int relu, int *counter, int grid, int parity) {
     constexpr int KV = MT >= 8 ? 2 : 4;  // 64-bit operand reads keep 8 accumulator tiles inside 256 VGPRs
     // more than 64 KB of dynamic LDS has to be opted into once per kernel
-    if (!zant_raise_lds_limit(ctx, reinterpret_cast<const void *>(&conv_f32_mfma_kernel<MT, WM, WN, KV, TT, POOL>), 160 * 1024)) return;
-    ZANT_KERNEL_NAME(ctx, "conv_f32_mfma_kernel<%d,%d,%d,%d,%d,%s>", MT, WM, WN, KV, TT, POOL ? "true" : "false");
-    hipLaunchKernelGGL((conv_f32_mfma_kernel<MT, WM, WN, KV, TT, POOL>), dim3(grid), dim3(WM * WN * 64), p.lds_bytes + bias_lds_bytes(g),
-                       ctx->stream, x, wp, bias, y, g, p.t, relu, counter, parity);
+    if (!zant_raise_lds_limit(ctx, reinterpret_cast<const void *>(&conv_f32_mfma_kernel<MT, WM, WN, KV, TT, POOL, PACK>), 160 * 1024)) return;
+    PackGeom pk = {0, p.t.n_tiles, 0};
+    if (PACK) {
+        // a last round that fills at most one workgroup per CU is dealt out by workgroup number (both of the first two
+        // tiles of a workgroup are static, so the tail starts behind them)
+        pk.S = p.pack_S;
+        const int rem = p.t.n_tiles % grid;
+        if (rem > 0 && rem <= ctx->num_cus && p.t.n_tiles - rem >= 2 * grid) { pk.tail_start = p.t.n_tiles - rem; pk.tail_n = rem; }
+        ZANT_KERNEL_NAME(ctx, "conv_f32_mfma_kernel<%d,%d,%d,%d,%d,true,true>", MT, WM, WN, KV, TT);
+    } else {
+        ZANT_KERNEL_NAME(ctx, "conv_f32_mfma_kernel<%d,%d,%d,%d,%d,%s>", MT, WM, WN, KV, TT, POOL ? "true" : "false");
+    }
+    hipLaunchKernelGGL((conv_f32_mfma_kernel<MT, WM, WN, KV, TT, POOL, PACK>), dim3(grid), dim3(WM * WN * 64), p.lds_bytes + bias_lds_bytes(g),
+                       ctx->stream, x, wp, bias, y, g, p.t, relu, counter, parity, pk);
 }
 
 template <int MT, int WM, int WN, bool POOL>
@@ -835,6 +976,16 @@ void launch_mfma(zant_ctx *ctx, const float *x, const float *wp, const float *bi
 template <int WM, int WN>
 bool dispatch_mt(zant_ctx *ctx, const float *x, const float *wp, const float *bias, float *y, const ConvGeom &g,
                  const MfmaPlan &p, int relu, int *counter, int grid, bool pool, int parity) {
+    if (pool && p.pack_S > 0) {
+        if constexpr (WM == 2 && WN == 2) {
+            if (p.MT != 4) return false;
+            if (g.KH * g.KW == 9) launch_mfma_tt<4, WM, WN, 9, true, true>(ctx, x, wp, bias, y, g, p, relu, counter, grid, parity);
+            else launch_mfma_tt<4, WM, WN, 0, true, true>(ctx, x, wp, bias, y, g, p, relu, counter, grid, parity);
+            return true;
+        } else {
+            return false;
+        }
+    }
     if (pool) {
         switch (p.MT) {
         case 4: launch_mfma<4, WM, WN, true>(ctx, x, wp, bias, y, g, p, relu, counter, grid, parity); return true;
