@@ -106,7 +106,7 @@ int zant_hip_timer_stop(zant_ctx *ctx, float *elapsed_ms);
 int zant_hip_kernel_timing(zant_ctx *ctx, int enable);
 int zant_hip_kernel_ms(zant_ctx *ctx, float *elapsed_ms);
 /* The device function of the most recent operator's main kernel as a profiler's kernel trace names it, with its
- * template arguments (e.g. "conv_f32_mfma_kernel<4,2,2,4,9,true>"); "" where the launch site does not say.  The
+ * template arguments (e.g. "conv_f32_mfma_kernel<4,2,2,4,9,true,true>"); "" where the launch site does not say.  The
  * string lives in the context and changes with the next operator call. */
 const char *zant_hip_kernel_name(zant_ctx *ctx);
 

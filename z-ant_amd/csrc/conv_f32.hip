@@ -956,10 +956,8 @@ void launch_mfma_tt(zant_ctx *ctx, const float *x, const float *wp, const float 
         pk.S = p.pack_S;
         const int rem = p.t.n_tiles % grid;
         if (rem > 0 && rem <= ctx->num_cus && p.t.n_tiles - rem >= 2 * grid) { pk.tail_start = p.t.n_tiles - rem; pk.tail_n = rem; }
-        ZANT_KERNEL_NAME(ctx, "conv_f32_mfma_kernel<%d,%d,%d,%d,%d,true,true>", MT, WM, WN, KV, TT);
-    } else {
-        ZANT_KERNEL_NAME(ctx, "conv_f32_mfma_kernel<%d,%d,%d,%d,%d,%s>", MT, WM, WN, KV, TT, POOL ? "true" : "false");
     }
+    ZANT_KERNEL_NAME(ctx, "conv_f32_mfma_kernel<%d,%d,%d,%d,%d,%s,%s>", MT, WM, WN, KV, TT, POOL ? "true" : "false", PACK ? "true" : "false");
     hipLaunchKernelGGL((conv_f32_mfma_kernel<MT, WM, WN, KV, TT, POOL, PACK>), dim3(grid), dim3(WM * WN * 64), p.lds_bytes + bias_lds_bytes(g),
                        ctx->stream, x, wp, bias, y, g, p.t, relu, counter, parity, pk);
 }
