@@ -348,9 +348,17 @@ GEMM_MODE_CASES = [
 ]
 
 
+# ... and each of them exists for both tile shapes: 64 x 64 (four waves) while 128 x 64 tiles would leave more than half of
+# the CUs without one, 128 x 64 (eight waves) from there on.  `many_rows` grows M until the second shape is taken.
+@pytest.mark.parametrize("many_rows", [False, True], ids=["tile64x64", "tile128x64"])
 @pytest.mark.parametrize("M,K,N,ta,mis_a,mis_b,modes", GEMM_MODE_CASES)
-def test_gemm_copy_modes_vs_oracle(G, M, K, N, ta, mis_a, mis_b, modes):
+def test_gemm_copy_modes_vs_oracle(G, M, K, N, ta, mis_a, mis_b, modes, many_rows):
     import torch
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    n_tiles = -(-N // 64)
+    if many_rows:
+        M += 128 * (cus // 2 // n_tiles + 1)
+    assert (2 * -(-M // 128) * n_tiles > cus) == many_rows
     g = np.random.default_rng(M + 3 * K + 5 * N + ta)
     a = g.standard_normal((1, 1, K, M) if ta else (1, 1, M, K), dtype=np.float32)
     b = (g.standard_normal((1, 1, K, N)) * np.sqrt(2.0 / K)).astype(np.float32)
@@ -366,6 +374,6 @@ def test_gemm_copy_modes_vs_oracle(G, M, K, N, ta, mis_a, mis_b, modes):
     assert (A.data_ptr() % 16 != 0) == bool(mis_a) and (B.data_ptr() % 16 != 0) == bool(mis_b)
     y = torch.full((1, 1, M, N), -7.0, device="cuda:0")
     G.tm.gemm_lean(A, B, G.dev(c), 1.0, 1.0, bool(ta), False, y, "relu")
-    assert G.tm.context().kernel_name() == "gemm_f32_dma_kernel<1,4,2,%d,%d,5>" % modes
+    assert G.tm.context().kernel_name() == "gemm_f32_dma_kernel<1,%d,2,%d,%d,5>" % ((4 if many_rows else 2,) + modes)
     ref = zo.ReLU(zo.gemm(a, b, c, 1.0, 1.0, bool(ta), False))
     np.testing.assert_allclose(G.host(y), ref, rtol=G.RTOL, atol=G.ATOL)

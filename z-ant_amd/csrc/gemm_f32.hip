@@ -706,7 +706,12 @@ int run_gemm(zant_ctx *ctx, const float *A, const float *B, const float *C, floa
     }
     const int am = a_kc ? (g.a_vec ? KC16 : KC4) : RC4;
     const int bmode = b_kc ? (g.b_vec ? KC16 : KC4) : (g.b_vec ? RC16 : RC4);  // (b_vec with B stored [K][N]: N is a multiple of 4)
-    if (N > 32) dispatch_gemm_dma<1, 4, 2>(ctx, A, B, C, Y, g, am, bmode);  // 128 x 64 tile, 8 waves, 5 stages
+    // 128 x 64 tiles (8 waves, 5 stages) while they give at least every other CU one; below that 64 x 64 tiles (4 waves,
+    // two workgroups per CU): twice the tiles at half the work each (2048 x 256 x 4096: 144 -> 86 us), 4 % slower per
+    // flop where both fill the GPU.
+    const int64_t tiles_128 = ((M + 127) / 128) * ((N + 63) / 64);
+    if (N > 32 && 2 * tiles_128 <= ctx->num_cus) dispatch_gemm_dma<1, 2, 2>(ctx, A, B, C, Y, g, am, bmode);
+    else if (N > 32) dispatch_gemm_dma<1, 4, 2>(ctx, A, B, C, Y, g, am, bmode);
     else launch_gemm<1, 4, 1>(ctx, A, B, C, Y, g, a_kc, b_kc);              // 128 x 32 tile
     ZANT_LAUNCH_CHECK(ctx);
     return ZANT_OK;
