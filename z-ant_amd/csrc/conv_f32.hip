@@ -78,8 +78,8 @@ __device__ __forceinline__ float vmax3(float a, float b, float c) {
     return r;
 }
 
-// Window-packed tiles of the pooled kernel: window slots per tile; the tiles from `tail_start` on (tail_n of them, the
-// last partial round) are handed out one per workgroup, to workgroups 0 .. tail_n-1.
+// S: window-packed tiles of the pooled kernel, window slots per tile.  Every kernel: the tiles from `tail_start` on
+// (tail_n of them, the last partial round) are handed out one per workgroup, to workgroups 0 .. tail_n-1.
 struct PackGeom { int S, tail_start, tail_n; };
 
 // A few zero words that padding lanes of the asynchronous global->LDS copies read from.
@@ -271,8 +271,8 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
     int *ptab = reinterpret_cast<int *>(lds + 2 * buf_floats);     // [P1s]: img << 24 | patch row << 12 | patch column
     int *ttab0 = ptab + (PACK ? 0 : t.P1s);                        // [2][P1s]: per tile, a position's element offset in
     int *ttab1 = ttab0 + t.P1s;                                    //   the image group, -1 where the patch is padding
-    int *sched = ttab1 + t.P1s;                                    // [2]: tile ids handed out by thread 0
-    float *bias_l = reinterpret_cast<float *>(sched + 2);          // [n_kblocks * K_BLK]: the bias, zero past K
+    int *sched = ttab1 + t.P1s;                                    // [2]: tile ids handed out by thread 0; [2]: tail tile taken
+    float *bias_l = reinterpret_cast<float *>(sched + 4);          // [n_kblocks * K_BLK]: the bias, zero past K
     int *wtab = reinterpret_cast<int *>(bias_l + t.n_kblocks * K_BLK);  // PACK: [NB * windows per image][2]
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -357,7 +357,10 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
     } else {
         out_pos[0] = 0;
     }
-    if (tid == 0) sched[0] = blockIdx.x + gridDim.x;  // the second tile is static, later ones come from the counter
+    if (tid == 0) {
+        sched[0] = blockIdx.x + gridDim.x;  // the second tile is static, later ones come from the counter
+        sched[2] = 0;
+    }
     // Two counters take turns: this launch draws from tile_counters[parity] and re-arms the other one for the next
     // launch of the same operator, so that packed weights and counters can be kept across calls without a reset pass.
     if (tid == 0 && blockIdx.x == 0) tile_counters[parity ^ 1] = 2 * int(gridDim.x);
@@ -422,7 +425,6 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
             }
         }
     };
-    bool tail_taken = false;  // (thread 0) this workgroup has had its tile of the last, partial round
     {
         int coff;
         decode(cur, cn0, coh0, ckb, coff, cp1);
@@ -484,14 +486,12 @@ conv_f32_mfma_kernel(const float *__restrict__ x, const float *__restrict__ wp, 
                 nxt = __builtin_amdgcn_readfirstlane(sched[tile_par]);  // written at least one barrier ago
                 if (tid == 0) {
                     int drawn = atomicAdd(tile_counters + parity, 1);
-                    if constexpr (PACK) {
-                        // The tiles of the last, partial round belong to the first workgroups by number, one each (they
-                        // sit on different CUs): drawn freely, two of them can land on one CU and run at half speed
-                        // while other CUs idle, which is a whole round again.
-                        if (drawn >= pk.tail_start) {
-                            drawn = (!tail_taken && int(blockIdx.x) < pk.tail_n) ? pk.tail_start + int(blockIdx.x) : t.n_tiles;
-                            tail_taken = true;
-                        }
+                    // The tiles of a last round that fills at most one workgroup per CU belong to the first workgroups by
+                    // number, one each (they sit on different CUs): drawn freely, two of them land on one CU -- its two
+                    // workgroups finish together -- and run at half speed while other CUs idle, a whole round again.
+                    if (drawn >= pk.tail_start) {
+                        drawn = (sched[2] == 0 && int(blockIdx.x) < pk.tail_n) ? pk.tail_start + int(blockIdx.x) : t.n_tiles;
+                        sched[2] = 1;
                     }
                     sched[tile_par ^ 1] = drawn;
                 }
@@ -883,7 +883,8 @@ struct MfmaPlan : TilePlan {
 
 // Tile shape with the best useful-lane fraction whose LDS footprint allows two workgroups per CU.
 // LDS the kernel keeps beyond the planner's count: the bias of every output channel (padded to whole channel blocks)
-inline size_t bias_lds_bytes(const ConvGeom &g) { return size_t((g.K + 63) / 64) * 64 * sizeof(float); }
+// (and two more scheduler words)
+inline size_t bias_lds_bytes(const ConvGeom &g) { return size_t((g.K + 63) / 64) * 64 * sizeof(float) + 8; }
 
 // Window-packed plan for the pooled kernel (MT = 4: one group of 32 window slots per wave): tiles of S = WM*32 pooling
 // windows cut from the batch's flat window sequence.  The patch stages every image a run of S windows can touch.
@@ -949,14 +950,11 @@ void launch_mfma_tt(zant_ctx *ctx, const float *x, const float *wp, const float 
     constexpr int KV = MT >= 8 ? 2 : 4;  // 64-bit operand reads keep 8 accumulator tiles inside 256 VGPRs
     // more than 64 KB of dynamic LDS has to be opted into once per kernel
     if (!zant_raise_lds_limit(ctx, reinterpret_cast<const void *>(&conv_f32_mfma_kernel<MT, WM, WN, KV, TT, POOL, PACK>), 160 * 1024)) return;
-    PackGeom pk = {0, p.t.n_tiles, 0};
-    if (PACK) {
-        // a last round that fills at most one workgroup per CU is dealt out by workgroup number (both of the first two
-        // tiles of a workgroup are static, so the tail starts behind them)
-        pk.S = p.pack_S;
-        const int rem = p.t.n_tiles % grid;
-        if (rem > 0 && rem <= ctx->num_cus && p.t.n_tiles - rem >= 2 * grid) { pk.tail_start = p.t.n_tiles - rem; pk.tail_n = rem; }
-    }
+    PackGeom pk = {PACK ? p.pack_S : 0, p.t.n_tiles, 0};
+    // a last round that fills at most one workgroup per CU is dealt out by workgroup number (both of the first two tiles
+    // of a workgroup are static, so the tail starts behind them)
+    const int rem = p.t.n_tiles % grid;
+    if (rem > 0 && rem <= ctx->num_cus && p.t.n_tiles - rem >= 2 * grid) { pk.tail_start = p.t.n_tiles - rem; pk.tail_n = rem; }
     ZANT_KERNEL_NAME(ctx, "conv_f32_mfma_kernel<%d,%d,%d,%d,%d,%s,%s>", MT, WM, WN, KV, TT, POOL ? "true" : "false", PACK ? "true" : "false");
     hipLaunchKernelGGL((conv_f32_mfma_kernel<MT, WM, WN, KV, TT, POOL, PACK>), dim3(grid), dim3(WM * WN * 64), p.lds_bytes + bias_lds_bytes(g),
                        ctx->stream, x, wp, bias, y, g, p.t, relu, counter, parity, pk);
