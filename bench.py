@@ -28,8 +28,8 @@ if ROOT not in sys.path:
 # profile names, and reported only when the kernel this run launched for the dominant node is that same function
 # (otherwise null: the figure would describe a kernel that no longer runs).
 MEASURED_HBM_BYTES = {
-    "conv_f32_mfma_kernel<4,2,2,4,9,true,true>": 119.69e6,
-    "conv_f32_c1k3_pool_mfma_kernel<true,true>": 103.53e6,
+    "conv_f32_mfma_kernel<4,2,2,4,9,true,true>": 119.79e6,
+    "conv_f32_c1k3_pool_mfma_kernel<true,true>": 103.63e6,
     "gemm_f32_dma_kernel<1,4,2,0,0,5>": 60.91e6,  # the model's first Gemm (B packed at load)
     "gemm_f32_dma_kernel<1,4,2,0,3,5>": 60.93e6,  # the same shape through gemm_lean (B row-major)
     "gemm_f32_skinny_kernel<3>": 8.88e6,
